@@ -1,0 +1,126 @@
+/*
+ * oxk_oracle.h — CPU restatement of oxidize-c's quantized-matvec arithmetic.
+ *
+ * TEST INFRASTRUCTURE ONLY.  This library is the checker the HIP kernels are
+ * compared against; nothing in the shipped library links, loads or calls it.
+ *
+ * Every function restates one reference function (cited below, paths relative
+ * to the reference checkout, oxidize-c/...) in plain scalar C, compiled with
+ * -ffp-contract=off exactly like the reference (oxidize-c/Makefile:20-21).
+ * Unlike the reference, the dot functions can also hand back the per-sub-block
+ * int32 sums, which are the quantities the GPU path must reproduce bit for bit.
+ *
+ * Pinning status (what each function was checked against):
+ *   oxo_f16_to_f32        all 65536 inputs vs numpy float16 and vs the compiled
+ *                         reference; KATs of tests/test_oxk.c:8-47
+ *   oxo_f32_to_f16_bits   dense sample + ties/subnormals vs compiled reference
+ *   oxo_scale_min_k4      KATs tests/test_oxk.c:72-103; exhaustive byte triples
+ *                         vs compiled reference
+ *   oxo_quantize_q8_k/0   compiled reference through oc_matvec_quantized (the
+ *                         activation is left in `temp`); invariants (bsums)
+ *   oxo_dot_*             compiled reference scalar + dispatched kernels on the
+ *                         raw-block generator of tests/test_oxk_avx2_parity.c,
+ *                         closed forms, dequantised double-precision cross-check
+ *   oxo_matvec_*          compiled reference entry points, float bits
+ * No function is "parity unpinned".
+ */
+#ifndef OXK_ORACLE_H
+#define OXK_ORACLE_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* GGUF type ids used on this path (include/oxidize/quant.h:94-110). */
+enum {
+    OXO_Q8_0   = 7,
+    OXO_Q4_K_S = 12,
+    OXO_Q4_K_M = 13,
+    OXO_Q6_K   = 16,
+};
+
+#define OXO_QK_K        256u
+#define OXO_QK8_0       32u
+#define OXO_Q4_K_BYTES  144u
+#define OXO_Q6_K_BYTES  210u
+#define OXO_Q8_0_BYTES  34u
+#define OXO_Q8_K_BYTES  292u
+
+/* src/compute/oxk.c:26-56 */
+float    oxo_f16_to_f32(uint16_t h);
+/* src/compute/flash_attention.c:149-185 (round-half-up, not RNE) */
+uint16_t oxo_f32_to_f16_bits(float v);
+/* src/compute/oxk.c:60-75 */
+void     oxo_scale_min_k4(unsigned j, const uint8_t scales[12],
+                          uint8_t *sc, uint8_t *mn);
+
+/* src/compute/matvec.c:276-316 — n must be a multiple of 256. */
+void oxo_quantize_q8_k(const float *x, size_t n, uint8_t *out);
+/* src/compute/matvec.c:130-155 — n must be a multiple of 32. */
+void oxo_quantize_q8_0(const float *x, size_t n, uint8_t *out);
+
+/* src/compute/oxk.c:243-297.  `sub` (optional) receives 8 int32 per block:
+ * S_j = sum over sub-block j of nibble * q8.  `posmin` (optional) receives
+ * 2 int32 per block: {sum_j sc_j*S_j, sum_j m_j*B_j}. */
+float oxo_dot_q4_k_q8_k(const uint8_t *row, size_t blocks, const uint8_t *act,
+                        int32_t *sub, int32_t *posmin);
+/* src/compute/oxk.c:913-964.  `grp` (optional) receives 16 int32 per block. */
+float oxo_dot_q6_k_q8_k(const uint8_t *row, size_t blocks, const uint8_t *act,
+                        int32_t *grp);
+/* src/compute/oxk.c:224-241 (block-sequential scalar chain).  `isum`
+ * (optional) receives one int32 per block. */
+float oxo_dot_q8_0_q8_0(const uint8_t *row, size_t blocks, const uint8_t *act,
+                        int32_t *isum);
+
+/* 0 = not eligible for the integer path, 1 = Q8_0 activation, 2 = Q8_K
+ * (src/compute/matvec.c:99-127 restricted to the types above) and the stride
+ * rule of src/compute/matvec.c:961-985. */
+int oxo_act_kind(uint32_t qtype, size_t cols);
+int oxo_stride_ok(uint32_t qtype, size_t cols, size_t row_bytes);
+
+/* src/compute/matvec.c:833-907 (integer path only).  Returns 0 when handled,
+ * 1 when the reference would have taken its dequantise-to-f32 path (which
+ * this oracle does not restate).  `temp` receives the quantised activation. */
+int oxo_matvec_quantized(uint32_t qtype, const uint8_t *data, size_t rows,
+                         size_t cols, size_t row_bytes, const float *input,
+                         float *output, float *temp);
+/* src/compute/matvec.c:1525-1594 */
+int oxo_matvec_quantized_fused(const uint32_t *qtypes,
+                               const uint8_t *const *datas, const size_t *rows,
+                               size_t cols, const size_t *row_bytes,
+                               size_t n_outs, const float *input,
+                               float *const *outs, float *temp);
+/* src/compute/matvec.c:1597-1680 */
+int oxo_matvec_quantized_multi_input(const uint32_t *qtypes,
+                                     const uint8_t *const *datas,
+                                     const size_t *rows, size_t cols,
+                                     const size_t *row_bytes, size_t n_outs,
+                                     const float *const *inputs,
+                                     float *const *outs, float *temp);
+/* src/compute/matvec.c:1263-1488 (integer path; every output is the same
+ * single-vector dot, so no tiling is restated). */
+int oxo_matvec_quantized_batch(uint32_t qtype, const uint8_t *data,
+                               size_t rows, size_t cols, size_t row_bytes,
+                               const float *inputs, size_t in_stride,
+                               float *outputs, size_t out_stride, size_t n_vec,
+                               uint8_t *act_scratch, size_t act_bytes);
+/* src/compute/matvec.c:997-1014 with the default 4 MiB tile. */
+size_t oxo_matvec_batch_scratch_bytes(size_t max_cols);
+
+/* MoE routing as the prefill caller does it (src/model/llama.c:5965-6031):
+ * softmax over n_expert logits, top-k by repeated strict-greater scan (ties
+ * keep the lower index), optional renormalisation.  ids/weights: n_tok*k. */
+void oxo_moe_route(const float *logits, size_t n_tok, size_t n_expert,
+                   size_t k, int renorm, int32_t *ids, float *weights);
+
+/* Dequantise one row to f32 (src/compute/quantization.c:486-503, :633-670,
+ * :723-766) — used only as an independent cross-check of the layouts. */
+int oxo_dequant_row(uint32_t qtype, const uint8_t *row, size_t cols, float *out);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,66 @@
+"""Seeded synthetic tensors (raw Q4_K / Q6_K / Q8_0 blocks, f32 activations).
+
+Thin ctypes wrapper over ``liboxsynth.so`` (built from ``csrc/synth.c``).  The
+generator is integer-only, so the same seed gives the same bytes everywhere.
+Shapes and distributions follow the benchmark configurations: Q4_K d/dmin
+~ |N(0,0.02)|, 6-bit scales/mins uniform, nibbles uniform; Q6_K int8 scales in
+[-32,31], codes uniform; Q8_0 int8 in [-127,127], d ~ |N(0,0.01)|.
+"""
+import ctypes
+import os
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB = None
+
+Q8_0, Q4_K, Q6_K = 7, 13, 16
+BLOCK_BYTES = {Q8_0: 34, Q4_K: 144, 12: 144, Q6_K: 210}
+BLOCK_ELEMS = {Q8_0: 32, Q4_K: 256, 12: 256, Q6_K: 256}
+
+
+def _lib():
+    global _LIB
+    if _LIB is None:
+        path = os.path.join(_HERE, "liboxsynth.so")
+        if not os.path.exists(path):
+            raise RuntimeError(
+                "liboxsynth.so is not built; run `python -c 'import __graft_entry__ as g; g.build()'`")
+        lib = ctypes.CDLL(path)
+        for name in ("oxs_fill_q4_k", "oxs_fill_q6_k", "oxs_fill_q8_0"):
+            getattr(lib, name).argtypes = [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_uint64,
+                                           ctypes.c_uint64, ctypes.c_float]
+            getattr(lib, name).restype = None
+        lib.oxs_fill_normal_f32.argtypes = [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_uint64,
+                                            ctypes.c_uint64, ctypes.c_float]
+        lib.oxs_fill_normal_f32.restype = None
+        _LIB = lib
+    return _LIB
+
+
+def row_bytes(qtype, cols):
+    return cols // BLOCK_ELEMS[qtype] * BLOCK_BYTES[qtype]
+
+
+def weights(qtype, rows, cols, seed=0, stream=0, sigma=None, out=None):
+    """rows x cols matrix of raw blocks of `qtype`, as a flat uint8 array."""
+    if cols % BLOCK_ELEMS[qtype]:
+        raise ValueError("cols must be a whole number of blocks")
+    n_blocks = rows * (cols // BLOCK_ELEMS[qtype])
+    nbytes = n_blocks * BLOCK_BYTES[qtype]
+    if out is None:
+        out = np.empty(nbytes, dtype=np.uint8)
+    assert out.dtype == np.uint8 and out.size == nbytes and out.flags.c_contiguous
+    fn = {Q8_0: "oxs_fill_q8_0", Q4_K: "oxs_fill_q4_k", 12: "oxs_fill_q4_k",
+          Q6_K: "oxs_fill_q6_k"}[qtype]
+    if sigma is None:
+        sigma = 0.01 if qtype == Q8_0 else 0.02
+    getattr(_lib(), fn)(out.ctypes.data, n_blocks, seed, stream, sigma)
+    return out
+
+
+def normal(n, seed=0, stream=1000, scale=1.0):
+    """n float32 values ~ N(0,1)*scale."""
+    out = np.empty(n, dtype=np.float32)
+    _lib().oxs_fill_normal_f32(out.ctypes.data, n, seed, stream, scale)
+    return out
