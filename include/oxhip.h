@@ -1,0 +1,240 @@
+/*
+ * oxhip.h — C ABI of liboxhip: MI355X (gfx950) quantized matvec / matmul.
+ *
+ * Two layers, both plain C (pointers and sizes only):
+ *
+ *   1. Drop-in host API — same argument lists as the reference's
+ *      oxidize-c/include/oxidize/matvec.h.  Host pointers in, host pointers
+ *      out; weights are uploaded once (explicitly via oxh_weight_register or
+ *      on first sight) and stay resident in HBM.  The oxh_matvec_* functions
+ *      return a status; the oc_matvec_* symbols are the reference's own names
+ *      and signatures (void) layered on top of them.
+ *
+ *   2. Device-resident API — asynchronous launches on a caller stream over
+ *      device pointers, modelled on the reference's device ABI
+ *      (oxidize-c/include/oxidize/cuda_mmq.h:17-20, :57-72, :128-143).
+ *
+ * There is no CPU fallback anywhere in this library.  A shape the reference's
+ * integer path declines (oxidize-c/src/compute/matvec.c:99-127, :961-985)
+ * yields OXH_DECLINED so the caller can run its own CPU code; every other
+ * failure is an error code plus a message retrievable with oxh_last_error().
+ */
+#ifndef OXHIP_H
+#define OXHIP_H
+
+#include <stdbool.h>
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ─── status ──────────────────────────────────────────────────────────── */
+
+#define OXH_OK            0
+#define OXH_DECLINED      1   /* not an integer-path shape/type; nothing was written */
+#define OXH_ERR_HIP      (-1) /* a HIP runtime call failed                   */
+#define OXH_ERR_ARG      (-2) /* NULL pointer / overflow / bad size          */
+#define OXH_ERR_NO_DEVICE (-3)
+#define OXH_ERR_TOO_WIDE (-4) /* cols beyond what one workgroup can stage    */
+#define OXH_ERR_NOMEM    (-5)
+
+/* GGUF quantization type ids handled here; values are ABI
+ * (oxidize-c/include/oxidize/quant.h:94-110). */
+#define OXH_Q8_0    7u
+#define OXH_Q4_K_S 12u
+#define OXH_Q4_K_M 13u
+#define OXH_Q6_K   16u
+
+/* Block geometry (oxidize-c/include/oxidize/oxk.h:46-66). */
+#define OXH_QK_K         256u
+#define OXH_QK8_0         32u
+#define OXH_Q4_K_BYTES   144u
+#define OXH_Q6_K_BYTES   210u
+#define OXH_Q8_0_BYTES    34u
+#define OXH_Q8_K_BYTES   292u
+
+/* Thread-local text of the last failure on this thread ("" if none). */
+const char *oxh_last_error(void);
+
+/* ─── layer 2: device-resident, stream-ordered ────────────────────────── */
+
+/* Select the device and create the library's internal stream.  Idempotent.
+ * Replaces oc_cuda_init's device selection (oxidize-c/src/backends/cuda.cu:633). */
+int oxh_init(int device);
+void oxh_shutdown(void);
+
+/* 0 = declined, 1 = pairs with Q8_0 activations, 2 = pairs with Q8_K.
+ * Replaces fused_act_kind (oxidize-c/src/compute/matvec.c:99-127) and
+ * oc_cuda_mmq_supported (oxidize-c/include/oxidize/cuda_mmq.h:38-42). */
+int oxh_act_kind(uint32_t qtype, size_t cols);
+/* Packed row size for (qtype, cols), 0 if declined.  Replaces
+ * oc_cuda_mmq_row_bytes (cuda_mmq.h:44-48); no padding is ever added, the
+ * device layout is the on-disk layout. */
+size_t oxh_row_bytes(uint32_t qtype, size_t cols);
+/* Bytes of one quantised activation vector of `cols` values for `qtype`. */
+size_t oxh_act_bytes(uint32_t qtype, size_t cols);
+
+/* Activation quantisers.  d_x: n_vec vectors of `cols` floats, `in_stride`
+ * floats apart.  d_act: n_vec activations back to back, each in the exact
+ * byte format of the reference: Q8_K [f32 d][256 i8][16 i16 sums] per 256
+ * values (oxidize-c/src/compute/matvec.c:276-316), Q8_0 [f16 d][32 i8] per 32
+ * (matvec.c:130-155).  Replaces oc_cuda_mmq_quantize_x (cuda_mmq.h:128-132). */
+int oxh_quantize_q8_k(const float *d_x, size_t in_stride, size_t n_vec,
+                      size_t cols, void *d_act, void *stream);
+int oxh_quantize_q8_0(const float *d_x, size_t in_stride, size_t n_vec,
+                      size_t cols, void *d_act, void *stream);
+
+/* One weight matrix (or expert slice) of a grouped launch. */
+typedef struct OxhSegment {
+    const void *d_w;      /* packed rows, row stride = oxh_row_bytes()        */
+    float      *d_out;    /* output vector 0; vector v at d_out + v*out_stride */
+    size_t      rows;
+    size_t      act_first;/* index of this segment's first activation in d_acts */
+} OxhSegment;
+
+/* Decode GEMV over pre-quantised activations:
+ *   out[v][r] = dot(W[r], act[act_first + v])   for v < n_vec (1..8)
+ * for every segment, in ONE launch.  Covers the reference's row kernels
+ * oc_oxk_dot_rows_{q4_k,q6_k}_q8_k / _q8_0_q8_0 (oxidize-c/src/compute/oxk.c:
+ * 1447-1465) as used by matvec_fused_slice, matvec_fused_multi_slice and
+ * matvec_fused_multi_input_slice (matvec.c:640-797) and the small-batch
+ * rows path (matvec.c:1079-1102); the device analogue is
+ * oc_cuda_mmq_matvec / _matvec_expert (cuda_mmq.h:57-72).  Segments live in
+ * HOST memory and are copied into the launch. */
+int oxh_gemv_segments(uint32_t qtype, const OxhSegment *segs, size_t n_segs,
+                      size_t cols, const void *d_acts, size_t n_vec,
+                      size_t out_stride, void *stream);
+
+/* Prefill matmul on int8 MFMA: out[v*out_stride + r] = dot(W[r], act[v]) for
+ * v < n_vec (any count), Q8_K activations.  Replaces the prepared-row batch
+ * kernels oc_oxk_q4_k_prep_row + oc_oxk_dot_q4_k_prepped_multi
+ * (oxidize-c/src/compute/oxk.c:316-366, :787-836) driven by
+ * matvec_batch_prep_slice (matvec.c:1198-1228). */
+int oxh_mmq(uint32_t qtype, const void *d_w, size_t rows, size_t cols,
+            const void *d_acts, size_t n_vec, float *d_out, size_t out_stride,
+            void *stream);
+
+/* Test hook: the integer sub-block sums the GEMV kernel forms, written by the
+ * same device code path.  Q4_K: 8 int32 per super-block (S_j), Q6_K: 16 per
+ * super-block, Q8_0: 1 per block; layout [row][block][j].  The reference
+ * exposes no such API; the values are the intermediates of
+ * oxidize-c/src/compute/oxk.c:263-283, :932-954, :234-237. */
+int oxh_debug_subblock_sums(uint32_t qtype, const void *d_w, size_t rows,
+                            size_t cols, const void *d_act, int32_t *d_sums,
+                            void *stream);
+
+/* Device memory / stream / event plumbing so that C callers never include
+ * HIP headers (as cuda_mmq.h does with its void* stream). */
+int  oxh_malloc(void **d_ptr, size_t bytes);
+int  oxh_free(void *d_ptr);
+int  oxh_memcpy_h2d(void *d_dst, const void *h_src, size_t bytes, void *stream);
+int  oxh_memcpy_d2h(void *h_dst, const void *d_src, size_t bytes, void *stream);
+int  oxh_memset(void *d_dst, int value, size_t bytes, void *stream);
+int  oxh_stream_create(void **stream);
+int  oxh_stream_destroy(void *stream);
+int  oxh_stream_sync(void *stream);   /* NULL = the library's internal stream */
+int  oxh_event_create(void **event);
+int  oxh_event_destroy(void *event);
+int  oxh_event_record(void *event, void *stream);
+int  oxh_event_sync(void *event);
+int  oxh_event_elapsed_ms(void *start, void *stop, float *ms);
+/* name (<=255 chars), compute units, clock MHz, memory bytes. */
+int  oxh_device_info(char *name, size_t name_len, int *n_cu, int *clock_mhz,
+                     size_t *mem_bytes);
+
+/* ─── layer 1: drop-in host API ───────────────────────────────────────── */
+
+/* Make the bytes at [h_data, h_data+bytes) resident in HBM and remember the
+ * mapping, so later calls that pass any pointer inside that range (a whole
+ * tensor or an expert slice of a stacked tensor) run without an upload.
+ * Modelled on oc_cuda_init's weight upload (oxidize-c/src/backends/cuda.cu:
+ * 633-712).  Unregistered weights are registered on first use.  As in the
+ * reference, weights are taken to be immutable while registered: the host
+ * bytes are not looked at again, so unregister before reusing the memory. */
+int oxh_weight_register(const void *h_data, size_t bytes);
+int oxh_weight_unregister(const void *h_data);
+/* Drop every registered range (the host memory may then be reused or freed). */
+int oxh_weight_clear(void);
+/* Device address backing a registered host pointer, or NULL. */
+const void *oxh_weight_device_ptr(const void *h_data);
+
+/* Same arguments and results as oc_matvec_quantized
+ * (oxidize-c/include/oxidize/matvec.h:50-52; matvec.c:833-907): output[r] =
+ * dot(W[r], Q8(input)); `temp` (>= cols floats) receives the quantised
+ * activation bytes exactly as the reference leaves them there. */
+int oxh_matvec_quantized(uint32_t qtype, const uint8_t *data, size_t rows,
+                         size_t cols, size_t row_bytes, const float *input,
+                         float *output, float *temp);
+/* oc_matvec_quantized_fused (matvec.h:62-66; matvec.c:1525-1594). */
+int oxh_matvec_quantized_fused(const uint32_t *qtypes,
+                               const uint8_t *const *datas, const size_t *rows,
+                               size_t cols, const size_t *row_bytes,
+                               size_t n_outs, const float *input,
+                               float *const *outs, float *temp);
+/* oc_matvec_quantized_multi_input (matvec.h:72-76; matvec.c:1597-1680). */
+int oxh_matvec_quantized_multi_input(const uint32_t *qtypes,
+                                     const uint8_t *const *datas,
+                                     const size_t *rows, size_t cols,
+                                     const size_t *row_bytes, size_t n_outs,
+                                     const float *const *inputs,
+                                     float *const *outs, float *temp);
+/* oc_matvec_quantized_batch (matvec.h:118-124; matvec.c:1263-1488).
+ * `act_scratch`/`act_bytes` keep the reference's meaning for eligibility
+ * (NULL or too small for one activation => OXH_DECLINED); the quantised
+ * activations themselves stay on the device. */
+int oxh_matvec_quantized_batch(uint32_t qtype, const uint8_t *data,
+                               size_t rows, size_t cols, size_t row_bytes,
+                               const float *inputs, size_t in_stride,
+                               float *outputs, size_t out_stride, size_t n_vec,
+                               float *temp, uint8_t *act_scratch,
+                               size_t act_bytes);
+
+/* The reference's own symbols (matvec.h:50-52, :62-66, :72-76, :118-124,
+ * :132, :146-147, :81-88).  They call the oxh_ functions above.  Because they
+ * return void, a decline or failure is routed to the handler installed with
+ * oxh_set_decline_handler(); with no handler installed the process prints the
+ * error and aborts — it never silently computes on the CPU. */
+typedef struct {
+    size_t activation_quantizations;
+    size_t parallel_dispatches;
+    size_t fallback_calls;
+} OcMatvecFusedTestStats;
+
+void oc_matvec_quantized(uint32_t qtype, const uint8_t *data, size_t rows,
+                         size_t cols, size_t row_bytes, const float *input,
+                         float *output, float *temp);
+void oc_matvec_quantized_fused(const uint32_t *qtypes,
+                               const uint8_t *const *datas, const size_t *rows,
+                               size_t cols, const size_t *row_bytes,
+                               size_t n_outs, const float *input,
+                               float *const *outs, float *temp);
+void oc_matvec_quantized_multi_input(const uint32_t *qtypes,
+                                     const uint8_t *const *datas,
+                                     const size_t *rows, size_t cols,
+                                     const size_t *row_bytes, size_t n_outs,
+                                     const float *const *inputs,
+                                     float *const *outs, float *temp);
+void oc_matvec_quantized_batch(uint32_t qtype, const uint8_t *data,
+                               size_t rows, size_t cols, size_t row_bytes,
+                               const float *inputs, size_t in_stride,
+                               float *outputs, size_t out_stride, size_t n_vec,
+                               float *temp, uint8_t *act_scratch,
+                               size_t act_bytes);
+size_t oc_matvec_batch_scratch_bytes(size_t max_cols);
+void oc_matvec_set_fused(bool enabled);
+bool oc_matvec_fused_enabled(void);
+void oc_matvec_fused_test_reset(void);
+OcMatvecFusedTestStats oc_matvec_fused_test_stats(void);
+
+/* Called by the void oc_matvec_* symbols when the oxh_ call did not return
+ * OXH_OK.  `which` is 0 single, 1 fused, 2 multi_input, 3 batch; `status` is
+ * the oxh_ status.  A maintainer points this at the original CPU functions. */
+typedef void (*OxhDeclineHandler)(int which, int status, void *user);
+void oxh_set_decline_handler(OxhDeclineHandler fn, void *user);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* OXHIP_H */

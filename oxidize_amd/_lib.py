@@ -1,0 +1,107 @@
+"""ctypes binding of liboxhip.so (the C ABI declared in include/oxhip.h).
+
+Loading fails loudly when the library has not been built: there is no Python
+or CPU implementation behind these calls.
+"""
+import ctypes
+import os
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "liboxhip.so")
+
+OK, DECLINED = 0, 1
+ERR_HIP, ERR_ARG, ERR_NO_DEVICE, ERR_TOO_WIDE, ERR_NOMEM = -1, -2, -3, -4, -5
+
+V = ctypes.c_void_p
+Z = ctypes.c_size_t
+U32 = ctypes.c_uint32
+I = ctypes.c_int
+
+
+class OxhSegment(ctypes.Structure):
+    _fields_ = [("d_w", V), ("d_out", V), ("rows", Z), ("act_first", Z)]
+
+
+class OcMatvecFusedTestStats(ctypes.Structure):
+    _fields_ = [("activation_quantizations", Z), ("parallel_dispatches", Z),
+                ("fallback_calls", Z)]
+
+
+# name -> (restype, argtypes); every symbol include/oxhip.h declares
+SIGNATURES = {
+    "oxh_last_error": (ctypes.c_char_p, []),
+    "oxh_init": (I, [I]),
+    "oxh_shutdown": (None, []),
+    "oxh_act_kind": (I, [U32, Z]),
+    "oxh_row_bytes": (Z, [U32, Z]),
+    "oxh_act_bytes": (Z, [U32, Z]),
+    "oxh_quantize_q8_k": (I, [V, Z, Z, Z, V, V]),
+    "oxh_quantize_q8_0": (I, [V, Z, Z, Z, V, V]),
+    "oxh_gemv_segments": (I, [U32, ctypes.POINTER(OxhSegment), Z, Z, V, Z, Z, V]),
+    "oxh_mmq": (I, [U32, V, Z, Z, V, Z, V, Z, V]),
+    "oxh_debug_subblock_sums": (I, [U32, V, Z, Z, V, V, V]),
+    "oxh_malloc": (I, [ctypes.POINTER(V), Z]),
+    "oxh_free": (I, [V]),
+    "oxh_memcpy_h2d": (I, [V, V, Z, V]),
+    "oxh_memcpy_d2h": (I, [V, V, Z, V]),
+    "oxh_memset": (I, [V, I, Z, V]),
+    "oxh_stream_create": (I, [ctypes.POINTER(V)]),
+    "oxh_stream_destroy": (I, [V]),
+    "oxh_stream_sync": (I, [V]),
+    "oxh_event_create": (I, [ctypes.POINTER(V)]),
+    "oxh_event_destroy": (I, [V]),
+    "oxh_event_record": (I, [V, V]),
+    "oxh_event_sync": (I, [V]),
+    "oxh_event_elapsed_ms": (I, [V, V, ctypes.POINTER(ctypes.c_float)]),
+    "oxh_device_info": (I, [ctypes.c_char_p, Z, ctypes.POINTER(I), ctypes.POINTER(I),
+                            ctypes.POINTER(Z)]),
+    "oxh_weight_register": (I, [V, Z]),
+    "oxh_weight_unregister": (I, [V]),
+    "oxh_weight_clear": (I, []),
+    "oxh_weight_device_ptr": (V, [V]),
+    "oxh_matvec_quantized": (I, [U32, V, Z, Z, Z, V, V, V]),
+    "oxh_matvec_quantized_fused": (I, [V, V, V, Z, V, Z, V, V, V]),
+    "oxh_matvec_quantized_multi_input": (I, [V, V, V, Z, V, Z, V, V, V]),
+    "oxh_matvec_quantized_batch": (I, [U32, V, Z, Z, Z, V, Z, V, Z, Z, V, V, Z]),
+    "oc_matvec_quantized": (None, [U32, V, Z, Z, Z, V, V, V]),
+    "oc_matvec_quantized_fused": (None, [V, V, V, Z, V, Z, V, V, V]),
+    "oc_matvec_quantized_multi_input": (None, [V, V, V, Z, V, Z, V, V, V]),
+    "oc_matvec_quantized_batch": (None, [U32, V, Z, Z, Z, V, Z, V, Z, Z, V, V, Z]),
+    "oc_matvec_batch_scratch_bytes": (Z, [Z]),
+    "oc_matvec_set_fused": (None, [ctypes.c_bool]),
+    "oc_matvec_fused_enabled": (ctypes.c_bool, []),
+    "oc_matvec_fused_test_reset": (None, []),
+    "oc_matvec_fused_test_stats": (OcMatvecFusedTestStats, []),
+    "oxh_set_decline_handler": (None, [V, V]),
+}
+
+_LIB = None
+
+
+class OxhError(RuntimeError):
+    def __init__(self, status, message):
+        super().__init__("liboxhip status %d: %s" % (status, message))
+        self.status = status
+
+
+def lib():
+    global _LIB
+    if _LIB is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(
+                "liboxhip.so has not been built (expected %s); run "
+                "`python -c 'import __graft_entry__ as g; g.build()'`" % LIB_PATH)
+        handle = ctypes.CDLL(LIB_PATH)
+        for name, (res, args) in SIGNATURES.items():
+            fn = getattr(handle, name)
+            fn.restype = res
+            fn.argtypes = args
+        _LIB = handle
+    return _LIB
+
+
+def check(status):
+    """Raise on anything but OXH_OK."""
+    if status != OK:
+        raise OxhError(status, lib().oxh_last_error().decode("utf-8", "replace"))
+    return status

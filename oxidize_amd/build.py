@@ -1,0 +1,63 @@
+"""Build recipes for the native libraries (run on a CPU-only machine too).
+
+    liboxhip.so    HIP kernels + C host layer (hipcc cross-compiles gfx950)
+    liboxsynth.so  synthetic tensor generator (gcc)
+
+Everything is built in-tree next to this file so that the shared objects
+travel with the source tree.
+"""
+import os
+import shutil
+import subprocess
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(HERE)
+CSRC = os.path.join(HERE, "csrc")
+INCLUDE = os.path.join(ROOT, "include")
+
+HIPCC = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+CC = os.environ.get("CC", "gcc")
+
+# -ffp-contract=off: the block terms must round exactly like the reference's
+# C code.  -packed-fp32-ops is switched off on purpose for this target.
+HIP_FLAGS = ["--offload-arch=gfx950", "-O3", "-fPIC", "-std=c++17", "-ffp-contract=off",
+             "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+             "-Wall", "-Wno-unused-command-line-argument"]
+C_FLAGS = ["-std=c11", "-O2", "-fPIC", "-Wall", "-Wextra", "-ffp-contract=off"]
+
+
+def _run(cmd):
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError("command failed: %s\n%s" % (" ".join(cmd), proc.stdout))
+    return proc.stdout
+
+
+def build_oxhip(verbose=False):
+    obj_hip = os.path.join(CSRC, "oxh_kernels.o")
+    obj_c = os.path.join(CSRC, "oc_matvec.o")
+    out = os.path.join(HERE, "liboxhip.so")
+    log = _run([HIPCC] + HIP_FLAGS + ["-I", INCLUDE, "-I", CSRC, "-c",
+                                     os.path.join(CSRC, "oxh_kernels.hip"), "-o", obj_hip])
+    log += _run([CC] + C_FLAGS + ["-I", INCLUDE, "-I", CSRC, "-c",
+                                  os.path.join(CSRC, "oc_matvec.c"), "-o", obj_c])
+    log += _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", out, obj_hip, obj_c,
+                 "-lpthread", "-Wno-unused-command-line-argument"])
+    if verbose and log.strip():
+        print(log)
+    return out
+
+
+def build_synth():
+    out = os.path.join(HERE, "liboxsynth.so")
+    _run([CC] + C_FLAGS + ["-fopenmp", "-shared", "-o", out, os.path.join(CSRC, "synth.c")])
+    return out
+
+
+def build_all(verbose=False):
+    return [build_oxhip(verbose), build_synth()]
+
+
+if __name__ == "__main__":
+    for path in build_all(verbose=True):
+        print("built", path)

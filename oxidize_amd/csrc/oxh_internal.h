@@ -1,0 +1,24 @@
+/* oxh_internal.h — symbols shared between the HIP translation unit and the C
+ * host layer of liboxhip; not part of the public ABI. */
+#ifndef OXH_INTERNAL_H
+#define OXH_INTERNAL_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* printf-style with exactly two %s slots (either may be NULL). */
+void oxh_set_error(const char *fmt, const char *a, const char *b);
+/* The stream created by oxh_init(). */
+void *oxh_internal_stream(void);
+/* Largest n_vec (1..8) one GEMV launch can stage for (qtype, cols); 0 when
+ * even a single activation does not fit. */
+size_t oxh_gemv_max_nvec(uint32_t qtype, size_t cols);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,792 @@
+/*
+ * oxh_kernels.hip — gfx950 kernels and the thin device-resident C ABI of
+ * liboxhip (layer 2 of include/oxhip.h).
+ *
+ * Arithmetic contract (all paths relative to the reference checkout):
+ *   Q8_K / Q8_0 activation bytes  oxidize-c/src/compute/matvec.c:276-316, :130-155
+ *   f32 -> f16 (round half up)    oxidize-c/src/compute/flash_attention.c:149-185
+ *   Q4_K x Q8_K block dot         oxidize-c/src/compute/oxk.c:243-297
+ *   Q6_K x Q8_K block dot         oxidize-c/src/compute/oxk.c:913-964
+ *   Q8_0 x Q8_0 block dot         oxidize-c/src/compute/oxk.c:224-241
+ *
+ * All integer sums are exact, so they may be formed in any order.  The f32
+ * part keeps the reference's order: one term per block, rounded exactly as
+ * `dw*dq*(float)pos - dmin*dq*(float)min_acc`, then a strictly sequential sum
+ * over the blocks of a row starting from 0.0f.  Float contraction is disabled
+ * for this file (build flag -ffp-contract=off and the pragma below).
+ *
+ * Wave64 only.  Build: hipcc --offload-arch=gfx950 -O3 -ffp-contract=off
+ *   -Xclang -target-feature -Xclang -packed-fp32-ops
+ */
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <string.h>
+
+#include "oxhip.h"
+#include "oxh_internal.h"
+
+#pragma clang fp contract(off)
+
+/* ─── error plumbing ──────────────────────────────────────────────────── */
+
+static thread_local char g_err[512] = "";
+
+extern "C" const char *oxh_last_error(void) { return g_err; }
+
+extern "C" void oxh_set_error(const char *fmt, const char *a, const char *b)
+{
+    snprintf(g_err, sizeof g_err, fmt, a ? a : "", b ? b : "");
+}
+
+static int hip_fail(hipError_t e, const char *what)
+{
+    snprintf(g_err, sizeof g_err, "HIP error in %s: %s", what, hipGetErrorString(e));
+    return OXH_ERR_HIP;
+}
+
+#define HIP_TRY(call)                                                          \
+    do {                                                                       \
+        hipError_t e_ = (call);                                                \
+        if (e_ != hipSuccess) return hip_fail(e_, #call);                      \
+    } while (0)
+
+static int arg_fail(const char *what)
+{
+    snprintf(g_err, sizeof g_err, "invalid argument: %s", what);
+    return OXH_ERR_ARG;
+}
+
+/* ─── small device helpers ────────────────────────────────────────────── */
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+/* 16-byte vector with only 2-byte alignment: Q6_K (210 B) and Q8_0 (34 B)
+ * blocks start on even addresses.  gfx9+ under HSA runs with unaligned
+ * global access enabled, and the compiler emits one global_load_dwordx4. */
+struct __attribute__((packed, aligned(2))) U32x4u2 { uint32_t x, y, z, w; };
+struct __attribute__((packed, aligned(2))) U32u2 { uint32_t v; };
+
+__device__ __forceinline__ int dot4(uint32_t a, uint32_t b, int c)
+{
+    return __builtin_amdgcn_sdot4((int)a, (int)b, c, false);
+}
+
+/* Sum over the four lanes of a quad; every lane receives the total. */
+__device__ __forceinline__ int quad_sum(int v)
+{
+    v += __builtin_amdgcn_update_dpp(0, v, 0xB1, 0xF, 0xF, false); /* lanes ^1 */
+    v += __builtin_amdgcn_update_dpp(0, v, 0x4E, 0xF, 0xF, false); /* lanes ^2 */
+    return v;
+}
+
+/* Exact binary16 -> binary32 including subnormals (integer-only so it does
+ * not depend on the wave's denormal mode). */
+__device__ __forceinline__ float half_bits_to_float(uint32_t h)
+{
+    const uint32_t sign = (h & 0x8000u) << 16;
+    const uint32_t e = (h >> 10) & 31u;
+    const uint32_t m = h & 0x3FFu;
+    uint32_t bits;
+    if (e == 31u) {
+        bits = sign | 0x7F800000u | (m << 13);
+    } else if (e != 0u) {
+        bits = sign | ((e + 112u) << 23) | (m << 13);
+    } else if (m == 0u) {
+        bits = sign;
+    } else {
+        const uint32_t lz = (uint32_t)__clz((int)m) - 21u;   /* shifts to bit 10 */
+        bits = sign | ((113u - lz) << 23) | (((m << lz) & 0x3FFu) << 13);
+    }
+    return __uint_as_float(bits);
+}
+
+/* binary32 -> binary16 bits, round-half-UP on the dropped bits
+ * (flash_attention.c:149-185). */
+__device__ __forceinline__ uint32_t float_to_half_bits_half_up(float v)
+{
+    const uint32_t u = __float_as_uint(v);
+    const uint32_t sign = (u >> 16) & 0x8000u;
+    const int e32 = (int)((u >> 23) & 0xFFu);
+    const uint32_t man = u & 0x7FFFFFu;
+    if (e32 == 255) {
+        if (man == 0u) return sign | 0x7C00u;
+        uint32_t payload = man >> 13;
+        if (payload == 0u) payload = 1u;
+        return sign | 0x7C00u | payload;
+    }
+    const int e16 = e32 - 112;
+    if (e16 >= 31) return sign | 0x7C00u;
+    if (e16 >= 1) {
+        uint32_t out = ((uint32_t)e16 << 10) | (man >> 13);
+        if (man & 0x1000u) {
+            out += 1u;
+            if (out >= 0x7C00u) return sign | 0x7C00u;
+        }
+        return sign | out;
+    }
+    if (e16 < -10) return sign;
+    const uint32_t full = man | 0x800000u;
+    const uint32_t sh = (uint32_t)(14 - e16);
+    uint32_t out = full >> sh;
+    if ((full >> (sh - 1u)) & 1u) out += 1u;
+    return sign | out;
+}
+
+__device__ __forceinline__ int quantize_one(float x, float inv)
+{
+    /* lrintf under round-to-nearest-even == v_rndne_f32 + convert */
+    int v = (int)rintf(x * inv);
+    v = v > 127 ? 127 : v;
+    v = v < -128 ? -128 : v;
+    return v;
+}
+
+/* ─── activation quantisers ───────────────────────────────────────────── */
+
+/* One wave per 256-value block; lane l owns values 4l..4l+3. */
+__global__ __launch_bounds__(256) void
+k_quantize_q8_k(const float *__restrict__ x, size_t in_stride, uint32_t blocks_per_vec,
+                uint32_t total_blocks, uint8_t *__restrict__ act)
+{
+    const uint32_t lane = threadIdx.x & 63u;
+    const uint32_t gb = blockIdx.x * 4u + (threadIdx.x >> 6);
+    if (gb >= total_blocks) return;
+    const uint32_t vec = gb / blocks_per_vec;
+    const uint32_t blk = gb - vec * blocks_per_vec;
+    const float *src = x + (size_t)vec * in_stride + (size_t)blk * 256u + 4u * lane;
+    const float v0 = src[0], v1 = src[1], v2 = src[2], v3 = src[3];
+
+    /* max |x| over the block; NaNs never win a '>' comparison in the
+     * reference's scan, fmaxf drops them the same way */
+    float amax = fmaxf(fmaxf(fabsf(v0), fabsf(v1)), fmaxf(fabsf(v2), fabsf(v3)));
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) amax = fmaxf(amax, __shfl_xor(amax, m, 64));
+
+    const float d = amax / 127.0f;
+    const float inv = (d != 0.0f) ? 1.0f / d : 0.0f;
+    const int q0 = quantize_one(v0, inv), q1 = quantize_one(v1, inv);
+    const int q2 = quantize_one(v2, inv), q3 = quantize_one(v3, inv);
+
+    uint8_t *dst = act + (size_t)gb * OXH_Q8_K_BYTES;
+    const uint32_t packed = (uint32_t)(q0 & 255) | ((uint32_t)(q1 & 255) << 8) |
+                            ((uint32_t)(q2 & 255) << 16) | ((uint32_t)(q3 & 255) << 24);
+    reinterpret_cast<uint32_t *>(dst + 4)[lane] = packed;
+    if (lane == 0) *reinterpret_cast<float *>(dst) = d;
+
+    const int s = quad_sum(q0 + q1 + q2 + q3);   /* 16 values = one bsum group */
+    if ((lane & 3u) == 0u)
+        reinterpret_cast<int16_t *>(dst + 260)[lane >> 2] = (int16_t)s;
+}
+
+/* One wave per 8 blocks of 32 values; lane l owns values 4l..4l+3 of the
+ * 256-value span, i.e. 8 lanes per block. */
+__global__ __launch_bounds__(256) void
+k_quantize_q8_0(const float *__restrict__ x, size_t in_stride, uint32_t blocks_per_vec,
+                uint32_t n_vec, uint8_t *__restrict__ act)
+{
+    const uint32_t lane = threadIdx.x & 63u;
+    const uint32_t spans_per_vec = (blocks_per_vec + 7u) / 8u;
+    const uint32_t gs = blockIdx.x * 4u + (threadIdx.x >> 6);
+    if (gs >= spans_per_vec * n_vec) return;
+    const uint32_t vec = gs / spans_per_vec;
+    const uint32_t span = gs - vec * spans_per_vec;
+    const uint32_t blk = span * 8u + (lane >> 3);
+    const bool live = blk < blocks_per_vec;
+    float v0 = 0.f, v1 = 0.f, v2 = 0.f, v3 = 0.f;
+    if (live) {
+        const float *src = x + (size_t)vec * in_stride + (size_t)blk * 32u + 4u * (lane & 7u);
+        v0 = src[0]; v1 = src[1]; v2 = src[2]; v3 = src[3];
+    }
+    float amax = fmaxf(fmaxf(fabsf(v0), fabsf(v1)), fmaxf(fabsf(v2), fabsf(v3)));
+#pragma unroll
+    for (int m = 4; m >= 1; m >>= 1) amax = fmaxf(amax, __shfl_xor(amax, m, 64));
+    const float d = amax / 127.0f;
+    const float inv = (d != 0.0f) ? 1.0f / d : 0.0f;
+    const int q0 = quantize_one(v0, inv), q1 = quantize_one(v1, inv);
+    const int q2 = quantize_one(v2, inv), q3 = quantize_one(v3, inv);
+    if (!live) return;
+    uint8_t *dst = act + ((size_t)vec * blocks_per_vec + blk) * OXH_Q8_0_BYTES;
+    /* the block starts on an even address only: 16-bit stores */
+    uint16_t *q16 = reinterpret_cast<uint16_t *>(dst + 2 + 4u * (lane & 7u));
+    q16[0] = (uint16_t)((q0 & 255) | ((q1 & 255) << 8));
+    q16[1] = (uint16_t)((q2 & 255) | ((q3 & 255) << 8));
+    if ((lane & 7u) == 0u)
+        *reinterpret_cast<uint16_t *>(dst) = (uint16_t)float_to_half_bits_half_up(d);
+}
+
+/* ─── decode GEMV ─────────────────────────────────────────────────────── */
+
+#define OXH_MAX_SEGS 32
+#define OXH_GEMV_WAVES 4          /* waves per workgroup */
+#define OXH_MAX_NV 8
+
+/* Bytes of LDS one staged Q8_K activation takes: 256 B of values, 16 B of
+ * sub-block sums and 4 B of scale per block, rounded up so the next
+ * activation's 16-byte vectors stay aligned. */
+__host__ __device__ static inline uint32_t q8k_lds_bytes(uint32_t blocks)
+{
+    return (blocks * (256u + 16u + 4u) + 15u) & ~15u;
+}
+
+struct SegTable {
+    const uint8_t *w[OXH_MAX_SEGS];
+    float *out[OXH_MAX_SEGS];
+    uint32_t rows[OXH_MAX_SEGS];
+    uint32_t act_first[OXH_MAX_SEGS];
+    uint32_t wg_begin[OXH_MAX_SEGS + 1];   /* first workgroup of each segment */
+    uint32_t n;
+};
+
+struct GemvParams {
+    uint32_t blocks;        /* weight blocks per row                        */
+    uint32_t magic;         /* ceil(2^32 / blocks), for g / blocks          */
+    uint32_t rows_per_wave; /* RW                                           */
+    uint32_t n_vec;         /* activations per segment (1..8)               */
+    uint32_t act_bytes;     /* bytes of one quantised activation            */
+    uint32_t out_stride;    /* floats between output vectors                */
+    uint32_t term_stride;   /* blocks + 1 (LDS row pitch of the term table) */
+    int32_t *dump;          /* debug: sub-block sums, or NULL               */
+};
+
+/* LDS layout for the Q8_K-activation kernels (per workgroup), in this order:
+ *   per activation v: q  [4][blocks*4] x 16 B   values of (block, 64-span s),
+ *                        quarter i, at ((i*blocks*4) + block*4 + s)
+ *                     bs [blocks*4]   x 4 B    Q4_K: B_{2s} | B_{2s+1}<<16
+ *                     dq [blocks]     x 4 B
+ *   terms: [waves][n_vec][rows_per_wave][term_stride] f32
+ * For Q6_K the q array is indexed by (block, unit u=(n,lh)), quarter k, and
+ * bs holds 4 x int32 per unit (32*bsum of its 4 groups), see k_gemv_q6_k. */
+
+__device__ __forceinline__ uint32_t find_segment(const SegTable &t, uint32_t wg)
+{
+    uint32_t s = 0;
+    while (s + 1 < t.n && wg >= t.wg_begin[s + 1]) s++;
+    return s;
+}
+
+/* Q4_K x Q8_K.  Four lanes per super-block: lane (b, s) owns nibble bytes
+ * [32s, 32s+32) of block b, i.e. sub-blocks 2s (low nibbles) and 2s+1 (high
+ * nibbles), elements [64s, 64s+64).  16 blocks = 2304 contiguous bytes per
+ * wave pass. */
+template <bool DUMP>
+__global__ __launch_bounds__(OXH_GEMV_WAVES * 64) void
+k_gemv_q4_k(const SegTable segs, const GemvParams p, const uint8_t *__restrict__ acts)
+{
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    const uint32_t tid = threadIdx.x;
+    const uint32_t lane = tid & 63u;
+    const uint32_t wave = tid >> 6;
+    const uint32_t B = p.blocks;
+    const uint32_t NV = p.n_vec;
+
+    const uint32_t seg = find_segment(segs, blockIdx.x);
+    const uint32_t wg_in_seg = blockIdx.x - segs.wg_begin[seg];
+    const uint32_t seg_rows = segs.rows[seg];
+
+    const uint32_t act_lds = q8k_lds_bytes(B);               /* per activation */
+    float *const terms = reinterpret_cast<float *>(lds + (size_t)act_lds * NV) +
+                         (size_t)wave * NV * p.rows_per_wave * p.term_stride;
+
+    /* stage the segment's activations */
+    for (uint32_t v = 0; v < NV; v++) {
+        const uint8_t *a = acts + (size_t)(segs.act_first[seg] + v) * p.act_bytes;
+        uint8_t *base = lds + (size_t)v * act_lds;
+        uint32_t *qd = reinterpret_cast<uint32_t *>(base);
+        uint32_t *bs = reinterpret_cast<uint32_t *>(base + B * 256u);
+        float *dq = reinterpret_cast<float *>(base + B * 256u + B * 16u);
+        for (uint32_t j = tid; j < B * 64u; j += OXH_GEMV_WAVES * 64u) {
+            const uint32_t blk = j >> 6, w = j & 63u;
+            const uint32_t c = w >> 2, s = c >> 2, i = c & 3u;
+            const uint32_t val = *reinterpret_cast<const uint32_t *>(a + (size_t)blk * 292u + 4u + 4u * w);
+            qd[((i * B * 4u) + blk * 4u + s) * 4u + (w & 3u)] = val;
+        }
+        for (uint32_t j = tid; j < B * 4u; j += OXH_GEMV_WAVES * 64u) {
+            const uint32_t blk = j >> 2, s = j & 3u;
+            const uint32_t *sp = reinterpret_cast<const uint32_t *>(a + (size_t)blk * 292u + 260u) + 2u * s;
+            const uint32_t p0 = sp[0], p1 = sp[1];
+            const int b0 = (int)(int16_t)(p0 & 0xFFFFu) + (int)(int16_t)(p0 >> 16);
+            const int b1 = (int)(int16_t)(p1 & 0xFFFFu) + (int)(int16_t)(p1 >> 16);
+            bs[j] = ((uint32_t)b0 & 0xFFFFu) | ((uint32_t)b1 << 16);
+        }
+        for (uint32_t j = tid; j < B; j += OXH_GEMV_WAVES * 64u)
+            dq[j] = *reinterpret_cast<const float *>(a + (size_t)j * 292u);
+    }
+    __syncthreads();
+
+    const uint32_t RW = p.rows_per_wave;
+    const uint32_t row0 = (wg_in_seg * OXH_GEMV_WAVES + wave) * RW;
+    if (row0 >= seg_rows) return;
+    const uint32_t nrows = min(RW, seg_rows - row0);
+    const uint32_t nblk = nrows * B;
+    const uint32_t s = lane & 3u;
+    const bool hi = s >= 2u;
+    const uint32_t sh = (s & 1u) * 16u;
+    const uint32_t mask_a = hi ? 0x0F0F0F0Fu : 0x3F3F3F3Fu;
+    const uint32_t mask_b = hi ? 0x30303030u : 0u;
+
+    const uint8_t *wbase = segs.w[seg] + (size_t)row0 * B * 144u;
+
+    for (uint32_t g0 = 0; g0 < nblk; g0 += 16u) {
+        const uint32_t g = g0 + (lane >> 2);
+        const bool live = g < nblk;
+        const uint32_t gc = live ? g : 0u;
+        const uint32_t r = (B == 1u) ? gc : __umulhi(gc, p.magic);
+        const uint32_t blk = gc - r * B;
+        const uint8_t *wb = wbase + (size_t)gc * 144u;
+        const u32x4 hdr = *reinterpret_cast<const u32x4 *>(wb);
+        const u32x4 na = *reinterpret_cast<const u32x4 *>(wb + 16u + 32u * s);
+        const u32x4 nb = *reinterpret_cast<const u32x4 *>(wb + 32u + 32u * s);
+
+        /* 6-bit scale/min unpack for this lane's two sub-blocks */
+        const uint32_t u0 = hdr.y, u1 = hdr.z, u2 = hdr.w;
+        const uint32_t scw = ((hi ? u2 : u0) & mask_a) | ((u0 >> 2) & mask_b);
+        const uint32_t mnw = ((hi ? (u2 >> 4) : u1) & mask_a) | ((u1 >> 2) & mask_b);
+        const int sc_a = (int)((scw >> sh) & 0xFFu), sc_b = (int)((scw >> (sh + 8u)) & 0xFFu);
+        const int mn_a = (int)((mnw >> sh) & 0xFFu), mn_b = (int)((mnw >> (sh + 8u)) & 0xFFu);
+        const float dw = half_bits_to_float(hdr.x & 0xFFFFu);
+        const float dmin = half_bits_to_float(hdr.x >> 16);
+
+        const uint32_t slot = blk * 4u + s;
+        for (uint32_t v = 0; v < NV; v++) {
+            const uint8_t *base = lds + (size_t)v * act_lds;
+            const u32x4 *qv = reinterpret_cast<const u32x4 *>(base);
+            const u32x4 a0 = qv[slot], a1 = qv[B * 4u + slot];
+            const u32x4 a2 = qv[B * 8u + slot], a3 = qv[B * 12u + slot];
+            const uint32_t bsp = reinterpret_cast<const uint32_t *>(base + B * 256u)[slot];
+            const float dq = reinterpret_cast<const float *>(base + B * 256u + B * 16u)[blk];
+
+            int s_lo = 0, s_hi = 0;
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                s_lo = dot4(na[k] & 0x0F0F0F0Fu, a0[k], s_lo);
+                s_lo = dot4(nb[k] & 0x0F0F0F0Fu, a1[k], s_lo);
+                s_hi = dot4((na[k] >> 4) & 0x0F0F0F0Fu, a2[k], s_hi);
+                s_hi = dot4((nb[k] >> 4) & 0x0F0F0F0Fu, a3[k], s_hi);
+            }
+            if (DUMP) {
+                if (live) {
+                    int32_t *o = p.dump + ((size_t)(row0 * B + gc)) * 8u + 2u * s;
+                    o[0] = s_lo;
+                    o[1] = s_hi;
+                }
+            }
+            int pos = sc_a * s_lo + sc_b * s_hi;
+            int mn = mn_a * (int)(int16_t)(bsp & 0xFFFFu) + mn_b * ((int)bsp >> 16);
+            pos = quad_sum(pos);
+            mn = quad_sum(mn);
+            const float t_pos = dw * dq;
+            const float t_min = dmin * dq;
+            const float up = t_pos * (float)pos;
+            const float dn = t_min * (float)mn;
+            if (live && s == 0u)
+                terms[((size_t)v * RW + r) * p.term_stride + blk] = up - dn;
+        }
+    }
+
+    /* strictly sequential per-row sums, one lane per (vector, row) */
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    for (uint32_t idx = lane; idx < NV * nrows; idx += 64u) {
+        const uint32_t v = idx / nrows, r = idx - v * nrows;
+        const float *t = terms + ((size_t)v * RW + r) * p.term_stride;
+        float sum = 0.0f;
+        for (uint32_t b = 0; b < B; b++) sum += t[b];
+        segs.out[seg][(size_t)v * p.out_stride + row0 + r] = sum;
+    }
+}
+
+/* ─── host side of layer 2 ────────────────────────────────────────────── */
+
+static int g_device = -1;
+static hipStream_t g_stream = nullptr;
+static int g_n_cu = 0;
+
+extern "C" int oxh_init(int device)
+{
+    if (g_device >= 0) {
+        if (device == g_device) return OXH_OK;
+        return arg_fail("oxh_init: already initialised on another device");
+    }
+    int n = 0;
+    hipError_t e = hipGetDeviceCount(&n);
+    if (e != hipSuccess || n <= 0) {
+        snprintf(g_err, sizeof g_err, "no HIP device available (%s)",
+                 e == hipSuccess ? "device count is 0" : hipGetErrorString(e));
+        return OXH_ERR_NO_DEVICE;
+    }
+    if (device < 0 || device >= n) return arg_fail("oxh_init: device index out of range");
+    HIP_TRY(hipSetDevice(device));
+    hipDeviceProp_t prop;
+    HIP_TRY(hipGetDeviceProperties(&prop, device));
+    g_n_cu = prop.multiProcessorCount;
+    HIP_TRY(hipStreamCreateWithFlags(&g_stream, hipStreamNonBlocking));
+    g_device = device;
+    return OXH_OK;
+}
+
+extern "C" void oxh_shutdown(void)
+{
+    if (g_device < 0) return;
+    if (g_stream) (void)hipStreamDestroy(g_stream);
+    g_stream = nullptr;
+    g_device = -1;
+}
+
+static int ensure_init(void)
+{
+    if (g_device >= 0) return OXH_OK;
+    return oxh_init(0);
+}
+
+static hipStream_t pick_stream(void *stream)
+{
+    return stream ? (hipStream_t)stream : g_stream;
+}
+
+extern "C" void *oxh_internal_stream(void) { return (void *)g_stream; }
+
+extern "C" int oxh_act_kind(uint32_t qtype, size_t cols)
+{
+    switch (qtype) {
+    case OXH_Q8_0:   return (cols % OXH_QK8_0 == 0) ? 1 : 0;
+    case OXH_Q4_K_S:
+    case OXH_Q4_K_M:
+    case OXH_Q6_K:   return (cols % OXH_QK_K == 0) ? 2 : 0;
+    default:         return 0;
+    }
+}
+
+static size_t block_bytes(uint32_t qtype)
+{
+    switch (qtype) {
+    case OXH_Q8_0:   return OXH_Q8_0_BYTES;
+    case OXH_Q4_K_S:
+    case OXH_Q4_K_M: return OXH_Q4_K_BYTES;
+    case OXH_Q6_K:   return OXH_Q6_K_BYTES;
+    default:         return 0;
+    }
+}
+
+extern "C" size_t oxh_row_bytes(uint32_t qtype, size_t cols)
+{
+    const int kind = oxh_act_kind(qtype, cols);
+    if (!kind) return 0;
+    const size_t nb = kind == 2 ? cols / OXH_QK_K : cols / OXH_QK8_0;
+    const size_t bb = block_bytes(qtype);
+    if (nb != 0 && bb > SIZE_MAX / nb) return 0;
+    return nb * bb;
+}
+
+extern "C" size_t oxh_act_bytes(uint32_t qtype, size_t cols)
+{
+    const int kind = oxh_act_kind(qtype, cols);
+    if (!kind) return 0;
+    return kind == 2 ? cols / OXH_QK_K * OXH_Q8_K_BYTES : cols / OXH_QK8_0 * OXH_Q8_0_BYTES;
+}
+
+extern "C" int oxh_quantize_q8_k(const float *d_x, size_t in_stride, size_t n_vec,
+                                 size_t cols, void *d_act, void *stream)
+{
+    int rc = ensure_init();
+    if (rc) return rc;
+    if (n_vec == 0 || cols == 0) return OXH_OK;
+    if (!d_x || !d_act) return arg_fail("oxh_quantize_q8_k: NULL pointer");
+    if (cols % OXH_QK_K) return arg_fail("oxh_quantize_q8_k: cols not a multiple of 256");
+    if (in_stride < cols) return arg_fail("oxh_quantize_q8_k: in_stride < cols");
+    const size_t bpv = cols / OXH_QK_K;
+    if (bpv > 0xFFFFFFFFull / n_vec) return arg_fail("oxh_quantize_q8_k: too many blocks");
+    const uint32_t total = (uint32_t)(bpv * n_vec);
+    hipLaunchKernelGGL(k_quantize_q8_k, dim3((total + 3u) / 4u), dim3(256), 0,
+                       pick_stream(stream), d_x, in_stride, (uint32_t)bpv, total,
+                       (uint8_t *)d_act);
+    HIP_TRY(hipGetLastError());
+    return OXH_OK;
+}
+
+extern "C" int oxh_quantize_q8_0(const float *d_x, size_t in_stride, size_t n_vec,
+                                 size_t cols, void *d_act, void *stream)
+{
+    int rc = ensure_init();
+    if (rc) return rc;
+    if (n_vec == 0 || cols == 0) return OXH_OK;
+    if (!d_x || !d_act) return arg_fail("oxh_quantize_q8_0: NULL pointer");
+    if (cols % OXH_QK8_0) return arg_fail("oxh_quantize_q8_0: cols not a multiple of 32");
+    if (in_stride < cols) return arg_fail("oxh_quantize_q8_0: in_stride < cols");
+    const size_t bpv = cols / OXH_QK8_0;
+    const size_t spans = (bpv + 7u) / 8u;
+    if (spans > 0xFFFFFFFFull / n_vec || n_vec > 0xFFFFFFFFull)
+        return arg_fail("oxh_quantize_q8_0: too many blocks");
+    const uint32_t total = (uint32_t)(spans * n_vec);
+    hipLaunchKernelGGL(k_quantize_q8_0, dim3((total + 3u) / 4u), dim3(256), 0,
+                       pick_stream(stream), d_x, in_stride, (uint32_t)bpv,
+                       (uint32_t)n_vec, (uint8_t *)d_act);
+    HIP_TRY(hipGetLastError());
+    return OXH_OK;
+}
+
+/* Rows each wave takes: large enough to amortise the per-row tail, small
+ * enough that the launch still has several waves per SIMD on every CU. */
+static uint32_t choose_rows_per_wave(size_t total_rows, uint32_t blocks, uint32_t lanes_per_block)
+{
+    const size_t target_waves = (size_t)(g_n_cu > 0 ? g_n_cu : 256) * 16u;
+    size_t rw = total_rows / target_waves;
+    if (rw < 1) rw = 1;
+    if (rw > 16) rw = 16;
+    /* whole passes when possible: rw*blocks a multiple of blocks-per-pass */
+    const uint32_t per_pass = 64u / lanes_per_block;
+    while (rw > 1 && ((rw * blocks) % per_pass) != 0) rw--;
+    return (uint32_t)rw;
+}
+
+static size_t gemv_lds_bytes(uint32_t blocks, size_t n_vec, uint32_t rows_per_wave)
+{
+    return n_vec * (size_t)q8k_lds_bytes(blocks) +
+           (size_t)OXH_GEMV_WAVES * n_vec * rows_per_wave * (blocks + 1u) * 4u;
+}
+
+extern "C" size_t oxh_gemv_max_nvec(uint32_t qtype, size_t cols)
+{
+    if (oxh_act_kind(qtype, cols) != 2) return 0;
+    const size_t blocks = cols / OXH_QK_K;
+    if (blocks > 0xFFFFu) return 0;
+    size_t nv = OXH_MAX_NV;
+    while (nv > 0 && gemv_lds_bytes((uint32_t)blocks, nv, 1) > 65536u) nv--;
+    return nv;
+}
+
+static int launch_gemv(uint32_t qtype, const OxhSegment *segs, size_t n_segs, size_t cols,
+                       const void *d_acts, size_t n_vec, size_t out_stride, int32_t *dump,
+                       void *stream)
+{
+    int rc = ensure_init();
+    if (rc) return rc;
+    if (n_segs == 0) return OXH_OK;
+    if (!segs || !d_acts) return arg_fail("gemv: NULL pointer");
+    if (n_vec < 1 || n_vec > OXH_MAX_NV) return arg_fail("gemv: n_vec must be 1..8");
+    if (n_segs > OXH_MAX_SEGS) return arg_fail("gemv: more than 32 segments in one launch");
+    const int kind = oxh_act_kind(qtype, cols);
+    if (!kind) {
+        snprintf(g_err, sizeof g_err, "gemv: qtype %u with cols %zu has no integer path", qtype, cols);
+        return OXH_DECLINED;
+    }
+    if (qtype != OXH_Q4_K_S && qtype != OXH_Q4_K_M) {
+        snprintf(g_err, sizeof g_err, "gemv: qtype %u kernel not built yet", qtype);
+        return OXH_ERR_ARG;
+    }
+    const size_t blocks = cols / OXH_QK_K;
+    size_t total_rows = 0, max_act = 0;
+    for (size_t i = 0; i < n_segs; i++) {
+        if (segs[i].rows > 0xFFFFFFFFull / (blocks * 8u)) return arg_fail("gemv: segment too large");
+        if (segs[i].rows && (!segs[i].d_w || !segs[i].d_out)) return arg_fail("gemv: NULL segment pointer");
+        total_rows += segs[i].rows;
+        if (segs[i].act_first > max_act) max_act = segs[i].act_first;
+    }
+    if (total_rows == 0) return OXH_OK;
+    if (out_stride > 0xFFFFFFFFull || max_act + n_vec > 0xFFFFFFFFull) return arg_fail("gemv: stride too large");
+
+    GemvParams p;
+    p.blocks = (uint32_t)blocks;
+    p.magic = (uint32_t)((0x100000000ull + blocks - 1u) / blocks);
+    p.rows_per_wave = choose_rows_per_wave(total_rows, p.blocks, 4);
+    p.n_vec = (uint32_t)n_vec;
+    p.act_bytes = (uint32_t)(blocks * OXH_Q8_K_BYTES);
+    p.out_stride = (uint32_t)out_stride;
+    p.term_stride = p.blocks + 1u;
+    p.dump = dump;
+
+    size_t lds = gemv_lds_bytes(p.blocks, n_vec, p.rows_per_wave);
+    while (lds > 65536u && p.rows_per_wave > 1) {
+        p.rows_per_wave--;
+        lds = gemv_lds_bytes(p.blocks, n_vec, p.rows_per_wave);
+    }
+    if (lds > 65536u) {
+        snprintf(g_err, sizeof g_err, "gemv: cols %zu x n_vec %zu needs %zu B of LDS (max 65536)",
+                 cols, n_vec, lds);
+        return OXH_ERR_TOO_WIDE;
+    }
+
+    SegTable t;
+    memset(&t, 0, sizeof t);
+    uint32_t wg = 0;
+    uint32_t n = 0;
+    const uint32_t rows_per_wg = p.rows_per_wave * OXH_GEMV_WAVES;
+    for (size_t i = 0; i < n_segs; i++) {
+        if (segs[i].rows == 0) continue;
+        t.w[n] = (const uint8_t *)segs[i].d_w;
+        t.out[n] = segs[i].d_out;
+        t.rows[n] = (uint32_t)segs[i].rows;
+        t.act_first[n] = (uint32_t)segs[i].act_first;
+        t.wg_begin[n] = wg;
+        wg += (uint32_t)((segs[i].rows + rows_per_wg - 1u) / rows_per_wg);
+        n++;
+    }
+    t.wg_begin[n] = wg;
+    t.n = n;
+
+    if (dump)
+        hipLaunchKernelGGL(k_gemv_q4_k<true>, dim3(wg), dim3(OXH_GEMV_WAVES * 64), lds,
+                           pick_stream(stream), t, p, (const uint8_t *)d_acts);
+    else
+        hipLaunchKernelGGL(k_gemv_q4_k<false>, dim3(wg), dim3(OXH_GEMV_WAVES * 64), lds,
+                           pick_stream(stream), t, p, (const uint8_t *)d_acts);
+    HIP_TRY(hipGetLastError());
+    return OXH_OK;
+}
+
+extern "C" int oxh_gemv_segments(uint32_t qtype, const OxhSegment *segs, size_t n_segs,
+                                 size_t cols, const void *d_acts, size_t n_vec,
+                                 size_t out_stride, void *stream)
+{
+    return launch_gemv(qtype, segs, n_segs, cols, d_acts, n_vec, out_stride, nullptr, stream);
+}
+
+extern "C" int oxh_debug_subblock_sums(uint32_t qtype, const void *d_w, size_t rows,
+                                       size_t cols, const void *d_act, int32_t *d_sums,
+                                       void *stream)
+{
+    if (!d_sums) return arg_fail("oxh_debug_subblock_sums: NULL output");
+    int rc = ensure_init();
+    if (rc) return rc;
+    float *scratch = nullptr;
+    HIP_TRY(hipMalloc((void **)&scratch, (rows ? rows : 1) * sizeof(float)));
+    OxhSegment s = { d_w, scratch, rows, 0 };
+    rc = launch_gemv(qtype, &s, 1, cols, d_act, 1, rows, d_sums, stream);
+    hipError_t e = hipStreamSynchronize(pick_stream(stream));
+    (void)hipFree(scratch);
+    if (rc) return rc;
+    if (e != hipSuccess) return hip_fail(e, "hipStreamSynchronize");
+    return OXH_OK;
+}
+
+extern "C" int oxh_mmq(uint32_t, const void *, size_t, size_t, const void *, size_t,
+                       float *, size_t, void *)
+{
+    snprintf(g_err, sizeof g_err, "oxh_mmq: not built yet");
+    return OXH_ERR_ARG;
+}
+
+/* ─── memory / stream / event plumbing ────────────────────────────────── */
+
+extern "C" int oxh_malloc(void **d_ptr, size_t bytes)
+{
+    int rc = ensure_init();
+    if (rc) return rc;
+    if (!d_ptr) return arg_fail("oxh_malloc: NULL");
+    hipError_t e = hipMalloc(d_ptr, bytes ? bytes : 1);
+    if (e == hipErrorOutOfMemory) {
+        snprintf(g_err, sizeof g_err, "out of device memory allocating %zu bytes", bytes);
+        (void)hipGetLastError();
+        return OXH_ERR_NOMEM;
+    }
+    if (e != hipSuccess) return hip_fail(e, "hipMalloc");
+    return OXH_OK;
+}
+
+extern "C" int oxh_free(void *d_ptr)
+{
+    if (!d_ptr) return OXH_OK;
+    HIP_TRY(hipFree(d_ptr));
+    return OXH_OK;
+}
+
+extern "C" int oxh_memcpy_h2d(void *d_dst, const void *h_src, size_t bytes, void *stream)
+{
+    int rc = ensure_init();
+    if (rc) return rc;
+    if (bytes == 0) return OXH_OK;
+    HIP_TRY(hipMemcpyAsync(d_dst, h_src, bytes, hipMemcpyHostToDevice, pick_stream(stream)));
+    return OXH_OK;
+}
+
+extern "C" int oxh_memcpy_d2h(void *h_dst, const void *d_src, size_t bytes, void *stream)
+{
+    int rc = ensure_init();
+    if (rc) return rc;
+    if (bytes == 0) return OXH_OK;
+    HIP_TRY(hipMemcpyAsync(h_dst, d_src, bytes, hipMemcpyDeviceToHost, pick_stream(stream)));
+    return OXH_OK;
+}
+
+extern "C" int oxh_memset(void *d_dst, int value, size_t bytes, void *stream)
+{
+    int rc = ensure_init();
+    if (rc) return rc;
+    if (bytes == 0) return OXH_OK;
+    HIP_TRY(hipMemsetAsync(d_dst, value, bytes, pick_stream(stream)));
+    return OXH_OK;
+}
+
+extern "C" int oxh_stream_create(void **stream)
+{
+    int rc = ensure_init();
+    if (rc) return rc;
+    hipStream_t s;
+    HIP_TRY(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));
+    *stream = (void *)s;
+    return OXH_OK;
+}
+
+extern "C" int oxh_stream_destroy(void *stream)
+{
+    if (stream) HIP_TRY(hipStreamDestroy((hipStream_t)stream));
+    return OXH_OK;
+}
+
+extern "C" int oxh_stream_sync(void *stream)
+{
+    int rc = ensure_init();
+    if (rc) return rc;
+    HIP_TRY(hipStreamSynchronize(pick_stream(stream)));
+    return OXH_OK;
+}
+
+extern "C" int oxh_event_create(void **event)
+{
+    int rc = ensure_init();
+    if (rc) return rc;
+    hipEvent_t e;
+    HIP_TRY(hipEventCreate(&e));
+    *event = (void *)e;
+    return OXH_OK;
+}
+
+extern "C" int oxh_event_destroy(void *event)
+{
+    if (event) HIP_TRY(hipEventDestroy((hipEvent_t)event));
+    return OXH_OK;
+}
+
+extern "C" int oxh_event_record(void *event, void *stream)
+{
+    HIP_TRY(hipEventRecord((hipEvent_t)event, pick_stream(stream)));
+    return OXH_OK;
+}
+
+extern "C" int oxh_event_sync(void *event)
+{
+    HIP_TRY(hipEventSynchronize((hipEvent_t)event));
+    return OXH_OK;
+}
+
+extern "C" int oxh_event_elapsed_ms(void *start, void *stop, float *ms)
+{
+    HIP_TRY(hipEventElapsedTime(ms, (hipEvent_t)start, (hipEvent_t)stop));
+    return OXH_OK;
+}
+
+extern "C" int oxh_device_info(char *name, size_t name_len, int *n_cu, int *clock_mhz,
+                               size_t *mem_bytes)
+{
+    int rc = ensure_init();
+    if (rc) return rc;
+    hipDeviceProp_t prop;
+    HIP_TRY(hipGetDeviceProperties(&prop, g_device));
+    if (name && name_len) {
+        strncpy(name, prop.name, name_len - 1);
+        name[name_len - 1] = 0;
+    }
+    if (n_cu) *n_cu = prop.multiProcessorCount;
+    if (clock_mhz) *clock_mhz = prop.clockRate / 1000;
+    if (mem_bytes) *mem_bytes = prop.totalGlobalMem;
+    return OXH_OK;
+}

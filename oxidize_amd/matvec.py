@@ -1,0 +1,163 @@
+"""Host-side mirror of the reference's quantized-matvec interface over numpy
+arrays, calling straight into liboxhip's C ABI.
+
+Names and argument meaning follow oxidize-c/include/oxidize/matvec.h:
+``matvec_quantized``, ``matvec_quantized_fused``,
+``matvec_quantized_multi_input``, ``matvec_quantized_batch``.  Each returns the
+library status (0 handled, 1 declined) and raises :class:`OxhError` on errors.
+The ``Device*`` helpers wrap the device-resident layer for benchmarks.
+"""
+import ctypes
+
+import numpy as np
+
+from . import _lib
+from ._lib import DECLINED, OK, OxhError, OxhSegment, check, lib
+
+Q8_0, Q4_K_S, Q4_K_M, Q6_K = 7, 12, 13, 16
+
+
+def _p(a):
+    return None if a is None else ctypes.c_void_p(a.ctypes.data)
+
+
+def _status(rc):
+    if rc in (OK, DECLINED):
+        return rc
+    return check(rc)
+
+
+def _ptrs(arrays):
+    return (ctypes.c_void_p * len(arrays))(*[a.ctypes.data for a in arrays])
+
+
+def _sizes(values):
+    return (ctypes.c_size_t * len(values))(*[int(v) for v in values])
+
+
+def _u32s(values):
+    return (ctypes.c_uint32 * len(values))(*[int(v) for v in values])
+
+
+def matvec_quantized(qtype, data, rows, cols, row_bytes, x, out, temp):
+    """out[r] = dot(W[r], Q8(x)); `temp` receives the quantised activation."""
+    return _status(lib().oxh_matvec_quantized(qtype, _p(data), rows, cols, row_bytes,
+                                              _p(x), _p(out), _p(temp)))
+
+
+def matvec_quantized_fused(qtypes, datas, rows, cols, row_bytes, x, outs, temp):
+    n = len(datas)
+    return _status(lib().oxh_matvec_quantized_fused(
+        _u32s(qtypes), _ptrs(datas), _sizes(rows), cols, _sizes(row_bytes), n, _p(x),
+        _ptrs(outs), _p(temp)))
+
+
+def matvec_quantized_multi_input(qtypes, datas, rows, cols, row_bytes, xs, outs, temp):
+    n = len(datas)
+    return _status(lib().oxh_matvec_quantized_multi_input(
+        _u32s(qtypes), _ptrs(datas), _sizes(rows), cols, _sizes(row_bytes), n, _ptrs(xs),
+        _ptrs(outs), _p(temp)))
+
+
+def matvec_quantized_batch(qtype, data, rows, cols, row_bytes, xs, in_stride, outs,
+                           out_stride, n_vec, temp, act_scratch):
+    nbytes = 0 if act_scratch is None else act_scratch.nbytes
+    return _status(lib().oxh_matvec_quantized_batch(
+        qtype, _p(data), rows, cols, row_bytes, _p(xs), in_stride, _p(outs), out_stride,
+        n_vec, _p(temp), _p(act_scratch), nbytes))
+
+
+def batch_scratch_bytes(max_cols):
+    return lib().oc_matvec_batch_scratch_bytes(max_cols)
+
+
+# ─── device-resident layer ──────────────────────────────────────────────
+
+
+class DeviceBuffer:
+    """A hipMalloc'd range owned by this object."""
+
+    def __init__(self, nbytes):
+        self.nbytes = int(nbytes)
+        ptr = ctypes.c_void_p()
+        check(lib().oxh_malloc(ctypes.byref(ptr), self.nbytes))
+        self.ptr = ptr.value
+
+    @classmethod
+    def from_host(cls, array):
+        array = np.ascontiguousarray(array)
+        buf = cls(array.nbytes)
+        buf.upload(array)
+        return buf
+
+    def upload(self, array, offset=0):
+        array = np.ascontiguousarray(array)
+        assert offset + array.nbytes <= self.nbytes
+        check(lib().oxh_memcpy_h2d(ctypes.c_void_p(self.ptr + offset), _p(array),
+                                   array.nbytes, None))
+        check(lib().oxh_stream_sync(None))
+
+    def download(self, dtype, count, offset=0):
+        out = np.empty(count, dtype=dtype)
+        assert offset + out.nbytes <= self.nbytes
+        check(lib().oxh_memcpy_d2h(_p(out), ctypes.c_void_p(self.ptr + offset), out.nbytes, None))
+        check(lib().oxh_stream_sync(None))
+        return out
+
+    def free(self):
+        if self.ptr:
+            lib().oxh_stream_sync(None)
+            lib().oxh_free(ctypes.c_void_p(self.ptr))
+            self.ptr = 0
+
+    def __del__(self):
+        try:
+            self.free()
+        except Exception:
+            pass
+
+
+def act_bytes(qtype, cols):
+    return lib().oxh_act_bytes(qtype, cols)
+
+
+def quantize(qtype, d_x, in_stride, n_vec, cols, d_act, stream=None):
+    kind = lib().oxh_act_kind(qtype, cols)
+    fn = lib().oxh_quantize_q8_k if kind == 2 else lib().oxh_quantize_q8_0
+    check(fn(ctypes.c_void_p(d_x), in_stride, n_vec, cols, ctypes.c_void_p(d_act), stream))
+
+
+def make_segments(items):
+    """items: iterable of (d_w, d_out, rows, act_first) with integer addresses."""
+    items = list(items)
+    segs = (OxhSegment * len(items))()
+    for s, (w, o, r, a) in zip(segs, items):
+        s.d_w, s.d_out, s.rows, s.act_first = w, o, r, a
+    return segs
+
+
+def gemv_segments(qtype, segs, cols, d_acts, n_vec=1, out_stride=0, stream=None):
+    check(lib().oxh_gemv_segments(qtype, segs, len(segs), cols, ctypes.c_void_p(d_acts),
+                                  n_vec, out_stride, stream))
+
+
+def mmq(qtype, d_w, rows, cols, d_acts, n_vec, d_out, out_stride, stream=None):
+    check(lib().oxh_mmq(qtype, ctypes.c_void_p(d_w), rows, cols, ctypes.c_void_p(d_acts),
+                        n_vec, ctypes.c_void_p(d_out), out_stride, stream))
+
+
+def debug_subblock_sums(qtype, d_w, rows, cols, d_act, d_sums, stream=None):
+    check(lib().oxh_debug_subblock_sums(qtype, ctypes.c_void_p(d_w), rows, cols,
+                                        ctypes.c_void_p(d_act), ctypes.c_void_p(d_sums), stream))
+
+
+def sync(stream=None):
+    check(lib().oxh_stream_sync(stream))
+
+
+def device_info():
+    name = ctypes.create_string_buffer(256)
+    n_cu, mhz, mem = ctypes.c_int(), ctypes.c_int(), ctypes.c_size_t()
+    check(lib().oxh_device_info(name, 256, ctypes.byref(n_cu), ctypes.byref(mhz), ctypes.byref(mem)))
+    return {"name": name.value.decode(), "n_cu": n_cu.value, "clock_mhz": mhz.value,
+            "mem_bytes": mem.value}
