@@ -229,6 +229,18 @@ __host__ __device__ static inline uint32_t q8k_lds_bytes(uint32_t blocks)
     return (blocks * (256u + 16u + 4u) + 15u) & ~15u;
 }
 
+/* Q6_K pairing: 256 B of values, 16 x int32 pre-scaled group sums, scale. */
+__host__ __device__ static inline uint32_t q8k6_lds_bytes(uint32_t blocks)
+{
+    return (blocks * (256u + 64u + 4u) + 15u) & ~15u;
+}
+
+/* Q8_0 activation: 32 B of values and the decoded f32 scale per block. */
+__host__ __device__ static inline uint32_t q80_lds_bytes(uint32_t blocks)
+{
+    return (blocks * (32u + 4u) + 15u) & ~15u;
+}
+
 struct SegTable {
     const uint8_t *w[OXH_MAX_SEGS];
     float *out[OXH_MAX_SEGS];
@@ -264,6 +276,10 @@ __device__ __forceinline__ uint32_t find_segment(const SegTable &t, uint32_t wg)
     while (s + 1 < t.n && wg >= t.wg_begin[s + 1]) s++;
     return s;
 }
+
+__device__ __forceinline__ void
+row_sums(const float *terms, uint32_t lane, uint32_t NV, uint32_t nrows, uint32_t RW,
+         uint32_t B, uint32_t term_stride, float *out, uint32_t out_stride, uint32_t row0);
 
 /* Q4_K x Q8_K.  Four lanes per super-block: lane (b, s) owns nibble bytes
  * [32s, 32s+32) of block b, i.e. sub-blocks 2s (low nibbles) and 2s+1 (high
@@ -384,15 +400,220 @@ k_gemv_q4_k(const SegTable segs, const GemvParams p, const uint8_t *__restrict__
         }
     }
 
-    /* strictly sequential per-row sums, one lane per (vector, row) */
+    row_sums(terms, lane, NV, nrows, RW, B, p.term_stride, segs.out[seg], p.out_stride, row0);
+}
+
+/* Shared tail: strictly sequential per-row sums, one lane per (vector, row). */
+__device__ __forceinline__ void
+row_sums(const float *terms, uint32_t lane, uint32_t NV, uint32_t nrows, uint32_t RW,
+         uint32_t B, uint32_t term_stride, float *out, uint32_t out_stride, uint32_t row0)
+{
     __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
     for (uint32_t idx = lane; idx < NV * nrows; idx += 64u) {
         const uint32_t v = idx / nrows, r = idx - v * nrows;
-        const float *t = terms + ((size_t)v * RW + r) * p.term_stride;
+        const float *t = terms + ((size_t)v * RW + r) * term_stride;
         float sum = 0.0f;
         for (uint32_t b = 0; b < B; b++) sum += t[b];
-        segs.out[seg][(size_t)v * p.out_stride + row0 + r] = sum;
+        out[(size_t)v * out_stride + row0 + r] = sum;
     }
+}
+
+/* Q6_K x Q8_K.  Four lanes per super-block: lane (b, u) with u = 2n + lh owns
+ * the 64 weights e = 128n + 32k + 16lh + i (k < 4, i < 16): 16 bytes of ql at
+ * 64n+16lh (low nibbles -> k=0, high -> k=2), 16 bytes at 64n+32+16lh (k=1,
+ * k=3) and 16 bytes of qh at 32n+16lh (two bits per k).  Each k is one
+ * 16-weight scale group g = 8n + 2k + lh.  Blocks are 210 bytes, so every
+ * load here is only 2-byte aligned. */
+template <bool DUMP>
+__global__ __launch_bounds__(OXH_GEMV_WAVES * 64) void
+k_gemv_q6_k(const SegTable segs, const GemvParams p, const uint8_t *__restrict__ acts)
+{
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    const uint32_t tid = threadIdx.x;
+    const uint32_t lane = tid & 63u;
+    const uint32_t wave = tid >> 6;
+    const uint32_t B = p.blocks;
+    const uint32_t NV = p.n_vec;
+
+    const uint32_t seg = find_segment(segs, blockIdx.x);
+    const uint32_t wg_in_seg = blockIdx.x - segs.wg_begin[seg];
+    const uint32_t seg_rows = segs.rows[seg];
+
+    const uint32_t act_lds = q8k6_lds_bytes(B);
+    float *const terms = reinterpret_cast<float *>(lds + (size_t)act_lds * NV) +
+                         (size_t)wave * NV * p.rows_per_wave * p.term_stride;
+
+    for (uint32_t v = 0; v < NV; v++) {
+        const uint8_t *a = acts + (size_t)(segs.act_first[seg] + v) * p.act_bytes;
+        uint8_t *base = lds + (size_t)v * act_lds;
+        uint32_t *qd = reinterpret_cast<uint32_t *>(base);
+        int32_t *bs = reinterpret_cast<int32_t *>(base + B * 256u);
+        float *dq = reinterpret_cast<float *>(base + B * 256u + B * 64u);
+        for (uint32_t j = tid; j < B * 64u; j += OXH_GEMV_WAVES * 64u) {
+            const uint32_t blk = j >> 6, w = j & 63u;
+            const uint32_t e = 4u * w;
+            const uint32_t n = e >> 7, k = (e >> 5) & 3u, lh = (e >> 4) & 1u;
+            const uint32_t val = *reinterpret_cast<const uint32_t *>(a + (size_t)blk * 292u + 4u + 4u * w);
+            qd[((k * B * 4u) + blk * 4u + 2u * n + lh) * 4u + (w & 3u)] = val;
+        }
+        for (uint32_t j = tid; j < B * 16u; j += OXH_GEMV_WAVES * 64u) {
+            const uint32_t blk = j >> 4, g = j & 15u;
+            const uint32_t n = g >> 3, k = (g >> 1) & 3u, lh = g & 1u;
+            const int16_t sum = *reinterpret_cast<const int16_t *>(a + (size_t)blk * 292u + 260u + 2u * g);
+            bs[(blk * 4u + 2u * n + lh) * 4u + k] = 32 * (int32_t)sum;
+        }
+        for (uint32_t j = tid; j < B; j += OXH_GEMV_WAVES * 64u)
+            dq[j] = *reinterpret_cast<const float *>(a + (size_t)j * 292u);
+    }
+    __syncthreads();
+
+    const uint32_t RW = p.rows_per_wave;
+    const uint32_t row0 = (wg_in_seg * OXH_GEMV_WAVES + wave) * RW;
+    if (row0 >= seg_rows) return;
+    const uint32_t nrows = min(RW, seg_rows - row0);
+    const uint32_t nblk = nrows * B;
+    const uint32_t u = lane & 3u;
+    const uint32_t n = u >> 1, lh = u & 1u;
+    const uint8_t *wbase = segs.w[seg] + (size_t)row0 * B * 210u;
+
+    for (uint32_t g0 = 0; g0 < nblk; g0 += 16u) {
+        const uint32_t g = g0 + (lane >> 2);
+        const bool live = g < nblk;
+        const uint32_t gc = live ? g : 0u;
+        const uint32_t r = (B == 1u) ? gc : __umulhi(gc, p.magic);
+        const uint32_t blk = gc - r * B;
+        const uint8_t *wb = wbase + (size_t)gc * 210u;
+        const U32x4u2 la = *reinterpret_cast<const U32x4u2 *>(wb + 64u * n + 16u * lh);
+        const U32x4u2 lb = *reinterpret_cast<const U32x4u2 *>(wb + 64u * n + 32u + 16u * lh);
+        const U32x4u2 hh = *reinterpret_cast<const U32x4u2 *>(wb + 128u + 32u * n + 16u * lh);
+        const uint32_t sc_lo = reinterpret_cast<const U32u2 *>(wb + 192u + 8u * n)->v;
+        const uint32_t sc_hi = reinterpret_cast<const U32u2 *>(wb + 196u + 8u * n)->v;
+        const uint32_t dbits = *reinterpret_cast<const uint16_t *>(wb + 208u);
+        /* scale bytes lh, lh+2 (low word) and lh+4, lh+6 (high word) */
+        const int sc0 = (int)(int8_t)(sc_lo >> (8u * lh));
+        const int sc1 = (int)(int8_t)(sc_lo >> (8u * lh + 16u));
+        const int sc2 = (int)(int8_t)(sc_hi >> (8u * lh));
+        const int sc3 = (int)(int8_t)(sc_hi >> (8u * lh + 16u));
+        const float dw = half_bits_to_float(dbits);
+        const uint32_t qa[4] = { la.x, la.y, la.z, la.w };
+        const uint32_t qb[4] = { lb.x, lb.y, lb.z, lb.w };
+        const uint32_t qh[4] = { hh.x, hh.y, hh.z, hh.w };
+
+        const uint32_t slot = blk * 4u + u;
+        for (uint32_t v = 0; v < NV; v++) {
+            const uint8_t *base = lds + (size_t)v * act_lds;
+            const u32x4 *qv = reinterpret_cast<const u32x4 *>(base);
+            const u32x4 a0 = qv[slot], a1 = qv[B * 4u + slot];
+            const u32x4 a2 = qv[B * 8u + slot], a3 = qv[B * 12u + slot];
+            const u32x4 off = reinterpret_cast<const u32x4 *>(base + B * 256u)[slot];
+            const float dq = reinterpret_cast<const float *>(base + B * 256u + B * 64u)[blk];
+
+            int g0s = 0, g1s = 0, g2s = 0, g3s = 0;
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const uint32_t c0 = (qa[i] & 0x0F0F0F0Fu) | ((qh[i] << 4) & 0x30303030u);
+                const uint32_t c1 = (qb[i] & 0x0F0F0F0Fu) | ((qh[i] << 2) & 0x30303030u);
+                const uint32_t c2 = ((qa[i] >> 4) & 0x0F0F0F0Fu) | (qh[i] & 0x30303030u);
+                const uint32_t c3 = ((qb[i] >> 4) & 0x0F0F0F0Fu) | ((qh[i] >> 2) & 0x30303030u);
+                g0s = dot4(c0, a0[i], g0s);
+                g1s = dot4(c1, a1[i], g1s);
+                g2s = dot4(c2, a2[i], g2s);
+                g3s = dot4(c3, a3[i], g3s);
+            }
+            if (DUMP) {
+                if (live) {
+                    int32_t *o = p.dump + ((size_t)(row0 * B + gc)) * 16u + 8u * n + lh;
+                    o[0] = g0s; o[2] = g1s; o[4] = g2s; o[6] = g3s;
+                }
+            }
+            /* sum_g sc_g * (G_g - 32*bsum_g) == pos - 32*minc, in integers */
+            int tot = sc0 * (g0s - (int)off[0]) + sc1 * (g1s - (int)off[1]) +
+                      sc2 * (g2s - (int)off[2]) + sc3 * (g3s - (int)off[3]);
+            tot = quad_sum(tot);
+            const float t = dw * dq;
+            if (live && u == 0u)
+                terms[((size_t)v * RW + r) * p.term_stride + blk] = t * (float)tot;
+        }
+    }
+    row_sums(terms, lane, NV, nrows, RW, B, p.term_stride, segs.out[seg], p.out_stride, row0);
+}
+
+/* Q8_0 x Q8_0.  One lane per 34-byte block, 64 blocks (2176 contiguous bytes)
+ * per wave pass.  The per-block integer dot is exact; the f32 result is the
+ * block-sequential chain of oxk.c:224-241 (the reference's x86 decode path
+ * accumulates the same terms in a different order, so f32 outputs agree with
+ * it to tolerance, not to the bit). */
+template <bool DUMP>
+__global__ __launch_bounds__(OXH_GEMV_WAVES * 64) void
+k_gemv_q8_0(const SegTable segs, const GemvParams p, const uint8_t *__restrict__ acts)
+{
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    const uint32_t tid = threadIdx.x;
+    const uint32_t lane = tid & 63u;
+    const uint32_t wave = tid >> 6;
+    const uint32_t B = p.blocks;
+    const uint32_t NV = p.n_vec;
+
+    const uint32_t seg = find_segment(segs, blockIdx.x);
+    const uint32_t wg_in_seg = blockIdx.x - segs.wg_begin[seg];
+    const uint32_t seg_rows = segs.rows[seg];
+
+    const uint32_t act_lds = q80_lds_bytes(B);
+    float *const terms = reinterpret_cast<float *>(lds + (size_t)act_lds * NV) +
+                         (size_t)wave * NV * p.rows_per_wave * p.term_stride;
+
+    for (uint32_t v = 0; v < NV; v++) {
+        const uint8_t *a = acts + (size_t)(segs.act_first[seg] + v) * p.act_bytes;
+        uint8_t *base = lds + (size_t)v * act_lds;
+        uint32_t *qd = reinterpret_cast<uint32_t *>(base);
+        float *dq = reinterpret_cast<float *>(base + B * 32u);
+        for (uint32_t j = tid; j < B * 8u; j += OXH_GEMV_WAVES * 64u) {
+            const uint32_t blk = j >> 3, w = j & 7u;
+            const uint32_t val = reinterpret_cast<const U32u2 *>(a + (size_t)blk * 34u + 2u + 4u * w)->v;
+            qd[(((w >> 2) * B) + blk) * 4u + (w & 3u)] = val;
+        }
+        for (uint32_t j = tid; j < B; j += OXH_GEMV_WAVES * 64u)
+            dq[j] = half_bits_to_float(*reinterpret_cast<const uint16_t *>(a + (size_t)j * 34u));
+    }
+    __syncthreads();
+
+    const uint32_t RW = p.rows_per_wave;
+    const uint32_t row0 = (wg_in_seg * OXH_GEMV_WAVES + wave) * RW;
+    if (row0 >= seg_rows) return;
+    const uint32_t nrows = min(RW, seg_rows - row0);
+    const uint32_t nblk = nrows * B;
+    const uint8_t *wbase = segs.w[seg] + (size_t)row0 * B * 34u;
+
+    for (uint32_t g0 = 0; g0 < nblk; g0 += 64u) {
+        const uint32_t g = g0 + lane;
+        const bool live = g < nblk;
+        const uint32_t gc = live ? g : 0u;
+        const uint32_t r = (B == 1u) ? gc : __umulhi(gc, p.magic);
+        const uint32_t blk = gc - r * B;
+        const uint8_t *wb = wbase + (size_t)gc * 34u;
+        const uint32_t dbits = *reinterpret_cast<const uint16_t *>(wb);
+        const U32x4u2 w0 = *reinterpret_cast<const U32x4u2 *>(wb + 2u);
+        const U32x4u2 w1 = *reinterpret_cast<const U32x4u2 *>(wb + 18u);
+        const float dw = half_bits_to_float(dbits);
+
+        for (uint32_t v = 0; v < NV; v++) {
+            const uint8_t *base = lds + (size_t)v * act_lds;
+            const u32x4 *qv = reinterpret_cast<const u32x4 *>(base);
+            const u32x4 a0 = qv[blk], a1 = qv[B + blk];
+            const float dq = reinterpret_cast<const float *>(base + B * 32u)[blk];
+            int isum = 0;
+            isum = dot4(w0.x, a0[0], isum); isum = dot4(w0.y, a0[1], isum);
+            isum = dot4(w0.z, a0[2], isum); isum = dot4(w0.w, a0[3], isum);
+            isum = dot4(w1.x, a1[0], isum); isum = dot4(w1.y, a1[1], isum);
+            isum = dot4(w1.z, a1[2], isum); isum = dot4(w1.w, a1[3], isum);
+            if (DUMP) {
+                if (live) p.dump[(size_t)row0 * B + gc] = isum;
+            }
+            const float t = dw * dq;
+            if (live) terms[((size_t)v * RW + r) * p.term_stride + blk] = t * (float)isum;
+        }
+    }
+    row_sums(terms, lane, NV, nrows, RW, B, p.term_stride, segs.out[seg], p.out_stride, row0);
 }
 
 /* ─── host side of layer 2 ────────────────────────────────────────────── */
@@ -538,19 +759,29 @@ static uint32_t choose_rows_per_wave(size_t total_rows, uint32_t blocks, uint32_
     return (uint32_t)rw;
 }
 
-static size_t gemv_lds_bytes(uint32_t blocks, size_t n_vec, uint32_t rows_per_wave)
+static bool is_q4k(uint32_t qtype) { return qtype == OXH_Q4_K_S || qtype == OXH_Q4_K_M; }
+
+static uint32_t act_lds_bytes(uint32_t qtype, uint32_t blocks)
 {
-    return n_vec * (size_t)q8k_lds_bytes(blocks) +
+    if (qtype == OXH_Q8_0) return q80_lds_bytes(blocks);
+    if (qtype == OXH_Q6_K) return q8k6_lds_bytes(blocks);
+    return q8k_lds_bytes(blocks);
+}
+
+static size_t gemv_lds_bytes(uint32_t qtype, uint32_t blocks, size_t n_vec, uint32_t rows_per_wave)
+{
+    return n_vec * (size_t)act_lds_bytes(qtype, blocks) +
            (size_t)OXH_GEMV_WAVES * n_vec * rows_per_wave * (blocks + 1u) * 4u;
 }
 
 extern "C" size_t oxh_gemv_max_nvec(uint32_t qtype, size_t cols)
 {
-    if (oxh_act_kind(qtype, cols) != 2) return 0;
-    const size_t blocks = cols / OXH_QK_K;
+    const int kind = oxh_act_kind(qtype, cols);
+    if (!kind) return 0;
+    const size_t blocks = kind == 2 ? cols / OXH_QK_K : cols / OXH_QK8_0;
     if (blocks > 0xFFFFu) return 0;
     size_t nv = OXH_MAX_NV;
-    while (nv > 0 && gemv_lds_bytes((uint32_t)blocks, nv, 1) > 65536u) nv--;
+    while (nv > 0 && gemv_lds_bytes(qtype, (uint32_t)blocks, nv, 1) > 65536u) nv--;
     return nv;
 }
 
@@ -569,35 +800,38 @@ static int launch_gemv(uint32_t qtype, const OxhSegment *segs, size_t n_segs, si
         snprintf(g_err, sizeof g_err, "gemv: qtype %u with cols %zu has no integer path", qtype, cols);
         return OXH_DECLINED;
     }
-    if (qtype != OXH_Q4_K_S && qtype != OXH_Q4_K_M) {
-        snprintf(g_err, sizeof g_err, "gemv: qtype %u kernel not built yet", qtype);
-        return OXH_ERR_ARG;
+    const size_t blocks = kind == 2 ? cols / OXH_QK_K : cols / OXH_QK8_0;
+    const size_t bbytes = block_bytes(qtype);
+    if (blocks > 0xFFFFu) {
+        snprintf(g_err, sizeof g_err, "gemv: cols %zu too wide", cols);
+        return OXH_ERR_TOO_WIDE;
     }
-    const size_t blocks = cols / OXH_QK_K;
     size_t total_rows = 0, max_act = 0;
     for (size_t i = 0; i < n_segs; i++) {
-        if (segs[i].rows > 0xFFFFFFFFull / (blocks * 8u)) return arg_fail("gemv: segment too large");
+        if (segs[i].rows > 0x7FFFFFFFull / (blocks * 16u)) return arg_fail("gemv: segment too large");
         if (segs[i].rows && (!segs[i].d_w || !segs[i].d_out)) return arg_fail("gemv: NULL segment pointer");
         total_rows += segs[i].rows;
         if (segs[i].act_first > max_act) max_act = segs[i].act_first;
     }
     if (total_rows == 0) return OXH_OK;
     if (out_stride > 0xFFFFFFFFull || max_act + n_vec > 0xFFFFFFFFull) return arg_fail("gemv: stride too large");
+    (void)bbytes;
 
+    const uint32_t lanes_per_block = qtype == OXH_Q8_0 ? 1u : 4u;
     GemvParams p;
     p.blocks = (uint32_t)blocks;
     p.magic = (uint32_t)((0x100000000ull + blocks - 1u) / blocks);
-    p.rows_per_wave = choose_rows_per_wave(total_rows, p.blocks, 4);
+    p.rows_per_wave = choose_rows_per_wave(total_rows, p.blocks, lanes_per_block);
     p.n_vec = (uint32_t)n_vec;
-    p.act_bytes = (uint32_t)(blocks * OXH_Q8_K_BYTES);
+    p.act_bytes = (uint32_t)oxh_act_bytes(qtype, cols);
     p.out_stride = (uint32_t)out_stride;
     p.term_stride = p.blocks + 1u;
     p.dump = dump;
 
-    size_t lds = gemv_lds_bytes(p.blocks, n_vec, p.rows_per_wave);
+    size_t lds = gemv_lds_bytes(qtype, p.blocks, n_vec, p.rows_per_wave);
     while (lds > 65536u && p.rows_per_wave > 1) {
         p.rows_per_wave--;
-        lds = gemv_lds_bytes(p.blocks, n_vec, p.rows_per_wave);
+        lds = gemv_lds_bytes(qtype, p.blocks, n_vec, p.rows_per_wave);
     }
     if (lds > 65536u) {
         snprintf(g_err, sizeof g_err, "gemv: cols %zu x n_vec %zu needs %zu B of LDS (max 65536)",
@@ -623,12 +857,19 @@ static int launch_gemv(uint32_t qtype, const OxhSegment *segs, size_t n_segs, si
     t.wg_begin[n] = wg;
     t.n = n;
 
-    if (dump)
-        hipLaunchKernelGGL(k_gemv_q4_k<true>, dim3(wg), dim3(OXH_GEMV_WAVES * 64), lds,
-                           pick_stream(stream), t, p, (const uint8_t *)d_acts);
-    else
-        hipLaunchKernelGGL(k_gemv_q4_k<false>, dim3(wg), dim3(OXH_GEMV_WAVES * 64), lds,
-                           pick_stream(stream), t, p, (const uint8_t *)d_acts);
+    const dim3 grid(wg), block(OXH_GEMV_WAVES * 64);
+    hipStream_t st = pick_stream(stream);
+    const uint8_t *a = (const uint8_t *)d_acts;
+    if (is_q4k(qtype)) {
+        if (dump) hipLaunchKernelGGL(k_gemv_q4_k<true>, grid, block, lds, st, t, p, a);
+        else      hipLaunchKernelGGL(k_gemv_q4_k<false>, grid, block, lds, st, t, p, a);
+    } else if (qtype == OXH_Q6_K) {
+        if (dump) hipLaunchKernelGGL(k_gemv_q6_k<true>, grid, block, lds, st, t, p, a);
+        else      hipLaunchKernelGGL(k_gemv_q6_k<false>, grid, block, lds, st, t, p, a);
+    } else {
+        if (dump) hipLaunchKernelGGL(k_gemv_q8_0<true>, grid, block, lds, st, t, p, a);
+        else      hipLaunchKernelGGL(k_gemv_q8_0<false>, grid, block, lds, st, t, p, a);
+    }
     HIP_TRY(hipGetLastError());
     return OXH_OK;
 }

@@ -1,0 +1,257 @@
+"""GPU parity for the Q6_K and Q8_0 decode GEMVs, the Q8_0 activation
+quantiser and the grouped entry points (fused / multi-input / batch), through
+the C ABI, against the CPU oracle.
+
+Bars: activation bytes and integer sub-block sums bit-exact for every type;
+f32 outputs bit-exact for Q4_K and Q6_K; Q8_0 f32 outputs bit-exact against the
+oracle's block-sequential chain and within |a-b| <= 1e-4 + 1e-5*|ref| of the
+compiled reference (whose x86 decode kernel sums the same terms in f32 lanes).
+"""
+import numpy as np
+import pytest
+
+import oxlibs
+from oxidize_amd import matvec as mv
+from oxidize_amd import synth
+
+pytestmark = pytest.mark.gpu
+
+Q80, Q4K, Q6K = 7, 13, 16
+
+
+def oracle_matvec(qtype, w, rows, cols, x):
+    o = oxlibs.oracle()
+    out = np.zeros(rows, np.float32)
+    temp = np.zeros(cols, np.float32)
+    rc = o.oxo_matvec_quantized(qtype, w.ctypes.data, rows, cols, synth.row_bytes(qtype, cols),
+                                x.ctypes.data, out.ctypes.data, temp.ctypes.data)
+    assert rc == 0
+    return out, temp
+
+
+def bits(a):
+    return np.ascontiguousarray(a).view(np.uint32)
+
+
+@pytest.mark.parametrize("cols", [32, 896, 4864, 4096])
+def test_quantize_q8_0_bytes_bit_exact(oxh, cols):
+    n_vec = 3
+    x = synth.normal(n_vec * cols, seed=4, stream=cols).reshape(n_vec, cols)
+    x[1, :32] = 0.0
+    x[2, :32] *= 1e-7          # f16 scale lands in the subnormal range
+    x[0, :32] *= 3e4           # large scale
+    nbytes = mv.act_bytes(Q80, cols)
+    d_x = mv.DeviceBuffer.from_host(x)
+    d_a = mv.DeviceBuffer(n_vec * nbytes)
+    mv.quantize(Q80, d_x.ptr, cols, n_vec, cols, d_a.ptr)
+    got = d_a.download(np.uint8, n_vec * nbytes).reshape(n_vec, nbytes)
+    o = oxlibs.oracle()
+    for v in range(n_vec):
+        want = np.zeros(nbytes, np.uint8)
+        o.oxo_quantize_q8_0(x[v].ctypes.data, cols, want.ctypes.data)
+        assert np.array_equal(got[v], want), "vector %d" % v
+
+
+@pytest.mark.parametrize("qtype,rows,cols", [
+    (Q6K, 1, 256), (Q6K, 9, 768), (Q6K, 100, 14336), (Q6K, 257, 4096), (Q6K, 33, 2816),
+    (Q80, 1, 32), (Q80, 5, 96), (Q80, 1000, 896), (Q80, 300, 4864), (Q80, 77, 4096),
+])
+def test_matvec_quantized_bits(oxh, qtype, rows, cols):
+    w = synth.weights(qtype, rows, cols, seed=21, stream=rows)
+    x = synth.normal(cols, seed=21, stream=9)
+    out = np.full(rows, np.nan, np.float32)
+    temp = np.zeros(cols, np.float32)
+    rc = mv.matvec_quantized(qtype, w, rows, cols, synth.row_bytes(qtype, cols), x, out, temp)
+    assert rc == 0
+    want, want_temp = oracle_matvec(qtype, w, rows, cols, x)
+    nact = mv.act_bytes(qtype, cols)
+    assert np.array_equal(temp.view(np.uint8)[:nact], want_temp.view(np.uint8)[:nact])
+    assert np.array_equal(bits(out), bits(want))
+    ref = oxlibs.ref()
+    if ref is not None:
+        r_out = np.zeros(rows, np.float32)
+        r_tmp = np.zeros(cols, np.float32)
+        ref.oc_matvec_quantized(qtype, w.ctypes.data, rows, cols, synth.row_bytes(qtype, cols),
+                                x.ctypes.data, r_out.ctypes.data, r_tmp.ctypes.data)
+        assert np.array_equal(temp.view(np.uint8)[:nact], r_tmp.view(np.uint8)[:nact])
+        if qtype == Q80:
+            assert np.all(np.abs(out - r_out) <= 1e-4 + 1e-5 * np.abs(r_out))
+        else:
+            assert np.array_equal(bits(out), bits(r_out))
+
+
+@pytest.mark.parametrize("qtype,cols,per_block", [(Q6K, 4096, 16), (Q80, 896, 1)])
+def test_subblock_sums_bit_exact(oxh, qtype, cols, per_block):
+    rows = 37
+    w = synth.weights(qtype, rows, cols, seed=6)
+    x = synth.normal(cols, seed=6)
+    o = oxlibs.oracle()
+    nact = mv.act_bytes(qtype, cols)
+    act = np.zeros(nact, np.uint8)
+    blocks = cols // synth.BLOCK_ELEMS[qtype]
+    rb = synth.row_bytes(qtype, cols)
+    want = np.zeros((rows, blocks, per_block), np.int32)
+    if qtype == Q6K:
+        o.oxo_quantize_q8_k(x.ctypes.data, cols, act.ctypes.data)
+        for r in range(rows):
+            o.oxo_dot_q6_k_q8_k(w[r * rb:].ctypes.data, blocks, act.ctypes.data, want[r].ctypes.data)
+    else:
+        o.oxo_quantize_q8_0(x.ctypes.data, cols, act.ctypes.data)
+        for r in range(rows):
+            o.oxo_dot_q8_0_q8_0(w[r * rb:].ctypes.data, blocks, act.ctypes.data, want[r].ctypes.data)
+    d_w = mv.DeviceBuffer.from_host(w)
+    d_a = mv.DeviceBuffer.from_host(act)
+    d_s = mv.DeviceBuffer(want.nbytes)
+    mv.debug_subblock_sums(qtype, d_w.ptr, rows, cols, d_a.ptr, d_s.ptr)
+    got = d_s.download(np.int32, want.size).reshape(want.shape)
+    assert np.array_equal(got, want)
+
+
+@pytest.mark.parametrize("qtype,cols,rows", [(Q4K, 4096, [4096, 1024, 1024]),
+                                             (Q4K, 2048, [300, 0, 5]),
+                                             (Q6K, 1024, [64, 64]),
+                                             (Q80, 896, [896, 128, 128])])
+def test_fused_equals_separate(oxh, qtype, cols, rows):
+    """oc_matvec_quantized_fused: bit-identical to one call per matrix, one
+    activation quantisation and one dispatch (tests/test_matvec_fused.c:88-136)."""
+    rb = synth.row_bytes(qtype, cols)
+    ws = [synth.weights(qtype, r, cols, seed=31, stream=i) if r else np.zeros(1, np.uint8)
+          for i, r in enumerate(rows)]
+    x = synth.normal(cols, seed=31, stream=99)
+    outs = [np.full(max(r, 1), np.nan, np.float32) for r in rows]
+    temp = np.zeros(cols, np.float32)
+    oxh.oc_matvec_fused_test_reset()
+    rc = mv.matvec_quantized_fused([qtype] * len(rows), ws, rows, cols, [rb] * len(rows), x, outs, temp)
+    assert rc == 0
+    st = oxh.oc_matvec_fused_test_stats()
+    assert (st.activation_quantizations, st.parallel_dispatches, st.fallback_calls) == (1, 1, 0)
+    for w, r, out in zip(ws, rows, outs):
+        if r == 0:
+            continue
+        want, _ = oracle_matvec(qtype, w, r, cols, x)
+        assert np.array_equal(bits(out[:r]), bits(want))
+
+
+def test_fused_mixed_types_falls_back_per_matrix(oxh):
+    cols = 1024
+    rows = [40, 24]
+    qts = [Q4K, Q6K]
+    ws = [synth.weights(q, r, cols, seed=32, stream=i) for i, (q, r) in enumerate(zip(qts, rows))]
+    x = synth.normal(cols, seed=32)
+    outs = [np.zeros(r, np.float32) for r in rows]
+    temp = np.zeros(cols, np.float32)
+    oxh.oc_matvec_fused_test_reset()
+    rc = mv.matvec_quantized_fused(qts, ws, rows, cols, [synth.row_bytes(q, cols) for q in qts],
+                                   x, outs, temp)
+    assert rc == 0
+    st = oxh.oc_matvec_fused_test_stats()
+    assert (st.activation_quantizations, st.parallel_dispatches, st.fallback_calls) == (2, 2, 2)
+    for q, w, r, out in zip(qts, ws, rows, outs):
+        want, _ = oracle_matvec(q, w, r, cols, x)
+        assert np.array_equal(bits(out), bits(want))
+
+
+@pytest.mark.parametrize("qtype,cols,rows", [(Q4K, 14336, [4096, 4096]), (Q4K, 768, [3, 17, 1, 40]),
+                                             (Q6K, 512, [10, 20]), (Q80, 64, [5, 6, 7])])
+def test_multi_input_equals_separate(oxh, qtype, cols, rows):
+    rb = synth.row_bytes(qtype, cols)
+    ws = [synth.weights(qtype, r, cols, seed=41, stream=i) for i, r in enumerate(rows)]
+    xs = [synth.normal(cols, seed=41, stream=200 + i) for i in range(len(rows))]
+    outs = [np.full(r, np.nan, np.float32) for r in rows]
+    temp = np.zeros(cols, np.float32)
+    oxh.oc_matvec_fused_test_reset()
+    rc = mv.matvec_quantized_multi_input([qtype] * len(rows), ws, rows, cols, [rb] * len(rows),
+                                         xs, outs, temp)
+    assert rc == 0
+    st = oxh.oc_matvec_fused_test_stats()
+    assert (st.activation_quantizations, st.parallel_dispatches, st.fallback_calls) == (len(rows), 1, 0)
+    for w, r, x, out in zip(ws, rows, xs, outs):
+        want, _ = oracle_matvec(qtype, w, r, cols, x)
+        assert np.array_equal(bits(out), bits(want))
+
+
+@pytest.mark.parametrize("qtype,rows,cols,n_vec,in_pad,out_pad", [
+    (Q4K, 96, 1024, 1, 0, 0), (Q4K, 96, 1024, 5, 3, 7), (Q4K, 64, 14336, 8, 0, 0),
+    (Q6K, 50, 512, 3, 16, 1), (Q80, 70, 896, 8, 0, 5), (Q80, 70, 896, 2, 4, 0),
+    (Q4K, 40, 512, 13, 0, 3), (Q6K, 24, 768, 11, 0, 0),
+])
+def test_batch_equals_single(oxh, qtype, rows, cols, n_vec, in_pad, out_pad):
+    """oc_matvec_quantized_batch: every output equals the single-vector call;
+    padded strides honoured and the padding left untouched
+    (tests/test_matvec_batch.c:86-99, :188-234)."""
+    in_stride, out_stride = cols + in_pad, rows + out_pad
+    w = synth.weights(qtype, rows, cols, seed=51)
+    xs = synth.normal(n_vec * in_stride, seed=51, stream=3).reshape(n_vec, in_stride)
+    outs = np.full((n_vec, out_stride), -7.25, np.float32)
+    temp = np.zeros(cols, np.float32)
+    scratch = np.zeros(mv.batch_scratch_bytes(cols), np.uint8)
+    rc = mv.matvec_quantized_batch(qtype, w, rows, cols, synth.row_bytes(qtype, cols), xs,
+                                   in_stride, outs, out_stride, n_vec, temp, scratch)
+    assert rc == 0
+    for v in range(n_vec):
+        want, _ = oracle_matvec(qtype, w, rows, cols, np.ascontiguousarray(xs[v, :cols]))
+        assert np.array_equal(bits(outs[v, :rows]), bits(want)), "vector %d" % v
+        assert np.all(outs[v, rows:] == -7.25)
+
+
+def test_declines_like_the_reference(oxh):
+    """Shapes the reference's integer path refuses come back OXH_DECLINED with
+    the outputs untouched (matvec.c:99-127, :961-985, :1290-1292)."""
+    out = np.full(8, 3.5, np.float32)
+    temp = np.zeros(4096, np.float32)
+    x = synth.normal(4096, seed=1)
+    w = synth.weights(Q4K, 8, 4096, seed=1)
+    rb = synth.row_bytes(Q4K, 4096)
+    # K-quant with cols not a multiple of 256 (e.g. n_embd = 896)
+    assert mv.matvec_quantized(Q4K, w, 8, 896, 504, x, out, temp) == mv.DECLINED
+    # padded row stride
+    assert mv.matvec_quantized(Q4K, w, 4, 4096, rb + 16, x, out, temp) == mv.DECLINED
+    # a type with no kernel here (F16 = 1)
+    assert mv.matvec_quantized(1, w, 8, 4096, 8192, x, out, temp) == mv.DECLINED
+    # global switch off
+    oxh.oc_matvec_set_fused(False)
+    try:
+        assert mv.matvec_quantized(Q4K, w, 8, 4096, rb, x, out, temp) == mv.DECLINED
+    finally:
+        oxh.oc_matvec_set_fused(True)
+    # batch without scratch / with scratch smaller than one activation
+    outs = np.full((2, 8), 3.5, np.float32)
+    xs = np.stack([x, x])
+    assert mv.matvec_quantized_batch(Q4K, w, 8, 4096, rb, xs, 4096, outs, 8, 2, temp, None) == mv.DECLINED
+    small = np.zeros(100, np.uint8)
+    assert mv.matvec_quantized_batch(Q4K, w, 8, 4096, rb, xs, 4096, outs, 8, 2, temp, small) == mv.DECLINED
+    assert np.all(out == 3.5) and np.all(outs == 3.5)
+    # and the same call with everything in order is handled
+    assert mv.matvec_quantized(Q4K, w, 8, 4096, rb, x, out, temp) == mv.OK
+
+
+def test_empty_inputs_are_no_ops(oxh):
+    x = synth.normal(256, seed=1)
+    w = synth.weights(Q4K, 1, 256, seed=1)
+    out = np.full(4, 1.5, np.float32)
+    temp = np.zeros(256, np.float32)
+    assert mv.matvec_quantized(Q4K, w, 0, 256, 144, x, out, temp) == mv.OK
+    assert mv.matvec_quantized_fused([], [], [], 256, [], x, [], temp) == mv.OK
+    scratch = np.zeros(4096, np.uint8)
+    assert mv.matvec_quantized_batch(Q4K, w, 1, 256, 144, x, 256, out, 1, 0, temp, scratch) == mv.OK
+    assert np.all(out == 1.5)
+
+
+def test_expert_slices_resolve_inside_a_registered_tensor(oxh):
+    """A stacked expert tensor registered once; calls pass slice pointers
+    (llama.c:4248-4251 stacks expert e at rows [e*rows, (e+1)*rows))."""
+    n_exp, rows, cols = 4, 48, 1024
+    rb = synth.row_bytes(Q4K, cols)
+    w = synth.weights(Q4K, n_exp * rows, cols, seed=61)
+    from oxidize_amd import _lib
+    _lib.check(oxh.oxh_weight_register(w.ctypes.data, w.nbytes))
+    base = oxh.oxh_weight_device_ptr(w.ctypes.data)
+    x = synth.normal(cols, seed=61)
+    temp = np.zeros(cols, np.float32)
+    for e in (2, 0, 3):
+        sl = w[e * rows * rb:(e + 1) * rows * rb]
+        assert oxh.oxh_weight_device_ptr(sl.ctypes.data) == base + e * rows * rb
+        out = np.zeros(rows, np.float32)
+        assert mv.matvec_quantized(Q4K, sl, rows, cols, rb, x, out, temp) == mv.OK
+        want, _ = oracle_matvec(Q4K, np.ascontiguousarray(sl), rows, cols, x)
+        assert np.array_equal(bits(out), bits(want))
