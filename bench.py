@@ -1,0 +1,193 @@
+#!/usr/bin/env python3
+"""Benchmark of the quantized-matvec hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+A step is one decode token of the Llama-3-8B-shaped GEMV set: 32 layers x
+{fused q/k/v, o, fused gate/up (Q4_K), down (Q6_K)}, every GEMV preceded by
+the Q8_K quantisation of its own f32 input, 256 launches replayed as one HIP
+graph.  All inputs are resident in HBM before the timed region starts.
+
+Prints ONE JSON line.  `value` is whole-step algorithmic GB/s (packed weights
+at their on-disk size + f32 activations in + f32 outputs out, divided by the
+wall time of the K timed steps).  `roofline` is the dominant kernel (the
+Q4_K gate/up GEMV, 28672 x 4096) timed with HIP events on the launch stream.
+`cpu_baseline` is the reference's own CPU code (oracle/_ref, or the oracle
+port when that was never built) on this host's cores over one layer.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0
+
+
+def cpu_baseline(layers_sample=1, min_seconds=1.5):
+    """The reference CPU path on the host cores over `layers_sample` layers of
+    the same workload (same shapes, same synthetic generator)."""
+    import ctypes
+
+    import numpy as np
+    sys.path.insert(0, os.path.join(ROOT, "tests"))
+    import oxlibs
+    from oxidize_amd import synth
+
+    ref = oxlibs.ref()
+    kind = "reference" if ref is not None else "port"
+    cores = min(16, os.cpu_count() or 1)
+    if ref is not None:
+        ref.oc_parallel_set_threads(cores)
+    else:
+        os.environ.setdefault("OMP_NUM_THREADS", str(cores))
+    orc = oxlibs.oracle()
+    ops = [(13, [4096, 1024, 1024], 4096), (13, [4096], 4096), (13, [14336, 14336], 4096),
+           (16, [4096], 14336)]
+    mats = []
+    nbytes = 0
+    for i, (qt, rows, cols) in enumerate(ops):
+        ws = [synth.weights(qt, r, cols, seed=0, stream=9000 + 10 * i + k) for k, r in enumerate(rows)]
+        x = synth.normal(cols, seed=0, stream=9900 + i)
+        outs = [np.zeros(r, np.float32) for r in rows]
+        temp = np.zeros(cols, np.float32)
+        mats.append((qt, rows, cols, ws, x, outs, temp))
+        nbytes += sum(w.nbytes for w in ws) + 4 * cols + 4 * sum(rows)
+
+    def one_layer():
+        for qt, rows, cols, ws, x, outs, temp in mats:
+            rb = synth.row_bytes(qt, cols)
+            n = len(rows)
+            if ref is not None:
+                ref.oc_matvec_quantized_fused(oxlibs.u32_array([qt] * n), oxlibs.ptr_array(ws),
+                                              oxlibs.size_array(rows), cols, oxlibs.size_array([rb] * n),
+                                              n, x.ctypes.data, oxlibs.ptr_array(outs), temp.ctypes.data)
+            else:
+                orc.oxo_matvec_quantized_fused(oxlibs.u32_array([qt] * n), oxlibs.ptr_array(ws),
+                                               oxlibs.size_array(rows), cols, oxlibs.size_array([rb] * n),
+                                               n, x.ctypes.data, oxlibs.ptr_array(outs), temp.ctypes.data)
+
+    one_layer()
+    reps, t0 = 0, time.perf_counter()
+    while True:
+        one_layer()
+        reps += 1
+        dt = time.perf_counter() - t0
+        if dt >= min_seconds and reps >= 3:
+            break
+    gbps = nbytes * reps / dt / 1e9
+    return {"value": round(gbps, 3), "unit": "GB/s", "cores": cores, "kind": kind,
+            "sample": "%d repetitions of one layer of the same decode set (qkv, o, gate/up Q4_K; "
+                      "down Q6_K; %.1f MB per repetition) through oc_matvec_quantized_fused, "
+                      "%.2f s wall" % (reps, nbytes / 1e6, dt)}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--layers", type=int, default=32, help=argparse.SUPPRESS)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-graph", action="store_true", help="launch kernels one by one")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this path is built and measured on ONE GPU; --gpus %d is not supported "
+              "(the work shards by output rows, see DESIGN.md)" % args.gpus, file=sys.stderr)
+        return 2
+
+    from oxidize_amd import _lib
+    from oxidize_amd import matvec as mv
+    from oxidize_amd.workloads import DecodeSet
+
+    lib = _lib.lib()
+    _lib.check(lib.oxh_init(0))
+    info = mv.device_info()
+
+    ds = DecodeSet(layers=args.layers, seed=0)
+    step_bytes = ds.bytes_per_step
+
+    graph = None
+    if not args.no_graph:
+        graph = mv.Graph()
+        with graph:
+            ds.launch_step()
+
+    def step():
+        if graph is not None:
+            graph.launch()
+        else:
+            ds.launch_step()
+
+    for _ in range(args.warmup):
+        step()
+    mv.sync()
+
+    e0, e1 = mv.Event(), mv.Event()
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(args.steps):
+        step()
+    e1.record()
+    mv.sync()
+    wall = time.perf_counter() - t0
+    ev_ms = e1.ms_since(e0)
+    ms_per_step = wall * 1e3 / args.steps
+    value = step_bytes * args.steps / wall / 1e9
+
+    # Dominant kernel: the Q4_K gate/up GEMV (2 x 14336 rows x 4096), timed
+    # back to back over the 32 layers' distinct weights (2.1 GB per sweep, so
+    # nothing is served from cache), HIP events on the launch stream.
+    gate_up = 2
+    _, qt, rows, cols, _ = ds.ops[gate_up]
+    k_bytes = sum(w.nbytes for w in ds.weights[0][gate_up]) + 4 * cols + 4 * sum(rows)
+    sweeps = max(3, min(10, args.steps))
+    for layer in range(ds.layers):
+        ds.launch_op(layer, gate_up, quantize=False)
+    mv.sync()
+    k0, k1 = mv.Event(), mv.Event()
+    k0.record()
+    for _ in range(sweeps):
+        for layer in range(ds.layers):
+            ds.launch_op(layer, gate_up, quantize=False)
+    k1.record()
+    mv.sync()
+    k_us = k1.ms_since(k0) * 1e3 / (sweeps * ds.layers)
+    achieved = k_bytes / k_us / 1e3   # GB/s
+
+    out = {
+        "metric": "q4k_gemv_hbm_gbps_llama3_8b_decode",
+        "value": round(value, 2),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "i8",
+        "data": "synthetic",
+        "config": {"workload": "llama3-8b decode GEMV set, batch 1, 32 layers: qkv+o+gate/up Q4_K, "
+                               "down Q6_K, Q8_K activations (BASELINE configs[1])",
+                   "layers": ds.layers, "launches_per_step": 8 * ds.layers,
+                   "bytes_per_step": step_bytes, "hip_graph": graph is not None},
+        "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBPS, 2),
+        "tokens_per_s_equiv": round(args.steps / wall, 1),
+        "gpu_event_ms_per_step": round(ev_ms / args.steps, 4),
+        "device": info,
+        "roofline": {"bound": "hbm", "kernel": "k_gemv_q4_k (gate/up 28672x4096)",
+                     "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "bytes_per_launch": k_bytes, "us_per_launch": round(k_us, 3)},
+    }
+    out["cpu_baseline"] = None if args.no_cpu else cpu_baseline()
+    print(json.dumps(out))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -140,6 +140,15 @@ int  oxh_event_destroy(void *event);
 int  oxh_event_record(void *event, void *stream);
 int  oxh_event_sync(void *event);
 int  oxh_event_elapsed_ms(void *start, void *stop, float *ms);
+/* Capture everything launched on `stream` between begin and end into a HIP
+ * graph and replay it with one call: a decode step is a few hundred short
+ * launches whose submission cost would otherwise dominate.  The device
+ * functions above record no memset nodes.  The reference's counterpart is the
+ * graph-replay decode of oxidize-c/src/backends/cuda_fast.cu (cuda.h:250-265). */
+int  oxh_graph_begin(void *stream);
+int  oxh_graph_end(void *stream, void **graph_exec);
+int  oxh_graph_launch(void *graph_exec, void *stream);
+int  oxh_graph_destroy(void *graph_exec);
 /* name (<=255 chars), compute units, clock MHz, memory bytes. */
 int  oxh_device_info(char *name, size_t name_len, int *n_cu, int *clock_mhz,
                      size_t *mem_bytes);

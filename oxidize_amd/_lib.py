@@ -53,6 +53,10 @@ SIGNATURES = {
     "oxh_event_record": (I, [V, V]),
     "oxh_event_sync": (I, [V]),
     "oxh_event_elapsed_ms": (I, [V, V, ctypes.POINTER(ctypes.c_float)]),
+    "oxh_graph_begin": (I, [V]),
+    "oxh_graph_end": (I, [V, ctypes.POINTER(V)]),
+    "oxh_graph_launch": (I, [V, V]),
+    "oxh_graph_destroy": (I, [V]),
     "oxh_device_info": (I, [ctypes.c_char_p, Z, ctypes.POINTER(I), ctypes.POINTER(I),
                             ctypes.POINTER(Z)]),
     "oxh_weight_register": (I, [V, Z]),

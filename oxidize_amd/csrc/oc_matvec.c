@@ -467,13 +467,13 @@ int oxh_matvec_quantized_batch(uint32_t qtype, const uint8_t *data, size_t rows,
     }
     if ((rc = quantize(kind, (const float *)g_dx.p, in_stride, n_vec, cols, g_dact.p))) return rc;
 
-    const size_t mmq_min = 16;
-    if (kind == 2 && n_vec >= mmq_min && (qtype == OXH_Q4_K_S || qtype == OXH_Q4_K_M)) {
-        rc = oxh_mmq(qtype, d_w, rows, cols, g_dact.p, n_vec, (float *)g_dout.p, rows, NULL);
-        if (rc == OXH_OK) goto copy_back;
-        /* fall through to the GEMV kernel over slices of the batch */
-    }
-    {
+    /* More vectors than the GEMV kernel keeps in flight: Q4_K goes to the
+     * int8-MFMA kernel; the other types walk the batch in GEMV-sized slices
+     * (every output is the same dot either way). */
+    if (n_vec > 8 && (qtype == OXH_Q4_K_S || qtype == OXH_Q4_K_M)) {
+        if ((rc = oxh_mmq(qtype, d_w, rows, cols, g_dact.p, n_vec, (float *)g_dout.p, rows, NULL)))
+            return rc;
+    } else {
         size_t step = oxh_gemv_max_nvec(qtype, cols);
         if (step == 0) {
             oxh_set_error("batch: cols too wide for one workgroup%s%s", NULL, NULL);
@@ -485,7 +485,6 @@ int oxh_matvec_quantized_batch(uint32_t qtype, const uint8_t *data, size_t rows,
             if ((rc = oxh_gemv_segments(qtype, &seg, 1, cols, g_dact.p, m, rows, NULL))) return rc;
         }
     }
-copy_back:
     if (out_stride == rows) {
         if ((rc = oxh_memcpy_d2h(outputs, g_dout.p, packed_out, NULL))) return rc;
     } else {

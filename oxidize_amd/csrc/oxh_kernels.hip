@@ -616,6 +616,152 @@ k_gemv_q8_0(const SegTable segs, const GemvParams p, const uint8_t *__restrict__
     row_sums(terms, lane, NV, nrows, RW, B, p.term_stride, segs.out[seg], p.out_stride, row0);
 }
 
+/* ─── prefill matmul (MMQ) ────────────────────────────────────────────── */
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+
+#define MMQ_WAVES 4
+#define MMQ_ROWS (MMQ_WAVES * 32)   /* weight rows per workgroup          */
+#define MMQ_TOK 64                  /* tokens per workgroup (two tiles)   */
+
+/* Q4_K weights x Q8_K activations on v_mfma_i32_32x32x32_i8.
+ *
+ * One MFMA covers 32 tokens x 32 weight rows x one 32-wide sub-block, so each
+ * result tile is exactly the sub-block sums S_j of oxk.c:263-270 for 1024
+ * (token, row) pairs.  M = tokens (A operand, int8 activations staged in
+ * LDS), N = weight rows (B operand, nibble codes unpacked in registers): the
+ * accumulator of lane l then belongs to weight row l%32, so the 6-bit scale
+ * is one register per lane and `pos += sc_j * S_j` is an integer multiply-add
+ * per accumulator.  The min term sum_j m_j*B_j is formed by a second MFMA per
+ * sub-block with the B operand set to m_j in every byte (sum_k m_j*q_k over
+ * the sub-block is m_j*B_j), accumulated over the whole super-block.
+ * Per super-block the f32 step is the reference's, in its order:
+ *   acc += (dw*dq)*(float)pos - (dmin*dq)*(float)min_acc      (oxk.c:286-294)
+ * so every output is bit-identical to the single-vector GEMV.
+ *
+ * Lane l supplies, for both operands, the 16 values k = 16*(l/32) .. +15 of
+ * the sub-block; A and B use the same assignment, so the product does not
+ * depend on how the hardware numbers k internally. */
+__global__ __launch_bounds__(MMQ_WAVES * 64) void
+k_mmq_q4_k(const uint8_t *__restrict__ w, uint32_t rows, uint32_t B,
+           const uint8_t *__restrict__ acts, uint32_t n_vec, float *__restrict__ out,
+           size_t out_stride)
+{
+    __shared__ __attribute__((aligned(16))) uint8_t lds_q[MMQ_TOK * 256];
+    __shared__ float lds_dq[MMQ_TOK];
+
+    const uint32_t tid = threadIdx.x;
+    const uint32_t lane = tid & 63u;
+    const uint32_t wave = tid >> 6;
+    const uint32_t n = lane & 31u;          /* weight row / token within a tile */
+    const uint32_t h = lane >> 5;           /* which 16 of the sub-block's 32   */
+    const uint32_t row_base = blockIdx.x * MMQ_ROWS + wave * 32u;
+    const uint32_t tok_base = blockIdx.y * MMQ_TOK;
+    const uint32_t row = row_base + n;
+    const uint32_t row_c = row < rows ? row : rows - 1u;
+    const uint8_t *wrow = w + (size_t)row_c * B * 144u;
+    const size_t act_stride = (size_t)B * 292u;
+
+    float acc[2][16];
+#pragma unroll
+    for (int t = 0; t < 2; t++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) acc[t][i] = 0.0f;
+
+    for (uint32_t b = 0; b < B; b++) {
+        __syncthreads();
+        /* stage this super-block of 64 tokens: value dword wd of token t goes
+         * to [tile][j][h][token-in-tile] x 16 B */
+        for (uint32_t idx = tid; idx < MMQ_TOK * 64u; idx += MMQ_WAVES * 64u) {
+            const uint32_t t = idx >> 6, wd = idx & 63u;
+            const uint32_t tok = tok_base + t;
+            uint32_t val = 0u;
+            if (tok < n_vec)
+                val = *reinterpret_cast<const uint32_t *>(acts + (size_t)tok * act_stride +
+                                                          (size_t)b * 292u + 4u + 4u * wd);
+            const uint32_t j = wd >> 3, hh = (wd >> 2) & 1u;
+            const uint32_t slot = (((t >> 5) * 8u + j) * 2u + hh) * 32u + (t & 31u);
+            reinterpret_cast<uint32_t *>(lds_q)[slot * 4u + (wd & 3u)] = val;
+        }
+        if (tid < MMQ_TOK) {
+            const uint32_t tok = tok_base + tid;
+            lds_dq[tid] = tok < n_vec
+                ? *reinterpret_cast<const float *>(acts + (size_t)tok * act_stride + (size_t)b * 292u)
+                : 0.0f;
+        }
+        /* this lane's weights: header and its half of each 32-byte nibble group */
+        const uint8_t *wb = wrow + (size_t)b * 144u;
+        const u32x4 hdr = *reinterpret_cast<const u32x4 *>(wb);
+        u32x4 nib[4];
+#pragma unroll
+        for (int gp = 0; gp < 4; gp++)
+            nib[gp] = *reinterpret_cast<const u32x4 *>(wb + 16u + 32u * gp + 16u * h);
+        __syncthreads();
+
+        const uint32_t u0 = hdr.y, u1 = hdr.z, u2 = hdr.w;
+        const uint32_t sc_lo = u0 & 0x3F3F3F3Fu;
+        const uint32_t mn_lo = u1 & 0x3F3F3F3Fu;
+        const uint32_t sc_hi = (u2 & 0x0F0F0F0Fu) | ((u0 >> 2) & 0x30303030u);
+        const uint32_t mn_hi = ((u2 >> 4) & 0x0F0F0F0Fu) | ((u1 >> 2) & 0x30303030u);
+        const float dw = half_bits_to_float(hdr.x & 0xFFFFu);
+        const float dmin = half_bits_to_float(hdr.x >> 16);
+
+        v16i pos[2], mn[2];
+#pragma unroll
+        for (int t = 0; t < 2; t++)
+#pragma unroll
+            for (int i = 0; i < 16; i++) { pos[t][i] = 0; mn[t][i] = 0; }
+
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const u32x4 raw = nib[j >> 1];
+            v4i bw;
+#pragma unroll
+            for (int k = 0; k < 4; k++)
+                bw[k] = (int)((j & 1) ? ((raw[k] >> 4) & 0x0F0F0F0Fu) : (raw[k] & 0x0F0F0F0Fu));
+            const uint32_t scw = j < 4 ? sc_lo : sc_hi;
+            const uint32_t mnw = j < 4 ? mn_lo : mn_hi;
+            const int sc = (int)((scw >> (8 * (j & 3))) & 0xFFu);
+            const int mj = (int)(((mnw >> (8 * (j & 3))) & 0xFFu) * 0x01010101u);
+            const v4i bm = { mj, mj, mj, mj };
+#pragma unroll
+            for (int t = 0; t < 2; t++) {
+                const v4i a = *reinterpret_cast<const v4i *>(
+                    lds_q + ((((uint32_t)t * 8u + (uint32_t)j) * 2u + h) * 32u + n) * 16u);
+                const v16i zero = { 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0 };
+                const v16i sj = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, bw, zero, 0, 0, 0);
+#pragma unroll
+                for (int i = 0; i < 16; i++) pos[t][i] += __mul24(sc, sj[i]);
+                mn[t] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, bm, mn[t], 0, 0, 0);
+            }
+        }
+        /* accumulator i of lane l is token 8*(i/4) + 4*(l/32) + i%4 of the tile */
+#pragma unroll
+        for (int t = 0; t < 2; t++)
+#pragma unroll
+            for (int i = 0; i < 16; i++) {
+                const uint32_t m = 8u * (uint32_t)(i >> 2) + 4u * h + (uint32_t)(i & 3);
+                const float dq = lds_dq[t * 32 + m];
+                const float t_pos = dw * dq;
+                const float t_min = dmin * dq;
+                const float up = t_pos * (float)pos[t][i];
+                const float dn = t_min * (float)mn[t][i];
+                acc[t][i] += up - dn;
+            }
+    }
+    if (row < rows) {
+#pragma unroll
+        for (int t = 0; t < 2; t++)
+#pragma unroll
+            for (int i = 0; i < 16; i++) {
+                const uint32_t m = 8u * (uint32_t)(i >> 2) + 4u * h + (uint32_t)(i & 3);
+                const uint32_t tok = tok_base + (uint32_t)t * 32u + m;
+                if (tok < n_vec) out[(size_t)tok * out_stride + row] = acc[t][i];
+            }
+    }
+}
+
 /* ─── host side of layer 2 ────────────────────────────────────────────── */
 
 static int g_device = -1;
@@ -899,11 +1045,29 @@ extern "C" int oxh_debug_subblock_sums(uint32_t qtype, const void *d_w, size_t r
     return OXH_OK;
 }
 
-extern "C" int oxh_mmq(uint32_t, const void *, size_t, size_t, const void *, size_t,
-                       float *, size_t, void *)
+extern "C" int oxh_mmq(uint32_t qtype, const void *d_w, size_t rows, size_t cols,
+                       const void *d_acts, size_t n_vec, float *d_out, size_t out_stride,
+                       void *stream)
 {
-    snprintf(g_err, sizeof g_err, "oxh_mmq: not built yet");
-    return OXH_ERR_ARG;
+    int rc = ensure_init();
+    if (rc) return rc;
+    if (rows == 0 || n_vec == 0) return OXH_OK;
+    if (!d_w || !d_acts || !d_out) return arg_fail("oxh_mmq: NULL pointer");
+    if (!is_q4k(qtype) || oxh_act_kind(qtype, cols) != 2) {
+        snprintf(g_err, sizeof g_err, "oxh_mmq: qtype %u with cols %zu has no MFMA kernel", qtype, cols);
+        return OXH_DECLINED;
+    }
+    if (out_stride < rows) return arg_fail("oxh_mmq: out_stride < rows");
+    const size_t blocks = cols / OXH_QK_K;
+    if (rows > 0x7FFFFFFFull || n_vec > 0x7FFFFFFFull || blocks > 0xFFFFFFull)
+        return arg_fail("oxh_mmq: dimension too large");
+    const dim3 grid((uint32_t)((rows + MMQ_ROWS - 1) / MMQ_ROWS),
+                    (uint32_t)((n_vec + MMQ_TOK - 1) / MMQ_TOK));
+    hipLaunchKernelGGL(k_mmq_q4_k, grid, dim3(MMQ_WAVES * 64), 0, pick_stream(stream),
+                       (const uint8_t *)d_w, (uint32_t)rows, (uint32_t)blocks,
+                       (const uint8_t *)d_acts, (uint32_t)n_vec, d_out, out_stride);
+    HIP_TRY(hipGetLastError());
+    return OXH_OK;
 }
 
 /* ─── memory / stream / event plumbing ────────────────────────────────── */
@@ -1012,6 +1176,39 @@ extern "C" int oxh_event_sync(void *event)
 extern "C" int oxh_event_elapsed_ms(void *start, void *stop, float *ms)
 {
     HIP_TRY(hipEventElapsedTime(ms, (hipEvent_t)start, (hipEvent_t)stop));
+    return OXH_OK;
+}
+
+extern "C" int oxh_graph_begin(void *stream)
+{
+    int rc = ensure_init();
+    if (rc) return rc;
+    HIP_TRY(hipStreamBeginCapture(pick_stream(stream), hipStreamCaptureModeThreadLocal));
+    return OXH_OK;
+}
+
+extern "C" int oxh_graph_end(void *stream, void **graph_exec)
+{
+    if (!graph_exec) return arg_fail("oxh_graph_end: NULL");
+    hipGraph_t graph = nullptr;
+    HIP_TRY(hipStreamEndCapture(pick_stream(stream), &graph));
+    hipGraphExec_t exec = nullptr;
+    hipError_t e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+    (void)hipGraphDestroy(graph);
+    if (e != hipSuccess) return hip_fail(e, "hipGraphInstantiate");
+    *graph_exec = (void *)exec;
+    return OXH_OK;
+}
+
+extern "C" int oxh_graph_launch(void *graph_exec, void *stream)
+{
+    HIP_TRY(hipGraphLaunch((hipGraphExec_t)graph_exec, pick_stream(stream)));
+    return OXH_OK;
+}
+
+extern "C" int oxh_graph_destroy(void *graph_exec)
+{
+    if (graph_exec) HIP_TRY(hipGraphExecDestroy((hipGraphExec_t)graph_exec));
     return OXH_OK;
 }
 

@@ -161,3 +161,46 @@ def device_info():
     check(lib().oxh_device_info(name, 256, ctypes.byref(n_cu), ctypes.byref(mhz), ctypes.byref(mem)))
     return {"name": name.value.decode(), "n_cu": n_cu.value, "clock_mhz": mhz.value,
             "mem_bytes": mem.value}
+
+
+class Graph:
+    """Capture of everything launched on `stream` inside the with-block."""
+
+    def __init__(self, stream=None):
+        self.stream = stream
+        self.exec = ctypes.c_void_p()
+
+    def __enter__(self):
+        check(lib().oxh_graph_begin(self.stream))
+        return self
+
+    def __exit__(self, exc_type, exc, tb):
+        rc = lib().oxh_graph_end(self.stream, ctypes.byref(self.exec))
+        if exc_type is None:
+            check(rc)
+        return False
+
+    def launch(self):
+        check(lib().oxh_graph_launch(self.exec, self.stream))
+
+    def destroy(self):
+        if self.exec:
+            lib().oxh_graph_destroy(self.exec)
+            self.exec = ctypes.c_void_p()
+
+
+class Event:
+    def __init__(self):
+        self.handle = ctypes.c_void_p()
+        check(lib().oxh_event_create(ctypes.byref(self.handle)))
+
+    def record(self, stream=None):
+        check(lib().oxh_event_record(self.handle, stream))
+
+    def sync(self):
+        check(lib().oxh_event_sync(self.handle))
+
+    def ms_since(self, start):
+        ms = ctypes.c_float()
+        check(lib().oxh_event_elapsed_ms(start.handle, self.handle, ctypes.byref(ms)))
+        return ms.value

@@ -1,0 +1,177 @@
+"""Writes tests/golden/*.npz: input/output vectors taken from the COMPILED
+REFERENCE (oracle/_ref/liboxref.so, built by `make -C oracle` from the
+reference checkout).  Run in the build container only; the fixtures are
+committed, this script documents how they were made.
+
+    python tests/golden/make_golden.py
+
+Every array is data: inputs and the reference's outputs for them.
+"""
+import ctypes
+import os
+import sys
+import zlib
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(os.path.dirname(HERE))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "tests"))
+
+import oxlibs  # noqa: E402
+from oxidize_amd import synth  # noqa: E402
+
+Q80, Q4K, Q6K = 7, 13, 16
+
+
+def xorshift_bytes(n, seed):
+    """The byte stream of the reference's raw-block tests
+    (tests/test_oxk_avx2_parity.c:125-131): xorshift32, low byte of each draw."""
+    out = np.empty(n, np.uint8)
+    s = seed & 0xFFFFFFFF
+    for i in range(n):
+        s ^= (s << 13) & 0xFFFFFFFF
+        s ^= s >> 17
+        s ^= (s << 5) & 0xFFFFFFFF
+        out[i] = s & 0xFF
+    return out
+
+
+def finite_scale_bits(rng, n):
+    """f16 bit patterns of finite positive scales in [0.0005, 0.0405]."""
+    vals = (0.0005 + rng.integers(0, 1000, n) * 4e-5).astype(np.float32)
+    return vals.astype(np.float16).view(np.uint16)
+
+
+def main():
+    ref = oxlibs.ref()
+    if ref is None:
+        raise SystemExit("oracle/_ref/liboxref.so missing: run `make -C oracle` first")
+    ref.oc_parallel_set_threads(1)
+    rng = np.random.default_rng(20240607)
+
+    # ── scalar helpers ────────────────────────────────────────────────────
+    h = np.arange(65536, dtype=np.uint16)
+    f16_to_f32 = np.empty(65536, np.uint32)
+    two = (ctypes.c_uint8 * 2)()
+    for i in range(65536):
+        two[0], two[1] = i & 255, i >> 8
+        f16_to_f32[i] = np.float32(ref.oc_oxk_f16_le_to_f32(two)).view(np.uint32)
+    # f32 -> f16: random magnitudes, exact ties, subnormal range, overflow edge
+    parts = [rng.standard_normal(3000).astype(np.float32) * s
+             for s in (1e-9, 1e-7, 6e-6, 1e-4, 1e-2, 1.0, 300.0, 7e4)]
+    ties = ((np.arange(0x33000000, 0x47800000, 0x2000, dtype=np.uint32) | 0x1000)).view(np.float32)
+    near = ((np.arange(0x33000000, 0x47800000, 0x2000, dtype=np.uint32) | 0x0FFF)).view(np.float32)
+    edge = np.array([0.0, -0.0, 65504.0, 65519.99, 65520.0, 1e10, -1e10, np.inf, -np.inf,
+                     5.9604645e-8, 2.9802322e-8, 2.98e-8, 6.0975552e-5, 6.1035156e-5],
+                    dtype=np.float32)
+    f32_in = np.concatenate(parts + [ties[::37], near[::41], edge]).astype(np.float32)
+    f32_to_f16 = np.array([ref.oc_f32_to_f16_bits(float(v)) for v in f32_in], dtype=np.uint16)
+
+    scales = rng.integers(0, 256, (512, 12), dtype=np.uint8)
+    sc_out = np.empty((512, 8, 2), np.uint8)
+    a = ctypes.c_uint8()
+    b = ctypes.c_uint8()
+    for i in range(512):
+        for j in range(8):
+            ref.oc_oxk_get_scale_min_k4(j, scales[i].ctypes.data, ctypes.byref(a), ctypes.byref(b))
+            sc_out[i, j] = (a.value, b.value)
+    np.savez_compressed(os.path.join(HERE, "scalar_helpers.npz"),
+                        f16_to_f32_bits=f16_to_f32, f32_in=f32_in, f32_to_f16_bits=f32_to_f16,
+                        k4_scales=scales, k4_sc_min=sc_out)
+
+    # ── raw-block dots (random bytes, finite scales, acts in [-127,127]) ──
+    nb, trials = 12, 24
+    out = {}
+    for name, qt, bsize, d_offs in (("q4_k", Q4K, 144, (0, 2)), ("q6_k", Q6K, 210, (208,)),
+                                    ("q8_0", Q80, 34, (0,))):
+        w = xorshift_bytes(trials * nb * bsize, 0x9E3779B9 ^ qt).reshape(trials, nb, bsize)
+        for off in d_offs:
+            bits = finite_scale_bits(rng, trials * nb).reshape(trials, nb)
+            w[:, :, off] = bits & 0xFF
+            w[:, :, off + 1] = bits >> 8
+        if qt == Q80:
+            act = np.zeros((trials, nb, 34), np.uint8)
+            bits = finite_scale_bits(rng, trials * nb).reshape(trials, nb)
+            act[:, :, 0] = bits & 0xFF
+            act[:, :, 1] = bits >> 8
+            act[:, :, 2:] = rng.integers(-127, 128, (trials, nb, 32)).astype(np.int8).view(np.uint8)
+        else:
+            act = np.zeros((trials, nb, 292), np.uint8)
+            d = (0.001 + rng.integers(0, 1000, (trials, nb)) * 2e-5).astype(np.float32)
+            act[:, :, 0:4] = d.view(np.uint8).reshape(trials, nb, 4)
+            q = rng.integers(-127, 128, (trials, nb, 256)).astype(np.int8)
+            act[:, :, 4:260] = q.view(np.uint8)
+            bs = q.reshape(trials, nb, 16, 16).sum(axis=3).astype(np.int16)
+            act[:, :, 260:292] = bs.view(np.uint8).reshape(trials, nb, 32)
+        scalar = np.empty((trials, 2), np.uint32)
+        disp = np.empty((trials, 2), np.uint32)
+        fs = getattr(ref, "oc_oxk_dot_%s_%s_scalar" % (name, "q8_0" if qt == Q80 else "q8_k"))
+        fd = getattr(ref, "oc_oxk_dot_%s_%s" % (name, "q8_0" if qt == Q80 else "q8_k"))
+        for t in range(trials):
+            wt = np.ascontiguousarray(w[t])
+            at = np.ascontiguousarray(act[t])
+            for k, blocks in enumerate((1, nb)):
+                scalar[t, k] = np.float32(fs(wt.ctypes.data, blocks, at.ctypes.data)).view(np.uint32)
+                disp[t, k] = np.float32(fd(wt.ctypes.data, blocks, at.ctypes.data)).view(np.uint32)
+        out[name + "_w"] = w
+        out[name + "_act"] = act
+        out[name + "_scalar_bits"] = scalar
+        out[name + "_dispatched_bits"] = disp
+    np.savez_compressed(os.path.join(HERE, "raw_block_dots.npz"), **out)
+
+    # ── API level: small matrices stored whole ───────────────────────────
+    api = {}
+    for name, qt, rows, cols in (("q4_k", Q4K, 48, 1024), ("q6_k", Q6K, 24, 768), ("q8_0", Q80, 40, 896)):
+        rb = synth.row_bytes(qt, cols)
+        w = synth.weights(qt, rows, cols, seed=7, stream=qt)
+        x = synth.normal(cols, seed=7, stream=100 + qt)
+        o = np.zeros(rows, np.float32)
+        temp = np.zeros(cols, np.float32)
+        ref.oc_matvec_quantized(qt, w.ctypes.data, rows, cols, rb, x.ctypes.data, o.ctypes.data,
+                                temp.ctypes.data)
+        nact = cols // synth.BLOCK_ELEMS[qt] * (34 if qt == Q80 else 292)
+        api[name + "_w"] = w
+        api[name + "_x"] = x
+        api[name + "_shape"] = np.array([rows, cols, rb], np.int64)
+        api[name + "_out_bits"] = o.view(np.uint32).copy()
+        api[name + "_act"] = temp.view(np.uint8)[:nact].copy()
+        # batch with padded strides, 5 vectors
+        n_vec, in_stride, out_stride = 5, cols + 8, rows + 3
+        xs = synth.normal(n_vec * in_stride, seed=8, stream=qt).reshape(n_vec, in_stride)
+        outs = np.full((n_vec, out_stride), -1.0, np.float32)
+        scratch = np.zeros(ref.oc_matvec_batch_scratch_bytes(cols), np.uint8)
+        ref.oc_matvec_quantized_batch(qt, w.ctypes.data, rows, cols, rb, xs.ctypes.data, in_stride,
+                                      outs.ctypes.data, out_stride, n_vec, temp.ctypes.data,
+                                      scratch.ctypes.data, scratch.nbytes)
+        api[name + "_batch_x"] = xs
+        api[name + "_batch_out_bits"] = outs.view(np.uint32).copy()
+    np.savez_compressed(os.path.join(HERE, "matvec_api.npz"), **api)
+
+    # ── full-size benchmark configuration 0 and friends: checksums ───────
+    big = {}
+    for name, qt, rows, cols in (("cfg0_q4k_4096x4096", Q4K, 4096, 4096),
+                                 ("down_q6k_4096x14336", Q6K, 4096, 14336),
+                                 ("ffn_q80_4864x896", Q80, 4864, 896)):
+        rb = synth.row_bytes(qt, cols)
+        w = synth.weights(qt, rows, cols, seed=0, stream=0)
+        x = synth.normal(cols, seed=0, stream=1000)
+        o = np.zeros(rows, np.float32)
+        temp = np.zeros(cols, np.float32)
+        ref.oc_matvec_quantized(qt, w.ctypes.data, rows, cols, rb, x.ctypes.data, o.ctypes.data,
+                                temp.ctypes.data)
+        nact = cols // synth.BLOCK_ELEMS[qt] * (34 if qt == Q80 else 292)
+        big[name + "_crc_w"] = np.array([zlib.crc32(w.tobytes())], np.uint32)
+        big[name + "_crc_x"] = np.array([zlib.crc32(x.tobytes())], np.uint32)
+        big[name + "_crc_act"] = np.array([zlib.crc32(temp.view(np.uint8)[:nact].tobytes())], np.uint32)
+        big[name + "_crc_out"] = np.array([zlib.crc32(o.tobytes())], np.uint32)
+        big[name + "_out"] = o.copy()
+    np.savez_compressed(os.path.join(HERE, "full_size.npz"), **big)
+    for f in sorted(os.listdir(HERE)):
+        if f.endswith(".npz"):
+            print(f, os.path.getsize(os.path.join(HERE, f)))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,117 @@
+"""CPU tests of the shipped library's C ABI and host logic (no GPU needed):
+every symbol include/oxhip.h declares is exported, the eligibility helpers
+agree with the oracle's restatement of the reference's rules, declines happen
+before any device work, and without a device the library fails loudly instead
+of computing anything."""
+import ctypes
+import os
+import re
+
+import numpy as np
+
+import oxlibs
+from oxidize_amd import _lib, synth
+from oxidize_amd import matvec as mv
+
+ROOT = oxlibs.ROOT
+
+
+def declared_functions():
+    text = open(os.path.join(ROOT, "include", "oxhip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    names = re.findall(r"\b((?:oxh|oc)_[a-z0-9_]+)\s*\(", text)
+    return sorted(set(names))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = _lib.lib()
+    names = declared_functions()
+    assert len(names) >= 40
+    for n in names:
+        assert hasattr(lib, n), "missing export: " + n
+    assert set(_lib.SIGNATURES) == set(names)
+
+
+def test_no_oracle_or_reference_symbols_in_the_product():
+    out = os.popen("nm -D --defined-only %s" % _lib.LIB_PATH).read()
+    assert "oxo_" not in out
+    needed = os.popen("readelf -d %s" % _lib.LIB_PATH).read()
+    assert "oxoracle" not in needed and "oxref" not in needed
+
+
+def test_shape_helpers_match_the_reference_rules():
+    lib = _lib.lib()
+    o = oxlibs.oracle()
+    for qt in (0, 1, 2, 7, 8, 12, 13, 14, 16, 25):
+        for cols in (0, 32, 96, 256, 896, 900, 2816, 4096, 14336):
+            want = o.oxo_act_kind(qt, cols) if qt in (7, 12, 13, 16) else 0
+            assert lib.oxh_act_kind(qt, cols) == want
+    assert lib.oxh_row_bytes(13, 4096) == 2304
+    assert lib.oxh_row_bytes(16, 14336) == 11760
+    assert lib.oxh_row_bytes(7, 896) == 952
+    assert lib.oxh_row_bytes(13, 896) == 0
+    assert lib.oxh_act_bytes(13, 4096) == 4672
+    assert lib.oxh_act_bytes(7, 896) == 952
+    for cols in (0, 31, 256, 896, 4096, 14336, 1 << 20, 3 << 20):
+        assert lib.oc_matvec_batch_scratch_bytes(cols) == o.oxo_matvec_batch_scratch_bytes(cols)
+
+
+def test_fused_switch_and_counters():
+    lib = _lib.lib()
+    assert lib.oc_matvec_fused_enabled() is True
+    lib.oc_matvec_set_fused(False)
+    assert lib.oc_matvec_fused_enabled() is False
+    lib.oc_matvec_set_fused(True)
+    lib.oc_matvec_fused_test_reset()
+    st = lib.oc_matvec_fused_test_stats()
+    assert (st.activation_quantizations, st.parallel_dispatches, st.fallback_calls) == (0, 0, 0)
+
+
+def test_declines_need_no_device():
+    x = synth.normal(4096, seed=1)
+    w = synth.weights(13, 2, 4096, seed=1)
+    out = np.full(2, 9.0, np.float32)
+    temp = np.zeros(4096, np.float32)
+    assert mv.matvec_quantized(13, w, 2, 896, 504, x, out, temp) == mv.DECLINED
+    assert mv.matvec_quantized(13, w, 2, 4096, 2320, x, out, temp) == mv.DECLINED
+    assert mv.matvec_quantized(2, w, 2, 4096, 8192, x, out, temp) == mv.DECLINED
+    assert b"declined" in _lib.lib().oxh_last_error()
+    assert np.all(out == 9.0)
+
+
+def test_without_a_device_the_library_reports_it():
+    """In a GPU-less container the compute entry points must return an error
+    (never a result): there is no CPU path behind them."""
+    lib = _lib.lib()
+    rc = lib.oxh_init(0)
+    if rc == 0:
+        return                                   # a GPU is present: covered by the gpu tests
+    assert rc == _lib.ERR_NO_DEVICE
+    assert b"no HIP device" in lib.oxh_last_error()
+    x = synth.normal(256, seed=1)
+    w = synth.weights(13, 4, 256, seed=1)
+    out = np.full(4, 9.0, np.float32)
+    temp = np.zeros(256, np.float32)
+    try:
+        mv.matvec_quantized(13, w, 4, 256, 144, x, out, temp)
+    except mv.OxhError as e:
+        assert e.status == _lib.ERR_NO_DEVICE
+    else:
+        raise AssertionError("expected an error without a device")
+    assert np.all(out == 9.0)
+
+
+def test_synthetic_generator_is_deterministic():
+    a = synth.weights(13, 64, 1024, seed=5, stream=2)
+    b = synth.weights(13, 64, 1024, seed=5, stream=2)
+    c = synth.weights(13, 64, 1024, seed=6, stream=2)
+    assert np.array_equal(a, b) and not np.array_equal(a, c)
+    blk = a.reshape(-1, 144)
+    d = blk[:, :2].copy().view(np.float16).astype(np.float32)
+    assert np.all(np.isfinite(d)) and np.all(d >= 0) and 0.012 < d.mean() < 0.020
+    x = synth.normal(1 << 16, seed=0)
+    assert abs(float(x.mean())) < 0.02 and abs(float(x.std()) - 1.0) < 0.02
+    q = synth.weights(7, 16, 896, seed=1).reshape(-1, 34)[:, 2:].copy().view(np.int8)
+    assert q.min() >= -127 and q.max() <= 127
+    s6 = synth.weights(16, 4, 512, seed=1).reshape(-1, 210)[:, 192:208].copy().view(np.int8)
+    assert s6.min() >= -32 and s6.max() <= 31

@@ -1,0 +1,372 @@
+"""CPU tests that pin the oracle (oracle/liboxoracle.so):
+
+  * against the golden vectors taken from the compiled reference
+    (tests/golden/*.npz, made by tests/golden/make_golden.py),
+  * against the known-answer tests the reference's own suite holds
+    (oxidize-c/tests/test_oxk.c, test_oxk_extended.c, test_quant.c),
+  * against what the mathematics fixes: closed forms, a dequantised
+    double-precision dot product, invariants of the activation format,
+  * and, when oracle/_ref/liboxref.so is present, against the live reference.
+"""
+import ctypes
+import os
+import zlib
+
+import numpy as np
+import pytest
+
+import oxlibs
+from oxidize_amd import synth
+
+GOLD = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+Q80, Q4K, Q6K = 7, 13, 16
+O = oxlibs.oracle()
+
+
+def load(name):
+    return np.load(os.path.join(GOLD, name))
+
+
+def f32bits(x):
+    return np.float32(x).view(np.uint32)
+
+
+def f16_le(v):
+    b = np.float16(v).view(np.uint16)
+    return [int(b) & 255, int(b) >> 8]
+
+
+# ─── scalar helpers ─────────────────────────────────────────────────────
+
+def test_f16_to_f32_all_values_vs_reference_and_numpy():
+    g = load("scalar_helpers.npz")
+    mine = np.array([f32bits(O.oxo_f16_to_f32(i)) for i in range(65536)], dtype=np.uint32)
+    assert np.array_equal(mine, g["f16_to_f32_bits"])
+    h = np.arange(65536, dtype=np.uint16).view(np.float16)
+    finite = np.isfinite(h)
+    assert np.array_equal(mine[finite], h[finite].astype(np.float32).view(np.uint32))
+
+
+@pytest.mark.parametrize("lo,hi,value", [(0, 0, 0.0), (0x00, 0x3C, 1.0), (0x00, 0xBC, -1.0),
+                                         (0x00, 0x38, 0.5), (0x00, 0x40, 2.0), (0x00, 0x64, 1024.0)])
+def test_f16_known_answers(lo, hi, value):
+    # oxidize-c/tests/test_oxk.c:8-47
+    assert O.oxo_f16_to_f32(lo | (hi << 8)) == value
+
+
+def test_f32_to_f16_half_up_vs_reference():
+    g = load("scalar_helpers.npz")
+    mine = np.array([O.oxo_f32_to_f16_bits(float(v)) for v in g["f32_in"]], dtype=np.uint16)
+    assert np.array_equal(mine, g["f32_to_f16_bits"])
+
+
+def test_f32_to_f16_is_half_up_not_nearest_even():
+    # 1 + 2^-11 is an exact tie between 0x3C00 and 0x3C01: RNE keeps the even
+    # 0x3C00, the reference's rule goes up.
+    tie = np.uint32(0x3F801000).view(np.float32)
+    assert O.oxo_f32_to_f16_bits(float(tie)) == 0x3C01
+    assert np.float32(tie).astype(np.float16).view(np.uint16) == 0x3C00
+    assert O.oxo_f32_to_f16_bits(65520.0) == 0x7C00          # carries into inf
+    assert O.oxo_f32_to_f16_bits(2.9802322e-8) == 0x0001     # half the smallest subnormal rounds up
+    assert O.oxo_f32_to_f16_bits(2.9e-8) == 0x0000
+
+
+def test_scale_min_k4_known_answers_and_golden():
+    # oxidize-c/tests/test_oxk.c:72-103
+    sc, mn = ctypes.c_uint8(), ctypes.c_uint8()
+    s = (ctypes.c_uint8 * 12)()
+    s[0], s[4] = 42, 17
+    O.oxo_scale_min_k4(0, s, ctypes.byref(sc), ctypes.byref(mn))
+    assert (sc.value, mn.value) == (42, 17)
+    s = (ctypes.c_uint8 * 12)()
+    s[0], s[4], s[8] = 0xC0, 0x80, 0x9A
+    O.oxo_scale_min_k4(4, s, ctypes.byref(sc), ctypes.byref(mn))
+    assert (sc.value, mn.value) == (0x0A | (3 << 4), 0x09 | (2 << 4))
+    g = load("scalar_helpers.npz")
+    for i in range(g["k4_scales"].shape[0]):
+        row = np.ascontiguousarray(g["k4_scales"][i])
+        for j in range(8):
+            O.oxo_scale_min_k4(j, row.ctypes.data, ctypes.byref(sc), ctypes.byref(mn))
+            assert (sc.value, mn.value) == tuple(g["k4_sc_min"][i, j])
+
+
+# ─── activation quantisers ──────────────────────────────────────────────
+
+def numpy_q8(x, group):
+    """Independent numpy statement of d = amax/127, q = rint(x * (1/d))."""
+    x = x.reshape(-1, group).astype(np.float32)
+    amax = np.abs(x).max(axis=1)
+    d = (amax / np.float32(127.0)).astype(np.float32)
+    with np.errstate(divide="ignore"):
+        inv = np.where(d != 0, np.float32(1.0) / d, np.float32(0.0)).astype(np.float32)
+    q = np.clip(np.rint((x * inv[:, None]).astype(np.float32)), -128, 127).astype(np.int8)
+    return d, q
+
+
+def test_quantize_q8_k_against_numpy_and_invariants():
+    cols = 4096
+    x = synth.normal(cols, seed=0, stream=1000)
+    x[256:512] = 0.0
+    out = np.zeros(cols // 256 * 292, np.uint8)
+    O.oxo_quantize_q8_k(x.ctypes.data, cols, out.ctypes.data)
+    blk = out.reshape(-1, 292)
+    d, q = numpy_q8(x, 256)
+    assert np.array_equal(blk[:, :4].copy().view(np.float32).ravel(), d)
+    assert np.array_equal(blk[:, 4:260].copy().view(np.int8), q)
+    bs = blk[:, 260:].copy().view(np.int16)
+    assert np.array_equal(bs, q.reshape(-1, 16, 16).sum(axis=2).astype(np.int16))
+    assert np.all(blk[1] == 0)                       # all-zero block
+    assert np.abs(q).max() == 127
+
+
+def test_quantize_q8_0_against_numpy():
+    cols = 896
+    x = synth.normal(cols, seed=0, stream=1000)
+    out = np.zeros(cols // 32 * 34, np.uint8)
+    O.oxo_quantize_q8_0(x.ctypes.data, cols, out.ctypes.data)
+    blk = out.reshape(-1, 34)
+    d, q = numpy_q8(x, 32)
+    assert np.array_equal(blk[:, 2:].copy().view(np.int8), q)
+    want = np.array([O.oxo_f32_to_f16_bits(float(v)) for v in d], dtype=np.uint16)
+    assert np.array_equal(blk[:, :2].copy().view(np.uint16).ravel(), want)
+
+
+# ─── block dots ─────────────────────────────────────────────────────────
+
+def dot(name, w, blocks, act, extra=None):
+    w = np.ascontiguousarray(w)
+    act = np.ascontiguousarray(act)
+    if name == "q4_k":
+        return O.oxo_dot_q4_k_q8_k(w.ctypes.data, blocks, act.ctypes.data, extra, None)
+    if name == "q6_k":
+        return O.oxo_dot_q6_k_q8_k(w.ctypes.data, blocks, act.ctypes.data, extra)
+    return O.oxo_dot_q8_0_q8_0(w.ctypes.data, blocks, act.ctypes.data, extra)
+
+
+@pytest.mark.parametrize("name", ["q4_k", "q6_k", "q8_0"])
+def test_raw_block_dots_float_bits_vs_reference(name):
+    g = load("raw_block_dots.npz")
+    w, act = g[name + "_w"], g[name + "_act"]
+    for t in range(w.shape[0]):
+        for k, blocks in enumerate((1, w.shape[1])):
+            got = f32bits(dot(name, w[t], blocks, act[t]))
+            assert got == g[name + "_scalar_bits"][t, k]
+            assert got == g[name + "_dispatched_bits"][t, k]
+
+
+def test_known_answer_dots():
+    # Q8_0 ones -> 32, twos*threes -> 192 (oxidize-c/tests/test_oxk.c:105-133)
+    w = np.array([0x00, 0x3C] + [1] * 32, np.uint8)
+    assert dot("q8_0", w, 1, w) == 32.0
+    w2 = np.array([0x00, 0x3C] + [2] * 32, np.uint8)
+    a3 = np.array([0x00, 0x3C] + [3] * 32, np.uint8)
+    assert dot("q8_0", w2, 1, a3) == 192.0
+    # all-zero K blocks -> 0 (oxidize-c/tests/test_oxk_extended.c:213-270)
+    assert dot("q4_k", np.zeros(144, np.uint8), 1, np.zeros(292, np.uint8)) == 0.0
+    assert dot("q6_k", np.zeros(210, np.uint8), 1, np.zeros(292, np.uint8)) == 0.0
+
+
+def q8k_block(d, q):
+    blk = np.zeros(292, np.uint8)
+    blk[:4] = np.array([d], np.float32).view(np.uint8)
+    blk[4:260] = np.asarray(q, np.int8).view(np.uint8)
+    blk[260:] = np.asarray(q, np.int8).reshape(16, 16).sum(axis=1).astype(np.int16).view(np.uint8)
+    return blk
+
+
+def q4k_block(d, dmin, sc, mn, nib):
+    blk = np.zeros(144, np.uint8)
+    blk[0:2], blk[2:4] = f16_le(d), f16_le(dmin)
+    for j in range(4):
+        blk[4 + j] = sc[j] | ((sc[j + 4] >> 4) << 6)
+        blk[8 + j] = mn[j] | ((mn[j + 4] >> 4) << 6)
+        blk[12 + j] = (sc[j + 4] & 15) | ((mn[j + 4] & 15) << 4)
+    nib = np.asarray(nib, np.uint8).reshape(4, 2, 32)      # [gp][low/high][l]
+    blk[16:] = (nib[:, 0, :] | (nib[:, 1, :] << 4)).ravel()
+    return blk
+
+
+def test_q4_k_closed_form():
+    # all nibbles n, all scales s, all mins m, all activations a:
+    # dq*(d*256*s*n*a) - dq*(dmin*256*m*a), every factor exact in f32
+    d, dmin, dq, s, m, n, a = 0.5, 0.25, 0.125, 3, 5, 7, 2
+    w = q4k_block(d, dmin, [s] * 8, [m] * 8, [n] * 256)
+    act = q8k_block(dq, [a] * 256)
+    assert dot("q4_k", w, 1, act) == dq * d * 256 * s * n * a - dq * dmin * 256 * m * a
+
+
+def test_q4_k_each_sub_block_uses_its_own_scale_and_nibble_half():
+    # one-hot: only sub-block j has a non-zero scale -> result isolates S_j
+    rng = np.random.default_rng(5)
+    nib = rng.integers(0, 16, 256)
+    q = rng.integers(-127, 128, 256)
+    act = q8k_block(1.0, q)
+    for j in range(8):
+        sc = [0] * 8
+        sc[j] = 1
+        w = q4k_block(1.0, 0.0, sc, [0] * 8, nib)
+        want = int(np.dot(nib[32 * j:32 * j + 32], q[32 * j:32 * j + 32]))
+        sub = np.zeros(8, np.int32)
+        got = dot("q4_k", w, 1, act, sub.ctypes.data)
+        assert got == float(want)
+        assert sub[j] == want
+    # and the min term alone: scales 0, min j = 1 -> -dmin * sum(q over sub-block j)
+    for j in range(8):
+        mn = [0] * 8
+        mn[j] = 1
+        w = q4k_block(1.0, 1.0, [0] * 8, mn, nib)
+        assert dot("q4_k", w, 1, act) == -float(q[32 * j:32 * j + 32].sum())
+
+
+def test_q6_k_codes_zero_give_minus_32_times_scale_sum():
+    # all codes 0 -> every weight is d*sc*(-32)  (oxidize-c/tests/test_quant.c:290-310)
+    blk = np.zeros(210, np.uint8)
+    blk[192:208] = np.arange(1, 17, dtype=np.int8).view(np.uint8)
+    blk[208:210] = f16_le(1.0)
+    q = np.arange(256) % 7 - 3
+    act = q8k_block(1.0, q)
+    want = sum(-32 * (g + 1) * int(q[16 * g:16 * g + 16].sum()) for g in range(16))
+    assert dot("q6_k", blk, 1, act) == float(want)
+
+
+@pytest.mark.parametrize("name,qt,group", [("q4_k", Q4K, 256), ("q6_k", Q6K, 256), ("q8_0", Q80, 32)])
+def test_dot_agrees_with_dequantised_double_precision(name, qt, group):
+    """Kernel-vs-layout check of oxidize-c/tests/test_oxk_gguf_layout.c:104-141:
+    dot the dequantised weights with the dequantised activation in double."""
+    cols = 2048
+    w = synth.weights(qt, 1, cols, seed=9, stream=qt)
+    x = synth.normal(cols, seed=9)
+    wf = np.zeros(cols, np.float32)
+    assert O.oxo_dequant_row(qt, w.ctypes.data, cols, wf.ctypes.data) == 0
+    if qt == Q80:
+        act = np.zeros(cols // 32 * 34, np.uint8)
+        O.oxo_quantize_q8_0(x.ctypes.data, cols, act.ctypes.data)
+        b = act.reshape(-1, 34)
+        dq = b[:, :2].copy().view(np.float16).astype(np.float64)
+        xq = b[:, 2:].copy().view(np.int8).astype(np.float64) * dq
+    else:
+        act = np.zeros(cols // 256 * 292, np.uint8)
+        O.oxo_quantize_q8_k(x.ctypes.data, cols, act.ctypes.data)
+        b = act.reshape(-1, 292)
+        dq = b[:, :4].copy().view(np.float32).astype(np.float64)
+        xq = b[:, 4:260].copy().view(np.int8).astype(np.float64) * dq
+    want = float(np.dot(wf.astype(np.float64), xq.ravel()))
+    got = dot(name, w, cols // group, act)
+    scale = float(np.abs(wf.astype(np.float64) * xq.ravel()).sum())
+    assert abs(got - want) <= 1e-6 * scale
+
+
+def test_every_weight_byte_influences_the_dot():
+    # oxidize-c/tests/test_quant.c:569-583, applied to the dot kernels
+    rng = np.random.default_rng(3)
+    for name, qt, size in (("q4_k", Q4K, 144), ("q6_k", Q6K, 210), ("q8_0", Q80, 34)):
+        group = 32 if qt == Q80 else 256
+        w = synth.weights(qt, 1, group, seed=13, stream=qt)
+        if qt == Q80:
+            act = np.concatenate([np.array(f16_le(0.5), np.uint8),
+                                  rng.integers(1, 100, 32).astype(np.uint8)])
+        else:
+            act = q8k_block(0.5, rng.integers(1, 100, 256))
+        base = f32bits(dot(name, w, 1, act))
+        for i in range(size):
+            w2 = w.copy()
+            w2[i] ^= 0x15 if qt != Q80 or i >= 2 else 0x04
+            assert f32bits(dot(name, w2, 1, act)) != base, "%s byte %d" % (name, i)
+
+
+# ─── API level ──────────────────────────────────────────────────────────
+
+@pytest.mark.parametrize("name,qt", [("q4_k", Q4K), ("q6_k", Q6K), ("q8_0", Q80)])
+def test_matvec_and_batch_vs_reference_goldens(name, qt):
+    g = load("matvec_api.npz")
+    rows, cols, rb = (int(v) for v in g[name + "_shape"])
+    w, x = g[name + "_w"], g[name + "_x"]
+    out = np.zeros(rows, np.float32)
+    temp = np.zeros(cols, np.float32)
+    assert O.oxo_matvec_quantized(qt, w.ctypes.data, rows, cols, rb, x.ctypes.data,
+                                  out.ctypes.data, temp.ctypes.data) == 0
+    act = g[name + "_act"]
+    assert np.array_equal(temp.view(np.uint8)[:act.size], act)
+    ref_out = g[name + "_out_bits"].view(np.float32)
+    if qt == Q80:   # the reference's decode kernel reassociates the f32 sum
+        assert np.all(np.abs(out - ref_out) <= 1e-4 + 1e-5 * np.abs(ref_out))
+    else:
+        assert np.array_equal(out.view(np.uint32), g[name + "_out_bits"])
+    xs = g[name + "_batch_x"]
+    n_vec, in_stride = xs.shape
+    want = g[name + "_batch_out_bits"].view(np.float32)
+    out_stride = want.shape[1]
+    outs = np.full((n_vec, out_stride), -1.0, np.float32)
+    scratch = np.zeros(O.oxo_matvec_batch_scratch_bytes(cols), np.uint8)
+    assert O.oxo_matvec_quantized_batch(qt, w.ctypes.data, rows, cols, rb, xs.ctypes.data, in_stride,
+                                        outs.ctypes.data, out_stride, n_vec, scratch.ctypes.data,
+                                        scratch.nbytes) == 0
+    if qt == Q80:
+        assert np.all(np.abs(outs - want) <= 1e-4 + 1e-5 * np.abs(want))
+    else:
+        assert np.array_equal(outs.view(np.uint32), want.view(np.uint32))
+    assert np.all(outs[:, rows:] == -1.0)
+
+
+@pytest.mark.parametrize("name,qt,rows,cols", [("cfg0_q4k_4096x4096", Q4K, 4096, 4096),
+                                               ("down_q6k_4096x14336", Q6K, 4096, 14336),
+                                               ("ffn_q80_4864x896", Q80, 4864, 896)])
+def test_full_size_configs_vs_reference_checksums(name, qt, rows, cols):
+    g = load("full_size.npz")
+    w = synth.weights(qt, rows, cols, seed=0, stream=0)
+    x = synth.normal(cols, seed=0, stream=1000)
+    assert zlib.crc32(w.tobytes()) == int(g[name + "_crc_w"][0])      # generator is stable
+    assert zlib.crc32(x.tobytes()) == int(g[name + "_crc_x"][0])
+    out = np.zeros(rows, np.float32)
+    temp = np.zeros(cols, np.float32)
+    assert O.oxo_matvec_quantized(qt, w.ctypes.data, rows, cols, synth.row_bytes(qt, cols),
+                                  x.ctypes.data, out.ctypes.data, temp.ctypes.data) == 0
+    nact = cols // synth.BLOCK_ELEMS[qt] * (34 if qt == Q80 else 292)
+    assert zlib.crc32(temp.view(np.uint8)[:nact].tobytes()) == int(g[name + "_crc_act"][0])
+    if qt == Q80:
+        assert np.all(np.abs(out - g[name + "_out"]) <= 1e-4 + 1e-5 * np.abs(g[name + "_out"]))
+    else:
+        assert zlib.crc32(out.tobytes()) == int(g[name + "_crc_out"][0])
+
+
+def test_eligibility_rules():
+    # oxidize-c/src/compute/matvec.c:99-127, :961-985
+    assert O.oxo_act_kind(Q4K, 4096) == 2 and O.oxo_act_kind(Q4K, 896) == 0
+    assert O.oxo_act_kind(Q6K, 256) == 2 and O.oxo_act_kind(12, 512) == 2
+    assert O.oxo_act_kind(Q80, 896) == 1 and O.oxo_act_kind(Q80, 900) == 0
+    assert O.oxo_act_kind(0, 4096) == 0 and O.oxo_act_kind(1, 4096) == 0
+    assert O.oxo_stride_ok(Q4K, 4096, 2304) == 1 and O.oxo_stride_ok(Q4K, 4096, 2320) == 0
+    assert O.oxo_stride_ok(Q6K, 14336, 11760) == 1 and O.oxo_stride_ok(Q80, 896, 952) == 1
+    assert O.oxo_matvec_batch_scratch_bytes(4096) == 4 << 20
+
+
+def test_moe_route_brute_force():
+    """Top-2 of 8 by softmax probability (oxidize-c/src/model/llama.c:5965-6031):
+    selection is order-only, so it must equal a stable descending sort."""
+    logits = synth.normal(16 * 8, seed=0, stream=4242).reshape(16, 8)
+    ids = np.zeros((16, 2), np.int32)
+    wts = np.zeros((16, 2), np.float32)
+    O.oxo_moe_route(logits.ctypes.data, 16, 8, 2, 1, ids.ctypes.data, wts.ctypes.data)
+    for t in range(16):
+        order = np.argsort(-logits[t], kind="stable")[:2]
+        assert list(ids[t]) == list(order)
+        p = np.exp(logits[t].astype(np.float64) - logits[t].max())
+        p /= p.sum()
+        assert np.allclose(wts[t], p[order] / p[order].sum(), rtol=1e-5)
+        assert abs(wts[t].sum() - 1.0) < 1e-6
+
+
+@pytest.mark.skipif(oxlibs.ref() is None, reason="compiled reference not present")
+def test_oracle_vs_live_reference_many_rows():
+    ref = oxlibs.ref()
+    ref.oc_parallel_set_threads(2)
+    for qt, rows, cols in ((Q4K, 700, 4096), (Q6K, 300, 14336), (Q4K, 513, 2816), (Q6K, 64, 256)):
+        rb = synth.row_bytes(qt, cols)
+        w = synth.weights(qt, rows, cols, seed=77, stream=rows)
+        x = synth.normal(cols, seed=77)
+        a, b = np.zeros(rows, np.float32), np.zeros(rows, np.float32)
+        ta, tb = np.zeros(cols, np.float32), np.zeros(cols, np.float32)
+        O.oxo_matvec_quantized(qt, w.ctypes.data, rows, cols, rb, x.ctypes.data, a.ctypes.data, ta.ctypes.data)
+        ref.oc_matvec_quantized(qt, w.ctypes.data, rows, cols, rb, x.ctypes.data, b.ctypes.data, tb.ctypes.data)
+        assert np.array_equal(a.view(np.uint32), b.view(np.uint32))
+        assert np.array_equal(ta.view(np.uint8), tb.view(np.uint8))
