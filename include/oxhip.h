@@ -107,6 +107,18 @@ int oxh_gemv_segments(uint32_t qtype, const OxhSegment *segs, size_t n_segs,
                       size_t cols, const void *d_acts, size_t n_vec,
                       size_t out_stride, void *stream);
 
+/* Same launch with the activation quantisation fused into the kernel: d_x
+ * holds the f32 input vectors (`x_stride` floats apart, indexed like d_acts),
+ * every workgroup quantises the vectors of its segment straight into LDS —
+ * one kernel per decode matmul instead of two, which is what
+ * oc_matvec_quantized does in one call (matvec.c:860-881).  When d_act_out is
+ * not NULL the quantised bytes are also stored there (reference format,
+ * oxh_act_bytes() per vector). */
+int oxh_gemv_segments_f32(uint32_t qtype, const OxhSegment *segs, size_t n_segs,
+                          size_t cols, const float *d_x, size_t x_stride,
+                          void *d_act_out, size_t n_vec, size_t out_stride,
+                          void *stream);
+
 /* Prefill matmul on int8 MFMA: out[v*out_stride + r] = dot(W[r], act[v]) for
  * v < n_vec (any count), Q8_K activations.  Replaces the prepared-row batch
  * kernels oc_oxk_q4_k_prep_row + oc_oxk_dot_q4_k_prepped_multi

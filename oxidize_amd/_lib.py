@@ -38,6 +38,7 @@ SIGNATURES = {
     "oxh_quantize_q8_k": (I, [V, Z, Z, Z, V, V]),
     "oxh_quantize_q8_0": (I, [V, Z, Z, Z, V, V]),
     "oxh_gemv_segments": (I, [U32, ctypes.POINTER(OxhSegment), Z, Z, V, Z, Z, V]),
+    "oxh_gemv_segments_f32": (I, [U32, ctypes.POINTER(OxhSegment), Z, Z, V, Z, V, Z, Z, V]),
     "oxh_mmq": (I, [U32, V, Z, Z, V, Z, V, Z, V]),
     "oxh_debug_subblock_sums": (I, [U32, V, Z, Z, V, V, V]),
     "oxh_malloc": (I, [ctypes.POINTER(V), Z]),

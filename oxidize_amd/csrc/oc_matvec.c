@@ -274,9 +274,11 @@ int oxh_matvec_quantized(uint32_t qtype, const uint8_t *data, size_t rows,
     if ((rc = reserve(&g_dout, obytes))) return rc;
 
     if ((rc = oxh_memcpy_h2d(g_dx.p, input, cols * sizeof(float), NULL))) return rc;
-    if ((rc = quantize(kind, (const float *)g_dx.p, cols, 1, cols, g_dact.p))) return rc;
+    /* one launch: quantise the activation inside the GEMV kernel */
     OxhSegment seg = { d_w, (float *)g_dout.p, rows, 0 };
-    if ((rc = oxh_gemv_segments(qtype, &seg, 1, cols, g_dact.p, 1, rows, NULL))) return rc;
+    if ((rc = oxh_gemv_segments_f32(qtype, &seg, 1, cols, (const float *)g_dx.p, cols, g_dact.p, 1,
+                                    rows, NULL)))
+        return rc;
     if ((rc = oxh_memcpy_d2h(output, g_dout.p, obytes, NULL))) return rc;
     if ((rc = oxh_memcpy_d2h(temp, g_dact.p, abytes, NULL))) return rc;
     return oxh_stream_sync(NULL);
@@ -286,7 +288,7 @@ int oxh_matvec_quantized(uint32_t qtype, const uint8_t *data, size_t rows,
 
 /* Shared body: n_outs matrices of one eligible type.  `inputs` has either one
  * vector (shared) or n_outs vectors. */
-static int grouped(uint32_t qtype, int kind, const uint8_t *const *datas,
+static int grouped(uint32_t qtype, const uint8_t *const *datas,
                    const size_t *rows, size_t cols, const size_t *row_bytes,
                    size_t n_outs, const float *const *inputs, size_t n_inputs,
                    float *const *outs)
@@ -312,8 +314,6 @@ static int grouped(uint32_t qtype, int kind, const uint8_t *const *datas,
         if ((rc = oxh_memcpy_h2d((float *)g_dx.p + i * cols, inputs[i], cols * sizeof(float), NULL)))
             return rc;
     }
-    if ((rc = quantize(kind, (const float *)g_dx.p, cols, n_inputs, cols, g_dact.p))) return rc;
-
     enum { CHUNK = 32 };
     OxhSegment segs[CHUNK];
     size_t done_rows = 0;
@@ -334,7 +334,9 @@ static int grouped(uint32_t qtype, int kind, const uint8_t *const *datas,
             segs[i].act_first = n_inputs == 1 ? 0 : k;
             done_rows += rows[k];
         }
-        if ((rc = oxh_gemv_segments(qtype, segs, n, cols, g_dact.p, 1, 0, NULL))) return rc;
+        if ((rc = oxh_gemv_segments_f32(qtype, segs, n, cols, (const float *)g_dx.p, cols, NULL, 1, 0,
+                                        NULL)))
+            return rc;
     }
     size_t off = 0;
     for (size_t k = 0; k < n_outs; k++) {
@@ -367,8 +369,7 @@ int oxh_matvec_quantized_fused(const uint32_t *qtypes, const uint8_t *const *dat
         /* matvec.c:1571-1573 */
         g_stats.activation_quantizations++;
         g_stats.parallel_dispatches++;
-        return grouped(qtypes[0], oxh_act_kind(qtypes[0], cols), datas, rows, cols,
-                       row_bytes, n_outs, &input, 1, outs);
+        return grouped(qtypes[0], datas, rows, cols, row_bytes, n_outs, &input, 1, outs);
     }
     /* mixed types (or an all-empty group): one call per matrix, matvec.c:1579-1593 */
     if (temp == NULL) return declined("temp is NULL");
@@ -404,8 +405,7 @@ int oxh_matvec_quantized_multi_input(const uint32_t *qtypes, const uint8_t *cons
         /* matvec.c:1661-1662 */
         g_stats.activation_quantizations += n_outs;
         g_stats.parallel_dispatches++;
-        return grouped(qtypes[0], oxh_act_kind(qtypes[0], cols), datas, rows, cols,
-                       row_bytes, n_outs, inputs, n_outs, outs);
+        return grouped(qtypes[0], datas, rows, cols, row_bytes, n_outs, inputs, n_outs, outs);
     }
     if (temp == NULL) return declined("temp is NULL");
     for (size_t k = 0; k < n_outs; k++) {
@@ -465,12 +465,12 @@ int oxh_matvec_quantized_batch(uint32_t qtype, const uint8_t *data, size_t rows,
                                      cols * sizeof(float), NULL)))
                 return rc;
     }
-    if ((rc = quantize(kind, (const float *)g_dx.p, in_stride, n_vec, cols, g_dact.p))) return rc;
-
     /* More vectors than the GEMV kernel keeps in flight: Q4_K goes to the
-     * int8-MFMA kernel; the other types walk the batch in GEMV-sized slices
+     * int8-MFMA kernel behind a stand-alone quantiser launch; everything else
+     * walks the batch in GEMV-sized slices with the quantisation fused in
      * (every output is the same dot either way). */
     if (n_vec > 8 && (qtype == OXH_Q4_K_S || qtype == OXH_Q4_K_M)) {
+        if ((rc = quantize(kind, (const float *)g_dx.p, in_stride, n_vec, cols, g_dact.p))) return rc;
         if ((rc = oxh_mmq(qtype, d_w, rows, cols, g_dact.p, n_vec, (float *)g_dout.p, rows, NULL)))
             return rc;
     } else {
@@ -482,7 +482,9 @@ int oxh_matvec_quantized_batch(uint32_t qtype, const uint8_t *data, size_t rows,
         for (size_t v0 = 0; v0 < n_vec; v0 += step) {
             const size_t m = n_vec - v0 < step ? n_vec - v0 : step;
             OxhSegment seg = { d_w, (float *)g_dout.p + v0 * rows, rows, v0 };
-            if ((rc = oxh_gemv_segments(qtype, &seg, 1, cols, g_dact.p, m, rows, NULL))) return rc;
+            if ((rc = oxh_gemv_segments_f32(qtype, &seg, 1, cols, (const float *)g_dx.p, in_stride,
+                                            NULL, m, rows, NULL)))
+                return rc;
         }
     }
     if (out_stride == rows) {

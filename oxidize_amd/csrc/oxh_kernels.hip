@@ -21,6 +21,7 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 #include <stdio.h>
+#include <stdlib.h>
 #include <string.h>
 
 #include "oxhip.h"
@@ -78,6 +79,49 @@ __device__ __forceinline__ int quad_sum(int v)
     v += __builtin_amdgcn_update_dpp(0, v, 0xB1, 0xF, 0xF, false); /* lanes ^1 */
     v += __builtin_amdgcn_update_dpp(0, v, 0x4E, 0xF, 0xF, false); /* lanes ^2 */
     return v;
+}
+
+/* Maximum over the wave; every lane receives it.  Quad and row steps are DPP
+ * (xor 1, xor 2, mirror within 8, mirror within 16), the four row results
+ * are combined through scalar registers. */
+__device__ __forceinline__ float dpp_max_step(float v, const int ctrl_sel)
+{
+    int o;
+    switch (ctrl_sel) {
+    case 0:  o = __builtin_amdgcn_update_dpp(0, __float_as_int(v), 0xB1, 0xF, 0xF, false); break;
+    case 1:  o = __builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x4E, 0xF, 0xF, false); break;
+    case 2:  o = __builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x141, 0xF, 0xF, false); break;
+    default: o = __builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x140, 0xF, 0xF, false); break;
+    }
+    return fmaxf(v, __int_as_float(o));
+}
+
+/* max over each aligned group of 8 lanes */
+__device__ __forceinline__ float oct_max(float v)
+{
+    v = dpp_max_step(v, 0);
+    v = dpp_max_step(v, 1);
+    v = dpp_max_step(v, 2);
+    return v;
+}
+
+__device__ __forceinline__ float wave_max(float v)
+{
+    v = oct_max(v);
+    v = dpp_max_step(v, 3);
+    const int b = __float_as_int(v);
+    const float r0 = __int_as_float(__builtin_amdgcn_readlane(b, 0));
+    const float r1 = __int_as_float(__builtin_amdgcn_readlane(b, 16));
+    const float r2 = __int_as_float(__builtin_amdgcn_readlane(b, 32));
+    const float r3 = __int_as_float(__builtin_amdgcn_readlane(b, 48));
+    return fmaxf(fmaxf(r0, r1), fmaxf(r2, r3));
+}
+
+/* binary16 -> binary32 with the hardware converter (exact for every input,
+ * subnormals included: f16 denormals are never flushed on this target). */
+__device__ __forceinline__ float half_to_float_hw(uint32_t h)
+{
+    return (float)__builtin_bit_cast(_Float16, (uint16_t)h);
 }
 
 /* Exact binary16 -> binary32 including subnormals (integer-only so it does
@@ -215,552 +259,8 @@ k_quantize_q8_0(const float *__restrict__ x, size_t in_stride, uint32_t blocks_p
         *reinterpret_cast<uint16_t *>(dst) = (uint16_t)float_to_half_bits_half_up(d);
 }
 
-/* ─── decode GEMV ─────────────────────────────────────────────────────── */
-
-#define OXH_MAX_SEGS 32
-#define OXH_GEMV_WAVES 4          /* waves per workgroup */
-#define OXH_MAX_NV 8
-
-/* Bytes of LDS one staged Q8_K activation takes: 256 B of values, 16 B of
- * sub-block sums and 4 B of scale per block, rounded up so the next
- * activation's 16-byte vectors stay aligned. */
-__host__ __device__ static inline uint32_t q8k_lds_bytes(uint32_t blocks)
-{
-    return (blocks * (256u + 16u + 4u) + 15u) & ~15u;
-}
-
-/* Q6_K pairing: 256 B of values, 16 x int32 pre-scaled group sums, scale. */
-__host__ __device__ static inline uint32_t q8k6_lds_bytes(uint32_t blocks)
-{
-    return (blocks * (256u + 64u + 4u) + 15u) & ~15u;
-}
-
-/* Q8_0 activation: 32 B of values and the decoded f32 scale per block. */
-__host__ __device__ static inline uint32_t q80_lds_bytes(uint32_t blocks)
-{
-    return (blocks * (32u + 4u) + 15u) & ~15u;
-}
-
-struct SegTable {
-    const uint8_t *w[OXH_MAX_SEGS];
-    float *out[OXH_MAX_SEGS];
-    uint32_t rows[OXH_MAX_SEGS];
-    uint32_t act_first[OXH_MAX_SEGS];
-    uint32_t wg_begin[OXH_MAX_SEGS + 1];   /* first workgroup of each segment */
-    uint32_t n;
-};
-
-struct GemvParams {
-    uint32_t blocks;        /* weight blocks per row                        */
-    uint32_t magic;         /* ceil(2^32 / blocks), for g / blocks          */
-    uint32_t rows_per_wave; /* RW                                           */
-    uint32_t n_vec;         /* activations per segment (1..8)               */
-    uint32_t act_bytes;     /* bytes of one quantised activation            */
-    uint32_t out_stride;    /* floats between output vectors                */
-    uint32_t term_stride;   /* blocks + 1 (LDS row pitch of the term table) */
-    int32_t *dump;          /* debug: sub-block sums, or NULL               */
-};
-
-/* LDS layout for the Q8_K-activation kernels (per workgroup), in this order:
- *   per activation v: q  [4][blocks*4] x 16 B   values of (block, 64-span s),
- *                        quarter i, at ((i*blocks*4) + block*4 + s)
- *                     bs [blocks*4]   x 4 B    Q4_K: B_{2s} | B_{2s+1}<<16
- *                     dq [blocks]     x 4 B
- *   terms: [waves][n_vec][rows_per_wave][term_stride] f32
- * For Q6_K the q array is indexed by (block, unit u=(n,lh)), quarter k, and
- * bs holds 4 x int32 per unit (32*bsum of its 4 groups), see k_gemv_q6_k. */
-
-__device__ __forceinline__ uint32_t find_segment(const SegTable &t, uint32_t wg)
-{
-    uint32_t s = 0;
-    while (s + 1 < t.n && wg >= t.wg_begin[s + 1]) s++;
-    return s;
-}
-
-__device__ __forceinline__ void
-row_sums(const float *terms, uint32_t lane, uint32_t NV, uint32_t nrows, uint32_t RW,
-         uint32_t B, uint32_t term_stride, float *out, uint32_t out_stride, uint32_t row0);
-
-/* Q4_K x Q8_K.  Four lanes per super-block: lane (b, s) owns nibble bytes
- * [32s, 32s+32) of block b, i.e. sub-blocks 2s (low nibbles) and 2s+1 (high
- * nibbles), elements [64s, 64s+64).  16 blocks = 2304 contiguous bytes per
- * wave pass. */
-template <bool DUMP>
-__global__ __launch_bounds__(OXH_GEMV_WAVES * 64) void
-k_gemv_q4_k(const SegTable segs, const GemvParams p, const uint8_t *__restrict__ acts)
-{
-    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
-    const uint32_t tid = threadIdx.x;
-    const uint32_t lane = tid & 63u;
-    const uint32_t wave = tid >> 6;
-    const uint32_t B = p.blocks;
-    const uint32_t NV = p.n_vec;
-
-    const uint32_t seg = find_segment(segs, blockIdx.x);
-    const uint32_t wg_in_seg = blockIdx.x - segs.wg_begin[seg];
-    const uint32_t seg_rows = segs.rows[seg];
-
-    const uint32_t act_lds = q8k_lds_bytes(B);               /* per activation */
-    float *const terms = reinterpret_cast<float *>(lds + (size_t)act_lds * NV) +
-                         (size_t)wave * NV * p.rows_per_wave * p.term_stride;
-
-    /* stage the segment's activations */
-    for (uint32_t v = 0; v < NV; v++) {
-        const uint8_t *a = acts + (size_t)(segs.act_first[seg] + v) * p.act_bytes;
-        uint8_t *base = lds + (size_t)v * act_lds;
-        uint32_t *qd = reinterpret_cast<uint32_t *>(base);
-        uint32_t *bs = reinterpret_cast<uint32_t *>(base + B * 256u);
-        float *dq = reinterpret_cast<float *>(base + B * 256u + B * 16u);
-        for (uint32_t j = tid; j < B * 64u; j += OXH_GEMV_WAVES * 64u) {
-            const uint32_t blk = j >> 6, w = j & 63u;
-            const uint32_t c = w >> 2, s = c >> 2, i = c & 3u;
-            const uint32_t val = *reinterpret_cast<const uint32_t *>(a + (size_t)blk * 292u + 4u + 4u * w);
-            qd[((i * B * 4u) + blk * 4u + s) * 4u + (w & 3u)] = val;
-        }
-        for (uint32_t j = tid; j < B * 4u; j += OXH_GEMV_WAVES * 64u) {
-            const uint32_t blk = j >> 2, s = j & 3u;
-            const uint32_t *sp = reinterpret_cast<const uint32_t *>(a + (size_t)blk * 292u + 260u) + 2u * s;
-            const uint32_t p0 = sp[0], p1 = sp[1];
-            const int b0 = (int)(int16_t)(p0 & 0xFFFFu) + (int)(int16_t)(p0 >> 16);
-            const int b1 = (int)(int16_t)(p1 & 0xFFFFu) + (int)(int16_t)(p1 >> 16);
-            bs[j] = ((uint32_t)b0 & 0xFFFFu) | ((uint32_t)b1 << 16);
-        }
-        for (uint32_t j = tid; j < B; j += OXH_GEMV_WAVES * 64u)
-            dq[j] = *reinterpret_cast<const float *>(a + (size_t)j * 292u);
-    }
-    __syncthreads();
-
-    const uint32_t RW = p.rows_per_wave;
-    const uint32_t row0 = (wg_in_seg * OXH_GEMV_WAVES + wave) * RW;
-    if (row0 >= seg_rows) return;
-    const uint32_t nrows = min(RW, seg_rows - row0);
-    const uint32_t nblk = nrows * B;
-    const uint32_t s = lane & 3u;
-    const bool hi = s >= 2u;
-    const uint32_t sh = (s & 1u) * 16u;
-    const uint32_t mask_a = hi ? 0x0F0F0F0Fu : 0x3F3F3F3Fu;
-    const uint32_t mask_b = hi ? 0x30303030u : 0u;
-
-    const uint8_t *wbase = segs.w[seg] + (size_t)row0 * B * 144u;
-
-    for (uint32_t g0 = 0; g0 < nblk; g0 += 16u) {
-        const uint32_t g = g0 + (lane >> 2);
-        const bool live = g < nblk;
-        const uint32_t gc = live ? g : 0u;
-        const uint32_t r = (B == 1u) ? gc : __umulhi(gc, p.magic);
-        const uint32_t blk = gc - r * B;
-        const uint8_t *wb = wbase + (size_t)gc * 144u;
-        const u32x4 hdr = *reinterpret_cast<const u32x4 *>(wb);
-        const u32x4 na = *reinterpret_cast<const u32x4 *>(wb + 16u + 32u * s);
-        const u32x4 nb = *reinterpret_cast<const u32x4 *>(wb + 32u + 32u * s);
-
-        /* 6-bit scale/min unpack for this lane's two sub-blocks */
-        const uint32_t u0 = hdr.y, u1 = hdr.z, u2 = hdr.w;
-        const uint32_t scw = ((hi ? u2 : u0) & mask_a) | ((u0 >> 2) & mask_b);
-        const uint32_t mnw = ((hi ? (u2 >> 4) : u1) & mask_a) | ((u1 >> 2) & mask_b);
-        const int sc_a = (int)((scw >> sh) & 0xFFu), sc_b = (int)((scw >> (sh + 8u)) & 0xFFu);
-        const int mn_a = (int)((mnw >> sh) & 0xFFu), mn_b = (int)((mnw >> (sh + 8u)) & 0xFFu);
-        const float dw = half_bits_to_float(hdr.x & 0xFFFFu);
-        const float dmin = half_bits_to_float(hdr.x >> 16);
-
-        const uint32_t slot = blk * 4u + s;
-        for (uint32_t v = 0; v < NV; v++) {
-            const uint8_t *base = lds + (size_t)v * act_lds;
-            const u32x4 *qv = reinterpret_cast<const u32x4 *>(base);
-            const u32x4 a0 = qv[slot], a1 = qv[B * 4u + slot];
-            const u32x4 a2 = qv[B * 8u + slot], a3 = qv[B * 12u + slot];
-            const uint32_t bsp = reinterpret_cast<const uint32_t *>(base + B * 256u)[slot];
-            const float dq = reinterpret_cast<const float *>(base + B * 256u + B * 16u)[blk];
-
-            int s_lo = 0, s_hi = 0;
-#pragma unroll
-            for (int k = 0; k < 4; k++) {
-                s_lo = dot4(na[k] & 0x0F0F0F0Fu, a0[k], s_lo);
-                s_lo = dot4(nb[k] & 0x0F0F0F0Fu, a1[k], s_lo);
-                s_hi = dot4((na[k] >> 4) & 0x0F0F0F0Fu, a2[k], s_hi);
-                s_hi = dot4((nb[k] >> 4) & 0x0F0F0F0Fu, a3[k], s_hi);
-            }
-            if (DUMP) {
-                if (live) {
-                    int32_t *o = p.dump + ((size_t)(row0 * B + gc)) * 8u + 2u * s;
-                    o[0] = s_lo;
-                    o[1] = s_hi;
-                }
-            }
-            int pos = sc_a * s_lo + sc_b * s_hi;
-            int mn = mn_a * (int)(int16_t)(bsp & 0xFFFFu) + mn_b * ((int)bsp >> 16);
-            pos = quad_sum(pos);
-            mn = quad_sum(mn);
-            const float t_pos = dw * dq;
-            const float t_min = dmin * dq;
-            const float up = t_pos * (float)pos;
-            const float dn = t_min * (float)mn;
-            if (live && s == 0u)
-                terms[((size_t)v * RW + r) * p.term_stride + blk] = up - dn;
-        }
-    }
-
-    row_sums(terms, lane, NV, nrows, RW, B, p.term_stride, segs.out[seg], p.out_stride, row0);
-}
-
-/* Shared tail: strictly sequential per-row sums, one lane per (vector, row). */
-__device__ __forceinline__ void
-row_sums(const float *terms, uint32_t lane, uint32_t NV, uint32_t nrows, uint32_t RW,
-         uint32_t B, uint32_t term_stride, float *out, uint32_t out_stride, uint32_t row0)
-{
-    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
-    for (uint32_t idx = lane; idx < NV * nrows; idx += 64u) {
-        const uint32_t v = idx / nrows, r = idx - v * nrows;
-        const float *t = terms + ((size_t)v * RW + r) * term_stride;
-        float sum = 0.0f;
-        for (uint32_t b = 0; b < B; b++) sum += t[b];
-        out[(size_t)v * out_stride + row0 + r] = sum;
-    }
-}
-
-/* Q6_K x Q8_K.  Four lanes per super-block: lane (b, u) with u = 2n + lh owns
- * the 64 weights e = 128n + 32k + 16lh + i (k < 4, i < 16): 16 bytes of ql at
- * 64n+16lh (low nibbles -> k=0, high -> k=2), 16 bytes at 64n+32+16lh (k=1,
- * k=3) and 16 bytes of qh at 32n+16lh (two bits per k).  Each k is one
- * 16-weight scale group g = 8n + 2k + lh.  Blocks are 210 bytes, so every
- * load here is only 2-byte aligned. */
-template <bool DUMP>
-__global__ __launch_bounds__(OXH_GEMV_WAVES * 64) void
-k_gemv_q6_k(const SegTable segs, const GemvParams p, const uint8_t *__restrict__ acts)
-{
-    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
-    const uint32_t tid = threadIdx.x;
-    const uint32_t lane = tid & 63u;
-    const uint32_t wave = tid >> 6;
-    const uint32_t B = p.blocks;
-    const uint32_t NV = p.n_vec;
-
-    const uint32_t seg = find_segment(segs, blockIdx.x);
-    const uint32_t wg_in_seg = blockIdx.x - segs.wg_begin[seg];
-    const uint32_t seg_rows = segs.rows[seg];
-
-    const uint32_t act_lds = q8k6_lds_bytes(B);
-    float *const terms = reinterpret_cast<float *>(lds + (size_t)act_lds * NV) +
-                         (size_t)wave * NV * p.rows_per_wave * p.term_stride;
-
-    for (uint32_t v = 0; v < NV; v++) {
-        const uint8_t *a = acts + (size_t)(segs.act_first[seg] + v) * p.act_bytes;
-        uint8_t *base = lds + (size_t)v * act_lds;
-        uint32_t *qd = reinterpret_cast<uint32_t *>(base);
-        int32_t *bs = reinterpret_cast<int32_t *>(base + B * 256u);
-        float *dq = reinterpret_cast<float *>(base + B * 256u + B * 64u);
-        for (uint32_t j = tid; j < B * 64u; j += OXH_GEMV_WAVES * 64u) {
-            const uint32_t blk = j >> 6, w = j & 63u;
-            const uint32_t e = 4u * w;
-            const uint32_t n = e >> 7, k = (e >> 5) & 3u, lh = (e >> 4) & 1u;
-            const uint32_t val = *reinterpret_cast<const uint32_t *>(a + (size_t)blk * 292u + 4u + 4u * w);
-            qd[((k * B * 4u) + blk * 4u + 2u * n + lh) * 4u + (w & 3u)] = val;
-        }
-        for (uint32_t j = tid; j < B * 16u; j += OXH_GEMV_WAVES * 64u) {
-            const uint32_t blk = j >> 4, g = j & 15u;
-            const uint32_t n = g >> 3, k = (g >> 1) & 3u, lh = g & 1u;
-            const int16_t sum = *reinterpret_cast<const int16_t *>(a + (size_t)blk * 292u + 260u + 2u * g);
-            bs[(blk * 4u + 2u * n + lh) * 4u + k] = 32 * (int32_t)sum;
-        }
-        for (uint32_t j = tid; j < B; j += OXH_GEMV_WAVES * 64u)
-            dq[j] = *reinterpret_cast<const float *>(a + (size_t)j * 292u);
-    }
-    __syncthreads();
-
-    const uint32_t RW = p.rows_per_wave;
-    const uint32_t row0 = (wg_in_seg * OXH_GEMV_WAVES + wave) * RW;
-    if (row0 >= seg_rows) return;
-    const uint32_t nrows = min(RW, seg_rows - row0);
-    const uint32_t nblk = nrows * B;
-    const uint32_t u = lane & 3u;
-    const uint32_t n = u >> 1, lh = u & 1u;
-    const uint8_t *wbase = segs.w[seg] + (size_t)row0 * B * 210u;
-
-    for (uint32_t g0 = 0; g0 < nblk; g0 += 16u) {
-        const uint32_t g = g0 + (lane >> 2);
-        const bool live = g < nblk;
-        const uint32_t gc = live ? g : 0u;
-        const uint32_t r = (B == 1u) ? gc : __umulhi(gc, p.magic);
-        const uint32_t blk = gc - r * B;
-        const uint8_t *wb = wbase + (size_t)gc * 210u;
-        const U32x4u2 la = *reinterpret_cast<const U32x4u2 *>(wb + 64u * n + 16u * lh);
-        const U32x4u2 lb = *reinterpret_cast<const U32x4u2 *>(wb + 64u * n + 32u + 16u * lh);
-        const U32x4u2 hh = *reinterpret_cast<const U32x4u2 *>(wb + 128u + 32u * n + 16u * lh);
-        const uint32_t sc_lo = reinterpret_cast<const U32u2 *>(wb + 192u + 8u * n)->v;
-        const uint32_t sc_hi = reinterpret_cast<const U32u2 *>(wb + 196u + 8u * n)->v;
-        const uint32_t dbits = *reinterpret_cast<const uint16_t *>(wb + 208u);
-        /* scale bytes lh, lh+2 (low word) and lh+4, lh+6 (high word) */
-        const int sc0 = (int)(int8_t)(sc_lo >> (8u * lh));
-        const int sc1 = (int)(int8_t)(sc_lo >> (8u * lh + 16u));
-        const int sc2 = (int)(int8_t)(sc_hi >> (8u * lh));
-        const int sc3 = (int)(int8_t)(sc_hi >> (8u * lh + 16u));
-        const float dw = half_bits_to_float(dbits);
-        const uint32_t qa[4] = { la.x, la.y, la.z, la.w };
-        const uint32_t qb[4] = { lb.x, lb.y, lb.z, lb.w };
-        const uint32_t qh[4] = { hh.x, hh.y, hh.z, hh.w };
-
-        const uint32_t slot = blk * 4u + u;
-        for (uint32_t v = 0; v < NV; v++) {
-            const uint8_t *base = lds + (size_t)v * act_lds;
-            const u32x4 *qv = reinterpret_cast<const u32x4 *>(base);
-            const u32x4 a0 = qv[slot], a1 = qv[B * 4u + slot];
-            const u32x4 a2 = qv[B * 8u + slot], a3 = qv[B * 12u + slot];
-            const u32x4 off = reinterpret_cast<const u32x4 *>(base + B * 256u)[slot];
-            const float dq = reinterpret_cast<const float *>(base + B * 256u + B * 64u)[blk];
-
-            int g0s = 0, g1s = 0, g2s = 0, g3s = 0;
-#pragma unroll
-            for (int i = 0; i < 4; i++) {
-                const uint32_t c0 = (qa[i] & 0x0F0F0F0Fu) | ((qh[i] << 4) & 0x30303030u);
-                const uint32_t c1 = (qb[i] & 0x0F0F0F0Fu) | ((qh[i] << 2) & 0x30303030u);
-                const uint32_t c2 = ((qa[i] >> 4) & 0x0F0F0F0Fu) | (qh[i] & 0x30303030u);
-                const uint32_t c3 = ((qb[i] >> 4) & 0x0F0F0F0Fu) | ((qh[i] >> 2) & 0x30303030u);
-                g0s = dot4(c0, a0[i], g0s);
-                g1s = dot4(c1, a1[i], g1s);
-                g2s = dot4(c2, a2[i], g2s);
-                g3s = dot4(c3, a3[i], g3s);
-            }
-            if (DUMP) {
-                if (live) {
-                    int32_t *o = p.dump + ((size_t)(row0 * B + gc)) * 16u + 8u * n + lh;
-                    o[0] = g0s; o[2] = g1s; o[4] = g2s; o[6] = g3s;
-                }
-            }
-            /* sum_g sc_g * (G_g - 32*bsum_g) == pos - 32*minc, in integers */
-            int tot = sc0 * (g0s - (int)off[0]) + sc1 * (g1s - (int)off[1]) +
-                      sc2 * (g2s - (int)off[2]) + sc3 * (g3s - (int)off[3]);
-            tot = quad_sum(tot);
-            const float t = dw * dq;
-            if (live && u == 0u)
-                terms[((size_t)v * RW + r) * p.term_stride + blk] = t * (float)tot;
-        }
-    }
-    row_sums(terms, lane, NV, nrows, RW, B, p.term_stride, segs.out[seg], p.out_stride, row0);
-}
-
-/* Q8_0 x Q8_0.  One lane per 34-byte block, 64 blocks (2176 contiguous bytes)
- * per wave pass.  The per-block integer dot is exact; the f32 result is the
- * block-sequential chain of oxk.c:224-241 (the reference's x86 decode path
- * accumulates the same terms in a different order, so f32 outputs agree with
- * it to tolerance, not to the bit). */
-template <bool DUMP>
-__global__ __launch_bounds__(OXH_GEMV_WAVES * 64) void
-k_gemv_q8_0(const SegTable segs, const GemvParams p, const uint8_t *__restrict__ acts)
-{
-    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
-    const uint32_t tid = threadIdx.x;
-    const uint32_t lane = tid & 63u;
-    const uint32_t wave = tid >> 6;
-    const uint32_t B = p.blocks;
-    const uint32_t NV = p.n_vec;
-
-    const uint32_t seg = find_segment(segs, blockIdx.x);
-    const uint32_t wg_in_seg = blockIdx.x - segs.wg_begin[seg];
-    const uint32_t seg_rows = segs.rows[seg];
-
-    const uint32_t act_lds = q80_lds_bytes(B);
-    float *const terms = reinterpret_cast<float *>(lds + (size_t)act_lds * NV) +
-                         (size_t)wave * NV * p.rows_per_wave * p.term_stride;
-
-    for (uint32_t v = 0; v < NV; v++) {
-        const uint8_t *a = acts + (size_t)(segs.act_first[seg] + v) * p.act_bytes;
-        uint8_t *base = lds + (size_t)v * act_lds;
-        uint32_t *qd = reinterpret_cast<uint32_t *>(base);
-        float *dq = reinterpret_cast<float *>(base + B * 32u);
-        for (uint32_t j = tid; j < B * 8u; j += OXH_GEMV_WAVES * 64u) {
-            const uint32_t blk = j >> 3, w = j & 7u;
-            const uint32_t val = reinterpret_cast<const U32u2 *>(a + (size_t)blk * 34u + 2u + 4u * w)->v;
-            qd[(((w >> 2) * B) + blk) * 4u + (w & 3u)] = val;
-        }
-        for (uint32_t j = tid; j < B; j += OXH_GEMV_WAVES * 64u)
-            dq[j] = half_bits_to_float(*reinterpret_cast<const uint16_t *>(a + (size_t)j * 34u));
-    }
-    __syncthreads();
-
-    const uint32_t RW = p.rows_per_wave;
-    const uint32_t row0 = (wg_in_seg * OXH_GEMV_WAVES + wave) * RW;
-    if (row0 >= seg_rows) return;
-    const uint32_t nrows = min(RW, seg_rows - row0);
-    const uint32_t nblk = nrows * B;
-    const uint8_t *wbase = segs.w[seg] + (size_t)row0 * B * 34u;
-
-    for (uint32_t g0 = 0; g0 < nblk; g0 += 64u) {
-        const uint32_t g = g0 + lane;
-        const bool live = g < nblk;
-        const uint32_t gc = live ? g : 0u;
-        const uint32_t r = (B == 1u) ? gc : __umulhi(gc, p.magic);
-        const uint32_t blk = gc - r * B;
-        const uint8_t *wb = wbase + (size_t)gc * 34u;
-        const uint32_t dbits = *reinterpret_cast<const uint16_t *>(wb);
-        const U32x4u2 w0 = *reinterpret_cast<const U32x4u2 *>(wb + 2u);
-        const U32x4u2 w1 = *reinterpret_cast<const U32x4u2 *>(wb + 18u);
-        const float dw = half_bits_to_float(dbits);
-
-        for (uint32_t v = 0; v < NV; v++) {
-            const uint8_t *base = lds + (size_t)v * act_lds;
-            const u32x4 *qv = reinterpret_cast<const u32x4 *>(base);
-            const u32x4 a0 = qv[blk], a1 = qv[B + blk];
-            const float dq = reinterpret_cast<const float *>(base + B * 32u)[blk];
-            int isum = 0;
-            isum = dot4(w0.x, a0[0], isum); isum = dot4(w0.y, a0[1], isum);
-            isum = dot4(w0.z, a0[2], isum); isum = dot4(w0.w, a0[3], isum);
-            isum = dot4(w1.x, a1[0], isum); isum = dot4(w1.y, a1[1], isum);
-            isum = dot4(w1.z, a1[2], isum); isum = dot4(w1.w, a1[3], isum);
-            if (DUMP) {
-                if (live) p.dump[(size_t)row0 * B + gc] = isum;
-            }
-            const float t = dw * dq;
-            if (live) terms[((size_t)v * RW + r) * p.term_stride + blk] = t * (float)isum;
-        }
-    }
-    row_sums(terms, lane, NV, nrows, RW, B, p.term_stride, segs.out[seg], p.out_stride, row0);
-}
-
-/* ─── prefill matmul (MMQ) ────────────────────────────────────────────── */
-
-typedef int v4i __attribute__((ext_vector_type(4)));
-typedef int v16i __attribute__((ext_vector_type(16)));
-
-#define MMQ_WAVES 4
-#define MMQ_ROWS (MMQ_WAVES * 32)   /* weight rows per workgroup          */
-#define MMQ_TOK 64                  /* tokens per workgroup (two tiles)   */
-
-/* Q4_K weights x Q8_K activations on v_mfma_i32_32x32x32_i8.
- *
- * One MFMA covers 32 tokens x 32 weight rows x one 32-wide sub-block, so each
- * result tile is exactly the sub-block sums S_j of oxk.c:263-270 for 1024
- * (token, row) pairs.  M = tokens (A operand, int8 activations staged in
- * LDS), N = weight rows (B operand, nibble codes unpacked in registers): the
- * accumulator of lane l then belongs to weight row l%32, so the 6-bit scale
- * is one register per lane and `pos += sc_j * S_j` is an integer multiply-add
- * per accumulator.  The min term sum_j m_j*B_j is formed by a second MFMA per
- * sub-block with the B operand set to m_j in every byte (sum_k m_j*q_k over
- * the sub-block is m_j*B_j), accumulated over the whole super-block.
- * Per super-block the f32 step is the reference's, in its order:
- *   acc += (dw*dq)*(float)pos - (dmin*dq)*(float)min_acc      (oxk.c:286-294)
- * so every output is bit-identical to the single-vector GEMV.
- *
- * Lane l supplies, for both operands, the 16 values k = 16*(l/32) .. +15 of
- * the sub-block; A and B use the same assignment, so the product does not
- * depend on how the hardware numbers k internally. */
-__global__ __launch_bounds__(MMQ_WAVES * 64) void
-k_mmq_q4_k(const uint8_t *__restrict__ w, uint32_t rows, uint32_t B,
-           const uint8_t *__restrict__ acts, uint32_t n_vec, float *__restrict__ out,
-           size_t out_stride)
-{
-    __shared__ __attribute__((aligned(16))) uint8_t lds_q[MMQ_TOK * 256];
-    __shared__ float lds_dq[MMQ_TOK];
-
-    const uint32_t tid = threadIdx.x;
-    const uint32_t lane = tid & 63u;
-    const uint32_t wave = tid >> 6;
-    const uint32_t n = lane & 31u;          /* weight row / token within a tile */
-    const uint32_t h = lane >> 5;           /* which 16 of the sub-block's 32   */
-    const uint32_t row_base = blockIdx.x * MMQ_ROWS + wave * 32u;
-    const uint32_t tok_base = blockIdx.y * MMQ_TOK;
-    const uint32_t row = row_base + n;
-    const uint32_t row_c = row < rows ? row : rows - 1u;
-    const uint8_t *wrow = w + (size_t)row_c * B * 144u;
-    const size_t act_stride = (size_t)B * 292u;
-
-    float acc[2][16];
-#pragma unroll
-    for (int t = 0; t < 2; t++)
-#pragma unroll
-        for (int i = 0; i < 16; i++) acc[t][i] = 0.0f;
-
-    for (uint32_t b = 0; b < B; b++) {
-        __syncthreads();
-        /* stage this super-block of 64 tokens: value dword wd of token t goes
-         * to [tile][j][h][token-in-tile] x 16 B */
-        for (uint32_t idx = tid; idx < MMQ_TOK * 64u; idx += MMQ_WAVES * 64u) {
-            const uint32_t t = idx >> 6, wd = idx & 63u;
-            const uint32_t tok = tok_base + t;
-            uint32_t val = 0u;
-            if (tok < n_vec)
-                val = *reinterpret_cast<const uint32_t *>(acts + (size_t)tok * act_stride +
-                                                          (size_t)b * 292u + 4u + 4u * wd);
-            const uint32_t j = wd >> 3, hh = (wd >> 2) & 1u;
-            const uint32_t slot = (((t >> 5) * 8u + j) * 2u + hh) * 32u + (t & 31u);
-            reinterpret_cast<uint32_t *>(lds_q)[slot * 4u + (wd & 3u)] = val;
-        }
-        if (tid < MMQ_TOK) {
-            const uint32_t tok = tok_base + tid;
-            lds_dq[tid] = tok < n_vec
-                ? *reinterpret_cast<const float *>(acts + (size_t)tok * act_stride + (size_t)b * 292u)
-                : 0.0f;
-        }
-        /* this lane's weights: header and its half of each 32-byte nibble group */
-        const uint8_t *wb = wrow + (size_t)b * 144u;
-        const u32x4 hdr = *reinterpret_cast<const u32x4 *>(wb);
-        u32x4 nib[4];
-#pragma unroll
-        for (int gp = 0; gp < 4; gp++)
-            nib[gp] = *reinterpret_cast<const u32x4 *>(wb + 16u + 32u * gp + 16u * h);
-        __syncthreads();
-
-        const uint32_t u0 = hdr.y, u1 = hdr.z, u2 = hdr.w;
-        const uint32_t sc_lo = u0 & 0x3F3F3F3Fu;
-        const uint32_t mn_lo = u1 & 0x3F3F3F3Fu;
-        const uint32_t sc_hi = (u2 & 0x0F0F0F0Fu) | ((u0 >> 2) & 0x30303030u);
-        const uint32_t mn_hi = ((u2 >> 4) & 0x0F0F0F0Fu) | ((u1 >> 2) & 0x30303030u);
-        const float dw = half_bits_to_float(hdr.x & 0xFFFFu);
-        const float dmin = half_bits_to_float(hdr.x >> 16);
-
-        v16i pos[2], mn[2];
-#pragma unroll
-        for (int t = 0; t < 2; t++)
-#pragma unroll
-            for (int i = 0; i < 16; i++) { pos[t][i] = 0; mn[t][i] = 0; }
-
-#pragma unroll
-        for (int j = 0; j < 8; j++) {
-            const u32x4 raw = nib[j >> 1];
-            v4i bw;
-#pragma unroll
-            for (int k = 0; k < 4; k++)
-                bw[k] = (int)((j & 1) ? ((raw[k] >> 4) & 0x0F0F0F0Fu) : (raw[k] & 0x0F0F0F0Fu));
-            const uint32_t scw = j < 4 ? sc_lo : sc_hi;
-            const uint32_t mnw = j < 4 ? mn_lo : mn_hi;
-            const int sc = (int)((scw >> (8 * (j & 3))) & 0xFFu);
-            const int mj = (int)(((mnw >> (8 * (j & 3))) & 0xFFu) * 0x01010101u);
-            const v4i bm = { mj, mj, mj, mj };
-#pragma unroll
-            for (int t = 0; t < 2; t++) {
-                const v4i a = *reinterpret_cast<const v4i *>(
-                    lds_q + ((((uint32_t)t * 8u + (uint32_t)j) * 2u + h) * 32u + n) * 16u);
-                const v16i zero = { 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0 };
-                const v16i sj = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, bw, zero, 0, 0, 0);
-#pragma unroll
-                for (int i = 0; i < 16; i++) pos[t][i] += __mul24(sc, sj[i]);
-                mn[t] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, bm, mn[t], 0, 0, 0);
-            }
-        }
-        /* accumulator i of lane l is token 8*(i/4) + 4*(l/32) + i%4 of the tile */
-#pragma unroll
-        for (int t = 0; t < 2; t++)
-#pragma unroll
-            for (int i = 0; i < 16; i++) {
-                const uint32_t m = 8u * (uint32_t)(i >> 2) + 4u * h + (uint32_t)(i & 3);
-                const float dq = lds_dq[t * 32 + m];
-                const float t_pos = dw * dq;
-                const float t_min = dmin * dq;
-                const float up = t_pos * (float)pos[t][i];
-                const float dn = t_min * (float)mn[t][i];
-                acc[t][i] += up - dn;
-            }
-    }
-    if (row < rows) {
-#pragma unroll
-        for (int t = 0; t < 2; t++)
-#pragma unroll
-            for (int i = 0; i < 16; i++) {
-                const uint32_t m = 8u * (uint32_t)(i >> 2) + 4u * h + (uint32_t)(i & 3);
-                const uint32_t tok = tok_base + (uint32_t)t * 32u + m;
-                if (tok < n_vec) out[(size_t)tok * out_stride + row] = acc[t][i];
-            }
-    }
-}
+#include "gemv_kernels.inc"
+#include "mmq_kernels.inc"
 
 /* ─── host side of layer 2 ────────────────────────────────────────────── */
 
@@ -891,20 +391,6 @@ extern "C" int oxh_quantize_q8_0(const float *d_x, size_t in_stride, size_t n_ve
     return OXH_OK;
 }
 
-/* Rows each wave takes: large enough to amortise the per-row tail, small
- * enough that the launch still has several waves per SIMD on every CU. */
-static uint32_t choose_rows_per_wave(size_t total_rows, uint32_t blocks, uint32_t lanes_per_block)
-{
-    const size_t target_waves = (size_t)(g_n_cu > 0 ? g_n_cu : 256) * 16u;
-    size_t rw = total_rows / target_waves;
-    if (rw < 1) rw = 1;
-    if (rw > 16) rw = 16;
-    /* whole passes when possible: rw*blocks a multiple of blocks-per-pass */
-    const uint32_t per_pass = 64u / lanes_per_block;
-    while (rw > 1 && ((rw * blocks) % per_pass) != 0) rw--;
-    return (uint32_t)rw;
-}
-
 static bool is_q4k(uint32_t qtype) { return qtype == OXH_Q4_K_S || qtype == OXH_Q4_K_M; }
 
 static uint32_t act_lds_bytes(uint32_t qtype, uint32_t blocks)
@@ -914,10 +400,37 @@ static uint32_t act_lds_bytes(uint32_t qtype, uint32_t blocks)
     return q8k_lds_bytes(blocks);
 }
 
-static size_t gemv_lds_bytes(uint32_t qtype, uint32_t blocks, size_t n_vec, uint32_t rows_per_wave)
+static size_t gemv_lds_bytes(uint32_t qtype, uint32_t blocks, size_t n_vec, uint32_t waves,
+                             uint32_t rows_cap)
 {
     return n_vec * (size_t)act_lds_bytes(qtype, blocks) +
-           (size_t)OXH_GEMV_WAVES * n_vec * rows_per_wave * (blocks + 1u) * 4u;
+           (size_t)waves * n_vec * rows_cap * (blocks + 1u) * 4u;
+}
+
+static uint32_t env_u32(const char *name, uint32_t dflt, uint32_t lo, uint32_t hi)
+{
+    const char *e = getenv(name);
+    if (!e || !*e) return dflt;
+    const long v = strtol(e, nullptr, 10);
+    if (v < (long)lo || v > (long)hi) return dflt;
+    return (uint32_t)v;
+}
+
+/* Launch shape knobs (tuning aids; the defaults are what the benchmarks use):
+ * OXH_GEMV_WAVES = waves per workgroup (1..16), OXH_GEMV_WG_PER_CU = how many
+ * workgroups per compute unit the grid is sized for. */
+static uint32_t gemv_waves(void)
+{
+    static uint32_t w = 0;
+    if (!w) w = env_u32("OXH_GEMV_WAVES", 16, 1, 16);
+    return w;
+}
+
+static uint32_t gemv_wg_per_cu(void)
+{
+    static uint32_t w = 0;
+    if (!w) w = env_u32("OXH_GEMV_WG_PER_CU", 2, 1, 64);
+    return w;
 }
 
 extern "C" size_t oxh_gemv_max_nvec(uint32_t qtype, size_t cols)
@@ -927,18 +440,25 @@ extern "C" size_t oxh_gemv_max_nvec(uint32_t qtype, size_t cols)
     const size_t blocks = kind == 2 ? cols / OXH_QK_K : cols / OXH_QK8_0;
     if (blocks > 0xFFFFu) return 0;
     size_t nv = OXH_MAX_NV;
-    while (nv > 0 && gemv_lds_bytes(qtype, (uint32_t)blocks, nv, 1) > 65536u) nv--;
+    while (nv > 0 && gemv_lds_bytes(qtype, (uint32_t)blocks, nv, 1, 1) > 65536u) nv--;
     return nv;
 }
 
+struct GemvIo {
+    const void *d_acts;     /* pre-quantised activations, or NULL            */
+    const float *d_x;       /* f32 inputs to quantise in the kernel, or NULL */
+    size_t x_stride;
+    void *d_act_out;        /* optional store of the quantised bytes         */
+};
+
 static int launch_gemv(uint32_t qtype, const OxhSegment *segs, size_t n_segs, size_t cols,
-                       const void *d_acts, size_t n_vec, size_t out_stride, int32_t *dump,
+                       const GemvIo &io, size_t n_vec, size_t out_stride, int32_t *dump,
                        void *stream)
 {
     int rc = ensure_init();
     if (rc) return rc;
     if (n_segs == 0) return OXH_OK;
-    if (!segs || !d_acts) return arg_fail("gemv: NULL pointer");
+    if (!segs || (!io.d_acts && !io.d_x)) return arg_fail("gemv: NULL pointer");
     if (n_vec < 1 || n_vec > OXH_MAX_NV) return arg_fail("gemv: n_vec must be 1..8");
     if (n_segs > OXH_MAX_SEGS) return arg_fail("gemv: more than 32 segments in one launch");
     const int kind = oxh_act_kind(qtype, cols);
@@ -947,11 +467,11 @@ static int launch_gemv(uint32_t qtype, const OxhSegment *segs, size_t n_segs, si
         return OXH_DECLINED;
     }
     const size_t blocks = kind == 2 ? cols / OXH_QK_K : cols / OXH_QK8_0;
-    const size_t bbytes = block_bytes(qtype);
     if (blocks > 0xFFFFu) {
         snprintf(g_err, sizeof g_err, "gemv: cols %zu too wide", cols);
         return OXH_ERR_TOO_WIDE;
     }
+    if (io.d_x && io.x_stride < cols) return arg_fail("gemv: x_stride < cols");
     size_t total_rows = 0, max_act = 0;
     for (size_t i = 0; i < n_segs; i++) {
         if (segs[i].rows > 0x7FFFFFFFull / (blocks * 16u)) return arg_fail("gemv: segment too large");
@@ -960,36 +480,56 @@ static int launch_gemv(uint32_t qtype, const OxhSegment *segs, size_t n_segs, si
         if (segs[i].act_first > max_act) max_act = segs[i].act_first;
     }
     if (total_rows == 0) return OXH_OK;
-    if (out_stride > 0xFFFFFFFFull || max_act + n_vec > 0xFFFFFFFFull) return arg_fail("gemv: stride too large");
-    (void)bbytes;
+    if (out_stride > 0xFFFFFFFFull || io.x_stride > 0xFFFFFFFFull || max_act + n_vec > 0xFFFFFFFFull)
+        return arg_fail("gemv: stride too large");
 
-    const uint32_t lanes_per_block = qtype == OXH_Q8_0 ? 1u : 4u;
+    /* Deal workgroups to segments in proportion to their rows; every wave
+     * then owns ceil(rows / waves) whole rows of its segment. */
+    uint32_t W = gemv_waves();
+    const size_t target = (size_t)(g_n_cu > 0 ? g_n_cu : 256) * gemv_wg_per_cu();
+    uint32_t cap_limit = GEMV_ROWS_CAP;
+    uint32_t n_wg[OXH_MAX_SEGS];
+    uint32_t rows_cap = 1;
+    for (;;) {
+        rows_cap = 1;
+        for (size_t i = 0; i < n_segs; i++) {
+            const size_t rows = segs[i].rows;
+            if (rows == 0) { n_wg[i] = 0; continue; }
+            size_t share = (target * rows + total_rows / 2) / total_rows;
+            const size_t lo = (rows + (size_t)W * cap_limit - 1) / ((size_t)W * cap_limit);
+            const size_t hi = (rows + W - 1) / W;
+            if (share < lo) share = lo;
+            if (share > hi) share = hi;
+            if (share < 1) share = 1;
+            n_wg[i] = (uint32_t)share;
+            const uint32_t rpw = (uint32_t)((rows + share * W - 1) / (share * W));   /* q + (rem != 0) */
+            if (rpw > rows_cap) rows_cap = rpw;
+        }
+        if (gemv_lds_bytes(qtype, (uint32_t)blocks, n_vec, W, rows_cap) <= 65536u) break;
+        if (cap_limit > 1) { cap_limit = rows_cap > 1 ? rows_cap - 1 : 1; continue; }
+        if (W > 1) { W /= 2; cap_limit = GEMV_ROWS_CAP; continue; }
+        snprintf(g_err, sizeof g_err, "gemv: cols %zu x n_vec %zu does not fit 64 KiB of LDS", cols, n_vec);
+        return OXH_ERR_TOO_WIDE;
+    }
+    const size_t lds = gemv_lds_bytes(qtype, (uint32_t)blocks, n_vec, W, rows_cap);
+
     GemvParams p;
+    memset(&p, 0, sizeof p);
     p.blocks = (uint32_t)blocks;
     p.magic = (uint32_t)((0x100000000ull + blocks - 1u) / blocks);
-    p.rows_per_wave = choose_rows_per_wave(total_rows, p.blocks, lanes_per_block);
     p.n_vec = (uint32_t)n_vec;
     p.act_bytes = (uint32_t)oxh_act_bytes(qtype, cols);
     p.out_stride = (uint32_t)out_stride;
     p.term_stride = p.blocks + 1u;
+    p.rows_cap = rows_cap;
+    p.x = io.d_x;
+    p.x_stride = (uint32_t)io.x_stride;
+    p.act_out = (uint8_t *)io.d_act_out;
     p.dump = dump;
-
-    size_t lds = gemv_lds_bytes(qtype, p.blocks, n_vec, p.rows_per_wave);
-    while (lds > 65536u && p.rows_per_wave > 1) {
-        p.rows_per_wave--;
-        lds = gemv_lds_bytes(qtype, p.blocks, n_vec, p.rows_per_wave);
-    }
-    if (lds > 65536u) {
-        snprintf(g_err, sizeof g_err, "gemv: cols %zu x n_vec %zu needs %zu B of LDS (max 65536)",
-                 cols, n_vec, lds);
-        return OXH_ERR_TOO_WIDE;
-    }
 
     SegTable t;
     memset(&t, 0, sizeof t);
-    uint32_t wg = 0;
-    uint32_t n = 0;
-    const uint32_t rows_per_wg = p.rows_per_wave * OXH_GEMV_WAVES;
+    uint32_t wg = 0, n = 0;
     for (size_t i = 0; i < n_segs; i++) {
         if (segs[i].rows == 0) continue;
         t.w[n] = (const uint8_t *)segs[i].d_w;
@@ -997,25 +537,27 @@ static int launch_gemv(uint32_t qtype, const OxhSegment *segs, size_t n_segs, si
         t.rows[n] = (uint32_t)segs[i].rows;
         t.act_first[n] = (uint32_t)segs[i].act_first;
         t.wg_begin[n] = wg;
-        wg += (uint32_t)((segs[i].rows + rows_per_wg - 1u) / rows_per_wg);
+        t.rows_q[n] = (uint32_t)(segs[i].rows / ((size_t)n_wg[i] * W));
+        t.rows_rem[n] = (uint32_t)(segs[i].rows % ((size_t)n_wg[i] * W));
+        wg += n_wg[i];
         n++;
     }
     t.wg_begin[n] = wg;
     t.n = n;
 
-    const dim3 grid(wg), block(OXH_GEMV_WAVES * 64);
+    const dim3 grid(wg), block(W * 64u);
     hipStream_t st = pick_stream(stream);
-    const uint8_t *a = (const uint8_t *)d_acts;
-    if (is_q4k(qtype)) {
-        if (dump) hipLaunchKernelGGL(k_gemv_q4_k<true>, grid, block, lds, st, t, p, a);
-        else      hipLaunchKernelGGL(k_gemv_q4_k<false>, grid, block, lds, st, t, p, a);
-    } else if (qtype == OXH_Q6_K) {
-        if (dump) hipLaunchKernelGGL(k_gemv_q6_k<true>, grid, block, lds, st, t, p, a);
-        else      hipLaunchKernelGGL(k_gemv_q6_k<false>, grid, block, lds, st, t, p, a);
-    } else {
-        if (dump) hipLaunchKernelGGL(k_gemv_q8_0<true>, grid, block, lds, st, t, p, a);
-        else      hipLaunchKernelGGL(k_gemv_q8_0<false>, grid, block, lds, st, t, p, a);
-    }
+    const uint8_t *a = (const uint8_t *)io.d_acts;
+#define OXH_LAUNCH(KERNEL)                                                              \
+    do {                                                                                \
+        if (dump)            hipLaunchKernelGGL((KERNEL<0, true>), grid, block, lds, st, t, p, a);  \
+        else if (n_vec == 1) hipLaunchKernelGGL((KERNEL<1, false>), grid, block, lds, st, t, p, a); \
+        else                 hipLaunchKernelGGL((KERNEL<0, false>), grid, block, lds, st, t, p, a); \
+    } while (0)
+    if (is_q4k(qtype))          OXH_LAUNCH(k_gemv_q4_k);
+    else if (qtype == OXH_Q6_K) OXH_LAUNCH(k_gemv_q6_k);
+    else                        OXH_LAUNCH(k_gemv_q8_0);
+#undef OXH_LAUNCH
     HIP_TRY(hipGetLastError());
     return OXH_OK;
 }
@@ -1024,7 +566,19 @@ extern "C" int oxh_gemv_segments(uint32_t qtype, const OxhSegment *segs, size_t 
                                  size_t cols, const void *d_acts, size_t n_vec,
                                  size_t out_stride, void *stream)
 {
-    return launch_gemv(qtype, segs, n_segs, cols, d_acts, n_vec, out_stride, nullptr, stream);
+    if (!d_acts && n_segs) return arg_fail("oxh_gemv_segments: NULL activations");
+    const GemvIo io = { d_acts, nullptr, 0, nullptr };
+    return launch_gemv(qtype, segs, n_segs, cols, io, n_vec, out_stride, nullptr, stream);
+}
+
+extern "C" int oxh_gemv_segments_f32(uint32_t qtype, const OxhSegment *segs, size_t n_segs,
+                                     size_t cols, const float *d_x, size_t x_stride,
+                                     void *d_act_out, size_t n_vec, size_t out_stride,
+                                     void *stream)
+{
+    if (!d_x && n_segs) return arg_fail("oxh_gemv_segments_f32: NULL input");
+    const GemvIo io = { nullptr, d_x, x_stride, d_act_out };
+    return launch_gemv(qtype, segs, n_segs, cols, io, n_vec, out_stride, nullptr, stream);
 }
 
 extern "C" int oxh_debug_subblock_sums(uint32_t qtype, const void *d_w, size_t rows,
@@ -1037,7 +591,8 @@ extern "C" int oxh_debug_subblock_sums(uint32_t qtype, const void *d_w, size_t r
     float *scratch = nullptr;
     HIP_TRY(hipMalloc((void **)&scratch, (rows ? rows : 1) * sizeof(float)));
     OxhSegment s = { d_w, scratch, rows, 0 };
-    rc = launch_gemv(qtype, &s, 1, cols, d_act, 1, rows, d_sums, stream);
+    const GemvIo io = { d_act, nullptr, 0, nullptr };
+    rc = launch_gemv(qtype, &s, 1, cols, io, 1, rows, d_sums, stream);
     hipError_t e = hipStreamSynchronize(pick_stream(stream));
     (void)hipFree(scratch);
     if (rc) return rc;

@@ -141,6 +141,14 @@ def gemv_segments(qtype, segs, cols, d_acts, n_vec=1, out_stride=0, stream=None)
                                   n_vec, out_stride, stream))
 
 
+def gemv_segments_f32(qtype, segs, cols, d_x, x_stride, d_act_out=None, n_vec=1, out_stride=0,
+                      stream=None):
+    """GEMV with the activation quantisation fused into the kernel."""
+    check(lib().oxh_gemv_segments_f32(qtype, segs, len(segs), cols, ctypes.c_void_p(d_x), x_stride,
+                                      None if d_act_out is None else ctypes.c_void_p(d_act_out),
+                                      n_vec, out_stride, stream))
+
+
 def mmq(qtype, d_w, rows, cols, d_acts, n_vec, d_out, out_stride, stream=None):
     check(lib().oxh_mmq(qtype, ctypes.c_void_p(d_w), rows, cols, ctypes.c_void_p(d_acts),
                         n_vec, ctypes.c_void_p(d_out), out_stride, stream))

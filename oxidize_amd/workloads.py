@@ -84,16 +84,22 @@ class DecodeSet:
     def ops_per_step(self):
         return sum(2 * sum(rows) * cols for _, _, rows, cols, _ in self.ops) * self.layers
 
-    def launch_op(self, layer, op, stream=None, quantize=True):
+    def launch_op(self, layer, op, stream=None, fused=True):
+        """One decode matmul from its f32 input: a single launch that quantises
+        the activation inside the GEMV kernel (fused=True, what the host API
+        does), or the stand-alone quantiser followed by the GEMV."""
         name, qt, rows, cols, _ = self.ops[op]
-        if quantize:
+        if fused:
+            mv.gemv_segments_f32(qt, self.segments[layer][op], cols, self.x[layer][op].ptr, cols,
+                                 self.act[layer][op].ptr, 1, 0, stream)
+        else:
             mv.quantize(qt, self.x[layer][op].ptr, cols, 1, cols, self.act[layer][op].ptr, stream)
-        mv.gemv_segments(qt, self.segments[layer][op], cols, self.act[layer][op].ptr, 1, 0, stream)
+            mv.gemv_segments(qt, self.segments[layer][op], cols, self.act[layer][op].ptr, 1, 0, stream)
 
-    def launch_step(self, stream=None):
+    def launch_step(self, stream=None, fused=True):
         for layer in range(self.layers):
             for op in range(len(self.ops)):
-                self.launch_op(layer, op, stream)
+                self.launch_op(layer, op, stream, fused)
 
     def output(self, layer, op):
         rows = sum(self.ops[op][2])

@@ -283,3 +283,55 @@ def test_mmq_batch_bit_identical_to_single_vector(oxh, rows, cols, n_vec, out_pa
                                         sc2.ctypes.data, sc2.nbytes) == 0
     assert np.array_equal(bits(outs[:, :rows]), bits(want))
     assert np.all(outs[:, rows:] == -7.25)
+
+
+@pytest.mark.parametrize("qtype,cols,d_off", [(Q4K, 1024, 0), (Q6K, 1024, 208), (Q80, 256, 0)])
+def test_subnormal_and_extreme_f16_weight_scales(oxh, qtype, cols, d_off):
+    """f16 block scales in the subnormal range, at the largest finite value and
+    negative: the f16 -> f32 step must be exact for every bit pattern."""
+    rows = 64
+    w = synth.weights(qtype, rows, cols, seed=81)
+    bsz = synth.BLOCK_BYTES[qtype]
+    blk = w.reshape(-1, bsz)
+    pats = np.array([0x0001, 0x0002, 0x03FF, 0x0400, 0x7BFF, 0x8001, 0x83FF, 0xBC00, 0x0000, 0x8000,
+                     0x0155, 0x3555], np.uint16)
+    sel = pats[np.arange(blk.shape[0]) % pats.size]
+    blk[:, d_off] = sel & 0xFF
+    blk[:, d_off + 1] = sel >> 8
+    if qtype == Q4K:
+        sel2 = pats[(np.arange(blk.shape[0]) * 5 + 3) % pats.size]
+        blk[:, 2] = sel2 & 0xFF
+        blk[:, 3] = sel2 >> 8
+    x = synth.normal(cols, seed=81)
+    out = np.zeros(rows, np.float32)
+    temp = np.zeros(cols, np.float32)
+    assert mv.matvec_quantized(qtype, w, rows, cols, synth.row_bytes(qtype, cols), x, out, temp) == 0
+    want, _ = oracle_matvec(qtype, w, rows, cols, x)
+    assert np.array_equal(bits(out), bits(want))
+
+
+@pytest.mark.parametrize("qtype,rows,cols,n_vec", [(Q4K, 100, 4096, 1), (Q6K, 60, 2048, 3), (Q80, 90, 896, 8)])
+def test_prequantised_and_fused_paths_agree(oxh, qtype, rows, cols, n_vec):
+    """Layer 2: quantiser kernel + GEMV over stored Q8 bytes gives the same
+    outputs and the same activation bytes as the single fused launch."""
+    w = synth.weights(qtype, rows, cols, seed=91)
+    xs = synth.normal(n_vec * cols, seed=91).reshape(n_vec, cols)
+    d_w = mv.DeviceBuffer.from_host(w)
+    d_x = mv.DeviceBuffer.from_host(xs)
+    nact = mv.act_bytes(qtype, cols)
+    d_a1, d_a2 = mv.DeviceBuffer(n_vec * nact), mv.DeviceBuffer(n_vec * nact)
+    d_o1, d_o2 = mv.DeviceBuffer(n_vec * rows * 4), mv.DeviceBuffer(n_vec * rows * 4)
+    mv.quantize(qtype, d_x.ptr, cols, n_vec, cols, d_a1.ptr)
+    mv.gemv_segments(qtype, mv.make_segments([(d_w.ptr, d_o1.ptr, rows, 0)]), cols, d_a1.ptr, n_vec, rows)
+    mv.gemv_segments_f32(qtype, mv.make_segments([(d_w.ptr, d_o2.ptr, rows, 0)]), cols, d_x.ptr, cols,
+                         d_a2.ptr, n_vec, rows)
+    a1 = d_a1.download(np.uint8, n_vec * nact)
+    a2 = d_a2.download(np.uint8, n_vec * nact)
+    o1 = d_o1.download(np.float32, n_vec * rows)
+    o2 = d_o2.download(np.float32, n_vec * rows)
+    assert np.array_equal(a1, a2)
+    assert np.array_equal(bits(o1), bits(o2))
+    o = oxlibs.oracle()
+    for v in range(n_vec):
+        want, _ = oracle_matvec(qtype, w, rows, cols, np.ascontiguousarray(xs[v]))
+        assert np.array_equal(bits(o1[v * rows:(v + 1) * rows]), bits(want))
