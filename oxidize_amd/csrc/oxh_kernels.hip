@@ -429,7 +429,7 @@ static uint32_t gemv_waves(void)
 static uint32_t gemv_wg_per_cu(void)
 {
     static uint32_t w = 0;
-    if (!w) w = env_u32("OXH_GEMV_WG_PER_CU", 2, 1, 64);
+    if (!w) w = env_u32("OXH_GEMV_WG_PER_CU", 1, 1, 64);
     return w;
 }
 
