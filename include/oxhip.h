@@ -92,11 +92,14 @@ typedef struct OxhSegment {
     float      *d_out;    /* output vector 0; vector v at d_out + v*out_stride */
     size_t      rows;
     size_t      act_first;/* index of this segment's first activation in d_acts */
+    size_t      n_vec;    /* activations of this segment (1..8); 0 = the launch's n_vec */
 } OxhSegment;
 
 /* Decode GEMV over pre-quantised activations:
  *   out[v][r] = dot(W[r], act[act_first + v])   for v < n_vec (1..8)
- * for every segment, in ONE launch.  Covers the reference's row kernels
+ * for every segment, in ONE launch (a segment may override n_vec with its own
+ * count: expert e of an MoE layer takes only the m_e tokens routed to it,
+ * llama.c:6151-6169).  Covers the reference's row kernels
  * oc_oxk_dot_rows_{q4_k,q6_k}_q8_k / _q8_0_q8_0 (oxidize-c/src/compute/oxk.c:
  * 1447-1465) as used by matvec_fused_slice, matvec_fused_multi_slice and
  * matvec_fused_multi_input_slice (matvec.c:640-797) and the small-batch

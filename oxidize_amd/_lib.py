@@ -19,7 +19,7 @@ I = ctypes.c_int
 
 
 class OxhSegment(ctypes.Structure):
-    _fields_ = [("d_w", V), ("d_out", V), ("rows", Z), ("act_first", Z)]
+    _fields_ = [("d_w", V), ("d_out", V), ("rows", Z), ("act_first", Z), ("n_vec", Z)]
 
 
 class OcMatvecFusedTestStats(ctypes.Structure):

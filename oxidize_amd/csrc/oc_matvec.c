@@ -275,7 +275,7 @@ int oxh_matvec_quantized(uint32_t qtype, const uint8_t *data, size_t rows,
 
     if ((rc = oxh_memcpy_h2d(g_dx.p, input, cols * sizeof(float), NULL))) return rc;
     /* one launch: quantise the activation inside the GEMV kernel */
-    OxhSegment seg = { d_w, (float *)g_dout.p, rows, 0 };
+    OxhSegment seg = { d_w, (float *)g_dout.p, rows, 0, 0 };
     if ((rc = oxh_gemv_segments_f32(qtype, &seg, 1, cols, (const float *)g_dx.p, cols, g_dact.p, 1,
                                     rows, NULL)))
         return rc;
@@ -332,6 +332,7 @@ static int grouped(uint32_t qtype, const uint8_t *const *datas,
             segs[i].d_out = (float *)g_dout.p + done_rows;
             segs[i].rows = rows[k];
             segs[i].act_first = n_inputs == 1 ? 0 : k;
+            segs[i].n_vec = 0;
             done_rows += rows[k];
         }
         if ((rc = oxh_gemv_segments_f32(qtype, segs, n, cols, (const float *)g_dx.p, cols, NULL, 1, 0,
@@ -481,7 +482,7 @@ int oxh_matvec_quantized_batch(uint32_t qtype, const uint8_t *data, size_t rows,
         }
         for (size_t v0 = 0; v0 < n_vec; v0 += step) {
             const size_t m = n_vec - v0 < step ? n_vec - v0 : step;
-            OxhSegment seg = { d_w, (float *)g_dout.p + v0 * rows, rows, v0 };
+            OxhSegment seg = { d_w, (float *)g_dout.p + v0 * rows, rows, v0, 0 };
             if ((rc = oxh_gemv_segments_f32(qtype, &seg, 1, cols, (const float *)g_dx.p, in_stride,
                                             NULL, m, rows, NULL)))
                 return rc;

@@ -264,6 +264,8 @@ k_quantize_q8_0(const float *__restrict__ x, size_t in_stride, uint32_t blocks_p
 
 /* ─── host side of layer 2 ────────────────────────────────────────────── */
 
+static hipError_t raise_all_lds_ceilings(void);
+
 static int g_device = -1;
 static hipStream_t g_stream = nullptr;
 static int g_n_cu = 0;
@@ -287,6 +289,7 @@ extern "C" int oxh_init(int device)
     HIP_TRY(hipGetDeviceProperties(&prop, device));
     g_n_cu = prop.multiProcessorCount;
     HIP_TRY(hipStreamCreateWithFlags(&g_stream, hipStreamNonBlocking));
+    HIP_TRY(raise_all_lds_ceilings());
     g_device = device;
     return OXH_OK;
 }
@@ -391,6 +394,31 @@ extern "C" int oxh_quantize_q8_0(const float *d_x, size_t in_stride, size_t n_ve
     return OXH_OK;
 }
 
+/* gfx950 has 160 KiB of LDS per CU; one workgroup may take all of it once the
+ * kernel's dynamic-LDS ceiling is raised (done once in oxh_init). */
+#define GEMV_LDS_LIMIT (160u * 1024u)
+
+template <typename K>
+static hipError_t raise_lds_ceiling(K kernel)
+{
+    return hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)GEMV_LDS_LIMIT);
+}
+
+static hipError_t raise_all_lds_ceilings(void)
+{
+    hipError_t e;
+#define OXH_RAISE(KERNEL)                                                     \
+    if ((e = raise_lds_ceiling(KERNEL<0, true>)) != hipSuccess) return e;     \
+    if ((e = raise_lds_ceiling(KERNEL<1, false>)) != hipSuccess) return e;    \
+    if ((e = raise_lds_ceiling(KERNEL<0, false>)) != hipSuccess) return e;
+    OXH_RAISE(k_gemv_q4_k)
+    OXH_RAISE(k_gemv_q6_k)
+    OXH_RAISE(k_gemv_q8_0)
+#undef OXH_RAISE
+    return hipSuccess;
+}
+
 static bool is_q4k(uint32_t qtype) { return qtype == OXH_Q4_K_S || qtype == OXH_Q4_K_M; }
 
 static uint32_t act_lds_bytes(uint32_t qtype, uint32_t blocks)
@@ -440,7 +468,7 @@ extern "C" size_t oxh_gemv_max_nvec(uint32_t qtype, size_t cols)
     const size_t blocks = kind == 2 ? cols / OXH_QK_K : cols / OXH_QK8_0;
     if (blocks > 0xFFFFu) return 0;
     size_t nv = OXH_MAX_NV;
-    while (nv > 0 && gemv_lds_bytes(qtype, (uint32_t)blocks, nv, 1, 1) > 65536u) nv--;
+    while (nv > 0 && gemv_lds_bytes(qtype, (uint32_t)blocks, nv, 1, 1) > GEMV_LDS_LIMIT) nv--;
     return nv;
 }
 
@@ -460,6 +488,7 @@ static int launch_gemv(uint32_t qtype, const OxhSegment *segs, size_t n_segs, si
     if (n_segs == 0) return OXH_OK;
     if (!segs || (!io.d_acts && !io.d_x)) return arg_fail("gemv: NULL pointer");
     if (n_vec < 1 || n_vec > OXH_MAX_NV) return arg_fail("gemv: n_vec must be 1..8");
+    const size_t n_vec_default = n_vec;
     if (n_segs > OXH_MAX_SEGS) return arg_fail("gemv: more than 32 segments in one launch");
     const int kind = oxh_act_kind(qtype, cols);
     if (!kind) {
@@ -473,13 +502,23 @@ static int launch_gemv(uint32_t qtype, const OxhSegment *segs, size_t n_segs, si
     }
     if (io.d_x && io.x_stride < cols) return arg_fail("gemv: x_stride < cols");
     size_t total_rows = 0, max_act = 0;
+    /* a segment may carry its own activation count; the launch value is the default */
+    size_t max_nv = 0;
+    bool all_one = true;
     for (size_t i = 0; i < n_segs; i++) {
+        const size_t nv = segs[i].n_vec ? segs[i].n_vec : n_vec;
+        if (nv < 1 || nv > OXH_MAX_NV) return arg_fail("gemv: segment n_vec must be 1..8");
+        if (segs[i].rows) {
+            if (nv > max_nv) max_nv = nv;
+            if (nv != 1) all_one = false;
+        }
         if (segs[i].rows > 0x7FFFFFFFull / (blocks * 16u)) return arg_fail("gemv: segment too large");
         if (segs[i].rows && (!segs[i].d_w || !segs[i].d_out)) return arg_fail("gemv: NULL segment pointer");
         total_rows += segs[i].rows;
         if (segs[i].act_first > max_act) max_act = segs[i].act_first;
     }
     if (total_rows == 0) return OXH_OK;
+    n_vec = max_nv;                        /* sizes LDS from here on */
     if (out_stride > 0xFFFFFFFFull || io.x_stride > 0xFFFFFFFFull || max_act + n_vec > 0xFFFFFFFFull)
         return arg_fail("gemv: stride too large");
 
@@ -505,10 +544,10 @@ static int launch_gemv(uint32_t qtype, const OxhSegment *segs, size_t n_segs, si
             const uint32_t rpw = (uint32_t)((rows + share * W - 1) / (share * W));   /* q + (rem != 0) */
             if (rpw > rows_cap) rows_cap = rpw;
         }
-        if (gemv_lds_bytes(qtype, (uint32_t)blocks, n_vec, W, rows_cap) <= 65536u) break;
+        if (gemv_lds_bytes(qtype, (uint32_t)blocks, n_vec, W, rows_cap) <= GEMV_LDS_LIMIT) break;
         if (cap_limit > 1) { cap_limit = rows_cap > 1 ? rows_cap - 1 : 1; continue; }
         if (W > 1) { W /= 2; cap_limit = GEMV_ROWS_CAP; continue; }
-        snprintf(g_err, sizeof g_err, "gemv: cols %zu x n_vec %zu does not fit 64 KiB of LDS", cols, n_vec);
+        snprintf(g_err, sizeof g_err, "gemv: cols %zu x n_vec %zu does not fit 160 KiB of LDS", cols, n_vec);
         return OXH_ERR_TOO_WIDE;
     }
     const size_t lds = gemv_lds_bytes(qtype, (uint32_t)blocks, n_vec, W, rows_cap);
@@ -517,7 +556,6 @@ static int launch_gemv(uint32_t qtype, const OxhSegment *segs, size_t n_segs, si
     memset(&p, 0, sizeof p);
     p.blocks = (uint32_t)blocks;
     p.magic = (uint32_t)((0x100000000ull + blocks - 1u) / blocks);
-    p.n_vec = (uint32_t)n_vec;
     p.act_bytes = (uint32_t)oxh_act_bytes(qtype, cols);
     p.out_stride = (uint32_t)out_stride;
     p.term_stride = p.blocks + 1u;
@@ -536,6 +574,7 @@ static int launch_gemv(uint32_t qtype, const OxhSegment *segs, size_t n_segs, si
         t.out[n] = segs[i].d_out;
         t.rows[n] = (uint32_t)segs[i].rows;
         t.act_first[n] = (uint32_t)segs[i].act_first;
+        t.nv[n] = (uint32_t)(segs[i].n_vec ? segs[i].n_vec : n_vec_default);
         t.wg_begin[n] = wg;
         t.rows_q[n] = (uint32_t)(segs[i].rows / ((size_t)n_wg[i] * W));
         t.rows_rem[n] = (uint32_t)(segs[i].rows % ((size_t)n_wg[i] * W));
@@ -551,7 +590,7 @@ static int launch_gemv(uint32_t qtype, const OxhSegment *segs, size_t n_segs, si
 #define OXH_LAUNCH(KERNEL)                                                              \
     do {                                                                                \
         if (dump)            hipLaunchKernelGGL((KERNEL<0, true>), grid, block, lds, st, t, p, a);  \
-        else if (n_vec == 1) hipLaunchKernelGGL((KERNEL<1, false>), grid, block, lds, st, t, p, a); \
+        else if (all_one)    hipLaunchKernelGGL((KERNEL<1, false>), grid, block, lds, st, t, p, a); \
         else                 hipLaunchKernelGGL((KERNEL<0, false>), grid, block, lds, st, t, p, a); \
     } while (0)
     if (is_q4k(qtype))          OXH_LAUNCH(k_gemv_q4_k);
@@ -590,7 +629,7 @@ extern "C" int oxh_debug_subblock_sums(uint32_t qtype, const void *d_w, size_t r
     if (rc) return rc;
     float *scratch = nullptr;
     HIP_TRY(hipMalloc((void **)&scratch, (rows ? rows : 1) * sizeof(float)));
-    OxhSegment s = { d_w, scratch, rows, 0 };
+    OxhSegment s = { d_w, scratch, rows, 0, 0 };
     const GemvIo io = { d_act, nullptr, 0, nullptr };
     rc = launch_gemv(qtype, &s, 1, cols, io, 1, rows, d_sums, stream);
     hipError_t e = hipStreamSynchronize(pick_stream(stream));

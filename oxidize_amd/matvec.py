@@ -128,11 +128,13 @@ def quantize(qtype, d_x, in_stride, n_vec, cols, d_act, stream=None):
 
 
 def make_segments(items):
-    """items: iterable of (d_w, d_out, rows, act_first) with integer addresses."""
+    """items: iterable of (d_w, d_out, rows, act_first[, n_vec]) with integer
+    addresses; n_vec 0/omitted = the launch's n_vec."""
     items = list(items)
     segs = (OxhSegment * len(items))()
-    for s, (w, o, r, a) in zip(segs, items):
-        s.d_w, s.d_out, s.rows, s.act_first = w, o, r, a
+    for s, it in zip(segs, items):
+        s.d_w, s.d_out, s.rows, s.act_first = it[0], it[1], it[2], it[3]
+        s.n_vec = it[4] if len(it) > 4 else 0
     return segs
 
 

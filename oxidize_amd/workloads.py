@@ -108,3 +108,107 @@ class DecodeSet:
     def activation(self, layer, op):
         _, qt, _, cols, _ = self.ops[op]
         return self.act[layer][op].download(np.uint8, mv.act_bytes(qt, cols))
+
+
+def route_top_k(logits, k=2, renorm=True):
+    """Token -> expert routing as the reference's MoE layers do it
+    (llama.c:5965-6031): softmax over the expert logits, the k largest
+    probabilities by repeated strict-greater scan (ties keep the lower index),
+    gate weights renormalised over the selected experts.  Host-side caller
+    logic, not part of the matmul path; it only decides which GEMVs run."""
+    logits = np.asarray(logits, dtype=np.float32)
+    n_tok, n_exp = logits.shape
+    ids = np.zeros((n_tok, k), np.int32)
+    wts = np.zeros((n_tok, k), np.float32)
+    for t in range(n_tok):
+        p = np.exp(logits[t] - logits[t].max()).astype(np.float32)
+        p = (p * np.float32(1.0 / float(p.astype(np.float64).sum()))).astype(np.float32)
+        order = list(range(n_exp))
+        for i in range(k):
+            best = i
+            for c in range(i + 1, n_exp):
+                if p[order[c]] > p[order[best]]:
+                    best = c
+            order[i], order[best] = order[best], order[i]
+            ids[t, i] = order[i]
+        sel = p[ids[t]].astype(np.float64)
+        norm = sel.sum() if renorm else 1.0
+        wts[t] = (sel / (norm if norm > 0 else 1.0)).astype(np.float32)
+    return ids, wts
+
+
+def group_by_expert(ids, n_expert):
+    """Counting sort of the (token, slot) pairs by expert, token order kept
+    inside an expert (llama.c:6060-6069).  Returns (offsets[n_expert+1],
+    token index per sorted pair)."""
+    pairs = [(int(e), t) for t in range(ids.shape[0]) for e in ids[t]]
+    counts = np.bincount([e for e, _ in pairs], minlength=n_expert)
+    offsets = np.concatenate([[0], np.cumsum(counts)]).astype(np.int64)
+    fill = offsets[:-1].copy()
+    tok = np.zeros(len(pairs), np.int64)
+    for e, t in pairs:
+        tok[fill[e]] = t
+        fill[e] += 1
+    return offsets, tok
+
+
+class MoESet:
+    """Mixtral-8x7B-shaped expert GEMVs: 8 experts, top-2 routing of 16 decode
+    tokens; gate/up 14336 x 4096 and down 4096 x 14336 per expert, all Q4_K,
+    stacked expert-major as the reference stores them (llama.c:4248-4251).
+    Every expert's matrices are applied only to the tokens routed to it: ONE
+    launch for all experts' gate+up, ONE for all experts' down, each expert a
+    segment with its own activation count."""
+
+    def __init__(self, n_expert=8, top_k=2, n_tok=16, hidden=4096, ffn=14336, seed=0, keep_host=False):
+        self.n_expert, self.top_k, self.n_tok = n_expert, top_k, n_tok
+        self.hidden, self.ffn = hidden, ffn
+        self.logits = synth.normal(n_tok * n_expert, seed=seed, stream=4242).reshape(n_tok, n_expert)
+        self.ids, self.gate_w = route_top_k(self.logits, top_k)
+        self.offsets, self.pair_tok = group_by_expert(self.ids, n_expert)
+        n_pairs = n_tok * top_k
+        rb_gu, rb_dn = synth.row_bytes(Q4K, hidden), synth.row_bytes(Q4K, ffn)
+        self.host = {}
+        self.w = {}
+        for name, rows, cols, stream in (("gate", ffn, hidden, 700), ("up", ffn, hidden, 701),
+                                         ("down", hidden, ffn, 702)):
+            w = synth.weights(Q4K, n_expert * rows, cols, seed=seed, stream=stream)
+            self.w[name] = mv.DeviceBuffer.from_host(w)
+            if keep_host:
+                self.host[name] = w
+        self.x_tok = synth.normal(n_tok * hidden, seed=seed, stream=4300).reshape(n_tok, hidden)
+        self.xg = np.ascontiguousarray(self.x_tok[self.pair_tok])            # gathered per pair
+        self.h = synth.normal(n_pairs * ffn, seed=seed, stream=4301).reshape(n_pairs, ffn)
+        self.d_xg = mv.DeviceBuffer.from_host(self.xg)
+        self.d_h = mv.DeviceBuffer.from_host(self.h)
+        self.d_gate = mv.DeviceBuffer(n_pairs * ffn * 4)
+        self.d_up = mv.DeviceBuffer(n_pairs * ffn * 4)
+        self.d_down = mv.DeviceBuffer(n_pairs * hidden * 4)
+        gu, dn = [], []
+        self.hit = 0
+        for e in range(n_expert):
+            lo, hi = int(self.offsets[e]), int(self.offsets[e + 1])
+            if hi > lo:
+                self.hit += 1
+            for c0 in range(lo, hi, 8):
+                m = min(8, hi - c0)
+                gu.append((self.w["gate"].ptr + e * ffn * rb_gu, self.d_gate.ptr + c0 * ffn * 4, ffn, c0, m))
+                gu.append((self.w["up"].ptr + e * ffn * rb_gu, self.d_up.ptr + c0 * ffn * 4, ffn, c0, m))
+                dn.append((self.w["down"].ptr + e * hidden * rb_dn, self.d_down.ptr + c0 * hidden * 4, hidden, c0, m))
+        self.seg_gu = [mv.make_segments(gu[i:i + 32]) for i in range(0, len(gu), 32)]
+        self.seg_dn = [mv.make_segments(dn[i:i + 32]) for i in range(0, len(dn), 32)]
+        per_expert = (2 * ffn * rb_gu + hidden * rb_dn)
+        self.bytes_per_step = self.hit * per_expert + n_pairs * 4 * (hidden + 2 * ffn + ffn + hidden)
+        self.ops_per_step = n_pairs * 2 * 3 * ffn * hidden
+
+    def launch_step(self, stream=None):
+        for segs in self.seg_gu:
+            mv.gemv_segments_f32(Q4K, segs, self.hidden, self.d_xg.ptr, self.hidden, None, 1, self.ffn, stream)
+        for segs in self.seg_dn:
+            mv.gemv_segments_f32(Q4K, segs, self.ffn, self.d_h.ptr, self.ffn, None, 1, self.hidden, stream)
+
+    def outputs(self):
+        n_pairs = self.n_tok * self.top_k
+        return (self.d_gate.download(np.float32, n_pairs * self.ffn).reshape(n_pairs, self.ffn),
+                self.d_up.download(np.float32, n_pairs * self.ffn).reshape(n_pairs, self.ffn),
+                self.d_down.download(np.float32, n_pairs * self.hidden).reshape(n_pairs, self.hidden))

@@ -1,0 +1,168 @@
+"""GPU parity at the benchmark configurations' real shapes, through the C ABI.
+
+  config 0   Q4_K 4096x4096, seed 0: outputs and activation bytes against the
+             checksums taken from the compiled reference (tests/golden)
+  config 1   one full Llama-3-8B layer of the decode set (qkv, o, gate/up, down)
+             bit-exact against the oracle, plus a determinism check over layers
+  config 2   Q8_0 lm_head 151936x896 with batch 1 and 8
+  config 3   MMQ prefill 512 x 4096 against 14336/4096 rows: sampled tokens
+             bit-exact against the oracle, linearity-free property: every
+             token's output equals the single-vector GEMV of that token
+  config 4   Mixtral-shaped expert GEMVs (8 experts, top-2, 16 tokens)
+"""
+import os
+import zlib
+
+import numpy as np
+import pytest
+
+import oxlibs
+from oxidize_amd import matvec as mv
+from oxidize_amd import synth, workloads
+
+pytestmark = pytest.mark.gpu
+GOLD = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+Q80, Q4K, Q6K = 7, 13, 16
+
+
+def bits(a):
+    return np.ascontiguousarray(a).view(np.uint32)
+
+
+def oracle_matvec(qtype, w, rows, cols, x):
+    o = oxlibs.oracle()
+    out = np.zeros(rows, np.float32)
+    temp = np.zeros(cols, np.float32)
+    assert o.oxo_matvec_quantized(qtype, w.ctypes.data, rows, cols, synth.row_bytes(qtype, cols),
+                                  x.ctypes.data, out.ctypes.data, temp.ctypes.data) == 0
+    return out, temp
+
+
+@pytest.mark.parametrize("name,qt,rows,cols", [("cfg0_q4k_4096x4096", Q4K, 4096, 4096),
+                                               ("down_q6k_4096x14336", Q6K, 4096, 14336),
+                                               ("ffn_q80_4864x896", Q80, 4864, 896)])
+def test_config0_against_reference_checksums(oxh, name, qt, rows, cols):
+    g = np.load(os.path.join(GOLD, "full_size.npz"))
+    w = synth.weights(qt, rows, cols, seed=0, stream=0)
+    x = synth.normal(cols, seed=0, stream=1000)
+    out = np.zeros(rows, np.float32)
+    temp = np.zeros(cols, np.float32)
+    assert mv.matvec_quantized(qt, w, rows, cols, synth.row_bytes(qt, cols), x, out, temp) == 0
+    nact = mv.act_bytes(qt, cols)
+    assert zlib.crc32(temp.view(np.uint8)[:nact].tobytes()) == int(g[name + "_crc_act"][0])
+    if qt == Q80:
+        ref = g[name + "_out"]
+        assert np.all(np.abs(out - ref) <= 1e-4 + 1e-5 * np.abs(ref))
+    else:
+        assert zlib.crc32(out.tobytes()) == int(g[name + "_crc_out"][0])
+        assert np.array_equal(bits(out), bits(g[name + "_out"]))
+
+
+def test_config1_decode_layer_bit_exact_and_repeatable(oxh):
+    ds = workloads.DecodeSet(layers=2, seed=0, keep_host=(0, 1))
+    ds.launch_step()
+    mv.sync()
+    first = [[ds.output(layer, op) for op in range(4)] for layer in range(2)]
+    for layer in range(2):
+        for op, (name, qt, rows, cols, _) in enumerate(ds.ops):
+            x = ds.x_host[(layer, op)]
+            off = 0
+            o = oxlibs.oracle()
+            act = np.zeros(mv.act_bytes(qt, cols), np.uint8)
+            o.oxo_quantize_q8_k(x.ctypes.data, cols, act.ctypes.data)
+            assert np.array_equal(ds.activation(layer, op), act), (layer, name)
+            for seg, r in enumerate(rows):
+                want, _ = oracle_matvec(qt, ds.host[(layer, op, seg)], r, cols, x)
+                assert np.array_equal(bits(first[layer][op][off:off + r]), bits(want)), (layer, name, seg)
+                off += r
+    # replay through a HIP graph: identical bits every time
+    g = mv.Graph()
+    with g:
+        ds.launch_step()
+    for _ in range(3):
+        g.launch()
+        mv.sync()
+        for layer in range(2):
+            for op in range(4):
+                assert np.array_equal(bits(ds.output(layer, op)), bits(first[layer][op]))
+    g.destroy()
+
+
+@pytest.mark.parametrize("n_vec", [1, 8])
+def test_config2_q8_0_lm_head(oxh, n_vec):
+    rows, cols = 151936, 896
+    w = synth.weights(Q80, rows, cols, seed=0, stream=5)
+    xs = synth.normal(n_vec * cols, seed=0, stream=6).reshape(n_vec, cols)
+    outs = np.zeros((n_vec, rows), np.float32)
+    temp = np.zeros(cols, np.float32)
+    scratch = np.zeros(mv.batch_scratch_bytes(cols), np.uint8)
+    assert mv.matvec_quantized_batch(Q80, w, rows, cols, synth.row_bytes(Q80, cols), xs, cols, outs,
+                                     rows, n_vec, temp, scratch) == 0
+    for v in range(n_vec):
+        want, _ = oracle_matvec(Q80, w, rows, cols, np.ascontiguousarray(xs[v]))
+        assert np.array_equal(bits(outs[v]), bits(want))
+    ref = oxlibs.ref()
+    if ref is not None:
+        r_out = np.zeros(rows, np.float32)
+        ref.oc_matvec_quantized(Q80, w.ctypes.data, rows, cols, synth.row_bytes(Q80, cols),
+                                xs[0].ctypes.data, r_out.ctypes.data, temp.ctypes.data)
+        assert np.all(np.abs(outs[0] - r_out) <= 1e-4 + 1e-5 * np.abs(r_out))
+
+
+@pytest.mark.parametrize("rows", [14336, 4096])
+def test_config3_mmq_prefill_512_tokens(oxh, rows):
+    cols, n_vec = 4096, 512
+    w = synth.weights(Q4K, rows, cols, seed=0, stream=0)
+    xs = synth.normal(n_vec * cols, seed=0, stream=2000).reshape(n_vec, cols)
+    d_w = mv.DeviceBuffer.from_host(w)
+    d_x = mv.DeviceBuffer.from_host(xs)
+    nact = mv.act_bytes(Q4K, cols)
+    d_a = mv.DeviceBuffer(n_vec * nact)
+    d_o = mv.DeviceBuffer(n_vec * rows * 4)
+    mv.quantize(Q4K, d_x.ptr, cols, n_vec, cols, d_a.ptr)
+    mv.mmq(Q4K, d_w.ptr, rows, cols, d_a.ptr, n_vec, d_o.ptr, rows)
+    out = d_o.download(np.float32, n_vec * rows).reshape(n_vec, rows)
+    acts = d_a.download(np.uint8, n_vec * nact).reshape(n_vec, nact)
+    o = oxlibs.oracle()
+    for v in (0, 1, 31, 32, 63, 64, 255, 300, 511):
+        want, wtemp = oracle_matvec(Q4K, w, rows, cols, np.ascontiguousarray(xs[v]))
+        assert np.array_equal(acts[v], wtemp.view(np.uint8)[:nact]), v
+        assert np.array_equal(bits(out[v]), bits(want)), v
+    # every token, a slice of rows: the MFMA path against the GEMV kernel on the same device data
+    d_o2 = mv.DeviceBuffer(8 * rows * 4)
+    for v0 in (8, 120, 504):
+        segs = mv.make_segments([(d_w.ptr, d_o2.ptr, rows, v0)])
+        mv.gemv_segments(Q4K, segs, cols, d_a.ptr, 8, rows)
+        got = d_o2.download(np.float32, 8 * rows).reshape(8, rows)
+        assert np.array_equal(bits(got), bits(out[v0:v0 + 8]))
+
+
+def test_config4_moe_expert_gemvs(oxh):
+    ms = workloads.MoESet(seed=0, keep_host=True)
+    o = oxlibs.oracle()
+    ids = np.zeros((16, 2), np.int32)
+    wts = np.zeros((16, 2), np.float32)
+    o.oxo_moe_route(ms.logits.ctypes.data, 16, 8, 2, 1, ids.ctypes.data, wts.ctypes.data)
+    assert np.array_equal(ids, ms.ids)
+    assert np.allclose(wts, ms.gate_w, rtol=1e-6)
+    assert ms.offsets[-1] == 32 and sorted(ms.pair_tok[:ms.offsets[1]]) == list(ms.pair_tok[:ms.offsets[1]])
+    ms.launch_step()
+    mv.sync()
+    gate, up, down = ms.outputs()
+    rb_gu, rb_dn = synth.row_bytes(Q4K, 4096), synth.row_bytes(Q4K, 14336)
+    rng = np.random.default_rng(0)
+    for e in range(8):
+        lo, hi = int(ms.offsets[e]), int(ms.offsets[e + 1])
+        for pidx in range(lo, hi):
+            if rng.random() > 0.4 and pidx not in (lo, hi - 1):
+                continue
+            wg = ms.host["gate"][e * 14336 * rb_gu:(e + 1) * 14336 * rb_gu]
+            wu = ms.host["up"][e * 14336 * rb_gu:(e + 1) * 14336 * rb_gu]
+            wd = ms.host["down"][e * 4096 * rb_dn:(e + 1) * 4096 * rb_dn]
+            x = np.ascontiguousarray(ms.xg[pidx])
+            assert np.array_equal(x, ms.x_tok[ms.pair_tok[pidx]])
+            assert e in ms.ids[ms.pair_tok[pidx]]
+            assert np.array_equal(bits(gate[pidx]), bits(oracle_matvec(Q4K, wg, 14336, 4096, x)[0]))
+            assert np.array_equal(bits(up[pidx]), bits(oracle_matvec(Q4K, wu, 14336, 4096, x)[0]))
+            h = np.ascontiguousarray(ms.h[pidx])
+            assert np.array_equal(bits(down[pidx]), bits(oracle_matvec(Q4K, wd, 4096, 14336, h)[0]))
