@@ -416,6 +416,7 @@ static hipError_t raise_all_lds_ceilings(void)
     OXH_RAISE(k_gemv_q6_k)
     OXH_RAISE(k_gemv_q8_0)
 #undef OXH_RAISE
+    if ((e = raise_lds_ceiling(k_mmq_q4_k)) != hipSuccess) return e;
     return hipSuccess;
 }
 
@@ -657,7 +658,7 @@ extern "C" int oxh_mmq(uint32_t qtype, const void *d_w, size_t rows, size_t cols
         return arg_fail("oxh_mmq: dimension too large");
     const dim3 grid((uint32_t)((rows + MMQ_ROWS - 1) / MMQ_ROWS),
                     (uint32_t)((n_vec + MMQ_TOK - 1) / MMQ_TOK));
-    hipLaunchKernelGGL(k_mmq_q4_k, grid, dim3(MMQ_WAVES * 64), 0, pick_stream(stream),
+    hipLaunchKernelGGL(k_mmq_q4_k, grid, dim3(MMQ_WAVES * 64), MMQ_LDS_BYTES, pick_stream(stream),
                        (const uint8_t *)d_w, (uint32_t)rows, (uint32_t)blocks,
                        (const uint8_t *)d_acts, (uint32_t)n_vec, d_out, out_stride);
     HIP_TRY(hipGetLastError());
