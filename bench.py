@@ -25,6 +25,112 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
+# HBM bytes one gate/up launch moves, from two rocprofv3 --pmc runs (FETCH_SIZE
+# 32407.5 KiB x 2.000, WRITE_SIZE 116.58 KiB x 1.000; the factors are what the
+# same counters read for a 256 MiB device-to-device copy).  Not measured live.
+GATE_UP_TRAFFIC_BYTES = 66489528
+INT8_PEAK_TOPS = 5033.0     # dense int8 MFMA: 256 CU x 2.4 GHz x 8192 op/clk/CU
+
+
+def timed(fn, reps, mv):
+    """Average microseconds of fn() over `reps` back-to-back calls (HIP events)."""
+    fn()
+    mv.sync()
+    e0, e1 = mv.Event(), mv.Event()
+    e0.record()
+    for _ in range(reps):
+        fn()
+    e1.record()
+    mv.sync()
+    return e1.ms_since(e0) * 1e3 / reps
+
+
+def secondary_figures(mv, synth):
+    """The other benchmark configurations, measured the same way (inputs
+    resident, HIP events on the launch stream).  Reported next to the headline
+    figure, never folded into it."""
+    from oxidize_amd.workloads import MoESet
+    out = {}
+    Q80, Q4K = 7, 13
+    # MMQ prefill (configuration 3): 512 tokens, Q4_K 14336x4096 and 4096x4096
+    cols, n_vec = 4096, 512
+    x = synth.normal(n_vec * cols, seed=0, stream=2000)
+    d_x = mv.DeviceBuffer.from_host(x)
+    d_a = mv.DeviceBuffer(n_vec * mv.act_bytes(Q4K, cols))
+    mmq = {}
+    for rows in (14336, 4096):
+        w = synth.weights(Q4K, rows, cols, seed=0, stream=0)
+        copies = [mv.DeviceBuffer.from_host(w) for _ in range(3)]
+        d_o = mv.DeviceBuffer(n_vec * rows * 4)
+        state = {"i": 0}
+
+        def run():
+            state["i"] += 1
+            mv.quantize(Q4K, d_x.ptr, cols, n_vec, cols, d_a.ptr)
+            mv.mmq(Q4K, copies[state["i"] % 3].ptr, rows, cols, d_a.ptr, n_vec, d_o.ptr, rows)
+
+        us = timed(run, 12, mv)
+        ops = 2.0 * rows * cols * n_vec
+        mmq["%dx%dx%d" % (rows, cols, n_vec)] = {
+            "us": round(us, 2), "tops": round(ops / us / 1e6, 1),
+            "frac_of_int8_peak": round(ops / us / 1e6 / INT8_PEAK_TOPS, 4),
+            "includes": "Q8_K quantisation of the 512 activations + k_mmq_q4_k"}
+        for c in copies:
+            c.free()
+    out["mmq_prefill_q4k"] = mmq
+    d_x.free()
+    d_a.free()
+    # Q8_0 lm_head (configuration 2), batch 1 and 8
+    rows, cols = 151936, 896
+    w = synth.weights(Q80, rows, cols, seed=0, stream=5)
+    copies = [mv.DeviceBuffer.from_host(w) for _ in range(3)]
+    q8 = {}
+    for nv in (1, 8):
+        xs = synth.normal(nv * cols, seed=0, stream=6)
+        d_x = mv.DeviceBuffer.from_host(xs)
+        d_o = mv.DeviceBuffer(nv * rows * 4)
+        state = {"i": 0}
+
+        def run():
+            state["i"] += 1
+            segs = mv.make_segments([(copies[state["i"] % 3].ptr, d_o.ptr, rows, 0)])
+            mv.gemv_segments_f32(Q80, segs, cols, d_x.ptr, cols, None, nv, rows)
+
+        us = timed(run, 12, mv)
+        nbytes = w.nbytes + nv * 4 * (cols + rows)
+        q8["batch%d" % nv] = {"us": round(us, 2), "gbps": round(nbytes / us / 1e3, 1),
+                              "frac_of_hbm_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBPS, 4)}
+        d_x.free()
+        d_o.free()
+    out["q8_0_lm_head_151936x896"] = q8
+    for c in copies:
+        c.free()
+    # Mixtral-shaped expert GEMVs (configuration 4)
+    ms = MoESet(seed=0)
+    us = timed(ms.launch_step, 10, mv)
+    out["moe_8x_top2_16tok_q4k"] = {
+        "us": round(us, 2), "experts_hit": ms.hit, "gbps": round(ms.bytes_per_step / us / 1e3, 1),
+        "frac_of_hbm_peak": round(ms.bytes_per_step / us / 1e3 / HBM_PEAK_GBPS, 4),
+        "note": "792.7 MB of expert weights fit the 256 MB last-level cache only in part; "
+                "two launches (all experts' gate+up, all experts' down)"}
+    return out
+
+
+def traffic_probe(mv, ds):
+    """For `rocprofv3 --pmc FETCH_SIZE` / `WRITE_SIZE` runs: three 256 MiB
+    device-to-device copies (a kernel of known traffic to scale the counters
+    by), then one gate/up GEMV per layer.  Prints nothing."""
+    import ctypes
+    from oxidize_amd import _lib
+    n = 256 << 20
+    a, b = mv.DeviceBuffer(n), mv.DeviceBuffer(n)
+    _lib.check(_lib.lib().oxh_memset(ctypes.c_void_p(a.ptr), 1, n, None))
+    for _ in range(3):
+        _lib.check(_lib.lib().oxh_memcpy_d2d(ctypes.c_void_p(b.ptr), ctypes.c_void_p(a.ptr), n, None))
+    mv.sync()
+    for layer in range(ds.layers):
+        ds.launch_op(layer, 2)
+    mv.sync()
 
 
 def cpu_baseline(layers_sample=1, min_seconds=1.5):
@@ -93,6 +199,8 @@ def main():
     ap.add_argument("--layers", type=int, default=32, help=argparse.SUPPRESS)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-graph", action="store_true", help="launch kernels one by one")
+    ap.add_argument("--no-extra", action="store_true", help="skip the secondary configurations")
+    ap.add_argument("--probe", choices=["traffic"], help="run a counter-collection workload and exit")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this path is built and measured on ONE GPU; --gpus %d is not supported "
@@ -109,6 +217,9 @@ def main():
 
     ds = DecodeSet(layers=args.layers, seed=0)
     step_bytes = ds.bytes_per_step
+    if args.probe == "traffic":
+        traffic_probe(mv, ds)
+        return 0
 
     graph = None
     if not args.no_graph:
@@ -181,9 +292,12 @@ def main():
         "device": info,
         "roofline": {"bound": "hbm", "kernel": "k_gemv_q4_k (gate/up 28672x4096)",
                      "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": GATE_UP_TRAFFIC_BYTES,
                      "bytes_per_launch": k_bytes, "us_per_launch": round(k_us, 3)},
     }
+    if not args.no_extra:
+        from oxidize_amd import synth
+        out["extra"] = secondary_figures(mv, synth)
     out["cpu_baseline"] = None if args.no_cpu else cpu_baseline()
     print(json.dumps(out))
     return 0

@@ -146,6 +146,7 @@ int  oxh_malloc(void **d_ptr, size_t bytes);
 int  oxh_free(void *d_ptr);
 int  oxh_memcpy_h2d(void *d_dst, const void *h_src, size_t bytes, void *stream);
 int  oxh_memcpy_d2h(void *h_dst, const void *d_src, size_t bytes, void *stream);
+int  oxh_memcpy_d2d(void *d_dst, const void *d_src, size_t bytes, void *stream);
 int  oxh_memset(void *d_dst, int value, size_t bytes, void *stream);
 int  oxh_stream_create(void **stream);
 int  oxh_stream_destroy(void *stream);

@@ -45,6 +45,7 @@ SIGNATURES = {
     "oxh_free": (I, [V]),
     "oxh_memcpy_h2d": (I, [V, V, Z, V]),
     "oxh_memcpy_d2h": (I, [V, V, Z, V]),
+    "oxh_memcpy_d2d": (I, [V, V, Z, V]),
     "oxh_memset": (I, [V, I, Z, V]),
     "oxh_stream_create": (I, [ctypes.POINTER(V)]),
     "oxh_stream_destroy": (I, [V]),

@@ -707,6 +707,15 @@ extern "C" int oxh_memcpy_d2h(void *h_dst, const void *d_src, size_t bytes, void
     return OXH_OK;
 }
 
+extern "C" int oxh_memcpy_d2d(void *d_dst, const void *d_src, size_t bytes, void *stream)
+{
+    int rc = ensure_init();
+    if (rc) return rc;
+    if (bytes == 0) return OXH_OK;
+    HIP_TRY(hipMemcpyAsync(d_dst, d_src, bytes, hipMemcpyDeviceToDevice, pick_stream(stream)));
+    return OXH_OK;
+}
+
 extern "C" int oxh_memset(void *d_dst, int value, size_t bytes, void *stream)
 {
     int rc = ensure_init();
