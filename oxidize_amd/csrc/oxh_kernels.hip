@@ -455,11 +455,18 @@ static uint32_t gemv_waves(void)
     return w;
 }
 
-static uint32_t gemv_wg_per_cu(void)
+/* One 16-wave workgroup per CU is resident at a time.  A launch sized at one
+ * workgroup per CU starts every wave at once, which is best while a wave has
+ * only a handful of passes; past ~8 passes per wave a second round of
+ * workgroups balances the tail better (measured: Q8_0 151936 x 896 goes from
+ * 50 us to 35 us, the Llama decode shapes are best at one). */
+static uint32_t gemv_wg_per_cu(size_t total_passes, uint32_t waves)
 {
-    static uint32_t w = 0;
-    if (!w) w = env_u32("OXH_GEMV_WG_PER_CU", 1, 1, 64);
-    return w;
+    static int forced = -1;
+    if (forced < 0) forced = (int)env_u32("OXH_GEMV_WG_PER_CU", 0, 0, 64);
+    if (forced > 0) return (uint32_t)forced;
+    const size_t one_round = (size_t)(g_n_cu > 0 ? g_n_cu : 256) * waves;
+    return total_passes > one_round * 8u ? 2u : 1u;
 }
 
 extern "C" size_t oxh_gemv_max_nvec(uint32_t qtype, size_t cols)
@@ -526,7 +533,9 @@ static int launch_gemv(uint32_t qtype, const OxhSegment *segs, size_t n_segs, si
     /* Deal workgroups to segments in proportion to their rows; every wave
      * then owns ceil(rows / waves) whole rows of its segment. */
     uint32_t W = gemv_waves();
-    const size_t target = (size_t)(g_n_cu > 0 ? g_n_cu : 256) * gemv_wg_per_cu();
+    const size_t blocks_per_pass = qtype == OXH_Q8_0 ? 64u : 16u;
+    const size_t target = (size_t)(g_n_cu > 0 ? g_n_cu : 256) *
+                          gemv_wg_per_cu(total_rows * blocks / blocks_per_pass, W);
     uint32_t cap_limit = GEMV_ROWS_CAP;
     uint32_t n_wg[OXH_MAX_SEGS];
     uint32_t rows_cap = 1;
