@@ -416,7 +416,9 @@ static hipError_t raise_all_lds_ceilings(void)
     OXH_RAISE(k_gemv_q6_k)
     OXH_RAISE(k_gemv_q8_0)
 #undef OXH_RAISE
-    if ((e = raise_lds_ceiling(k_mmq_q4_k)) != hipSuccess) return e;
+    if ((e = raise_lds_ceiling(k_mmq_q4_k<1>)) != hipSuccess) return e;
+    if ((e = raise_lds_ceiling(k_mmq_q4_k<2>)) != hipSuccess) return e;
+    if ((e = raise_lds_ceiling(k_mmq_q4_k<4>)) != hipSuccess) return e;
     return hipSuccess;
 }
 
@@ -665,11 +667,29 @@ extern "C" int oxh_mmq(uint32_t qtype, const void *d_w, size_t rows, size_t cols
     const size_t blocks = cols / OXH_QK_K;
     if (rows > 0x7FFFFFFFull || n_vec > 0x7FFFFFFFull || blocks > 0xFFFFFFull)
         return arg_fail("oxh_mmq: dimension too large");
-    const dim3 grid((uint32_t)((rows + MMQ_ROWS - 1) / MMQ_ROWS),
-                    (uint32_t)((n_vec + MMQ_TOK - 1) / MMQ_TOK));
-    hipLaunchKernelGGL(k_mmq_q4_k, grid, dim3(MMQ_WAVES * 64), MMQ_LDS_BYTES, pick_stream(stream),
-                       (const uint8_t *)d_w, (uint32_t)rows, (uint32_t)blocks,
-                       (const uint8_t *)d_acts, (uint32_t)n_vec, d_out, out_stride);
+    /* the kernel addresses a workgroup's 256 rows and 128 tokens with 32-bit lane offsets */
+    if (blocks * 292u * 128u > 0xFFFFFFFFull)
+        return arg_fail("oxh_mmq: cols too large");
+    const uint32_t row_tiles = (uint32_t)((rows + MMQ_ROWS - 1) / MMQ_ROWS);
+#define MMQ_LAUNCH(TT)                                                                              \
+    hipLaunchKernelGGL(k_mmq_q4_k<TT>, dim3(row_tiles, (uint32_t)((n_vec + 32u * TT - 1) / (32u * TT))), \
+                       dim3(MMQ_WAVES * 64), MmqGeom<TT>::LDS_BYTES, pick_stream(stream),            \
+                       (const uint8_t *)d_w, (uint32_t)rows, (uint32_t)blocks,                       \
+                       (const uint8_t *)d_acts, (uint32_t)n_vec, d_out, out_stride)
+    /* Token tiles per wave: four amortise the operand build best, but a launch
+     * needs about one workgroup per CU; take the largest count that still
+     * gives one, and never more tiles than the batch fills. */
+    const size_t cus = (size_t)(g_n_cu > 0 ? g_n_cu : 256);
+    const size_t need = cus - cus / 8;
+    int tt = 4;
+    while (tt > 1 && (n_vec <= 16u * (size_t)tt || row_tiles * ((n_vec + 32u * tt - 1) / (32u * tt)) < need)) tt >>= 1;
+    static int forced = -1;                 /* OXH_MMQ_TILES = 1, 2 or 4 overrides the choice */
+    if (forced < 0) forced = (int)env_u32("OXH_MMQ_TILES", 0, 0, 4);
+    if (forced == 1 || forced == 2 || forced == 4) tt = forced;
+    if (tt == 1) MMQ_LAUNCH(1);
+    else if (tt == 2) MMQ_LAUNCH(2);
+    else MMQ_LAUNCH(4);
+#undef MMQ_LAUNCH
     HIP_TRY(hipGetLastError());
     return OXH_OK;
 }
