@@ -28,7 +28,7 @@ HBM_PEAK_GBPS = 8000.0
 # HBM bytes one gate/up launch moves, from two rocprofv3 --pmc runs (FETCH_SIZE
 # 32407.5 KiB x 2.000, WRITE_SIZE 116.58 KiB x 1.000; the factors are what the
 # same counters read for a 256 MiB device-to-device copy).  Not measured live.
-GATE_UP_TRAFFIC_BYTES = 66489528
+GATE_UP_TRAFFIC_BYTES = 66497512
 INT8_PEAK_TOPS = 5033.0     # dense int8 MFMA: 256 CU x 2.4 GHz x 8192 op/clk/CU
 
 
@@ -69,12 +69,19 @@ def secondary_figures(mv, synth):
             mv.quantize(Q4K, d_x.ptr, cols, n_vec, cols, d_a.ptr)
             mv.mmq(Q4K, copies[state["i"] % 3].ptr, rows, cols, d_a.ptr, n_vec, d_o.ptr, rows)
 
+        def run_mma_only():
+            state["i"] += 1
+            mv.mmq(Q4K, copies[state["i"] % 3].ptr, rows, cols, d_a.ptr, n_vec, d_o.ptr, rows)
+
         us = timed(run, 12, mv)
+        us_mma = timed(run_mma_only, 12, mv)
         ops = 2.0 * rows * cols * n_vec
         mmq["%dx%dx%d" % (rows, cols, n_vec)] = {
             "us": round(us, 2), "tops": round(ops / us / 1e6, 1),
             "frac_of_int8_peak": round(ops / us / 1e6 / INT8_PEAK_TOPS, 4),
-            "includes": "Q8_K quantisation of the 512 activations + k_mmq_q4_k"}
+            "includes": "Q8_K quantisation of the 512 activations + k_mmq_q4_k",
+            "mfma_kernel_only_us": round(us_mma, 2),
+            "mfma_kernel_only_frac_of_int8_peak": round(ops / us_mma / 1e6 / INT8_PEAK_TOPS, 4)}
         for c in copies:
             c.free()
     out["mmq_prefill_q4k"] = mmq
@@ -133,7 +140,22 @@ def traffic_probe(mv, ds):
     mv.sync()
 
 
-def cpu_baseline(layers_sample=1, min_seconds=1.5):
+def mmq_probe(mv, synth):
+    """For `rocprofv3 --pmc` runs on the MFMA kernel: quantise 512 activations
+    of 4096 values, then three 14336 x 4096 x 512 launches.  Prints nothing."""
+    Q4K = 13
+    rows, cols, n_vec = 14336, 4096, 512
+    d_w = mv.DeviceBuffer.from_host(synth.weights(Q4K, rows, cols, seed=0, stream=0))
+    d_x = mv.DeviceBuffer.from_host(synth.normal(n_vec * cols, seed=0, stream=2000))
+    d_a = mv.DeviceBuffer(n_vec * mv.act_bytes(Q4K, cols))
+    d_o = mv.DeviceBuffer(n_vec * rows * 4)
+    mv.quantize(Q4K, d_x.ptr, cols, n_vec, cols, d_a.ptr)
+    for _ in range(3):
+        mv.mmq(Q4K, d_w.ptr, rows, cols, d_a.ptr, n_vec, d_o.ptr, rows)
+    mv.sync()
+
+
+def cpu_baseline(layers_sample=1, min_seconds=2.5):
     """The reference CPU path on the host cores over `layers_sample` layers of
     the same workload (same shapes, same synthetic generator)."""
     import ctypes
@@ -200,7 +222,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-graph", action="store_true", help="launch kernels one by one")
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary configurations")
-    ap.add_argument("--probe", choices=["traffic"], help="run a counter-collection workload and exit")
+    ap.add_argument("--probe", choices=["traffic", "mmq"], help="run a counter-collection workload and exit")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this path is built and measured on ONE GPU; --gpus %d is not supported "
@@ -214,6 +236,11 @@ def main():
     lib = _lib.lib()
     _lib.check(lib.oxh_init(0))
     info = mv.device_info()
+
+    if args.probe == "mmq":
+        from oxidize_amd import synth
+        mmq_probe(mv, synth)
+        return 0
 
     ds = DecodeSet(layers=args.layers, seed=0)
     step_bytes = ds.bytes_per_step
