@@ -119,7 +119,8 @@ def secondary_figures(mv, synth):
         "us": round(us, 2), "experts_hit": ms.hit, "gbps": round(ms.bytes_per_step / us / 1e3, 1),
         "frac_of_hbm_peak": round(ms.bytes_per_step / us / 1e3 / HBM_PEAK_GBPS, 4),
         "note": "792.7 MB of expert weights fit the 256 MB last-level cache only in part; "
-                "two launches (all experts' gate+up, all experts' down)"}
+                "per step: Q8_K quantisation + one MFMA launch for all experts' gate+up, the same for "
+                "all experts' down, each expert over its own tokens only"}
     return out
 
 

@@ -416,9 +416,9 @@ static hipError_t raise_all_lds_ceilings(void)
     OXH_RAISE(k_gemv_q6_k)
     OXH_RAISE(k_gemv_q8_0)
 #undef OXH_RAISE
-    if ((e = raise_lds_ceiling(k_mmq_q4_k<1>)) != hipSuccess) return e;
-    if ((e = raise_lds_ceiling(k_mmq_q4_k<2>)) != hipSuccess) return e;
-    if ((e = raise_lds_ceiling(k_mmq_q4_k<4>)) != hipSuccess) return e;
+    if ((e = raise_lds_ceiling(k_mmq_q4_k<2, 2, 8>)) != hipSuccess) return e;
+    if ((e = raise_lds_ceiling(k_mmq_q4_k<4, 2, 8>)) != hipSuccess) return e;
+    if ((e = raise_lds_ceiling(k_mmq_q4_k<8, 2, 8>)) != hipSuccess) return e;
     return hipSuccess;
 }
 
@@ -489,6 +489,54 @@ struct GemvIo {
     void *d_act_out;        /* optional store of the quantised bytes         */
 };
 
+/* Q4_K with three or more activations per weight goes to the matrix cores:
+ * the dot-instruction GEMV repeats its integer work per activation and stops
+ * keeping up with the weight stream there (OXH_GEMV_MFMA_MIN_NV moves the
+ * threshold; 0 = never).  The MFMA kernel reads Q8_K activations, so an f32
+ * launch qualifies only if it has somewhere to put the quantised bytes. */
+static bool gemv_wants_mfma(uint32_t qtype, const GemvIo &io, size_t max_nv, const int32_t *dump)
+{
+    static int min_nv = -1;
+    if (min_nv < 0) min_nv = (int)env_u32("OXH_GEMV_MFMA_MIN_NV", 3, 0, 64);
+    if (!is_q4k(qtype) || dump || min_nv == 0 || max_nv < (size_t)min_nv) return false;
+    return io.d_acts != nullptr || io.d_act_out != nullptr;
+}
+
+static int launch_mmq_segments(const OxhSegment *segs, size_t n_segs, size_t cols, size_t blocks,
+                               const GemvIo &io, size_t n_vec_default, size_t n_acts,
+                               size_t out_stride, void *stream)
+{
+    typedef MmqGeom<1, 1, 4> G;
+    if (blocks * 292u * 256u > 0xFFFFFFFFull) return arg_fail("gemv: cols too large");
+    const uint8_t *acts = (const uint8_t *)io.d_acts;
+    if (!acts) {
+        int rc = oxh_quantize_q8_k(io.d_x, io.x_stride, n_acts, cols, io.d_act_out, stream);
+        if (rc) return rc;
+        acts = (const uint8_t *)io.d_act_out;
+    }
+    SegTable t;
+    memset(&t, 0, sizeof t);
+    uint32_t wg = 0, n = 0;
+    for (size_t i = 0; i < n_segs; i++) {
+        if (segs[i].rows == 0) continue;
+        t.w[n] = (const uint8_t *)segs[i].d_w;
+        t.out[n] = segs[i].d_out;
+        t.rows[n] = (uint32_t)segs[i].rows;
+        t.act_first[n] = (uint32_t)segs[i].act_first;
+        t.nv[n] = (uint32_t)(segs[i].n_vec ? segs[i].n_vec : n_vec_default);
+        t.wg_begin[n] = wg;
+        wg += (uint32_t)((segs[i].rows + G::ROWS - 1) / G::ROWS);
+        n++;
+    }
+    t.wg_begin[n] = wg;
+    t.n = n;
+    auto kernel = k_mmq_q4_k_segments<1, 1, 4>;
+    hipLaunchKernelGGL(kernel, dim3(wg), dim3(4 * 64), G::LDS_BYTES,
+                       pick_stream(stream), t, (uint32_t)blocks, acts, out_stride);
+    HIP_TRY(hipGetLastError());
+    return OXH_OK;
+}
+
 static int launch_gemv(uint32_t qtype, const OxhSegment *segs, size_t n_segs, size_t cols,
                        const GemvIo &io, size_t n_vec, size_t out_stride, int32_t *dump,
                        void *stream)
@@ -528,6 +576,9 @@ static int launch_gemv(uint32_t qtype, const OxhSegment *segs, size_t n_segs, si
         if (segs[i].act_first > max_act) max_act = segs[i].act_first;
     }
     if (total_rows == 0) return OXH_OK;
+    if (gemv_wants_mfma(qtype, io, max_nv, dump))
+        return launch_mmq_segments(segs, n_segs, cols, blocks, io, n_vec_default, max_act + max_nv,
+                                   out_stride, stream);
     n_vec = max_nv;                        /* sizes LDS from here on */
     if (out_stride > 0xFFFFFFFFull || io.x_stride > 0xFFFFFFFFull || max_act + n_vec > 0xFFFFFFFFull)
         return arg_fail("gemv: stride too large");
@@ -651,6 +702,18 @@ extern "C" int oxh_debug_subblock_sums(uint32_t qtype, const void *d_w, size_t r
     return OXH_OK;
 }
 
+template <int TC, int RC, int WAVES>
+static void mmq_launch(const void *d_w, size_t rows, size_t blocks, const void *d_acts, size_t n_vec,
+                       float *d_out, size_t out_stride, void *stream)
+{
+    typedef MmqGeom<TC, RC, WAVES> G;
+    const dim3 grid((uint32_t)((rows + G::ROWS - 1) / G::ROWS), (uint32_t)((n_vec + G::TOK - 1) / G::TOK));
+    auto kernel = k_mmq_q4_k<TC, RC, WAVES>;
+    hipLaunchKernelGGL(kernel, grid, dim3(WAVES * 64), G::LDS_BYTES, pick_stream(stream),
+                       (const uint8_t *)d_w, (uint32_t)rows, (uint32_t)blocks,
+                       (const uint8_t *)d_acts, (uint32_t)n_vec, d_out, out_stride);
+}
+
 extern "C" int oxh_mmq(uint32_t qtype, const void *d_w, size_t rows, size_t cols,
                        const void *d_acts, size_t n_vec, float *d_out, size_t out_stride,
                        void *stream)
@@ -667,29 +730,29 @@ extern "C" int oxh_mmq(uint32_t qtype, const void *d_w, size_t rows, size_t cols
     const size_t blocks = cols / OXH_QK_K;
     if (rows > 0x7FFFFFFFull || n_vec > 0x7FFFFFFFull || blocks > 0xFFFFFFull)
         return arg_fail("oxh_mmq: dimension too large");
-    /* the kernel addresses a workgroup's 256 rows and 128 tokens with 32-bit lane offsets */
-    if (blocks * 292u * 128u > 0xFFFFFFFFull)
+    /* the kernel addresses a workgroup's rows and tokens with 32-bit lane offsets */
+    if (blocks * 292u * 256u > 0xFFFFFFFFull)
         return arg_fail("oxh_mmq: cols too large");
-    const uint32_t row_tiles = (uint32_t)((rows + MMQ_ROWS - 1) / MMQ_ROWS);
-#define MMQ_LAUNCH(TT)                                                                              \
-    hipLaunchKernelGGL(k_mmq_q4_k<TT>, dim3(row_tiles, (uint32_t)((n_vec + 32u * TT - 1) / (32u * TT))), \
-                       dim3(MMQ_WAVES * 64), MmqGeom<TT>::LDS_BYTES, pick_stream(stream),            \
-                       (const uint8_t *)d_w, (uint32_t)rows, (uint32_t)blocks,                       \
-                       (const uint8_t *)d_acts, (uint32_t)n_vec, d_out, out_stride)
-    /* Token tiles per wave: four amortise the operand build best, but a launch
-     * needs about one workgroup per CU; take the largest count that still
-     * gives one, and never more tiles than the batch fills. */
-    const size_t cus = (size_t)(g_n_cu > 0 ? g_n_cu : 256);
-    const size_t need = cus - cus / 8;
-    int tt = 4;
-    while (tt > 1 && (n_vec <= 16u * (size_t)tt || row_tiles * ((n_vec + 32u * tt - 1) / (32u * tt)) < need)) tt >>= 1;
-    static int forced = -1;                 /* OXH_MMQ_TILES = 1, 2 or 4 overrides the choice */
+    static int forced = -1;                 /* OXH_MMQ_TILES = 1, 2 or 4 forces the prefill shape with that many 32-token tiles */
     if (forced < 0) forced = (int)env_u32("OXH_MMQ_TILES", 0, 0, 4);
-    if (forced == 1 || forced == 2 || forced == 4) tt = forced;
-    if (tt == 1) MMQ_LAUNCH(1);
-    else if (tt == 2) MMQ_LAUNCH(2);
-    else MMQ_LAUNCH(4);
-#undef MMQ_LAUNCH
+    const bool force = forced == 1 || forced == 2 || forced == 4;
+    if (!force && n_vec <= 16) mmq_launch<1, 1, 4>(d_w, rows, blocks, d_acts, n_vec, d_out, out_stride, stream);           /* small batch: bound by the weight stream */
+    else if (!force && n_vec <= 32) mmq_launch<2, 1, 4>(d_w, rows, blocks, d_acts, n_vec, d_out, out_stride, stream);
+    else {
+        /* Prefill shape.  32-token tiles per wave: four amortise the operand
+         * build best, but a launch needs about one workgroup per CU; take the
+         * largest count that still gives one, and never more tiles than the
+         * batch fills. */
+        const size_t row_tiles = (rows + 255) / 256;
+        const size_t cus = (size_t)(g_n_cu > 0 ? g_n_cu : 256);
+        const size_t need = cus - cus / 8;
+        int tt = 4;
+        while (tt > 1 && (n_vec <= 16u * (size_t)tt || row_tiles * ((n_vec + 32u * tt - 1) / (32u * tt)) < need)) tt >>= 1;
+        if (force) tt = forced;
+        if (tt == 1) mmq_launch<2, 2, 8>(d_w, rows, blocks, d_acts, n_vec, d_out, out_stride, stream);
+        else if (tt == 2) mmq_launch<4, 2, 8>(d_w, rows, blocks, d_acts, n_vec, d_out, out_stride, stream);
+        else mmq_launch<8, 2, 8>(d_w, rows, blocks, d_acts, n_vec, d_out, out_stride, stream);
+    }
     HIP_TRY(hipGetLastError());
     return OXH_OK;
 }

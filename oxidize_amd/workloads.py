@@ -184,6 +184,10 @@ class MoESet:
         self.d_gate = mv.DeviceBuffer(n_pairs * ffn * 4)
         self.d_up = mv.DeviceBuffer(n_pairs * ffn * 4)
         self.d_down = mv.DeviceBuffer(n_pairs * hidden * 4)
+        # room for the quantised activations: with it, launches of three or more
+        # activations per expert run on the matrix cores
+        self.d_act_x = mv.DeviceBuffer(n_pairs * mv.act_bytes(Q4K, hidden))
+        self.d_act_h = mv.DeviceBuffer(n_pairs * mv.act_bytes(Q4K, ffn))
         gu, dn = [], []
         self.hit = 0
         for e in range(n_expert):
@@ -203,9 +207,11 @@ class MoESet:
 
     def launch_step(self, stream=None):
         for segs in self.seg_gu:
-            mv.gemv_segments_f32(Q4K, segs, self.hidden, self.d_xg.ptr, self.hidden, None, 1, self.ffn, stream)
+            mv.gemv_segments_f32(Q4K, segs, self.hidden, self.d_xg.ptr, self.hidden, self.d_act_x.ptr, 1,
+                                 self.ffn, stream)
         for segs in self.seg_dn:
-            mv.gemv_segments_f32(Q4K, segs, self.ffn, self.d_h.ptr, self.ffn, None, 1, self.hidden, stream)
+            mv.gemv_segments_f32(Q4K, segs, self.ffn, self.d_h.ptr, self.ffn, self.d_act_h.ptr, 1,
+                                 self.hidden, stream)
 
     def outputs(self):
         n_pairs = self.n_tok * self.top_k
