@@ -416,9 +416,8 @@ static hipError_t raise_all_lds_ceilings(void)
     OXH_RAISE(k_gemv_q6_k)
     OXH_RAISE(k_gemv_q8_0)
 #undef OXH_RAISE
-    if ((e = raise_lds_ceiling(k_mmq_q4_k<2, 2, 8>)) != hipSuccess) return e;
-    if ((e = raise_lds_ceiling(k_mmq_q4_k<4, 2, 8>)) != hipSuccess) return e;
     if ((e = raise_lds_ceiling(k_mmq_q4_k<8, 2, 8>)) != hipSuccess) return e;
+    if ((e = raise_lds_ceiling(k_mmq_q4_k<4, 1, 8>)) != hipSuccess) return e;
     return hipSuccess;
 }
 
@@ -733,26 +732,24 @@ extern "C" int oxh_mmq(uint32_t qtype, const void *d_w, size_t rows, size_t cols
     /* the kernel addresses a workgroup's rows and tokens with 32-bit lane offsets */
     if (blocks * 292u * 256u > 0xFFFFFFFFull)
         return arg_fail("oxh_mmq: cols too large");
-    static int forced = -1;                 /* OXH_MMQ_TILES = 1, 2 or 4 forces the prefill shape with that many 32-token tiles */
-    if (forced < 0) forced = (int)env_u32("OXH_MMQ_TILES", 0, 0, 4);
-    const bool force = forced == 1 || forced == 2 || forced == 4;
-    if (!force && n_vec <= 16) mmq_launch<1, 1, 4>(d_w, rows, blocks, d_acts, n_vec, d_out, out_stride, stream);           /* small batch: bound by the weight stream */
-    else if (!force && n_vec <= 32) mmq_launch<2, 1, 4>(d_w, rows, blocks, d_acts, n_vec, d_out, out_stride, stream);
-    else {
-        /* Prefill shape.  32-token tiles per wave: four amortise the operand
-         * build best, but a launch needs about one workgroup per CU; take the
-         * largest count that still gives one, and never more tiles than the
-         * batch fills. */
-        const size_t row_tiles = (rows + 255) / 256;
-        const size_t cus = (size_t)(g_n_cu > 0 ? g_n_cu : 256);
-        const size_t need = cus - cus / 8;
-        int tt = 4;
-        while (tt > 1 && (n_vec <= 16u * (size_t)tt || row_tiles * ((n_vec + 32u * tt - 1) / (32u * tt)) < need)) tt >>= 1;
-        if (force) tt = forced;
-        if (tt == 1) mmq_launch<2, 2, 8>(d_w, rows, blocks, d_acts, n_vec, d_out, out_stride, stream);
-        else if (tt == 2) mmq_launch<4, 2, 8>(d_w, rows, blocks, d_acts, n_vec, d_out, out_stride, stream);
-        else mmq_launch<8, 2, 8>(d_w, rows, blocks, d_acts, n_vec, d_out, out_stride, stream);
+    /* Shape: the largest tile that still gives (nearly) every CU a workgroup;
+     * OXH_MMQ_SHAPE = 1..4 forces 256x128, 128x64, 64x32, 64x16 (rows x tokens). */
+    static int forced = -1;
+    if (forced < 0) forced = (int)env_u32("OXH_MMQ_SHAPE", 0, 0, 4);
+    const size_t cus = (size_t)(g_n_cu > 0 ? g_n_cu : 256);
+    const size_t need = cus - cus / 8;
+    int shape = forced;
+    if (!shape) {
+        if (n_vec <= 16) shape = 4;
+        else if (n_vec <= 32) shape = 3;
+        else if (((rows + 255) / 256) * ((n_vec + 127) / 128) >= need) shape = 1;
+        else if (((rows + 127) / 128) * ((n_vec + 63) / 64) >= need) shape = 2;
+        else shape = 3;
     }
+    if (shape == 1)      mmq_launch<8, 2, 8>(d_w, rows, blocks, d_acts, n_vec, d_out, out_stride, stream);
+    else if (shape == 2) mmq_launch<4, 1, 8>(d_w, rows, blocks, d_acts, n_vec, d_out, out_stride, stream);
+    else if (shape == 3) mmq_launch<2, 1, 4>(d_w, rows, blocks, d_acts, n_vec, d_out, out_stride, stream);
+    else                 mmq_launch<1, 1, 4>(d_w, rows, blocks, d_acts, n_vec, d_out, out_stride, stream);
     HIP_TRY(hipGetLastError());
     return OXH_OK;
 }

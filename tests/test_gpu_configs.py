@@ -138,15 +138,15 @@ def test_config3_mmq_prefill_512_tokens(oxh, rows):
 
 
 @pytest.mark.parametrize("rows,cols,n_vec", [
-    (7165, 512, 507),       # 28 row tiles x 8 token tiles of 64 = 224 workgroups
-    (14329, 256, 500),      # 56 row tiles x 4 token tiles of 128 = 224 workgroups
-    (4100, 512, 40),        # too few workgroups for the wide tiles: 17 x 2 of 32 tokens
+    (7165, 512, 507),       # 256x128 tiles would be 28 x 4 workgroups: 128x64 tiles, 56 x 8
+    (14329, 256, 500),      # 256x128 tiles: 56 x 4 = 224 workgroups
+    (4100, 512, 40),        # too few workgroups for either: 64x32 tiles, 65 x 2
 ])
 def test_mmq_tile_variants_ragged(oxh, rows, cols, n_vec):
-    """The MFMA kernel comes in three tile widths (32, 64, 128 tokens per
-    workgroup), picked from the launch size; these shapes select the two wider
-    ones on a 256-CU device and leave the last row tile and the last token
-    tile partly filled.  Every output is checked against the GEMV kernel on
+    """The MFMA kernel comes in several tile shapes (256x128, 128x64, 64x32,
+    64x16 rows x tokens), picked from the launch size; these cases select the
+    first three on a 256-CU device and leave the last row tile and the last
+    token tile partly filled.  Every output is checked against the GEMV kernel on
     the same device data, and a sample of tokens against the oracle."""
     info = mv.device_info()
     if info["n_cu"] != 256:
