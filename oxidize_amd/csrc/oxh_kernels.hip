@@ -518,16 +518,15 @@ static int launch_mmq_segments(const OxhSegment *segs, size_t n_segs, size_t col
     uint32_t wg = 0, n = 0;
     for (size_t i = 0; i < n_segs; i++) {
         if (segs[i].rows == 0) continue;
-        t.w[n] = (const uint8_t *)segs[i].d_w;
-        t.out[n] = segs[i].d_out;
-        t.rows[n] = (uint32_t)segs[i].rows;
-        t.act_first[n] = (uint32_t)segs[i].act_first;
-        t.nv[n] = (uint32_t)(segs[i].n_vec ? segs[i].n_vec : n_vec_default);
-        t.wg_begin[n] = wg;
+        t.s[n].w = (const uint8_t *)segs[i].d_w;
+        t.s[n].out = segs[i].d_out;
+        t.s[n].rows = (uint32_t)segs[i].rows;
+        t.s[n].act_first = (uint32_t)segs[i].act_first;
+        t.s[n].nv = (uint32_t)(segs[i].n_vec ? segs[i].n_vec : n_vec_default);
+        t.s[n].wg_begin = wg;
         wg += (uint32_t)((segs[i].rows + G::ROWS - 1) / G::ROWS);
         n++;
     }
-    t.wg_begin[n] = wg;
     t.n = n;
     auto kernel = k_mmq_q4_k_segments<1, 1, 4>;
     hipLaunchKernelGGL(kernel, dim3(wg), dim3(4 * 64), G::LDS_BYTES,
@@ -632,18 +631,17 @@ static int launch_gemv(uint32_t qtype, const OxhSegment *segs, size_t n_segs, si
     uint32_t wg = 0, n = 0;
     for (size_t i = 0; i < n_segs; i++) {
         if (segs[i].rows == 0) continue;
-        t.w[n] = (const uint8_t *)segs[i].d_w;
-        t.out[n] = segs[i].d_out;
-        t.rows[n] = (uint32_t)segs[i].rows;
-        t.act_first[n] = (uint32_t)segs[i].act_first;
-        t.nv[n] = (uint32_t)(segs[i].n_vec ? segs[i].n_vec : n_vec_default);
-        t.wg_begin[n] = wg;
-        t.rows_q[n] = (uint32_t)(segs[i].rows / ((size_t)n_wg[i] * W));
-        t.rows_rem[n] = (uint32_t)(segs[i].rows % ((size_t)n_wg[i] * W));
+        t.s[n].w = (const uint8_t *)segs[i].d_w;
+        t.s[n].out = segs[i].d_out;
+        t.s[n].rows = (uint32_t)segs[i].rows;
+        t.s[n].act_first = (uint32_t)segs[i].act_first;
+        t.s[n].nv = (uint32_t)(segs[i].n_vec ? segs[i].n_vec : n_vec_default);
+        t.s[n].wg_begin = wg;
+        t.s[n].rows_q = (uint32_t)(segs[i].rows / ((size_t)n_wg[i] * W));
+        t.s[n].rows_rem = (uint32_t)(segs[i].rows % ((size_t)n_wg[i] * W));
         wg += n_wg[i];
         n++;
     }
-    t.wg_begin[n] = wg;
     t.n = n;
 
     const dim3 grid(wg), block(W * 64u);
