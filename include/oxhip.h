@@ -143,6 +143,11 @@ int oxh_debug_subblock_sums(uint32_t qtype, const void *d_w, size_t rows,
 /* Device memory / stream / event plumbing so that C callers never include
  * HIP headers (as cuda_mmq.h does with its void* stream). */
 int  oxh_malloc(void **d_ptr, size_t bytes);
+/* Page-locked host memory (hipHostMalloc): copies to and from it are true
+ * asynchronous DMA.  The host-pointer entry points stage their small inputs
+ * and outputs through such buffers. */
+int  oxh_host_alloc(void **h_ptr, size_t bytes);
+int  oxh_host_free(void *h_ptr);
 int  oxh_free(void *d_ptr);
 int  oxh_memcpy_h2d(void *d_dst, const void *h_src, size_t bytes, void *stream);
 int  oxh_memcpy_d2h(void *h_dst, const void *d_src, size_t bytes, void *stream);

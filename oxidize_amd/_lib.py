@@ -42,6 +42,8 @@ SIGNATURES = {
     "oxh_mmq": (I, [U32, V, Z, Z, V, Z, V, Z, V]),
     "oxh_debug_subblock_sums": (I, [U32, V, Z, Z, V, V, V]),
     "oxh_malloc": (I, [ctypes.POINTER(V), Z]),
+    "oxh_host_alloc": (I, [ctypes.POINTER(V), Z]),
+    "oxh_host_free": (I, [V]),
     "oxh_free": (I, [V]),
     "oxh_memcpy_h2d": (I, [V, V, Z, V]),
     "oxh_memcpy_d2h": (I, [V, V, Z, V]),

@@ -193,6 +193,38 @@ typedef struct {
 
 static DevBuf g_dx, g_dact, g_dout;
 
+/* Page-locked host staging for the decode-sized entry points: the caller's
+ * vectors are ordinary pageable memory, and a copy between pageable memory and
+ * the device is a synchronous two-step affair inside the runtime (about 12 us
+ * each, three per call).  Staged through pinned buffers a call is one DMA in,
+ * the launch, one DMA out (output and quantised activation together). */
+typedef struct {
+    void *p;
+    size_t bytes;
+} HostBuf;
+
+static HostBuf g_hin, g_hout;
+
+static int reserve_host(HostBuf *b, size_t bytes)
+{
+    if (b->bytes >= bytes) return OXH_OK;
+    int rc = oxh_stream_sync(NULL);
+    if (rc) return rc;
+    if (b->p) {
+        rc = oxh_host_free(b->p);
+        b->p = NULL;
+        b->bytes = 0;
+        if (rc) return rc;
+    }
+    size_t want = bytes < (1u << 18) ? (1u << 18) : bytes + bytes / 4;
+    rc = oxh_host_alloc(&b->p, want);
+    if (rc) return rc;
+    b->bytes = want;
+    return OXH_OK;
+}
+
+static size_t align16(size_t n) { return (n + 15u) & ~(size_t)15u; }
+
 static int reserve(DevBuf *b, size_t bytes)
 {
     if (b->bytes >= bytes) return OXH_OK;
@@ -269,19 +301,25 @@ int oxh_matvec_quantized(uint32_t qtype, const uint8_t *data, size_t rows,
     if (rc) return rc;
     const uint8_t *d_w;
     if ((rc = resident_ptr(data, wbytes, &d_w))) return rc;
+    /* device and pinned-host images: [output rows][quantised activation] */
+    const size_t act_off = align16(obytes);
     if ((rc = reserve(&g_dx, cols * sizeof(float)))) return rc;
-    if ((rc = reserve(&g_dact, abytes))) return rc;
-    if ((rc = reserve(&g_dout, obytes))) return rc;
+    if ((rc = reserve(&g_dout, act_off + abytes))) return rc;
+    if ((rc = reserve_host(&g_hin, cols * sizeof(float)))) return rc;
+    if ((rc = reserve_host(&g_hout, act_off + abytes))) return rc;
 
-    if ((rc = oxh_memcpy_h2d(g_dx.p, input, cols * sizeof(float), NULL))) return rc;
+    memcpy(g_hin.p, input, cols * sizeof(float));
+    if ((rc = oxh_memcpy_h2d(g_dx.p, g_hin.p, cols * sizeof(float), NULL))) return rc;
     /* one launch: quantise the activation inside the GEMV kernel */
     OxhSegment seg = { d_w, (float *)g_dout.p, rows, 0, 0 };
-    if ((rc = oxh_gemv_segments_f32(qtype, &seg, 1, cols, (const float *)g_dx.p, cols, g_dact.p, 1,
-                                    rows, NULL)))
+    if ((rc = oxh_gemv_segments_f32(qtype, &seg, 1, cols, (const float *)g_dx.p, cols,
+                                    (uint8_t *)g_dout.p + act_off, 1, rows, NULL)))
         return rc;
-    if ((rc = oxh_memcpy_d2h(output, g_dout.p, obytes, NULL))) return rc;
-    if ((rc = oxh_memcpy_d2h(temp, g_dact.p, abytes, NULL))) return rc;
-    return oxh_stream_sync(NULL);
+    if ((rc = oxh_memcpy_d2h(g_hout.p, g_dout.p, act_off + abytes, NULL))) return rc;
+    if ((rc = oxh_stream_sync(NULL))) return rc;
+    memcpy(output, g_hout.p, obytes);
+    memcpy(temp, (const uint8_t *)g_hout.p + act_off, abytes);
+    return OXH_OK;
 }
 
 /* ─── grouped launches (fused / multi-input) ──────────────────────────── */
@@ -308,12 +346,14 @@ static int grouped(uint32_t qtype, const uint8_t *const *datas,
     if ((rc = reserve(&g_dx, xbytes))) return rc;
     if ((rc = reserve(&g_dact, actbytes))) return rc;
     if ((rc = reserve(&g_dout, total_rows * sizeof(float)))) return rc;
+    if ((rc = reserve_host(&g_hin, xbytes))) return rc;
+    if ((rc = reserve_host(&g_hout, total_rows * sizeof(float)))) return rc;
 
     for (size_t i = 0; i < n_inputs; i++) {
         if (!inputs[i]) return bad_arg("grouped: NULL input");
-        if ((rc = oxh_memcpy_h2d((float *)g_dx.p + i * cols, inputs[i], cols * sizeof(float), NULL)))
-            return rc;
+        memcpy((float *)g_hin.p + i * cols, inputs[i], cols * sizeof(float));
     }
+    if ((rc = oxh_memcpy_h2d(g_dx.p, g_hin.p, xbytes, NULL))) return rc;
     enum { CHUNK = 32 };
     OxhSegment segs[CHUNK];
     size_t done_rows = 0;
@@ -339,14 +379,14 @@ static int grouped(uint32_t qtype, const uint8_t *const *datas,
                                         NULL)))
             return rc;
     }
+    if ((rc = oxh_memcpy_d2h(g_hout.p, g_dout.p, total_rows * sizeof(float), NULL))) return rc;
+    if ((rc = oxh_stream_sync(NULL))) return rc;
     size_t off = 0;
     for (size_t k = 0; k < n_outs; k++) {
-        if (rows[k] &&
-            (rc = oxh_memcpy_d2h(outs[k], (float *)g_dout.p + off, rows[k] * sizeof(float), NULL)))
-            return rc;
+        if (rows[k]) memcpy(outs[k], (const float *)g_hout.p + off, rows[k] * sizeof(float));
         off += rows[k];
     }
-    return oxh_stream_sync(NULL);
+    return OXH_OK;
 }
 
 int oxh_matvec_quantized_fused(const uint32_t *qtypes, const uint8_t *const *datas,

@@ -754,6 +754,28 @@ extern "C" int oxh_mmq(uint32_t qtype, const void *d_w, size_t rows, size_t cols
 
 /* ─── memory / stream / event plumbing ────────────────────────────────── */
 
+extern "C" int oxh_host_alloc(void **h_ptr, size_t bytes)
+{
+    int rc = ensure_init();
+    if (rc) return rc;
+    if (!h_ptr) return arg_fail("oxh_host_alloc: NULL");
+    hipError_t e = hipHostMalloc(h_ptr, bytes ? bytes : 1, hipHostMallocDefault);
+    if (e == hipErrorOutOfMemory) {
+        snprintf(g_err, sizeof g_err, "out of host memory pinning %zu bytes", bytes);
+        (void)hipGetLastError();
+        return OXH_ERR_NOMEM;
+    }
+    if (e != hipSuccess) return hip_fail(e, "hipHostMalloc");
+    return OXH_OK;
+}
+
+extern "C" int oxh_host_free(void *h_ptr)
+{
+    if (!h_ptr) return OXH_OK;
+    HIP_TRY(hipHostFree(h_ptr));
+    return OXH_OK;
+}
+
 extern "C" int oxh_malloc(void **d_ptr, size_t bytes)
 {
     int rc = ensure_init();
