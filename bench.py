@@ -227,7 +227,7 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this path is built and measured on ONE GPU; --gpus %d is not supported "
-              "(the work shards by output rows, see DESIGN.md)" % args.gpus, file=sys.stderr)
+              "(the work would shard by output rows across GPUs; nothing here launches a second rank)" % args.gpus, file=sys.stderr)
         return 2
 
     from oxidize_amd import _lib
