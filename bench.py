@@ -87,6 +87,32 @@ def secondary_figures(mv, synth):
     out["mmq_prefill_q4k"] = mmq
     d_x.free()
     d_a.free()
+    # the down projection of the same model is Q6_K: 4096 x 14336, 512 tokens
+    Q6K = 16
+    rows, cols = 4096, 14336
+    x = synth.normal(n_vec * cols, seed=0, stream=2001)
+    d_x = mv.DeviceBuffer.from_host(x)
+    d_a = mv.DeviceBuffer(n_vec * mv.act_bytes(Q6K, cols))
+    w = synth.weights(Q6K, rows, cols, seed=0, stream=3)
+    copies = [mv.DeviceBuffer.from_host(w) for _ in range(3)]
+    d_o = mv.DeviceBuffer(n_vec * rows * 4)
+    mv.quantize(Q6K, d_x.ptr, cols, n_vec, cols, d_a.ptr)
+    state = {"i": 0}
+
+    def run_q6():
+        state["i"] += 1
+        mv.mmq(Q6K, copies[state["i"] % 3].ptr, rows, cols, d_a.ptr, n_vec, d_o.ptr, rows)
+
+    us = timed(run_q6, 12, mv)
+    ops = 2.0 * rows * cols * n_vec
+    out["mmq_prefill_q6k"] = {"%dx%dx%d" % (rows, cols, n_vec): {
+        "mfma_kernel_only_us": round(us, 2), "tops": round(ops / us / 1e6, 1),
+        "mfma_kernel_only_frac_of_int8_peak": round(ops / us / 1e6 / INT8_PEAK_TOPS, 4)}}
+    for c in copies:
+        c.free()
+    d_x.free()
+    d_a.free()
+    d_o.free()
     # Q8_0 lm_head (configuration 2), batch 1 and 8
     rows, cols = 151936, 896
     w = synth.weights(Q80, rows, cols, seed=0, stream=5)

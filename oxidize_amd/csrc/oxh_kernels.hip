@@ -418,6 +418,8 @@ static hipError_t raise_all_lds_ceilings(void)
 #undef OXH_RAISE
     if ((e = raise_lds_ceiling(k_mmq_q4_k<8, 2, 8>)) != hipSuccess) return e;
     if ((e = raise_lds_ceiling(k_mmq_q4_k<4, 1, 8>)) != hipSuccess) return e;
+    if ((e = raise_lds_ceiling(k_mmq_q6_k<8, 1, 8>)) != hipSuccess) return e;
+    if ((e = raise_lds_ceiling(k_mmq_q6_k<4, 1, 8>)) != hipSuccess) return e;
     return hipSuccess;
 }
 
@@ -711,6 +713,18 @@ static void mmq_launch(const void *d_w, size_t rows, size_t blocks, const void *
                        (const uint8_t *)d_acts, (uint32_t)n_vec, d_out, out_stride);
 }
 
+template <int TC, int RC, int WAVES>
+static void mmq6_launch(const void *d_w, size_t rows, size_t blocks, const void *d_acts, size_t n_vec,
+                        float *d_out, size_t out_stride, void *stream)
+{
+    typedef Mmq6Geom<TC, RC, WAVES> G;
+    const dim3 grid((uint32_t)((rows + G::ROWS - 1) / G::ROWS), (uint32_t)((n_vec + G::TOK - 1) / G::TOK));
+    auto kernel = k_mmq_q6_k<TC, RC, WAVES>;
+    hipLaunchKernelGGL(kernel, grid, dim3(WAVES * 64), G::LDS_BYTES, pick_stream(stream),
+                       (const uint8_t *)d_w, (uint32_t)rows, (uint32_t)blocks,
+                       (const uint8_t *)d_acts, (uint32_t)n_vec, d_out, out_stride);
+}
+
 extern "C" int oxh_mmq(uint32_t qtype, const void *d_w, size_t rows, size_t cols,
                        const void *d_acts, size_t n_vec, float *d_out, size_t out_stride,
                        void *stream)
@@ -719,7 +733,7 @@ extern "C" int oxh_mmq(uint32_t qtype, const void *d_w, size_t rows, size_t cols
     if (rc) return rc;
     if (rows == 0 || n_vec == 0) return OXH_OK;
     if (!d_w || !d_acts || !d_out) return arg_fail("oxh_mmq: NULL pointer");
-    if (!is_q4k(qtype) || oxh_act_kind(qtype, cols) != 2) {
+    if ((!is_q4k(qtype) && qtype != OXH_Q6_K) || oxh_act_kind(qtype, cols) != 2) {
         snprintf(g_err, sizeof g_err, "oxh_mmq: qtype %u with cols %zu has no MFMA kernel", qtype, cols);
         return OXH_DECLINED;
     }
@@ -743,6 +757,22 @@ extern "C" int oxh_mmq(uint32_t qtype, const void *d_w, size_t rows, size_t cols
         else if (((rows + 255) / 256) * ((n_vec + 127) / 128) >= need) shape = 1;
         else if (((rows + 127) / 128) * ((n_vec + 63) / 64) >= need) shape = 2;
         else shape = 3;
+    }
+    if (qtype == OXH_Q6_K) {
+        /* one 16-row chunk per wave throughout: 128x128, 128x64, 64x32, 64x16 */
+        if (!forced) {
+            if (n_vec <= 16) shape = 4;
+            else if (n_vec <= 32) shape = 3;
+            else if (((rows + 127) / 128) * ((n_vec + 127) / 128) >= need) shape = 1;
+            else if (((rows + 127) / 128) * ((n_vec + 63) / 64) >= need) shape = 2;
+            else shape = 3;
+        }
+        if (shape == 1)      mmq6_launch<8, 1, 8>(d_w, rows, blocks, d_acts, n_vec, d_out, out_stride, stream);
+        else if (shape == 2) mmq6_launch<4, 1, 8>(d_w, rows, blocks, d_acts, n_vec, d_out, out_stride, stream);
+        else if (shape == 3) mmq6_launch<2, 1, 4>(d_w, rows, blocks, d_acts, n_vec, d_out, out_stride, stream);
+        else                 mmq6_launch<1, 1, 4>(d_w, rows, blocks, d_acts, n_vec, d_out, out_stride, stream);
+        HIP_TRY(hipGetLastError());
+        return OXH_OK;
     }
     if (shape == 1)      mmq_launch<8, 2, 8>(d_w, rows, blocks, d_acts, n_vec, d_out, out_stride, stream);
     else if (shape == 2) mmq_launch<4, 1, 8>(d_w, rows, blocks, d_acts, n_vec, d_out, out_stride, stream);

@@ -137,12 +137,15 @@ def test_config3_mmq_prefill_512_tokens(oxh, rows):
         assert np.array_equal(bits(got), bits(out[v0:v0 + 8]))
 
 
-@pytest.mark.parametrize("rows,cols,n_vec", [
-    (7165, 512, 507),       # 256x128 tiles would be 28 x 4 workgroups: 128x64 tiles, 56 x 8
-    (14329, 256, 500),      # 256x128 tiles: 56 x 4 = 224 workgroups
-    (4100, 512, 40),        # too few workgroups for either: 64x32 tiles, 65 x 2
+@pytest.mark.parametrize("qtype,rows,cols,n_vec", [
+    (Q4K, 7165, 512, 507),      # 256x128 tiles would be 28 x 4 workgroups: 128x64 tiles, 56 x 8
+    (Q4K, 14329, 256, 500),     # 256x128 tiles: 56 x 4 = 224 workgroups
+    (Q4K, 4100, 512, 40),       # too few workgroups for either: 64x32 tiles, 65 x 2
+    (Q6K, 7165, 512, 507),      # Q6_K: 128x128 tiles, 56 x 4
+    (Q6K, 3600, 256, 500),      # Q6_K: 128x64 tiles, 29 x 8
+    (Q6K, 4100, 512, 40),       # Q6_K: 64x32 tiles
 ])
-def test_mmq_tile_variants_ragged(oxh, rows, cols, n_vec):
+def test_mmq_tile_variants_ragged(oxh, qtype, rows, cols, n_vec):
     """The MFMA kernel comes in several tile shapes (256x128, 128x64, 64x32,
     64x16 rows x tokens), picked from the launch size; these cases select the
     first three on a 256-CU device and leave the last row tile and the last
@@ -151,27 +154,27 @@ def test_mmq_tile_variants_ragged(oxh, rows, cols, n_vec):
     info = mv.device_info()
     if info["n_cu"] != 256:
         pytest.skip("tile choice is tied to 256 compute units")
-    w = synth.weights(Q4K, rows, cols, seed=5, stream=rows)
+    w = synth.weights(qtype, rows, cols, seed=5, stream=rows)
     xs = synth.normal(n_vec * cols, seed=5, stream=n_vec).reshape(n_vec, cols)
     d_w = mv.DeviceBuffer.from_host(w)
     d_x = mv.DeviceBuffer.from_host(xs)
-    nact = mv.act_bytes(Q4K, cols)
+    nact = mv.act_bytes(qtype, cols)
     d_a = mv.DeviceBuffer(n_vec * nact)
     stride = rows + 3
     d_o = mv.DeviceBuffer(n_vec * stride * 4)
     d_o.upload(np.full(n_vec * stride, -7.25, np.float32))
-    mv.quantize(Q4K, d_x.ptr, cols, n_vec, cols, d_a.ptr)
-    mv.mmq(Q4K, d_w.ptr, rows, cols, d_a.ptr, n_vec, d_o.ptr, stride)
+    mv.quantize(qtype, d_x.ptr, cols, n_vec, cols, d_a.ptr)
+    mv.mmq(qtype, d_w.ptr, rows, cols, d_a.ptr, n_vec, d_o.ptr, stride)
     out = d_o.download(np.float32, n_vec * stride).reshape(n_vec, stride)
     assert np.all(out[:, rows:] == -7.25)
     for v in (0, 31, 32, n_vec // 2, n_vec - 1):
-        want, _ = oracle_matvec(Q4K, w, rows, cols, np.ascontiguousarray(xs[v]))
+        want, _ = oracle_matvec(qtype, w, rows, cols, np.ascontiguousarray(xs[v]))
         assert np.array_equal(bits(out[v, :rows]), bits(want)), v
     d_o2 = mv.DeviceBuffer(8 * rows * 4)
     for v0 in range(0, n_vec, 8):
         nv = min(8, n_vec - v0)
         segs = mv.make_segments([(d_w.ptr, d_o2.ptr, rows, v0)])
-        mv.gemv_segments(Q4K, segs, cols, d_a.ptr, nv, rows)
+        mv.gemv_segments(qtype, segs, cols, d_a.ptr, nv, rows)
         got = d_o2.download(np.float32, 8 * rows).reshape(8, rows)[:nv]
         assert np.array_equal(bits(got), bits(out[v0:v0 + nv, :rows])), v0
 

@@ -257,28 +257,30 @@ def test_expert_slices_resolve_inside_a_registered_tensor(oxh):
         assert np.array_equal(bits(out), bits(want))
 
 
+@pytest.mark.parametrize("qtype", [Q4K, Q6K])
 @pytest.mark.parametrize("rows,cols,n_vec,out_pad", [
     (32, 256, 32, 0), (130, 1024, 9, 0), (128, 4096, 64, 0), (200, 2816, 100, 5),
     (257, 512, 65, 1), (64, 14336, 40, 0),
 ])
-def test_mmq_batch_bit_identical_to_single_vector(oxh, rows, cols, n_vec, out_pad):
-    """More than 8 vectors of Q4_K go through the int8-MFMA kernel; the
-    reference promises batch == single-vector to the bit for K-quants
+def test_mmq_batch_bit_identical_to_single_vector(oxh, qtype, rows, cols, n_vec, out_pad):
+    """More than 8 vectors of Q4_K or Q6_K go through the int8-MFMA kernels;
+    the reference promises batch == single-vector to the bit for K-quants
     (matvec.h:115-117, tests/test_matvec_batch.c:86-99)."""
+    Q4K_ = qtype
     out_stride = rows + out_pad
-    w = synth.weights(Q4K, rows, cols, seed=71, stream=rows)
+    w = synth.weights(Q4K_, rows, cols, seed=71, stream=rows)
     xs = synth.normal(n_vec * cols, seed=71, stream=n_vec).reshape(n_vec, cols)
     xs[3, :256] = 0.0
     outs = np.full((n_vec, out_stride), -7.25, np.float32)
     temp = np.zeros(cols, np.float32)
     scratch = np.zeros(mv.batch_scratch_bytes(cols), np.uint8)
-    rc = mv.matvec_quantized_batch(Q4K, w, rows, cols, synth.row_bytes(Q4K, cols), xs, cols, outs,
+    rc = mv.matvec_quantized_batch(qtype, w, rows, cols, synth.row_bytes(qtype, cols), xs, cols, outs,
                                    out_stride, n_vec, temp, scratch)
     assert rc == 0
     o = oxlibs.oracle()
     want = np.zeros((n_vec, rows), np.float32)
     sc2 = np.zeros(o.oxo_matvec_batch_scratch_bytes(cols), np.uint8)
-    assert o.oxo_matvec_quantized_batch(Q4K, w.ctypes.data, rows, cols, synth.row_bytes(Q4K, cols),
+    assert o.oxo_matvec_quantized_batch(qtype, w.ctypes.data, rows, cols, synth.row_bytes(qtype, cols),
                                         xs.ctypes.data, cols, want.ctypes.data, rows, n_vec,
                                         sc2.ctypes.data, sc2.nbytes) == 0
     assert np.array_equal(bits(outs[:, :rows]), bits(want))
