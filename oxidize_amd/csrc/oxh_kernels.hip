@@ -499,11 +499,11 @@ static bool gemv_wants_mfma(uint32_t qtype, const GemvIo &io, size_t max_nv, con
 {
     static int min_nv = -1;
     if (min_nv < 0) min_nv = (int)env_u32("OXH_GEMV_MFMA_MIN_NV", 3, 0, 64);
-    if (!is_q4k(qtype) || dump || min_nv == 0 || max_nv < (size_t)min_nv) return false;
+    if ((!is_q4k(qtype) && qtype != OXH_Q6_K) || dump || min_nv == 0 || max_nv < (size_t)min_nv) return false;
     return io.d_acts != nullptr || io.d_act_out != nullptr;
 }
 
-static int launch_mmq_segments(const OxhSegment *segs, size_t n_segs, size_t cols, size_t blocks,
+static int launch_mmq_segments(uint32_t qtype, const OxhSegment *segs, size_t n_segs, size_t cols, size_t blocks,
                                const GemvIo &io, size_t n_vec_default, size_t n_acts,
                                size_t out_stride, void *stream)
 {
@@ -530,9 +530,17 @@ static int launch_mmq_segments(const OxhSegment *segs, size_t n_segs, size_t col
         n++;
     }
     t.n = n;
-    auto kernel = k_mmq_q4_k_segments<1, 1, 4>;
-    hipLaunchKernelGGL(kernel, dim3(wg), dim3(4 * 64), G::LDS_BYTES,
-                       pick_stream(stream), t, (uint32_t)blocks, acts, out_stride);
+    if (qtype == OXH_Q6_K) {
+        typedef Mmq6Geom<1, 1, 4> G6;                       /* same 64-row tiles */
+        static_assert(G6::ROWS == G::ROWS, "segment tiling is shared by both formats");
+        auto kernel = k_mmq_q6_k_segments<1, 1, 4>;
+        hipLaunchKernelGGL(kernel, dim3(wg), dim3(4 * 64), G6::LDS_BYTES,
+                           pick_stream(stream), t, (uint32_t)blocks, acts, out_stride);
+    } else {
+        auto kernel = k_mmq_q4_k_segments<1, 1, 4>;
+        hipLaunchKernelGGL(kernel, dim3(wg), dim3(4 * 64), G::LDS_BYTES,
+                           pick_stream(stream), t, (uint32_t)blocks, acts, out_stride);
+    }
     HIP_TRY(hipGetLastError());
     return OXH_OK;
 }
@@ -577,7 +585,7 @@ static int launch_gemv(uint32_t qtype, const OxhSegment *segs, size_t n_segs, si
     }
     if (total_rows == 0) return OXH_OK;
     if (gemv_wants_mfma(qtype, io, max_nv, dump))
-        return launch_mmq_segments(segs, n_segs, cols, blocks, io, n_vec_default, max_act + max_nv,
+        return launch_mmq_segments(qtype, segs, n_segs, cols, blocks, io, n_vec_default, max_act + max_nv,
                                    out_stride, stream);
     n_vec = max_nv;                        /* sizes LDS from here on */
     if (out_stride > 0xFFFFFFFFull || io.x_stride > 0xFFFFFFFFull || max_act + n_vec > 0xFFFFFFFFull)
