@@ -45,12 +45,15 @@ extern "C" {
 #define OXH_Q8_0    7u
 #define OXH_Q4_K_S 12u
 #define OXH_Q4_K_M 13u
+#define OXH_Q5_K_S 14u
+#define OXH_Q5_K_M 15u
 #define OXH_Q6_K   16u
 
 /* Block geometry (oxidize-c/include/oxidize/oxk.h:46-66). */
 #define OXH_QK_K         256u
 #define OXH_QK8_0         32u
 #define OXH_Q4_K_BYTES   144u
+#define OXH_Q5_K_BYTES   176u
 #define OXH_Q6_K_BYTES   210u
 #define OXH_Q8_0_BYTES    34u
 #define OXH_Q8_K_BYTES   292u
@@ -100,8 +103,8 @@ typedef struct OxhSegment {
  * for every segment, in ONE launch (a segment may override n_vec with its own
  * count: expert e of an MoE layer takes only the m_e tokens routed to it,
  * llama.c:6151-6169).  Covers the reference's row kernels
- * oc_oxk_dot_rows_{q4_k,q6_k}_q8_k / _q8_0_q8_0 (oxidize-c/src/compute/oxk.c:
- * 1447-1465) as used by matvec_fused_slice, matvec_fused_multi_slice and
+ * oc_oxk_dot_rows_{q4_k,q5_k,q6_k}_q8_k / _q8_0_q8_0 (oxidize-c/src/compute/oxk.c:
+ * 1447-1488) as used by matvec_fused_slice, matvec_fused_multi_slice and
  * matvec_fused_multi_input_slice (matvec.c:640-797) and the small-batch
  * rows path (matvec.c:1079-1102); the device analogue is
  * oc_cuda_mmq_matvec / _matvec_expert (cuda_mmq.h:57-72).  Segments live in
@@ -132,10 +135,10 @@ int oxh_mmq(uint32_t qtype, const void *d_w, size_t rows, size_t cols,
             void *stream);
 
 /* Test hook: the integer sub-block sums the GEMV kernel forms, written by the
- * same device code path.  Q4_K: 8 int32 per super-block (S_j), Q6_K: 16 per
+ * same device code path.  Q4_K and Q5_K: 8 int32 per super-block (S_j), Q6_K: 16 per
  * super-block, Q8_0: 1 per block; layout [row][block][j].  The reference
  * exposes no such API; the values are the intermediates of
- * oxidize-c/src/compute/oxk.c:263-283, :932-954, :234-237. */
+ * oxidize-c/src/compute/oxk.c:263-283, :870-886, :932-954, :234-237. */
 int oxh_debug_subblock_sums(uint32_t qtype, const void *d_w, size_t rows,
                             size_t cols, const void *d_act, int32_t *d_sums,
                             void *stream);

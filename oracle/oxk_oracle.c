@@ -226,6 +226,58 @@ float oxo_dot_q4_k_q8_k(const uint8_t *row, size_t blocks, const uint8_t *act,
     return sum;
 }
 
+float oxo_dot_q5_k_q8_k(const uint8_t *row, size_t blocks, const uint8_t *act,
+                        int32_t *sub, int32_t *posmin)
+{
+    float sum = 0.0f;
+    for (size_t b = 0; b < blocks; b++) {
+        const uint8_t *w = row + b * OXO_Q5_K_BYTES;
+        const uint8_t *a = act + b * OXO_Q8_K_BYTES;
+        const float dw = oxo_f16_to_f32(rd_u16(w));
+        const float dmin = oxo_f16_to_f32(rd_u16(w + 2));
+        float dq;
+        memcpy(&dq, a, 4);
+        const int8_t *q = (const int8_t *)(a + 4);
+        const uint8_t *hbits = w + 16;      /* 32 bytes: bit j of byte l is the fifth bit of element 32j + l */
+        const uint8_t *nib = w + 48;
+
+        uint8_t sc[8], mn[8];
+        scale_min_all(w + 4, sc, mn);
+
+        /* sub-block j = elements [32j, 32j+32): the nibble comes from where
+         * Q4_K keeps it, the fifth bit of element 32j + l is bit j of hbits[l] */
+        int32_t S[8];
+        for (int j = 0; j < 8; j++) {
+            const uint8_t *src = nib + 32 * (j >> 1);
+            const int shift = (j & 1) * 4;
+            int32_t acc = 0;
+            for (int l = 0; l < 32; l++) {
+                const int32_t code = (int32_t)((src[l] >> shift) & 15) +
+                                     (int32_t)(((hbits[l] >> j) & 1) << 4);
+                acc += code * (int32_t)q[32 * j + l];
+            }
+            S[j] = acc;
+        }
+        int32_t pos = 0, mins = 0;
+        for (int j = 0; j < 8; j++) {
+            int16_t b0, b1;
+            memcpy(&b0, a + 260 + 4 * j, 2);
+            memcpy(&b1, a + 262 + 4 * j, 2);
+            pos += (int32_t)sc[j] * S[j];
+            mins += (int32_t)mn[j] * ((int32_t)b0 + (int32_t)b1);
+        }
+        if (sub) memcpy(sub + 8 * b, S, sizeof S);
+        if (posmin) { posmin[2 * b] = pos; posmin[2 * b + 1] = mins; }
+
+        const float t_pos = dw * dq;
+        const float t_min = dmin * dq;
+        const float up = t_pos * (float)pos;
+        const float dn = t_min * (float)mins;
+        sum += up - dn;
+    }
+    return sum;
+}
+
 float oxo_dot_q6_k_q8_k(const uint8_t *row, size_t blocks, const uint8_t *act,
                         int32_t *grp)
 {
@@ -297,6 +349,8 @@ static size_t block_bytes(uint32_t qtype)
     case OXO_Q8_0:   return OXO_Q8_0_BYTES;
     case OXO_Q4_K_S:
     case OXO_Q4_K_M: return OXO_Q4_K_BYTES;
+    case OXO_Q5_K_S:
+    case OXO_Q5_K_M: return OXO_Q5_K_BYTES;
     case OXO_Q6_K:   return OXO_Q6_K_BYTES;
     default:         return 0;
     }
@@ -308,6 +362,8 @@ int oxo_act_kind(uint32_t qtype, size_t cols)
     case OXO_Q8_0:   return (cols % OXO_QK8_0 == 0) ? 1 : 0;
     case OXO_Q4_K_S:
     case OXO_Q4_K_M:
+    case OXO_Q5_K_S:
+    case OXO_Q5_K_M:
     case OXO_Q6_K:   return (cols % OXO_QK_K == 0) ? 2 : 0;
     default:         return 0;
     }
@@ -331,6 +387,8 @@ static float row_dot(uint32_t qtype, const uint8_t *row, size_t blocks,
     switch (qtype) {
     case OXO_Q8_0:   return oxo_dot_q8_0_q8_0(row, blocks, act, NULL);
     case OXO_Q6_K:   return oxo_dot_q6_k_q8_k(row, blocks, act, NULL);
+    case OXO_Q5_K_S:
+    case OXO_Q5_K_M: return oxo_dot_q5_k_q8_k(row, blocks, act, NULL, NULL);
     default:         return oxo_dot_q4_k_q8_k(row, blocks, act, NULL, NULL);
     }
 }
@@ -505,6 +563,22 @@ int oxo_dequant_row(uint32_t qtype, const uint8_t *row, size_t cols, float *out)
                 const int code = (int)((k < 2 ? (lo & 15u) : (lo >> 4)) |
                                        (((hi >> (2 * k)) & 3u) << 4)) - 32;
                 out[256 * b + e] = d * (float)sc[e >> 4] * (float)code;
+            }
+        } else if (qtype == OXO_Q5_K_S || qtype == OXO_Q5_K_M) {
+            const uint8_t *w = row + b * OXO_Q5_K_BYTES;
+            const float d = oxo_f16_to_f32(rd_u16(w));
+            const float dmin = oxo_f16_to_f32(rd_u16(w + 2));
+            uint8_t sc[8], mn[8];
+            for (unsigned j = 0; j < 8; j++)
+                oxo_scale_min_k4(j, w + 4, &sc[j], &mn[j]);
+            for (int e = 0; e < 256; e++) {
+                const int j = e >> 5, l = e & 31;
+                const unsigned byte = w[48 + 32 * (j >> 1) + l];
+                const unsigned code = ((j & 1) ? (byte >> 4) : (byte & 15u)) +
+                                      (((w[16 + l] >> j) & 1u) ? 16u : 0u);
+                const float ds = d * (float)sc[j];
+                const float ms = dmin * (float)mn[j];
+                out[256 * b + e] = ds * (float)code - ms;
             }
         } else {
             const uint8_t *w = row + b * OXO_Q4_K_BYTES;

@@ -39,12 +39,15 @@ enum {
     OXO_Q8_0   = 7,
     OXO_Q4_K_S = 12,
     OXO_Q4_K_M = 13,
+    OXO_Q5_K_S = 14,
+    OXO_Q5_K_M = 15,
     OXO_Q6_K   = 16,
 };
 
 #define OXO_QK_K        256u
 #define OXO_QK8_0       32u
 #define OXO_Q4_K_BYTES  144u
+#define OXO_Q5_K_BYTES  176u
 #define OXO_Q6_K_BYTES  210u
 #define OXO_Q8_0_BYTES  34u
 #define OXO_Q8_K_BYTES  292u
@@ -66,6 +69,11 @@ void oxo_quantize_q8_0(const float *x, size_t n, uint8_t *out);
  * S_j = sum over sub-block j of nibble * q8.  `posmin` (optional) receives
  * 2 int32 per block: {sum_j sc_j*S_j, sum_j m_j*B_j}. */
 float oxo_dot_q4_k_q8_k(const uint8_t *row, size_t blocks, const uint8_t *act,
+                        int32_t *sub, int32_t *posmin);
+/* src/compute/oxk.c:849-911 (same scale/min decode and f32 expression as
+ * Q4_K; the fifth bit of element 32j + l is bit j of byte l of the 32-byte
+ * plane at block offset 16).  `sub` and `posmin` as for Q4_K. */
+float oxo_dot_q5_k_q8_k(const uint8_t *row, size_t blocks, const uint8_t *act,
                         int32_t *sub, int32_t *posmin);
 /* src/compute/oxk.c:913-964.  `grp` (optional) receives 16 int32 per block. */
 float oxo_dot_q6_k_q8_k(const uint8_t *row, size_t blocks, const uint8_t *act,
@@ -117,7 +125,7 @@ void oxo_moe_route(const float *logits, size_t n_tok, size_t n_expert,
                    size_t k, int renorm, int32_t *ids, float *weights);
 
 /* Dequantise one row to f32 (src/compute/quantization.c:486-503, :633-670,
- * :723-766) — used only as an independent cross-check of the layouts. */
+ * :672-721, :723-766) — used only as an independent cross-check of the layouts. */
 int oxo_dequant_row(uint32_t qtype, const uint8_t *row, size_t cols, float *out);
 
 #ifdef __cplusplus

@@ -6,6 +6,7 @@
  *   Q8_K / Q8_0 activation bytes  oxidize-c/src/compute/matvec.c:276-316, :130-155
  *   f32 -> f16 (round half up)    oxidize-c/src/compute/flash_attention.c:149-185
  *   Q4_K x Q8_K block dot         oxidize-c/src/compute/oxk.c:243-297
+ *   Q5_K x Q8_K block dot         oxidize-c/src/compute/oxk.c:849-911
  *   Q6_K x Q8_K block dot         oxidize-c/src/compute/oxk.c:913-964
  *   Q8_0 x Q8_0 block dot         oxidize-c/src/compute/oxk.c:224-241
  *
@@ -321,6 +322,8 @@ extern "C" int oxh_act_kind(uint32_t qtype, size_t cols)
     case OXH_Q8_0:   return (cols % OXH_QK8_0 == 0) ? 1 : 0;
     case OXH_Q4_K_S:
     case OXH_Q4_K_M:
+    case OXH_Q5_K_S:
+    case OXH_Q5_K_M:
     case OXH_Q6_K:   return (cols % OXH_QK_K == 0) ? 2 : 0;
     default:         return 0;
     }
@@ -332,6 +335,8 @@ static size_t block_bytes(uint32_t qtype)
     case OXH_Q8_0:   return OXH_Q8_0_BYTES;
     case OXH_Q4_K_S:
     case OXH_Q4_K_M: return OXH_Q4_K_BYTES;
+    case OXH_Q5_K_S:
+    case OXH_Q5_K_M: return OXH_Q5_K_BYTES;
     case OXH_Q6_K:   return OXH_Q6_K_BYTES;
     default:         return 0;
     }
@@ -413,6 +418,7 @@ static hipError_t raise_all_lds_ceilings(void)
     if ((e = raise_lds_ceiling(KERNEL<1, false>)) != hipSuccess) return e;    \
     if ((e = raise_lds_ceiling(KERNEL<0, false>)) != hipSuccess) return e;
     OXH_RAISE(k_gemv_q4_k)
+    OXH_RAISE(k_gemv_q5_k)
     OXH_RAISE(k_gemv_q6_k)
     OXH_RAISE(k_gemv_q8_0)
 #undef OXH_RAISE
@@ -424,6 +430,7 @@ static hipError_t raise_all_lds_ceilings(void)
 }
 
 static bool is_q4k(uint32_t qtype) { return qtype == OXH_Q4_K_S || qtype == OXH_Q4_K_M; }
+static bool is_q5k(uint32_t qtype) { return qtype == OXH_Q5_K_S || qtype == OXH_Q5_K_M; }
 
 static uint32_t act_lds_bytes(uint32_t qtype, uint32_t blocks)
 {
@@ -664,6 +671,7 @@ static int launch_gemv(uint32_t qtype, const OxhSegment *segs, size_t n_segs, si
         else                 hipLaunchKernelGGL((KERNEL<0, false>), grid, block, lds, st, t, p, a); \
     } while (0)
     if (is_q4k(qtype))          OXH_LAUNCH(k_gemv_q4_k);
+    else if (is_q5k(qtype))     OXH_LAUNCH(k_gemv_q5_k);
     else if (qtype == OXH_Q6_K) OXH_LAUNCH(k_gemv_q6_k);
     else                        OXH_LAUNCH(k_gemv_q8_0);
 #undef OXH_LAUNCH

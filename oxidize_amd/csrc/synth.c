@@ -1,6 +1,6 @@
 /*
  * synth.c — seeded synthetic tensors for the quantized-matvec benchmarks and
- * tests: raw Q4_K / Q6_K / Q8_0 weight blocks and f32 activations.
+ * tests: raw Q4_K / Q5_K / Q6_K / Q8_0 weight blocks and f32 activations.
  *
  * Everything is integer arithmetic plus exactly-representable float steps, so
  * the same (seed, stream, index) yields the same bits on every machine and at
@@ -12,6 +12,8 @@
  *
  * Block contents follow the layouts the kernels consume (GGUF):
  *   Q4_K 144 B: f16 d, f16 dmin, 12 B packed 6-bit scales/mins, 128 B nibbles
+ *   Q5_K 176 B: f16 d, f16 dmin, 12 B packed 6-bit scales/mins, 32 B fifth-bit
+ *               plane, 128 B nibbles
  *   Q6_K 210 B: 128 B ql, 64 B qh, 16 int8 scales, f16 d
  *   Q8_0  34 B: f16 d, 32 int8
  */
@@ -116,6 +118,36 @@ void oxs_fill_q4_k(uint8_t *dst, size_t n_blocks, uint64_t seed,
             s[j + 8] = (uint8_t)((sc[j + 4] & 15u) | ((mn[j + 4] & 15u) << 4));
         }
         for (int i = 0; i < 16; i++) {
+            const uint64_t w = next64(&r);
+            memcpy(blk + 16 + 8 * i, &w, 8);
+        }
+    }
+}
+
+/* Q5_K blocks: the Q4_K header, then 32 bytes of fifth bits and 128 bytes of
+ * nibbles, all uniform (codes uniform in [0,31]). */
+void oxs_fill_q5_k(uint8_t *dst, size_t n_blocks, uint64_t seed,
+                   uint64_t stream, float sigma)
+{
+#pragma omp parallel for schedule(static)
+    for (long b = 0; b < (long)n_blocks; b++) {
+        Rng r = rng_for(seed, stream, (uint64_t)b);
+        uint8_t *blk = dst + (size_t)b * 176u;
+        put16(blk, half_abs_normal(&r, sigma));
+        put16(blk + 2, half_abs_normal(&r, sigma));
+        uint8_t sc[8], mn[8];
+        uint64_t u = next64(&r), v = next64(&r);
+        for (int j = 0; j < 8; j++) {
+            sc[j] = (uint8_t)((u >> (6 * j)) & 63u);
+            mn[j] = (uint8_t)((v >> (6 * j)) & 63u);
+        }
+        uint8_t *s = blk + 4;
+        for (int j = 0; j < 4; j++) {
+            s[j]     = (uint8_t)(sc[j] | ((sc[j + 4] >> 4) << 6));
+            s[j + 4] = (uint8_t)(mn[j] | ((mn[j + 4] >> 4) << 6));
+            s[j + 8] = (uint8_t)((sc[j + 4] & 15u) | ((mn[j + 4] & 15u) << 4));
+        }
+        for (int i = 0; i < 20; i++) {
             const uint64_t w = next64(&r);
             memcpy(blk + 16 + 8 * i, &w, 8);
         }

@@ -14,7 +14,7 @@ import numpy as np
 from . import _lib
 from ._lib import DECLINED, OK, OxhError, OxhSegment, check, lib
 
-Q8_0, Q4_K_S, Q4_K_M, Q6_K = 7, 12, 13, 16
+Q8_0, Q4_K_S, Q4_K_M, Q5_K_S, Q5_K_M, Q6_K = 7, 12, 13, 14, 15, 16
 
 
 def _p(a):

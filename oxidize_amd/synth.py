@@ -1,9 +1,10 @@
-"""Seeded synthetic tensors (raw Q4_K / Q6_K / Q8_0 blocks, f32 activations).
+"""Seeded synthetic tensors (raw Q4_K / Q5_K / Q6_K / Q8_0 blocks, f32 activations).
 
 Thin ctypes wrapper over ``liboxsynth.so`` (built from ``csrc/synth.c``).  The
 generator is integer-only, so the same seed gives the same bytes everywhere.
 Shapes and distributions follow the benchmark configurations: Q4_K d/dmin
-~ |N(0,0.02)|, 6-bit scales/mins uniform, nibbles uniform; Q6_K int8 scales in
+~ |N(0,0.02)|, 6-bit scales/mins uniform, nibbles uniform (Q5_K: the same plus a
+uniform fifth-bit plane); Q6_K int8 scales in
 [-32,31], codes uniform; Q8_0 int8 in [-127,127], d ~ |N(0,0.01)|.
 """
 import ctypes
@@ -14,9 +15,9 @@ import numpy as np
 _HERE = os.path.dirname(os.path.abspath(__file__))
 _LIB = None
 
-Q8_0, Q4_K, Q6_K = 7, 13, 16
-BLOCK_BYTES = {Q8_0: 34, Q4_K: 144, 12: 144, Q6_K: 210}
-BLOCK_ELEMS = {Q8_0: 32, Q4_K: 256, 12: 256, Q6_K: 256}
+Q8_0, Q4_K, Q5_K, Q6_K = 7, 13, 15, 16
+BLOCK_BYTES = {Q8_0: 34, Q4_K: 144, 12: 144, Q5_K: 176, 14: 176, Q6_K: 210}
+BLOCK_ELEMS = {Q8_0: 32, Q4_K: 256, 12: 256, Q5_K: 256, 14: 256, Q6_K: 256}
 
 
 def _lib():
@@ -27,7 +28,7 @@ def _lib():
             raise RuntimeError(
                 "liboxsynth.so is not built; run `python -c 'import __graft_entry__ as g; g.build()'`")
         lib = ctypes.CDLL(path)
-        for name in ("oxs_fill_q4_k", "oxs_fill_q6_k", "oxs_fill_q8_0"):
+        for name in ("oxs_fill_q4_k", "oxs_fill_q5_k", "oxs_fill_q6_k", "oxs_fill_q8_0"):
             getattr(lib, name).argtypes = [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_uint64,
                                            ctypes.c_uint64, ctypes.c_float]
             getattr(lib, name).restype = None
@@ -52,7 +53,7 @@ def weights(qtype, rows, cols, seed=0, stream=0, sigma=None, out=None):
         out = np.empty(nbytes, dtype=np.uint8)
     assert out.dtype == np.uint8 and out.size == nbytes and out.flags.c_contiguous
     fn = {Q8_0: "oxs_fill_q8_0", Q4_K: "oxs_fill_q4_k", 12: "oxs_fill_q4_k",
-          Q6_K: "oxs_fill_q6_k"}[qtype]
+          Q5_K: "oxs_fill_q5_k", 14: "oxs_fill_q5_k", Q6_K: "oxs_fill_q6_k"}[qtype]
     if sigma is None:
         sigma = 0.01 if qtype == Q8_0 else 0.02
     getattr(_lib(), fn)(out.ctypes.data, n_blocks, seed, stream, sigma)

@@ -5,6 +5,8 @@ committed, this script documents how they were made.
 
     python tests/golden/make_golden.py
 
+    python tests/golden/make_golden.py q5_k     # only q5_k.npz
+
 Every array is data: inputs and the reference's outputs for them.
 """
 import ctypes
@@ -22,7 +24,7 @@ sys.path.insert(0, os.path.join(ROOT, "tests"))
 import oxlibs  # noqa: E402
 from oxidize_amd import synth  # noqa: E402
 
-Q80, Q4K, Q6K = 7, 13, 16
+Q80, Q4K, Q5K, Q6K = 7, 13, 15, 16
 
 
 def xorshift_bytes(n, seed):
@@ -44,11 +46,91 @@ def finite_scale_bits(rng, n):
     return vals.astype(np.float16).view(np.uint16)
 
 
+def q8k_acts(rng, trials, nb):
+    act = np.zeros((trials, nb, 292), np.uint8)
+    d = (0.001 + rng.integers(0, 1000, (trials, nb)) * 2e-5).astype(np.float32)
+    act[:, :, 0:4] = d.view(np.uint8).reshape(trials, nb, 4)
+    q = rng.integers(-127, 128, (trials, nb, 256)).astype(np.int8)
+    act[:, :, 4:260] = q.view(np.uint8)
+    bs = q.reshape(trials, nb, 16, 16).sum(axis=3).astype(np.int16)
+    act[:, :, 260:292] = bs.view(np.uint8).reshape(trials, nb, 32)
+    return act
+
+
+def q5_k(ref):
+    """q5_k.npz: the same three kinds of vectors as the other files, for Q5_K
+    (a file and a generator of its own, so the older fixtures stay byte for
+    byte what they were)."""
+    rng = np.random.default_rng(20240915)
+    out = {}
+    nb, trials = 12, 24
+    w = xorshift_bytes(trials * nb * 176, 0x9E3779B9 ^ Q5K).reshape(trials, nb, 176)
+    for off in (0, 2):
+        bits = finite_scale_bits(rng, trials * nb).reshape(trials, nb)
+        w[:, :, off] = bits & 0xFF
+        w[:, :, off + 1] = bits >> 8
+    act = q8k_acts(rng, trials, nb)
+    scalar = np.empty((trials, 2), np.uint32)
+    disp = np.empty((trials, 2), np.uint32)
+    for t in range(trials):
+        wt = np.ascontiguousarray(w[t])
+        at = np.ascontiguousarray(act[t])
+        for k, blocks in enumerate((1, nb)):
+            scalar[t, k] = np.float32(ref.oc_oxk_dot_q5_k_q8_k_scalar(
+                wt.ctypes.data, blocks, at.ctypes.data)).view(np.uint32)
+            disp[t, k] = np.float32(ref.oc_oxk_dot_q5_k_q8_k(
+                wt.ctypes.data, blocks, at.ctypes.data)).view(np.uint32)
+    out["raw_w"], out["raw_act"] = w, act
+    out["raw_scalar_bits"], out["raw_dispatched_bits"] = scalar, disp
+
+    # API level, both type ids
+    for qt, rows, cols in ((15, 40, 1280), (14, 9, 256)):
+        rb = synth.row_bytes(qt, cols)
+        wm = synth.weights(qt, rows, cols, seed=7, stream=qt)
+        x = synth.normal(cols, seed=7, stream=100 + qt)
+        o = np.zeros(rows, np.float32)
+        temp = np.zeros(cols, np.float32)
+        ref.oc_matvec_quantized(qt, wm.ctypes.data, rows, cols, rb, x.ctypes.data, o.ctypes.data,
+                                temp.ctypes.data)
+        key = "api%d_" % qt
+        out[key + "w"], out[key + "x"] = wm, x
+        out[key + "shape"] = np.array([rows, cols, rb], np.int64)
+        out[key + "out_bits"] = o.view(np.uint32).copy()
+        out[key + "act"] = temp.view(np.uint8)[:cols // 256 * 292].copy()
+        n_vec, in_stride, out_stride = 5, cols + 8, rows + 3
+        xs = synth.normal(n_vec * in_stride, seed=8, stream=qt).reshape(n_vec, in_stride)
+        outs = np.full((n_vec, out_stride), -1.0, np.float32)
+        scratch = np.zeros(ref.oc_matvec_batch_scratch_bytes(cols), np.uint8)
+        ref.oc_matvec_quantized_batch(qt, wm.ctypes.data, rows, cols, rb, xs.ctypes.data, in_stride,
+                                      outs.ctypes.data, out_stride, n_vec, temp.ctypes.data,
+                                      scratch.ctypes.data, scratch.nbytes)
+        out[key + "batch_x"] = xs
+        out[key + "batch_out_bits"] = outs.view(np.uint32).copy()
+
+    # full-size shapes: checksums and the f32 outputs
+    for name, rows, cols in (("big_4096x4096", 4096, 4096), ("big_4096x14336", 4096, 14336)):
+        rb = synth.row_bytes(Q5K, cols)
+        wm = synth.weights(Q5K, rows, cols, seed=0, stream=0)
+        x = synth.normal(cols, seed=0, stream=1000)
+        o = np.zeros(rows, np.float32)
+        temp = np.zeros(cols, np.float32)
+        ref.oc_matvec_quantized(Q5K, wm.ctypes.data, rows, cols, rb, x.ctypes.data, o.ctypes.data,
+                                temp.ctypes.data)
+        out[name + "_crc_w"] = np.array([zlib.crc32(wm.tobytes())], np.uint32)
+        out[name + "_crc_x"] = np.array([zlib.crc32(x.tobytes())], np.uint32)
+        out[name + "_crc_out"] = np.array([zlib.crc32(o.tobytes())], np.uint32)
+        out[name + "_out"] = o.copy()
+    np.savez_compressed(os.path.join(HERE, "q5_k.npz"), **out)
+
+
 def main():
     ref = oxlibs.ref()
     if ref is None:
         raise SystemExit("oracle/_ref/liboxref.so missing: run `make -C oracle` first")
     ref.oc_parallel_set_threads(1)
+    q5_k(ref)
+    if sys.argv[1:] == ["q5_k"]:
+        return
     rng = np.random.default_rng(20240607)
 
     # ── scalar helpers ────────────────────────────────────────────────────

@@ -39,6 +39,7 @@ def oracle():
         lib.oxo_quantize_q8_k.argtypes = [V, Z, V]; lib.oxo_quantize_q8_k.restype = None
         lib.oxo_quantize_q8_0.argtypes = [V, Z, V]; lib.oxo_quantize_q8_0.restype = None
         lib.oxo_dot_q4_k_q8_k.argtypes = [V, Z, V, V, V]; lib.oxo_dot_q4_k_q8_k.restype = F
+        lib.oxo_dot_q5_k_q8_k.argtypes = [V, Z, V, V, V]; lib.oxo_dot_q5_k_q8_k.restype = F
         lib.oxo_dot_q6_k_q8_k.argtypes = [V, Z, V, V]; lib.oxo_dot_q6_k_q8_k.restype = F
         lib.oxo_dot_q8_0_q8_0.argtypes = [V, Z, V, V]; lib.oxo_dot_q8_0_q8_0.restype = F
         lib.oxo_act_kind.argtypes = [U32, Z]; lib.oxo_act_kind.restype = ctypes.c_int
@@ -73,7 +74,7 @@ def ref():
         lib.oc_f32_to_f16_bits.argtypes = [F]; lib.oc_f32_to_f16_bits.restype = ctypes.c_uint16
         lib.oc_oxk_get_scale_min_k4.argtypes = [ctypes.c_uint, V, V, V]
         lib.oc_oxk_get_scale_min_k4.restype = None
-        for n in ("q4_k_q8_k", "q6_k_q8_k", "q8_0_q8_0"):
+        for n in ("q4_k_q8_k", "q5_k_q8_k", "q6_k_q8_k", "q8_0_q8_0"):
             for suf in ("", "_scalar"):
                 f = getattr(lib, "oc_oxk_dot_" + n + suf)
                 f.argtypes = [V, Z, V]; f.restype = F

@@ -19,7 +19,7 @@ import oxlibs
 from oxidize_amd import synth
 
 GOLD = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
-Q80, Q4K, Q6K = 7, 13, 16
+Q80, Q4K, Q5K, Q6K = 7, 13, 15, 16
 O = oxlibs.oracle()
 
 
@@ -138,6 +138,8 @@ def dot(name, w, blocks, act, extra=None):
     act = np.ascontiguousarray(act)
     if name == "q4_k":
         return O.oxo_dot_q4_k_q8_k(w.ctypes.data, blocks, act.ctypes.data, extra, None)
+    if name == "q5_k":
+        return O.oxo_dot_q5_k_q8_k(w.ctypes.data, blocks, act.ctypes.data, extra, None)
     if name == "q6_k":
         return O.oxo_dot_q6_k_q8_k(w.ctypes.data, blocks, act.ctypes.data, extra)
     return O.oxo_dot_q8_0_q8_0(w.ctypes.data, blocks, act.ctypes.data, extra)
@@ -164,6 +166,7 @@ def test_known_answer_dots():
     # all-zero K blocks -> 0 (oxidize-c/tests/test_oxk_extended.c:213-270)
     assert dot("q4_k", np.zeros(144, np.uint8), 1, np.zeros(292, np.uint8)) == 0.0
     assert dot("q6_k", np.zeros(210, np.uint8), 1, np.zeros(292, np.uint8)) == 0.0
+    assert dot("q5_k", np.zeros(176, np.uint8), 1, np.zeros(292, np.uint8)) == 0.0
 
 
 def q8k_block(d, q):
@@ -218,6 +221,97 @@ def test_q4_k_each_sub_block_uses_its_own_scale_and_nibble_half():
         assert dot("q4_k", w, 1, act) == -float(q[32 * j:32 * j + 32].sum())
 
 
+def q5k_block(d, dmin, sc, mn, codes):
+    """Q5_K from 256 codes in [0,31]: the Q4_K header, then the fifth bits
+    (bit j of byte l belongs to element 32j + l), then the nibbles."""
+    codes = np.asarray(codes, np.uint8)
+    q4 = q4k_block(d, dmin, sc, mn, codes & 15)
+    hi = (codes >> 4).reshape(8, 32)
+    plane = np.zeros(32, np.uint8)
+    for j in range(8):
+        plane |= (hi[j] << j).astype(np.uint8)
+    return np.concatenate([q4[:16], plane, q4[16:]])
+
+
+def test_q5_k_raw_block_dots_float_bits_vs_reference():
+    g = load("q5_k.npz")
+    w, act = g["raw_w"], g["raw_act"]
+    for t in range(w.shape[0]):
+        for k, blocks in enumerate((1, w.shape[1])):
+            got = f32bits(dot("q5_k", w[t], blocks, act[t]))
+            assert got == g["raw_scalar_bits"][t, k]
+            assert got == g["raw_dispatched_bits"][t, k]
+
+
+def test_q5_k_closed_form_and_fifth_bit_placement():
+    d, dmin, dq, s, m, a = 0.5, 0.25, 0.125, 3, 5, 2
+    for code in (7, 16, 23, 31):
+        w = q5k_block(d, dmin, [s] * 8, [m] * 8, [code] * 256)
+        act = q8k_block(dq, [a] * 256)
+        assert dot("q5_k", w, 1, act) == dq * d * 256 * s * code * a - dq * dmin * 256 * m * a
+    # one element with only its fifth bit set, one non-zero scale: the result is
+    # 16 * that element's activation, for every element position
+    rng = np.random.default_rng(11)
+    q = rng.integers(-127, 128, 256)
+    act = q8k_block(1.0, q)
+    for e in list(range(0, 256, 37)) + [31, 32, 63, 64, 255]:
+        codes = np.zeros(256, np.uint8)
+        codes[e] = 16
+        sc = [0] * 8
+        sc[e // 32] = 1
+        w = q5k_block(1.0, 0.0, sc, [0] * 8, codes)
+        sub = np.zeros(8, np.int32)
+        assert dot("q5_k", w, 1, act, sub.ctypes.data) == 16.0 * q[e]
+        assert sub[e // 32] == 16 * q[e] and np.count_nonzero(sub) == (1 if q[e] else 0)
+    # one-hot scales isolate each sub-block's integer sum
+    codes = rng.integers(0, 32, 256)
+    for j in range(8):
+        sc = [0] * 8
+        sc[j] = 1
+        w = q5k_block(1.0, 0.0, sc, [0] * 8, codes)
+        assert dot("q5_k", w, 1, act) == float(np.dot(codes[32 * j:32 * j + 32], q[32 * j:32 * j + 32]))
+
+
+@pytest.mark.parametrize("qt", [15, 14])
+def test_q5_k_matvec_and_batch_vs_reference_goldens(qt):
+    g = load("q5_k.npz")
+    key = "api%d_" % qt
+    rows, cols, rb = (int(v) for v in g[key + "shape"])
+    w, x = g[key + "w"], g[key + "x"]
+    out = np.zeros(rows, np.float32)
+    temp = np.zeros(cols, np.float32)
+    assert O.oxo_matvec_quantized(qt, w.ctypes.data, rows, cols, rb, x.ctypes.data,
+                                  out.ctypes.data, temp.ctypes.data) == 0
+    act = g[key + "act"]
+    assert np.array_equal(temp.view(np.uint8)[:act.size], act)
+    assert np.array_equal(out.view(np.uint32), g[key + "out_bits"])
+    xs = g[key + "batch_x"]
+    n_vec, in_stride = xs.shape
+    want = g[key + "batch_out_bits"]
+    out_stride = want.shape[1]
+    outs = np.full((n_vec, out_stride), -1.0, np.float32)
+    scratch = np.zeros(O.oxo_matvec_batch_scratch_bytes(cols), np.uint8)
+    assert O.oxo_matvec_quantized_batch(qt, w.ctypes.data, rows, cols, rb, xs.ctypes.data, in_stride,
+                                        outs.ctypes.data, out_stride, n_vec, scratch.ctypes.data,
+                                        scratch.nbytes) == 0
+    assert np.array_equal(outs.view(np.uint32), want)
+
+
+@pytest.mark.parametrize("name,rows,cols", [("big_4096x4096", 4096, 4096), ("big_4096x14336", 4096, 14336)])
+def test_q5_k_full_size_vs_reference_checksums(name, rows, cols):
+    g = load("q5_k.npz")
+    w = synth.weights(Q5K, rows, cols, seed=0, stream=0)
+    x = synth.normal(cols, seed=0, stream=1000)
+    assert zlib.crc32(w.tobytes()) == int(g[name + "_crc_w"][0])
+    assert zlib.crc32(x.tobytes()) == int(g[name + "_crc_x"][0])
+    out = np.zeros(rows, np.float32)
+    temp = np.zeros(cols, np.float32)
+    assert O.oxo_matvec_quantized(Q5K, w.ctypes.data, rows, cols, synth.row_bytes(Q5K, cols),
+                                  x.ctypes.data, out.ctypes.data, temp.ctypes.data) == 0
+    assert zlib.crc32(out.tobytes()) == int(g[name + "_crc_out"][0])
+    assert np.array_equal(out, g[name + "_out"])
+
+
 def test_q6_k_codes_zero_give_minus_32_times_scale_sum():
     # all codes 0 -> every weight is d*sc*(-32)  (oxidize-c/tests/test_quant.c:290-310)
     blk = np.zeros(210, np.uint8)
@@ -229,7 +323,8 @@ def test_q6_k_codes_zero_give_minus_32_times_scale_sum():
     assert dot("q6_k", blk, 1, act) == float(want)
 
 
-@pytest.mark.parametrize("name,qt,group", [("q4_k", Q4K, 256), ("q6_k", Q6K, 256), ("q8_0", Q80, 32)])
+@pytest.mark.parametrize("name,qt,group", [("q4_k", Q4K, 256), ("q5_k", Q5K, 256), ("q6_k", Q6K, 256),
+                                           ("q8_0", Q80, 32)])
 def test_dot_agrees_with_dequantised_double_precision(name, qt, group):
     """Kernel-vs-layout check of oxidize-c/tests/test_oxk_gguf_layout.c:104-141:
     dot the dequantised weights with the dequantised activation in double."""
@@ -259,7 +354,7 @@ def test_dot_agrees_with_dequantised_double_precision(name, qt, group):
 def test_every_weight_byte_influences_the_dot():
     # oxidize-c/tests/test_quant.c:569-583, applied to the dot kernels
     rng = np.random.default_rng(3)
-    for name, qt, size in (("q4_k", Q4K, 144), ("q6_k", Q6K, 210), ("q8_0", Q80, 34)):
+    for name, qt, size in (("q4_k", Q4K, 144), ("q5_k", Q5K, 176), ("q6_k", Q6K, 210), ("q8_0", Q80, 34)):
         group = 32 if qt == Q80 else 256
         w = synth.weights(qt, 1, group, seed=13, stream=qt)
         if qt == Q80:
@@ -335,6 +430,8 @@ def test_eligibility_rules():
     assert O.oxo_act_kind(Q6K, 256) == 2 and O.oxo_act_kind(12, 512) == 2
     assert O.oxo_act_kind(Q80, 896) == 1 and O.oxo_act_kind(Q80, 900) == 0
     assert O.oxo_act_kind(0, 4096) == 0 and O.oxo_act_kind(1, 4096) == 0
+    assert O.oxo_act_kind(14, 512) == 2 and O.oxo_act_kind(Q5K, 4096) == 2 and O.oxo_act_kind(Q5K, 4000) == 0
+    assert O.oxo_stride_ok(Q5K, 4096, 2816) == 1 and O.oxo_stride_ok(Q5K, 4096, 2304) == 0
     assert O.oxo_stride_ok(Q4K, 4096, 2304) == 1 and O.oxo_stride_ok(Q4K, 4096, 2320) == 0
     assert O.oxo_stride_ok(Q6K, 14336, 11760) == 1 and O.oxo_stride_ok(Q80, 896, 952) == 1
     assert O.oxo_matvec_batch_scratch_bytes(4096) == 4 << 20
@@ -360,7 +457,8 @@ def test_moe_route_brute_force():
 def test_oracle_vs_live_reference_many_rows():
     ref = oxlibs.ref()
     ref.oc_parallel_set_threads(2)
-    for qt, rows, cols in ((Q4K, 700, 4096), (Q6K, 300, 14336), (Q4K, 513, 2816), (Q6K, 64, 256)):
+    for qt, rows, cols in ((Q4K, 700, 4096), (Q6K, 300, 14336), (Q4K, 513, 2816), (Q6K, 64, 256),
+                           (Q5K, 300, 4096), (14, 65, 768)):
         rb = synth.row_bytes(qt, cols)
         w = synth.weights(qt, rows, cols, seed=77, stream=rows)
         x = synth.normal(cols, seed=77)
