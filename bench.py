@@ -113,6 +113,42 @@ def secondary_figures(mv, synth):
     d_x.free()
     d_a.free()
     d_o.free()
+    # Q5_K (the other K-quant behind the same API): decode GEMV and 512-token
+    # prefill at the gate/up shape, 28672 x 4096
+    Q5K = 15
+    rows, cols = 28672, 4096
+    w = synth.weights(Q5K, rows, cols, seed=0, stream=4)
+    copies = [mv.DeviceBuffer.from_host(w) for _ in range(8)]    # 646 MB: beyond the last-level cache
+    x = synth.normal(n_vec * cols, seed=0, stream=2002)
+    d_x = mv.DeviceBuffer.from_host(x)
+    d_a = mv.DeviceBuffer(n_vec * mv.act_bytes(Q5K, cols))
+    d_o = mv.DeviceBuffer(n_vec * rows * 4)
+    segs = [mv.make_segments([(c.ptr, d_o.ptr, rows, 0)]) for c in copies]
+    state = {"i": 0}
+
+    def run_q5_gemv():
+        state["i"] += 1
+        mv.gemv_segments_f32(Q5K, segs[state["i"] % 8], cols, d_x.ptr, cols, None, 1, rows)
+
+    def run_q5_mmq():
+        state["i"] += 1
+        mv.mmq(Q5K, copies[state["i"] % 8].ptr, rows, cols, d_a.ptr, n_vec, d_o.ptr, rows)
+
+    us = timed(run_q5_gemv, 32, mv)
+    nbytes = w.nbytes + 4 * cols + 4 * rows
+    mv.quantize(Q5K, d_x.ptr, cols, n_vec, cols, d_a.ptr)
+    us_mma = timed(run_q5_mmq, 12, mv)
+    ops = 2.0 * rows * cols * n_vec
+    out["q5k_28672x4096"] = {
+        "gemv_batch1": {"us": round(us, 2), "gbps": round(nbytes / us / 1e3, 1),
+                        "frac_of_hbm_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBPS, 4)},
+        "mmq_512_tokens": {"mfma_kernel_only_us": round(us_mma, 2), "tops": round(ops / us_mma / 1e6, 1),
+                           "mfma_kernel_only_frac_of_int8_peak": round(ops / us_mma / 1e6 / INT8_PEAK_TOPS, 4)}}
+    for c in copies:
+        c.free()
+    d_x.free()
+    d_a.free()
+    d_o.free()
     # Q8_0 lm_head (configuration 2), batch 1 and 8
     rows, cols = 151936, 896
     w = synth.weights(Q80, rows, cols, seed=0, stream=5)

@@ -506,11 +506,12 @@ int oxh_matvec_quantized_batch(uint32_t qtype, const uint8_t *data, size_t rows,
                                      cols * sizeof(float), NULL)))
                 return rc;
     }
-    /* More vectors than the GEMV kernel keeps in flight: Q4_K and Q6_K go to the
+    /* More vectors than the GEMV kernel keeps in flight: Q4_K, Q5_K and Q6_K go to the
      * int8-MFMA kernel behind a stand-alone quantiser launch; everything else
      * walks the batch in GEMV-sized slices with the quantisation fused in
      * (every output is the same dot either way). */
-    if (n_vec > 8 && (qtype == OXH_Q4_K_S || qtype == OXH_Q4_K_M || qtype == OXH_Q6_K)) {
+    if (n_vec > 8 && (qtype == OXH_Q4_K_S || qtype == OXH_Q4_K_M || qtype == OXH_Q5_K_S ||
+                      qtype == OXH_Q5_K_M || qtype == OXH_Q6_K)) {
         if ((rc = quantize(kind, (const float *)g_dx.p, in_stride, n_vec, cols, g_dact.p))) return rc;
         if ((rc = oxh_mmq(qtype, d_w, rows, cols, g_dact.p, n_vec, (float *)g_dout.p, rows, NULL)))
             return rc;

@@ -424,6 +424,8 @@ static hipError_t raise_all_lds_ceilings(void)
 #undef OXH_RAISE
     if ((e = raise_lds_ceiling(k_mmq_q4_k<8, 2, 8>)) != hipSuccess) return e;
     if ((e = raise_lds_ceiling(k_mmq_q4_k<4, 1, 8>)) != hipSuccess) return e;
+    if ((e = raise_lds_ceiling(k_mmq_q5_k<8, 1, 8>)) != hipSuccess) return e;
+    if ((e = raise_lds_ceiling(k_mmq_q5_k<4, 1, 8>)) != hipSuccess) return e;
     if ((e = raise_lds_ceiling(k_mmq_q6_k<8, 1, 8>)) != hipSuccess) return e;
     if ((e = raise_lds_ceiling(k_mmq_q6_k<4, 1, 8>)) != hipSuccess) return e;
     return hipSuccess;
@@ -506,7 +508,8 @@ static bool gemv_wants_mfma(uint32_t qtype, const GemvIo &io, size_t max_nv, con
 {
     static int min_nv = -1;
     if (min_nv < 0) min_nv = (int)env_u32("OXH_GEMV_MFMA_MIN_NV", 3, 0, 64);
-    if ((!is_q4k(qtype) && qtype != OXH_Q6_K) || dump || min_nv == 0 || max_nv < (size_t)min_nv) return false;
+    if ((!is_q4k(qtype) && !is_q5k(qtype) && qtype != OXH_Q6_K) || dump || min_nv == 0 ||
+        max_nv < (size_t)min_nv) return false;
     return io.d_acts != nullptr || io.d_act_out != nullptr;
 }
 
@@ -542,6 +545,12 @@ static int launch_mmq_segments(uint32_t qtype, const OxhSegment *segs, size_t n_
         static_assert(G6::ROWS == G::ROWS, "segment tiling is shared by both formats");
         auto kernel = k_mmq_q6_k_segments<1, 1, 4>;
         hipLaunchKernelGGL(kernel, dim3(wg), dim3(4 * 64), G6::LDS_BYTES,
+                           pick_stream(stream), t, (uint32_t)blocks, acts, out_stride);
+    } else if (is_q5k(qtype)) {
+        typedef MmqGeom<1, 1, 4, true> G5;
+        static_assert(G5::ROWS == G::ROWS, "segment tiling is shared by all formats");
+        auto kernel = k_mmq_q5_k_segments<1, 1, 4>;
+        hipLaunchKernelGGL(kernel, dim3(wg), dim3(4 * 64), G5::LDS_BYTES,
                            pick_stream(stream), t, (uint32_t)blocks, acts, out_stride);
     } else {
         auto kernel = k_mmq_q4_k_segments<1, 1, 4>;
@@ -730,6 +739,18 @@ static void mmq_launch(const void *d_w, size_t rows, size_t blocks, const void *
 }
 
 template <int TC, int RC, int WAVES>
+static void mmq5_launch(const void *d_w, size_t rows, size_t blocks, const void *d_acts, size_t n_vec,
+                        float *d_out, size_t out_stride, void *stream)
+{
+    typedef MmqGeom<TC, RC, WAVES, true> G;
+    const dim3 grid((uint32_t)((rows + G::ROWS - 1) / G::ROWS), (uint32_t)((n_vec + G::TOK - 1) / G::TOK));
+    auto kernel = k_mmq_q5_k<TC, RC, WAVES>;
+    hipLaunchKernelGGL(kernel, grid, dim3(WAVES * 64), G::LDS_BYTES, pick_stream(stream),
+                       (const uint8_t *)d_w, (uint32_t)rows, (uint32_t)blocks,
+                       (const uint8_t *)d_acts, (uint32_t)n_vec, d_out, out_stride);
+}
+
+template <int TC, int RC, int WAVES>
 static void mmq6_launch(const void *d_w, size_t rows, size_t blocks, const void *d_acts, size_t n_vec,
                         float *d_out, size_t out_stride, void *stream)
 {
@@ -749,7 +770,7 @@ extern "C" int oxh_mmq(uint32_t qtype, const void *d_w, size_t rows, size_t cols
     if (rc) return rc;
     if (rows == 0 || n_vec == 0) return OXH_OK;
     if (!d_w || !d_acts || !d_out) return arg_fail("oxh_mmq: NULL pointer");
-    if ((!is_q4k(qtype) && qtype != OXH_Q6_K) || oxh_act_kind(qtype, cols) != 2) {
+    if ((!is_q4k(qtype) && !is_q5k(qtype) && qtype != OXH_Q6_K) || oxh_act_kind(qtype, cols) != 2) {
         snprintf(g_err, sizeof g_err, "oxh_mmq: qtype %u with cols %zu has no MFMA kernel", qtype, cols);
         return OXH_DECLINED;
     }
@@ -774,7 +795,7 @@ extern "C" int oxh_mmq(uint32_t qtype, const void *d_w, size_t rows, size_t cols
         else if (((rows + 127) / 128) * ((n_vec + 63) / 64) >= need) shape = 2;
         else shape = 3;
     }
-    if (qtype == OXH_Q6_K) {
+    if (qtype == OXH_Q6_K || is_q5k(qtype)) {
         /* one 16-row chunk per wave throughout: 128x128, 128x64, 64x32, 64x16 */
         if (!forced) {
             if (n_vec <= 16) shape = 4;
@@ -782,6 +803,14 @@ extern "C" int oxh_mmq(uint32_t qtype, const void *d_w, size_t rows, size_t cols
             else if (((rows + 127) / 128) * ((n_vec + 127) / 128) >= need) shape = 1;
             else if (((rows + 127) / 128) * ((n_vec + 63) / 64) >= need) shape = 2;
             else shape = 3;
+        }
+        if (is_q5k(qtype)) {
+            if (shape == 1)      mmq5_launch<8, 1, 8>(d_w, rows, blocks, d_acts, n_vec, d_out, out_stride, stream);
+            else if (shape == 2) mmq5_launch<4, 1, 8>(d_w, rows, blocks, d_acts, n_vec, d_out, out_stride, stream);
+            else if (shape == 3) mmq5_launch<2, 1, 4>(d_w, rows, blocks, d_acts, n_vec, d_out, out_stride, stream);
+            else                 mmq5_launch<1, 1, 4>(d_w, rows, blocks, d_acts, n_vec, d_out, out_stride, stream);
+            HIP_TRY(hipGetLastError());
+            return OXH_OK;
         }
         if (shape == 1)      mmq6_launch<8, 1, 8>(d_w, rows, blocks, d_acts, n_vec, d_out, out_stride, stream);
         else if (shape == 2) mmq6_launch<4, 1, 8>(d_w, rows, blocks, d_acts, n_vec, d_out, out_stride, stream);

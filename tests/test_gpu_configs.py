@@ -22,7 +22,7 @@ from oxidize_amd import synth, workloads
 
 pytestmark = pytest.mark.gpu
 GOLD = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
-Q80, Q4K, Q6K = 7, 13, 16
+Q80, Q4K, Q5K, Q6K = 7, 13, 15, 16
 
 
 def bits(a):
@@ -128,13 +128,14 @@ def test_config3_mmq_prefill_512_tokens(oxh, rows):
         want, wtemp = oracle_matvec(Q4K, w, rows, cols, np.ascontiguousarray(xs[v]))
         assert np.array_equal(acts[v], wtemp.view(np.uint8)[:nact]), v
         assert np.array_equal(bits(out[v]), bits(want)), v
-    # every token, a slice of rows: the MFMA path against the GEMV kernel on the same device data
-    d_o2 = mv.DeviceBuffer(8 * rows * 4)
-    for v0 in (8, 120, 504):
+    # the MFMA path against the dot-instruction GEMV kernel on the same device data
+    # (two activations per launch: three or more would run on the matrix cores too)
+    d_o2 = mv.DeviceBuffer(2 * rows * 4)
+    for v0 in (8, 10, 120, 126, 504, 510):
         segs = mv.make_segments([(d_w.ptr, d_o2.ptr, rows, v0)])
-        mv.gemv_segments(Q4K, segs, cols, d_a.ptr, 8, rows)
-        got = d_o2.download(np.float32, 8 * rows).reshape(8, rows)
-        assert np.array_equal(bits(got), bits(out[v0:v0 + 8]))
+        mv.gemv_segments(Q4K, segs, cols, d_a.ptr, 2, rows)
+        got = d_o2.download(np.float32, 2 * rows).reshape(2, rows)
+        assert np.array_equal(bits(got), bits(out[v0:v0 + 2]))
 
 
 @pytest.mark.parametrize("qtype,rows,cols,n_vec", [
@@ -144,13 +145,18 @@ def test_config3_mmq_prefill_512_tokens(oxh, rows):
     (Q6K, 7165, 512, 507),      # Q6_K: 128x128 tiles, 56 x 4
     (Q6K, 3600, 256, 500),      # Q6_K: 128x64 tiles, 29 x 8
     (Q6K, 4100, 512, 40),       # Q6_K: 64x32 tiles
+    (Q5K, 7165, 512, 507),      # Q5_K: 128x128 tiles, 56 x 4
+    (Q5K, 3600, 256, 500),      # Q5_K: 128x64 tiles, 29 x 8
+    (Q5K, 4100, 512, 40),       # Q5_K: 64x32 tiles
 ])
 def test_mmq_tile_variants_ragged(oxh, qtype, rows, cols, n_vec):
     """The MFMA kernel comes in several tile shapes (256x128, 128x64, 64x32,
     64x16 rows x tokens), picked from the launch size; these cases select the
     first three on a 256-CU device and leave the last row tile and the last
-    token tile partly filled.  Every output is checked against the GEMV kernel on
-    the same device data, and a sample of tokens against the oracle."""
+    token tile partly filled.  Every output is checked against the
+    dot-instruction GEMV kernel on the same device data (two activations per
+    launch: three or more would run on the matrix cores too), and a sample of
+    tokens against the oracle."""
     info = mv.device_info()
     if info["n_cu"] != 256:
         pytest.skip("tile choice is tied to 256 compute units")
@@ -170,13 +176,13 @@ def test_mmq_tile_variants_ragged(oxh, qtype, rows, cols, n_vec):
     for v in (0, 31, 32, n_vec // 2, n_vec - 1):
         want, _ = oracle_matvec(qtype, w, rows, cols, np.ascontiguousarray(xs[v]))
         assert np.array_equal(bits(out[v, :rows]), bits(want)), v
-    d_o2 = mv.DeviceBuffer(8 * rows * 4)
-    for v0 in range(0, n_vec, 8):
-        nv = min(8, n_vec - v0)
-        segs = mv.make_segments([(d_w.ptr, d_o2.ptr, rows, v0)])
+    d_o2 = mv.DeviceBuffer(n_vec * rows * 4)
+    for v0 in range(0, n_vec, 2):
+        nv = min(2, n_vec - v0)
+        segs = mv.make_segments([(d_w.ptr, d_o2.ptr + v0 * rows * 4, rows, v0)])
         mv.gemv_segments(qtype, segs, cols, d_a.ptr, nv, rows)
-        got = d_o2.download(np.float32, 8 * rows).reshape(8, rows)[:nv]
-        assert np.array_equal(bits(got), bits(out[v0:v0 + nv, :rows])), v0
+    got = d_o2.download(np.float32, n_vec * rows).reshape(n_vec, rows)
+    assert np.array_equal(bits(got), bits(out[:, :rows]))
 
 
 def test_config4_moe_expert_gemvs(oxh):
