@@ -125,10 +125,51 @@ int oxh_gemv_segments_f32(uint32_t qtype, const OxhSegment *segs, size_t n_segs,
                           void *d_act_out, size_t n_vec, size_t out_stride,
                           void *stream);
 
+/* The same launch with one more step fused in front of the quantiser, so that
+ * a decode layer needs no stand-alone normalisation or activation kernel and
+ * no f32 round trip between its matmuls:
+ *   OXH_PRO_RMSNORM  quantises x[i] * inv_rms * d_b[i] with
+ *                    inv_rms = 1/sqrt(mean(x^2) + eps); d_b = the norm weight,
+ *                    cols floats shared by all vectors.  Replaces
+ *                    oc_rms_norm_f32 (oxidize-c/src/compute/activation.c:16-22)
+ *                    / k_f_rmsnorm (oxidize-c/src/backends/cuda_fast.cu:155-168)
+ *                    followed by the matvec.  With d_add != NULL the
+ *                    vector normalised is x + d_add (laid out like d_x) and,
+ *                    when d_sum_out != NULL, that sum is stored there: the
+ *                    residual update and the next norm in one step
+ *                    (k_f_residual_rms, cuda_fast.cu:171-189).
+ *   OXH_PRO_SWIGLU   quantises silu(x[i]) * d_b[v][i]; x = the gate vectors,
+ *                    d_b = the up vectors laid out like d_x.  Replaces
+ *                    oc_swiglu_inplace_f32 (activation.c:92-99) / k_f_swiglu
+ *                    (cuda_fast.cu:477-485) followed by the down projection.
+ * d_out (optional, laid out like d_x) receives the f32 result of the
+ * prologue.  No stored result may overlap an input or the other stored
+ * result: every workgroup reads the inputs while one per segment stores.  pro == NULL is oxh_gemv_segments_f32.
+ * These are float operations: the normalised / activated values agree with
+ * the reference's to rounding (its own SIMD variants differ from one another
+ * in summation order), and everything after them, quantised bytes included,
+ * is the exact integer path applied to those values.  Launches with a
+ * prologue always use the dot-instruction kernels (n_vec <= 8). */
+#define OXH_PRO_RMSNORM 1u
+#define OXH_PRO_SWIGLU  2u
+typedef struct OxhPrologue {
+    uint32_t     kind;
+    float        eps;     /* RMSNORM */
+    const float *d_b;
+    float       *d_out;
+    const float *d_add;     /* RMSNORM only, optional */
+    float       *d_sum_out; /* RMSNORM with d_add only, optional */
+} OxhPrologue;
+int oxh_gemv_segments_fused(uint32_t qtype, const OxhSegment *segs, size_t n_segs,
+                            size_t cols, const float *d_x, size_t x_stride,
+                            const OxhPrologue *pro, void *d_act_out, size_t n_vec,
+                            size_t out_stride, void *stream);
+
 /* Prefill matmul on int8 MFMA: out[v*out_stride + r] = dot(W[r], act[v]) for
- * v < n_vec (any count), Q8_K activations.  Replaces the prepared-row batch
- * kernels oc_oxk_q4_k_prep_row + oc_oxk_dot_q4_k_prepped_multi
- * (oxidize-c/src/compute/oxk.c:316-366, :787-836) driven by
+ * v < n_vec (any count), Q8_K activations, Q4_K / Q5_K / Q6_K weights.
+ * Replaces the prepared-row batch kernels oc_oxk_q4_k_prep_row (and
+ * oc_oxk_q5_k_prep_row, oc_oxk_q6_k_prep_row) + oc_oxk_dot_q4_k_prepped_multi
+ * (oxidize-c/src/compute/oxk.c:316-366, :372-373, :787-836) driven by
  * matvec_batch_prep_slice (matvec.c:1198-1228). */
 int oxh_mmq(uint32_t qtype, const void *d_w, size_t rows, size_t cols,
             const void *d_acts, size_t n_vec, float *d_out, size_t out_stride,

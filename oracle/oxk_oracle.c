@@ -539,6 +539,26 @@ void oxo_moe_route(const float *logits, size_t n_tok, size_t n_expert,
     free(order);
 }
 
+/* ─── float steps in front of the quantiser ───────────────────────────── */
+
+void oxo_rms_norm_f32(const float *x, const float *weight, float *out, size_t n,
+                      float eps)
+{
+    float ss = 0.0f;
+    for (size_t i = 0; i < n; i++) ss += x[i] * x[i];
+    const float inv = 1.0f / sqrtf(ss / (float)n + eps);
+    for (size_t i = 0; i < n; i++) out[i] = x[i] * inv * weight[i];
+}
+
+void oxo_swiglu_f32(const float *gate, const float *up, float *out, size_t n)
+{
+    for (size_t i = 0; i < n; i++) {
+        const float g = gate[i];
+        const float sig = 1.0f / (1.0f + expf(-g));
+        out[i] = g * sig * up[i];
+    }
+}
+
 /* ─── dequantisation (layout cross-check only) ────────────────────────── */
 
 int oxo_dequant_row(uint32_t qtype, const uint8_t *row, size_t cols, float *out)

@@ -22,6 +22,9 @@
  *                         raw-block generator of tests/test_oxk_avx2_parity.c,
  *                         closed forms, dequantised double-precision cross-check
  *   oxo_matvec_*          compiled reference entry points, float bits
+ *   oxo_rms_norm_f32,     compiled reference (oc_rms_norm_f32, oc_swiglu_inplace_f32)
+ *   oxo_swiglu_f32        to 1e-6 relative, double-precision numpy, closed
+ *                         forms (constant vector, silu(0) = 0, large |g|)
  * No function is "parity unpinned".
  */
 #ifndef OXK_ORACLE_H
@@ -123,6 +126,16 @@ size_t oxo_matvec_batch_scratch_bytes(size_t max_cols);
  * keep the lower index), optional renormalisation.  ids/weights: n_tok*k. */
 void oxo_moe_route(const float *logits, size_t n_tok, size_t n_expert,
                    size_t k, int renorm, int32_t *ids, float *weights);
+
+/* The float steps a decode layer runs in front of the quantiser, scalar forms:
+ * RMSNorm (src/compute/activation.c:16-22 with the scalar dot and apply of
+ * src/compute/attn_kernels.c:6-11, :28-33) and SwiGLU
+ * (src/compute/activation.c:92-99).  The reference's x86 builds sum the
+ * squares in SIMD lanes and use a polynomial exp, so they agree with these
+ * to rounding, not to the bit. */
+void oxo_rms_norm_f32(const float *x, const float *weight, float *out, size_t n,
+                      float eps);
+void oxo_swiglu_f32(const float *gate, const float *up, float *out, size_t n);
 
 /* Dequantise one row to f32 (src/compute/quantization.c:486-503, :633-670,
  * :672-721, :723-766) — used only as an independent cross-check of the layouts. */

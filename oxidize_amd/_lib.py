@@ -22,6 +22,11 @@ class OxhSegment(ctypes.Structure):
     _fields_ = [("d_w", V), ("d_out", V), ("rows", Z), ("act_first", Z), ("n_vec", Z)]
 
 
+class OxhPrologue(ctypes.Structure):
+    _fields_ = [("kind", U32), ("eps", ctypes.c_float), ("d_b", V), ("d_out", V), ("d_add", V),
+                ("d_sum_out", V)]
+
+
 class OcMatvecFusedTestStats(ctypes.Structure):
     _fields_ = [("activation_quantizations", Z), ("parallel_dispatches", Z),
                 ("fallback_calls", Z)]
@@ -39,6 +44,8 @@ SIGNATURES = {
     "oxh_quantize_q8_0": (I, [V, Z, Z, Z, V, V]),
     "oxh_gemv_segments": (I, [U32, ctypes.POINTER(OxhSegment), Z, Z, V, Z, Z, V]),
     "oxh_gemv_segments_f32": (I, [U32, ctypes.POINTER(OxhSegment), Z, Z, V, Z, V, Z, Z, V]),
+    "oxh_gemv_segments_fused": (I, [U32, ctypes.POINTER(OxhSegment), Z, Z, V, Z,
+                                    ctypes.POINTER(OxhPrologue), V, Z, Z, V]),
     "oxh_mmq": (I, [U32, V, Z, Z, V, Z, V, Z, V]),
     "oxh_debug_subblock_sums": (I, [U32, V, Z, Z, V, V, V]),
     "oxh_malloc": (I, [ctypes.POINTER(V), Z]),

@@ -422,6 +422,18 @@ static hipError_t raise_all_lds_ceilings(void)
     OXH_RAISE(k_gemv_q6_k)
     OXH_RAISE(k_gemv_q8_0)
 #undef OXH_RAISE
+#define OXH_RAISE_PRO(KERNEL)                                                                     \
+    if ((e = raise_lds_ceiling(KERNEL<1, GEMV_PRO_RMSNORM>)) != hipSuccess) return e;             \
+    if ((e = raise_lds_ceiling(KERNEL<0, GEMV_PRO_RMSNORM>)) != hipSuccess) return e;             \
+    if ((e = raise_lds_ceiling(KERNEL<1, GEMV_PRO_SWIGLU>)) != hipSuccess) return e;              \
+    if ((e = raise_lds_ceiling(KERNEL<0, GEMV_PRO_SWIGLU>)) != hipSuccess) return e;              \
+    if ((e = raise_lds_ceiling(KERNEL<1, GEMV_PRO_ADD_RMSNORM>)) != hipSuccess) return e;         \
+    if ((e = raise_lds_ceiling(KERNEL<0, GEMV_PRO_ADD_RMSNORM>)) != hipSuccess) return e;
+    OXH_RAISE_PRO(k_gemv_q4_k_pro)
+    OXH_RAISE_PRO(k_gemv_q5_k_pro)
+    OXH_RAISE_PRO(k_gemv_q6_k_pro)
+    OXH_RAISE_PRO(k_gemv_q8_0_pro)
+#undef OXH_RAISE_PRO
     if ((e = raise_lds_ceiling(k_mmq_q4_k<8, 2, 8>)) != hipSuccess) return e;
     if ((e = raise_lds_ceiling(k_mmq_q4_k<4, 1, 8>)) != hipSuccess) return e;
     if ((e = raise_lds_ceiling(k_mmq_q5_k<8, 1, 8>)) != hipSuccess) return e;
@@ -497,6 +509,7 @@ struct GemvIo {
     const float *d_x;       /* f32 inputs to quantise in the kernel, or NULL */
     size_t x_stride;
     void *d_act_out;        /* optional store of the quantised bytes         */
+    const OxhPrologue *pro; /* fused prologue in front of the quantiser, or NULL */
 };
 
 /* Q4_K with three or more activations per weight goes to the matrix cores:
@@ -510,6 +523,8 @@ static bool gemv_wants_mfma(uint32_t qtype, const GemvIo &io, size_t max_nv, con
     if (min_nv < 0) min_nv = (int)env_u32("OXH_GEMV_MFMA_MIN_NV", 3, 0, 64);
     if ((!is_q4k(qtype) && !is_q5k(qtype) && qtype != OXH_Q6_K) || dump || min_nv == 0 ||
         max_nv < (size_t)min_nv) return false;
+    /* a prologue lives in the GEMV kernels' quantiser only */
+    if (io.pro) return false;
     return io.d_acts != nullptr || io.d_act_out != nullptr;
 }
 
@@ -651,6 +666,15 @@ static int launch_gemv(uint32_t qtype, const OxhSegment *segs, size_t n_segs, si
     p.x_stride = (uint32_t)io.x_stride;
     p.act_out = (uint8_t *)io.d_act_out;
     p.dump = dump;
+    uint32_t pro = io.pro ? io.pro->kind : 0u;
+    if (pro) {
+        p.pro_b = io.pro->d_b;
+        p.pro_out = io.pro->d_out;
+        p.pro_eps = io.pro->eps;
+        p.pro_add = io.pro->d_add;
+        p.pro_sum_out = io.pro->d_sum_out;
+        if (pro == OXH_PRO_RMSNORM && io.pro->d_add) pro = GEMV_PRO_ADD_RMSNORM;
+    }
 
     SegTable t;
     memset(&t, 0, sizeof t);
@@ -679,10 +703,24 @@ static int launch_gemv(uint32_t qtype, const OxhSegment *segs, size_t n_segs, si
         else if (all_one)    hipLaunchKernelGGL((KERNEL<1, false>), grid, block, lds, st, t, p, a); \
         else                 hipLaunchKernelGGL((KERNEL<0, false>), grid, block, lds, st, t, p, a); \
     } while (0)
-    if (is_q4k(qtype))          OXH_LAUNCH(k_gemv_q4_k);
-    else if (is_q5k(qtype))     OXH_LAUNCH(k_gemv_q5_k);
-    else if (qtype == OXH_Q6_K) OXH_LAUNCH(k_gemv_q6_k);
-    else                        OXH_LAUNCH(k_gemv_q8_0);
+#define OXH_LAUNCH_PRO(KERNEL, PRO)                                                     \
+    do {                                                                                \
+        if (all_one) hipLaunchKernelGGL((KERNEL<1, PRO>), grid, block, lds, st, t, p, a); \
+        else         hipLaunchKernelGGL((KERNEL<0, PRO>), grid, block, lds, st, t, p, a); \
+    } while (0)
+#define OXH_LAUNCH_ANY(PLAIN, WITH_PRO)                                                 \
+    do {                                                                                \
+        if (pro == GEMV_PRO_ADD_RMSNORM) OXH_LAUNCH_PRO(WITH_PRO, GEMV_PRO_ADD_RMSNORM); \
+        else if (pro == OXH_PRO_RMSNORM) OXH_LAUNCH_PRO(WITH_PRO, GEMV_PRO_RMSNORM);    \
+        else if (pro == OXH_PRO_SWIGLU) OXH_LAUNCH_PRO(WITH_PRO, GEMV_PRO_SWIGLU);      \
+        else                            OXH_LAUNCH(PLAIN);                              \
+    } while (0)
+    if (is_q4k(qtype))          OXH_LAUNCH_ANY(k_gemv_q4_k, k_gemv_q4_k_pro);
+    else if (is_q5k(qtype))     OXH_LAUNCH_ANY(k_gemv_q5_k, k_gemv_q5_k_pro);
+    else if (qtype == OXH_Q6_K) OXH_LAUNCH_ANY(k_gemv_q6_k, k_gemv_q6_k_pro);
+    else                        OXH_LAUNCH_ANY(k_gemv_q8_0, k_gemv_q8_0_pro);
+#undef OXH_LAUNCH_ANY
+#undef OXH_LAUNCH_PRO
 #undef OXH_LAUNCH
     HIP_TRY(hipGetLastError());
     return OXH_OK;
@@ -693,7 +731,7 @@ extern "C" int oxh_gemv_segments(uint32_t qtype, const OxhSegment *segs, size_t 
                                  size_t out_stride, void *stream)
 {
     if (!d_acts && n_segs) return arg_fail("oxh_gemv_segments: NULL activations");
-    const GemvIo io = { d_acts, nullptr, 0, nullptr };
+    const GemvIo io = { d_acts, nullptr, 0, nullptr, nullptr };
     return launch_gemv(qtype, segs, n_segs, cols, io, n_vec, out_stride, nullptr, stream);
 }
 
@@ -703,7 +741,50 @@ extern "C" int oxh_gemv_segments_f32(uint32_t qtype, const OxhSegment *segs, siz
                                      void *stream)
 {
     if (!d_x && n_segs) return arg_fail("oxh_gemv_segments_f32: NULL input");
-    const GemvIo io = { nullptr, d_x, x_stride, d_act_out };
+    const GemvIo io = { nullptr, d_x, x_stride, d_act_out, nullptr };
+    return launch_gemv(qtype, segs, n_segs, cols, io, n_vec, out_stride, nullptr, stream);
+}
+
+extern "C" int oxh_gemv_segments_fused(uint32_t qtype, const OxhSegment *segs, size_t n_segs,
+                                       size_t cols, const float *d_x, size_t x_stride,
+                                       const OxhPrologue *pro, void *d_act_out, size_t n_vec,
+                                       size_t out_stride, void *stream)
+{
+    if (!d_x && n_segs) return arg_fail("oxh_gemv_segments_fused: NULL input");
+    if (pro) {
+        if (pro->kind != OXH_PRO_RMSNORM && pro->kind != OXH_PRO_SWIGLU)
+            return arg_fail("oxh_gemv_segments_fused: unknown prologue kind");
+        if ((pro->d_add || pro->d_sum_out) && pro->kind != OXH_PRO_RMSNORM)
+            return arg_fail("oxh_gemv_segments_fused: d_add / d_sum_out go with OXH_PRO_RMSNORM");
+        if (pro->d_sum_out && !pro->d_add)
+            return arg_fail("oxh_gemv_segments_fused: d_sum_out without d_add");
+        if (!pro->d_b && n_segs) return arg_fail("oxh_gemv_segments_fused: prologue operand is NULL");
+        if (pro->kind == OXH_PRO_RMSNORM && !(pro->eps >= 0.0f))
+            return arg_fail("oxh_gemv_segments_fused: eps must be >= 0");
+        /* every workgroup reads all of x while the first one of each segment
+         * stores the result: the two must not overlap */
+        if ((pro->d_out || pro->d_sum_out) && n_segs) {
+            size_t max_act = 0;
+            for (size_t i = 0; i < n_segs; i++) {
+                const size_t nv = segs[i].n_vec ? segs[i].n_vec : n_vec;
+                if (segs[i].rows && segs[i].act_first + nv > max_act) max_act = segs[i].act_first + nv;
+            }
+            const size_t span = max_act ? ((max_act - 1) * x_stride + cols) * sizeof(float) : 0;
+            const size_t bspan = pro->kind == OXH_PRO_SWIGLU ? span : cols * sizeof(float);
+            const char *ins[3] = { (const char *)d_x, (const char *)pro->d_b, (const char *)pro->d_add };
+            const size_t in_span[3] = { span, bspan, span };
+            const char *outs[2] = { (const char *)pro->d_out, (const char *)pro->d_sum_out };
+            for (int o = 0; o < 2; o++) {
+                if (!outs[o]) continue;
+                for (int i = 0; i < 3; i++)
+                    if (ins[i] && outs[o] < ins[i] + in_span[i] && ins[i] < outs[o] + span)
+                        return arg_fail("oxh_gemv_segments_fused: a stored result overlaps an input");
+            }
+            if (outs[0] && outs[1] && outs[0] < outs[1] + span && outs[1] < outs[0] + span)
+                return arg_fail("oxh_gemv_segments_fused: the two stored results overlap");
+        }
+    }
+    const GemvIo io = { nullptr, d_x, x_stride, d_act_out, pro };
     return launch_gemv(qtype, segs, n_segs, cols, io, n_vec, out_stride, nullptr, stream);
 }
 
@@ -717,7 +798,7 @@ extern "C" int oxh_debug_subblock_sums(uint32_t qtype, const void *d_w, size_t r
     float *scratch = nullptr;
     HIP_TRY(hipMalloc((void **)&scratch, (rows ? rows : 1) * sizeof(float)));
     OxhSegment s = { d_w, scratch, rows, 0, 0 };
-    const GemvIo io = { d_act, nullptr, 0, nullptr };
+    const GemvIo io = { d_act, nullptr, 0, nullptr, nullptr };
     rc = launch_gemv(qtype, &s, 1, cols, io, 1, rows, d_sums, stream);
     hipError_t e = hipStreamSynchronize(pick_stream(stream));
     (void)hipFree(scratch);

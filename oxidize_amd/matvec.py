@@ -12,7 +12,7 @@ import ctypes
 import numpy as np
 
 from . import _lib
-from ._lib import DECLINED, OK, OxhError, OxhSegment, check, lib
+from ._lib import DECLINED, OK, OxhError, OxhPrologue, OxhSegment, check, lib
 
 Q8_0, Q4_K_S, Q4_K_M, Q5_K_S, Q5_K_M, Q6_K = 7, 12, 13, 14, 15, 16
 
@@ -149,6 +149,23 @@ def gemv_segments_f32(qtype, segs, cols, d_x, x_stride, d_act_out=None, n_vec=1,
     check(lib().oxh_gemv_segments_f32(qtype, segs, len(segs), cols, ctypes.c_void_p(d_x), x_stride,
                                       None if d_act_out is None else ctypes.c_void_p(d_act_out),
                                       n_vec, out_stride, stream))
+
+
+PRO_RMSNORM, PRO_SWIGLU = 1, 2
+
+
+def gemv_segments_fused(qtype, segs, cols, d_x, x_stride, kind, d_b, eps=0.0, d_pro_out=None,
+                        d_act_out=None, n_vec=1, out_stride=0, stream=None, d_add=None, d_sum_out=None):
+    """GEMV with RMSNorm (d_b = norm weight; optionally of x + d_add, the sum
+    stored to d_sum_out) or SwiGLU (d_x = gate, d_b = up) and the activation
+    quantisation fused into the kernel."""
+    def vp(a):
+        return None if a is None else ctypes.c_void_p(a)
+    pro = OxhPrologue(kind, eps, ctypes.c_void_p(d_b), vp(d_pro_out), vp(d_add), vp(d_sum_out))
+    check(lib().oxh_gemv_segments_fused(qtype, segs, len(segs), cols, ctypes.c_void_p(d_x), x_stride,
+                                        ctypes.byref(pro),
+                                        None if d_act_out is None else ctypes.c_void_p(d_act_out),
+                                        n_vec, out_stride, stream))
 
 
 def mmq(qtype, d_w, rows, cols, d_acts, n_vec, d_out, out_stride, stream=None):

@@ -6,6 +6,7 @@ committed, this script documents how they were made.
     python tests/golden/make_golden.py
 
     python tests/golden/make_golden.py q5_k     # only q5_k.npz
+    python tests/golden/make_golden.py float    # only float_steps.npz
 
 Every array is data: inputs and the reference's outputs for them.
 """
@@ -123,13 +124,39 @@ def q5_k(ref):
     np.savez_compressed(os.path.join(HERE, "q5_k.npz"), **out)
 
 
+def float_steps(ref):
+    """float_steps.npz: RMSNorm and SwiGLU as the compiled reference computes
+    them (oc_rms_norm_f32, oc_swiglu_inplace_f32)."""
+    out = {}
+    for n in (256, 896, 4096):
+        x = synth.normal(n, seed=11, stream=n) * np.float32(3.0)
+        w = (synth.normal(n, seed=12, stream=n) * np.float32(0.1) + np.float32(1.0)).astype(np.float32)
+        for eps in (1e-5, 1e-6):
+            o = np.zeros(n, np.float32)
+            ref.oc_rms_norm_f32(x.ctypes.data, w.ctypes.data, o.ctypes.data, n, eps)
+            out["rms_%d_%g_out" % (n, eps)] = o
+        out["rms_%d_x" % n], out["rms_%d_w" % n] = x, w
+    g = np.concatenate([synth.normal(4000, seed=13) * np.float32(4.0),
+                        np.array([0.0, -0.0, 1e-8, -1e-8, 20.0, -20.0, 87.9, -87.9, 100.0, -100.0,
+                                  1e4, -1e4], np.float32),
+                        np.linspace(-12, 12, 84, dtype=np.float32)]).astype(np.float32)
+    u = synth.normal(g.size, seed=14)
+    o = g.copy()
+    ref.oc_swiglu_inplace_f32(o.ctypes.data, u.ctypes.data, g.size)
+    out["swiglu_gate"], out["swiglu_up"], out["swiglu_out"] = g, u, o
+    np.savez_compressed(os.path.join(HERE, "float_steps.npz"), **out)
+
+
 def main():
     ref = oxlibs.ref()
     if ref is None:
         raise SystemExit("oracle/_ref/liboxref.so missing: run `make -C oracle` first")
     ref.oc_parallel_set_threads(1)
-    q5_k(ref)
-    if sys.argv[1:] == ["q5_k"]:
+    if sys.argv[1:] != ["float"]:
+        q5_k(ref)
+    if sys.argv[1:] != ["q5_k"]:
+        float_steps(ref)
+    if sys.argv[1:] in (["q5_k"], ["float"]):
         return
     rng = np.random.default_rng(20240607)
 

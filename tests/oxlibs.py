@@ -56,6 +56,8 @@ def oracle():
         lib.oxo_matvec_batch_scratch_bytes.restype = Z
         lib.oxo_moe_route.argtypes = [V, Z, Z, Z, ctypes.c_int, V, V]; lib.oxo_moe_route.restype = None
         lib.oxo_dequant_row.argtypes = [U32, V, Z, V]; lib.oxo_dequant_row.restype = ctypes.c_int
+        lib.oxo_rms_norm_f32.argtypes = [V, V, V, Z, F]; lib.oxo_rms_norm_f32.restype = None
+        lib.oxo_swiglu_f32.argtypes = [V, V, V, Z]; lib.oxo_swiglu_f32.restype = None
         _ORACLE = lib
     return _ORACLE
 
@@ -91,6 +93,9 @@ def ref():
         lib.oc_parallel_set_threads.argtypes = [Z]; lib.oc_parallel_set_threads.restype = ctypes.c_int
         lib.oc_parallel_n_threads.restype = Z
         lib.oc_quant_dequant_row.argtypes = [U32, V, Z, V, Z]; lib.oc_quant_dequant_row.restype = ctypes.c_int
+        if hasattr(lib, "oc_rms_norm_f32"):
+            lib.oc_rms_norm_f32.argtypes = [V, V, V, Z, F]; lib.oc_rms_norm_f32.restype = None
+            lib.oc_swiglu_inplace_f32.argtypes = [V, V, Z]; lib.oc_swiglu_inplace_f32.restype = None
         _REF = lib
     return _REF
 

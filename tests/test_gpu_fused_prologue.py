@@ -1,0 +1,199 @@
+"""GPU parity for the GEMV launches with a fused prologue (RMSNorm or SwiGLU in
+front of the activation quantiser), through the C ABI.
+
+Two bars, because the prologue is float arithmetic and everything after it is
+the integer path:
+  * the prologue's f32 result (stored on request) agrees with the oracle's
+    scalar restatement of the reference within FLOAT_RTOL relative -- the
+    reference's own SIMD variants differ from its scalar form by as much;
+  * given exactly those f32 values, the quantised activation bytes and the
+    outputs are bit-identical to the oracle's quantise + block dot, and to the
+    library's own launch without a prologue over the same values.
+"""
+import numpy as np
+import pytest
+
+import oxlibs
+from oxidize_amd import _lib
+from oxidize_amd import matvec as mv
+from oxidize_amd import synth
+
+pytestmark = pytest.mark.gpu
+
+Q80, Q4K, Q5K, Q6K = 7, 13, 15, 16
+FLOAT_RTOL = 4e-6
+
+
+def bits(a):
+    return np.ascontiguousarray(a).view(np.uint32)
+
+
+def oracle_matvec(qtype, w, rows, cols, x):
+    o = oxlibs.oracle()
+    out = np.zeros(rows, np.float32)
+    temp = np.zeros(cols, np.float32)
+    assert o.oxo_matvec_quantized(qtype, w.ctypes.data, rows, cols, synth.row_bytes(qtype, cols),
+                                  x.ctypes.data, out.ctypes.data, temp.ctypes.data) == 0
+    return out, temp
+
+
+def run_fused(qtype, w, rows, cols, xs, kind, b, eps=0.0):
+    """-> (prologue f32 result, activation bytes, outputs), all from the device."""
+    n_vec = xs.shape[0]
+    d_w = mv.DeviceBuffer.from_host(w)
+    d_x = mv.DeviceBuffer.from_host(xs)
+    d_b = mv.DeviceBuffer.from_host(b)
+    nact = mv.act_bytes(qtype, cols)
+    d_y = mv.DeviceBuffer(n_vec * cols * 4)
+    d_a = mv.DeviceBuffer(n_vec * nact)
+    d_o = mv.DeviceBuffer(n_vec * rows * 4)
+    segs = mv.make_segments([(d_w.ptr, d_o.ptr, rows, 0)])
+    mv.gemv_segments_fused(qtype, segs, cols, d_x.ptr, cols, kind, d_b.ptr, eps, d_y.ptr, d_a.ptr,
+                           n_vec, rows)
+    y = d_y.download(np.float32, n_vec * cols).reshape(n_vec, cols)
+    acts = d_a.download(np.uint8, n_vec * nact).reshape(n_vec, nact)
+    out = d_o.download(np.float32, n_vec * rows).reshape(n_vec, rows)
+    # the same values through the launch without a prologue
+    d_o2 = mv.DeviceBuffer(n_vec * rows * 4)
+    segs2 = mv.make_segments([(d_w.ptr, d_o2.ptr, rows, 0)])
+    mv.gemv_segments_f32(qtype, segs2, cols, d_y.ptr, cols, None, n_vec, rows)
+    out2 = d_o2.download(np.float32, n_vec * rows).reshape(n_vec, rows)
+    assert np.array_equal(bits(out), bits(out2))
+    return y, acts, out
+
+
+def check_integer_path(qtype, w, rows, cols, y, acts, out):
+    nact = acts.shape[1]
+    for v in range(y.shape[0]):
+        want, wtemp = oracle_matvec(qtype, w, rows, cols, np.ascontiguousarray(y[v]))
+        assert np.array_equal(acts[v], wtemp.view(np.uint8)[:nact]), "activation bytes, vector %d" % v
+        assert np.array_equal(bits(out[v]), bits(want)), "outputs, vector %d" % v
+
+
+CASES = [
+    (Q4K, 300, 256, 1), (Q4K, 4096, 4096, 1), (Q4K, 700, 14336, 1), (Q4K, 64, 18432, 1),
+    (Q4K, 200, 4096, 3), (Q4K, 64, 18432, 2), (Q5K, 333, 4096, 1), (Q5K, 100, 2048, 8),
+    (Q6K, 4096, 14336, 1), (Q6K, 50, 512, 5), (Q80, 1000, 896, 1), (Q80, 300, 4864, 1),
+    (Q80, 90, 96, 4), (Q80, 5, 32, 1),
+]
+
+
+@pytest.mark.parametrize("qtype,rows,cols,n_vec", CASES)
+def test_rmsnorm_prologue(oxh, qtype, rows, cols, n_vec):
+    w = synth.weights(qtype, rows, cols, seed=3, stream=rows)
+    xs = (synth.normal(n_vec * cols, seed=3, stream=cols) * np.float32(2.5)).reshape(n_vec, cols)
+    if n_vec > 1:
+        xs[1] *= np.float32(1e-3)
+    gamma = (synth.normal(cols, seed=4, stream=cols) * np.float32(0.2) + np.float32(1.0)).astype(np.float32)
+    eps = 1e-5
+    y, acts, out = run_fused(qtype, w, rows, cols, xs, mv.PRO_RMSNORM, gamma, eps)
+    o = oxlibs.oracle()
+    for v in range(n_vec):
+        want = np.zeros(cols, np.float32)
+        o.oxo_rms_norm_f32(xs[v].ctypes.data, gamma.ctypes.data, want.ctypes.data, cols, eps)
+        assert np.all(np.abs(y[v] - want) <= FLOAT_RTOL * np.abs(want)), "vector %d" % v
+        xd = xs[v].astype(np.float64)
+        exact = xd / np.sqrt((xd * xd).mean() + eps) * gamma
+        assert np.all(np.abs(y[v] - exact) <= FLOAT_RTOL * np.abs(exact))
+    check_integer_path(qtype, w, rows, cols, y, acts, out)
+
+
+@pytest.mark.parametrize("qtype,rows,cols,n_vec", CASES)
+def test_swiglu_prologue(oxh, qtype, rows, cols, n_vec):
+    w = synth.weights(qtype, rows, cols, seed=5, stream=rows)
+    gate = (synth.normal(n_vec * cols, seed=5, stream=cols) * np.float32(3.0)).reshape(n_vec, cols)
+    up = synth.normal(n_vec * cols, seed=6, stream=cols).reshape(n_vec, cols)
+    gate[0, :8] = np.array([0.0, -0.0, 30.0, -30.0, 88.5, -88.5, 1e-9, -100.0], np.float32)[:min(8, cols)]
+    y, acts, out = run_fused(qtype, w, rows, cols, gate, mv.PRO_SWIGLU, up)
+    o = oxlibs.oracle()
+    for v in range(n_vec):
+        want = np.zeros(cols, np.float32)
+        o.oxo_swiglu_f32(gate[v].ctypes.data, up[v].ctypes.data, want.ctypes.data, cols)
+        assert np.all(np.abs(y[v] - want) <= FLOAT_RTOL * np.abs(want) + 1e-30), "vector %d" % v
+    check_integer_path(qtype, w, rows, cols, y, acts, out)
+
+
+@pytest.mark.parametrize("qtype,rows,cols,n_vec", [(Q4K, 4096, 4096, 1), (Q4K, 64, 18432, 2), (Q6K, 50, 512, 5),
+                                                  (Q5K, 333, 4096, 1), (Q80, 300, 4864, 1), (Q80, 90, 96, 4)])
+def test_residual_add_rmsnorm_prologue(oxh, qtype, rows, cols, n_vec):
+    """x + add is stored bit-exactly (one f32 addition per element), normalised
+    like the oracle normalises that sum, and quantised / multiplied exactly."""
+    w = synth.weights(qtype, rows, cols, seed=13, stream=rows)
+    xs = (synth.normal(n_vec * cols, seed=13, stream=cols) * np.float32(2.0)).reshape(n_vec, cols)
+    add = synth.normal(n_vec * cols, seed=14, stream=cols).reshape(n_vec, cols)
+    gamma = (synth.normal(cols, seed=15, stream=cols) * np.float32(0.2) + np.float32(1.0)).astype(np.float32)
+    eps = 1e-5
+    d_w = mv.DeviceBuffer.from_host(w)
+    d_x, d_add, d_g = (mv.DeviceBuffer.from_host(a) for a in (xs, add, gamma))
+    nact = mv.act_bytes(qtype, cols)
+    d_y, d_s = mv.DeviceBuffer(n_vec * cols * 4), mv.DeviceBuffer(n_vec * cols * 4)
+    d_a, d_o = mv.DeviceBuffer(n_vec * nact), mv.DeviceBuffer(n_vec * rows * 4)
+    segs = mv.make_segments([(d_w.ptr, d_o.ptr, rows, 0)])
+    mv.gemv_segments_fused(qtype, segs, cols, d_x.ptr, cols, mv.PRO_RMSNORM, d_g.ptr, eps, d_y.ptr, d_a.ptr,
+                           n_vec, rows, d_add=d_add.ptr, d_sum_out=d_s.ptr)
+    total = d_s.download(np.float32, n_vec * cols).reshape(n_vec, cols)
+    assert np.array_equal(bits(total), bits(xs + add))
+    y = d_y.download(np.float32, n_vec * cols).reshape(n_vec, cols)
+    o = oxlibs.oracle()
+    for v in range(n_vec):
+        want = np.zeros(cols, np.float32)
+        o.oxo_rms_norm_f32(total[v].ctypes.data, gamma.ctypes.data, want.ctypes.data, cols, eps)
+        assert np.all(np.abs(y[v] - want) <= FLOAT_RTOL * np.abs(want)), "vector %d" % v
+    acts = d_a.download(np.uint8, n_vec * nact).reshape(n_vec, nact)
+    out = d_o.download(np.float32, n_vec * rows).reshape(n_vec, rows)
+    check_integer_path(qtype, w, rows, cols, y, acts, out)
+
+
+def test_rmsnorm_prologue_with_several_segments(oxh):
+    """q, k and v share one normalised input (one launch); and a launch whose
+    segments each take their own vector (the multi-input form)."""
+    cols, rows = 4096, [4096, 1024, 1024]
+    ws = [synth.weights(Q4K, r, cols, seed=7, stream=i) for i, r in enumerate(rows)]
+    xs = synth.normal(3 * cols, seed=7, stream=50).reshape(3, cols)
+    gamma = (synth.normal(cols, seed=8) * np.float32(0.1) + np.float32(1.0)).astype(np.float32)
+    d_ws = [mv.DeviceBuffer.from_host(w) for w in ws]
+    d_os = [mv.DeviceBuffer(r * 4) for r in rows]
+    d_x = mv.DeviceBuffer.from_host(xs)
+    d_g = mv.DeviceBuffer.from_host(gamma)
+    d_y = mv.DeviceBuffer(3 * cols * 4)
+    for shared in (True, False):
+        segs = mv.make_segments([(d_ws[i].ptr, d_os[i].ptr, rows[i], 0 if shared else i) for i in range(3)])
+        d_y.upload(np.zeros(3 * cols, np.float32))
+        mv.gemv_segments_fused(Q4K, segs, cols, d_x.ptr, cols, mv.PRO_RMSNORM, d_g.ptr, 1e-6, d_y.ptr,
+                               None, 1, 0)
+        y = d_y.download(np.float32, 3 * cols).reshape(3, cols)
+        for i in range(3):
+            v = 0 if shared else i
+            want, _ = oracle_matvec(Q4K, ws[i], rows[i], cols, np.ascontiguousarray(y[v]))
+            assert np.array_equal(bits(d_os[i].download(np.float32, rows[i])), bits(want))
+        if shared:
+            assert np.all(y[1:] == 0.0)
+
+
+def test_fused_prologue_argument_checks(oxh):
+    cols, rows = 512, 16
+    w = synth.weights(Q4K, rows, cols, seed=9)
+    d_w = mv.DeviceBuffer.from_host(w)
+    d_x = mv.DeviceBuffer.from_host(synth.normal(cols, seed=9))
+    d_b = mv.DeviceBuffer.from_host(np.ones(cols, np.float32))
+    d_o = mv.DeviceBuffer(rows * 4)
+    segs = mv.make_segments([(d_w.ptr, d_o.ptr, rows, 0)])
+    for bad in (lambda: mv.gemv_segments_fused(Q4K, segs, cols, d_x.ptr, cols, 7, d_b.ptr),
+                lambda: mv.gemv_segments_fused(Q4K, segs, cols, d_x.ptr, cols, mv.PRO_RMSNORM, 0),
+                lambda: mv.gemv_segments_fused(Q4K, segs, cols, d_x.ptr, cols, mv.PRO_RMSNORM, d_b.ptr,
+                                               -1.0),
+                # the stored result may not overlap an input
+                lambda: mv.gemv_segments_fused(Q4K, segs, cols, d_x.ptr, cols, mv.PRO_RMSNORM, d_b.ptr,
+                                               1e-5, d_x.ptr + 64),
+                lambda: mv.gemv_segments_fused(Q4K, segs, cols, d_x.ptr, cols, mv.PRO_SWIGLU, d_b.ptr,
+                                               0.0, d_b.ptr),
+                # the residual form belongs to RMSNorm, and a stored sum needs something added
+                lambda: mv.gemv_segments_fused(Q4K, segs, cols, d_x.ptr, cols, mv.PRO_SWIGLU, d_b.ptr,
+                                               d_add=d_b.ptr),
+                lambda: mv.gemv_segments_fused(Q4K, segs, cols, d_x.ptr, cols, mv.PRO_RMSNORM, d_b.ptr,
+                                               1e-5, d_sum_out=d_o.ptr),
+                lambda: mv.gemv_segments_fused(Q4K, segs, cols, d_x.ptr, cols, mv.PRO_RMSNORM, d_b.ptr,
+                                               1e-5, d_add=d_b.ptr, d_sum_out=d_x.ptr)):
+        with pytest.raises(_lib.OxhError) as e:
+            bad()
+        assert e.value.status == _lib.ERR_ARG

@@ -424,6 +424,56 @@ def test_full_size_configs_vs_reference_checksums(name, qt, rows, cols):
         assert zlib.crc32(out.tobytes()) == int(g[name + "_crc_out"][0])
 
 
+# ─── float steps in front of the quantiser ──────────────────────────────
+
+FLOAT_RTOL = 4e-6      # scalar, SIMD-lane and tree summation orders differ by rounding only
+
+
+def test_rms_norm_vs_reference_goldens_and_double_precision():
+    g = load("float_steps.npz")
+    for n in (256, 896, 4096):
+        x, w = g["rms_%d_x" % n], g["rms_%d_w" % n]
+        for eps in (1e-5, 1e-6):
+            out = np.zeros(n, np.float32)
+            O.oxo_rms_norm_f32(x.ctypes.data, w.ctypes.data, out.ctypes.data, n, eps)
+            want = g["rms_%d_%g_out" % (n, eps)]
+            assert np.all(np.abs(out - want) <= FLOAT_RTOL * np.abs(want))
+            xd = x.astype(np.float64)
+            exact = xd / np.sqrt((xd * xd).mean() + eps) * w
+            assert np.all(np.abs(out - exact) <= FLOAT_RTOL * np.abs(exact))
+    # closed form: a constant vector c with unit weights normalises to c/sqrt(c^2 + eps)
+    x = np.full(512, 3.0, np.float32)
+    out = np.zeros(512, np.float32)
+    ones = np.ones(512, np.float32)
+    O.oxo_rms_norm_f32(x.ctypes.data, ones.ctypes.data, out.ctypes.data, 512, 0.0)
+    assert np.all(out == 1.0)
+    # the weight multiplies element-wise and the sign of x survives
+    w = np.arange(512, dtype=np.float32)
+    x[::2] = -3.0
+    O.oxo_rms_norm_f32(x.ctypes.data, w.ctypes.data, out.ctypes.data, 512, 0.0)
+    assert np.array_equal(out, np.where(np.arange(512) % 2 == 0, -w, w))
+
+
+def test_swiglu_vs_reference_goldens_and_double_precision():
+    g = load("float_steps.npz")
+    gate, up, want = g["swiglu_gate"], g["swiglu_up"], g["swiglu_out"]
+    out = np.zeros(gate.size, np.float32)
+    O.oxo_swiglu_f32(gate.ctypes.data, up.ctypes.data, out.ctypes.data, gate.size)
+    # the reference's x86 exp clamps its argument at +-88: beyond that silu(g) is
+    # 0 or g to more digits than f32 holds, but a denormal-range product may differ
+    assert np.all(np.abs(out - want) <= FLOAT_RTOL * np.abs(want) + 1e-30)
+    gd = gate.astype(np.float64)
+    with np.errstate(over="ignore"):
+        exact = gd / (1.0 + np.exp(-gd)) * up
+    assert np.all(np.abs(out - exact) <= FLOAT_RTOL * np.abs(exact) + 1e-30)
+    z, ones = np.zeros(4, np.float32), np.ones(4, np.float32)
+    O.oxo_swiglu_f32(z.ctypes.data, ones.ctypes.data, out.ctypes.data, 4)
+    assert np.all(out[:4] == 0.0)
+    big, two = np.array([50.0, -50.0], np.float32), np.array([2.0, 2.0], np.float32)
+    O.oxo_swiglu_f32(big.ctypes.data, two.ctypes.data, out.ctypes.data, 2)
+    assert out[0] == 100.0 and abs(out[1]) < 1e-18
+
+
 def test_eligibility_rules():
     # oxidize-c/src/compute/matvec.c:99-127, :961-985
     assert O.oxo_act_kind(Q4K, 4096) == 2 and O.oxo_act_kind(Q4K, 896) == 0
