@@ -96,7 +96,17 @@ typedef struct OxhSegment {
     size_t      rows;
     size_t      act_first;/* index of this segment's first activation in d_acts */
     size_t      n_vec;    /* activations of this segment (1..8); 0 = the launch's n_vec */
+    const void *d_w_pair; /* NULL, or a second matrix of the same type and shape: the
+                             segment then writes silu(dot(W[r], a)) * dot(W_pair[r], a) */
 } OxhSegment;
+
+/* A segment with d_w_pair set computes the gate and up projections of a
+ * SwiGLU feed-forward block in one pass and writes only their combination
+ * h[r] = silu(gate[r]) * up[r] (f32, the expression of
+ * oxidize-c/src/compute/activation.c:92-99 / k_f_swiglu,
+ * oxidize-c/src/backends/cuda_fast.cu:477-485): every wave walks its rows of
+ * both matrices, so no gate / up vector ever reaches memory.  Paired
+ * launches always use the dot-instruction kernels (n_vec <= 8). */
 
 /* Decode GEMV over pre-quantised activations:
  *   out[v][r] = dot(W[r], act[act_first + v])   for v < n_vec (1..8)

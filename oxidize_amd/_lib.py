@@ -19,7 +19,8 @@ I = ctypes.c_int
 
 
 class OxhSegment(ctypes.Structure):
-    _fields_ = [("d_w", V), ("d_out", V), ("rows", Z), ("act_first", Z), ("n_vec", Z)]
+    _fields_ = [("d_w", V), ("d_out", V), ("rows", Z), ("act_first", Z), ("n_vec", Z),
+                ("d_w_pair", V)]
 
 
 class OxhPrologue(ctypes.Structure):

@@ -311,7 +311,7 @@ int oxh_matvec_quantized(uint32_t qtype, const uint8_t *data, size_t rows,
     memcpy(g_hin.p, input, cols * sizeof(float));
     if ((rc = oxh_memcpy_h2d(g_dx.p, g_hin.p, cols * sizeof(float), NULL))) return rc;
     /* one launch: quantise the activation inside the GEMV kernel */
-    OxhSegment seg = { d_w, (float *)g_dout.p, rows, 0, 0 };
+    OxhSegment seg = { d_w, (float *)g_dout.p, rows, 0, 0, NULL };
     if ((rc = oxh_gemv_segments_f32(qtype, &seg, 1, cols, (const float *)g_dx.p, cols,
                                     (uint8_t *)g_dout.p + act_off, 1, rows, NULL)))
         return rc;
@@ -373,6 +373,7 @@ static int grouped(uint32_t qtype, const uint8_t *const *datas,
             segs[i].rows = rows[k];
             segs[i].act_first = n_inputs == 1 ? 0 : k;
             segs[i].n_vec = 0;
+            segs[i].d_w_pair = NULL;
             done_rows += rows[k];
         }
         if ((rc = oxh_gemv_segments_f32(qtype, segs, n, cols, (const float *)g_dx.p, cols, NULL, 1, 0,
@@ -523,7 +524,7 @@ int oxh_matvec_quantized_batch(uint32_t qtype, const uint8_t *data, size_t rows,
         }
         for (size_t v0 = 0; v0 < n_vec; v0 += step) {
             const size_t m = n_vec - v0 < step ? n_vec - v0 : step;
-            OxhSegment seg = { d_w, (float *)g_dout.p + v0 * rows, rows, v0, 0 };
+            OxhSegment seg = { d_w, (float *)g_dout.p + v0 * rows, rows, v0, 0, NULL };
             if ((rc = oxh_gemv_segments_f32(qtype, &seg, 1, cols, (const float *)g_dx.p, in_stride,
                                             NULL, m, rows, NULL)))
                 return rc;

@@ -422,18 +422,22 @@ static hipError_t raise_all_lds_ceilings(void)
     OXH_RAISE(k_gemv_q6_k)
     OXH_RAISE(k_gemv_q8_0)
 #undef OXH_RAISE
+#define OXH_RAISE_PRO1(KERNEL, PRO)                                                               \
+    if ((e = raise_lds_ceiling(KERNEL<1, PRO, false>)) != hipSuccess) return e;                   \
+    if ((e = raise_lds_ceiling(KERNEL<0, PRO, false>)) != hipSuccess) return e;                   \
+    if ((e = raise_lds_ceiling(KERNEL<1, PRO, true>)) != hipSuccess) return e;                    \
+    if ((e = raise_lds_ceiling(KERNEL<0, PRO, true>)) != hipSuccess) return e;
 #define OXH_RAISE_PRO(KERNEL)                                                                     \
-    if ((e = raise_lds_ceiling(KERNEL<1, GEMV_PRO_RMSNORM>)) != hipSuccess) return e;             \
-    if ((e = raise_lds_ceiling(KERNEL<0, GEMV_PRO_RMSNORM>)) != hipSuccess) return e;             \
-    if ((e = raise_lds_ceiling(KERNEL<1, GEMV_PRO_SWIGLU>)) != hipSuccess) return e;              \
-    if ((e = raise_lds_ceiling(KERNEL<0, GEMV_PRO_SWIGLU>)) != hipSuccess) return e;              \
-    if ((e = raise_lds_ceiling(KERNEL<1, GEMV_PRO_ADD_RMSNORM>)) != hipSuccess) return e;         \
-    if ((e = raise_lds_ceiling(KERNEL<0, GEMV_PRO_ADD_RMSNORM>)) != hipSuccess) return e;
+    OXH_RAISE_PRO1(KERNEL, GEMV_PRO_NONE)                                                         \
+    OXH_RAISE_PRO1(KERNEL, GEMV_PRO_RMSNORM)                                                      \
+    OXH_RAISE_PRO1(KERNEL, GEMV_PRO_SWIGLU)                                                       \
+    OXH_RAISE_PRO1(KERNEL, GEMV_PRO_ADD_RMSNORM)
     OXH_RAISE_PRO(k_gemv_q4_k_pro)
     OXH_RAISE_PRO(k_gemv_q5_k_pro)
     OXH_RAISE_PRO(k_gemv_q6_k_pro)
     OXH_RAISE_PRO(k_gemv_q8_0_pro)
 #undef OXH_RAISE_PRO
+#undef OXH_RAISE_PRO1
     if ((e = raise_lds_ceiling(k_mmq_q4_k<8, 2, 8>)) != hipSuccess) return e;
     if ((e = raise_lds_ceiling(k_mmq_q4_k<4, 1, 8>)) != hipSuccess) return e;
     if ((e = raise_lds_ceiling(k_mmq_q5_k<8, 1, 8>)) != hipSuccess) return e;
@@ -555,6 +559,7 @@ static int launch_mmq_segments(uint32_t qtype, const OxhSegment *segs, size_t n_
         n++;
     }
     t.n = n;
+    for (uint32_t i = 1; i < 4 && i < n; i++) t.bound[i - 1] = t.s[i].wg_begin;
     if (qtype == OXH_Q6_K) {
         typedef Mmq6Geom<1, 1, 4> G6;                       /* same 64-row tiles */
         static_assert(G6::ROWS == G::ROWS, "segment tiling is shared by both formats");
@@ -601,21 +606,26 @@ static int launch_gemv(uint32_t qtype, const OxhSegment *segs, size_t n_segs, si
     size_t total_rows = 0, max_act = 0;
     /* a segment may carry its own activation count; the launch value is the default */
     size_t max_nv = 0;
-    bool all_one = true;
+    bool all_one = true, any_pair = false;
+    /* a paired segment walks two matrices: it counts twice wherever work is sized */
+    size_t total_work = 0;
     for (size_t i = 0; i < n_segs; i++) {
         const size_t nv = segs[i].n_vec ? segs[i].n_vec : n_vec;
         if (nv < 1 || nv > OXH_MAX_NV) return arg_fail("gemv: segment n_vec must be 1..8");
         if (segs[i].rows) {
             if (nv > max_nv) max_nv = nv;
             if (nv != 1) all_one = false;
+            if (segs[i].d_w_pair) any_pair = true;
         }
-        if (segs[i].rows > 0x7FFFFFFFull / (blocks * 16u)) return arg_fail("gemv: segment too large");
+        if (segs[i].rows > 0x3FFFFFFFull / (blocks * 16u)) return arg_fail("gemv: segment too large");
         if (segs[i].rows && (!segs[i].d_w || !segs[i].d_out)) return arg_fail("gemv: NULL segment pointer");
         total_rows += segs[i].rows;
+        total_work += segs[i].rows * (segs[i].d_w_pair ? 2u : 1u);
         if (segs[i].act_first > max_act) max_act = segs[i].act_first;
     }
     if (total_rows == 0) return OXH_OK;
-    if (gemv_wants_mfma(qtype, io, max_nv, dump))
+    if (any_pair && dump) return arg_fail("gemv: no sub-block dump of a paired launch");
+    if (!any_pair && gemv_wants_mfma(qtype, io, max_nv, dump))
         return launch_mmq_segments(qtype, segs, n_segs, cols, blocks, io, n_vec_default, max_act + max_nv,
                                    out_stride, stream);
     n_vec = max_nv;                        /* sizes LDS from here on */
@@ -627,7 +637,7 @@ static int launch_gemv(uint32_t qtype, const OxhSegment *segs, size_t n_segs, si
     uint32_t W = gemv_waves();
     const size_t blocks_per_pass = qtype == OXH_Q8_0 ? 64u : 16u;
     const size_t target = (size_t)(g_n_cu > 0 ? g_n_cu : 256) *
-                          gemv_wg_per_cu(total_rows * blocks / blocks_per_pass, W);
+                          gemv_wg_per_cu(total_work * blocks / blocks_per_pass, W);
     uint32_t cap_limit = GEMV_ROWS_CAP;
     uint32_t n_wg[OXH_MAX_SEGS];
     uint32_t rows_cap = 1;
@@ -636,14 +646,16 @@ static int launch_gemv(uint32_t qtype, const OxhSegment *segs, size_t n_segs, si
         for (size_t i = 0; i < n_segs; i++) {
             const size_t rows = segs[i].rows;
             if (rows == 0) { n_wg[i] = 0; continue; }
-            size_t share = (target * rows + total_rows / 2) / total_rows;
-            const size_t lo = (rows + (size_t)W * cap_limit - 1) / ((size_t)W * cap_limit);
+            const size_t mult = segs[i].d_w_pair ? 2u : 1u;     /* table rows per owned row */
+            size_t share = (target * rows * mult + total_work / 2) / total_work;
+            const size_t own_limit = cap_limit / mult ? cap_limit / mult : 1u;
+            const size_t lo = (rows + (size_t)W * own_limit - 1) / ((size_t)W * own_limit);
             const size_t hi = (rows + W - 1) / W;
             if (share < lo) share = lo;
             if (share > hi) share = hi;
             if (share < 1) share = 1;
             n_wg[i] = (uint32_t)share;
-            const uint32_t rpw = (uint32_t)((rows + share * W - 1) / (share * W));   /* q + (rem != 0) */
+            const uint32_t rpw = (uint32_t)((rows + share * W - 1) / (share * W) * mult);   /* (q + (rem != 0)) * mult */
             if (rpw > rows_cap) rows_cap = rpw;
         }
         if (gemv_lds_bytes(qtype, (uint32_t)blocks, n_vec, W, rows_cap) <= GEMV_LDS_LIMIT) break;
@@ -678,10 +690,13 @@ static int launch_gemv(uint32_t qtype, const OxhSegment *segs, size_t n_segs, si
 
     SegTable t;
     memset(&t, 0, sizeof t);
+    PairTable pairs;
+    memset(&pairs, 0, sizeof pairs);
     uint32_t wg = 0, n = 0;
     for (size_t i = 0; i < n_segs; i++) {
         if (segs[i].rows == 0) continue;
         t.s[n].w = (const uint8_t *)segs[i].d_w;
+        pairs.w2[n] = (const uint8_t *)segs[i].d_w_pair;
         t.s[n].out = segs[i].d_out;
         t.s[n].rows = (uint32_t)segs[i].rows;
         t.s[n].act_first = (uint32_t)segs[i].act_first;
@@ -693,6 +708,7 @@ static int launch_gemv(uint32_t qtype, const OxhSegment *segs, size_t n_segs, si
         n++;
     }
     t.n = n;
+    for (uint32_t i = 1; i < 4 && i < n; i++) t.bound[i - 1] = t.s[i].wg_begin;
 
     const dim3 grid(wg), block(W * 64u);
     hipStream_t st = pick_stream(stream);
@@ -705,14 +721,20 @@ static int launch_gemv(uint32_t qtype, const OxhSegment *segs, size_t n_segs, si
     } while (0)
 #define OXH_LAUNCH_PRO(KERNEL, PRO)                                                     \
     do {                                                                                \
-        if (all_one) hipLaunchKernelGGL((KERNEL<1, PRO>), grid, block, lds, st, t, p, a); \
-        else         hipLaunchKernelGGL((KERNEL<0, PRO>), grid, block, lds, st, t, p, a); \
+        if (any_pair) {                                                                 \
+            if (all_one) hipLaunchKernelGGL((KERNEL<1, PRO, true>), grid, block, lds, st, t, p, a, pairs);  \
+            else         hipLaunchKernelGGL((KERNEL<0, PRO, true>), grid, block, lds, st, t, p, a, pairs);  \
+        } else {                                                                        \
+            if (all_one) hipLaunchKernelGGL((KERNEL<1, PRO, false>), grid, block, lds, st, t, p, a, pairs); \
+            else         hipLaunchKernelGGL((KERNEL<0, PRO, false>), grid, block, lds, st, t, p, a, pairs); \
+        }                                                                               \
     } while (0)
 #define OXH_LAUNCH_ANY(PLAIN, WITH_PRO)                                                 \
     do {                                                                                \
         if (pro == GEMV_PRO_ADD_RMSNORM) OXH_LAUNCH_PRO(WITH_PRO, GEMV_PRO_ADD_RMSNORM); \
         else if (pro == OXH_PRO_RMSNORM) OXH_LAUNCH_PRO(WITH_PRO, GEMV_PRO_RMSNORM);    \
         else if (pro == OXH_PRO_SWIGLU) OXH_LAUNCH_PRO(WITH_PRO, GEMV_PRO_SWIGLU);      \
+        else if (any_pair)              OXH_LAUNCH_PRO(WITH_PRO, GEMV_PRO_NONE);        \
         else                            OXH_LAUNCH(PLAIN);                              \
     } while (0)
     if (is_q4k(qtype))          OXH_LAUNCH_ANY(k_gemv_q4_k, k_gemv_q4_k_pro);
@@ -797,7 +819,7 @@ extern "C" int oxh_debug_subblock_sums(uint32_t qtype, const void *d_w, size_t r
     if (rc) return rc;
     float *scratch = nullptr;
     HIP_TRY(hipMalloc((void **)&scratch, (rows ? rows : 1) * sizeof(float)));
-    OxhSegment s = { d_w, scratch, rows, 0, 0 };
+    OxhSegment s = { d_w, scratch, rows, 0, 0, nullptr };
     const GemvIo io = { d_act, nullptr, 0, nullptr, nullptr };
     rc = launch_gemv(qtype, &s, 1, cols, io, 1, rows, d_sums, stream);
     hipError_t e = hipStreamSynchronize(pick_stream(stream));

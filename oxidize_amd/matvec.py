@@ -128,13 +128,15 @@ def quantize(qtype, d_x, in_stride, n_vec, cols, d_act, stream=None):
 
 
 def make_segments(items):
-    """items: iterable of (d_w, d_out, rows, act_first[, n_vec]) with integer
-    addresses; n_vec 0/omitted = the launch's n_vec."""
+    """items: iterable of (d_w, d_out, rows, act_first[, n_vec[, d_w_pair]]) with
+    integer addresses; n_vec 0/omitted = the launch's n_vec; d_w_pair = the second
+    matrix of a gate/up pair (the segment then writes silu(gate) * up)."""
     items = list(items)
     segs = (OxhSegment * len(items))()
     for s, it in zip(segs, items):
         s.d_w, s.d_out, s.rows, s.act_first = it[0], it[1], it[2], it[3]
         s.n_vec = it[4] if len(it) > 4 else 0
+        s.d_w_pair = it[5] if len(it) > 5 else None
     return segs
 
 

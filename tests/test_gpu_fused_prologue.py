@@ -197,3 +197,80 @@ def test_fused_prologue_argument_checks(oxh):
         with pytest.raises(_lib.OxhError) as e:
             bad()
         assert e.value.status == _lib.ERR_ARG
+
+
+# ─── paired gate / up matrices: h = silu(W_gate x) * (W_up x) in one pass ───
+
+def paired_case(qtype, rows, cols, n_vec, seed):
+    wg = synth.weights(qtype, rows, cols, seed=seed, stream=1)
+    wu = synth.weights(qtype, rows, cols, seed=seed, stream=2)
+    xs = synth.normal(n_vec * cols, seed=seed, stream=3).reshape(n_vec, cols)
+    return wg, wu, xs
+
+
+def check_paired(qtype, wg, wu, rows, cols, x_used, h):
+    """h against the oracle: gate and up exactly, their combination to rounding."""
+    o = oxlibs.oracle()
+    for v in range(x_used.shape[0]):
+        gate, _ = oracle_matvec(qtype, wg, rows, cols, np.ascontiguousarray(x_used[v]))
+        up, _ = oracle_matvec(qtype, wu, rows, cols, np.ascontiguousarray(x_used[v]))
+        want = np.zeros(rows, np.float32)
+        o.oxo_swiglu_f32(gate.ctypes.data, up.ctypes.data, want.ctypes.data, rows)
+        assert np.all(np.abs(h[v] - want) <= FLOAT_RTOL * np.abs(want) + 1e-30), "vector %d" % v
+
+
+@pytest.mark.parametrize("qtype,rows,cols,n_vec", [
+    (Q4K, 14336, 4096, 1), (Q4K, 77, 512, 1), (Q4K, 1000, 1024, 3), (Q4K, 140000, 256, 1),
+    (Q5K, 700, 2048, 1), (Q6K, 2000, 1024, 2), (Q80, 4864, 896, 1), (Q80, 100, 64, 8),
+])
+def test_paired_gate_up_swiglu(oxh, qtype, rows, cols, n_vec):
+    wg, wu, xs = paired_case(qtype, rows, cols, n_vec, seed=21)
+    d_g, d_u, d_x = (mv.DeviceBuffer.from_host(a) for a in (wg, wu, xs))
+    d_h = mv.DeviceBuffer(n_vec * rows * 4)
+    segs = mv.make_segments([(d_g.ptr, d_h.ptr, rows, 0, 0, d_u.ptr)])
+    mv.gemv_segments_f32(qtype, segs, cols, d_x.ptr, cols, None, n_vec, rows)
+    h = d_h.download(np.float32, n_vec * rows).reshape(n_vec, rows)
+    check_paired(qtype, wg, wu, rows, cols, xs, h)
+    # the same from the library's own separate launches: identical gate and up bits go in
+    d_go, d_uo = mv.DeviceBuffer(n_vec * rows * 4), mv.DeviceBuffer(n_vec * rows * 4)
+    for d_w, d_o in ((d_g, d_go), (d_u, d_uo)):
+        mv.gemv_segments_f32(qtype, mv.make_segments([(d_w.ptr, d_o.ptr, rows, 0)]), cols, d_x.ptr, cols,
+                             None, n_vec, rows)
+    gate = d_go.download(np.float32, n_vec * rows)
+    up = d_uo.download(np.float32, n_vec * rows)
+    want = np.zeros(n_vec * rows, np.float32)
+    oxlibs.oracle().oxo_swiglu_f32(gate.ctypes.data, up.ctypes.data, want.ctypes.data, want.size)
+    assert np.all(np.abs(h.ravel() - want) <= FLOAT_RTOL * np.abs(want) + 1e-30)
+    # pre-quantised activations take the same path
+    nact = mv.act_bytes(qtype, cols)
+    d_a = mv.DeviceBuffer(n_vec * nact)
+    mv.quantize(qtype, d_x.ptr, cols, n_vec, cols, d_a.ptr)
+    d_h2 = mv.DeviceBuffer(n_vec * rows * 4)
+    mv.gemv_segments(qtype, mv.make_segments([(d_g.ptr, d_h2.ptr, rows, 0, 0, d_u.ptr)]), cols, d_a.ptr,
+                     n_vec, rows)
+    assert np.array_equal(bits(d_h2.download(np.float32, n_vec * rows)), bits(h.ravel()))
+
+
+def test_paired_with_rmsnorm_prologue_and_mixed_segments(oxh):
+    """A feed-forward block's first launch: x + residual -> RMSNorm -> gate/up ->
+    SwiGLU; and a launch that mixes a paired and a plain segment."""
+    rows, cols = 2000, 4096
+    wg, wu, xs = paired_case(Q4K, rows, cols, 1, seed=22)
+    res = synth.normal(cols, seed=22, stream=9).reshape(1, cols)
+    gamma = (synth.normal(cols, seed=23) * np.float32(0.1) + np.float32(1.0)).astype(np.float32)
+    d_g, d_u, d_x, d_r, d_gm = (mv.DeviceBuffer.from_host(a) for a in (wg, wu, xs, res, gamma))
+    d_h, d_y, d_s = mv.DeviceBuffer(rows * 4), mv.DeviceBuffer(cols * 4), mv.DeviceBuffer(cols * 4)
+    segs = mv.make_segments([(d_g.ptr, d_h.ptr, rows, 0, 0, d_u.ptr)])
+    mv.gemv_segments_fused(Q4K, segs, cols, d_x.ptr, cols, mv.PRO_RMSNORM, d_gm.ptr, 1e-5, d_y.ptr, None,
+                           1, rows, d_add=d_r.ptr, d_sum_out=d_s.ptr)
+    assert np.array_equal(bits(d_s.download(np.float32, cols)), bits((xs + res).ravel()))
+    y = d_y.download(np.float32, cols).reshape(1, cols)
+    check_paired(Q4K, wg, wu, rows, cols, y, d_h.download(np.float32, rows).reshape(1, rows))
+    # mixed: segment 0 paired, segment 1 a plain matrix over the same input
+    w3 = synth.weights(Q4K, 300, cols, seed=24)
+    d_w3, d_o3 = mv.DeviceBuffer.from_host(w3), mv.DeviceBuffer(300 * 4)
+    segs = mv.make_segments([(d_g.ptr, d_h.ptr, rows, 0, 0, d_u.ptr), (d_w3.ptr, d_o3.ptr, 300, 0)])
+    mv.gemv_segments_f32(Q4K, segs, cols, d_x.ptr, cols, None, 1, 0)
+    check_paired(Q4K, wg, wu, rows, cols, xs, d_h.download(np.float32, rows).reshape(1, rows))
+    want, _ = oracle_matvec(Q4K, w3, 300, cols, np.ascontiguousarray(xs[0]))
+    assert np.array_equal(bits(d_o3.download(np.float32, 300)), bits(want))
