@@ -45,6 +45,24 @@ def timed(fn, reps, mv):
     return e1.ms_since(e0) * 1e3 / reps
 
 
+def chain_figure(mv, ds, steps):
+    """The same 32 layers as a dependent chain, with the float steps a decode
+    layer runs between its matmuls (residual add + RMSNorm in front of q/k/v and
+    of gate/up, SwiGLU behind gate/up) fused into the four GEMV launches."""
+    from oxidize_amd.workloads import DecodeChain
+    chain = DecodeChain(ds)
+    graph = mv.Graph()
+    with graph:
+        chain.launch_step()
+    us = timed(graph.launch, max(5, steps), mv)
+    nbytes = chain.bytes_per_step
+    return {"us_per_step": round(us, 1), "gbps": round(nbytes / us / 1e3, 1),
+            "frac_of_hbm_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBPS, 4),
+            "launches_per_step": 4 * ds.layers, "bytes_per_step": nbytes,
+            "note": "attention itself is outside this library: the q projection stands in for its "
+                    "output so that every launch depends on the previous one"}
+
+
 def secondary_figures(mv, synth):
     """The other benchmark configurations, measured the same way (inputs
     resident, HIP events on the launch stream).  Reported next to the headline
@@ -388,6 +406,7 @@ def main():
     if not args.no_extra:
         from oxidize_amd import synth
         out["extra"] = secondary_figures(mv, synth)
+        out["extra"]["decode_chain_fused"] = chain_figure(mv, ds, args.steps)
     out["cpu_baseline"] = None if args.no_cpu else cpu_baseline()
     print(json.dumps(out))
     return 0

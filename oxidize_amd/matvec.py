@@ -117,6 +117,10 @@ class DeviceBuffer:
             pass
 
 
+def copy_d2d(d_dst, d_src, nbytes, stream=None):
+    check(lib().oxh_memcpy_d2d(ctypes.c_void_p(d_dst), ctypes.c_void_p(d_src), nbytes, stream))
+
+
 def act_bytes(qtype, cols):
     return lib().oxh_act_bytes(qtype, cols)
 

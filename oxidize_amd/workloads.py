@@ -110,6 +110,97 @@ class DecodeSet:
         return self.act[layer][op].download(np.uint8, mv.act_bytes(qt, cols))
 
 
+class DecodeChain:
+    """The same matrices as a ``DecodeSet``, launched as the dependent chain a
+    decode step really is, with the float steps between the matmuls fused into
+    the GEMV launches (four launches per layer, nothing leaves the device):
+
+      1. q/k/v = W_qkv . Q8K(rmsnorm(x + f) * g_attn)      x <- x + f   (f: the previous
+                                                            layer's feed-forward output)
+      2. o     = W_o . Q8K(a)                               a: attention output
+      3. h     = silu(W_gate . n) * (W_up . n),  n = Q8K(rmsnorm(x + o) * g_ffn),  x <- x + o
+      4. f     = W_down . Q8K(h)
+
+    Attention itself (RoPE, KV cache, softmax) is not part of this library; its
+    output is stood in for by the q projection so that every launch still
+    depends on the one before it.  The residual stream alternates between two
+    buffers because a launch may not store over a vector it reads."""
+
+    def __init__(self, dset, eps=1e-5, seed=0, capture=False):
+        self.d = dset
+        self.eps = eps
+        h, ffn, layers = dset.hidden, dset.ffn, dset.layers
+        self.g_attn_host = [(synth.normal(h, seed=seed, stream=300000 + l) * np.float32(0.1) + np.float32(1.0))
+                            .astype(np.float32) for l in range(layers)]
+        self.g_ffn_host = [(synth.normal(h, seed=seed, stream=310000 + l) * np.float32(0.1) + np.float32(1.0))
+                           .astype(np.float32) for l in range(layers)]
+        self.g_attn = [mv.DeviceBuffer.from_host(g) for g in self.g_attn_host]
+        self.g_ffn = [mv.DeviceBuffer.from_host(g) for g in self.g_ffn_host]
+        self.x0_host = synth.normal(h, seed=seed, stream=320000)
+        self.f0_host = np.zeros(h, np.float32)
+        self.x0 = mv.DeviceBuffer.from_host(self.x0_host)
+        self.f0 = mv.DeviceBuffer.from_host(self.f0_host)
+        self.res = [mv.DeviceBuffer(h * 4) for _ in range(3)]     # residual stream, rotating
+        self.qkv = mv.DeviceBuffer((h + 2 * dset.kv) * 4)
+        self.o = mv.DeviceBuffer(h * 4)
+        self.h = mv.DeviceBuffer(ffn * 4)
+        self.f = mv.DeviceBuffer(h * 4)
+        # per-stage copies for the parity test: [layer] -> dict of DeviceBuffers
+        self.capture = capture
+        self.cap = [dict(n1=mv.DeviceBuffer(h * 4), x1=mv.DeviceBuffer(h * 4), qkv=mv.DeviceBuffer((h + 2 * dset.kv) * 4),
+                         o=mv.DeviceBuffer(h * 4), n2=mv.DeviceBuffer(h * 4), x2=mv.DeviceBuffer(h * 4),
+                         h=mv.DeviceBuffer(ffn * 4), f=mv.DeviceBuffer(h * 4))
+                    for _ in range(layers)] if capture else None
+        self.segs = []
+        for l in range(layers):
+            w = dset.weights[l]
+            off, qkv_items = 0, []
+            for seg, r in enumerate(dset.ops[0][2]):
+                qkv_items.append((w[0][seg].ptr, self.qkv.ptr + off * 4, r, 0))
+                off += r
+            self.segs.append(dict(
+                qkv=mv.make_segments(qkv_items),
+                o=mv.make_segments([(w[1][0].ptr, self.o.ptr, h, 0)]),
+                gate_up=mv.make_segments([(w[2][0].ptr, self.h.ptr, ffn, 0, 0, w[2][1].ptr)]),
+                down=mv.make_segments([(w[3][0].ptr, self.f.ptr, h, 0)])))
+
+    @property
+    def bytes_per_step(self):
+        """Packed weights once, plus what the four launches of a layer read and
+        write in f32: x, f, g, x' / q,k,v out; a in, o out; x, o, g in, x', h
+        out; h in, f out."""
+        d = self.d
+        h, kv, ffn = d.hidden, d.kv, d.ffn
+        per_layer = 4 * ((3 * h + h + (h + 2 * kv)) + (h + h) + (3 * h + h + ffn) + (ffn + h))
+        return d.weight_bytes + d.layers * per_layer
+
+    def launch_step(self, stream=None):
+        d = self.d
+        h = d.hidden
+        x, f = self.x0, self.f0
+        turn = 0
+        for l in range(d.layers):
+            sg = self.segs[l]
+            cap = self.cap[l] if self.capture else None
+            # three buffers in rotation: a launch never stores over a vector it reads
+            x1, x2 = self.res[turn % 3], self.res[(turn + 1) % 3]
+            turn += 2
+            mv.gemv_segments_fused(Q4K, sg["qkv"], h, x.ptr, h, mv.PRO_RMSNORM, self.g_attn[l].ptr, self.eps,
+                                   cap["n1"].ptr if cap else None, None, 1, 0, stream, d_add=f.ptr,
+                                   d_sum_out=x1.ptr)
+            mv.gemv_segments_f32(Q4K, sg["o"], h, self.qkv.ptr, h, None, 1, 0, stream)
+            mv.gemv_segments_fused(Q4K, sg["gate_up"], h, x1.ptr, h, mv.PRO_RMSNORM, self.g_ffn[l].ptr, self.eps,
+                                   cap["n2"].ptr if cap else None, None, 1, 0, stream, d_add=self.o.ptr,
+                                   d_sum_out=x2.ptr)
+            mv.gemv_segments_f32(Q6K, sg["down"], d.ffn, self.h.ptr, d.ffn, None, 1, 0, stream)
+            if cap:
+                for name, src in (("x1", x1), ("qkv", self.qkv), ("o", self.o), ("x2", x2), ("h", self.h),
+                                  ("f", self.f)):
+                    mv.copy_d2d(cap[name].ptr, src.ptr, cap[name].nbytes, stream)
+            x, f = x2, self.f
+        self.last_x = x
+
+
 def route_top_k(logits, k=2, renorm=True):
     """Token -> expert routing as the reference's MoE layers do it
     (llama.c:5965-6031): softmax over the expert logits, the k largest

@@ -274,3 +274,56 @@ def test_paired_with_rmsnorm_prologue_and_mixed_segments(oxh):
     check_paired(Q4K, wg, wu, rows, cols, xs, d_h.download(np.float32, rows).reshape(1, rows))
     want, _ = oracle_matvec(Q4K, w3, 300, cols, np.ascontiguousarray(xs[0]))
     assert np.array_equal(bits(d_o3.download(np.float32, 300)), bits(want))
+
+
+def test_decode_chain_stage_by_stage(oxh):
+    """Two layers of the dependent decode chain (four launches per layer, float
+    steps fused into the GEMVs).  Every stage is checked against the oracle
+    applied to the stage's own inputs as the device produced them: sums and
+    integer paths to the bit, RMSNorm and SwiGLU to rounding."""
+    from oxidize_amd.workloads import DecodeChain, DecodeSet
+    hidden, kv, ffn, layers = 1024, 256, 2816, 2
+    ds = DecodeSet(hidden=hidden, kv=kv, ffn=ffn, layers=layers, seed=3, keep_host=range(layers))
+    ch = DecodeChain(ds, eps=1e-5, seed=3, capture=True)
+    ch.launch_step()
+    mv.sync()
+    o = oxlibs.oracle()
+
+    def rms(x, g):
+        out = np.zeros(x.size, np.float32)
+        o.oxo_rms_norm_f32(x.ctypes.data, g.ctypes.data, out.ctypes.data, x.size, 1e-5)
+        return out
+
+    x, f = ch.x0_host, ch.f0_host
+    for l in range(layers):
+        c = {k: b.download(np.float32, b.nbytes // 4) for k, b in ch.cap[l].items()}
+        assert np.array_equal(bits(c["x1"]), bits(x + f))
+        want = rms(c["x1"], ch.g_attn_host[l])
+        assert np.all(np.abs(c["n1"] - want) <= FLOAT_RTOL * np.abs(want))
+        off = 0
+        for seg, r in enumerate((hidden, kv, kv)):
+            got, _ = oracle_matvec(Q4K, ds.host[(l, 0, seg)], r, hidden, c["n1"])
+            assert np.array_equal(bits(c["qkv"][off:off + r]), bits(got))
+            off += r
+        got, _ = oracle_matvec(Q4K, ds.host[(l, 1, 0)], hidden, hidden, np.ascontiguousarray(c["qkv"][:hidden]))
+        assert np.array_equal(bits(c["o"]), bits(got))
+        assert np.array_equal(bits(c["x2"]), bits(c["x1"] + c["o"]))
+        want = rms(c["x2"], ch.g_ffn_host[l])
+        assert np.all(np.abs(c["n2"] - want) <= FLOAT_RTOL * np.abs(want))
+        gate, _ = oracle_matvec(Q4K, ds.host[(l, 2, 0)], ffn, hidden, c["n2"])
+        up, _ = oracle_matvec(Q4K, ds.host[(l, 2, 1)], ffn, hidden, c["n2"])
+        want = np.zeros(ffn, np.float32)
+        o.oxo_swiglu_f32(gate.ctypes.data, up.ctypes.data, want.ctypes.data, ffn)
+        assert np.all(np.abs(c["h"] - want) <= FLOAT_RTOL * np.abs(want) + 1e-30)
+        got, _ = oracle_matvec(Q6K, ds.host[(l, 3, 0)], hidden, ffn, c["h"])
+        assert np.array_equal(bits(c["f"]), bits(got))
+        x, f = c["x2"], c["f"]
+    # a replay as one graph reproduces the eager run bit for bit
+    eager = ch.last_x.download(np.float32, hidden)
+    g = mv.Graph()
+    with g:
+        ch.launch_step(g.stream)
+    for _ in range(3):
+        g.launch()
+        mv.sync()
+        assert np.array_equal(bits(ch.last_x.download(np.float32, hidden)), bits(eager))
