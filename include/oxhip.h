@@ -39,6 +39,8 @@ extern "C" {
 #define OXH_ERR_NO_DEVICE (-3)
 #define OXH_ERR_TOO_WIDE (-4) /* cols beyond what one workgroup can stage    */
 #define OXH_ERR_NOMEM    (-5)
+#define OXH_ERR_FORMAT   (-6) /* a model file is malformed or truncated       */
+#define OXH_ERR_IO       (-7) /* a model file could not be opened or mapped   */
 
 /* GGUF quantization type ids handled here; values are ABI
  * (oxidize-c/include/oxidize/quant.h:94-110). */
@@ -48,6 +50,7 @@ extern "C" {
 #define OXH_Q5_K_S 14u
 #define OXH_Q5_K_M 15u
 #define OXH_Q6_K   16u
+#define OXH_QTYPE_UNKNOWN 0xffffffffu
 
 /* Block geometry (oxidize-c/include/oxidize/oxk.h:46-66). */
 #define OXH_QK_K         256u
@@ -227,6 +230,61 @@ int  oxh_graph_destroy(void *graph_exec);
 /* name (<=255 chars), compute units, clock MHz, memory bytes. */
 int  oxh_device_info(char *name, size_t name_len, int *n_cu, int *clock_mhz,
                      size_t *mem_bytes);
+
+/* ─── model files ─────────────────────────────────────────────────────── */
+
+/* GGUF v2 / v3 files: the tensor table as weight views for the entry points
+ * below, and the upload of every tensor this library has kernels for.
+ * Replaces oc_gguf_map_open / oc_gguf_map_tensor_get / oc_gguf_map_tensor_data
+ * (oxidize-c/include/oxidize/gguf.h:262-331, parser oxidize-c/src/format/
+ * gguf.c:322-505, same acceptance rules), view_from_info
+ * (oxidize-c/src/model/llama.c:108-127) and oc_cuda_init's upload loop
+ * (oxidize-c/src/backends/cuda.cu:633-712).  The file is mapped read-only and
+ * never copied on the host; a malformed file is OXH_ERR_FORMAT, never a crash. */
+#define OXH_GGUF_MAX_DIMS 8u
+
+typedef struct OxhGguf OxhGguf;
+
+typedef struct OxhTensor {
+    const char *name;       /* NUL-terminated, owned by the OxhGguf                     */
+    uint32_t    qtype;      /* type id as the matvec entry points take it (oxidize-c/
+                               include/oxidize/quant.h:92-140), OXH_QTYPE_UNKNOWN if the
+                               on-disk id is not one the reference maps                 */
+    uint32_t    ggml_type;  /* the on-disk id                                           */
+    uint32_t    n_dims;
+    uint64_t    dims[OXH_GGUF_MAX_DIMS];    /* dims[0] is the innermost                 */
+    uint64_t    offset;     /* from the start of the data section                       */
+    const void *data;       /* inside the mapping                                       */
+    size_t      nbytes;     /* 0 when the type has no fixed block layout here           */
+    size_t      rows;       /* product of dims[1..]: a stacked expert tensor is all its
+                               experts' rows, expert e at rows [e*dims[1], (e+1)*dims[1]) */
+    size_t      cols;       /* dims[0]                                                  */
+    size_t      row_bytes;  /* packed bytes of one row, 0 if cols is not whole blocks   */
+    int         resident;   /* made resident by oxh_gguf_register_all                   */
+} OxhTensor;
+
+int  oxh_gguf_open(const char *path, OxhGguf **out);
+/* Unregisters what oxh_gguf_register_all made resident and unmaps the file. */
+void oxh_gguf_close(OxhGguf *g);
+/* Any of the out pointers may be NULL. */
+int  oxh_gguf_info(const OxhGguf *g, uint32_t *version, uint64_t *alignment, uint64_t *data_start,
+                   size_t *n_tensors, size_t *n_metadata);
+int  oxh_gguf_tensor_at(const OxhGguf *g, size_t index, OxhTensor *out);
+/* OXH_DECLINED when there is no tensor of that name. */
+int  oxh_gguf_tensor_find(const OxhGguf *g, const char *name, OxhTensor *out);
+/* Metadata by key: OXH_DECLINED when the key is absent or of another kind
+ * (u64: any integer or bool that is not negative; f64: F32 or F64; str: the
+ * bytes inside the mapping, not NUL-terminated). */
+int  oxh_gguf_meta_u64(const OxhGguf *g, const char *key, uint64_t *out);
+int  oxh_gguf_meta_f64(const OxhGguf *g, const char *key, double *out);
+int  oxh_gguf_meta_str(const OxhGguf *g, const char *key, const char **data, size_t *len);
+/* Makes every matrix (2 or more dimensions) whose type and width have an
+ * integer path here resident in HBM, whole, so that later matvec calls on
+ * the tensor or on an expert slice of it find it there. */
+int  oxh_gguf_register_all(OxhGguf *g, size_t *n_registered, size_t *bytes);
+/* On-disk type id -> type id of the matvec entry points
+ * (oc_quant_type_from_ggml_id, oxidize-c/src/compute/quantization.c:2980-2988). */
+uint32_t oxh_qtype_from_ggml_id(uint32_t ggml_id);
 
 /* ─── layer 1: drop-in host API ───────────────────────────────────────── */
 

@@ -10,7 +10,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, "liboxhip.so")
 
 OK, DECLINED = 0, 1
-ERR_HIP, ERR_ARG, ERR_NO_DEVICE, ERR_TOO_WIDE, ERR_NOMEM = -1, -2, -3, -4, -5
+ERR_HIP, ERR_ARG, ERR_NO_DEVICE, ERR_TOO_WIDE, ERR_NOMEM, ERR_FORMAT, ERR_IO = -1, -2, -3, -4, -5, -6, -7
 
 V = ctypes.c_void_p
 Z = ctypes.c_size_t
@@ -26,6 +26,12 @@ class OxhSegment(ctypes.Structure):
 class OxhPrologue(ctypes.Structure):
     _fields_ = [("kind", U32), ("eps", ctypes.c_float), ("d_b", V), ("d_out", V), ("d_add", V),
                 ("d_sum_out", V)]
+
+
+class OxhTensor(ctypes.Structure):
+    _fields_ = [("name", ctypes.c_char_p), ("qtype", U32), ("ggml_type", U32), ("n_dims", U32),
+                ("dims", ctypes.c_uint64 * 8), ("offset", ctypes.c_uint64), ("data", V), ("nbytes", Z),
+                ("rows", Z), ("cols", Z), ("row_bytes", Z), ("resident", I)]
 
 
 class OcMatvecFusedTestStats(ctypes.Structure):
@@ -71,6 +77,17 @@ SIGNATURES = {
     "oxh_graph_destroy": (I, [V]),
     "oxh_device_info": (I, [ctypes.c_char_p, Z, ctypes.POINTER(I), ctypes.POINTER(I),
                             ctypes.POINTER(Z)]),
+    "oxh_gguf_open": (I, [ctypes.c_char_p, ctypes.POINTER(V)]),
+    "oxh_gguf_close": (None, [V]),
+    "oxh_gguf_info": (I, [V, ctypes.POINTER(U32), ctypes.POINTER(ctypes.c_uint64),
+                          ctypes.POINTER(ctypes.c_uint64), ctypes.POINTER(Z), ctypes.POINTER(Z)]),
+    "oxh_gguf_tensor_at": (I, [V, Z, ctypes.POINTER(OxhTensor)]),
+    "oxh_gguf_tensor_find": (I, [V, ctypes.c_char_p, ctypes.POINTER(OxhTensor)]),
+    "oxh_gguf_meta_u64": (I, [V, ctypes.c_char_p, ctypes.POINTER(ctypes.c_uint64)]),
+    "oxh_gguf_meta_f64": (I, [V, ctypes.c_char_p, ctypes.POINTER(ctypes.c_double)]),
+    "oxh_gguf_meta_str": (I, [V, ctypes.c_char_p, ctypes.POINTER(V), ctypes.POINTER(Z)]),
+    "oxh_gguf_register_all": (I, [V, ctypes.POINTER(Z), ctypes.POINTER(Z)]),
+    "oxh_qtype_from_ggml_id": (U32, [U32]),
     "oxh_weight_register": (I, [V, Z]),
     "oxh_weight_unregister": (I, [V]),
     "oxh_weight_clear": (I, []),

@@ -36,12 +36,15 @@ def _run(cmd):
 def build_oxhip(verbose=False):
     obj_hip = os.path.join(CSRC, "oxh_kernels.o")
     obj_c = os.path.join(CSRC, "oc_matvec.o")
+    obj_g = os.path.join(CSRC, "oxh_gguf.o")
     out = os.path.join(HERE, "liboxhip.so")
     log = _run([HIPCC] + HIP_FLAGS + ["-I", INCLUDE, "-I", CSRC, "-c",
                                      os.path.join(CSRC, "oxh_kernels.hip"), "-o", obj_hip])
     log += _run([CC] + C_FLAGS + ["-I", INCLUDE, "-I", CSRC, "-c",
                                   os.path.join(CSRC, "oc_matvec.c"), "-o", obj_c])
-    log += _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", out, obj_hip, obj_c,
+    log += _run([CC] + C_FLAGS + ["-I", INCLUDE, "-I", CSRC, "-c",
+                                  os.path.join(CSRC, "oxh_gguf.c"), "-o", obj_g])
+    log += _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", out, obj_hip, obj_c, obj_g,
                  "-lpthread", "-Wno-unused-command-line-argument"])
     if verbose and log.strip():
         print(log)

@@ -82,7 +82,9 @@ static Resident *find_range(const uint8_t *p, size_t bytes)
 {
     for (size_t i = 0; i < g_nres; i++) {
         const Resident *r = &g_res[i];
-        if (p >= r->h && p - r->h <= (ptrdiff_t)r->bytes &&
+        /* p must lie inside the range: the end of one tensor is the start of the
+         * next in a mapped model file */
+        if (p >= r->h && (size_t)(p - r->h) < r->bytes &&
             bytes <= r->bytes - (size_t)(p - r->h))
             return &g_res[i];
     }
