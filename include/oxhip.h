@@ -188,6 +188,18 @@ int oxh_mmq(uint32_t qtype, const void *d_w, size_t rows, size_t cols,
             const void *d_acts, size_t n_vec, float *d_out, size_t out_stride,
             void *stream);
 
+/* Embedding lookup: out[t*out_stride ..] = row d_ids[t] of a packed matrix,
+ * expanded to f32 in the reference's dequantisation arithmetic (bit-identical
+ * to oc_quant_dequant_row, oxidize-c/src/compute/quantization.c:2781-2795), so
+ * the token-embedding table stays quantized in HBM and the ids never leave
+ * the device.  Replaces oc_cuda_mmq_get_row / _get_row_dev / _get_row_batch
+ * (oxidize-c/include/oxidize/cuda_mmq.h:74-93).  Q4_K, Q5_K, Q6_K and Q8_0;
+ * d_ids is device memory (at most 65535 per call); an id >= rows gives a row
+ * of zeros; d_out and out_stride*4 must be multiples of 16 bytes. */
+int oxh_get_rows(uint32_t qtype, const void *d_w, size_t rows, size_t cols,
+                 const uint32_t *d_ids, size_t n_ids, float *d_out, size_t out_stride,
+                 void *stream);
+
 /* Test hook: the integer sub-block sums the GEMV kernel forms, written by the
  * same device code path.  Q4_K and Q5_K: 8 int32 per super-block (S_j), Q6_K: 16 per
  * super-block, Q8_0: 1 per block; layout [row][block][j].  The reference

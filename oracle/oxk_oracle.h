@@ -22,6 +22,7 @@
  *                         raw-block generator of tests/test_oxk_avx2_parity.c,
  *                         closed forms, dequantised double-precision cross-check
  *   oxo_matvec_*          compiled reference entry points, float bits
+ *   oxo_dequant_row       compiled reference oc_quant_dequant_row, float bits
  *   oxo_rms_norm_f32,     compiled reference (oc_rms_norm_f32, oc_swiglu_inplace_f32)
  *   oxo_swiglu_f32        to 1e-6 relative, double-precision numpy, closed
  *                         forms (constant vector, silu(0) = 0, large |g|)
@@ -138,7 +139,8 @@ void oxo_rms_norm_f32(const float *x, const float *weight, float *out, size_t n,
 void oxo_swiglu_f32(const float *gate, const float *up, float *out, size_t n);
 
 /* Dequantise one row to f32 (src/compute/quantization.c:486-503, :633-670,
- * :672-721, :723-766) — used only as an independent cross-check of the layouts. */
+ * :672-721, :723-766): the checker of the embedding lookup, and an independent
+ * cross-check of the layouts behind the dot functions. */
 int oxo_dequant_row(uint32_t qtype, const uint8_t *row, size_t cols, float *out);
 
 #ifdef __cplusplus

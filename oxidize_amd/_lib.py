@@ -54,6 +54,7 @@ SIGNATURES = {
     "oxh_gemv_segments_fused": (I, [U32, ctypes.POINTER(OxhSegment), Z, Z, V, Z,
                                     ctypes.POINTER(OxhPrologue), V, Z, Z, V]),
     "oxh_mmq": (I, [U32, V, Z, Z, V, Z, V, Z, V]),
+    "oxh_get_rows": (I, [U32, V, Z, Z, V, Z, V, Z, V]),
     "oxh_debug_subblock_sums": (I, [U32, V, Z, Z, V, V, V]),
     "oxh_malloc": (I, [ctypes.POINTER(V), Z]),
     "oxh_host_alloc": (I, [ctypes.POINTER(V), Z]),

@@ -260,6 +260,76 @@ k_quantize_q8_0(const float *__restrict__ x, size_t in_stride, uint32_t blocks_p
         *reinterpret_cast<uint16_t *>(dst) = (uint16_t)float_to_half_bits_half_up(d);
 }
 
+/* ─── embedding lookup: packed rows -> f32 ────────────────────────────── */
+
+/* out[t][:] = dequantised row ids[t] of a packed matrix, in the reference's
+ * arithmetic (oxidize-c/src/compute/quantization.c:486-503 Q8_0, :633-670
+ * Q4_K, :672-721 Q5_K, :723-766 Q6_K), so the values equal the CPU path's to
+ * the bit.  One wave per 256 values, lane l producing values 4l .. 4l+3 (they
+ * share a sub-block / scale group); grid.y walks the ids.  An id beyond the
+ * matrix yields a row of zeros rather than a read outside it.
+ * KIND: 0 Q4_K, 1 Q5_K, 2 Q6_K, 3 Q8_0. */
+template <int KIND>
+__global__ __launch_bounds__(256) void
+k_get_rows(const uint8_t *__restrict__ w, uint32_t rows, uint32_t cols, uint32_t row_bytes,
+           const uint32_t *__restrict__ ids, float *__restrict__ out, size_t out_stride)
+{
+    const uint32_t lane = threadIdx.x & 63u;
+    const uint32_t unit = blockIdx.x * 4u + (threadIdx.x >> 6);     /* 256-value span of the row */
+    const uint32_t e0 = unit * 256u + 4u * lane;                    /* this lane's first element */
+    if (e0 >= cols) return;
+    const uint32_t id = ids[blockIdx.y];
+    float *dst = out + (size_t)blockIdx.y * out_stride + e0;
+    float v[4] = { 0.0f, 0.0f, 0.0f, 0.0f };
+    if (id < rows) {
+        const uint8_t *row = w + (size_t)id * row_bytes;
+        if (KIND == 3) {
+            const uint8_t *blk = row + (size_t)(e0 >> 5) * 34u;
+            const float d = half_to_float_hw(*reinterpret_cast<const uint16_t *>(blk));
+            const uint32_t q = reinterpret_cast<const U32u2 *>(blk + 2u + (e0 & 31u))->v;
+#pragma unroll
+            for (int i = 0; i < 4; i++) v[i] = (float)(int8_t)(q >> (8 * i)) * d;
+        } else if (KIND == 2) {
+            const uint8_t *blk = row + (size_t)unit * 210u;
+            const uint32_t e = 4u * lane, n = e >> 7, k = (e >> 5) & 3u, l32 = e & 31u;
+            const uint32_t lo = reinterpret_cast<const U32u2 *>(blk + 64u * n + 32u * (k & 1u) + l32)->v;
+            const uint32_t hi = reinterpret_cast<const U32u2 *>(blk + 128u + 32u * n + l32)->v;
+            const float d = half_to_float_hw(*reinterpret_cast<const uint16_t *>(blk + 208u));
+            const float sc = (float)(int8_t)blk[192u + (e >> 4)];
+            const float ds = d * sc;
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const uint32_t lb = (lo >> (8 * i)) & 0xFFu, hb = (hi >> (8 * i)) & 0xFFu;
+                const int code = (int)((k < 2u ? (lb & 15u) : (lb >> 4)) | (((hb >> (2u * k)) & 3u) << 4)) - 32;
+                v[i] = ds * (float)code;
+            }
+        } else {
+            const uint32_t bs = KIND == 1 ? 176u : 144u;
+            const uint8_t *blk = row + (size_t)unit * bs;
+            const uint32_t e = 4u * lane, j = e >> 5, l32 = e & 31u;
+            const uint32_t hdr = *reinterpret_cast<const uint32_t *>(blk);
+            const float d = half_to_float_hw(hdr & 0xFFFFu), dmin = half_to_float_hw(hdr >> 16);
+            /* 6-bit scale and min of sub-block j (oxk.c:60-75) */
+            const uint8_t *q = blk + 4u;
+            uint32_t sc, mn;
+            if (j < 4u) { sc = q[j] & 63u; mn = q[j + 4u] & 63u; }
+            else { sc = (q[j + 4u] & 15u) | ((q[j - 4u] >> 6) << 4); mn = (q[j + 4u] >> 4) | ((q[j] >> 6) << 4); }
+            const float ds = d * (float)sc, ms = dmin * (float)mn;
+            const uint32_t nib = *reinterpret_cast<const uint32_t *>(blk + (KIND == 1 ? 48u : 16u) + 32u * (j >> 1) + l32);
+            uint32_t fifth = 0u;
+            if (KIND == 1) fifth = *reinterpret_cast<const uint32_t *>(blk + 16u + l32) >> j;
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const uint32_t byte = (nib >> (8 * i)) & 0xFFu;
+                uint32_t code = (j & 1u) ? (byte >> 4) : (byte & 15u);
+                if (KIND == 1) code += ((fifth >> (8 * i)) & 1u) << 4;
+                v[i] = ds * (float)code - ms;
+            }
+        }
+    }
+    *reinterpret_cast<float4 *>(dst) = make_float4(v[0], v[1], v[2], v[3]);
+}
+
 #include "gemv_kernels.inc"
 #include "mmq_kernels.inc"
 
@@ -926,6 +996,39 @@ extern "C" int oxh_mmq(uint32_t qtype, const void *d_w, size_t rows, size_t cols
     else if (shape == 2) mmq_launch<4, 1, 8>(d_w, rows, blocks, d_acts, n_vec, d_out, out_stride, stream);
     else if (shape == 3) mmq_launch<2, 1, 4>(d_w, rows, blocks, d_acts, n_vec, d_out, out_stride, stream);
     else                 mmq_launch<1, 1, 4>(d_w, rows, blocks, d_acts, n_vec, d_out, out_stride, stream);
+    HIP_TRY(hipGetLastError());
+    return OXH_OK;
+}
+
+extern "C" int oxh_get_rows(uint32_t qtype, const void *d_w, size_t rows, size_t cols,
+                            const uint32_t *d_ids, size_t n_ids, float *d_out, size_t out_stride,
+                            void *stream)
+{
+    int rc = ensure_init();
+    if (rc) return rc;
+    if (n_ids == 0) return OXH_OK;
+    if (!d_w || !d_ids || !d_out) return arg_fail("oxh_get_rows: NULL pointer");
+    const size_t rb = oxh_row_bytes(qtype, cols);
+    if (rb == 0) {
+        snprintf(g_err, sizeof g_err, "oxh_get_rows: qtype %u with cols %zu has no kernel here", qtype, cols);
+        return OXH_DECLINED;
+    }
+    if (out_stride < cols) return arg_fail("oxh_get_rows: out_stride < cols");
+    if (rows > 0xFFFFFFFFull || cols > 0xFFFFFFFFull || rb > 0xFFFFFFFFull || n_ids > 65535u)
+        return arg_fail("oxh_get_rows: dimension too large (at most 65535 ids per call)");
+    if ((out_stride & 3u) || ((uintptr_t)d_out & 15u))
+        return arg_fail("oxh_get_rows: output rows must be 16-byte aligned");
+    const dim3 grid((uint32_t)((cols + 1023u) / 1024u), (uint32_t)n_ids), block(256);
+    hipStream_t st = pick_stream(stream);
+    const uint8_t *w = (const uint8_t *)d_w;
+#define OXH_GET_ROWS(KIND)                                                                   \
+    hipLaunchKernelGGL(k_get_rows<KIND>, grid, block, 0, st, w, (uint32_t)rows, (uint32_t)cols, \
+                       (uint32_t)rb, d_ids, d_out, out_stride)
+    if (is_q4k(qtype))          OXH_GET_ROWS(0);
+    else if (is_q5k(qtype))     OXH_GET_ROWS(1);
+    else if (qtype == OXH_Q6_K) OXH_GET_ROWS(2);
+    else                        OXH_GET_ROWS(3);
+#undef OXH_GET_ROWS
     HIP_TRY(hipGetLastError());
     return OXH_OK;
 }

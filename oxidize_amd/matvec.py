@@ -179,6 +179,11 @@ def mmq(qtype, d_w, rows, cols, d_acts, n_vec, d_out, out_stride, stream=None):
                         n_vec, ctypes.c_void_p(d_out), out_stride, stream))
 
 
+def get_rows(qtype, d_w, rows, cols, d_ids, n_ids, d_out, out_stride, stream=None):
+    check(lib().oxh_get_rows(qtype, ctypes.c_void_p(d_w), rows, cols, ctypes.c_void_p(d_ids), n_ids,
+                             ctypes.c_void_p(d_out), out_stride, stream))
+
+
 def debug_subblock_sums(qtype, d_w, rows, cols, d_act, d_sums, stream=None):
     check(lib().oxh_debug_subblock_sums(qtype, ctypes.c_void_p(d_w), rows, cols,
                                         ctypes.c_void_p(d_act), ctypes.c_void_p(d_sums), stream))

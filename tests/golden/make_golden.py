@@ -7,6 +7,7 @@ committed, this script documents how they were made.
 
     python tests/golden/make_golden.py q5_k     # only q5_k.npz
     python tests/golden/make_golden.py float    # only float_steps.npz
+    python tests/golden/make_golden.py dequant  # only dequant_rows.npz
 
 Every array is data: inputs and the reference's outputs for them.
 """
@@ -147,16 +148,36 @@ def float_steps(ref):
     np.savez_compressed(os.path.join(HERE, "float_steps.npz"), **out)
 
 
+def dequant_rows(ref):
+    """dequant_rows.npz: rows of every type the embedding lookup handles,
+    expanded by the compiled reference (oc_quant_dequant_row)."""
+    out = {}
+    for name, qt, cols in (("q4_k", 13, 768), ("q5_k", 15, 768), ("q6_k", 16, 768), ("q8_0", 7, 160)):
+        rows = 3
+        rb = synth.row_bytes(qt, cols)
+        w = synth.weights(qt, rows, cols, seed=17, stream=qt)
+        f = np.zeros((rows, cols), np.float32)
+        for r in range(rows):
+            rc = ref.oc_quant_dequant_row(qt, w[r * rb:].ctypes.data, rb, f[r].ctypes.data, cols)
+            assert rc == 0
+        out[name + "_w"], out[name + "_bits"] = w, f.view(np.uint32).copy()
+        out[name + "_shape"] = np.array([rows, cols, rb], np.int64)
+    np.savez_compressed(os.path.join(HERE, "dequant_rows.npz"), **out)
+
+
 def main():
     ref = oxlibs.ref()
     if ref is None:
         raise SystemExit("oracle/_ref/liboxref.so missing: run `make -C oracle` first")
     ref.oc_parallel_set_threads(1)
-    if sys.argv[1:] != ["float"]:
+    only = sys.argv[1] if len(sys.argv) > 1 else None
+    if only in (None, "q5_k"):
         q5_k(ref)
-    if sys.argv[1:] != ["q5_k"]:
+    if only in (None, "float"):
         float_steps(ref)
-    if sys.argv[1:] in (["q5_k"], ["float"]):
+    if only in (None, "dequant"):
+        dequant_rows(ref)
+    if only is not None:
         return
     rng = np.random.default_rng(20240607)
 

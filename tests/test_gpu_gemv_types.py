@@ -337,3 +337,33 @@ def test_prequantised_and_fused_paths_agree(oxh, qtype, rows, cols, n_vec):
     for v in range(n_vec):
         want, _ = oracle_matvec(qtype, w, rows, cols, np.ascontiguousarray(xs[v]))
         assert np.array_equal(bits(o1[v * rows:(v + 1) * rows]), bits(want))
+
+
+@pytest.mark.parametrize("qtype,rows,cols", [(Q4K, 1000, 4096), (15, 300, 1024), (Q6K, 500, 2816), (Q80, 2000, 896),
+                                             (Q80, 64, 32), (Q4K, 7, 256)])
+def test_embedding_rows_bit_identical_to_the_cpu_dequantisation(oxh, qtype, rows, cols):
+    """oxh_get_rows against the oracle's dequantisation (itself bit-identical
+    to the compiled reference's oc_quant_dequant_row): ids on the device, first
+    and last row, repeats, padded output stride, and an id beyond the matrix,
+    which must give zeros."""
+    w = synth.weights(qtype, rows, cols, seed=33, stream=rows)
+    rb = synth.row_bytes(qtype, cols)
+    ids = np.array([0, rows - 1, rows // 2, 0, rows, 0xFFFFFFFF, 1 % rows], np.uint32)
+    stride = cols + 8
+    d_w = mv.DeviceBuffer.from_host(w)
+    d_ids = mv.DeviceBuffer.from_host(ids)
+    d_o = mv.DeviceBuffer(ids.size * stride * 4)
+    d_o.upload(np.full(ids.size * stride, -7.25, np.float32))
+    mv.get_rows(qtype, d_w.ptr, rows, cols, d_ids.ptr, ids.size, d_o.ptr, stride)
+    got = d_o.download(np.float32, ids.size * stride).reshape(ids.size, stride)
+    o = oxlibs.oracle()
+    for t, i in enumerate(ids):
+        want = np.zeros(cols, np.float32)
+        if i < rows:
+            assert o.oxo_dequant_row(qtype, w[int(i) * rb:].ctypes.data, cols, want.ctypes.data) == 0
+        assert np.array_equal(bits(got[t, :cols]), bits(want)), "id %d" % i
+    assert np.all(got[:, cols:] == -7.25)
+    # a type without a kernel here declines
+    with pytest.raises(mv.OxhError) as e:
+        mv.get_rows(1, d_w.ptr, rows, cols, d_ids.ptr, ids.size, d_o.ptr, stride)
+    assert e.value.status == mv.DECLINED

@@ -474,6 +474,30 @@ def test_swiglu_vs_reference_goldens_and_double_precision():
     assert out[0] == 100.0 and abs(out[1]) < 1e-18
 
 
+@pytest.mark.parametrize("name,qt", [("q4_k", Q4K), ("q5_k", Q5K), ("q6_k", Q6K), ("q8_0", Q80)])
+def test_dequant_row_bits_vs_reference(name, qt):
+    """oxo_dequant_row is the checker of the embedding lookup: bit-identical to
+    the compiled reference's oc_quant_dequant_row on the committed vectors, and
+    live when the compiled reference is present."""
+    g = load("dequant_rows.npz")
+    rows, cols, rb = (int(v) for v in g[name + "_shape"])
+    w = g[name + "_w"]
+    for r in range(rows):
+        out = np.zeros(cols, np.float32)
+        assert O.oxo_dequant_row(qt, w[r * rb:].ctypes.data, cols, out.ctypes.data) == 0
+        assert np.array_equal(out.view(np.uint32), g[name + "_bits"][r])
+    ref = oxlibs.ref()
+    if ref is not None:
+        cols = 2048 if qt != Q80 else 896
+        rb = synth.row_bytes(qt, cols)
+        w = synth.weights(qt, 5, cols, seed=19, stream=qt)
+        for r in range(5):
+            a, b = np.zeros(cols, np.float32), np.zeros(cols, np.float32)
+            assert O.oxo_dequant_row(qt, w[r * rb:].ctypes.data, cols, a.ctypes.data) == 0
+            assert ref.oc_quant_dequant_row(qt, w[r * rb:].ctypes.data, rb, b.ctypes.data, cols) == 0
+            assert np.array_equal(a.view(np.uint32), b.view(np.uint32))
+
+
 def test_eligibility_rules():
     # oxidize-c/src/compute/matvec.c:99-127, :961-985
     assert O.oxo_act_kind(Q4K, 4096) == 2 and O.oxo_act_kind(Q4K, 896) == 0
