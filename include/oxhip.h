@@ -44,6 +44,10 @@ extern "C" {
 
 /* GGUF quantization type ids handled here; values are ABI
  * (oxidize-c/include/oxidize/quant.h:94-110). */
+#define OXH_Q4_0    3u
+#define OXH_Q4_1    4u
+#define OXH_Q5_0    5u
+#define OXH_Q5_1    6u
 #define OXH_Q8_0    7u
 #define OXH_Q4_K_S 12u
 #define OXH_Q4_K_M 13u
@@ -59,6 +63,10 @@ extern "C" {
 #define OXH_Q5_K_BYTES   176u
 #define OXH_Q6_K_BYTES   210u
 #define OXH_Q8_0_BYTES    34u
+#define OXH_Q4_0_BYTES    18u
+#define OXH_Q4_1_BYTES    20u
+#define OXH_Q5_0_BYTES    22u
+#define OXH_Q5_1_BYTES    24u
 #define OXH_Q8_K_BYTES   292u
 
 /* Thread-local text of the last failure on this thread ("" if none). */

@@ -341,11 +341,75 @@ float oxo_dot_q8_0_q8_0(const uint8_t *row, size_t blocks, const uint8_t *act,
     return sum;
 }
 
+/* The 32-value formats.  `isum` (optional) receives one int32 per block: the
+ * offset-corrected integer dot for Q4_0 / Q5_0, the plain code dot for Q4_1 /
+ * Q5_1 (whose second integer is the sum of the activation values). */
+static float dot_legacy(int five_bit, int has_min, const uint8_t *row, size_t blocks,
+                        const uint8_t *act, int32_t *isum)
+{
+    const size_t bytes = 18u + (has_min ? 2u : 0u) + (five_bit ? 4u : 0u);
+    const size_t qh_at = has_min ? 4u : 2u, qs_at = bytes - 16u;
+    float sum = 0.0f;
+    for (size_t b = 0; b < blocks; b++) {
+        const uint8_t *w = row + b * bytes;
+        const uint8_t *a = act + b * OXO_Q8_0_BYTES;
+        const float dw = oxo_f16_to_f32(rd_u16(w));
+        const float mw = has_min ? oxo_f16_to_f32(rd_u16(w + 2)) : 0.0f;
+        const float dq = oxo_f16_to_f32(rd_u16(a));
+        const int8_t *q = (const int8_t *)(a + 2);
+        uint32_t qh = 0;
+        if (five_bit) memcpy(&qh, w + qh_at, 4);
+        int32_t dotp = 0, qsum = 0;
+        for (int j = 0; j < 16; j++) {
+            /* low nibble of byte j = element j, high nibble = element j + 16 */
+            const int32_t x0 = (int32_t)(w[qs_at + j] & 15u) | (int32_t)(((qh >> j) & 1u) << 4);
+            const int32_t x1 = (int32_t)(w[qs_at + j] >> 4) | (int32_t)(((qh >> (j + 16)) & 1u) << 4);
+            dotp += x0 * (int32_t)q[j] + x1 * (int32_t)q[j + 16];
+            qsum += (int32_t)q[j] + (int32_t)q[j + 16];
+        }
+        if (has_min) {
+            if (isum) isum[b] = dotp;
+            const float t = dw * dq;
+            const float tm = mw * dq;
+            const float up = t * (float)dotp;
+            const float off = tm * (float)qsum;
+            sum += up + off;
+        } else {
+            const int32_t v = dotp - (five_bit ? 16 : 8) * qsum;
+            if (isum) isum[b] = v;
+            const float t = dw * dq;
+            sum += t * (float)v;
+        }
+    }
+    return sum;
+}
+
+float oxo_dot_q4_0_q8_0(const uint8_t *row, size_t blocks, const uint8_t *act, int32_t *isum)
+{
+    return dot_legacy(0, 0, row, blocks, act, isum);
+}
+float oxo_dot_q4_1_q8_0(const uint8_t *row, size_t blocks, const uint8_t *act, int32_t *isum)
+{
+    return dot_legacy(0, 1, row, blocks, act, isum);
+}
+float oxo_dot_q5_0_q8_0(const uint8_t *row, size_t blocks, const uint8_t *act, int32_t *isum)
+{
+    return dot_legacy(1, 0, row, blocks, act, isum);
+}
+float oxo_dot_q5_1_q8_0(const uint8_t *row, size_t blocks, const uint8_t *act, int32_t *isum)
+{
+    return dot_legacy(1, 1, row, blocks, act, isum);
+}
+
 /* ─── eligibility ─────────────────────────────────────────────────────── */
 
 static size_t block_bytes(uint32_t qtype)
 {
     switch (qtype) {
+    case OXO_Q4_0:   return 18u;
+    case OXO_Q4_1:   return 20u;
+    case OXO_Q5_0:   return 22u;
+    case OXO_Q5_1:   return 24u;
     case OXO_Q8_0:   return OXO_Q8_0_BYTES;
     case OXO_Q4_K_S:
     case OXO_Q4_K_M: return OXO_Q4_K_BYTES;
@@ -359,6 +423,10 @@ static size_t block_bytes(uint32_t qtype)
 int oxo_act_kind(uint32_t qtype, size_t cols)
 {
     switch (qtype) {
+    case OXO_Q4_0:
+    case OXO_Q4_1:
+    case OXO_Q5_0:
+    case OXO_Q5_1:
     case OXO_Q8_0:   return (cols % OXO_QK8_0 == 0) ? 1 : 0;
     case OXO_Q4_K_S:
     case OXO_Q4_K_M:
@@ -385,6 +453,10 @@ static float row_dot(uint32_t qtype, const uint8_t *row, size_t blocks,
                      const uint8_t *act)
 {
     switch (qtype) {
+    case OXO_Q4_0:   return oxo_dot_q4_0_q8_0(row, blocks, act, NULL);
+    case OXO_Q4_1:   return oxo_dot_q4_1_q8_0(row, blocks, act, NULL);
+    case OXO_Q5_0:   return oxo_dot_q5_0_q8_0(row, blocks, act, NULL);
+    case OXO_Q5_1:   return oxo_dot_q5_1_q8_0(row, blocks, act, NULL);
     case OXO_Q8_0:   return oxo_dot_q8_0_q8_0(row, blocks, act, NULL);
     case OXO_Q6_K:   return oxo_dot_q6_k_q8_k(row, blocks, act, NULL);
     case OXO_Q5_K_S:
@@ -565,6 +637,7 @@ int oxo_dequant_row(uint32_t qtype, const uint8_t *row, size_t cols, float *out)
 {
     const int kind = oxo_act_kind(qtype, cols);
     if (!kind) return 1;
+    if (qtype == OXO_Q4_0 || qtype == OXO_Q4_1 || qtype == OXO_Q5_0 || qtype == OXO_Q5_1) return 1;
     const size_t blocks = n_blocks(kind, cols);
     for (size_t b = 0; b < blocks; b++) {
         if (qtype == OXO_Q8_0) {

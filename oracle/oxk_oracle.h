@@ -40,6 +40,10 @@ extern "C" {
 
 /* GGUF type ids used on this path (include/oxidize/quant.h:94-110). */
 enum {
+    OXO_Q4_0   = 3,
+    OXO_Q4_1   = 4,
+    OXO_Q5_0   = 5,
+    OXO_Q5_1   = 6,
     OXO_Q8_0   = 7,
     OXO_Q4_K_S = 12,
     OXO_Q4_K_M = 13,
@@ -86,6 +90,14 @@ float oxo_dot_q6_k_q8_k(const uint8_t *row, size_t blocks, const uint8_t *act,
  * (optional) receives one int32 per block. */
 float oxo_dot_q8_0_q8_0(const uint8_t *row, size_t blocks, const uint8_t *act,
                         int32_t *isum);
+
+/* src/compute/oxk.c:88-113, :115-139, :141-165, :167-191 (scalar forms, the
+ * block-sequential f32 chain).  `isum` (optional): one int32 per block, the
+ * offset-corrected dot for Q4_0 / Q5_0, the plain code dot for Q4_1 / Q5_1. */
+float oxo_dot_q4_0_q8_0(const uint8_t *row, size_t blocks, const uint8_t *act, int32_t *isum);
+float oxo_dot_q4_1_q8_0(const uint8_t *row, size_t blocks, const uint8_t *act, int32_t *isum);
+float oxo_dot_q5_0_q8_0(const uint8_t *row, size_t blocks, const uint8_t *act, int32_t *isum);
+float oxo_dot_q5_1_q8_0(const uint8_t *row, size_t blocks, const uint8_t *act, int32_t *isum);
 
 /* 0 = not eligible for the integer path, 1 = Q8_0 activation, 2 = Q8_K
  * (src/compute/matvec.c:99-127 restricted to the types above) and the stride

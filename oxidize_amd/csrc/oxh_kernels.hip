@@ -389,6 +389,10 @@ extern "C" void *oxh_internal_stream(void) { return (void *)g_stream; }
 extern "C" int oxh_act_kind(uint32_t qtype, size_t cols)
 {
     switch (qtype) {
+    case OXH_Q4_0:
+    case OXH_Q4_1:
+    case OXH_Q5_0:
+    case OXH_Q5_1:
     case OXH_Q8_0:   return (cols % OXH_QK8_0 == 0) ? 1 : 0;
     case OXH_Q4_K_S:
     case OXH_Q4_K_M:
@@ -402,6 +406,10 @@ extern "C" int oxh_act_kind(uint32_t qtype, size_t cols)
 static size_t block_bytes(uint32_t qtype)
 {
     switch (qtype) {
+    case OXH_Q4_0:   return OXH_Q4_0_BYTES;
+    case OXH_Q4_1:   return OXH_Q4_1_BYTES;
+    case OXH_Q5_0:   return OXH_Q5_0_BYTES;
+    case OXH_Q5_1:   return OXH_Q5_1_BYTES;
     case OXH_Q8_0:   return OXH_Q8_0_BYTES;
     case OXH_Q4_K_S:
     case OXH_Q4_K_M: return OXH_Q4_K_BYTES;
@@ -491,6 +499,10 @@ static hipError_t raise_all_lds_ceilings(void)
     OXH_RAISE(k_gemv_q5_k)
     OXH_RAISE(k_gemv_q6_k)
     OXH_RAISE(k_gemv_q8_0)
+    OXH_RAISE(k_gemv_q4_0)
+    OXH_RAISE(k_gemv_q4_1)
+    OXH_RAISE(k_gemv_q5_0)
+    OXH_RAISE(k_gemv_q5_1)
 #undef OXH_RAISE
 #define OXH_RAISE_PRO1(KERNEL, PRO)                                                               \
     if ((e = raise_lds_ceiling(KERNEL<1, PRO, false>)) != hipSuccess) return e;                   \
@@ -506,6 +518,10 @@ static hipError_t raise_all_lds_ceilings(void)
     OXH_RAISE_PRO(k_gemv_q5_k_pro)
     OXH_RAISE_PRO(k_gemv_q6_k_pro)
     OXH_RAISE_PRO(k_gemv_q8_0_pro)
+    OXH_RAISE_PRO(k_gemv_q4_0_pro)
+    OXH_RAISE_PRO(k_gemv_q4_1_pro)
+    OXH_RAISE_PRO(k_gemv_q5_0_pro)
+    OXH_RAISE_PRO(k_gemv_q5_1_pro)
 #undef OXH_RAISE_PRO
 #undef OXH_RAISE_PRO1
     if ((e = raise_lds_ceiling(k_mmq_q4_k<8, 2, 8>)) != hipSuccess) return e;
@@ -522,7 +538,7 @@ static bool is_q5k(uint32_t qtype) { return qtype == OXH_Q5_K_S || qtype == OXH_
 
 static uint32_t act_lds_bytes(uint32_t qtype, uint32_t blocks)
 {
-    if (qtype == OXH_Q8_0) return q80_lds_bytes(blocks);
+    if (oxh_act_kind(qtype, 32) == 1) return q80_lds_bytes(blocks);
     if (qtype == OXH_Q6_K) return q8k6_lds_bytes(blocks);
     return q8k_lds_bytes(blocks);
 }
@@ -705,7 +721,7 @@ static int launch_gemv(uint32_t qtype, const OxhSegment *segs, size_t n_segs, si
     /* Deal workgroups to segments in proportion to their rows; every wave
      * then owns ceil(rows / waves) whole rows of its segment. */
     uint32_t W = gemv_waves();
-    const size_t blocks_per_pass = qtype == OXH_Q8_0 ? 64u : 16u;
+    const size_t blocks_per_pass = kind == 1 ? 64u : 16u;
     const size_t target = (size_t)(g_n_cu > 0 ? g_n_cu : 256) *
                           gemv_wg_per_cu(total_work * blocks / blocks_per_pass, W);
     uint32_t cap_limit = GEMV_ROWS_CAP;
@@ -810,6 +826,10 @@ static int launch_gemv(uint32_t qtype, const OxhSegment *segs, size_t n_segs, si
     if (is_q4k(qtype))          OXH_LAUNCH_ANY(k_gemv_q4_k, k_gemv_q4_k_pro);
     else if (is_q5k(qtype))     OXH_LAUNCH_ANY(k_gemv_q5_k, k_gemv_q5_k_pro);
     else if (qtype == OXH_Q6_K) OXH_LAUNCH_ANY(k_gemv_q6_k, k_gemv_q6_k_pro);
+    else if (qtype == OXH_Q4_0) OXH_LAUNCH_ANY(k_gemv_q4_0, k_gemv_q4_0_pro);
+    else if (qtype == OXH_Q4_1) OXH_LAUNCH_ANY(k_gemv_q4_1, k_gemv_q4_1_pro);
+    else if (qtype == OXH_Q5_0) OXH_LAUNCH_ANY(k_gemv_q5_0, k_gemv_q5_0_pro);
+    else if (qtype == OXH_Q5_1) OXH_LAUNCH_ANY(k_gemv_q5_1, k_gemv_q5_1_pro);
     else                        OXH_LAUNCH_ANY(k_gemv_q8_0, k_gemv_q8_0_pro);
 #undef OXH_LAUNCH_ANY
 #undef OXH_LAUNCH_PRO
@@ -1008,7 +1028,8 @@ extern "C" int oxh_get_rows(uint32_t qtype, const void *d_w, size_t rows, size_t
     if (rc) return rc;
     if (n_ids == 0) return OXH_OK;
     if (!d_w || !d_ids || !d_out) return arg_fail("oxh_get_rows: NULL pointer");
-    const size_t rb = oxh_row_bytes(qtype, cols);
+    const bool known = is_q4k(qtype) || is_q5k(qtype) || qtype == OXH_Q6_K || qtype == OXH_Q8_0;
+    const size_t rb = known ? oxh_row_bytes(qtype, cols) : 0;
     if (rb == 0) {
         snprintf(g_err, sizeof g_err, "oxh_get_rows: qtype %u with cols %zu has no kernel here", qtype, cols);
         return OXH_DECLINED;

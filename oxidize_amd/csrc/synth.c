@@ -16,6 +16,8 @@
  *               plane, 128 B nibbles
  *   Q6_K 210 B: 128 B ql, 64 B qh, 16 int8 scales, f16 d
  *   Q8_0  34 B: f16 d, 32 int8
+ *   Q4_0 18 B / Q4_1 20 B / Q5_0 22 B / Q5_1 24 B: f16 d [, f16 m][, 32 fifth
+ *               bits], 16 B nibbles
  */
 #include <stddef.h>
 #include <stdint.h>
@@ -190,6 +192,26 @@ void oxs_fill_q8_0(uint8_t *dst, size_t n_blocks, uint64_t seed,
             for (int k = 0; k < 4; k++)
                 blk[2 + i + k] =
                     (uint8_t)(int8_t)((int)(((w >> (16 * k)) & 0xFFFFu) % 255u) - 127);
+        }
+    }
+}
+
+/* The 32-value formats Q4_0 (18 B), Q4_1 (20 B), Q5_0 (22 B), Q5_1 (24 B):
+ * f16 d (and f16 m when has_min) ~ |N(0,sigma)|, every other byte uniform. */
+void oxs_fill_legacy(uint8_t *dst, size_t n_blocks, uint64_t seed, uint64_t stream,
+                     float sigma, uint32_t block_bytes, int has_min)
+{
+#pragma omp parallel for schedule(static)
+    for (long b = 0; b < (long)n_blocks; b++) {
+        Rng r = rng_for(seed, stream, (uint64_t)b);
+        uint8_t *blk = dst + (size_t)b * block_bytes;
+        put16(blk, half_abs_normal(&r, sigma));
+        uint32_t at = 2;
+        if (has_min) { put16(blk + 2, half_abs_normal(&r, sigma)); at = 4; }
+        uint64_t w = 0;
+        for (uint32_t i = at, k = 0; i < block_bytes; i++, k++) {
+            if ((k & 7u) == 0u) w = next64(&r);
+            blk[i] = (uint8_t)(w >> (8u * (k & 7u)));
         }
     }
 }

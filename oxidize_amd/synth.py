@@ -15,9 +15,11 @@ import numpy as np
 _HERE = os.path.dirname(os.path.abspath(__file__))
 _LIB = None
 
-Q8_0, Q4_K, Q5_K, Q6_K = 7, 13, 15, 16
-BLOCK_BYTES = {Q8_0: 34, Q4_K: 144, 12: 144, Q5_K: 176, 14: 176, Q6_K: 210}
-BLOCK_ELEMS = {Q8_0: 32, Q4_K: 256, 12: 256, Q5_K: 256, 14: 256, Q6_K: 256}
+Q4_0, Q4_1, Q5_0, Q5_1, Q8_0, Q4_K, Q5_K, Q6_K = 3, 4, 5, 6, 7, 13, 15, 16
+BLOCK_BYTES = {Q4_0: 18, Q4_1: 20, Q5_0: 22, Q5_1: 24, Q8_0: 34, Q4_K: 144, 12: 144, Q5_K: 176, 14: 176,
+               Q6_K: 210}
+BLOCK_ELEMS = {Q4_0: 32, Q4_1: 32, Q5_0: 32, Q5_1: 32, Q8_0: 32, Q4_K: 256, 12: 256, Q5_K: 256, 14: 256,
+               Q6_K: 256}
 
 
 def _lib():
@@ -32,6 +34,9 @@ def _lib():
             getattr(lib, name).argtypes = [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_uint64,
                                            ctypes.c_uint64, ctypes.c_float]
             getattr(lib, name).restype = None
+        lib.oxs_fill_legacy.argtypes = [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_uint64, ctypes.c_uint64,
+                                        ctypes.c_float, ctypes.c_uint32, ctypes.c_int]
+        lib.oxs_fill_legacy.restype = None
         lib.oxs_fill_normal_f32.argtypes = [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_uint64,
                                             ctypes.c_uint64, ctypes.c_float]
         lib.oxs_fill_normal_f32.restype = None
@@ -52,6 +57,10 @@ def weights(qtype, rows, cols, seed=0, stream=0, sigma=None, out=None):
     if out is None:
         out = np.empty(nbytes, dtype=np.uint8)
     assert out.dtype == np.uint8 and out.size == nbytes and out.flags.c_contiguous
+    if qtype in (Q4_0, Q4_1, Q5_0, Q5_1):
+        _lib().oxs_fill_legacy(out.ctypes.data, n_blocks, seed, stream, 0.02 if sigma is None else sigma,
+                               BLOCK_BYTES[qtype], int(qtype in (Q4_1, Q5_1)))
+        return out
     fn = {Q8_0: "oxs_fill_q8_0", Q4_K: "oxs_fill_q4_k", 12: "oxs_fill_q4_k",
           Q5_K: "oxs_fill_q5_k", 14: "oxs_fill_q5_k", Q6_K: "oxs_fill_q6_k"}[qtype]
     if sigma is None:

@@ -8,6 +8,7 @@ committed, this script documents how they were made.
     python tests/golden/make_golden.py q5_k     # only q5_k.npz
     python tests/golden/make_golden.py float    # only float_steps.npz
     python tests/golden/make_golden.py dequant  # only dequant_rows.npz
+    python tests/golden/make_golden.py legacy   # only legacy_formats.npz
 
 Every array is data: inputs and the reference's outputs for them.
 """
@@ -165,6 +166,52 @@ def dequant_rows(ref):
     np.savez_compressed(os.path.join(HERE, "dequant_rows.npz"), **out)
 
 
+LEGACY = (("q4_0", 3, 18), ("q4_1", 4, 20), ("q5_0", 5, 22), ("q5_1", 6, 24))
+
+
+def legacy_formats(ref):
+    """legacy_formats.npz: Q4_0 / Q4_1 / Q5_0 / Q5_1 against Q8_0 activations,
+    raw-block dots (scalar and dispatched kernels) and the matvec entry points."""
+    rng = np.random.default_rng(20241101)
+    out = {}
+    nb, trials = 12, 16
+    for name, qt, bsize in LEGACY:
+        w = xorshift_bytes(trials * nb * bsize, 0x9E3779B9 ^ qt).reshape(trials, nb, bsize)
+        for off in ((0, 2) if name.endswith("_1") else (0,)):
+            bits = finite_scale_bits(rng, trials * nb).reshape(trials, nb)
+            w[:, :, off] = bits & 0xFF
+            w[:, :, off + 1] = bits >> 8
+        act = np.zeros((trials, nb, 34), np.uint8)
+        bits = finite_scale_bits(rng, trials * nb).reshape(trials, nb)
+        act[:, :, 0] = bits & 0xFF
+        act[:, :, 1] = bits >> 8
+        act[:, :, 2:] = rng.integers(-127, 128, (trials, nb, 32)).astype(np.int8).view(np.uint8)
+        scalar = np.empty((trials, 2), np.uint32)
+        disp = np.empty((trials, 2), np.uint32)
+        fs = getattr(ref, "oc_oxk_dot_%s_q8_0_scalar" % name)
+        fd = getattr(ref, "oc_oxk_dot_%s_q8_0" % name)
+        for t in range(trials):
+            wt, at = np.ascontiguousarray(w[t]), np.ascontiguousarray(act[t])
+            for k, blocks in enumerate((1, nb)):
+                scalar[t, k] = np.float32(fs(wt.ctypes.data, blocks, at.ctypes.data)).view(np.uint32)
+                disp[t, k] = np.float32(fd(wt.ctypes.data, blocks, at.ctypes.data)).view(np.uint32)
+        out[name + "_w"], out[name + "_act"] = w, act
+        out[name + "_scalar_bits"], out[name + "_dispatched_bits"] = scalar, disp
+        rows, cols = 40, 896
+        rb = synth.row_bytes(qt, cols)
+        wm = synth.weights(qt, rows, cols, seed=7, stream=qt)
+        x = synth.normal(cols, seed=7, stream=100 + qt)
+        o = np.zeros(rows, np.float32)
+        temp = np.zeros(cols, np.float32)
+        ref.oc_matvec_quantized(qt, wm.ctypes.data, rows, cols, rb, x.ctypes.data, o.ctypes.data,
+                                temp.ctypes.data)
+        out[name + "_api_w"], out[name + "_api_x"] = wm, x
+        out[name + "_api_shape"] = np.array([rows, cols, rb], np.int64)
+        out[name + "_api_out"] = o.copy()
+        out[name + "_api_act"] = temp.view(np.uint8)[:cols // 32 * 34].copy()
+    np.savez_compressed(os.path.join(HERE, "legacy_formats.npz"), **out)
+
+
 def main():
     ref = oxlibs.ref()
     if ref is None:
@@ -177,6 +224,8 @@ def main():
         float_steps(ref)
     if only in (None, "dequant"):
         dequant_rows(ref)
+    if only in (None, "legacy"):
+        legacy_formats(ref)
     if only is not None:
         return
     rng = np.random.default_rng(20240607)

@@ -42,15 +42,16 @@ def test_no_oracle_or_reference_symbols_in_the_product():
 def test_shape_helpers_match_the_reference_rules():
     lib = _lib.lib()
     o = oxlibs.oracle()
-    for qt in (0, 1, 2, 7, 8, 12, 13, 14, 15, 16, 25):
+    for qt in (0, 1, 2, 3, 4, 5, 6, 7, 8, 12, 13, 14, 15, 16, 25):
         for cols in (0, 32, 96, 256, 896, 900, 2816, 4096, 14336):
-            want = o.oxo_act_kind(qt, cols) if qt in (7, 12, 13, 14, 15, 16) else 0
+            want = o.oxo_act_kind(qt, cols) if qt in (3, 4, 5, 6, 7, 12, 13, 14, 15, 16) else 0
             assert lib.oxh_act_kind(qt, cols) == want
     assert lib.oxh_row_bytes(13, 4096) == 2304
     assert lib.oxh_row_bytes(16, 14336) == 11760
     assert lib.oxh_row_bytes(7, 896) == 952
     assert lib.oxh_row_bytes(13, 896) == 0
     assert lib.oxh_row_bytes(15, 4096) == 2816 and lib.oxh_row_bytes(14, 256) == 176
+    assert [lib.oxh_row_bytes(q, 896) for q in (3, 4, 5, 6)] == [28 * 18, 28 * 20, 28 * 22, 28 * 24]
     assert lib.oxh_act_bytes(13, 4096) == 4672
     assert lib.oxh_act_bytes(7, 896) == 952
     for cols in (0, 31, 256, 896, 4096, 14336, 1 << 20, 3 << 20):

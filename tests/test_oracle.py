@@ -498,12 +498,83 @@ def test_dequant_row_bits_vs_reference(name, qt):
             assert np.array_equal(a.view(np.uint32), b.view(np.uint32))
 
 
+LEGACY = (("q4_0", 3, 18), ("q4_1", 4, 20), ("q5_0", 5, 22), ("q5_1", 6, 24))
+
+
+@pytest.mark.parametrize("name,qt,bsize", LEGACY)
+def test_legacy_formats_vs_reference_goldens(name, qt, bsize):
+    g = load("legacy_formats.npz")
+    fo = getattr(O, "oxo_dot_%s_q8_0" % name)
+    w, act = g[name + "_w"], g[name + "_act"]
+    for t in range(w.shape[0]):
+        wt, at = np.ascontiguousarray(w[t]), np.ascontiguousarray(act[t])
+        for k, blocks in enumerate((1, w.shape[1])):
+            got = f32bits(fo(wt.ctypes.data, blocks, at.ctypes.data, None))
+            assert got == g[name + "_scalar_bits"][t, k]
+            assert got == g[name + "_dispatched_bits"][t, k]
+    rows, cols, rb = (int(v) for v in g[name + "_api_shape"])
+    wm, x = g[name + "_api_w"], g[name + "_api_x"]
+    out = np.zeros(rows, np.float32)
+    temp = np.zeros(cols, np.float32)
+    assert O.oxo_matvec_quantized(qt, wm.ctypes.data, rows, cols, rb, x.ctypes.data, out.ctypes.data,
+                                  temp.ctypes.data) == 0
+    a = g[name + "_api_act"]
+    assert np.array_equal(temp.view(np.uint8)[:a.size], a)
+    want = g[name + "_api_out"]
+    assert np.all(np.abs(out - want) <= 1e-4 + 1e-5 * np.abs(want))
+
+
+@pytest.mark.parametrize("name,qt,bsize", LEGACY)
+def test_legacy_formats_closed_forms_and_layout(name, qt, bsize):
+    """Codes c everywhere, activations a everywhere: 32*(c - offset)*a*d*dq, plus
+    32*a*m*dq for the _1 formats; and one element at a time, which fixes the
+    nibble halves (byte i: low nibble = element i, high = element i + 16) and
+    the fifth-bit order."""
+    fo = getattr(O, "oxo_dot_%s_q8_0" % name)
+    has_m, five = name.endswith("_1"), name.startswith("q5")
+    qs_at = bsize - 16
+    d, m, dq, a = 0.5, 0.25, 0.125, 3
+    act = np.concatenate([np.array(f16_le(dq), np.uint8), np.full(32, a, np.int8).view(np.uint8)])
+    for code in ((5, 12) if not five else (5, 21, 31)):
+        blk = np.zeros(bsize, np.uint8)
+        blk[0:2] = f16_le(d)
+        if has_m:
+            blk[2:4] = f16_le(m)
+        blk[qs_at:] = (code & 15) | ((code & 15) << 4)
+        if five and code & 16:
+            blk[qs_at - 4:qs_at] = 0xFF
+        off = 0 if has_m else (16 if five else 8)
+        want = dq * d * 32 * (code - off) * a + (dq * m * 32 * a if has_m else 0.0)
+        assert fo(blk.ctypes.data, 1, act.ctypes.data, None) == want
+    rng = np.random.default_rng(9)
+    q = rng.integers(-127, 128, 32).astype(np.int8)
+    act = np.concatenate([np.array(f16_le(1.0), np.uint8), q.view(np.uint8)])
+    off = 0 if has_m else (16 if five else 8)
+    base_blk = np.zeros(bsize, np.uint8)
+    base_blk[0:2] = f16_le(1.0)
+    base = fo(base_blk.ctypes.data, 1, act.ctypes.data, None)          # all codes 0
+    assert base == float(-off * int(q.sum()))
+    for e in range(32):
+        blk = base_blk.copy()
+        blk[qs_at + (e & 15)] = 7 << (4 * (e >> 4))
+        isum = np.zeros(1, np.int32)
+        got = fo(blk.ctypes.data, 1, act.ctypes.data, isum.ctypes.data)
+        assert got == base + 7.0 * q[e], "element %d" % e
+        if five:
+            blk = base_blk.copy()
+            blk[qs_at - 4 + (e >> 3)] = 1 << (e & 7)
+            assert fo(blk.ctypes.data, 1, act.ctypes.data, None) == base + 16.0 * q[e], "fifth bit %d" % e
+
+
 def test_eligibility_rules():
     # oxidize-c/src/compute/matvec.c:99-127, :961-985
     assert O.oxo_act_kind(Q4K, 4096) == 2 and O.oxo_act_kind(Q4K, 896) == 0
     assert O.oxo_act_kind(Q6K, 256) == 2 and O.oxo_act_kind(12, 512) == 2
     assert O.oxo_act_kind(Q80, 896) == 1 and O.oxo_act_kind(Q80, 900) == 0
     assert O.oxo_act_kind(0, 4096) == 0 and O.oxo_act_kind(1, 4096) == 0
+    for qt, rb in ((3, 18), (4, 20), (5, 22), (6, 24)):
+        assert O.oxo_act_kind(qt, 896) == 1 and O.oxo_act_kind(qt, 900) == 0
+        assert O.oxo_stride_ok(qt, 896, 28 * rb) == 1 and O.oxo_stride_ok(qt, 896, 28 * rb + 2) == 0
     assert O.oxo_act_kind(14, 512) == 2 and O.oxo_act_kind(Q5K, 4096) == 2 and O.oxo_act_kind(Q5K, 4000) == 0
     assert O.oxo_stride_ok(Q5K, 4096, 2816) == 1 and O.oxo_stride_ok(Q5K, 4096, 2304) == 0
     assert O.oxo_stride_ok(Q4K, 4096, 2304) == 1 and O.oxo_stride_ok(Q4K, 4096, 2320) == 0
