@@ -201,6 +201,24 @@ def secondary_figures(mv, synth):
         "note": "792.7 MB of expert weights fit the 256 MB last-level cache only in part; "
                 "per step: Q8_K quantisation + one MFMA launch for all experts' gate+up, the same for "
                 "all experts' down, each expert over its own tokens only"}
+    # the same layer end to end with the routing on the device: router logits in, combined output out
+    layer = mv.MoeLayer(Q4K, Q4K, ms.w["gate"].ptr, ms.w["up"].ptr, ms.w["down"].ptr, ms.n_expert, ms.top_k,
+                        ms.hidden, ms.ffn, True, max_tok=ms.n_tok)
+    d_logits = mv.DeviceBuffer.from_host(ms.logits)
+    d_xt = mv.DeviceBuffer.from_host(ms.x_tok)
+    d_yt = mv.DeviceBuffer(ms.n_tok * ms.hidden * 4)
+    layer.forward(d_logits.ptr, d_xt.ptr, ms.n_tok, d_yt.ptr)
+    mv.sync()
+    graph = mv.Graph()
+    with graph:
+        layer.forward(d_logits.ptr, d_xt.ptr, ms.n_tok, d_yt.ptr)
+    us = timed(graph.launch, 10, mv)
+    out["moe_layer_device_routed_8x_top2_16tok_q4k"] = {
+        "us": round(us, 2), "gbps": round(ms.bytes_per_step / us / 1e3, 1),
+        "frac_of_hbm_peak": round(ms.bytes_per_step / us / 1e3 / HBM_PEAK_GBPS, 4),
+        "launches": 6,
+        "note": "oxh_moe_ffn as one graph: route + group, gather + Q8_K, gate/up of all experts, "
+                "silu(gate)*up + Q8_K, down of all experts, combine; no host step between them"}
     return out
 
 

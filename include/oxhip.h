@@ -208,6 +208,52 @@ int oxh_get_rows(uint32_t qtype, const void *d_w, size_t rows, size_t cols,
                  const uint32_t *d_ids, size_t n_ids, float *d_out, size_t out_stride,
                  void *stream);
 
+/* Mixture-of-experts feed-forward with the routing on the device.  For n_tok
+ * tokens (router logits [n_tok][n_expert], inputs [n_tok][hidden]):
+ *   route    softmax, the top_k experts per token, gate weights (renormalised
+ *            over the selected experts when `renorm`)
+ *   group    (token, expert) pairs sorted by expert, token order kept
+ *   experts  per expert and only for its own tokens: gate, up, silu(gate)*up,
+ *            down -- int8 MFMA over Q8_K activations
+ *   combine  out[token] = sum, in ascending expert order, of weight * down
+ * as oxidize-c/src/model/llama.c:5965-6160 does it on the host; the device
+ * analogues are k_moe_route (oxidize-c/src/backends/cuda.cu:495) and
+ * oc_cuda_mmq_matvec_expert (oxidize-c/include/oxidize/cuda_mmq.h:64-72).
+ * Nothing returns to the host between the steps and the launch sizes depend
+ * only on n_tok, so a layer is a fixed sequence that may be captured in a
+ * graph.  Expert matrices are stacked expert-major (expert e of gate/up at
+ * rows [e*ffn, (e+1)*ffn), of down at rows [e*hidden, (e+1)*hidden)); types
+ * Q4_K, Q5_K or Q6_K; at most 16 experts, top_k <= 8, n_tok <= 4096.
+ * Expert ids and the grouping are exact; gate weights and silu(gate)*up are
+ * float steps that agree with the reference to rounding; everything the
+ * integer path computes from them is exact. */
+typedef struct OxhMoe {
+    uint32_t    qtype_gate_up, qtype_down;
+    const void *d_w_gate, *d_w_up, *d_w_down;
+    size_t      n_expert, top_k, hidden, ffn;
+    int         renorm;
+} OxhMoe;
+int oxh_moe_workspace_bytes(const OxhMoe *m, size_t n_tok, size_t *bytes);
+/* d_workspace: oxh_moe_workspace_bytes() of device memory, 256-byte aligned,
+ * overwritten by every call. */
+int oxh_moe_ffn(const OxhMoe *m, const float *d_logits, const float *d_x, size_t x_stride,
+                size_t n_tok, float *d_out, size_t out_stride, void *d_workspace,
+                size_t workspace_bytes, void *stream);
+/* The routing and grouping step alone (n_expert <= 32).  ids, weights,
+ * slot_pos: n_tok*top_k entries, pair (t, j) at t*top_k + j; counts,
+ * offsets: per expert (offsets has n_expert + 1 entries); perm: the token of
+ * each sorted pair; slot_pos: where pair (t, j) landed in that order. */
+int oxh_moe_route(const float *d_logits, size_t n_tok, size_t n_expert, size_t top_k, int renorm,
+                  int32_t *d_ids, float *d_weights, uint32_t *d_counts, uint32_t *d_offsets,
+                  uint32_t *d_perm, uint32_t *d_slot_pos, void *stream);
+
+/* Test hook: byte offsets inside oxh_moe_ffn's workspace of, in this order,
+ * ids, weights, slot_pos, perm, counts, offsets, the gathered Q8_K activations,
+ * gate, up (f32 [pair][ffn]), the Q8_K form of silu(gate)*up, the down outputs
+ * (f32 [pair][hidden]), and the total size.  After a call the parity tests read
+ * every intermediate from there. */
+int oxh_debug_moe_workspace_parts(const OxhMoe *m, size_t n_tok, size_t parts[12]);
+
 /* Test hook: the integer sub-block sums the GEMV kernel forms, written by the
  * same device code path.  Q4_K and Q5_K: 8 int32 per super-block (S_j), Q6_K: 16 per
  * super-block, Q8_0: 1 per block; layout [row][block][j].  The reference

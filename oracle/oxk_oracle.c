@@ -692,3 +692,43 @@ int oxo_dequant_row(uint32_t qtype, const uint8_t *row, size_t cols, float *out)
     }
     return 0;
 }
+
+/* ─── MoE feed-forward ────────────────────────────────────────────────── */
+
+int oxo_moe_ffn(uint32_t qtype_gate_up, uint32_t qtype_down, const uint8_t *w_gate,
+                const uint8_t *w_up, const uint8_t *w_down, size_t n_expert, size_t k,
+                size_t hidden, size_t ffn, int renorm, const float *logits,
+                const float *x, size_t n_tok, float *out)
+{
+    const size_t rb_gu = n_blocks(oxo_act_kind(qtype_gate_up, hidden), hidden) * block_bytes(qtype_gate_up);
+    const size_t rb_dn = n_blocks(oxo_act_kind(qtype_down, ffn), ffn) * block_bytes(qtype_down);
+    int32_t *ids = (int32_t *)malloc(n_tok * k * sizeof(int32_t));
+    float *wts = (float *)malloc(n_tok * k * sizeof(float));
+    float *gate = (float *)malloc(ffn * sizeof(float));
+    float *up = (float *)malloc(ffn * sizeof(float));
+    float *down = (float *)malloc(hidden * sizeof(float));
+    float *temp = (float *)malloc(((hidden > ffn ? hidden : ffn) / 256u + 1u) * 296u);
+    int rc = 1;
+    if (!ids || !wts || !gate || !up || !down || !temp) goto done;
+    oxo_moe_route(logits, n_tok, n_expert, k, renorm, ids, wts);
+    memset(out, 0, n_tok * hidden * sizeof(float));
+    rc = 0;
+    /* experts in ascending order, each over its tokens in token order: what
+     * the counting sort plus the per-expert pass amount to */
+    for (size_t e = 0; e < n_expert && !rc; e++)
+        for (size_t t = 0; t < n_tok && !rc; t++)
+            for (size_t j = 0; j < k; j++) {
+                if ((size_t)ids[t * k + j] != e) continue;
+                const float *xt = x + t * hidden;
+                rc |= oxo_matvec_quantized(qtype_gate_up, w_gate + e * ffn * rb_gu, ffn, hidden, rb_gu, xt, gate, temp);
+                rc |= oxo_matvec_quantized(qtype_gate_up, w_up + e * ffn * rb_gu, ffn, hidden, rb_gu, xt, up, temp);
+                oxo_swiglu_f32(gate, up, gate, ffn);
+                rc |= oxo_matvec_quantized(qtype_down, w_down + e * hidden * rb_dn, hidden, ffn, rb_dn, gate, down, temp);
+                const float w = wts[t * k + j];
+                float *dst = out + t * hidden;
+                for (size_t i = 0; i < hidden; i++) dst[i] += w * down[i];
+            }
+done:
+    free(ids); free(wts); free(gate); free(up); free(down); free(temp);
+    return rc;
+}

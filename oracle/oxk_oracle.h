@@ -26,6 +26,12 @@
  *   oxo_rms_norm_f32,     compiled reference (oc_rms_norm_f32, oc_swiglu_inplace_f32)
  *   oxo_swiglu_f32        to 1e-6 relative, double-precision numpy, closed
  *                         forms (constant vector, silu(0) = 0, large |g|)
+ *   oxo_moe_route         brute force (argsort of a double-precision softmax)
+ *   oxo_moe_ffn           composition of the functions above; against a numpy
+ *                         restatement built from per-expert dense products of
+ *                         the dequantised matrices (loose tolerance: pins the
+ *                         routing, grouping, expert indexing and combination,
+ *                         not the rounding, which the parts pin)
  * No function is "parity unpinned".
  */
 #ifndef OXK_ORACLE_H
@@ -139,6 +145,16 @@ size_t oxo_matvec_batch_scratch_bytes(size_t max_cols);
  * keep the lower index), optional renormalisation.  ids/weights: n_tok*k. */
 void oxo_moe_route(const float *logits, size_t n_tok, size_t n_expert,
                    size_t k, int renorm, int32_t *ids, float *weights);
+
+/* One MoE feed-forward layer over n_tok tokens as src/model/llama.c:5965-6160
+ * runs it (quantised expert matrices, no shared or zero experts): route, then
+ * experts in ascending order, each over its tokens in token order: gate, up,
+ * SwiGLU, down, out[token] += weight * down.  Expert matrices stacked
+ * expert-major.  Returns 0 when every matvec took the integer path. */
+int oxo_moe_ffn(uint32_t qtype_gate_up, uint32_t qtype_down, const uint8_t *w_gate,
+                const uint8_t *w_up, const uint8_t *w_down, size_t n_expert, size_t k,
+                size_t hidden, size_t ffn, int renorm, const float *logits,
+                const float *x, size_t n_tok, float *out);
 
 /* The float steps a decode layer runs in front of the quantiser, scalar forms:
  * RMSNorm (src/compute/activation.c:16-22 with the scalar dot and apply of

@@ -28,6 +28,11 @@ class OxhPrologue(ctypes.Structure):
                 ("d_sum_out", V)]
 
 
+class OxhMoe(ctypes.Structure):
+    _fields_ = [("qtype_gate_up", U32), ("qtype_down", U32), ("d_w_gate", V), ("d_w_up", V), ("d_w_down", V),
+                ("n_expert", Z), ("top_k", Z), ("hidden", Z), ("ffn", Z), ("renorm", I)]
+
+
 class OxhTensor(ctypes.Structure):
     _fields_ = [("name", ctypes.c_char_p), ("qtype", U32), ("ggml_type", U32), ("n_dims", U32),
                 ("dims", ctypes.c_uint64 * 8), ("offset", ctypes.c_uint64), ("data", V), ("nbytes", Z),
@@ -56,6 +61,10 @@ SIGNATURES = {
     "oxh_mmq": (I, [U32, V, Z, Z, V, Z, V, Z, V]),
     "oxh_get_rows": (I, [U32, V, Z, Z, V, Z, V, Z, V]),
     "oxh_debug_subblock_sums": (I, [U32, V, Z, Z, V, V, V]),
+    "oxh_moe_workspace_bytes": (I, [ctypes.POINTER(OxhMoe), Z, ctypes.POINTER(Z)]),
+    "oxh_moe_ffn": (I, [ctypes.POINTER(OxhMoe), V, V, Z, Z, V, Z, V, Z, V]),
+    "oxh_moe_route": (I, [V, Z, Z, Z, I, V, V, V, V, V, V, V]),
+    "oxh_debug_moe_workspace_parts": (I, [ctypes.POINTER(OxhMoe), Z, ctypes.POINTER(Z * 12)]),
     "oxh_malloc": (I, [ctypes.POINTER(V), Z]),
     "oxh_host_alloc": (I, [ctypes.POINTER(V), Z]),
     "oxh_host_free": (I, [V]),

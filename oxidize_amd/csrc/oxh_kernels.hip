@@ -189,18 +189,29 @@ __device__ __forceinline__ int quantize_one(float x, float inv)
 
 /* ─── activation quantisers ───────────────────────────────────────────── */
 
-/* One wave per 256-value block; lane l owns values 4l..4l+3. */
+/* One wave per 256-value block; lane l owns values 4l..4l+3.  Two optional
+ * extras for the mixture-of-experts path: `row_index` makes output vector v
+ * read input row row_index[v] (the gather of each expert's tokens), and `up`
+ * (laid out like x, same row) makes the value quantised silu(x) * up. */
 __global__ __launch_bounds__(256) void
 k_quantize_q8_k(const float *__restrict__ x, size_t in_stride, uint32_t blocks_per_vec,
-                uint32_t total_blocks, uint8_t *__restrict__ act)
+                uint32_t total_blocks, uint8_t *__restrict__ act,
+                const uint32_t *__restrict__ row_index, const float *__restrict__ up)
 {
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t gb = blockIdx.x * 4u + (threadIdx.x >> 6);
     if (gb >= total_blocks) return;
     const uint32_t vec = gb / blocks_per_vec;
     const uint32_t blk = gb - vec * blocks_per_vec;
-    const float *src = x + (size_t)vec * in_stride + (size_t)blk * 256u + 4u * lane;
-    const float v0 = src[0], v1 = src[1], v2 = src[2], v3 = src[3];
+    const size_t at = (size_t)(row_index ? row_index[vec] : vec) * in_stride + (size_t)blk * 256u + 4u * lane;
+    const float *src = x + at;
+    float v0 = src[0], v1 = src[1], v2 = src[2], v3 = src[3];
+    if (up) {
+        const float *u = up + at;
+        const float s0 = 1.0f / (1.0f + expf(-v0)), s1 = 1.0f / (1.0f + expf(-v1));
+        const float s2 = 1.0f / (1.0f + expf(-v2)), s3 = 1.0f / (1.0f + expf(-v3));
+        v0 = v0 * s0 * u[0]; v1 = v1 * s1 * u[1]; v2 = v2 * s2 * u[2]; v3 = v3 * s3 * u[3];
+    }
 
     /* max |x| over the block; NaNs never win a '>' comparison in the
      * reference's scan, fmaxf drops them the same way */
@@ -332,6 +343,7 @@ k_get_rows(const uint8_t *__restrict__ w, uint32_t rows, uint32_t cols, uint32_t
 
 #include "gemv_kernels.inc"
 #include "mmq_kernels.inc"
+#include "moe_kernels.inc"
 
 /* ─── host side of layer 2 ────────────────────────────────────────────── */
 
@@ -451,7 +463,22 @@ extern "C" int oxh_quantize_q8_k(const float *d_x, size_t in_stride, size_t n_ve
     const uint32_t total = (uint32_t)(bpv * n_vec);
     hipLaunchKernelGGL(k_quantize_q8_k, dim3((total + 3u) / 4u), dim3(256), 0,
                        pick_stream(stream), d_x, in_stride, (uint32_t)bpv, total,
-                       (uint8_t *)d_act);
+                       (uint8_t *)d_act, (const uint32_t *)nullptr, (const float *)nullptr);
+    HIP_TRY(hipGetLastError());
+    return OXH_OK;
+}
+
+/* the gather / SwiGLU forms used by the mixture-of-experts layer */
+static int quantize_q8_k_ex(const float *d_x, size_t in_stride, size_t n_vec, size_t cols, void *d_act,
+                            const uint32_t *d_row_index, const float *d_up, void *stream)
+{
+    const size_t bpv = cols / OXH_QK_K;
+    if (n_vec == 0 || bpv == 0) return OXH_OK;
+    if (bpv > 0xFFFFFFFFull / n_vec) return arg_fail("moe: too many blocks");
+    const uint32_t total = (uint32_t)(bpv * n_vec);
+    hipLaunchKernelGGL(k_quantize_q8_k, dim3((total + 3u) / 4u), dim3(256), 0,
+                       pick_stream(stream), d_x, in_stride, (uint32_t)bpv, total,
+                       (uint8_t *)d_act, d_row_index, d_up);
     HIP_TRY(hipGetLastError());
     return OXH_OK;
 }
@@ -1050,6 +1077,179 @@ extern "C" int oxh_get_rows(uint32_t qtype, const void *d_w, size_t rows, size_t
     else if (qtype == OXH_Q6_K) OXH_GET_ROWS(2);
     else                        OXH_GET_ROWS(3);
 #undef OXH_GET_ROWS
+    HIP_TRY(hipGetLastError());
+    return OXH_OK;
+}
+
+/* ─── mixture of experts ──────────────────────────────────────────────── */
+
+static size_t align256(size_t v) { return (v + 255u) & ~(size_t)255u; }
+
+/* Workspace layout of oxh_moe_ffn (every part 256-byte aligned). */
+struct MoeLayout {
+    size_t ids, wts, slot_pos, perm, counts, offsets, act_x, gate, up, act_h, y, total;
+};
+
+static int moe_layout(const OxhMoe *m, size_t n_tok, MoeLayout *l)
+{
+    if (!m || m->n_expert == 0 || m->n_expert > OXH_MOE_MAX_EXPERTS / 2)
+        return arg_fail("moe: n_expert must be 1..16");
+    if (m->top_k == 0 || m->top_k > OXH_MOE_MAX_TOPK || m->top_k > m->n_expert)
+        return arg_fail("moe: top_k must be 1..8 and at most n_expert");
+    if (oxh_act_kind(m->qtype_gate_up, m->hidden) != 2 || oxh_act_kind(m->qtype_down, m->ffn) != 2) {
+        snprintf(g_err, sizeof g_err, "moe: expert matrices must be Q4_K, Q5_K or Q6_K with widths in whole "
+                 "256-blocks (types %u / %u, hidden %zu, ffn %zu)", m->qtype_gate_up, m->qtype_down, m->hidden, m->ffn);
+        return OXH_DECLINED;
+    }
+    if (n_tok == 0 || n_tok > 4096) return arg_fail("moe: n_tok must be 1..4096");
+    const size_t pairs = n_tok * m->top_k;
+    size_t at = 0;
+#define OXH_PART(FIELD, BYTES) l->FIELD = at; at = align256(at + (BYTES))
+    OXH_PART(ids, pairs * 4);
+    OXH_PART(wts, pairs * 4);
+    OXH_PART(slot_pos, pairs * 4);
+    OXH_PART(perm, pairs * 4);
+    OXH_PART(counts, OXH_MOE_MAX_EXPERTS * 4);
+    OXH_PART(offsets, (OXH_MOE_MAX_EXPERTS + 1) * 4);
+    OXH_PART(act_x, pairs * oxh_act_bytes(m->qtype_gate_up, m->hidden));
+    OXH_PART(gate, pairs * m->ffn * 4);
+    OXH_PART(up, pairs * m->ffn * 4);
+    OXH_PART(act_h, pairs * oxh_act_bytes(m->qtype_down, m->ffn));
+    OXH_PART(y, pairs * m->hidden * 4);
+#undef OXH_PART
+    l->total = at;
+    return OXH_OK;
+}
+
+extern "C" int oxh_moe_workspace_bytes(const OxhMoe *m, size_t n_tok, size_t *bytes)
+{
+    MoeLayout l;
+    const int rc = moe_layout(m, n_tok, &l);
+    if (rc) return rc;
+    if (bytes) *bytes = l.total;
+    return OXH_OK;
+}
+
+extern "C" int oxh_debug_moe_workspace_parts(const OxhMoe *m, size_t n_tok, size_t parts[12])
+{
+    MoeLayout l;
+    const int rc = moe_layout(m, n_tok, &l);
+    if (rc) return rc;
+    if (!parts) return arg_fail("oxh_debug_moe_workspace_parts: NULL pointer");
+    const size_t v[12] = { l.ids, l.wts, l.slot_pos, l.perm, l.counts, l.offsets, l.act_x, l.gate, l.up, l.act_h,
+                           l.y, l.total };
+    memcpy(parts, v, sizeof v);
+    return OXH_OK;
+}
+
+extern "C" int oxh_moe_route(const float *d_logits, size_t n_tok, size_t n_expert, size_t top_k, int renorm,
+                             int32_t *d_ids, float *d_weights, uint32_t *d_counts, uint32_t *d_offsets,
+                             uint32_t *d_perm, uint32_t *d_slot_pos, void *stream)
+{
+    int rc = ensure_init();
+    if (rc) return rc;
+    if (n_tok == 0) return OXH_OK;
+    if (!d_logits || !d_ids || !d_weights || !d_counts || !d_offsets || !d_perm || !d_slot_pos)
+        return arg_fail("oxh_moe_route: NULL pointer");
+    if (n_expert == 0 || n_expert > OXH_MOE_MAX_EXPERTS) return arg_fail("oxh_moe_route: n_expert must be 1..32");
+    if (top_k == 0 || top_k > OXH_MOE_MAX_TOPK || top_k > n_expert)
+        return arg_fail("oxh_moe_route: top_k must be 1..8 and at most n_expert");
+    if (n_tok > 4096) return arg_fail("oxh_moe_route: at most 4096 tokens per call");
+    /* a wave per token in the first phase, per expert in the second: up to 16 waves */
+    const size_t waves = n_tok > n_expert ? n_tok : n_expert;
+    const uint32_t threads = 64u * (uint32_t)(waves > 16 ? 16 : waves);
+    hipLaunchKernelGGL(k_moe_route, dim3(1), dim3(threads), 0, pick_stream(stream),
+                       d_logits, (uint32_t)n_tok, (uint32_t)n_expert, (uint32_t)top_k, renorm, d_ids, d_weights,
+                       d_counts, d_offsets, d_perm, d_slot_pos);
+    HIP_TRY(hipGetLastError());
+    return OXH_OK;
+}
+
+/* one launch of the MFMA tile kernel over all experts, activation runs from device memory */
+static int launch_experts(uint32_t qtype, const void *const *d_w, float *const *d_out, size_t n_mat,
+                          size_t n_expert, size_t rows, size_t cols, const void *d_acts, size_t out_stride,
+                          const uint32_t *d_counts, const uint32_t *d_offsets, void *stream)
+{
+    typedef MmqGeom<1, 1, 4> G;
+    const size_t blocks = cols / OXH_QK_K;
+    if (blocks * 292u * 256u > 0xFFFFFFFFull) return arg_fail("moe: cols too large");
+    const size_t rb = oxh_row_bytes(qtype, cols);
+    SegTable t;
+    memset(&t, 0, sizeof t);
+    uint32_t wg = 0, n = 0;
+    for (size_t mtx = 0; mtx < n_mat; mtx++)
+        for (size_t e = 0; e < n_expert; e++) {
+            t.s[n].w = (const uint8_t *)d_w[mtx] + e * rows * rb;
+            t.s[n].out = d_out[mtx];
+            t.s[n].rows = (uint32_t)rows;
+            t.s[n].act_first = (uint32_t)e;             /* the expert whose count and offset apply */
+            t.s[n].wg_begin = wg;
+            wg += (uint32_t)((rows + G::ROWS - 1) / G::ROWS);
+            n++;
+        }
+    t.n = n;
+    for (uint32_t i = 1; i < 4 && i < n; i++) t.bound[i - 1] = t.s[i].wg_begin;
+    const uint8_t *acts = (const uint8_t *)d_acts;
+    hipStream_t st = pick_stream(stream);
+    if (qtype == OXH_Q6_K) {
+        typedef Mmq6Geom<1, 1, 4> G6;
+        auto kernel = k_mmq_q6_k_experts<1, 1, 4>;
+        hipLaunchKernelGGL(kernel, dim3(wg), dim3(256), G6::LDS_BYTES, st, t, (uint32_t)blocks, acts, out_stride,
+                           d_counts, d_offsets);
+    } else if (is_q5k(qtype)) {
+        typedef MmqGeom<1, 1, 4, true> G5;
+        auto kernel = k_mmq_q45_k_experts<1, 1, 4, true>;
+        hipLaunchKernelGGL(kernel, dim3(wg), dim3(256), G5::LDS_BYTES, st, t, (uint32_t)blocks, acts, out_stride,
+                           d_counts, d_offsets);
+    } else {
+        auto kernel = k_mmq_q45_k_experts<1, 1, 4, false>;
+        hipLaunchKernelGGL(kernel, dim3(wg), dim3(256), G::LDS_BYTES, st, t, (uint32_t)blocks, acts, out_stride,
+                           d_counts, d_offsets);
+    }
+    HIP_TRY(hipGetLastError());
+    return OXH_OK;
+}
+
+extern "C" int oxh_moe_ffn(const OxhMoe *m, const float *d_logits, const float *d_x, size_t x_stride,
+                           size_t n_tok, float *d_out, size_t out_stride, void *d_workspace,
+                           size_t workspace_bytes, void *stream)
+{
+    int rc = ensure_init();
+    if (rc) return rc;
+    MoeLayout l;
+    if ((rc = moe_layout(m, n_tok, &l))) return rc;
+    if (!d_logits || !d_x || !d_out || !d_workspace || !m->d_w_gate || !m->d_w_up || !m->d_w_down)
+        return arg_fail("oxh_moe_ffn: NULL pointer");
+    if (workspace_bytes < l.total) return arg_fail("oxh_moe_ffn: workspace too small (see oxh_moe_workspace_bytes)");
+    if (x_stride < m->hidden || out_stride < m->hidden) return arg_fail("oxh_moe_ffn: stride < hidden");
+    if ((uintptr_t)d_workspace & 255u) return arg_fail("oxh_moe_ffn: workspace must be 256-byte aligned");
+    uint8_t *ws = (uint8_t *)d_workspace;
+    int32_t *ids = (int32_t *)(ws + l.ids);
+    float *wts = (float *)(ws + l.wts);
+    uint32_t *slot_pos = (uint32_t *)(ws + l.slot_pos), *perm = (uint32_t *)(ws + l.perm);
+    uint32_t *counts = (uint32_t *)(ws + l.counts), *offsets = (uint32_t *)(ws + l.offsets);
+    float *gate = (float *)(ws + l.gate), *up = (float *)(ws + l.up), *y = (float *)(ws + l.y);
+    const size_t pairs = n_tok * m->top_k;
+
+    /* 1. route and group; 2. gather + quantise each pair's token */
+    if ((rc = oxh_moe_route(d_logits, n_tok, m->n_expert, m->top_k, m->renorm, ids, wts, counts, offsets, perm,
+                            slot_pos, stream))) return rc;
+    if ((rc = quantize_q8_k_ex(d_x, x_stride, pairs, m->hidden, ws + l.act_x, perm, nullptr, stream))) return rc;
+    /* 3. gate and up of every expert over its own pairs */
+    const void *w_gu[2] = { m->d_w_gate, m->d_w_up };
+    float *o_gu[2] = { gate, up };
+    if ((rc = launch_experts(m->qtype_gate_up, w_gu, o_gu, 2, m->n_expert, m->ffn, m->hidden, ws + l.act_x,
+                             m->ffn, counts, offsets, stream))) return rc;
+    /* 4. h = silu(gate) * up, quantised; 5. down */
+    if ((rc = quantize_q8_k_ex(gate, m->ffn, pairs, m->ffn, ws + l.act_h, nullptr, up, stream))) return rc;
+    const void *w_dn[1] = { m->d_w_down };
+    float *o_dn[1] = { y };
+    if ((rc = launch_experts(m->qtype_down, w_dn, o_dn, 1, m->n_expert, m->hidden, m->ffn, ws + l.act_h,
+                             m->hidden, counts, offsets, stream))) return rc;
+    /* 6. combine in ascending expert order */
+    hipLaunchKernelGGL(k_moe_combine, dim3((uint32_t)((m->hidden + 255u) / 256u), (uint32_t)n_tok), dim3(256), 0,
+                       pick_stream(stream), (const float *)y, m->hidden, (const int32_t *)ids, (const float *)wts,
+                       (const uint32_t *)slot_pos, (uint32_t)m->top_k, (uint32_t)m->hidden, d_out, out_stride);
     HIP_TRY(hipGetLastError());
     return OXH_OK;
 }

@@ -184,6 +184,48 @@ def get_rows(qtype, d_w, rows, cols, d_ids, n_ids, d_out, out_stride, stream=Non
                              ctypes.c_void_p(d_out), out_stride, stream))
 
 
+def moe_route(d_logits, n_tok, n_expert, top_k, renorm, d_ids, d_wts, d_counts, d_offsets, d_perm, d_slot_pos,
+              stream=None):
+    vp = ctypes.c_void_p
+    check(lib().oxh_moe_route(vp(d_logits), n_tok, n_expert, top_k, int(renorm), vp(d_ids), vp(d_wts),
+                              vp(d_counts), vp(d_offsets), vp(d_perm), vp(d_slot_pos), stream))
+
+
+class MoeLayer:
+    """One mixture-of-experts feed-forward layer resident on the device
+    (routing, grouping, expert matrices and combination as
+    oxidize-c/src/model/llama.c:5965-6160); wraps oxh_moe_ffn and owns its
+    workspace, sized for `max_tok` tokens."""
+
+    PARTS = ("ids", "wts", "slot_pos", "perm", "counts", "offsets", "act_x", "gate", "up", "act_h", "y", "total")
+
+    def __init__(self, qtype_gate_up, qtype_down, d_w_gate, d_w_up, d_w_down, n_expert, top_k, hidden, ffn,
+                 renorm=True, max_tok=16):
+        self.desc = _lib.OxhMoe(qtype_gate_up, qtype_down, d_w_gate, d_w_up, d_w_down, n_expert, top_k, hidden,
+                                ffn, int(renorm))
+        self.n_expert, self.top_k, self.hidden, self.ffn, self.max_tok = n_expert, top_k, hidden, ffn, max_tok
+        need = ctypes.c_size_t()
+        status = lib().oxh_moe_workspace_bytes(ctypes.byref(self.desc), max_tok, ctypes.byref(need))
+        if status == DECLINED:
+            raise OxhError(status, lib().oxh_last_error().decode())
+        check(status)
+        self.workspace = DeviceBuffer(need.value)
+
+    def forward(self, d_logits, d_x, n_tok, d_out, x_stride=None, out_stride=None, stream=None):
+        if n_tok > self.max_tok:
+            raise ValueError("n_tok %d beyond the workspace's %d" % (n_tok, self.max_tok))
+        check(lib().oxh_moe_ffn(ctypes.byref(self.desc), ctypes.c_void_p(d_logits), ctypes.c_void_p(d_x),
+                                x_stride or self.hidden, n_tok, ctypes.c_void_p(d_out),
+                                out_stride or self.hidden, ctypes.c_void_p(self.workspace.ptr),
+                                self.workspace.nbytes, stream))
+
+    def parts(self, n_tok):
+        """Offsets of the intermediates inside the workspace (test hook)."""
+        v = (ctypes.c_size_t * 12)()
+        check(lib().oxh_debug_moe_workspace_parts(ctypes.byref(self.desc), n_tok, ctypes.byref(v)))
+        return dict(zip(self.PARTS, [int(x) for x in v]))
+
+
 def debug_subblock_sums(qtype, d_w, rows, cols, d_act, d_sums, stream=None):
     check(lib().oxh_debug_subblock_sums(qtype, ctypes.c_void_p(d_w), rows, cols,
                                         ctypes.c_void_p(d_act), ctypes.c_void_p(d_sums), stream))

@@ -58,6 +58,8 @@ def oracle():
         lib.oxo_matvec_batch_scratch_bytes.argtypes = [Z]
         lib.oxo_matvec_batch_scratch_bytes.restype = Z
         lib.oxo_moe_route.argtypes = [V, Z, Z, Z, ctypes.c_int, V, V]; lib.oxo_moe_route.restype = None
+        lib.oxo_moe_ffn.argtypes = [U32, U32, V, V, V, Z, Z, Z, Z, ctypes.c_int, V, V, Z, V]
+        lib.oxo_moe_ffn.restype = ctypes.c_int
         lib.oxo_dequant_row.argtypes = [U32, V, Z, V]; lib.oxo_dequant_row.restype = ctypes.c_int
         lib.oxo_rms_norm_f32.argtypes = [V, V, V, Z, F]; lib.oxo_rms_norm_f32.restype = None
         lib.oxo_swiglu_f32.argtypes = [V, V, V, Z]; lib.oxo_swiglu_f32.restype = None

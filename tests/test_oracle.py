@@ -598,6 +598,64 @@ def test_moe_route_brute_force():
         assert abs(wts[t].sum() - 1.0) < 1e-6
 
 
+def test_moe_route_ties_known_answers():
+    """Worked by hand from the swapping selection of llama.c:5998-6012: after
+    expert 3 wins the first round of [0, 0, 0, 5], the index list reads
+    [3, 1, 2, 0], so the equal rest is taken as 1, 2 (not 0, 1)."""
+    rows = np.array([[0, 0, 0, 5], [5, 0, 0, 0], [0, 5, 0, 0], [1, 1, 1, 1], [0, 2, 2, 0], [3, 0, 3, 0]], np.float32)
+    ids = np.zeros((6, 3), np.int32)
+    wts = np.zeros((6, 3), np.float32)
+    O.oxo_moe_route(rows.ctypes.data, 6, 4, 3, 0, ids.ctypes.data, wts.ctypes.data)
+    assert ids.tolist() == [[3, 1, 2], [0, 1, 2], [1, 0, 2], [0, 1, 2], [1, 2, 0], [0, 2, 1]]
+    assert np.allclose(wts[3], 0.25) and np.allclose(wts[0, 0], np.exp(5) / (np.exp(5) + 3), rtol=1e-6)
+
+
+def dequant_matrix(qt, w, rows, cols):
+    rb = synth.row_bytes(qt, cols)
+    out = np.zeros((rows, cols), np.float32)
+    for r in range(rows):
+        assert O.oxo_dequant_row(qt, w[r * rb:].ctypes.data, cols, out[r].ctypes.data) == 0
+    return out.astype(np.float64)
+
+
+@pytest.mark.parametrize("qt_gu,qt_dn,renorm", [(Q4K, Q6K, 1), (Q5K, Q4K, 0)])
+def test_moe_ffn_against_dense_restatement(qt_gu, qt_dn, renorm):
+    """The layer of oxidize-c/src/model/llama.c:5965-6160 written a second way:
+    double-precision dense products of the dequantised expert matrices, experts
+    picked by a stable sort.  Agreement is to the activation quantisation
+    (about 1 %), which is what a wrong expert index, a swapped gate/up, a
+    missing gate weight or a token gathered from the wrong row would exceed by
+    orders of magnitude."""
+    n_exp, k, hidden, ffn, n_tok = 4, 2, 256, 512, 7
+    rb_gu, rb_dn = synth.row_bytes(qt_gu, hidden), synth.row_bytes(qt_dn, ffn)
+    wg = synth.weights(qt_gu, n_exp * ffn, hidden, seed=5, stream=1)
+    wu = synth.weights(qt_gu, n_exp * ffn, hidden, seed=5, stream=2)
+    wd = synth.weights(qt_dn, n_exp * hidden, ffn, seed=5, stream=3)
+    logits = synth.normal(n_tok * n_exp, seed=5, stream=4).reshape(n_tok, n_exp)
+    logits[:, 3] = -30.0                                   # an expert nobody selects
+    x = synth.normal(n_tok * hidden, seed=5, stream=5).reshape(n_tok, hidden)
+    out = np.full((n_tok, hidden), np.nan, np.float32)
+    assert O.oxo_moe_ffn(qt_gu, qt_dn, wg.ctypes.data, wu.ctypes.data, wd.ctypes.data, n_exp, k, hidden, ffn,
+                         renorm, logits.ctypes.data, x.ctypes.data, n_tok, out.ctypes.data) == 0
+    G, U, D = (dequant_matrix(qt_gu, wg, n_exp * ffn, hidden), dequant_matrix(qt_gu, wu, n_exp * ffn, hidden),
+               dequant_matrix(qt_dn, wd, n_exp * hidden, ffn))
+    want = np.zeros((n_tok, hidden))
+    for t in range(n_tok):
+        p = np.exp(logits[t].astype(np.float64) - logits[t].max())
+        p /= p.sum()
+        sel = np.argsort(-logits[t], kind="stable")[:k]
+        assert 3 not in sel
+        gw = p[sel] / p[sel].sum() if renorm else p[sel]
+        for e, w in zip(sel, gw):
+            g = G[e * ffn:(e + 1) * ffn] @ x[t]
+            u = U[e * ffn:(e + 1) * ffn] @ x[t]
+            with np.errstate(over="ignore"):
+                h = g / (1.0 + np.exp(-g)) * u
+            want[t] += w * (D[e * hidden:(e + 1) * hidden] @ h)
+    scale = np.abs(want).max()
+    assert np.abs(out - want).max() < 0.03 * scale
+
+
 @pytest.mark.skipif(oxlibs.ref() is None, reason="compiled reference not present")
 def test_oracle_vs_live_reference_many_rows():
     ref = oxlibs.ref()
