@@ -557,6 +557,8 @@ static hipError_t raise_all_lds_ceilings(void)
     if ((e = raise_lds_ceiling(k_mmq_q5_k<4, 1, 8>)) != hipSuccess) return e;
     if ((e = raise_lds_ceiling(k_mmq_q6_k<8, 1, 8>)) != hipSuccess) return e;
     if ((e = raise_lds_ceiling(k_mmq_q6_k<4, 1, 8>)) != hipSuccess) return e;
+    if ((e = raise_lds_ceiling(k_mmq_q6_k_segments<1, 1, 4, 2>)) != hipSuccess) return e;
+    if ((e = raise_lds_ceiling(k_mmq_q6_k_experts<1, 1, 4, 2>)) != hipSuccess) return e;
     return hipSuccess;
 }
 
@@ -645,6 +647,16 @@ static bool gemv_wants_mfma(uint32_t qtype, const GemvIo &io, size_t max_nv, con
     return io.d_acts != nullptr || io.d_act_out != nullptr;
 }
 
+/* The 64-row MFMA tile keeps one super-block per wave on its way; a launch with
+ * at most two workgroups per CU cannot fill the memory system like that and
+ * takes the variant with two super-blocks per stage (twice the LDS). */
+static bool mmq_deep_stages(uint32_t wg)
+{
+    static const uint32_t force = env_u32("OXH_MMQ_DEEP", 2, 0, 2);     /* 0 never, 1 always, 2 by launch size */
+    if (force < 2u) return force == 1u;
+    return wg <= 2u * (uint32_t)(g_n_cu > 0 ? g_n_cu : 256);
+}
+
 static int launch_mmq_segments(uint32_t qtype, const OxhSegment *segs, size_t n_segs, size_t cols, size_t blocks,
                                const GemvIo &io, size_t n_vec_default, size_t n_acts,
                                size_t out_stride, void *stream)
@@ -673,23 +685,23 @@ static int launch_mmq_segments(uint32_t qtype, const OxhSegment *segs, size_t n_
     }
     t.n = n;
     for (uint32_t i = 1; i < 4 && i < n; i++) t.bound[i - 1] = t.s[i].wg_begin;
-    if (qtype == OXH_Q6_K) {
-        typedef Mmq6Geom<1, 1, 4> G6;                       /* same 64-row tiles */
-        static_assert(G6::ROWS == G::ROWS, "segment tiling is shared by both formats");
-        auto kernel = k_mmq_q6_k_segments<1, 1, 4>;
-        hipLaunchKernelGGL(kernel, dim3(wg), dim3(4 * 64), G6::LDS_BYTES,
-                           pick_stream(stream), t, (uint32_t)blocks, acts, out_stride);
-    } else if (is_q5k(qtype)) {
-        typedef MmqGeom<1, 1, 4, true> G5;
-        static_assert(G5::ROWS == G::ROWS, "segment tiling is shared by all formats");
-        auto kernel = k_mmq_q5_k_segments<1, 1, 4>;
-        hipLaunchKernelGGL(kernel, dim3(wg), dim3(4 * 64), G5::LDS_BYTES,
-                           pick_stream(stream), t, (uint32_t)blocks, acts, out_stride);
+    typedef Mmq6Geom<1, 1, 4> G6;                           /* same 64-row tiles */
+    typedef MmqGeom<1, 1, 4, true> G5;
+    static_assert(G6::ROWS == G::ROWS && G5::ROWS == G::ROWS, "segment tiling is shared by all formats");
+    hipStream_t st = pick_stream(stream);
+    const uint32_t nb = (uint32_t)blocks;
+#define OXH_SEG_LAUNCH(KERNEL, GEOM, KB)                                                              \
+    hipLaunchKernelGGL((KERNEL<1, 1, 4, KB>), dim3(wg), dim3(4 * 64), (KB) * GEOM::LDS_BYTES, st, t, nb, acts, out_stride)
+    if (mmq_deep_stages(wg)) {
+        if (qtype == OXH_Q6_K) OXH_SEG_LAUNCH(k_mmq_q6_k_segments, G6, 2);
+        else if (is_q5k(qtype)) OXH_SEG_LAUNCH(k_mmq_q5_k_segments, G5, 2);
+        else OXH_SEG_LAUNCH(k_mmq_q4_k_segments, G, 2);
     } else {
-        auto kernel = k_mmq_q4_k_segments<1, 1, 4>;
-        hipLaunchKernelGGL(kernel, dim3(wg), dim3(4 * 64), G::LDS_BYTES,
-                           pick_stream(stream), t, (uint32_t)blocks, acts, out_stride);
+        if (qtype == OXH_Q6_K) OXH_SEG_LAUNCH(k_mmq_q6_k_segments, G6, 1);
+        else if (is_q5k(qtype)) OXH_SEG_LAUNCH(k_mmq_q5_k_segments, G5, 1);
+        else OXH_SEG_LAUNCH(k_mmq_q4_k_segments, G, 1);
     }
+#undef OXH_SEG_LAUNCH
     HIP_TRY(hipGetLastError());
     return OXH_OK;
 }
@@ -1191,21 +1203,22 @@ static int launch_experts(uint32_t qtype, const void *const *d_w, float *const *
     for (uint32_t i = 1; i < 4 && i < n; i++) t.bound[i - 1] = t.s[i].wg_begin;
     const uint8_t *acts = (const uint8_t *)d_acts;
     hipStream_t st = pick_stream(stream);
-    if (qtype == OXH_Q6_K) {
-        typedef Mmq6Geom<1, 1, 4> G6;
-        auto kernel = k_mmq_q6_k_experts<1, 1, 4>;
-        hipLaunchKernelGGL(kernel, dim3(wg), dim3(256), G6::LDS_BYTES, st, t, (uint32_t)blocks, acts, out_stride,
-                           d_counts, d_offsets);
-    } else if (is_q5k(qtype)) {
-        typedef MmqGeom<1, 1, 4, true> G5;
-        auto kernel = k_mmq_q45_k_experts<1, 1, 4, true>;
-        hipLaunchKernelGGL(kernel, dim3(wg), dim3(256), G5::LDS_BYTES, st, t, (uint32_t)blocks, acts, out_stride,
-                           d_counts, d_offsets);
+    typedef Mmq6Geom<1, 1, 4> G6;
+    typedef MmqGeom<1, 1, 4, true> G5;
+    const uint32_t nb = (uint32_t)blocks;
+#define OXH_EXP_LAUNCH(KERNEL, GEOM, KB)                                                              \
+    hipLaunchKernelGGL(KERNEL, dim3(wg), dim3(256), (KB) * GEOM::LDS_BYTES, st, t, nb, acts, out_stride, \
+                       d_counts, d_offsets)
+    if (mmq_deep_stages(wg)) {
+        if (qtype == OXH_Q6_K) OXH_EXP_LAUNCH((k_mmq_q6_k_experts<1, 1, 4, 2>), G6, 2);
+        else if (is_q5k(qtype)) OXH_EXP_LAUNCH((k_mmq_q45_k_experts<1, 1, 4, true, 2>), G5, 2);
+        else OXH_EXP_LAUNCH((k_mmq_q45_k_experts<1, 1, 4, false, 2>), G, 2);
     } else {
-        auto kernel = k_mmq_q45_k_experts<1, 1, 4, false>;
-        hipLaunchKernelGGL(kernel, dim3(wg), dim3(256), G::LDS_BYTES, st, t, (uint32_t)blocks, acts, out_stride,
-                           d_counts, d_offsets);
+        if (qtype == OXH_Q6_K) OXH_EXP_LAUNCH((k_mmq_q6_k_experts<1, 1, 4, 1>), G6, 1);
+        else if (is_q5k(qtype)) OXH_EXP_LAUNCH((k_mmq_q45_k_experts<1, 1, 4, true, 1>), G5, 1);
+        else OXH_EXP_LAUNCH((k_mmq_q45_k_experts<1, 1, 4, false, 1>), G, 1);
     }
+#undef OXH_EXP_LAUNCH
     HIP_TRY(hipGetLastError());
     return OXH_OK;
 }
