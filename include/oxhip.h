@@ -201,7 +201,8 @@ int oxh_mmq(uint32_t qtype, const void *d_w, size_t rows, size_t cols,
  * to oc_quant_dequant_row, oxidize-c/src/compute/quantization.c:2781-2795), so
  * the token-embedding table stays quantized in HBM and the ids never leave
  * the device.  Replaces oc_cuda_mmq_get_row / _get_row_dev / _get_row_batch
- * (oxidize-c/include/oxidize/cuda_mmq.h:74-93).  Q4_K, Q5_K, Q6_K and Q8_0;
+ * (oxidize-c/include/oxidize/cuda_mmq.h:74-93).  Every type the matvec entry
+ * points take (Q4_K, Q5_K, Q6_K, Q8_0, Q4_0, Q4_1, Q5_0, Q5_1);
  * d_ids is device memory (at most 65535 per call); an id >= rows gives a row
  * of zeros; d_out and out_stride*4 must be multiples of 16 bytes. */
 int oxh_get_rows(uint32_t qtype, const void *d_w, size_t rows, size_t cols,

@@ -637,10 +637,28 @@ int oxo_dequant_row(uint32_t qtype, const uint8_t *row, size_t cols, float *out)
 {
     const int kind = oxo_act_kind(qtype, cols);
     if (!kind) return 1;
-    if (qtype == OXO_Q4_0 || qtype == OXO_Q4_1 || qtype == OXO_Q5_0 || qtype == OXO_Q5_1) return 1;
     const size_t blocks = n_blocks(kind, cols);
     for (size_t b = 0; b < blocks; b++) {
-        if (qtype == OXO_Q8_0) {
+        if (qtype == OXO_Q4_0 || qtype == OXO_Q4_1 || qtype == OXO_Q5_0 || qtype == OXO_Q5_1) {
+            /* src/compute/quantization.c:386-474: value i is the low nibble of
+             * byte i, value i + 16 the high nibble; fifth bit e of the 32-bit
+             * word belongs to value e */
+            const int has_m = qtype == OXO_Q4_1 || qtype == OXO_Q5_1;
+            const int has_h = qtype == OXO_Q5_0 || qtype == OXO_Q5_1;
+            const uint8_t *w = row + b * block_bytes(qtype);
+            const float d = oxo_f16_to_f32(rd_u16(w));
+            const float m = has_m ? oxo_f16_to_f32(rd_u16(w + 2)) : 0.0f;
+            const uint8_t *qh = w + (has_m ? 4 : 2);
+            const uint8_t *qs = qh + (has_h ? 4 : 0);
+            const uint32_t bits = has_h ? ((uint32_t)qh[0] | ((uint32_t)qh[1] << 8) |
+                                           ((uint32_t)qh[2] << 16) | ((uint32_t)qh[3] << 24)) : 0u;
+            for (unsigned e = 0; e < 32; e++) {
+                const unsigned nib = e < 16 ? (qs[e] & 15u) : (unsigned)(qs[e - 16] >> 4);
+                const unsigned code = nib | (((bits >> e) & 1u) << 4);
+                if (has_m) out[32 * b + e] = (float)code * d + m;
+                else       out[32 * b + e] = (float)((int)code - (has_h ? 16 : 8)) * d;
+            }
+        } else if (qtype == OXO_Q8_0) {
             const uint8_t *w = row + b * OXO_Q8_0_BYTES;
             const float d = oxo_f16_to_f32(rd_u16(w));
             for (int i = 0; i < 32; i++)

@@ -279,7 +279,7 @@ k_quantize_q8_0(const float *__restrict__ x, size_t in_stride, uint32_t blocks_p
  * the bit.  One wave per 256 values, lane l producing values 4l .. 4l+3 (they
  * share a sub-block / scale group); grid.y walks the ids.  An id beyond the
  * matrix yields a row of zeros rather than a read outside it.
- * KIND: 0 Q4_K, 1 Q5_K, 2 Q6_K, 3 Q8_0. */
+ * KIND: 0 Q4_K, 1 Q5_K, 2 Q6_K, 3 Q8_0, 4 Q4_0, 5 Q4_1, 6 Q5_0, 7 Q5_1. */
 template <int KIND>
 __global__ __launch_bounds__(256) void
 k_get_rows(const uint8_t *__restrict__ w, uint32_t rows, uint32_t cols, uint32_t row_bytes,
@@ -294,7 +294,24 @@ k_get_rows(const uint8_t *__restrict__ w, uint32_t rows, uint32_t cols, uint32_t
     float v[4] = { 0.0f, 0.0f, 0.0f, 0.0f };
     if (id < rows) {
         const uint8_t *row = w + (size_t)id * row_bytes;
-        if (KIND == 3) {
+        if (KIND >= 4) {
+            /* 32-value blocks [f16 d][f16 m: Q4_1, Q5_1][4 B fifth bits: Q5_0, Q5_1][16 B nibbles]; value i
+             * is the low nibble of byte i, value i + 16 the high nibble (quantization.c:386-474) */
+            const bool has_m = KIND == 5 || KIND == 7, has_h = KIND >= 6;
+            const uint32_t qh_at = has_m ? 4u : 2u, qs_at = qh_at + (has_h ? 4u : 0u);
+            const uint8_t *blk = row + (size_t)(e0 >> 5) * (qs_at + 16u);
+            const uint32_t i0 = e0 & 31u;
+            const float d = half_to_float_hw(*reinterpret_cast<const uint16_t *>(blk));
+            const float m = has_m ? half_to_float_hw(*reinterpret_cast<const uint16_t *>(blk + 2u)) : 0.0f;
+            const uint32_t q = reinterpret_cast<const U32u2 *>(blk + qs_at + (i0 & 15u))->v >> (i0 & 16u ? 4u : 0u);
+            const uint32_t h = has_h ? reinterpret_cast<const U32u2 *>(blk + qh_at)->v >> i0 : 0u;
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const uint32_t code = ((q >> (8 * i)) & 15u) | (((h >> i) & 1u) << 4);
+                if (has_m) v[i] = (float)code * d + m;
+                else v[i] = (float)((int)code - (has_h ? 16 : 8)) * d;
+            }
+        } else if (KIND == 3) {
             const uint8_t *blk = row + (size_t)(e0 >> 5) * 34u;
             const float d = half_to_float_hw(*reinterpret_cast<const uint16_t *>(blk));
             const uint32_t q = reinterpret_cast<const U32u2 *>(blk + 2u + (e0 & 31u))->v;
@@ -1067,8 +1084,7 @@ extern "C" int oxh_get_rows(uint32_t qtype, const void *d_w, size_t rows, size_t
     if (rc) return rc;
     if (n_ids == 0) return OXH_OK;
     if (!d_w || !d_ids || !d_out) return arg_fail("oxh_get_rows: NULL pointer");
-    const bool known = is_q4k(qtype) || is_q5k(qtype) || qtype == OXH_Q6_K || qtype == OXH_Q8_0;
-    const size_t rb = known ? oxh_row_bytes(qtype, cols) : 0;
+    const size_t rb = oxh_act_kind(qtype, cols) ? oxh_row_bytes(qtype, cols) : 0;   /* every type with a matvec kernel */
     if (rb == 0) {
         snprintf(g_err, sizeof g_err, "oxh_get_rows: qtype %u with cols %zu has no kernel here", qtype, cols);
         return OXH_DECLINED;
@@ -1087,6 +1103,10 @@ extern "C" int oxh_get_rows(uint32_t qtype, const void *d_w, size_t rows, size_t
     if (is_q4k(qtype))          OXH_GET_ROWS(0);
     else if (is_q5k(qtype))     OXH_GET_ROWS(1);
     else if (qtype == OXH_Q6_K) OXH_GET_ROWS(2);
+    else if (qtype == OXH_Q4_0) OXH_GET_ROWS(4);
+    else if (qtype == OXH_Q4_1) OXH_GET_ROWS(5);
+    else if (qtype == OXH_Q5_0) OXH_GET_ROWS(6);
+    else if (qtype == OXH_Q5_1) OXH_GET_ROWS(7);
     else                        OXH_GET_ROWS(3);
 #undef OXH_GET_ROWS
     HIP_TRY(hipGetLastError());

@@ -153,7 +153,8 @@ def dequant_rows(ref):
     """dequant_rows.npz: rows of every type the embedding lookup handles,
     expanded by the compiled reference (oc_quant_dequant_row)."""
     out = {}
-    for name, qt, cols in (("q4_k", 13, 768), ("q5_k", 15, 768), ("q6_k", 16, 768), ("q8_0", 7, 160)):
+    for name, qt, cols in (("q4_k", 13, 768), ("q5_k", 15, 768), ("q6_k", 16, 768), ("q8_0", 7, 160),
+                           ("q4_0", 3, 160), ("q4_1", 4, 160), ("q5_0", 5, 160), ("q5_1", 6, 160)):
         rows = 3
         rb = synth.row_bytes(qt, cols)
         w = synth.weights(qt, rows, cols, seed=17, stream=qt)

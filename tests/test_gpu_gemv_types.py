@@ -340,7 +340,8 @@ def test_prequantised_and_fused_paths_agree(oxh, qtype, rows, cols, n_vec):
 
 
 @pytest.mark.parametrize("qtype,rows,cols", [(Q4K, 1000, 4096), (15, 300, 1024), (Q6K, 500, 2816), (Q80, 2000, 896),
-                                             (Q80, 64, 32), (Q4K, 7, 256)])
+                                             (Q80, 64, 32), (Q4K, 7, 256), (3, 300, 896), (4, 300, 896),
+                                             (5, 300, 896), (6, 300, 896), (5, 9, 32), (6, 9, 1056)])
 def test_embedding_rows_bit_identical_to_the_cpu_dequantisation(oxh, qtype, rows, cols):
     """oxh_get_rows against the oracle's dequantisation (itself bit-identical
     to the compiled reference's oc_quant_dequant_row): ids on the device, first

@@ -474,7 +474,8 @@ def test_swiglu_vs_reference_goldens_and_double_precision():
     assert out[0] == 100.0 and abs(out[1]) < 1e-18
 
 
-@pytest.mark.parametrize("name,qt", [("q4_k", Q4K), ("q5_k", Q5K), ("q6_k", Q6K), ("q8_0", Q80)])
+@pytest.mark.parametrize("name,qt", [("q4_k", Q4K), ("q5_k", Q5K), ("q6_k", Q6K), ("q8_0", Q80), ("q4_0", 3),
+                                     ("q4_1", 4), ("q5_0", 5), ("q5_1", 6)])
 def test_dequant_row_bits_vs_reference(name, qt):
     """oxo_dequant_row is the checker of the embedding lookup: bit-identical to
     the compiled reference's oc_quant_dequant_row on the committed vectors, and
@@ -488,7 +489,7 @@ def test_dequant_row_bits_vs_reference(name, qt):
         assert np.array_equal(out.view(np.uint32), g[name + "_bits"][r])
     ref = oxlibs.ref()
     if ref is not None:
-        cols = 2048 if qt != Q80 else 896
+        cols = 2048 if qt in (Q4K, Q5K, Q6K) else 896
         rb = synth.row_bytes(qt, cols)
         w = synth.weights(qt, 5, cols, seed=19, stream=qt)
         for r in range(5):
