@@ -63,6 +63,12 @@ def chain_figure(mv, ds, steps):
                     "output so that every launch depends on the previous one"}
 
 
+def _lib_check_memset(buf):
+    import ctypes
+    from oxidize_amd import _lib
+    _lib.check(_lib.lib().oxh_memset(ctypes.c_void_p(buf.ptr), 0x5A, buf.nbytes, None))
+
+
 def secondary_figures(mv, synth):
     """The other benchmark configurations, measured the same way (inputs
     resident, HIP events on the launch stream).  Reported next to the headline
@@ -192,6 +198,26 @@ def secondary_figures(mv, synth):
     out["q8_0_lm_head_151936x896"] = q8
     for c in copies:
         c.free()
+    # What a kernel that only reads reaches on buffers the size of the decode set's matrices (launch
+    # cost included; twelve distinct buffers in turn, 793 MB, so that nothing comes from the last-level
+    # cache; one graph of twelve launches per replay): the ceiling the GEMV figures stand against here.
+    ceiling = {}
+    probe = [mv.DeviceBuffer(66060288) for _ in range(12)]
+    for b in probe:
+        _lib_check_memset(b)
+    for name, nbytes in (("gate_up_66MB", 66060288), ("down_q6k_48MB", 48168960), ("qkv_14MB", 14155776),
+                         ("o_9MB", 9437184)):
+        graph = mv.Graph()                      # replayed as a graph, like the decode set
+        with graph:
+            for b in probe:
+                mv.read_probe(b.ptr, nbytes)
+        us = timed(graph.launch, 8, mv) / len(probe)
+        graph.destroy()
+        ceiling[name] = {"us": round(us, 2), "gbps": round(nbytes / us / 1e3, 1),
+                         "frac_of_hbm_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBPS, 4)}
+    for b in probe:
+        b.free()
+    out["read_only_kernel_ceiling"] = ceiling
     # Mixtral-shaped expert GEMVs (configuration 4)
     ms = MoESet(seed=0)
     us = timed(ms.launch_step, 10, mv)

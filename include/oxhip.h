@@ -54,6 +54,9 @@ extern "C" {
 #define OXH_Q5_K_S 14u
 #define OXH_Q5_K_M 15u
 #define OXH_Q6_K   16u
+#define OXH_AL5    17u     /* the Q4_0 block layout under its own id (quantization.c:207-214) */
+#define OXH_AL6    19u     /* the Q5_0 layout */
+#define OXH_AL8    20u     /* the Q8_0 layout */
 #define OXH_QTYPE_UNKNOWN 0xffffffffu
 
 /* Block geometry (oxidize-c/include/oxidize/oxk.h:46-66). */
@@ -254,6 +257,13 @@ int oxh_moe_route(const float *d_logits, size_t n_tok, size_t n_expert, size_t t
  * (f32 [pair][hidden]), and the total size.  After a call the parity tests read
  * every intermediate from there. */
 int oxh_debug_moe_workspace_parts(const OxhMoe *m, size_t n_tok, size_t parts[12]);
+
+/* Measurement aid: one launch that only reads `bytes` of device memory (a
+ * workgroup per CU, 16-byte loads, nothing computed); d_sink may be NULL.
+ * Timed on a buffer the size of a weight matrix it gives the ceiling any
+ * kernel streaming that matrix once can reach on the device, launch cost
+ * included.  No counterpart in the reference. */
+int oxh_debug_read_probe(const void *d_buf, size_t bytes, uint32_t *d_sink, void *stream);
 
 /* Test hook: the integer sub-block sums the GEMV kernel forms, written by the
  * same device code path.  Q4_K and Q5_K: 8 int32 per super-block (S_j), Q6_K: 16 per

@@ -406,10 +406,13 @@ float oxo_dot_q5_1_q8_0(const uint8_t *row, size_t blocks, const uint8_t *act, i
 static size_t block_bytes(uint32_t qtype)
 {
     switch (qtype) {
+    case OXO_AL5:
     case OXO_Q4_0:   return 18u;
     case OXO_Q4_1:   return 20u;
+    case OXO_AL6:
     case OXO_Q5_0:   return 22u;
     case OXO_Q5_1:   return 24u;
+    case OXO_AL8:
     case OXO_Q8_0:   return OXO_Q8_0_BYTES;
     case OXO_Q4_K_S:
     case OXO_Q4_K_M: return OXO_Q4_K_BYTES;
@@ -424,10 +427,13 @@ int oxo_act_kind(uint32_t qtype, size_t cols)
 {
     switch (qtype) {
     case OXO_Q4_0:
+    case OXO_AL5:
     case OXO_Q4_1:
     case OXO_Q5_0:
+    case OXO_AL6:
     case OXO_Q5_1:
-    case OXO_Q8_0:   return (cols % OXO_QK8_0 == 0) ? 1 : 0;
+    case OXO_Q8_0:
+    case OXO_AL8:    return (cols % OXO_QK8_0 == 0) ? 1 : 0;
     case OXO_Q4_K_S:
     case OXO_Q4_K_M:
     case OXO_Q5_K_S:
@@ -453,10 +459,14 @@ static float row_dot(uint32_t qtype, const uint8_t *row, size_t blocks,
                      const uint8_t *act)
 {
     switch (qtype) {
+    /* AL5 / AL6 / AL8: the Q4_0 / Q5_0 / Q8_0 dots (src/compute/matvec.c:323-329) */
+    case OXO_AL5:
     case OXO_Q4_0:   return oxo_dot_q4_0_q8_0(row, blocks, act, NULL);
     case OXO_Q4_1:   return oxo_dot_q4_1_q8_0(row, blocks, act, NULL);
+    case OXO_AL6:
     case OXO_Q5_0:   return oxo_dot_q5_0_q8_0(row, blocks, act, NULL);
     case OXO_Q5_1:   return oxo_dot_q5_1_q8_0(row, blocks, act, NULL);
+    case OXO_AL8:
     case OXO_Q8_0:   return oxo_dot_q8_0_q8_0(row, blocks, act, NULL);
     case OXO_Q6_K:   return oxo_dot_q6_k_q8_k(row, blocks, act, NULL);
     case OXO_Q5_K_S:
@@ -635,6 +645,9 @@ void oxo_swiglu_f32(const float *gate, const float *up, float *out, size_t n)
 
 int oxo_dequant_row(uint32_t qtype, const uint8_t *row, size_t cols, float *out)
 {
+    if (qtype == OXO_AL5) qtype = OXO_Q4_0;     /* src/compute/quantization.c:781-800 */
+    if (qtype == OXO_AL6) qtype = OXO_Q5_0;
+    if (qtype == OXO_AL8) qtype = OXO_Q8_0;
     const int kind = oxo_act_kind(qtype, cols);
     if (!kind) return 1;
     const size_t blocks = n_blocks(kind, cols);

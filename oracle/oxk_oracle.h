@@ -56,6 +56,9 @@ enum {
     OXO_Q5_K_S = 14,
     OXO_Q5_K_M = 15,
     OXO_Q6_K   = 16,
+    OXO_AL5    = 17,    /* Q4_0 layout */
+    OXO_AL6    = 19,    /* Q5_0 layout */
+    OXO_AL8    = 20,    /* Q8_0 layout */
 };
 
 #define OXO_QK_K        256u

@@ -89,6 +89,10 @@ static const TypeRow k_types[] = {
     { 26, 33, 1, 4 },      /* I32 */
     { 27, 34, 1, 8 },      /* I64 */
     { 28, 35, 1, 8 },      /* F64 */
+    { 240, OXH_AL5, 32, 18 },
+    { 241, OXH_AL8, 32, 34 },
+    { 242, OXH_AL6, 32, 22 },
+    { 243, 18, 32, 14 },   /* AL5_XS */
 };
 
 static const TypeRow *type_row(uint32_t ggml_id)

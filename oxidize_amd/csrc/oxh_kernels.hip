@@ -358,6 +358,29 @@ k_get_rows(const uint8_t *__restrict__ w, uint32_t rows, uint32_t cols, uint32_t
     *reinterpret_cast<float4 *>(dst) = make_float4(v[0], v[1], v[2], v[3]);
 }
 
+/* Measurement aid: a kernel that only reads.  Each workgroup streams one
+ * contiguous share of the buffer with 16-byte loads, four in flight per lane,
+ * and folds the data into a value that is stored only if it matches a constant
+ * (so the loads cannot be dropped).  What it reaches on a buffer is the rate
+ * no GEMV over the same bytes can exceed on this device. */
+__global__ __launch_bounds__(1024) void
+k_read_probe(const u32x4 *__restrict__ p, size_t n16, uint32_t *__restrict__ sink)
+{
+    const size_t per = (n16 + gridDim.x - 1) / gridDim.x;
+    const size_t b = (size_t)blockIdx.x * per, e = b + per < n16 ? b + per : n16;
+    u32x4 acc = { 0u, 0u, 0u, 0u };
+    size_t i = b + threadIdx.x;
+    for (; i + 3u * blockDim.x < e; i += 4u * blockDim.x) {
+        u32x4 v[4];
+#pragma unroll
+        for (int k = 0; k < 4; k++) v[k] = __builtin_nontemporal_load(p + i + (size_t)k * blockDim.x);
+#pragma unroll
+        for (int k = 0; k < 4; k++) acc ^= v[k];
+    }
+    for (; i < e; i += blockDim.x) acc ^= p[i];
+    if ((acc.x ^ acc.y ^ acc.z ^ acc.w) == 0x5EED5EEDu && sink) *sink = 1u;
+}
+
 #include "gemv_kernels.inc"
 #include "mmq_kernels.inc"
 #include "moe_kernels.inc"
@@ -415,9 +438,22 @@ static hipStream_t pick_stream(void *stream)
 
 extern "C" void *oxh_internal_stream(void) { return (void *)g_stream; }
 
-extern "C" int oxh_act_kind(uint32_t qtype, size_t cols)
+/* AL5, AL6 and AL8 are the Q4_0, Q5_0 and Q8_0 block layouts under ids of
+ * their own (oxidize-c/src/compute/quantization.c:207-214; the encoder
+ * differs, the bytes and the dot do not: matvec.c:323-329). */
+static uint32_t canon_qtype(uint32_t qtype)
 {
     switch (qtype) {
+    case OXH_AL5: return OXH_Q4_0;
+    case OXH_AL6: return OXH_Q5_0;
+    case OXH_AL8: return OXH_Q8_0;
+    default:      return qtype;
+    }
+}
+
+extern "C" int oxh_act_kind(uint32_t qtype, size_t cols)
+{
+    switch (canon_qtype(qtype)) {
     case OXH_Q4_0:
     case OXH_Q4_1:
     case OXH_Q5_0:
@@ -434,7 +470,7 @@ extern "C" int oxh_act_kind(uint32_t qtype, size_t cols)
 
 static size_t block_bytes(uint32_t qtype)
 {
-    switch (qtype) {
+    switch (canon_qtype(qtype)) {
     case OXH_Q4_0:   return OXH_Q4_0_BYTES;
     case OXH_Q4_1:   return OXH_Q4_1_BYTES;
     case OXH_Q5_0:   return OXH_Q5_0_BYTES;
@@ -729,6 +765,7 @@ static int launch_gemv(uint32_t qtype, const OxhSegment *segs, size_t n_segs, si
 {
     int rc = ensure_init();
     if (rc) return rc;
+    qtype = canon_qtype(qtype);
     if (n_segs == 0) return OXH_OK;
     if (!segs || (!io.d_acts && !io.d_x)) return arg_fail("gemv: NULL pointer");
     if (n_vec < 1 || n_vec > OXH_MAX_NV) return arg_fail("gemv: n_vec must be 1..8");
@@ -956,6 +993,18 @@ extern "C" int oxh_gemv_segments_fused(uint32_t qtype, const OxhSegment *segs, s
     return launch_gemv(qtype, segs, n_segs, cols, io, n_vec, out_stride, nullptr, stream);
 }
 
+extern "C" int oxh_debug_read_probe(const void *d_buf, size_t bytes, uint32_t *d_sink, void *stream)
+{
+    int rc = ensure_init();
+    if (rc) return rc;
+    if (!d_buf || ((uintptr_t)d_buf & 15u)) return arg_fail("oxh_debug_read_probe: buffer must be 16-byte aligned");
+    if (bytes < 16) return OXH_OK;
+    hipLaunchKernelGGL(k_read_probe, dim3((uint32_t)(g_n_cu > 0 ? g_n_cu : 256)), dim3(1024), 0, pick_stream(stream),
+                       (const u32x4 *)d_buf, bytes / 16u, d_sink);
+    HIP_TRY(hipGetLastError());
+    return OXH_OK;
+}
+
 extern "C" int oxh_debug_subblock_sums(uint32_t qtype, const void *d_w, size_t rows,
                                        size_t cols, const void *d_act, int32_t *d_sums,
                                        void *stream)
@@ -1082,6 +1131,7 @@ extern "C" int oxh_get_rows(uint32_t qtype, const void *d_w, size_t rows, size_t
 {
     int rc = ensure_init();
     if (rc) return rc;
+    qtype = canon_qtype(qtype);
     if (n_ids == 0) return OXH_OK;
     if (!d_w || !d_ids || !d_out) return arg_fail("oxh_get_rows: NULL pointer");
     const size_t rb = oxh_act_kind(qtype, cols) ? oxh_row_bytes(qtype, cols) : 0;   /* every type with a matvec kernel */

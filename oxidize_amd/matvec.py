@@ -226,6 +226,11 @@ class MoeLayer:
         return dict(zip(self.PARTS, [int(x) for x in v]))
 
 
+def read_probe(d_buf, nbytes, stream=None):
+    """One launch that only reads `nbytes` at d_buf (measurement aid)."""
+    check(lib().oxh_debug_read_probe(ctypes.c_void_p(d_buf), nbytes, None, stream))
+
+
 def debug_subblock_sums(qtype, d_w, rows, cols, d_act, d_sums, stream=None):
     check(lib().oxh_debug_subblock_sums(qtype, ctypes.c_void_p(d_w), rows, cols,
                                         ctypes.c_void_p(d_act), ctypes.c_void_p(d_sums), stream))

@@ -170,6 +170,9 @@ def dequant_rows(ref):
 LEGACY = (("q4_0", 3, 18), ("q4_1", 4, 20), ("q5_0", 5, 22), ("q5_1", 6, 24))
 
 
+ALIASES = (("al5", 17, 3), ("al6", 19, 5), ("al8", 20, 7))
+
+
 def legacy_formats(ref):
     """legacy_formats.npz: Q4_0 / Q4_1 / Q5_0 / Q5_1 against Q8_0 activations,
     raw-block dots (scalar and dispatched kernels) and the matvec entry points."""
@@ -210,6 +213,21 @@ def legacy_formats(ref):
         out[name + "_api_shape"] = np.array([rows, cols, rb], np.int64)
         out[name + "_api_out"] = o.copy()
         out[name + "_api_act"] = temp.view(np.uint8)[:cols // 32 * 34].copy()
+    # AL5 / AL6 / AL8: the Q4_0 / Q5_0 / Q8_0 layouts under their own type ids
+    for name, qt, base in ALIASES:
+        rows, cols = 24, 896
+        rb = synth.row_bytes(base, cols)
+        wm = synth.weights(base, rows, cols, seed=8, stream=qt)
+        x = synth.normal(cols, seed=8, stream=200 + qt)
+        o, temp, deq = np.zeros(rows, np.float32), np.zeros(cols, np.float32), np.zeros((2, cols), np.float32)
+        ref.oc_matvec_quantized(qt, wm.ctypes.data, rows, cols, rb, x.ctypes.data, o.ctypes.data, temp.ctypes.data)
+        for r in range(2):
+            assert ref.oc_quant_dequant_row(qt, wm[r * rb:].ctypes.data, rb, deq[r].ctypes.data, cols) == 0
+        out[name + "_api_w"], out[name + "_api_x"] = wm, x
+        out[name + "_api_shape"] = np.array([rows, cols, rb], np.int64)
+        out[name + "_api_out"] = o.copy()
+        out[name + "_api_act"] = temp.view(np.uint8)[:cols // 32 * 34].copy()
+        out[name + "_dequant_bits"] = deq.view(np.uint32).copy()
     np.savez_compressed(os.path.join(HERE, "legacy_formats.npz"), **out)
 
 

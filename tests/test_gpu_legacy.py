@@ -142,3 +142,36 @@ def test_fused_prologue_and_paired_segments(oxh, name, qtype):
     o.oxo_swiglu_f32(gate.ctypes.data, up.ctypes.data, want.ctypes.data, rows)
     h = d_h.download(np.float32, rows)
     assert np.all(np.abs(h - want) <= FLOAT_RTOL * np.abs(want) + 1e-30)
+
+
+@pytest.mark.parametrize("alias,base", [(17, 3), (19, 5), (20, 7)])
+def test_alias_type_ids_run_the_base_layout(oxh, alias, base):
+    """AL5 / AL6 / AL8 (oxidize-c/src/compute/quantization.c:207-214): same
+    bytes, same dot, another id -- host entry point, device segments and the
+    embedding lookup give the base type's bits."""
+    rows, cols = 300, 896
+    rb = synth.row_bytes(base, cols)
+    w = synth.weights(base, rows, cols, seed=21, stream=alias)
+    x = synth.normal(cols, seed=21, stream=alias + 50)
+    outs = []
+    for t in (alias, base):
+        out, temp = np.zeros(rows, np.float32), np.zeros(cols, np.float32)
+        assert mv.matvec_quantized(t, w, rows, cols, rb, x, out, temp) == 0
+        outs.append((out, temp.copy()))
+    assert np.array_equal(bits(outs[0][0]), bits(outs[1][0]))
+    assert np.array_equal(outs[0][1].view(np.uint8), outs[1][1].view(np.uint8))
+    o = oxlibs.oracle()
+    want, t2 = np.zeros(rows, np.float32), np.zeros(cols, np.float32)
+    assert o.oxo_matvec_quantized(alias, w.ctypes.data, rows, cols, rb, x.ctypes.data, want.ctypes.data,
+                                  t2.ctypes.data) == 0
+    assert np.array_equal(bits(outs[0][0]), bits(want))
+    d_w = mv.DeviceBuffer.from_host(w)
+    ids = np.array([0, rows - 1, 7], np.uint32)
+    d_ids = mv.DeviceBuffer.from_host(ids)
+    d_o = mv.DeviceBuffer(ids.size * cols * 4)
+    mv.get_rows(alias, d_w.ptr, rows, cols, d_ids.ptr, ids.size, d_o.ptr, cols)
+    got = d_o.download(np.float32, ids.size * cols).reshape(ids.size, cols)
+    for k, i in enumerate(ids):
+        deq = np.zeros(cols, np.float32)
+        assert o.oxo_dequant_row(alias, w[int(i) * rb:].ctypes.data, cols, deq.ctypes.data) == 0
+        assert np.array_equal(bits(got[k]), bits(deq))

@@ -525,6 +525,33 @@ def test_legacy_formats_vs_reference_goldens(name, qt, bsize):
     assert np.all(np.abs(out - want) <= 1e-4 + 1e-5 * np.abs(want))
 
 
+@pytest.mark.parametrize("name,qt,base", [("al5", 17, 3), ("al6", 19, 5), ("al8", 20, 7)])
+def test_alias_types_vs_reference_goldens(name, qt, base):
+    """AL5 / AL6 / AL8 are the Q4_0 / Q5_0 / Q8_0 layouts under other ids
+    (oxidize-c/src/compute/quantization.c:207-214, matvec.c:323-329): the
+    compiled reference's outputs for the alias id, and the oracle's for the
+    alias and the base id, which must not differ by a bit."""
+    g = load("legacy_formats.npz")
+    rows, cols, rb = (int(v) for v in g[name + "_api_shape"])
+    wm, x = g[name + "_api_w"], g[name + "_api_x"]
+    outs = []
+    for t in (qt, base):
+        out, temp = np.zeros(rows, np.float32), np.zeros(cols, np.float32)
+        assert O.oxo_act_kind(t, cols) == 1 and O.oxo_stride_ok(t, cols, rb) == 1
+        assert O.oxo_matvec_quantized(t, wm.ctypes.data, rows, cols, rb, x.ctypes.data, out.ctypes.data,
+                                      temp.ctypes.data) == 0
+        a = g[name + "_api_act"]
+        assert np.array_equal(temp.view(np.uint8)[:a.size], a)
+        outs.append(out)
+    assert np.array_equal(outs[0].view(np.uint32), outs[1].view(np.uint32))
+    want = g[name + "_api_out"]
+    assert np.all(np.abs(outs[0] - want) <= 1e-4 + 1e-5 * np.abs(want))
+    for r in range(2):
+        deq = np.zeros(cols, np.float32)
+        assert O.oxo_dequant_row(qt, wm[r * rb:].ctypes.data, cols, deq.ctypes.data) == 0
+        assert np.array_equal(deq.view(np.uint32), g[name + "_dequant_bits"][r])
+
+
 @pytest.mark.parametrize("name,qt,bsize", LEGACY)
 def test_legacy_formats_closed_forms_and_layout(name, qt, bsize):
     """Codes c everywhere, activations a everywhere: 32*(c - offset)*a*d*dq, plus
