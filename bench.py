@@ -173,6 +173,31 @@ def secondary_figures(mv, synth):
     d_x.free()
     d_a.free()
     d_o.free()
+    # the remaining weight types behind the same entry points: batch-1 GEMV at the gate/up shape,
+    # eight distinct copies in turn (beyond the last-level cache)
+    others = {}
+    x = synth.normal(cols, seed=0, stream=2003)
+    d_x = mv.DeviceBuffer.from_host(x)
+    d_o = mv.DeviceBuffer(rows * 4)
+    for name, qt in (("q2_k", 8), ("q3_k", 10), ("q4_0", 3), ("q4_1", 4), ("q5_0", 5), ("q5_1", 6)):
+        w = synth.weights(qt, rows, cols, seed=0, stream=7)
+        copies = [mv.DeviceBuffer.from_host(w) for _ in range(8)]
+        segs = [mv.make_segments([(c.ptr, d_o.ptr, rows, 0)]) for c in copies]
+        state = {"i": 0}
+
+        def run_other():
+            state["i"] += 1
+            mv.gemv_segments_f32(qt, segs[state["i"] % 8], cols, d_x.ptr, cols, None, 1, rows)
+
+        us = timed(run_other, 32, mv)
+        nbytes = w.nbytes + 4 * cols + 4 * rows
+        others[name] = {"us": round(us, 2), "gbps": round(nbytes / us / 1e3, 1),
+                        "frac_of_hbm_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBPS, 4)}
+        for c in copies:
+            c.free()
+    d_x.free()
+    d_o.free()
+    out["other_types_gemv_28672x4096"] = others
     # Q8_0 lm_head (configuration 2), batch 1 and 8
     rows, cols = 151936, 896
     w = synth.weights(Q80, rows, cols, seed=0, stream=5)

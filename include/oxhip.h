@@ -49,6 +49,10 @@ extern "C" {
 #define OXH_Q5_0    5u
 #define OXH_Q5_1    6u
 #define OXH_Q8_0    7u
+#define OXH_Q2_K    8u
+#define OXH_Q3_K_S  9u     /* ids 9, 10, 11: one Q3_K block layout */
+#define OXH_Q3_K_M 10u
+#define OXH_Q3_K_L 11u
 #define OXH_Q4_K_S 12u
 #define OXH_Q4_K_M 13u
 #define OXH_Q5_K_S 14u
@@ -65,6 +69,8 @@ extern "C" {
 #define OXH_Q4_K_BYTES   144u
 #define OXH_Q5_K_BYTES   176u
 #define OXH_Q6_K_BYTES   210u
+#define OXH_Q2_K_BYTES    84u
+#define OXH_Q3_K_BYTES   110u
 #define OXH_Q8_0_BYTES    34u
 #define OXH_Q4_0_BYTES    18u
 #define OXH_Q4_1_BYTES    20u
@@ -205,7 +211,7 @@ int oxh_mmq(uint32_t qtype, const void *d_w, size_t rows, size_t cols,
  * the token-embedding table stays quantized in HBM and the ids never leave
  * the device.  Replaces oc_cuda_mmq_get_row / _get_row_dev / _get_row_batch
  * (oxidize-c/include/oxidize/cuda_mmq.h:74-93).  Every type the matvec entry
- * points take (Q4_K, Q5_K, Q6_K, Q8_0, Q4_0, Q4_1, Q5_0, Q5_1);
+ * points take (Q2_K ... Q6_K, Q8_0, Q4_0, Q4_1, Q5_0, Q5_1, the AL aliases);
  * d_ids is device memory (at most 65535 per call); an id >= rows gives a row
  * of zeros; d_out and out_stride*4 must be multiples of 16 bytes. */
 int oxh_get_rows(uint32_t qtype, const void *d_w, size_t rows, size_t cols,

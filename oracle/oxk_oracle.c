@@ -322,6 +322,90 @@ float oxo_dot_q6_k_q8_k(const uint8_t *row, size_t blocks, const uint8_t *act,
     return sum;
 }
 
+/* Q2_K and Q3_K walk their 2-bit codes alike: element e = 128*outer +
+ * 32*inner + l (l < 32) is bits [2*inner, 2*inner + 2) of qs[32*outer + l];
+ * Q3_K adds bit (4*outer + inner) of hmask[l] as the code's third bit
+ * (src/compute/oxk.c:512-590). */
+static unsigned q23_code(const uint8_t *qs, const uint8_t *hmask, unsigned e)
+{
+    const unsigned outer = e >> 7, inner = (e >> 5) & 3u, l = e & 31u;
+    unsigned c = (qs[32u * outer + l] >> (2u * inner)) & 3u;
+    if (hmask) c |= ((hmask[l] >> (4u * outer + inner)) & 1u) << 2;
+    return c;
+}
+
+/* the sixteen 6-bit scales of a Q3_K block, minus 32 (src/compute/oxk.c:556-573) */
+static void q3k_scales(const uint8_t *p, int8_t sc[16])
+{
+    uint32_t a[4];
+    for (unsigned i = 0; i < 3; i++)
+        a[i] = (uint32_t)p[4 * i] | ((uint32_t)p[4 * i + 1] << 8) | ((uint32_t)p[4 * i + 2] << 16) |
+               ((uint32_t)p[4 * i + 3] << 24);
+    const uint32_t t = a[2];
+    a[2] = ((a[0] >> 4) & 0x0F0F0F0Fu) | (((t >> 4) & 0x03030303u) << 4);
+    a[3] = ((a[1] >> 4) & 0x0F0F0F0Fu) | (((t >> 6) & 0x03030303u) << 4);
+    a[0] = (a[0] & 0x0F0F0F0Fu) | ((t & 0x03030303u) << 4);
+    a[1] = (a[1] & 0x0F0F0F0Fu) | (((t >> 2) & 0x03030303u) << 4);
+    for (unsigned i = 0; i < 4; i++)
+        for (unsigned j = 0; j < 4; j++)
+            sc[4 * i + j] = (int8_t)(int32_t)(((a[i] >> (8 * j)) & 0xFFu) - 32u);
+}
+
+float oxo_dot_q2_k_q8_k(const uint8_t *row, size_t blocks, const uint8_t *act, int32_t *grp)
+{
+    float sum = 0.0f;
+    for (size_t b = 0; b < blocks; b++) {
+        const uint8_t *w = row + b * OXO_Q2_K_BYTES;
+        const uint8_t *a = act + b * OXO_Q8_K_BYTES;
+        const float dw = oxo_f16_to_f32(rd_u16(w + 80));
+        const float dmin = oxo_f16_to_f32(rd_u16(w + 82));
+        float dq;
+        memcpy(&dq, a, 4);
+        const int8_t *q = (const int8_t *)(a + 4);
+        int32_t pos = 0, min_acc = 0;
+        for (unsigned g = 0; g < 16; g++) {
+            int32_t acc = 0;
+            for (unsigned i = 0; i < 16; i++)
+                acc += (int32_t)q23_code(w + 16, NULL, 16 * g + i) * (int32_t)q[16 * g + i];
+            int16_t bs;
+            memcpy(&bs, a + 260 + 2 * g, 2);
+            pos += (int32_t)(w[g] & 15u) * acc;
+            min_acc += (int32_t)(w[g] >> 4) * (int32_t)bs;
+            if (grp) grp[16 * b + g] = acc;
+        }
+        sum += dq * (dw * (float)pos - dmin * (float)min_acc);
+    }
+    return sum;
+}
+
+float oxo_dot_q3_k_q8_k(const uint8_t *row, size_t blocks, const uint8_t *act, int32_t *grp)
+{
+    float sum = 0.0f;
+    for (size_t b = 0; b < blocks; b++) {
+        const uint8_t *w = row + b * OXO_Q3_K_BYTES;
+        const uint8_t *a = act + b * OXO_Q8_K_BYTES;
+        const float dw = oxo_f16_to_f32(rd_u16(w + 108));
+        float dq;
+        memcpy(&dq, a, 4);
+        const int8_t *q = (const int8_t *)(a + 4);
+        int8_t sc[16];
+        q3k_scales(w + 96, sc);
+        int32_t pos = 0, off = 0;
+        for (unsigned g = 0; g < 16; g++) {
+            int32_t acc = 0;
+            for (unsigned i = 0; i < 16; i++)
+                acc += (int32_t)q23_code(w + 32, w, 16 * g + i) * (int32_t)q[16 * g + i];
+            int16_t bs;
+            memcpy(&bs, a + 260 + 2 * g, 2);
+            pos += (int32_t)sc[g] * acc;
+            off += (int32_t)sc[g] * (int32_t)bs;
+            if (grp) grp[16 * b + g] = acc;
+        }
+        sum += dw * dq * (float)(pos - 4 * off);
+    }
+    return sum;
+}
+
 float oxo_dot_q8_0_q8_0(const uint8_t *row, size_t blocks, const uint8_t *act,
                         int32_t *isum)
 {
@@ -419,6 +503,10 @@ static size_t block_bytes(uint32_t qtype)
     case OXO_Q5_K_S:
     case OXO_Q5_K_M: return OXO_Q5_K_BYTES;
     case OXO_Q6_K:   return OXO_Q6_K_BYTES;
+    case OXO_Q2_K:   return OXO_Q2_K_BYTES;
+    case OXO_Q3_K_S:
+    case OXO_Q3_K_M:
+    case OXO_Q3_K_L: return OXO_Q3_K_BYTES;
     default:         return 0;
     }
 }
@@ -434,6 +522,10 @@ int oxo_act_kind(uint32_t qtype, size_t cols)
     case OXO_Q5_1:
     case OXO_Q8_0:
     case OXO_AL8:    return (cols % OXO_QK8_0 == 0) ? 1 : 0;
+    case OXO_Q2_K:
+    case OXO_Q3_K_S:
+    case OXO_Q3_K_M:
+    case OXO_Q3_K_L:
     case OXO_Q4_K_S:
     case OXO_Q4_K_M:
     case OXO_Q5_K_S:
@@ -469,6 +561,10 @@ static float row_dot(uint32_t qtype, const uint8_t *row, size_t blocks,
     case OXO_AL8:
     case OXO_Q8_0:   return oxo_dot_q8_0_q8_0(row, blocks, act, NULL);
     case OXO_Q6_K:   return oxo_dot_q6_k_q8_k(row, blocks, act, NULL);
+    case OXO_Q2_K:   return oxo_dot_q2_k_q8_k(row, blocks, act, NULL);
+    case OXO_Q3_K_S:
+    case OXO_Q3_K_M:
+    case OXO_Q3_K_L: return oxo_dot_q3_k_q8_k(row, blocks, act, NULL);
     case OXO_Q5_K_S:
     case OXO_Q5_K_M: return oxo_dot_q5_k_q8_k(row, blocks, act, NULL, NULL);
     default:         return oxo_dot_q4_k_q8_k(row, blocks, act, NULL, NULL);
@@ -670,6 +766,26 @@ int oxo_dequant_row(uint32_t qtype, const uint8_t *row, size_t cols, float *out)
                 const unsigned code = nib | (((bits >> e) & 1u) << 4);
                 if (has_m) out[32 * b + e] = (float)code * d + m;
                 else       out[32 * b + e] = (float)((int)code - (has_h ? 16 : 8)) * d;
+            }
+        } else if (qtype == OXO_Q2_K) {
+            /* src/compute/quantization.c:521-561 */
+            const uint8_t *w = row + b * OXO_Q2_K_BYTES;
+            const float d = oxo_f16_to_f32(rd_u16(w + 80));
+            const float mn = oxo_f16_to_f32(rd_u16(w + 82));
+            for (unsigned e = 0; e < 256; e++) {
+                const float dl = d * (float)(w[e >> 4] & 15u);
+                const float ml = mn * (float)(w[e >> 4] >> 4);
+                out[256 * b + e] = dl * (float)q23_code(w + 16, NULL, e) - ml;
+            }
+        } else if (qtype == OXO_Q3_K_S || qtype == OXO_Q3_K_M || qtype == OXO_Q3_K_L) {
+            /* src/compute/quantization.c:563-630 */
+            const uint8_t *w = row + b * OXO_Q3_K_BYTES;
+            const float d = oxo_f16_to_f32(rd_u16(w + 108));
+            int8_t sc[16];
+            q3k_scales(w + 96, sc);
+            for (unsigned e = 0; e < 256; e++) {
+                const float dl = d * (float)sc[e >> 4];
+                out[256 * b + e] = dl * (float)((int)q23_code(w + 32, w, e) - 4);
             }
         } else if (qtype == OXO_Q8_0) {
             const uint8_t *w = row + b * OXO_Q8_0_BYTES;

@@ -51,6 +51,10 @@ enum {
     OXO_Q5_0   = 5,
     OXO_Q5_1   = 6,
     OXO_Q8_0   = 7,
+    OXO_Q2_K   = 8,
+    OXO_Q3_K_S = 9,
+    OXO_Q3_K_M = 10,
+    OXO_Q3_K_L = 11,
     OXO_Q4_K_S = 12,
     OXO_Q4_K_M = 13,
     OXO_Q5_K_S = 14,
@@ -63,6 +67,8 @@ enum {
 
 #define OXO_QK_K        256u
 #define OXO_QK8_0       32u
+#define OXO_Q2_K_BYTES  84u
+#define OXO_Q3_K_BYTES  110u
 #define OXO_Q4_K_BYTES  144u
 #define OXO_Q5_K_BYTES  176u
 #define OXO_Q6_K_BYTES  210u
@@ -95,6 +101,14 @@ float oxo_dot_q5_k_q8_k(const uint8_t *row, size_t blocks, const uint8_t *act,
 /* src/compute/oxk.c:913-964.  `grp` (optional) receives 16 int32 per block. */
 float oxo_dot_q6_k_q8_k(const uint8_t *row, size_t blocks, const uint8_t *act,
                         int32_t *grp);
+/* src/compute/oxk.c:592-622 (Q2_K: 16 bytes of 4-bit scale | 4-bit min, 64
+ * bytes of 2-bit codes, f16 d, f16 dmin; the block term is
+ * dq*(d*pos - dmin*min)) and :624-652 (Q3_K: 32 bytes of third bits, 64 bytes
+ * of 2-bit codes, sixteen 6-bit scales in 12 bytes, f16 d; codes 0..7 with a
+ * uniform offset of 4: d*dq*(pos - 4*off)).  `grp` (optional) receives the 16
+ * int32 group sums per block. */
+float oxo_dot_q2_k_q8_k(const uint8_t *row, size_t blocks, const uint8_t *act, int32_t *grp);
+float oxo_dot_q3_k_q8_k(const uint8_t *row, size_t blocks, const uint8_t *act, int32_t *grp);
 /* src/compute/oxk.c:224-241 (block-sequential scalar chain).  `isum`
  * (optional) receives one int32 per block. */
 float oxo_dot_q8_0_q8_0(const uint8_t *row, size_t blocks, const uint8_t *act,

@@ -279,7 +279,7 @@ k_quantize_q8_0(const float *__restrict__ x, size_t in_stride, uint32_t blocks_p
  * the bit.  One wave per 256 values, lane l producing values 4l .. 4l+3 (they
  * share a sub-block / scale group); grid.y walks the ids.  An id beyond the
  * matrix yields a row of zeros rather than a read outside it.
- * KIND: 0 Q4_K, 1 Q5_K, 2 Q6_K, 3 Q8_0, 4 Q4_0, 5 Q4_1, 6 Q5_0, 7 Q5_1. */
+ * KIND: 0 Q4_K, 1 Q5_K, 2 Q6_K, 3 Q8_0, 4 Q4_0, 5 Q4_1, 6 Q5_0, 7 Q5_1, 8 Q2_K, 9 Q3_K. */
 template <int KIND>
 __global__ __launch_bounds__(256) void
 k_get_rows(const uint8_t *__restrict__ w, uint32_t rows, uint32_t cols, uint32_t row_bytes,
@@ -294,7 +294,32 @@ k_get_rows(const uint8_t *__restrict__ w, uint32_t rows, uint32_t cols, uint32_t
     float v[4] = { 0.0f, 0.0f, 0.0f, 0.0f };
     if (id < rows) {
         const uint8_t *row = w + (size_t)id * row_bytes;
-        if (KIND >= 4) {
+        if (KIND >= 8) {
+            /* 2-bit codes: element 128n + 32k + l is bits [2k, 2k+2) of qs[32n + l]; Q3_K adds bit
+             * 4n + k of hmask[l] as the third bit (quantization.c:521-630) */
+            const uint8_t *blk = row + (size_t)unit * (KIND == 9 ? 110u : 84u);
+            const uint32_t e = 4u * lane, n = e >> 7, k = (e >> 5) & 3u, l32 = e & 31u, g = e >> 4;
+            if (KIND == 8) {
+                const uint32_t dd = *reinterpret_cast<const uint32_t *>(blk + 80u);
+                const uint32_t sb = blk[g];
+                const float dl = half_to_float_hw(dd & 0xFFFFu) * (float)(sb & 15u);
+                const float ml = half_to_float_hw(dd >> 16) * (float)(sb >> 4);
+                const uint32_t q = *reinterpret_cast<const uint32_t *>(blk + 16u + 32u * n + l32) >> (2u * k);
+#pragma unroll
+                for (int i = 0; i < 4; i++) v[i] = dl * (float)((q >> (8 * i)) & 3u) - ml;
+            } else {
+                const uint8_t *sp = blk + 96u;
+                const uint32_t lo4 = g < 8u ? (sp[g] & 15u) : (uint32_t)(sp[g - 8u] >> 4);
+                const uint32_t hi2 = (sp[8u + (g & 3u)] >> (2u * (g >> 2))) & 3u;
+                const float dl = half_to_float_hw(*reinterpret_cast<const uint16_t *>(blk + 108u)) *
+                                 (float)((int)(lo4 | (hi2 << 4)) - 32);
+                const uint32_t q = reinterpret_cast<const U32u2 *>(blk + 32u + 32u * n + l32)->v >> (2u * k);
+                const uint32_t h = reinterpret_cast<const U32u2 *>(blk + l32)->v >> (4u * n + k);
+#pragma unroll
+                for (int i = 0; i < 4; i++)
+                    v[i] = dl * (float)((int)(((q >> (8 * i)) & 3u) | (((h >> (8 * i)) & 1u) << 2)) - 4);
+            }
+        } else if (KIND >= 4) {
             /* 32-value blocks [f16 d][f16 m: Q4_1, Q5_1][4 B fifth bits: Q5_0, Q5_1][16 B nibbles]; value i
              * is the low nibble of byte i, value i + 16 the high nibble (quantization.c:386-474) */
             const bool has_m = KIND == 5 || KIND == 7, has_h = KIND >= 6;
@@ -447,6 +472,8 @@ static uint32_t canon_qtype(uint32_t qtype)
     case OXH_AL5: return OXH_Q4_0;
     case OXH_AL6: return OXH_Q5_0;
     case OXH_AL8: return OXH_Q8_0;
+    case OXH_Q3_K_S:                    /* one Q3_K layout under three ids */
+    case OXH_Q3_K_L: return OXH_Q3_K_M;
     default:      return qtype;
     }
 }
@@ -459,6 +486,8 @@ extern "C" int oxh_act_kind(uint32_t qtype, size_t cols)
     case OXH_Q5_0:
     case OXH_Q5_1:
     case OXH_Q8_0:   return (cols % OXH_QK8_0 == 0) ? 1 : 0;
+    case OXH_Q2_K:
+    case OXH_Q3_K_M:
     case OXH_Q4_K_S:
     case OXH_Q4_K_M:
     case OXH_Q5_K_S:
@@ -481,6 +510,8 @@ static size_t block_bytes(uint32_t qtype)
     case OXH_Q5_K_S:
     case OXH_Q5_K_M: return OXH_Q5_K_BYTES;
     case OXH_Q6_K:   return OXH_Q6_K_BYTES;
+    case OXH_Q2_K:   return OXH_Q2_K_BYTES;
+    case OXH_Q3_K_M: return OXH_Q3_K_BYTES;
     default:         return 0;
     }
 }
@@ -578,6 +609,8 @@ static hipError_t raise_all_lds_ceilings(void)
     OXH_RAISE(k_gemv_q4_k)
     OXH_RAISE(k_gemv_q5_k)
     OXH_RAISE(k_gemv_q6_k)
+    OXH_RAISE(k_gemv_q2_k)
+    OXH_RAISE(k_gemv_q3_k)
     OXH_RAISE(k_gemv_q8_0)
     OXH_RAISE(k_gemv_q4_0)
     OXH_RAISE(k_gemv_q4_1)
@@ -597,6 +630,8 @@ static hipError_t raise_all_lds_ceilings(void)
     OXH_RAISE_PRO(k_gemv_q4_k_pro)
     OXH_RAISE_PRO(k_gemv_q5_k_pro)
     OXH_RAISE_PRO(k_gemv_q6_k_pro)
+    OXH_RAISE_PRO(k_gemv_q2_k_pro)
+    OXH_RAISE_PRO(k_gemv_q3_k_pro)
     OXH_RAISE_PRO(k_gemv_q8_0_pro)
     OXH_RAISE_PRO(k_gemv_q4_0_pro)
     OXH_RAISE_PRO(k_gemv_q4_1_pro)
@@ -621,7 +656,8 @@ static bool is_q5k(uint32_t qtype) { return qtype == OXH_Q5_K_S || qtype == OXH_
 static uint32_t act_lds_bytes(uint32_t qtype, uint32_t blocks)
 {
     if (oxh_act_kind(qtype, 32) == 1) return q80_lds_bytes(blocks);
-    if (qtype == OXH_Q6_K) return q8k6_lds_bytes(blocks);
+    qtype = canon_qtype(qtype);
+    if (qtype == OXH_Q6_K || qtype == OXH_Q2_K || qtype == OXH_Q3_K_M) return q8k6_lds_bytes(blocks);
     return q8k_lds_bytes(blocks);
 }
 
@@ -919,6 +955,8 @@ static int launch_gemv(uint32_t qtype, const OxhSegment *segs, size_t n_segs, si
     if (is_q4k(qtype))          OXH_LAUNCH_ANY(k_gemv_q4_k, k_gemv_q4_k_pro);
     else if (is_q5k(qtype))     OXH_LAUNCH_ANY(k_gemv_q5_k, k_gemv_q5_k_pro);
     else if (qtype == OXH_Q6_K) OXH_LAUNCH_ANY(k_gemv_q6_k, k_gemv_q6_k_pro);
+    else if (qtype == OXH_Q2_K) OXH_LAUNCH_ANY(k_gemv_q2_k, k_gemv_q2_k_pro);
+    else if (qtype == OXH_Q3_K_M) OXH_LAUNCH_ANY(k_gemv_q3_k, k_gemv_q3_k_pro);
     else if (qtype == OXH_Q4_0) OXH_LAUNCH_ANY(k_gemv_q4_0, k_gemv_q4_0_pro);
     else if (qtype == OXH_Q4_1) OXH_LAUNCH_ANY(k_gemv_q4_1, k_gemv_q4_1_pro);
     else if (qtype == OXH_Q5_0) OXH_LAUNCH_ANY(k_gemv_q5_0, k_gemv_q5_0_pro);
@@ -1157,6 +1195,8 @@ extern "C" int oxh_get_rows(uint32_t qtype, const void *d_w, size_t rows, size_t
     else if (qtype == OXH_Q4_1) OXH_GET_ROWS(5);
     else if (qtype == OXH_Q5_0) OXH_GET_ROWS(6);
     else if (qtype == OXH_Q5_1) OXH_GET_ROWS(7);
+    else if (qtype == OXH_Q2_K) OXH_GET_ROWS(8);
+    else if (qtype == OXH_Q3_K_M) OXH_GET_ROWS(9);
     else                        OXH_GET_ROWS(3);
 #undef OXH_GET_ROWS
     HIP_TRY(hipGetLastError());

@@ -178,6 +178,32 @@ void oxs_fill_q6_k(uint8_t *dst, size_t n_blocks, uint64_t seed,
     }
 }
 
+/* Q2_K (84 B: 16 scale|min bytes, 64 code bytes, f16 d, f16 dmin) and Q3_K
+ * (110 B: 32 third-bit bytes, 64 code bytes, 12 scale bytes, f16 d): every
+ * payload byte uniform, the f16 scales ~ |N(0,sigma)|. */
+void oxs_fill_q23_k(uint8_t *dst, size_t n_blocks, uint64_t seed, uint64_t stream, float sigma,
+                    int is_q3)
+{
+    const size_t bytes = is_q3 ? 110u : 84u;
+#pragma omp parallel for schedule(static)
+    for (long b = 0; b < (long)n_blocks; b++) {
+        Rng r = rng_for(seed, stream, (uint64_t)b);
+        uint8_t *blk = dst + (size_t)b * bytes;
+        uint8_t raw[112];
+        for (int i = 0; i < 14; i++) {
+            const uint64_t w = next64(&r);
+            memcpy(raw + 8 * i, &w, 8);
+        }
+        memcpy(blk, raw, bytes);
+        if (is_q3) {
+            put16(blk + 108, half_abs_normal(&r, sigma));
+        } else {
+            put16(blk + 80, half_abs_normal(&r, sigma));
+            put16(blk + 82, half_abs_normal(&r, sigma));
+        }
+    }
+}
+
 /* Q8_0 blocks: int8 uniform in [-127,127], d ~ |N(0,sigma)|. */
 void oxs_fill_q8_0(uint8_t *dst, size_t n_blocks, uint64_t seed,
                    uint64_t stream, float sigma)

@@ -16,10 +16,11 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 _LIB = None
 
 Q4_0, Q4_1, Q5_0, Q5_1, Q8_0, Q4_K, Q5_K, Q6_K = 3, 4, 5, 6, 7, 13, 15, 16
+Q2_K, Q3_K = 8, 10                      # Q3_K also under ids 9 and 11 (the _S and _L variants)
 BLOCK_BYTES = {Q4_0: 18, Q4_1: 20, Q5_0: 22, Q5_1: 24, Q8_0: 34, Q4_K: 144, 12: 144, Q5_K: 176, 14: 176,
-               Q6_K: 210}
+               Q6_K: 210, Q2_K: 84, 9: 110, Q3_K: 110, 11: 110}
 BLOCK_ELEMS = {Q4_0: 32, Q4_1: 32, Q5_0: 32, Q5_1: 32, Q8_0: 32, Q4_K: 256, 12: 256, Q5_K: 256, 14: 256,
-               Q6_K: 256}
+               Q6_K: 256, Q2_K: 256, 9: 256, Q3_K: 256, 11: 256}
 
 
 def _lib():
@@ -37,6 +38,9 @@ def _lib():
         lib.oxs_fill_legacy.argtypes = [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_uint64, ctypes.c_uint64,
                                         ctypes.c_float, ctypes.c_uint32, ctypes.c_int]
         lib.oxs_fill_legacy.restype = None
+        lib.oxs_fill_q23_k.argtypes = [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_uint64, ctypes.c_uint64,
+                                       ctypes.c_float, ctypes.c_int]
+        lib.oxs_fill_q23_k.restype = None
         lib.oxs_fill_normal_f32.argtypes = [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_uint64,
                                             ctypes.c_uint64, ctypes.c_float]
         lib.oxs_fill_normal_f32.restype = None
@@ -60,6 +64,10 @@ def weights(qtype, rows, cols, seed=0, stream=0, sigma=None, out=None):
     if qtype in (Q4_0, Q4_1, Q5_0, Q5_1):
         _lib().oxs_fill_legacy(out.ctypes.data, n_blocks, seed, stream, 0.02 if sigma is None else sigma,
                                BLOCK_BYTES[qtype], int(qtype in (Q4_1, Q5_1)))
+        return out
+    if qtype in (Q2_K, 9, Q3_K, 11):
+        _lib().oxs_fill_q23_k(out.ctypes.data, n_blocks, seed, stream, 0.02 if sigma is None else sigma,
+                              int(qtype != Q2_K))
         return out
     fn = {Q8_0: "oxs_fill_q8_0", Q4_K: "oxs_fill_q4_k", 12: "oxs_fill_q4_k",
           Q5_K: "oxs_fill_q5_k", 14: "oxs_fill_q5_k", Q6_K: "oxs_fill_q6_k"}[qtype]

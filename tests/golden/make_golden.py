@@ -9,6 +9,7 @@ committed, this script documents how they were made.
     python tests/golden/make_golden.py float    # only float_steps.npz
     python tests/golden/make_golden.py dequant  # only dequant_rows.npz
     python tests/golden/make_golden.py legacy   # only legacy_formats.npz
+    python tests/golden/make_golden.py q23_k    # only q23_k.npz
 
 Every array is data: inputs and the reference's outputs for them.
 """
@@ -149,6 +150,71 @@ def float_steps(ref):
     np.savez_compressed(os.path.join(HERE, "float_steps.npz"), **out)
 
 
+def q23_k(ref):
+    """q23_k.npz: Q2_K (type id 8) and Q3_K (ids 9, 10, 11): raw-block dots by
+    the scalar and the dispatched kernels, the matvec entry points (single and
+    batch), dequantised rows and full-size checksums."""
+    rng = np.random.default_rng(20241125)
+    out = {}
+    nb, trials = 12, 24
+    for name, qt, bsize, scale_at in (("q2_k", 8, 84, (80, 82)), ("q3_k", 10, 110, (108,))):
+        w = xorshift_bytes(trials * nb * bsize, 0x9E3779B9 ^ qt).reshape(trials, nb, bsize)
+        for off in scale_at:
+            bits = finite_scale_bits(rng, trials * nb).reshape(trials, nb)
+            w[:, :, off] = bits & 0xFF
+            w[:, :, off + 1] = bits >> 8
+        act = q8k_acts(rng, trials, nb)
+        scalar = np.empty((trials, 2), np.uint32)
+        disp = np.empty((trials, 2), np.uint32)
+        fs, fd = getattr(ref, "oc_oxk_dot_%s_q8_k_scalar" % name), getattr(ref, "oc_oxk_dot_%s_q8_k" % name)
+        for t in range(trials):
+            wt, at = np.ascontiguousarray(w[t]), np.ascontiguousarray(act[t])
+            for k, blocks in enumerate((1, nb)):
+                scalar[t, k] = np.float32(fs(wt.ctypes.data, blocks, at.ctypes.data)).view(np.uint32)
+                disp[t, k] = np.float32(fd(wt.ctypes.data, blocks, at.ctypes.data)).view(np.uint32)
+        out[name + "_raw_w"], out[name + "_raw_act"] = w, act
+        out[name + "_raw_scalar_bits"], out[name + "_raw_dispatched_bits"] = scalar, disp
+    for qt, rows, cols in ((8, 40, 1280), (9, 9, 256), (10, 40, 1280), (11, 17, 512)):
+        rb = synth.row_bytes(qt, cols)
+        wm = synth.weights(qt, rows, cols, seed=7, stream=qt)
+        x = synth.normal(cols, seed=7, stream=100 + qt)
+        o = np.zeros(rows, np.float32)
+        temp = np.zeros(cols, np.float32)
+        ref.oc_matvec_quantized(qt, wm.ctypes.data, rows, cols, rb, x.ctypes.data, o.ctypes.data,
+                                temp.ctypes.data)
+        key = "api%d_" % qt
+        out[key + "w"], out[key + "x"] = wm, x
+        out[key + "shape"] = np.array([rows, cols, rb], np.int64)
+        out[key + "out_bits"] = o.view(np.uint32).copy()
+        out[key + "act"] = temp.view(np.uint8)[:cols // 256 * 292].copy()
+        n_vec, in_stride, out_stride = 5, cols + 8, rows + 3
+        xs = synth.normal(n_vec * in_stride, seed=8, stream=qt).reshape(n_vec, in_stride)
+        outs = np.full((n_vec, out_stride), -1.0, np.float32)
+        scratch = np.zeros(ref.oc_matvec_batch_scratch_bytes(cols), np.uint8)
+        ref.oc_matvec_quantized_batch(qt, wm.ctypes.data, rows, cols, rb, xs.ctypes.data, in_stride,
+                                      outs.ctypes.data, out_stride, n_vec, temp.ctypes.data,
+                                      scratch.ctypes.data, scratch.nbytes)
+        out[key + "batch_x"] = xs
+        out[key + "batch_out_bits"] = outs.view(np.uint32).copy()
+        deq = np.zeros((2, cols), np.float32)
+        for r in range(2):
+            assert ref.oc_quant_dequant_row(qt, wm[r * rb:].ctypes.data, rb, deq[r].ctypes.data, cols) == 0
+        out[key + "dequant_bits"] = deq.view(np.uint32).copy()
+    for qt, name in ((8, "big_q2_k_4096x4096"), (10, "big_q3_k_4096x4096")):
+        rows = cols = 4096
+        rb = synth.row_bytes(qt, cols)
+        wm = synth.weights(qt, rows, cols, seed=0, stream=0)
+        x = synth.normal(cols, seed=0, stream=1000)
+        o = np.zeros(rows, np.float32)
+        temp = np.zeros(cols, np.float32)
+        ref.oc_matvec_quantized(qt, wm.ctypes.data, rows, cols, rb, x.ctypes.data, o.ctypes.data,
+                                temp.ctypes.data)
+        out[name + "_crc_w"] = np.array([zlib.crc32(wm.tobytes())], np.uint32)
+        out[name + "_crc_out"] = np.array([zlib.crc32(o.tobytes())], np.uint32)
+        out[name + "_out"] = o.copy()
+    np.savez_compressed(os.path.join(HERE, "q23_k.npz"), **out)
+
+
 def dequant_rows(ref):
     """dequant_rows.npz: rows of every type the embedding lookup handles,
     expanded by the compiled reference (oc_quant_dequant_row)."""
@@ -245,6 +311,8 @@ def main():
         dequant_rows(ref)
     if only in (None, "legacy"):
         legacy_formats(ref)
+    if only in (None, "q23_k"):
+        q23_k(ref)
     if only is not None:
         return
     rng = np.random.default_rng(20240607)

@@ -312,6 +312,140 @@ def test_q5_k_full_size_vs_reference_checksums(name, rows, cols):
     assert np.array_equal(out, g[name + "_out"])
 
 
+# ── Q2_K and Q3_K ────────────────────────────────────────────────────────
+
+@pytest.mark.parametrize("name", ["q2_k", "q3_k"])
+def test_q23_k_raw_block_dots_float_bits_vs_reference(name):
+    g = load("q23_k.npz")
+    fo = getattr(O, "oxo_dot_%s_q8_k" % name)
+    w, act = g[name + "_raw_w"], g[name + "_raw_act"]
+    for t in range(w.shape[0]):
+        wt, at = np.ascontiguousarray(w[t]), np.ascontiguousarray(act[t])
+        for k, blocks in enumerate((1, w.shape[1])):
+            got = f32bits(fo(wt.ctypes.data, blocks, at.ctypes.data, None))
+            assert got == g[name + "_raw_scalar_bits"][t, k]
+            assert got == g[name + "_raw_dispatched_bits"][t, k]
+
+
+@pytest.mark.parametrize("qt", [8, 9, 10, 11])
+def test_q23_k_matvec_batch_and_dequant_vs_reference_goldens(qt):
+    g = load("q23_k.npz")
+    key = "api%d_" % qt
+    rows, cols, rb = (int(v) for v in g[key + "shape"])
+    w, x = g[key + "w"], g[key + "x"]
+    assert O.oxo_act_kind(qt, cols) == 2 and O.oxo_stride_ok(qt, cols, rb) == 1 and O.oxo_act_kind(qt, 300) == 0
+    out = np.zeros(rows, np.float32)
+    temp = np.zeros(cols, np.float32)
+    assert O.oxo_matvec_quantized(qt, w.ctypes.data, rows, cols, rb, x.ctypes.data,
+                                  out.ctypes.data, temp.ctypes.data) == 0
+    act = g[key + "act"]
+    assert np.array_equal(temp.view(np.uint8)[:act.size], act)
+    assert np.array_equal(out.view(np.uint32), g[key + "out_bits"])
+    xs = g[key + "batch_x"]
+    n_vec, in_stride = xs.shape
+    want = g[key + "batch_out_bits"]
+    out_stride = want.shape[1]
+    outs = np.full((n_vec, out_stride), -1.0, np.float32)
+    scratch = np.zeros(O.oxo_matvec_batch_scratch_bytes(cols), np.uint8)
+    assert O.oxo_matvec_quantized_batch(qt, w.ctypes.data, rows, cols, rb, xs.ctypes.data, in_stride,
+                                        outs.ctypes.data, out_stride, n_vec, scratch.ctypes.data,
+                                        scratch.nbytes) == 0
+    assert np.array_equal(outs.view(np.uint32), want)
+    for r in range(2):
+        deq = np.zeros(cols, np.float32)
+        assert O.oxo_dequant_row(qt, w[r * rb:].ctypes.data, cols, deq.ctypes.data) == 0
+        assert np.array_equal(deq.view(np.uint32), g[key + "dequant_bits"][r])
+
+
+@pytest.mark.parametrize("qt,name", [(8, "big_q2_k_4096x4096"), (10, "big_q3_k_4096x4096")])
+def test_q23_k_full_size_vs_reference_checksums(qt, name):
+    g = load("q23_k.npz")
+    w = synth.weights(qt, 4096, 4096, seed=0, stream=0)
+    x = synth.normal(4096, seed=0, stream=1000)
+    assert zlib.crc32(w.tobytes()) == int(g[name + "_crc_w"][0])
+    out = np.zeros(4096, np.float32)
+    temp = np.zeros(4096, np.float32)
+    assert O.oxo_matvec_quantized(qt, w.ctypes.data, 4096, 4096, synth.row_bytes(qt, 4096),
+                                  x.ctypes.data, out.ctypes.data, temp.ctypes.data) == 0
+    assert zlib.crc32(out.tobytes()) == int(g[name + "_crc_out"][0])
+    assert np.array_equal(out, g[name + "_out"])
+
+
+def test_q2_k_closed_form_and_element_placement():
+    """All codes c, scales s, mins m, activations a: dq*(d*256*s*c*a - dmin*256*m*a)
+    (oxidize-c/src/compute/oxk.c:592-622); then one code at a time, which fixes
+    element e = 128*outer + 32*inner + l <- bits 2*inner of qs[32*outer + l]
+    and group e/16's scale."""
+    d, dmin, dq, a = 0.5, 0.25, 0.125, 3
+    for c, s_, m in ((1, 5, 2), (3, 15, 15), (2, 0, 7)):
+        blk = np.zeros(84, np.uint8)
+        blk[0:16] = s_ | (m << 4)
+        blk[16:80] = c * 0x55
+        blk[80:82], blk[82:84] = f16_le(d), f16_le(dmin)
+        act = q8k_block(dq, np.full(256, a))
+        assert O.oxo_dot_q2_k_q8_k(blk.ctypes.data, 1, act.ctypes.data, None) == \
+            dq * (d * 256 * s_ * c * a - dmin * 256 * m * a)
+    rng = np.random.default_rng(5)
+    q = rng.integers(-127, 128, 256)
+    act = q8k_block(1.0, q)
+    scales = rng.integers(1, 16, 16)
+    for e in range(256):
+        blk = np.zeros(84, np.uint8)
+        blk[0:16] = scales                                  # mins 0
+        blk[80:82] = f16_le(1.0)
+        outer, inner, l = e >> 7, (e >> 5) & 3, e & 31
+        blk[16 + 32 * outer + l] = 3 << (2 * inner)
+        grp = np.zeros(16, np.int32)
+        got = O.oxo_dot_q2_k_q8_k(blk.ctypes.data, 1, act.ctypes.data, grp.ctypes.data)
+        assert got == float(3 * int(scales[e >> 4]) * int(q[e])), "element %d" % e
+        assert grp[e >> 4] == 3 * q[e] and np.count_nonzero(grp) == (1 if q[e] else 0)
+
+
+def test_q3_k_closed_form_and_element_placement():
+    """Codes 0..7 with a uniform offset of 4 and int8 scales sc - 32
+    (oxidize-c/src/compute/oxk.c:624-652): all-equal blocks, then one 2-bit code
+    and one third bit at a time (bit 4*outer + inner of hmask[l]), and each of
+    the sixteen 6-bit scales in turn."""
+    d, dq, a = 0.5, 0.25, 3
+
+    def pack_scales(sc):                                    # sixteen values 0..63 into 12 bytes
+        out = np.zeros(12, np.uint8)
+        for j in range(16):
+            lo, hi = sc[j] & 15, sc[j] >> 4
+            out[j % 8] |= lo << (4 * (j // 8))
+            out[8 + j % 4] |= hi << (2 * (j // 4))
+        return out
+
+    for code, raw_sc in ((7, 40), (0, 33), (5, 0), (4, 63)):
+        blk = np.zeros(110, np.uint8)
+        blk[0:32] = 0xFF if code & 4 else 0
+        blk[32:96] = (code & 3) * 0x55
+        blk[96:108] = pack_scales([raw_sc] * 16)
+        blk[108:110] = f16_le(d)
+        act = q8k_block(dq, np.full(256, a))
+        assert O.oxo_dot_q3_k_q8_k(blk.ctypes.data, 1, act.ctypes.data, None) == \
+            d * dq * 256 * (raw_sc - 32) * (code - 4) * a
+    rng = np.random.default_rng(6)
+    q = rng.integers(-127, 128, 256)
+    act = q8k_block(1.0, q)
+    raw = rng.integers(0, 64, 16)
+    raw[raw == 32] = 33
+    base_blk = np.zeros(110, np.uint8)
+    base_blk[96:108] = pack_scales(list(raw))
+    base_blk[108:110] = f16_le(1.0)
+    base = O.oxo_dot_q3_k_q8_k(base_blk.ctypes.data, 1, act.ctypes.data, None)      # every code 0 -> weight -4*sc
+    assert base == float(sum(-4 * (int(raw[g]) - 32) * int(q[16 * g:16 * g + 16].sum()) for g in range(16)))
+    for e in range(256):
+        outer, inner, l = e >> 7, (e >> 5) & 3, e & 31
+        sc = int(raw[e >> 4]) - 32
+        blk = base_blk.copy()
+        blk[32 + 32 * outer + l] = 2 << (2 * inner)
+        assert O.oxo_dot_q3_k_q8_k(blk.ctypes.data, 1, act.ctypes.data, None) == base + 2.0 * sc * q[e], e
+        blk = base_blk.copy()
+        blk[l] = 1 << (4 * outer + inner)
+        assert O.oxo_dot_q3_k_q8_k(blk.ctypes.data, 1, act.ctypes.data, None) == base + 4.0 * sc * q[e], e
+
+
 def test_q6_k_codes_zero_give_minus_32_times_scale_sum():
     # all codes 0 -> every weight is d*sc*(-32)  (oxidize-c/tests/test_quant.c:290-310)
     blk = np.zeros(210, np.uint8)
