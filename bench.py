@@ -207,12 +207,13 @@ def secondary_figures(mv, synth):
         xs = synth.normal(nv * cols, seed=0, stream=6)
         d_x = mv.DeviceBuffer.from_host(xs)
         d_o = mv.DeviceBuffer(nv * rows * 4)
+        d_qa = mv.DeviceBuffer(nv * mv.act_bytes(Q80, cols))    # room for the quantised activations
         state = {"i": 0}
 
         def run():
             state["i"] += 1
             segs = mv.make_segments([(copies[state["i"] % 3].ptr, d_o.ptr, rows, 0)])
-            mv.gemv_segments_f32(Q80, segs, cols, d_x.ptr, cols, None, nv, rows)
+            mv.gemv_segments_f32(Q80, segs, cols, d_x.ptr, cols, d_qa.ptr, nv, rows)
 
         us = timed(run, 12, mv)
         nbytes = w.nbytes + nv * 4 * (cols + rows)

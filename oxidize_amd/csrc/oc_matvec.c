@@ -527,8 +527,10 @@ int oxh_matvec_quantized_batch(uint32_t qtype, const uint8_t *data, size_t rows,
         for (size_t v0 = 0; v0 < n_vec; v0 += step) {
             const size_t m = n_vec - v0 < step ? n_vec - v0 : step;
             OxhSegment seg = { d_w, (float *)g_dout.p + v0 * rows, rows, v0, 0, NULL };
+            /* with room for the quantised activations a slice of several vectors may run on
+             * the matrix cores (same results; the library decides) */
             if ((rc = oxh_gemv_segments_f32(qtype, &seg, 1, cols, (const float *)g_dx.p, in_stride,
-                                            NULL, m, rows, NULL)))
+                                            g_dact.p, m, rows, NULL)))
                 return rc;
         }
     }

@@ -645,6 +645,7 @@ static hipError_t raise_all_lds_ceilings(void)
     if ((e = raise_lds_ceiling(k_mmq_q5_k<4, 1, 8>)) != hipSuccess) return e;
     if ((e = raise_lds_ceiling(k_mmq_q6_k<8, 1, 8>)) != hipSuccess) return e;
     if ((e = raise_lds_ceiling(k_mmq_q6_k<4, 1, 8>)) != hipSuccess) return e;
+    if ((e = raise_lds_ceiling(k_mfma_q8_0_segments<4>)) != hipSuccess) return e;
     if ((e = raise_lds_ceiling(k_mmq_q6_k_segments<1, 1, 4, 2>)) != hipSuccess) return e;
     if ((e = raise_lds_ceiling(k_mmq_q6_k_experts<1, 1, 4, 2>)) != hipSuccess) return e;
     return hipSuccess;
@@ -746,6 +747,53 @@ static bool mmq_deep_stages(uint32_t wg)
     return wg <= 2u * (uint32_t)(g_n_cu > 0 ? g_n_cu : 256);
 }
 
+/* Q8_0 launches with five or more activations per weight go to the MFMA kernel
+ * (OXH_Q80_MFMA_MIN_NV moves the threshold, 0 = never) when the quantised
+ * activations exist or have somewhere to go and the staged activations fit LDS. */
+static bool q80_wants_mfma(uint32_t qtype, const GemvIo &io, size_t max_nv, size_t blocks, const int32_t *dump)
+{
+    static int min_nv = -1;
+    if (min_nv < 0) min_nv = (int)env_u32("OXH_Q80_MFMA_MIN_NV", 5, 0, 64);
+    if (qtype != OXH_Q8_0 || dump || io.pro || min_nv == 0 || max_nv < (size_t)min_nv || max_nv > MQ80_TOK)
+        return false;
+    if ((size_t)mq80_lds_bytes((uint32_t)blocks, max_nv > 8 ? 16u : 8u, 4u) > GEMV_LDS_LIMIT) return false;
+    return io.d_acts != nullptr || io.d_act_out != nullptr;
+}
+
+static int launch_q80_mfma_segments(const OxhSegment *segs, size_t n_segs, size_t cols, size_t blocks,
+                                    const GemvIo &io, size_t n_vec_default, size_t n_acts, size_t out_stride,
+                                    void *stream)
+{
+    const uint8_t *acts = (const uint8_t *)io.d_acts;
+    if (!acts) {
+        int rc = oxh_quantize_q8_0(io.d_x, io.x_stride, n_acts, cols, io.d_act_out, stream);
+        if (rc) return rc;
+        acts = (const uint8_t *)io.d_act_out;
+    }
+    SegTable t;
+    memset(&t, 0, sizeof t);
+    uint32_t wg = 0, n = 0;
+    for (size_t i = 0; i < n_segs; i++) {
+        if (segs[i].rows == 0) continue;
+        t.s[n].w = (const uint8_t *)segs[i].d_w;
+        t.s[n].out = segs[i].d_out;
+        t.s[n].rows = (uint32_t)segs[i].rows;
+        t.s[n].act_first = (uint32_t)segs[i].act_first;
+        t.s[n].nv = (uint32_t)(segs[i].n_vec ? segs[i].n_vec : n_vec_default);
+        t.s[n].wg_begin = wg;
+        wg += (uint32_t)((segs[i].rows + 63u) / 64u);
+        n++;
+    }
+    t.n = n;
+    for (uint32_t i = 1; i < 4 && i < n; i++) t.bound[i - 1] = t.s[i].wg_begin;
+    uint32_t toks = 8u;
+    for (uint32_t i = 0; i < n; i++) if (t.s[i].nv > 8u) toks = 16u;
+    hipLaunchKernelGGL((k_mfma_q8_0_segments<4>), dim3(wg), dim3(256), mq80_lds_bytes((uint32_t)blocks, toks, 4u),
+                       pick_stream(stream), t, (uint32_t)blocks, acts, out_stride, toks);
+    HIP_TRY(hipGetLastError());
+    return OXH_OK;
+}
+
 static int launch_mmq_segments(uint32_t qtype, const OxhSegment *segs, size_t n_segs, size_t cols, size_t blocks,
                                const GemvIo &io, size_t n_vec_default, size_t n_acts,
                                size_t out_stride, void *stream)
@@ -843,6 +891,9 @@ static int launch_gemv(uint32_t qtype, const OxhSegment *segs, size_t n_segs, si
     if (!any_pair && gemv_wants_mfma(qtype, io, max_nv, dump))
         return launch_mmq_segments(qtype, segs, n_segs, cols, blocks, io, n_vec_default, max_act + max_nv,
                                    out_stride, stream);
+    if (!any_pair && q80_wants_mfma(qtype, io, max_nv, blocks, dump))
+        return launch_q80_mfma_segments(segs, n_segs, cols, blocks, io, n_vec_default, max_act + max_nv,
+                                        out_stride, stream);
     n_vec = max_nv;                        /* sizes LDS from here on */
     if (out_stride > 0xFFFFFFFFull || io.x_stride > 0xFFFFFFFFull || max_act + n_vec > 0xFFFFFFFFull)
         return arg_fail("gemv: stride too large");
