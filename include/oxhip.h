@@ -233,7 +233,8 @@ int oxh_get_rows(uint32_t qtype, const void *d_w, size_t rows, size_t cols,
  * only on n_tok, so a layer is a fixed sequence that may be captured in a
  * graph.  Expert matrices are stacked expert-major (expert e of gate/up at
  * rows [e*ffn, (e+1)*ffn), of down at rows [e*hidden, (e+1)*hidden)); types
- * Q4_K, Q5_K or Q6_K; at most 16 experts, top_k <= 8, n_tok <= 4096.
+ * Q4_K, Q5_K or Q6_K; at most 64 experts (the expert launches carry up to 32
+ * matrices each and repeat beyond that), top_k <= 8, n_tok <= 4096.
  * Expert ids and the grouping are exact; gate weights and silu(gate)*up are
  * float steps that agree with the reference to rounding; everything the
  * integer path computes from them is exact. */
@@ -249,7 +250,7 @@ int oxh_moe_workspace_bytes(const OxhMoe *m, size_t n_tok, size_t *bytes);
 int oxh_moe_ffn(const OxhMoe *m, const float *d_logits, const float *d_x, size_t x_stride,
                 size_t n_tok, float *d_out, size_t out_stride, void *d_workspace,
                 size_t workspace_bytes, void *stream);
-/* The routing and grouping step alone (n_expert <= 32).  ids, weights,
+/* The routing and grouping step alone (n_expert <= 64).  ids, weights,
  * slot_pos: n_tok*top_k entries, pair (t, j) at t*top_k + j; counts,
  * offsets: per expert (offsets has n_expert + 1 entries); perm: the token of
  * each sorted pair; slot_pos: where pair (t, j) landed in that order. */

@@ -1265,8 +1265,8 @@ struct MoeLayout {
 
 static int moe_layout(const OxhMoe *m, size_t n_tok, MoeLayout *l)
 {
-    if (!m || m->n_expert == 0 || m->n_expert > OXH_MOE_MAX_EXPERTS / 2)
-        return arg_fail("moe: n_expert must be 1..16");
+    if (!m || m->n_expert == 0 || m->n_expert > OXH_MOE_MAX_EXPERTS)
+        return arg_fail("moe: n_expert must be 1..64");
     if (m->top_k == 0 || m->top_k > OXH_MOE_MAX_TOPK || m->top_k > m->n_expert)
         return arg_fail("moe: top_k must be 1..8 and at most n_expert");
     if (oxh_act_kind(m->qtype_gate_up, m->hidden) != 2 || oxh_act_kind(m->qtype_down, m->ffn) != 2) {
@@ -1324,7 +1324,7 @@ extern "C" int oxh_moe_route(const float *d_logits, size_t n_tok, size_t n_exper
     if (n_tok == 0) return OXH_OK;
     if (!d_logits || !d_ids || !d_weights || !d_counts || !d_offsets || !d_perm || !d_slot_pos)
         return arg_fail("oxh_moe_route: NULL pointer");
-    if (n_expert == 0 || n_expert > OXH_MOE_MAX_EXPERTS) return arg_fail("oxh_moe_route: n_expert must be 1..32");
+    if (n_expert == 0 || n_expert > OXH_MOE_MAX_EXPERTS) return arg_fail("oxh_moe_route: n_expert must be 1..64");
     if (top_k == 0 || top_k > OXH_MOE_MAX_TOPK || top_k > n_expert)
         return arg_fail("oxh_moe_route: top_k must be 1..8 and at most n_expert");
     if (n_tok > 4096) return arg_fail("oxh_moe_route: at most 4096 tokens per call");
@@ -1347,21 +1347,6 @@ static int launch_experts(uint32_t qtype, const void *const *d_w, float *const *
     const size_t blocks = cols / OXH_QK_K;
     if (blocks * 292u * 256u > 0xFFFFFFFFull) return arg_fail("moe: cols too large");
     const size_t rb = oxh_row_bytes(qtype, cols);
-    SegTable t;
-    memset(&t, 0, sizeof t);
-    uint32_t wg = 0, n = 0;
-    for (size_t mtx = 0; mtx < n_mat; mtx++)
-        for (size_t e = 0; e < n_expert; e++) {
-            t.s[n].w = (const uint8_t *)d_w[mtx] + e * rows * rb;
-            t.s[n].out = d_out[mtx];
-            t.s[n].rows = (uint32_t)rows;
-            t.s[n].act_first = (uint32_t)e;             /* the expert whose count and offset apply */
-            t.s[n].wg_begin = wg;
-            wg += (uint32_t)((rows + G::ROWS - 1) / G::ROWS);
-            n++;
-        }
-    t.n = n;
-    for (uint32_t i = 1; i < 4 && i < n; i++) t.bound[i - 1] = t.s[i].wg_begin;
     const uint8_t *acts = (const uint8_t *)d_acts;
     hipStream_t st = pick_stream(stream);
     typedef Mmq6Geom<1, 1, 4> G6;
@@ -1370,14 +1355,34 @@ static int launch_experts(uint32_t qtype, const void *const *d_w, float *const *
 #define OXH_EXP_LAUNCH(KERNEL, GEOM, KB)                                                              \
     hipLaunchKernelGGL(KERNEL, dim3(wg), dim3(256), (KB) * GEOM::LDS_BYTES, st, t, nb, acts, out_stride, \
                        d_counts, d_offsets)
-    if (mmq_deep_stages(wg)) {
-        if (qtype == OXH_Q6_K) OXH_EXP_LAUNCH((k_mmq_q6_k_experts<1, 1, 4, 2>), G6, 2);
-        else if (is_q5k(qtype)) OXH_EXP_LAUNCH((k_mmq_q45_k_experts<1, 1, 4, true, 2>), G5, 2);
-        else OXH_EXP_LAUNCH((k_mmq_q45_k_experts<1, 1, 4, false, 2>), G, 2);
-    } else {
-        if (qtype == OXH_Q6_K) OXH_EXP_LAUNCH((k_mmq_q6_k_experts<1, 1, 4, 1>), G6, 1);
-        else if (is_q5k(qtype)) OXH_EXP_LAUNCH((k_mmq_q45_k_experts<1, 1, 4, true, 1>), G5, 1);
-        else OXH_EXP_LAUNCH((k_mmq_q45_k_experts<1, 1, 4, false, 1>), G, 1);
+    /* one segment per expert and matrix, at most OXH_MAX_SEGS of them per launch */
+    const size_t per_launch = OXH_MAX_SEGS / n_mat;
+    for (size_t e0 = 0; e0 < n_expert; e0 += per_launch) {
+        const size_t e1 = e0 + per_launch < n_expert ? e0 + per_launch : n_expert;
+        SegTable t;
+        memset(&t, 0, sizeof t);
+        uint32_t wg = 0, n = 0;
+        for (size_t mtx = 0; mtx < n_mat; mtx++)
+            for (size_t e = e0; e < e1; e++) {
+                t.s[n].w = (const uint8_t *)d_w[mtx] + e * rows * rb;
+                t.s[n].out = d_out[mtx];
+                t.s[n].rows = (uint32_t)rows;
+                t.s[n].act_first = (uint32_t)e;         /* the expert whose count and offset apply */
+                t.s[n].wg_begin = wg;
+                wg += (uint32_t)((rows + G::ROWS - 1) / G::ROWS);
+                n++;
+            }
+        t.n = n;
+        for (uint32_t i = 1; i < 4 && i < n; i++) t.bound[i - 1] = t.s[i].wg_begin;
+        if (mmq_deep_stages(wg)) {
+            if (qtype == OXH_Q6_K) OXH_EXP_LAUNCH((k_mmq_q6_k_experts<1, 1, 4, 2>), G6, 2);
+            else if (is_q5k(qtype)) OXH_EXP_LAUNCH((k_mmq_q45_k_experts<1, 1, 4, true, 2>), G5, 2);
+            else OXH_EXP_LAUNCH((k_mmq_q45_k_experts<1, 1, 4, false, 2>), G, 2);
+        } else {
+            if (qtype == OXH_Q6_K) OXH_EXP_LAUNCH((k_mmq_q6_k_experts<1, 1, 4, 1>), G6, 1);
+            else if (is_q5k(qtype)) OXH_EXP_LAUNCH((k_mmq_q45_k_experts<1, 1, 4, true, 1>), G5, 1);
+            else OXH_EXP_LAUNCH((k_mmq_q45_k_experts<1, 1, 4, false, 1>), G, 1);
+        }
     }
 #undef OXH_EXP_LAUNCH
     HIP_TRY(hipGetLastError());

@@ -46,7 +46,8 @@ def group(ids, n_expert):
 
 
 @pytest.mark.parametrize("n_tok,n_exp,k,renorm", [(1, 8, 2, 1), (16, 8, 2, 1), (100, 32, 8, 0), (1500, 3, 1, 1),
-                                                  (37, 16, 4, 1), (5, 2, 2, 0), (4096, 8, 2, 1)])
+                                                  (37, 16, 4, 1), (5, 2, 2, 0), (4096, 8, 2, 1), (300, 64, 8, 1),
+                                                  (9, 60, 4, 0)])
 def test_route_and_grouping(oxh, n_tok, n_exp, k, renorm):
     o = oxlibs.oracle()
     logits = synth.normal(n_tok * n_exp, seed=n_tok, stream=4242).reshape(n_tok, n_exp)
@@ -235,6 +236,12 @@ def test_layer_top1_and_all_experts(oxh):
     check_layer(Q4K, Q6K, 16, 8, 256, 512, 6, seed=4, renorm=1, skew=False)
 
 
+def test_layer_with_more_experts_than_one_launch_carries(oxh):
+    """40 and 64 experts: the gate/up launch carries 16 experts, the down launch 32, so both repeat."""
+    check_layer(Q4K, Q4K, 40, 4, 256, 256, 50, seed=8, skew=True)
+    check_layer(Q5K, Q6K, 64, 6, 256, 512, 23, seed=9, skew=False)
+
+
 def test_mixtral_shape_sampled_and_graph_replay(oxh):
     """8 experts, top-2, 16 tokens, 4096 x 14336 Q4_K: sampled pairs and rows
     stage by stage, the combination in full, and three graph replays."""
@@ -247,7 +254,7 @@ def test_mixtral_shape_sampled_and_graph_replay(oxh):
 def test_argument_checks(oxh):
     d = mv.DeviceBuffer(1 << 16)
     with pytest.raises(mv.OxhError):
-        mv.MoeLayer(Q4K, Q4K, d.ptr, d.ptr, d.ptr, 17, 2, 256, 256)          # too many experts
+        mv.MoeLayer(Q4K, Q4K, d.ptr, d.ptr, d.ptr, 65, 2, 256, 256)          # too many experts
     with pytest.raises(mv.OxhError):
         mv.MoeLayer(Q4K, Q4K, d.ptr, d.ptr, d.ptr, 4, 5, 256, 256)           # top_k > n_expert
     with pytest.raises(mv.OxhError):
@@ -260,4 +267,4 @@ def test_argument_checks(oxh):
                                       4, ctypes.c_void_p(d.ptr), 256, ctypes.c_void_p(layer.workspace.ptr), 128,
                                       None))                                  # workspace too small
     with pytest.raises(mv.OxhError):
-        mv.moe_route(d.ptr, 4, 33, 2, 1, d.ptr, d.ptr, d.ptr, d.ptr, d.ptr, d.ptr)
+        mv.moe_route(d.ptr, 4, 65, 2, 1, d.ptr, d.ptr, d.ptr, d.ptr, d.ptr, d.ptr)
