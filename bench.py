@@ -26,9 +26,9 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
 # HBM bytes one gate/up launch moves, from two rocprofv3 --pmc runs (FETCH_SIZE
-# 32407.5 KiB x 2.000, WRITE_SIZE 116.58 KiB x 1.000; the factors are what the
+# 32410.7 KiB x 2.000, WRITE_SIZE 116.57 KiB x 1.000; the factors are what the
 # same counters read for a 256 MiB device-to-device copy).  Not measured live.
-GATE_UP_TRAFFIC_BYTES = 66489724
+GATE_UP_TRAFFIC_BYTES = 66496518
 INT8_PEAK_TOPS = 5033.0     # dense int8 MFMA: 256 CU x 2.4 GHz x 8192 op/clk/CU
 
 
