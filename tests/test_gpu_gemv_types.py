@@ -405,3 +405,30 @@ def test_q8_0_small_batches_on_the_matrix_cores(oxh, rows, cols, nvs):
             assert np.array_equal(bits(got[v]), bits(want)), (nv, v)
         first += nv
     assert rb * rows == ws[0].nbytes
+
+
+@pytest.mark.parametrize("qtype,size", [(Q4K, 144), (15, 176), (Q6K, 210), (Q80, 34), (8, 84), (10, 110), (3, 18),
+                                        (4, 20), (5, 22), (6, 24)])
+def test_every_weight_byte_influences_its_row(oxh, qtype, size):
+    """oxidize-c/tests/test_quant.c:569-583 as a kernel test: one row per byte of
+    a block, that byte altered; every row must differ from the unaltered one
+    (no byte of any layout is ignored or read from the wrong place) and carry
+    the oracle's bits."""
+    group = 256 if size > 34 else 32
+    base = synth.weights(qtype, 1, group, seed=13, stream=qtype)
+    masks = (0x15, 0x6A)             # two alterations per byte: an integer change can cancel by chance
+    w = np.tile(base, 2 * size + 1).reshape(2 * size + 1, size)
+    for i in range(size):
+        for m, mask in enumerate(masks):
+            w[1 + 2 * i + m, i] ^= mask
+    w = np.ascontiguousarray(w.ravel())
+    x = (synth.normal(group, seed=13, stream=1) ** 2 + 0.25).astype(np.float32)      # all positive
+    rows = 2 * size + 1
+    out = np.zeros(rows, np.float32)
+    temp = np.zeros(group, np.float32)
+    assert mv.matvec_quantized(qtype, w, rows, group, size, x, out, temp) == 0
+    want, _ = oracle_matvec(qtype, w, rows, group, x)
+    assert np.array_equal(bits(out), bits(want))
+    ob = bits(out)
+    same = [i for i in range(size) if ob[1 + 2 * i] == ob[0] and ob[2 + 2 * i] == ob[0]]
+    assert not same, "bytes without influence: %s" % same
