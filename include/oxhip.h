@@ -149,7 +149,9 @@ int oxh_gemv_segments(uint32_t qtype, const OxhSegment *segs, size_t n_segs,
  * one kernel per decode matmul instead of two, which is what
  * oc_matvec_quantized does in one call (matvec.c:860-881).  When d_act_out is
  * not NULL the quantised bytes are also stored there (reference format,
- * oxh_act_bytes() per vector). */
+ * oxh_act_bytes() per vector, indexed like d_x; room for every vector up to
+ * the largest act_first + n_vec of any segment), and launches of several
+ * vectors per weight may then run on the matrix cores. */
 int oxh_gemv_segments_f32(uint32_t qtype, const OxhSegment *segs, size_t n_segs,
                           size_t cols, const float *d_x, size_t x_stride,
                           void *d_act_out, size_t n_vec, size_t out_stride,

@@ -866,7 +866,7 @@ static int launch_gemv(uint32_t qtype, const OxhSegment *segs, size_t n_segs, si
         return OXH_ERR_TOO_WIDE;
     }
     if (io.d_x && io.x_stride < cols) return arg_fail("gemv: x_stride < cols");
-    size_t total_rows = 0, max_act = 0;
+    size_t total_rows = 0, max_act = 0, act_end = 0;     /* act_end: one past the last activation any segment reads */
     /* a segment may carry its own activation count; the launch value is the default */
     size_t max_nv = 0;
     bool all_one = true, any_pair = false;
@@ -885,14 +885,15 @@ static int launch_gemv(uint32_t qtype, const OxhSegment *segs, size_t n_segs, si
         total_rows += segs[i].rows;
         total_work += segs[i].rows * (segs[i].d_w_pair ? 2u : 1u);
         if (segs[i].act_first > max_act) max_act = segs[i].act_first;
+        if (segs[i].rows && segs[i].act_first + nv > act_end) act_end = segs[i].act_first + nv;
     }
     if (total_rows == 0) return OXH_OK;
     if (any_pair && dump) return arg_fail("gemv: no sub-block dump of a paired launch");
     if (!any_pair && gemv_wants_mfma(qtype, io, max_nv, dump))
-        return launch_mmq_segments(qtype, segs, n_segs, cols, blocks, io, n_vec_default, max_act + max_nv,
+        return launch_mmq_segments(qtype, segs, n_segs, cols, blocks, io, n_vec_default, act_end,
                                    out_stride, stream);
     if (!any_pair && q80_wants_mfma(qtype, io, max_nv, blocks, dump))
-        return launch_q80_mfma_segments(segs, n_segs, cols, blocks, io, n_vec_default, max_act + max_nv,
+        return launch_q80_mfma_segments(segs, n_segs, cols, blocks, io, n_vec_default, act_end,
                                         out_stride, stream);
     n_vec = max_nv;                        /* sizes LDS from here on */
     if (out_stride > 0xFFFFFFFFull || io.x_stride > 0xFFFFFFFFull || max_act + n_vec > 0xFFFFFFFFull)
