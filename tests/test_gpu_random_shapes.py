@@ -65,3 +65,116 @@ def test_random_launch(oxh, seed):
             assert o.oxo_matvec_quantized(qt, w.ctypes.data, r, cols, rb, np.ascontiguousarray(xs[f + v]).ctypes.data,
                                           want.ctypes.data, temp.ctypes.data) == 0
             assert np.array_equal(bits(area[v, :r]), bits(want)), (qt, cols, r, n, f, v, with_buffer)
+
+
+def oracle_rows(qt, layout, w, rows, cols, x):
+    o = oxlibs.oracle()
+    want = np.zeros(rows, np.float32)
+    temp = np.zeros(cols, np.float32)
+    assert o.oxo_matvec_quantized(qt, w.ctypes.data, rows, cols, synth.row_bytes(layout, cols), x.ctypes.data,
+                                  want.ctypes.data, temp.ctypes.data) == 0
+    return want, temp
+
+
+@pytest.mark.parametrize("seed", range(51))
+def test_random_host_calls(oxh, seed):
+    """The reference's four entry points on host arrays with random shapes: single,
+    fused (shared input, possibly mixed types and empty matrices), multi-input,
+    and batch (1..40 vectors, padded strides)."""
+    rng = np.random.default_rng(5000 + seed)
+    qt = int(TYPES[seed % len(TYPES)])
+    layout = BASE.get(qt, qt)
+    group = synth.BLOCK_ELEMS[layout]
+    cols = int(rng.integers(1, 25 if group == 256 else 100)) * group
+    rb = synth.row_bytes(layout, cols)
+    temp = np.zeros(cols, np.float32)
+    which = seed % 3
+    if which == 0:                                             # fused and multi-input
+        n = int(rng.integers(1, 6))
+        rows = [int(rng.integers(0, 200)) for _ in range(n)]
+        qts = [qt] * n
+        if seed % 2 and n > 1:                                 # one matrix of another type with the same block width
+            other = 16 if group == 256 and layout != 16 else (7 if group == 32 and layout != 7 else qt)
+            qts[-1] = other
+        lays = [BASE.get(q, q) for q in qts]
+        ws = [synth.weights(l, r, cols, seed=seed, stream=i) if r else np.zeros(1, np.uint8)
+              for i, (l, r) in enumerate(zip(lays, rows))]
+        rbs = [synth.row_bytes(l, cols) for l in lays]
+        x = synth.normal(cols, seed=seed, stream=50)
+        outs = [np.full(max(r, 1), -3.5, np.float32) for r in rows]
+        assert mv.matvec_quantized_fused(qts, ws, rows, cols, rbs, x, outs, temp) == 0
+        for q, l, w, r, out in zip(qts, lays, ws, rows, outs):
+            if r:
+                assert np.array_equal(bits(out[:r]), bits(oracle_rows(q, l, w, r, cols, x)[0]))
+        xs = [synth.normal(cols, seed=seed, stream=60 + i) for i in range(n)]
+        outs = [np.full(max(r, 1), -3.5, np.float32) for r in rows]
+        assert mv.matvec_quantized_multi_input(qts, ws, rows, cols, rbs, xs, outs, temp) == 0
+        for q, l, w, r, xv, out in zip(qts, lays, ws, rows, xs, outs):
+            if r:
+                assert np.array_equal(bits(out[:r]), bits(oracle_rows(q, l, w, r, cols, xv)[0]))
+    else:                                                      # single and batch
+        rows = int(rng.integers(1, 400))
+        w = synth.weights(layout, rows, cols, seed=seed, stream=3)
+        x = synth.normal(cols, seed=seed, stream=51)
+        out = np.full(rows, -3.5, np.float32)
+        assert mv.matvec_quantized(qt, w, rows, cols, rb, x, out, temp) == 0
+        want, want_temp = oracle_rows(qt, layout, w, rows, cols, x)
+        nact = mv.act_bytes(qt, cols)
+        assert np.array_equal(temp.view(np.uint8)[:nact], want_temp.view(np.uint8)[:nact])
+        assert np.array_equal(bits(out), bits(want))
+        n_vec = int(rng.integers(1, 41))
+        in_stride, out_stride = cols + int(rng.integers(0, 3)) * 8, rows + int(rng.integers(0, 3))
+        xb = synth.normal(n_vec * in_stride, seed=seed, stream=52).reshape(n_vec, in_stride)
+        ob = np.full((n_vec, out_stride), -3.5, np.float32)
+        scratch = np.zeros(mv.batch_scratch_bytes(cols), np.uint8)
+        assert mv.matvec_quantized_batch(qt, w, rows, cols, rb, xb, in_stride, ob, out_stride, n_vec, temp,
+                                         scratch) == 0
+        assert np.all(ob[:, rows:] == -3.5)
+        for v in rng.choice(n_vec, size=min(n_vec, 6), replace=False):
+            want, _ = oracle_rows(qt, layout, w, rows, cols, np.ascontiguousarray(xb[v, :cols]))
+            assert np.array_equal(bits(ob[v, :rows]), bits(want)), (qt, rows, cols, n_vec, int(v))
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_random_prefill_and_lookup(oxh, seed):
+    """oxh_mmq (9..300 activations; Q4_K, Q5_K, Q6_K) with padded output stride, and
+    oxh_get_rows over random ids for every type."""
+    rng = np.random.default_rng(9000 + seed)
+    o = oxlibs.oracle()
+    qt = (13, 15, 16, 12, 14)[seed % 5]
+    layout = BASE.get(qt, qt)
+    cols = int(rng.integers(1, 20)) * 256
+    rows = int(rng.integers(1, 500))
+    n_vec = int(rng.integers(9, 301))
+    stride = rows + int(rng.integers(0, 3)) * 4
+    w = synth.weights(layout, rows, cols, seed=seed, stream=1)
+    xs = synth.normal(n_vec * cols, seed=seed, stream=2).reshape(n_vec, cols)
+    d_w, d_x = mv.DeviceBuffer.from_host(w), mv.DeviceBuffer.from_host(xs)
+    d_a = mv.DeviceBuffer(n_vec * mv.act_bytes(qt, cols))
+    d_o = mv.DeviceBuffer(n_vec * stride * 4)
+    d_o.upload(np.full(n_vec * stride, -3.5, np.float32))
+    mv.quantize(qt, d_x.ptr, cols, n_vec, cols, d_a.ptr)
+    mv.mmq(qt, d_w.ptr, rows, cols, d_a.ptr, n_vec, d_o.ptr, stride)
+    mv.sync()
+    got = d_o.download(np.float32, n_vec * stride).reshape(n_vec, stride)
+    assert np.all(got[:, rows:] == -3.5)
+    for v in list(rng.choice(n_vec, size=5, replace=False)) + [0, n_vec - 1]:
+        want, _ = oracle_rows(qt, layout, w, rows, cols, np.ascontiguousarray(xs[v]))
+        assert np.array_equal(bits(got[v, :rows]), bits(want)), (qt, rows, cols, n_vec, int(v))
+    # embedding lookup, any type
+    qt2 = int(TYPES[seed % len(TYPES)])
+    lay2 = BASE.get(qt2, qt2)
+    group = synth.BLOCK_ELEMS[lay2]
+    cols2 = int(rng.integers(1, 12)) * (256 if group == 256 else 32 * int(rng.integers(1, 9)))
+    rows2 = int(rng.integers(1, 200))
+    rb2 = synth.row_bytes(lay2, cols2)
+    w2 = synth.weights(lay2, rows2, cols2, seed=seed, stream=3)
+    ids = rng.integers(0, rows2, size=int(rng.integers(1, 40))).astype(np.uint32)
+    d_w2, d_ids = mv.DeviceBuffer.from_host(w2), mv.DeviceBuffer.from_host(ids)
+    d_r = mv.DeviceBuffer(ids.size * cols2 * 4)
+    mv.get_rows(qt2, d_w2.ptr, rows2, cols2, d_ids.ptr, ids.size, d_r.ptr, cols2)
+    got = d_r.download(np.float32, ids.size * cols2).reshape(ids.size, cols2)
+    for k, i in enumerate(ids):
+        deq = np.zeros(cols2, np.float32)
+        assert o.oxo_dequant_row(qt2, w2[int(i) * rb2:].ctypes.data, cols2, deq.ctypes.data) == 0
+        assert np.array_equal(bits(got[k]), bits(deq)), (qt2, cols2, int(i))
