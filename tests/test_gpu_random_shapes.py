@@ -178,3 +178,71 @@ def test_random_prefill_and_lookup(oxh, seed):
         deq = np.zeros(cols2, np.float32)
         assert o.oxo_dequant_row(qt2, w2[int(i) * rb2:].ctypes.data, cols2, deq.ctypes.data) == 0
         assert np.array_equal(bits(got[k]), bits(deq)), (qt2, cols2, int(i))
+
+
+@pytest.mark.parametrize("seed", range(51))
+def test_random_fused_prologue_launch(oxh, seed):
+    """RMSNorm, residual add + RMSNorm or SwiGLU in front of any weight type, one to three
+    segments, one to four input vectors, optionally a paired gate/up segment.  The float
+    step is read back from the device; from there on everything is exact: the quantised
+    bytes, plain segments' outputs, and the two halves of a pair before silu(gate)*up."""
+    rng = np.random.default_rng(7000 + seed)
+    o = oxlibs.oracle()
+    qt = int(TYPES[seed % len(TYPES)])
+    layout = BASE.get(qt, qt)
+    group = synth.BLOCK_ELEMS[layout]
+    cols = int(rng.integers(1, 17 if group == 256 else 60)) * group
+    n_vec = int(rng.integers(1, 5))
+    kind = ("rms", "add_rms", "swiglu")[seed % 3]
+    n_segs = int(rng.integers(1, 4))
+    rows = [int(rng.integers(1, 250)) for _ in range(n_segs)]
+    paired = [bool(rng.integers(0, 2)) and seed % 4 == 0 for _ in range(n_segs)]
+    ws = [synth.weights(layout, r, cols, seed=seed, stream=2 * i) for i, r in enumerate(rows)]
+    w2 = [synth.weights(layout, r, cols, seed=seed, stream=2 * i + 1) if p else None
+          for i, (r, p) in enumerate(zip(rows, paired))]
+    xs = (synth.normal(n_vec * cols, seed=seed, stream=90) * np.float32(1.7)).reshape(n_vec, cols)
+    b = synth.normal((n_vec if kind == "swiglu" else 1) * cols, seed=seed, stream=91)
+    add = synth.normal(n_vec * cols, seed=seed, stream=92).reshape(n_vec, cols)
+    d_ws = [mv.DeviceBuffer.from_host(w) for w in ws]
+    d_w2 = [mv.DeviceBuffer.from_host(w) if w is not None else None for w in w2]
+    d_x, d_b, d_add = mv.DeviceBuffer.from_host(xs), mv.DeviceBuffer.from_host(b), mv.DeviceBuffer.from_host(add)
+    nact = mv.act_bytes(qt, cols)
+    d_y, d_sum = mv.DeviceBuffer(n_vec * cols * 4), mv.DeviceBuffer(n_vec * cols * 4)
+    d_a = mv.DeviceBuffer(n_vec * nact)
+    stride = max(rows)
+    d_o = mv.DeviceBuffer(n_segs * n_vec * stride * 4)
+    items = [(d_w.ptr, d_o.ptr + i * n_vec * stride * 4, r, 0, 0, None if p is None else p.ptr)
+             for i, (d_w, r, p) in enumerate(zip(d_ws, rows, d_w2))]
+    eps = 1e-5
+    mv.gemv_segments_fused(qt, mv.make_segments(items), cols, d_x.ptr, cols,
+                           mv.PRO_SWIGLU if kind == "swiglu" else mv.PRO_RMSNORM, d_b.ptr, eps, d_y.ptr, d_a.ptr,
+                           n_vec, stride, None, d_add.ptr if kind == "add_rms" else None,
+                           d_sum.ptr if kind == "add_rms" else None)
+    mv.sync()
+    y = d_y.download(np.float32, n_vec * cols).reshape(n_vec, cols)
+    acts = d_a.download(np.uint8, n_vec * nact).reshape(n_vec, nact)
+    out = d_o.download(np.float32, n_segs * n_vec * stride).reshape(n_segs, n_vec, stride)
+    for v in range(n_vec):                                      # the float step, to rounding
+        want = np.zeros(cols, np.float32)
+        if kind == "swiglu":
+            o.oxo_swiglu_f32(xs[v].ctypes.data, b[v * cols:].ctypes.data, want.ctypes.data, cols)
+        else:
+            src = xs[v] + add[v] if kind == "add_rms" else xs[v]
+            src = np.ascontiguousarray(src, np.float32)
+            if kind == "add_rms":
+                got_sum = d_sum.download(np.float32, n_vec * cols).reshape(n_vec, cols)[v]
+                assert np.array_equal(bits(got_sum), bits(src))
+            o.oxo_rms_norm_f32(src.ctypes.data, b.ctypes.data, want.ctypes.data, cols, eps)
+        assert np.all(np.abs(y[v] - want) <= 4e-6 * np.abs(want) + 1e-30), (kind, v)
+    for i, (w, wp, r) in enumerate(zip(ws, w2, rows)):          # the integer path, exactly
+        for v in range(n_vec):
+            yv = np.ascontiguousarray(y[v])
+            want, temp = oracle_rows(qt, layout, w, r, cols, yv)
+            assert np.array_equal(acts[v], temp.view(np.uint8)[:nact])
+            if wp is None:
+                assert np.array_equal(bits(out[i, v, :r]), bits(want)), (qt, kind, i, v)
+            else:
+                up, _ = oracle_rows(qt, layout, wp, r, cols, yv)
+                h = np.zeros(r, np.float32)
+                o.oxo_swiglu_f32(want.ctypes.data, up.ctypes.data, h.ctypes.data, r)
+                assert np.all(np.abs(out[i, v, :r] - h) <= 4e-6 * np.abs(h) + 1e-30), (qt, kind, i, v)
