@@ -268,3 +268,17 @@ def test_argument_checks(oxh):
                                       None))                                  # workspace too small
     with pytest.raises(mv.OxhError):
         mv.moe_route(d.ptr, 4, 65, 2, 1, d.ptr, d.ptr, d.ptr, d.ptr, d.ptr, d.ptr)
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_random_layers(oxh, seed):
+    """Random expert counts (1..64), top-k, widths, token counts and type pairs, stage by stage."""
+    rng = np.random.default_rng(300 + seed)
+    n_exp = int(rng.integers(1, 65))
+    k = int(rng.integers(1, min(8, n_exp) + 1))
+    hidden, ffn = int(rng.integers(1, 4)) * 256, int(rng.integers(1, 4)) * 256
+    n_tok = int(rng.integers(1, 70))
+    qt_gu = (Q4K, Q5K, Q6K)[int(rng.integers(0, 3))]
+    qt_dn = (Q4K, Q5K, Q6K)[int(rng.integers(0, 3))]
+    check_layer(qt_gu, qt_dn, n_exp, k, hidden, ffn, n_tok, seed=40 + seed, renorm=seed & 1,
+                skew=n_exp >= 3 and k < n_exp - 1)
