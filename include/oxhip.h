@@ -59,6 +59,7 @@ extern "C" {
 #define OXH_Q5_K_M 15u
 #define OXH_Q6_K   16u
 #define OXH_AL5    17u     /* the Q4_0 block layout under its own id (quantization.c:207-214) */
+#define OXH_AL5_XS 18u     /* f16 d + thirty-two 3-bit codes (oxk.h:55) */
 #define OXH_AL6    19u     /* the Q5_0 layout */
 #define OXH_AL8    20u     /* the Q8_0 layout */
 #define OXH_QTYPE_UNKNOWN 0xffffffffu
@@ -69,6 +70,7 @@ extern "C" {
 #define OXH_Q4_K_BYTES   144u
 #define OXH_Q5_K_BYTES   176u
 #define OXH_Q6_K_BYTES   210u
+#define OXH_AL5_XS_BYTES  14u
 #define OXH_Q2_K_BYTES    84u
 #define OXH_Q3_K_BYTES   110u
 #define OXH_Q8_0_BYTES    34u

@@ -468,6 +468,37 @@ static float dot_legacy(int five_bit, int has_min, const uint8_t *row, size_t bl
     return sum;
 }
 
+/* the 3-bit code of element i: bits [3i, 3i+3) of the 12 packed bytes, least
+ * significant bit first (src/compute/oxk.c:206-218) */
+static unsigned al5_xs_code(const uint8_t *packed, unsigned i)
+{
+    unsigned v = 0;
+    for (unsigned bb = 0; bb < 3; bb++) {
+        const unsigned bit = 3u * i + bb;
+        v |= ((packed[bit >> 3] >> (bit & 7u)) & 1u) << bb;
+    }
+    return v;
+}
+
+float oxo_dot_al5_xs_q8_0(const uint8_t *row, size_t blocks, const uint8_t *act, int32_t *isum)
+{
+    float sum = 0.0f;
+    for (size_t b = 0; b < blocks; b++) {
+        const uint8_t *w = row + b * OXO_AL5_XS_BYTES;
+        const uint8_t *a = act + b * OXO_Q8_0_BYTES;
+        const float dw = oxo_f16_to_f32(rd_u16(w));
+        const float dq = oxo_f16_to_f32(rd_u16(a));
+        const int8_t *q = (const int8_t *)(a + 2);
+        int32_t acc = 0;
+        for (unsigned i = 0; i < 32; i++)
+            acc += ((int32_t)al5_xs_code(w + 2, i) - 4) * (int32_t)q[i];
+        if (isum) isum[b] = acc;
+        const float t = dw * dq;
+        sum += t * (float)acc;
+    }
+    return sum;
+}
+
 float oxo_dot_q4_0_q8_0(const uint8_t *row, size_t blocks, const uint8_t *act, int32_t *isum)
 {
     return dot_legacy(0, 0, row, blocks, act, isum);
@@ -498,6 +529,7 @@ static size_t block_bytes(uint32_t qtype)
     case OXO_Q5_1:   return 24u;
     case OXO_AL8:
     case OXO_Q8_0:   return OXO_Q8_0_BYTES;
+    case OXO_AL5_XS: return OXO_AL5_XS_BYTES;
     case OXO_Q4_K_S:
     case OXO_Q4_K_M: return OXO_Q4_K_BYTES;
     case OXO_Q5_K_S:
@@ -521,7 +553,8 @@ int oxo_act_kind(uint32_t qtype, size_t cols)
     case OXO_AL6:
     case OXO_Q5_1:
     case OXO_Q8_0:
-    case OXO_AL8:    return (cols % OXO_QK8_0 == 0) ? 1 : 0;
+    case OXO_AL8:
+    case OXO_AL5_XS: return (cols % OXO_QK8_0 == 0) ? 1 : 0;
     case OXO_Q2_K:
     case OXO_Q3_K_S:
     case OXO_Q3_K_M:
@@ -560,6 +593,7 @@ static float row_dot(uint32_t qtype, const uint8_t *row, size_t blocks,
     case OXO_Q5_1:   return oxo_dot_q5_1_q8_0(row, blocks, act, NULL);
     case OXO_AL8:
     case OXO_Q8_0:   return oxo_dot_q8_0_q8_0(row, blocks, act, NULL);
+    case OXO_AL5_XS: return oxo_dot_al5_xs_q8_0(row, blocks, act, NULL);
     case OXO_Q6_K:   return oxo_dot_q6_k_q8_k(row, blocks, act, NULL);
     case OXO_Q2_K:   return oxo_dot_q2_k_q8_k(row, blocks, act, NULL);
     case OXO_Q3_K_S:
@@ -767,6 +801,12 @@ int oxo_dequant_row(uint32_t qtype, const uint8_t *row, size_t cols, float *out)
                 if (has_m) out[32 * b + e] = (float)code * d + m;
                 else       out[32 * b + e] = (float)((int)code - (has_h ? 16 : 8)) * d;
             }
+        } else if (qtype == OXO_AL5_XS) {
+            /* src/compute/quantization.c:802-832 */
+            const uint8_t *w = row + b * OXO_AL5_XS_BYTES;
+            const float d = oxo_f16_to_f32(rd_u16(w));
+            for (unsigned i = 0; i < 32; i++)
+                out[32 * b + i] = (float)((int32_t)al5_xs_code(w + 2, i) - 4) * d;
         } else if (qtype == OXO_Q2_K) {
             /* src/compute/quantization.c:521-561 */
             const uint8_t *w = row + b * OXO_Q2_K_BYTES;

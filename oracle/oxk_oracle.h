@@ -61,12 +61,14 @@ enum {
     OXO_Q5_K_M = 15,
     OXO_Q6_K   = 16,
     OXO_AL5    = 17,    /* Q4_0 layout */
+    OXO_AL5_XS = 18,    /* f16 d + 32 three-bit codes in 12 bytes */
     OXO_AL6    = 19,    /* Q5_0 layout */
     OXO_AL8    = 20,    /* Q8_0 layout */
 };
 
 #define OXO_QK_K        256u
 #define OXO_QK8_0       32u
+#define OXO_AL5_XS_BYTES 14u
 #define OXO_Q2_K_BYTES  84u
 #define OXO_Q3_K_BYTES  110u
 #define OXO_Q4_K_BYTES  144u
@@ -121,6 +123,8 @@ float oxo_dot_q4_0_q8_0(const uint8_t *row, size_t blocks, const uint8_t *act, i
 float oxo_dot_q4_1_q8_0(const uint8_t *row, size_t blocks, const uint8_t *act, int32_t *isum);
 float oxo_dot_q5_0_q8_0(const uint8_t *row, size_t blocks, const uint8_t *act, int32_t *isum);
 float oxo_dot_q5_1_q8_0(const uint8_t *row, size_t blocks, const uint8_t *act, int32_t *isum);
+/* src/compute/oxk.c:195-222: codes 0..7 with an offset of 4, (dw*dq) * (float)isum per block */
+float oxo_dot_al5_xs_q8_0(const uint8_t *row, size_t blocks, const uint8_t *act, int32_t *isum);
 
 /* 0 = not eligible for the integer path, 1 = Q8_0 activation, 2 = Q8_K
  * (src/compute/matvec.c:99-127 restricted to the types above) and the stride

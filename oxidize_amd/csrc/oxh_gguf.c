@@ -92,7 +92,7 @@ static const TypeRow k_types[] = {
     { 240, OXH_AL5, 32, 18 },
     { 241, OXH_AL8, 32, 34 },
     { 242, OXH_AL6, 32, 22 },
-    { 243, 18, 32, 14 },   /* AL5_XS */
+    { 243, OXH_AL5_XS, 32, OXH_AL5_XS_BYTES },
 };
 
 static const TypeRow *type_row(uint32_t ggml_id)

@@ -279,7 +279,7 @@ k_quantize_q8_0(const float *__restrict__ x, size_t in_stride, uint32_t blocks_p
  * the bit.  One wave per 256 values, lane l producing values 4l .. 4l+3 (they
  * share a sub-block / scale group); grid.y walks the ids.  An id beyond the
  * matrix yields a row of zeros rather than a read outside it.
- * KIND: 0 Q4_K, 1 Q5_K, 2 Q6_K, 3 Q8_0, 4 Q4_0, 5 Q4_1, 6 Q5_0, 7 Q5_1, 8 Q2_K, 9 Q3_K. */
+ * KIND: 0 Q4_K, 1 Q5_K, 2 Q6_K, 3 Q8_0, 4 Q4_0, 5 Q4_1, 6 Q5_0, 7 Q5_1, 8 Q2_K, 9 Q3_K, 10 AL5_XS. */
 template <int KIND>
 __global__ __launch_bounds__(256) void
 k_get_rows(const uint8_t *__restrict__ w, uint32_t rows, uint32_t cols, uint32_t row_bytes,
@@ -294,7 +294,19 @@ k_get_rows(const uint8_t *__restrict__ w, uint32_t rows, uint32_t cols, uint32_t
     float v[4] = { 0.0f, 0.0f, 0.0f, 0.0f };
     if (id < rows) {
         const uint8_t *row = w + (size_t)id * row_bytes;
-        if (KIND >= 8) {
+        if (KIND == 10) {
+            /* thirty-two 3-bit codes behind an f16 d, element i at bits [3i, 3i+3) (quantization.c:802-832):
+             * this lane's four codes are twelve bits starting at bit 3*(e0 % 32), inside one or two of the
+             * block's six 16-bit words */
+            const uint8_t *blk = row + (size_t)(e0 >> 5) * 14u;
+            const float d = half_to_float_hw(*reinterpret_cast<const uint16_t *>(blk));
+            const uint32_t bit = 3u * (e0 & 31u), word = bit >> 4;          /* bit = 12 * (lane % 8) */
+            const uint32_t lo16 = *reinterpret_cast<const uint16_t *>(blk + 2u + 2u * word);
+            const uint32_t hi16 = word < 5u ? *reinterpret_cast<const uint16_t *>(blk + 4u + 2u * word) : 0u;
+            const uint32_t c = ((lo16 | (hi16 << 16)) >> (bit & 15u)) & 0xFFFu;
+#pragma unroll
+            for (int i = 0; i < 4; i++) v[i] = (float)((int)((c >> (3 * i)) & 7u) - 4) * d;
+        } else if (KIND >= 8) {
             /* 2-bit codes: element 128n + 32k + l is bits [2k, 2k+2) of qs[32n + l]; Q3_K adds bit
              * 4n + k of hmask[l] as the third bit (quantization.c:521-630) */
             const uint8_t *blk = row + (size_t)unit * (KIND == 9 ? 110u : 84u);
@@ -485,6 +497,7 @@ extern "C" int oxh_act_kind(uint32_t qtype, size_t cols)
     case OXH_Q4_1:
     case OXH_Q5_0:
     case OXH_Q5_1:
+    case OXH_AL5_XS:
     case OXH_Q8_0:   return (cols % OXH_QK8_0 == 0) ? 1 : 0;
     case OXH_Q2_K:
     case OXH_Q3_K_M:
@@ -504,6 +517,7 @@ static size_t block_bytes(uint32_t qtype)
     case OXH_Q4_1:   return OXH_Q4_1_BYTES;
     case OXH_Q5_0:   return OXH_Q5_0_BYTES;
     case OXH_Q5_1:   return OXH_Q5_1_BYTES;
+    case OXH_AL5_XS: return OXH_AL5_XS_BYTES;
     case OXH_Q8_0:   return OXH_Q8_0_BYTES;
     case OXH_Q4_K_S:
     case OXH_Q4_K_M: return OXH_Q4_K_BYTES;
@@ -616,6 +630,7 @@ static hipError_t raise_all_lds_ceilings(void)
     OXH_RAISE(k_gemv_q4_1)
     OXH_RAISE(k_gemv_q5_0)
     OXH_RAISE(k_gemv_q5_1)
+    OXH_RAISE(k_gemv_al5_xs)
 #undef OXH_RAISE
 #define OXH_RAISE_PRO1(KERNEL, PRO)                                                               \
     if ((e = raise_lds_ceiling(KERNEL<1, PRO, false>)) != hipSuccess) return e;                   \
@@ -637,6 +652,7 @@ static hipError_t raise_all_lds_ceilings(void)
     OXH_RAISE_PRO(k_gemv_q4_1_pro)
     OXH_RAISE_PRO(k_gemv_q5_0_pro)
     OXH_RAISE_PRO(k_gemv_q5_1_pro)
+    OXH_RAISE_PRO(k_gemv_al5_xs_pro)
 #undef OXH_RAISE_PRO
 #undef OXH_RAISE_PRO1
     if ((e = raise_lds_ceiling(k_mmq_q4_k<8, 2, 8>)) != hipSuccess) return e;
@@ -1013,6 +1029,7 @@ static int launch_gemv(uint32_t qtype, const OxhSegment *segs, size_t n_segs, si
     else if (qtype == OXH_Q4_1) OXH_LAUNCH_ANY(k_gemv_q4_1, k_gemv_q4_1_pro);
     else if (qtype == OXH_Q5_0) OXH_LAUNCH_ANY(k_gemv_q5_0, k_gemv_q5_0_pro);
     else if (qtype == OXH_Q5_1) OXH_LAUNCH_ANY(k_gemv_q5_1, k_gemv_q5_1_pro);
+    else if (qtype == OXH_AL5_XS) OXH_LAUNCH_ANY(k_gemv_al5_xs, k_gemv_al5_xs_pro);
     else                        OXH_LAUNCH_ANY(k_gemv_q8_0, k_gemv_q8_0_pro);
 #undef OXH_LAUNCH_ANY
 #undef OXH_LAUNCH_PRO
@@ -1247,6 +1264,7 @@ extern "C" int oxh_get_rows(uint32_t qtype, const void *d_w, size_t rows, size_t
     else if (qtype == OXH_Q4_1) OXH_GET_ROWS(5);
     else if (qtype == OXH_Q5_0) OXH_GET_ROWS(6);
     else if (qtype == OXH_Q5_1) OXH_GET_ROWS(7);
+    else if (qtype == OXH_AL5_XS) OXH_GET_ROWS(10);
     else if (qtype == OXH_Q2_K) OXH_GET_ROWS(8);
     else if (qtype == OXH_Q3_K_M) OXH_GET_ROWS(9);
     else                        OXH_GET_ROWS(3);

@@ -233,7 +233,7 @@ def dequant_rows(ref):
     np.savez_compressed(os.path.join(HERE, "dequant_rows.npz"), **out)
 
 
-LEGACY = (("q4_0", 3, 18), ("q4_1", 4, 20), ("q5_0", 5, 22), ("q5_1", 6, 24))
+LEGACY = (("q4_0", 3, 18), ("q4_1", 4, 20), ("q5_0", 5, 22), ("q5_1", 6, 24), ("al5_xs", 18, 14))
 
 
 ALIASES = (("al5", 17, 3), ("al6", 19, 5), ("al8", 20, 7))
@@ -279,6 +279,11 @@ def legacy_formats(ref):
         out[name + "_api_shape"] = np.array([rows, cols, rb], np.int64)
         out[name + "_api_out"] = o.copy()
         out[name + "_api_act"] = temp.view(np.uint8)[:cols // 32 * 34].copy()
+        if name == "al5_xs":
+            deq = np.zeros((2, cols), np.float32)
+            for r in range(2):
+                assert ref.oc_quant_dequant_row(qt, wm[r * rb:].ctypes.data, rb, deq[r].ctypes.data, cols) == 0
+            out[name + "_dequant_bits"] = deq.view(np.uint32).copy()
     # AL5 / AL6 / AL8: the Q4_0 / Q5_0 / Q8_0 layouts under their own type ids
     for name, qt, base in ALIASES:
         rows, cols = 24, 896

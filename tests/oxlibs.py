@@ -44,7 +44,7 @@ def oracle():
         lib.oxo_dot_q8_0_q8_0.argtypes = [V, Z, V, V]; lib.oxo_dot_q8_0_q8_0.restype = F
         lib.oxo_dot_q2_k_q8_k.argtypes = [V, Z, V, V]; lib.oxo_dot_q2_k_q8_k.restype = F
         lib.oxo_dot_q3_k_q8_k.argtypes = [V, Z, V, V]; lib.oxo_dot_q3_k_q8_k.restype = F
-        for n in ("q4_0", "q4_1", "q5_0", "q5_1"):
+        for n in ("q4_0", "q4_1", "q5_0", "q5_1", "al5_xs"):
             f = getattr(lib, "oxo_dot_%s_q8_0" % n)
             f.argtypes = [V, Z, V, V]; f.restype = F
         lib.oxo_act_kind.argtypes = [U32, Z]; lib.oxo_act_kind.restype = ctypes.c_int
@@ -84,7 +84,7 @@ def ref():
         lib.oc_oxk_get_scale_min_k4.argtypes = [ctypes.c_uint, V, V, V]
         lib.oc_oxk_get_scale_min_k4.restype = None
         for n in ("q2_k_q8_k", "q3_k_q8_k", "q4_k_q8_k", "q5_k_q8_k", "q6_k_q8_k", "q8_0_q8_0", "q4_0_q8_0", "q4_1_q8_0", "q5_0_q8_0",
-                  "q5_1_q8_0"):
+                  "q5_1_q8_0", "al5_xs_q8_0"):
             for suf in ("", "_scalar"):
                 f = getattr(lib, "oc_oxk_dot_" + n + suf)
                 f.argtypes = [V, Z, V]; f.restype = F

@@ -341,7 +341,8 @@ def test_prequantised_and_fused_paths_agree(oxh, qtype, rows, cols, n_vec):
 
 @pytest.mark.parametrize("qtype,rows,cols", [(Q4K, 1000, 4096), (15, 300, 1024), (Q6K, 500, 2816), (Q80, 2000, 896),
                                              (Q80, 64, 32), (Q4K, 7, 256), (3, 300, 896), (4, 300, 896),
-                                             (5, 300, 896), (6, 300, 896), (5, 9, 32), (6, 9, 1056)])
+                                             (5, 300, 896), (6, 300, 896), (5, 9, 32), (6, 9, 1056), (18, 200, 896),
+                                             (18, 3, 32)])
 def test_embedding_rows_bit_identical_to_the_cpu_dequantisation(oxh, qtype, rows, cols):
     """oxh_get_rows against the oracle's dequantisation (itself bit-identical
     to the compiled reference's oc_quant_dequant_row): ids on the device, first
@@ -408,7 +409,7 @@ def test_q8_0_small_batches_on_the_matrix_cores(oxh, rows, cols, nvs):
 
 
 @pytest.mark.parametrize("qtype,size", [(Q4K, 144), (15, 176), (Q6K, 210), (Q80, 34), (8, 84), (10, 110), (3, 18),
-                                        (4, 20), (5, 22), (6, 24)])
+                                        (4, 20), (5, 22), (6, 24), (18, 14)])
 def test_every_weight_byte_influences_its_row(oxh, qtype, size):
     """oxidize-c/tests/test_quant.c:569-583 as a kernel test: one row per byte of
     a block, that byte altered; every row must differ from the unaltered one

@@ -1,5 +1,5 @@
-"""GPU parity for the 32-value formats Q4_0, Q4_1, Q5_0 and Q5_1 (type ids 3-6,
-Q8_0 activations) through the C ABI.
+"""GPU parity for the 32-value formats Q4_0, Q4_1, Q5_0, Q5_1 (type ids 3-6) and
+AL5_XS (id 18; 3-bit codes), Q8_0 activations, through the C ABI.
 
 Bars: Q8_0 activation bytes and the per-block integers bit-exact; f32 outputs
 bit-exact against the oracle's block-sequential chain (oxk.c:88-191) and within
@@ -17,7 +17,7 @@ from oxidize_amd import synth
 pytestmark = pytest.mark.gpu
 
 GOLD = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "legacy_formats.npz")
-LEGACY = (("q4_0", 3), ("q4_1", 4), ("q5_0", 5), ("q5_1", 6))
+LEGACY = (("q4_0", 3), ("q4_1", 4), ("q5_0", 5), ("q5_1", 6), ("al5_xs", 18))
 FLOAT_RTOL = 4e-6
 
 

@@ -13,7 +13,7 @@ from oxidize_amd import synth
 
 pytestmark = pytest.mark.gpu
 
-TYPES = (3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15, 16, 17, 19, 20)
+TYPES = (3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15, 16, 17, 18, 19, 20)
 BASE = {17: 3, 19: 5, 20: 7, 9: 10, 11: 10, 12: 13, 14: 15}      # ids that share another id's layout
 
 

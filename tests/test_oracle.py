@@ -634,9 +634,10 @@ def test_dequant_row_bits_vs_reference(name, qt):
 
 
 LEGACY = (("q4_0", 3, 18), ("q4_1", 4, 20), ("q5_0", 5, 22), ("q5_1", 6, 24))
+LEGACY_ALL = LEGACY + (("al5_xs", 18, 14),)
 
 
-@pytest.mark.parametrize("name,qt,bsize", LEGACY)
+@pytest.mark.parametrize("name,qt,bsize", LEGACY_ALL)
 def test_legacy_formats_vs_reference_goldens(name, qt, bsize):
     g = load("legacy_formats.npz")
     fo = getattr(O, "oxo_dot_%s_q8_0" % name)
@@ -657,6 +658,41 @@ def test_legacy_formats_vs_reference_goldens(name, qt, bsize):
     assert np.array_equal(temp.view(np.uint8)[:a.size], a)
     want = g[name + "_api_out"]
     assert np.all(np.abs(out - want) <= 1e-4 + 1e-5 * np.abs(want))
+
+
+def test_al5_xs_closed_form_placement_and_dequant():
+    """Thirty-two 3-bit codes, least significant bit first, offset 4
+    (oxidize-c/src/compute/oxk.c:195-222): all-equal blocks, one code at a time,
+    and the dequantised rows of the compiled reference."""
+    d, dq, a = 0.5, 0.25, 3
+    act = np.concatenate([np.array(f16_le(dq), np.uint8), np.full(32, a, np.int8).view(np.uint8)])
+    for code in range(8):
+        bits_ = "".join(format(code, "03b")[::-1] for _ in range(32))
+        packed = np.array([int(bits_[8 * i:8 * i + 8][::-1], 2) for i in range(12)], np.uint8)
+        blk = np.concatenate([np.array(f16_le(d), np.uint8), packed])
+        assert O.oxo_dot_al5_xs_q8_0(blk.ctypes.data, 1, act.ctypes.data, None) == d * dq * 32 * (code - 4) * a
+    rng = np.random.default_rng(9)
+    q = rng.integers(-127, 128, 32).astype(np.int8)
+    act = np.concatenate([np.array(f16_le(1.0), np.uint8), q.view(np.uint8)])
+    base_blk = np.zeros(14, np.uint8)
+    base_blk[0:2] = f16_le(1.0)
+    base = O.oxo_dot_al5_xs_q8_0(base_blk.ctypes.data, 1, act.ctypes.data, None)
+    assert base == float(-4 * int(q.sum()))
+    for e in range(32):
+        for bit in range(3):
+            blk = base_blk.copy()
+            pos = 3 * e + bit
+            blk[2 + pos // 8] = 1 << (pos % 8)
+            isum = np.zeros(1, np.int32)
+            got = O.oxo_dot_al5_xs_q8_0(blk.ctypes.data, 1, act.ctypes.data, isum.ctypes.data)
+            assert got == base + float((1 << bit) * int(q[e])), (e, bit)
+    g = load("legacy_formats.npz")
+    rows, cols, rb = (int(v) for v in g["al5_xs_api_shape"])
+    wm = g["al5_xs_api_w"]
+    for r in range(2):
+        deq = np.zeros(cols, np.float32)
+        assert O.oxo_dequant_row(18, wm[r * rb:].ctypes.data, cols, deq.ctypes.data) == 0
+        assert np.array_equal(deq.view(np.uint32), g["al5_xs_dequant_bits"][r])
 
 
 @pytest.mark.parametrize("name,qt,base", [("al5", 17, 3), ("al6", 19, 5), ("al8", 20, 7)])
