@@ -519,7 +519,7 @@ int oxh_matvec_quantized_batch(uint32_t qtype, const uint8_t *data, size_t rows,
         if ((rc = oxh_mmq(qtype, d_w, rows, cols, g_dact.p, n_vec, (float *)g_dout.p, rows, NULL)))
             return rc;
     } else {
-        size_t step = oxh_gemv_max_nvec(qtype, cols);
+        size_t step = oxh_gemv_max_nvec_buffered(qtype, cols);
         if (step == 0) {
             oxh_set_error("batch: cols too wide for one workgroup%s%s", NULL, NULL);
             return OXH_ERR_TOO_WIDE;

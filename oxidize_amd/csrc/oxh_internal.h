@@ -17,6 +17,9 @@ void *oxh_internal_stream(void);
 /* Largest n_vec (1..8) one GEMV launch can stage for (qtype, cols); 0 when
  * even a single activation does not fit. */
 size_t oxh_gemv_max_nvec(uint32_t qtype, size_t cols);
+/* The same for a launch that passes a buffer for the quantised activations
+ * (up to 16 for Q8_0 weights, which then run on the matrix cores). */
+size_t oxh_gemv_max_nvec_buffered(uint32_t qtype, size_t cols);
 
 #ifdef __cplusplus
 }

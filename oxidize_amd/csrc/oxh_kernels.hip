@@ -729,6 +729,17 @@ extern "C" size_t oxh_gemv_max_nvec(uint32_t qtype, size_t cols)
     return nv;
 }
 
+/* Q8_0 launches that hand over a buffer for the quantised activations run on the MFMA kernel
+ * from five activations on, and that kernel takes up to sixteen. */
+extern "C" size_t oxh_gemv_max_nvec_buffered(uint32_t qtype, size_t cols)
+{
+    const size_t plain = oxh_gemv_max_nvec(qtype, cols);
+    if (canon_qtype(qtype) != OXH_Q8_0 || plain == 0) return plain;
+    static const uint32_t min_nv = env_u32("OXH_Q80_MFMA_MIN_NV", 5, 0, 64);
+    if (min_nv == 0 || min_nv > MQ80_TOK) return plain;
+    return (size_t)mq80_lds_bytes((uint32_t)(cols / OXH_QK8_0), MQ80_TOK, 4u) <= GEMV_LDS_LIMIT ? MQ80_TOK : plain;
+}
+
 struct GemvIo {
     const void *d_acts;     /* pre-quantised activations, or NULL            */
     const float *d_x;       /* f32 inputs to quantise in the kernel, or NULL */
@@ -868,7 +879,7 @@ static int launch_gemv(uint32_t qtype, const OxhSegment *segs, size_t n_segs, si
     qtype = canon_qtype(qtype);
     if (n_segs == 0) return OXH_OK;
     if (!segs || (!io.d_acts && !io.d_x)) return arg_fail("gemv: NULL pointer");
-    if (n_vec < 1 || n_vec > OXH_MAX_NV) return arg_fail("gemv: n_vec must be 1..8");
+    if (n_vec < 1 || n_vec > MQ80_TOK) return arg_fail("gemv: n_vec must be 1..8");
     const size_t n_vec_default = n_vec;
     if (n_segs > OXH_MAX_SEGS) return arg_fail("gemv: more than 32 segments in one launch");
     const int kind = oxh_act_kind(qtype, cols);
@@ -890,7 +901,7 @@ static int launch_gemv(uint32_t qtype, const OxhSegment *segs, size_t n_segs, si
     size_t total_work = 0;
     for (size_t i = 0; i < n_segs; i++) {
         const size_t nv = segs[i].n_vec ? segs[i].n_vec : n_vec;
-        if (nv < 1 || nv > OXH_MAX_NV) return arg_fail("gemv: segment n_vec must be 1..8");
+        if (nv < 1 || nv > MQ80_TOK) return arg_fail("gemv: segment n_vec must be 1..8");
         if (segs[i].rows) {
             if (nv > max_nv) max_nv = nv;
             if (nv != 1) all_one = false;
@@ -911,6 +922,10 @@ static int launch_gemv(uint32_t qtype, const OxhSegment *segs, size_t n_segs, si
     if (!any_pair && q80_wants_mfma(qtype, io, max_nv, blocks, dump))
         return launch_q80_mfma_segments(segs, n_segs, cols, blocks, io, n_vec_default, act_end,
                                         out_stride, stream);
+    /* only that kernel takes 9 to 16 activations per weight */
+    if (max_nv > OXH_MAX_NV)
+        return arg_fail("gemv: n_vec must be 1..8 (up to 16 only where the launch runs on the matrix cores: "
+                        "Q4_K, Q5_K, Q6_K or Q8_0 weights with a buffer for the quantised activations)");
     n_vec = max_nv;                        /* sizes LDS from here on */
     if (out_stride > 0xFFFFFFFFull || io.x_stride > 0xFFFFFFFFull || max_act + n_vec > 0xFFFFFFFFull)
         return arg_fail("gemv: stride too large");

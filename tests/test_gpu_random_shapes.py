@@ -21,7 +21,7 @@ def bits(a):
     return np.ascontiguousarray(a).view(np.uint32)
 
 
-@pytest.mark.parametrize("seed", range(136))
+@pytest.mark.parametrize("seed", range(144))
 def test_random_launch(oxh, seed):
     rng = np.random.default_rng(1000 + seed)
     qt = int(TYPES[seed % len(TYPES)])
@@ -31,11 +31,15 @@ def test_random_launch(oxh, seed):
     cols = blocks * group
     n_segs = int(rng.integers(1, 5))
     rows = [int(rng.integers(1, 300)) for _ in range(n_segs)]
+    with_buffer = bool(seed & 1)
+    # with a buffer for the quantised activations these types run on the matrix cores, up to 16 per weight
+    wide = with_buffer and layout in (7, 13, 15, 16)
     nvs = [int(rng.integers(1, 9)) for _ in range(n_segs)]
+    if wide:
+        nvs[0] = int(rng.integers(9, 17))
     firsts = [int(rng.integers(0, 4)) for _ in range(n_segs)]
     n_act = max(f + n for f, n in zip(firsts, nvs))
     pad = int(rng.integers(0, 3)) * 4
-    with_buffer = bool(seed & 1)
     ws = [synth.weights(layout, r, cols, seed=seed, stream=i) for i, r in enumerate(rows)]
     xs = synth.normal(n_act * cols, seed=seed, stream=77).reshape(n_act, cols)
     d_ws = [mv.DeviceBuffer.from_host(w) for w in ws]
