@@ -154,8 +154,8 @@ int oxh_gemv_segments(uint32_t qtype, const OxhSegment *segs, size_t n_segs,
  * oxh_act_bytes() per vector, indexed like d_x; room for every vector up to
  * the largest act_first + n_vec of any segment), and launches of several
  * vectors per weight may then run on the matrix cores (Q4_K, Q5_K, Q6_K from
- * three vectors, Q8_0 from five), which also lifts the limit on n_vec from 8
- * to 16. */
+ * three vectors, the 32-value formats from five), which also lifts the limit
+ * on n_vec from 8 to 16. */
 int oxh_gemv_segments_f32(uint32_t qtype, const OxhSegment *segs, size_t n_segs,
                           size_t cols, const float *d_x, size_t x_stride,
                           void *d_act_out, size_t n_vec, size_t out_stride,

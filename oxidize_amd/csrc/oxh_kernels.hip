@@ -661,7 +661,12 @@ static hipError_t raise_all_lds_ceilings(void)
     if ((e = raise_lds_ceiling(k_mmq_q5_k<4, 1, 8>)) != hipSuccess) return e;
     if ((e = raise_lds_ceiling(k_mmq_q6_k<8, 1, 8>)) != hipSuccess) return e;
     if ((e = raise_lds_ceiling(k_mmq_q6_k<4, 1, 8>)) != hipSuccess) return e;
-    if ((e = raise_lds_ceiling(k_mfma_q8_0_segments<4>)) != hipSuccess) return e;
+    if ((e = raise_lds_ceiling(k_mfma_q8_0_segments<4, 0>)) != hipSuccess) return e;
+    if ((e = raise_lds_ceiling(k_mfma_q8_0_segments<4, 1>)) != hipSuccess) return e;
+    if ((e = raise_lds_ceiling(k_mfma_q8_0_segments<4, 2>)) != hipSuccess) return e;
+    if ((e = raise_lds_ceiling(k_mfma_q8_0_segments<4, 3>)) != hipSuccess) return e;
+    if ((e = raise_lds_ceiling(k_mfma_q8_0_segments<4, 4>)) != hipSuccess) return e;
+    if ((e = raise_lds_ceiling(k_mfma_q8_0_segments<4, 5>)) != hipSuccess) return e;
     if ((e = raise_lds_ceiling(k_mmq_q6_k_segments<1, 1, 4, 2>)) != hipSuccess) return e;
     if ((e = raise_lds_ceiling(k_mmq_q6_k_experts<1, 1, 4, 2>)) != hipSuccess) return e;
     return hipSuccess;
@@ -729,12 +734,13 @@ extern "C" size_t oxh_gemv_max_nvec(uint32_t qtype, size_t cols)
     return nv;
 }
 
-/* Q8_0 launches that hand over a buffer for the quantised activations run on the MFMA kernel
- * from five activations on, and that kernel takes up to sixteen. */
+/* Launches over a 32-value format that hand over a buffer for the quantised activations run on the
+ * MFMA kernel from five activations on, and that kernel takes up to sixteen. */
 extern "C" size_t oxh_gemv_max_nvec_buffered(uint32_t qtype, size_t cols)
 {
     const size_t plain = oxh_gemv_max_nvec(qtype, cols);
-    if (canon_qtype(qtype) != OXH_Q8_0 || plain == 0) return plain;
+    if (oxh_act_kind(qtype, 32) != 1 || plain == 0) return plain;
+    if (cols / OXH_QK8_0 * block_bytes(qtype) < 16u) return plain;
     static const uint32_t min_nv = env_u32("OXH_Q80_MFMA_MIN_NV", 5, 0, 64);
     if (min_nv == 0 || min_nv > MQ80_TOK) return plain;
     return (size_t)mq80_lds_bytes((uint32_t)(cols / OXH_QK8_0), MQ80_TOK, 4u) <= GEMV_LDS_LIMIT ? MQ80_TOK : plain;
@@ -774,20 +780,22 @@ static bool mmq_deep_stages(uint32_t wg)
     return wg <= 2u * (uint32_t)(g_n_cu > 0 ? g_n_cu : 256);
 }
 
-/* Q8_0 launches with five or more activations per weight go to the MFMA kernel
- * (OXH_Q80_MFMA_MIN_NV moves the threshold, 0 = never) when the quantised
- * activations exist or have somewhere to go and the staged activations fit LDS. */
+/* Launches over a 32-value format (Q8_0, Q4_0, Q4_1, Q5_0, Q5_1, AL5_XS) with five or more
+ * activations per weight go to the MFMA kernel (OXH_Q80_MFMA_MIN_NV moves the threshold, 0 = never)
+ * when the quantised activations exist or have somewhere to go and the staged activations fit LDS. */
 static bool q80_wants_mfma(uint32_t qtype, const GemvIo &io, size_t max_nv, size_t blocks, const int32_t *dump)
 {
     static int min_nv = -1;
     if (min_nv < 0) min_nv = (int)env_u32("OXH_Q80_MFMA_MIN_NV", 5, 0, 64);
-    if (qtype != OXH_Q8_0 || dump || io.pro || min_nv == 0 || max_nv < (size_t)min_nv || max_nv > MQ80_TOK)
+    if (oxh_act_kind(qtype, 32) != 1 || dump || io.pro || min_nv == 0 || max_nv < (size_t)min_nv ||
+        max_nv > MQ80_TOK)
         return false;
+    if (blocks * block_bytes(qtype) < 16u) return false;        /* rows shorter than one 16-byte piece */
     if ((size_t)mq80_lds_bytes((uint32_t)blocks, max_nv > 8 ? 16u : 8u, 4u) > GEMV_LDS_LIMIT) return false;
     return io.d_acts != nullptr || io.d_act_out != nullptr;
 }
 
-static int launch_q80_mfma_segments(const OxhSegment *segs, size_t n_segs, size_t cols, size_t blocks,
+static int launch_q80_mfma_segments(uint32_t qtype, const OxhSegment *segs, size_t n_segs, size_t cols, size_t blocks,
                                     const GemvIo &io, size_t n_vec_default, size_t n_acts, size_t out_stride,
                                     void *stream)
 {
@@ -815,8 +823,19 @@ static int launch_q80_mfma_segments(const OxhSegment *segs, size_t n_segs, size_
     for (uint32_t i = 1; i < 4 && i < n; i++) t.bound[i - 1] = t.s[i].wg_begin;
     uint32_t toks = 8u;
     for (uint32_t i = 0; i < n; i++) if (t.s[i].nv > 8u) toks = 16u;
-    hipLaunchKernelGGL((k_mfma_q8_0_segments<4>), dim3(wg), dim3(256), mq80_lds_bytes((uint32_t)blocks, toks, 4u),
-                       pick_stream(stream), t, (uint32_t)blocks, acts, out_stride, toks);
+    const size_t lds = mq80_lds_bytes((uint32_t)blocks, toks, 4u);
+    hipStream_t st = pick_stream(stream);
+#define OXH_MQ80(LEG) hipLaunchKernelGGL((k_mfma_q8_0_segments<4, LEG>), dim3(wg), dim3(256), lds, st, t, \
+                                         (uint32_t)blocks, acts, out_stride, toks)
+    switch (qtype) {
+    case OXH_Q4_0:   OXH_MQ80(1); break;
+    case OXH_Q4_1:   OXH_MQ80(2); break;
+    case OXH_Q5_0:   OXH_MQ80(3); break;
+    case OXH_Q5_1:   OXH_MQ80(4); break;
+    case OXH_AL5_XS: OXH_MQ80(5); break;
+    default:         OXH_MQ80(0); break;
+    }
+#undef OXH_MQ80
     HIP_TRY(hipGetLastError());
     return OXH_OK;
 }
@@ -920,12 +939,12 @@ static int launch_gemv(uint32_t qtype, const OxhSegment *segs, size_t n_segs, si
         return launch_mmq_segments(qtype, segs, n_segs, cols, blocks, io, n_vec_default, act_end,
                                    out_stride, stream);
     if (!any_pair && q80_wants_mfma(qtype, io, max_nv, blocks, dump))
-        return launch_q80_mfma_segments(segs, n_segs, cols, blocks, io, n_vec_default, act_end,
+        return launch_q80_mfma_segments(qtype, segs, n_segs, cols, blocks, io, n_vec_default, act_end,
                                         out_stride, stream);
     /* only that kernel takes 9 to 16 activations per weight */
     if (max_nv > OXH_MAX_NV)
         return arg_fail("gemv: n_vec must be 1..8 (up to 16 only where the launch runs on the matrix cores: "
-                        "Q4_K, Q5_K, Q6_K or Q8_0 weights with a buffer for the quantised activations)");
+                        "not Q2_K or Q3_K, a buffer for the quantised activations, staged activations within LDS)");
     n_vec = max_nv;                        /* sizes LDS from here on */
     if (out_stride > 0xFFFFFFFFull || io.x_stride > 0xFFFFFFFFull || max_act + n_vec > 0xFFFFFFFFull)
         return arg_fail("gemv: stride too large");

@@ -371,37 +371,38 @@ def test_embedding_rows_bit_identical_to_the_cpu_dequantisation(oxh, qtype, rows
     assert e.value.status == mv.DECLINED
 
 
+@pytest.mark.parametrize("fmt", [Q80, 3, 4, 5, 6, 18])
 @pytest.mark.parametrize("rows,cols,nvs", [(151, 896, (5, 8)), (64, 32, (8,)), (1000, 4864, (6, 8)), (33, 2048, (7, 5)),
-                                           (4864, 896, (8, 8, 5))])
-def test_q8_0_small_batches_on_the_matrix_cores(oxh, rows, cols, nvs):
-    """Q8_0 launches with five or more activations per weight and a buffer for
+                                           (4864, 896, (8, 8, 5)), (70, 2336, (16, 9)), (20, 64, (12,))])
+def test_q8_0_small_batches_on_the_matrix_cores(oxh, fmt, rows, cols, nvs):
+    """Launches over a 32-value format with five or more activations per weight and a buffer for
     their quantised form run on the int8 MFMA kernel: per-block integers exact,
     f32 the block-sequential chain, so every output carries the oracle's bits.
     One segment per entry of `nvs`, each with its own run of activations and
     its own count; ragged rows; the same launch with fewer than five
     activations (dot-instruction kernel) as a cross-check of the segment logic."""
-    rb = synth.row_bytes(Q80, cols)
+    rb = synth.row_bytes(fmt, cols)
     n_act = sum(nvs)
-    ws = [synth.weights(Q80, rows, cols, seed=71, stream=i) for i in range(len(nvs))]
+    ws = [synth.weights(fmt, rows, cols, seed=71, stream=i) for i in range(len(nvs))]
     xs = synth.normal(n_act * cols, seed=71, stream=9).reshape(n_act, cols)
     d_ws = [mv.DeviceBuffer.from_host(w) for w in ws]
     d_x = mv.DeviceBuffer.from_host(xs)
-    d_act = mv.DeviceBuffer(n_act * mv.act_bytes(Q80, cols))
+    d_act = mv.DeviceBuffer(n_act * mv.act_bytes(fmt, cols))
     d_out = mv.DeviceBuffer(n_act * rows * 4)
     d_out.upload(np.full(n_act * rows, np.nan, np.float32))
     items, first = [], 0
     for d_w, nv in zip(d_ws, nvs):
         items.append((d_w.ptr, d_out.ptr + first * rows * 4, rows, first, nv))
         first += nv
-    mv.gemv_segments_f32(Q80, mv.make_segments(items), cols, d_x.ptr, cols, d_act.ptr, max(nvs), rows)
+    mv.gemv_segments_f32(fmt, mv.make_segments(items), cols, d_x.ptr, cols, d_act.ptr, max(nvs), rows)
     mv.sync()
     got = d_out.download(np.float32, n_act * rows).reshape(n_act, rows)
     o = oxlibs.oracle()
-    acts = d_act.download(np.uint8, n_act * mv.act_bytes(Q80, cols)).reshape(n_act, -1)
+    acts = d_act.download(np.uint8, n_act * mv.act_bytes(fmt, cols)).reshape(n_act, -1)
     first = 0
     for w, nv in zip(ws, nvs):
         for v in range(first, first + nv):
-            want, temp = oracle_matvec(Q80, w, rows, cols, np.ascontiguousarray(xs[v]))
+            want, temp = oracle_matvec(fmt, w, rows, cols, np.ascontiguousarray(xs[v]))
             assert np.array_equal(acts[v], temp.view(np.uint8)[:acts.shape[1]])
             assert np.array_equal(bits(got[v]), bits(want)), (nv, v)
         first += nv
