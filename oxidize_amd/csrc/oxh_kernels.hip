@@ -669,6 +669,9 @@ static hipError_t raise_all_lds_ceilings(void)
     if ((e = raise_lds_ceiling(k_mfma_q8_0_segments<4, 5>)) != hipSuccess) return e;
     if ((e = raise_lds_ceiling(k_mmq_q6_k_segments<1, 1, 4, 2>)) != hipSuccess) return e;
     if ((e = raise_lds_ceiling(k_mmq_q6_k_experts<1, 1, 4, 2>)) != hipSuccess) return e;
+    if ((e = raise_lds_ceiling(k_mmq_q6_k_experts<4, 1, 8, 1>)) != hipSuccess) return e;
+    if ((e = raise_lds_ceiling(k_mmq_q45_k_experts<4, 1, 8, false, 1>)) != hipSuccess) return e;
+    if ((e = raise_lds_ceiling(k_mmq_q45_k_experts<4, 1, 8, true, 1>)) != hipSuccess) return e;
     return hipSuccess;
 }
 
@@ -1392,21 +1395,26 @@ extern "C" int oxh_moe_route(const float *d_logits, size_t n_tok, size_t n_exper
 }
 
 /* one launch of the MFMA tile kernel over all experts, activation runs from device memory */
-static int launch_experts(uint32_t qtype, const void *const *d_w, float *const *d_out, size_t n_mat,
-                          size_t n_expert, size_t rows, size_t cols, const void *d_acts, size_t out_stride,
-                          const uint32_t *d_counts, const uint32_t *d_offsets, void *stream)
+/* one or more launches of the MFMA tile kernel over all experts, activation runs from device memory.
+ * `avg_tokens` = pairs per expert on average: from about two dozen on, the 128-row x 64-token tile
+ * (eight waves) re-streams an expert's weights four times less often than the 64 x 16 one. */
+template <int TC, int WAVES>
+static int launch_experts_tiled(uint32_t qtype, const void *const *d_w, float *const *d_out, size_t n_mat,
+                                size_t n_expert, size_t rows, size_t cols, const void *d_acts, size_t out_stride,
+                                const uint32_t *d_counts, const uint32_t *d_offsets, void *stream)
 {
-    typedef MmqGeom<1, 1, 4> G;
+    typedef MmqGeom<TC, 1, WAVES> G;
+    typedef Mmq6Geom<TC, 1, WAVES> G6;
+    typedef MmqGeom<TC, 1, WAVES, true> G5;
+    static_assert(G6::ROWS == G::ROWS && G5::ROWS == G::ROWS, "row tiling is shared by all formats");
     const size_t blocks = cols / OXH_QK_K;
     if (blocks * 292u * 256u > 0xFFFFFFFFull) return arg_fail("moe: cols too large");
     const size_t rb = oxh_row_bytes(qtype, cols);
     const uint8_t *acts = (const uint8_t *)d_acts;
     hipStream_t st = pick_stream(stream);
-    typedef Mmq6Geom<1, 1, 4> G6;
-    typedef MmqGeom<1, 1, 4, true> G5;
     const uint32_t nb = (uint32_t)blocks;
 #define OXH_EXP_LAUNCH(KERNEL, GEOM, KB)                                                              \
-    hipLaunchKernelGGL(KERNEL, dim3(wg), dim3(256), (KB) * GEOM::LDS_BYTES, st, t, nb, acts, out_stride, \
+    hipLaunchKernelGGL(KERNEL, dim3(wg), dim3(WAVES * 64), (KB) * GEOM::LDS_BYTES, st, t, nb, acts, out_stride, \
                        d_counts, d_offsets)
     /* one segment per expert and matrix, at most OXH_MAX_SEGS of them per launch */
     const size_t per_launch = OXH_MAX_SEGS / n_mat;
@@ -1427,19 +1435,32 @@ static int launch_experts(uint32_t qtype, const void *const *d_w, float *const *
             }
         t.n = n;
         for (uint32_t i = 1; i < 4 && i < n; i++) t.bound[i - 1] = t.s[i].wg_begin;
-        if (mmq_deep_stages(wg)) {
-            if (qtype == OXH_Q6_K) OXH_EXP_LAUNCH((k_mmq_q6_k_experts<1, 1, 4, 2>), G6, 2);
-            else if (is_q5k(qtype)) OXH_EXP_LAUNCH((k_mmq_q45_k_experts<1, 1, 4, true, 2>), G5, 2);
-            else OXH_EXP_LAUNCH((k_mmq_q45_k_experts<1, 1, 4, false, 2>), G, 2);
+        /* two super-blocks per stage only for the small tile (the large one has no LDS to spare) */
+        if (TC == 1 && mmq_deep_stages(wg)) {
+            if (qtype == OXH_Q6_K) OXH_EXP_LAUNCH((k_mmq_q6_k_experts<TC, 1, WAVES, TC == 1 ? 2 : 1>), G6, TC == 1 ? 2 : 1);
+            else if (is_q5k(qtype)) OXH_EXP_LAUNCH((k_mmq_q45_k_experts<TC, 1, WAVES, true, TC == 1 ? 2 : 1>), G5, TC == 1 ? 2 : 1);
+            else OXH_EXP_LAUNCH((k_mmq_q45_k_experts<TC, 1, WAVES, false, TC == 1 ? 2 : 1>), G, TC == 1 ? 2 : 1);
         } else {
-            if (qtype == OXH_Q6_K) OXH_EXP_LAUNCH((k_mmq_q6_k_experts<1, 1, 4, 1>), G6, 1);
-            else if (is_q5k(qtype)) OXH_EXP_LAUNCH((k_mmq_q45_k_experts<1, 1, 4, true, 1>), G5, 1);
-            else OXH_EXP_LAUNCH((k_mmq_q45_k_experts<1, 1, 4, false, 1>), G, 1);
+            if (qtype == OXH_Q6_K) OXH_EXP_LAUNCH((k_mmq_q6_k_experts<TC, 1, WAVES, 1>), G6, 1);
+            else if (is_q5k(qtype)) OXH_EXP_LAUNCH((k_mmq_q45_k_experts<TC, 1, WAVES, true, 1>), G5, 1);
+            else OXH_EXP_LAUNCH((k_mmq_q45_k_experts<TC, 1, WAVES, false, 1>), G, 1);
         }
     }
 #undef OXH_EXP_LAUNCH
     HIP_TRY(hipGetLastError());
     return OXH_OK;
+}
+
+static int launch_experts(uint32_t qtype, const void *const *d_w, float *const *d_out, size_t n_mat,
+                          size_t n_expert, size_t rows, size_t cols, const void *d_acts, size_t out_stride,
+                          const uint32_t *d_counts, const uint32_t *d_offsets, size_t avg_tokens, void *stream)
+{
+    static const uint32_t big_from = env_u32("OXH_MOE_BIG_TILE_FROM", 24, 0, 4096);     /* 0 = never */
+    if (big_from && avg_tokens >= big_from)
+        return launch_experts_tiled<4, 8>(qtype, d_w, d_out, n_mat, n_expert, rows, cols, d_acts, out_stride,
+                                          d_counts, d_offsets, stream);
+    return launch_experts_tiled<1, 4>(qtype, d_w, d_out, n_mat, n_expert, rows, cols, d_acts, out_stride,
+                                      d_counts, d_offsets, stream);
 }
 
 extern "C" int oxh_moe_ffn(const OxhMoe *m, const float *d_logits, const float *d_x, size_t x_stride,
@@ -1470,14 +1491,15 @@ extern "C" int oxh_moe_ffn(const OxhMoe *m, const float *d_logits, const float *
     /* 3. gate and up of every expert over its own pairs */
     const void *w_gu[2] = { m->d_w_gate, m->d_w_up };
     float *o_gu[2] = { gate, up };
+    const size_t avg_tokens = pairs / m->n_expert;
     if ((rc = launch_experts(m->qtype_gate_up, w_gu, o_gu, 2, m->n_expert, m->ffn, m->hidden, ws + l.act_x,
-                             m->ffn, counts, offsets, stream))) return rc;
+                             m->ffn, counts, offsets, avg_tokens, stream))) return rc;
     /* 4. h = silu(gate) * up, quantised; 5. down */
     if ((rc = quantize_q8_k_ex(gate, m->ffn, pairs, m->ffn, ws + l.act_h, nullptr, up, stream))) return rc;
     const void *w_dn[1] = { m->d_w_down };
     float *o_dn[1] = { y };
     if ((rc = launch_experts(m->qtype_down, w_dn, o_dn, 1, m->n_expert, m->hidden, m->ffn, ws + l.act_h,
-                             m->hidden, counts, offsets, stream))) return rc;
+                             m->hidden, counts, offsets, avg_tokens, stream))) return rc;
     /* 6. combine in ascending expert order */
     hipLaunchKernelGGL(k_moe_combine, dim3((uint32_t)((m->hidden + 255u) / 256u), (uint32_t)n_tok), dim3(256), 0,
                        pick_stream(stream), (const float *)y, m->hidden, (const int32_t *)ids, (const float *)wts,

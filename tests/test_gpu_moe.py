@@ -236,6 +236,15 @@ def test_layer_top1_and_all_experts(oxh):
     check_layer(Q4K, Q6K, 16, 8, 256, 512, 6, seed=4, renorm=1, skew=False)
 
 
+@pytest.mark.parametrize("qt_gu,qt_dn", [(Q4K, Q6K), (Q5K, Q4K), (Q6K, Q5K)])
+def test_layer_with_prefill_sized_token_counts(oxh, qt_gu, qt_dn):
+    """150 pairs per expert on average: the expert launches take the 128-row x 64-token tile and walk
+    three token tiles per expert, the popular expert more."""
+    check_layer(qt_gu, qt_dn, 4, 2, 512, 768, 300, seed=21, sample=lambda n, offsets: sorted(
+        set(int(v) for v in offsets[:-1] if v < n) | set(int(v) - 1 for v in offsets[1:] if v > 0) |
+        set(range(0, n, 37))))
+
+
 def test_layer_with_more_experts_than_one_launch_carries(oxh):
     """40 and 64 experts: the gate/up launch carries 16 experts, the down launch 32, so both repeat."""
     check_layer(Q4K, Q4K, 40, 4, 256, 256, 50, seed=8, skew=True)
