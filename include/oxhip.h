@@ -211,6 +211,16 @@ int oxh_mmq(uint32_t qtype, const void *d_w, size_t rows, size_t cols,
             const void *d_acts, size_t n_vec, float *d_out, size_t out_stride,
             void *stream);
 
+/* A Q3_K matrix rewritten as a Q6_K matrix that gives bit-identical results:
+ * Q3_K's d * (sc - 32) * (code - 4) is Q6_K's d * sc6 * (code6 - 32) with
+ * code6 = code + 28 and sc6 = sc - 32, over the same groups in the same
+ * element order, and the two block terms (oxidize-c/src/compute/oxk.c:624-652,
+ * :913-964) are the same float of the same integer.  The reference prepares
+ * Q3_K rows into its Q6_K batch layout the same way (oxk.c:734-745).  Lets a
+ * prefill over Q3_K weights run on oxh_mmq(OXH_Q6_K, ...); d_q6k must hold
+ * rows * (cols/256) * 210 bytes. */
+int oxh_q3_k_as_q6_k(const void *d_w, size_t rows, size_t cols, void *d_q6k, void *stream);
+
 /* Embedding lookup: out[t*out_stride ..] = row d_ids[t] of a packed matrix,
  * expanded to f32 in the reference's dequantisation arithmetic (bit-identical
  * to oc_quant_dequant_row, oxidize-c/src/compute/quantization.c:2781-2795), so

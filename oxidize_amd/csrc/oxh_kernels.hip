@@ -418,6 +418,70 @@ k_read_probe(const u32x4 *__restrict__ p, size_t n16, uint32_t *__restrict__ sin
     if ((acc.x ^ acc.y ^ acc.z ^ acc.w) == 0x5EED5EEDu && sink) *sink = 1u;
 }
 
+/* Q3_K rows rewritten as Q6_K rows, exactly.  A Q3_K weight is d * (sc - 32) * (code - 4) with a
+ * 3-bit code; Q6_K's is d * sc6 * (code6 - 32) with a 6-bit code and an int8 scale, over the same
+ * sixteen groups in the same element order (element 128n + 32k + l).  With code6 = code + 28 and
+ * sc6 = sc - 32 the two are the same integer times the same d, so the block term
+ * d*dq*(float)(pos - 4*off) of oxk.c:624-652 and d*dq*(float)(pos - 32*minc) of oxk.c:913-964 are the
+ * same float: the reference itself prepares Q3_K rows into its Q6_K batch layout (oxk.c:734-745).
+ * Four lanes per block, split like the Q6_K GEMV: lane (n, lh) owns l = 16lh .. 16lh+15 of half n.
+ *   low nibble of code + 28:  q2 | 12 when the third bit h is 0 (28 + q2 = 16 + 12 + q2), q2 when it
+ *   is 1 (32 + q2);  upper two bits: 1 when h = 0, 2 when h = 1. */
+__global__ __launch_bounds__(256) void
+k_q3k_to_q6k(const uint8_t *__restrict__ src, uint8_t *__restrict__ dst, uint32_t n_blocks)
+{
+    const uint32_t t = blockIdx.x * 256u + threadIdx.x;
+    const uint32_t b = t >> 2, u = t & 3u, n = u >> 1, lh = u & 1u;
+    if (b >= n_blocks) return;
+    const uint8_t *s = src + (size_t)b * 110u;
+    uint8_t *d = dst + (size_t)b * 210u;
+    const U32x4u2 hm = *reinterpret_cast<const U32x4u2 *>(s + 16u * lh);
+    const U32x4u2 qs = *reinterpret_cast<const U32x4u2 *>(s + 32u + 32u * n + 16u * lh);
+    const uint32_t h4[4] = { hm.x, hm.y, hm.z, hm.w }, q4[4] = { qs.x, qs.y, qs.z, qs.w };
+    uint32_t la[4], lb[4], hh[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        uint32_t nib[4], hi2[4];
+#pragma unroll
+        for (uint32_t k = 0; k < 4u; k++) {
+            const uint32_t q2 = (q4[i] >> (2u * k)) & 0x03030303u;
+            const uint32_t h = (h4[i] >> (4u * n + k)) & 0x01010101u;
+            const uint32_t nh = h ^ 0x01010101u;
+            nib[k] = q2 | (nh << 2) | (nh << 3);
+            hi2[k] = (h << 1) | nh;
+        }
+        la[i] = nib[0] | (nib[2] << 4);
+        lb[i] = nib[1] | (nib[3] << 4);
+        hh[i] = hi2[0] | (hi2[1] << 2) | (hi2[2] << 4) | (hi2[3] << 6);
+    }
+    U32x4u2 o;
+    o.x = la[0]; o.y = la[1]; o.z = la[2]; o.w = la[3];
+    *reinterpret_cast<U32x4u2 *>(d + 64u * n + 16u * lh) = o;
+    o.x = lb[0]; o.y = lb[1]; o.z = lb[2]; o.w = lb[3];
+    *reinterpret_cast<U32x4u2 *>(d + 64u * n + 32u + 16u * lh) = o;
+    o.x = hh[0]; o.y = hh[1]; o.z = hh[2]; o.w = hh[3];
+    *reinterpret_cast<U32x4u2 *>(d + 128u + 32u * n + 16u * lh) = o;
+    if (u == 0u) {
+        /* the sixteen 6-bit scales (oxk.c:556-573), minus 32, as int8; then d */
+        const U32u2 *p = reinterpret_cast<const U32u2 *>(s + 96u);
+        const uint32_t a0 = p[0].v, a1 = p[1].v, tt = p[2].v;
+        uint32_t w[4];
+        w[0] = (a0 & 0x0F0F0F0Fu) | ((tt & 0x03030303u) << 4);
+        w[1] = (a1 & 0x0F0F0F0Fu) | (((tt >> 2) & 0x03030303u) << 4);
+        w[2] = ((a0 >> 4) & 0x0F0F0F0Fu) | (((tt >> 4) & 0x03030303u) << 4);
+        w[3] = ((a1 >> 4) & 0x0F0F0F0Fu) | (((tt >> 6) & 0x03030303u) << 4);
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            /* x - 32 per byte, x in 0..63: clear bit 5 when set, else set the top three bits */
+            const uint32_t below = (~w[i]) & 0x20202020u;
+            w[i] = (w[i] & 0x1F1F1F1Fu) | below | (below << 1) | (below << 2);
+        }
+        o.x = w[0]; o.y = w[1]; o.z = w[2]; o.w = w[3];
+        *reinterpret_cast<U32x4u2 *>(d + 192u) = o;
+        *reinterpret_cast<uint16_t *>(d + 208u) = *reinterpret_cast<const uint16_t *>(s + 108u);
+    }
+}
+
 #include "gemv_kernels.inc"
 #include "mmq_kernels.inc"
 #include "moe_kernels.inc"
@@ -1306,6 +1370,22 @@ extern "C" int oxh_get_rows(uint32_t qtype, const void *d_w, size_t rows, size_t
     else if (qtype == OXH_Q3_K_M) OXH_GET_ROWS(9);
     else                        OXH_GET_ROWS(3);
 #undef OXH_GET_ROWS
+    HIP_TRY(hipGetLastError());
+    return OXH_OK;
+}
+
+extern "C" int oxh_q3_k_as_q6_k(const void *d_w, size_t rows, size_t cols, void *d_q6k, void *stream)
+{
+    int rc = ensure_init();
+    if (rc) return rc;
+    if (rows == 0) return OXH_OK;
+    if (!d_w || !d_q6k) return arg_fail("oxh_q3_k_as_q6_k: NULL pointer");
+    if (cols == 0 || cols % OXH_QK_K) return arg_fail("oxh_q3_k_as_q6_k: cols must be a whole number of 256-blocks");
+    const size_t blocks = cols / OXH_QK_K;
+    if (rows > 0x3FFFFFFFull / blocks) return arg_fail("oxh_q3_k_as_q6_k: matrix too large");
+    const uint32_t n_blocks = (uint32_t)(rows * blocks);
+    hipLaunchKernelGGL(k_q3k_to_q6k, dim3((n_blocks * 4u + 255u) / 256u), dim3(256), 0, pick_stream(stream),
+                       (const uint8_t *)d_w, (uint8_t *)d_q6k, n_blocks);
     HIP_TRY(hipGetLastError());
     return OXH_OK;
 }

@@ -226,6 +226,11 @@ class MoeLayer:
         return dict(zip(self.PARTS, [int(x) for x in v]))
 
 
+def q3_k_as_q6_k(d_w, rows, cols, d_q6k, stream=None):
+    """Rewrite a Q3_K matrix as a Q6_K one with bit-identical results (for oxh_mmq)."""
+    check(lib().oxh_q3_k_as_q6_k(ctypes.c_void_p(d_w), rows, cols, ctypes.c_void_p(d_q6k), stream))
+
+
 def read_probe(d_buf, nbytes, stream=None):
     """One launch that only reads `nbytes` at d_buf (measurement aid)."""
     check(lib().oxh_debug_read_probe(ctypes.c_void_p(d_buf), nbytes, None, stream))

@@ -252,3 +252,46 @@ def test_declines_what_the_reference_declines(oxh):
     assert mv.matvec_quantized(Q2K, w, 4, 300, 84, x, out, temp) == mv.DECLINED      # cols not in whole blocks
     x = np.zeros(256, np.float32)
     assert mv.matvec_quantized(Q3K, w, 3, 256, 112, x, out, temp) == mv.DECLINED     # padded row stride
+
+
+def test_q3k_rewritten_as_q6k_bytes(oxh):
+    """The device rewrite against the element-by-element numpy statement: raw random blocks (every
+    scale value, every third-bit pattern) and generator blocks, block counts that do and do not fill
+    the last workgroup."""
+    from q3k_rewrite import q3k_as_q6k
+    g = np.load(GOLD)
+    raw = np.ascontiguousarray(g["q3_k_raw_w"]).reshape(-1)                 # 288 blocks
+    rng = np.random.default_rng(3)
+    rnd = rng.integers(0, 256, 110 * 1027, dtype=np.uint8)
+    for w, rows, cols in ((raw, 24, 12 * 256), (rnd, 1027, 256), (rnd[:110], 1, 256),
+                          (synth.weights(Q3K, 130, 2048, seed=8), 130, 2048)):
+        d_w = mv.DeviceBuffer.from_host(w)
+        d_o = mv.DeviceBuffer(rows * (cols // 256) * 210)
+        mv.q3_k_as_q6_k(d_w.ptr, rows, cols, d_o.ptr)
+        assert np.array_equal(d_o.download(np.uint8, rows * (cols // 256) * 210), q3k_as_q6k(w))
+    with pytest.raises(Exception):
+        mv.q3_k_as_q6_k(d_w.ptr, 1, 200, d_o.ptr)
+    mv.q3_k_as_q6_k(0, 0, 256, 0)           # no rows: nothing to do
+
+
+@pytest.mark.parametrize("qt,rows,cols,n_vec", [(Q3K, 300, 2048, 9), (Q3KS, 65, 256, 16), (Q3KL, 1, 512, 33),
+                                                (Q3K, 1000, 4096, 100), (Q3K, 4096, 4096, 512)])
+def test_q3k_prefill_batches_on_the_matrix_cores(oxh, qt, rows, cols, n_vec):
+    """More than eight vectors of Q3_K weights go through the rewrite and the Q6_K tile kernel: every
+    output still has the bits of the single-vector Q3_K dot."""
+    rb = synth.row_bytes(qt, cols)
+    w = synth.weights(qt, rows, cols, seed=61, stream=n_vec)
+    in_stride, out_stride = cols + 8, rows + 3
+    xb = synth.normal(n_vec * in_stride, seed=62, stream=n_vec).reshape(n_vec, in_stride)
+    ob = np.full((n_vec, out_stride), -1.0, np.float32)
+    temp = np.zeros(cols, np.float32)
+    scratch = np.zeros(mv.batch_scratch_bytes(cols), np.uint8)
+    assert mv.matvec_quantized_batch(qt, w, rows, cols, rb, xb, in_stride, ob, out_stride, n_vec, temp,
+                                     scratch) == 0
+    assert np.all(ob[:, rows:] == -1.0)
+    o = oxlibs.oracle()
+    want = np.zeros((n_vec, out_stride), np.float32)
+    act = np.zeros(scratch.size, np.uint8)
+    assert o.oxo_matvec_quantized_batch(qt, w.ctypes.data, rows, cols, rb, xb.ctypes.data, in_stride,
+                                        want.ctypes.data, out_stride, n_vec, act.ctypes.data, act.size) == 0
+    assert np.array_equal(bits(ob[:, :rows]), bits(want[:, :rows]))

@@ -327,6 +327,30 @@ def test_q23_k_raw_block_dots_float_bits_vs_reference(name):
             assert got == g[name + "_raw_dispatched_bits"][t, k]
 
 
+def test_q3_k_rewritten_as_q6_k_is_the_same_dot_and_the_same_row():
+    # the rewrite the batch path of the library uses for Q3_K weights: the Q6_K dot of the rewritten
+    # blocks has the float bits of the Q3_K dot (which the reference vectors above pin), and the rows
+    # dequantise to the same floats
+    from q3k_rewrite import q3k_as_q6k
+    g = load("q23_k.npz")
+    w, act = g["q3_k_raw_w"], g["q3_k_raw_act"]
+    for t in range(w.shape[0]):
+        at = np.ascontiguousarray(act[t])
+        w6 = q3k_as_q6k(w[t])
+        for k, blocks in enumerate((1, w.shape[1])):
+            got = f32bits(O.oxo_dot_q6_k_q8_k(w6.ctypes.data, blocks, at.ctypes.data, None))
+            assert got == g["q3_k_raw_scalar_bits"][t, k]
+    rows, cols = 9, 1024
+    w3 = synth.weights(10, rows, cols, seed=77)
+    w6 = q3k_as_q6k(w3)
+    a = np.zeros((rows, cols), np.float32)
+    b = np.zeros((rows, cols), np.float32)
+    for r in range(rows):
+        assert O.oxo_dequant_row(10, w3[r * (cols // 256) * 110:].ctypes.data, cols, a[r].ctypes.data) == 0
+        assert O.oxo_dequant_row(16, w6[r * (cols // 256) * 210:].ctypes.data, cols, b[r].ctypes.data) == 0
+    assert np.array_equal(a.view(np.uint32), b.view(np.uint32))
+
+
 @pytest.mark.parametrize("qt", [8, 9, 10, 11])
 def test_q23_k_matvec_batch_and_dequant_vs_reference_goldens(qt):
     g = load("q23_k.npz")
