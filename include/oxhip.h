@@ -221,6 +221,16 @@ int oxh_mmq(uint32_t qtype, const void *d_w, size_t rows, size_t cols,
  * rows * (cols/256) * 210 bytes. */
 int oxh_q3_k_as_q6_k(const void *d_w, size_t rows, size_t cols, void *d_q6k, void *stream);
 
+/* A Q2_K matrix widened for the matrix cores: 210-byte blocks whose 6-bit
+ * fields hold scale * code (at most 45), followed by the sixteen group minima
+ * as nibbles, dmin and d (oxk.c:592-622 gives the arithmetic: the block term
+ * dq * (d * sum sc*code*q - dmin * sum m*bsum), which the tile kernel
+ * reproduces to the bit).  The result is not a GGUF type: oxh_mmq accepts it
+ * under OXH_Q2_K_WIDE and nothing else does.  d_wide must hold
+ * rows * (cols/256) * 210 bytes. */
+#define OXH_Q2_K_WIDE 0x1008u
+int oxh_q2_k_widen(const void *d_w, size_t rows, size_t cols, void *d_wide, void *stream);
+
 /* Embedding lookup: out[t*out_stride ..] = row d_ids[t] of a packed matrix,
  * expanded to f32 in the reference's dequantisation arithmetic (bit-identical
  * to oc_quant_dequant_row, oxidize-c/src/compute/quantization.c:2781-2795), so

@@ -63,6 +63,7 @@ SIGNATURES = {
     "oxh_debug_subblock_sums": (I, [U32, V, Z, Z, V, V, V]),
     "oxh_debug_read_probe": (I, [V, Z, V, V]),
     "oxh_q3_k_as_q6_k": (I, [V, Z, Z, V, V]),
+    "oxh_q2_k_widen": (I, [V, Z, Z, V, V]),
     "oxh_moe_workspace_bytes": (I, [ctypes.POINTER(OxhMoe), Z, ctypes.POINTER(Z)]),
     "oxh_moe_ffn": (I, [ctypes.POINTER(OxhMoe), V, V, Z, Z, V, Z, V, Z, V]),
     "oxh_moe_route": (I, [V, Z, Z, Z, I, V, V, V, V, V, V, V]),

@@ -518,15 +518,20 @@ int oxh_matvec_quantized_batch(uint32_t qtype, const uint8_t *data, size_t rows,
         if ((rc = quantize(kind, (const float *)g_dx.p, in_stride, n_vec, cols, g_dact.p))) return rc;
         if ((rc = oxh_mmq(qtype, d_w, rows, cols, g_dact.p, n_vec, (float *)g_dout.p, rows, NULL)))
             return rc;
-    } else if (n_vec > 8 && (qtype == OXH_Q3_K_S || qtype == OXH_Q3_K_M || qtype == OXH_Q3_K_L)) {
-        /* Q3_K has no MFMA kernel of its own, but it is exactly a Q6_K matrix in other bytes: rewrite it
+    } else if (n_vec > 8 && (qtype == OXH_Q2_K || qtype == OXH_Q3_K_S || qtype == OXH_Q3_K_M ||
+                             qtype == OXH_Q3_K_L)) {
+        /* No MFMA kernel reads these blocks as they are.  Q3_K is exactly a Q6_K matrix in other bytes
+         * and Q2_K widens to 210-byte blocks with scale * code in the 6-bit fields: rewrite the matrix
          * for this call, as the reference prepares its batch rows (oxk.c:734-745), and use that kernel */
         size_t prep_bytes;
         if (!mul_ok(rows, cols / OXH_QK_K * OXH_Q6_K_BYTES, &prep_bytes)) return bad_arg("batch: size overflow");
         if ((rc = reserve(&g_dprep, prep_bytes))) return rc;
-        if ((rc = oxh_q3_k_as_q6_k(d_w, rows, cols, g_dprep.p, NULL))) return rc;
+        if (qtype == OXH_Q2_K) rc = oxh_q2_k_widen(d_w, rows, cols, g_dprep.p, NULL);
+        else                   rc = oxh_q3_k_as_q6_k(d_w, rows, cols, g_dprep.p, NULL);
+        if (rc) return rc;
         if ((rc = quantize(kind, (const float *)g_dx.p, in_stride, n_vec, cols, g_dact.p))) return rc;
-        if ((rc = oxh_mmq(OXH_Q6_K, g_dprep.p, rows, cols, g_dact.p, n_vec, (float *)g_dout.p, rows, NULL)))
+        if ((rc = oxh_mmq(qtype == OXH_Q2_K ? OXH_Q2_K_WIDE : OXH_Q6_K, g_dprep.p, rows, cols, g_dact.p, n_vec,
+                          (float *)g_dout.p, rows, NULL)))
             return rc;
     } else {
         size_t step = oxh_gemv_max_nvec_buffered(qtype, cols);

@@ -482,6 +482,67 @@ k_q3k_to_q6k(const uint8_t *__restrict__ src, uint8_t *__restrict__ dst, uint32_
     }
 }
 
+/* Q2_K rows widened to 210-byte blocks for the tile kernel's Q2 mode.  A Q2_K weight is
+ * d * sc * code - dmin * m with 4-bit sc and m per group of 16 and a 2-bit code (oxk.c:592-622), over
+ * the groups and the element order of Q6_K.  sc * code is at most 45 and goes into the 6-bit field
+ * of the Q6_K layout (low nibbles in bytes 0..127, upper two bits in bytes 128..191); bytes 192..199
+ * take the sixteen minima as nibbles (group g in byte g / 2, even groups low), bytes 200..201 dmin,
+ * bytes 202..207 zero, bytes 208..209 d.  Lane split as in k_q3k_to_q6k. */
+__global__ __launch_bounds__(256) void
+k_q2k_widen(const uint8_t *__restrict__ src, uint8_t *__restrict__ dst, uint32_t n_blocks)
+{
+    const uint32_t t = blockIdx.x * 256u + threadIdx.x;
+    const uint32_t b = t >> 2, u = t & 3u, n = u >> 1, lh = u & 1u;
+    if (b >= n_blocks) return;
+    const uint8_t *s = src + (size_t)b * 84u;
+    uint8_t *d = dst + (size_t)b * 210u;
+    const U32x4u2 sm = *reinterpret_cast<const U32x4u2 *>(s);
+    const U32x4u2 qs = *reinterpret_cast<const U32x4u2 *>(s + 16u + 32u * n + 16u * lh);
+    const uint32_t q4[4] = { qs.x, qs.y, qs.z, qs.w };
+    const uint32_t sw[4] = { sm.x, sm.y, sm.z, sm.w };
+    /* scale of group 8n + 2k + lh: byte 2k + lh of words 2n, 2n + 1 */
+    uint32_t sc[4];
+#pragma unroll
+    for (uint32_t k = 0; k < 4u; k++) {
+        const uint32_t word = n ? sw[2u + (k >> 1)] : sw[k >> 1];
+        sc[k] = (word >> (16u * (k & 1u) + 8u * lh)) & 15u;
+    }
+    uint32_t la[4], lb[4], hh[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        uint32_t p[4];
+#pragma unroll
+        for (uint32_t k = 0; k < 4u; k++)
+            p[k] = ((q4[i] >> (2u * k)) & 0x03030303u) * sc[k];      /* at most 45 per byte: no carries */
+        la[i] = (p[0] & 0x0F0F0F0Fu) | ((p[2] & 0x0F0F0F0Fu) << 4);
+        lb[i] = (p[1] & 0x0F0F0F0Fu) | ((p[3] & 0x0F0F0F0Fu) << 4);
+        hh[i] = ((p[0] >> 4) & 0x03030303u) | (((p[1] >> 4) & 0x03030303u) << 2) |
+                (((p[2] >> 4) & 0x03030303u) << 4) | (((p[3] >> 4) & 0x03030303u) << 6);
+    }
+    U32x4u2 o;
+    o.x = la[0]; o.y = la[1]; o.z = la[2]; o.w = la[3];
+    *reinterpret_cast<U32x4u2 *>(d + 64u * n + 16u * lh) = o;
+    o.x = lb[0]; o.y = lb[1]; o.z = lb[2]; o.w = lb[3];
+    *reinterpret_cast<U32x4u2 *>(d + 64u * n + 32u + 16u * lh) = o;
+    o.x = hh[0]; o.y = hh[1]; o.z = hh[2]; o.w = hh[3];
+    *reinterpret_cast<U32x4u2 *>(d + 128u + 32u * n + 16u * lh) = o;
+    if (u == 0u) {
+        uint32_t pk[4];
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const uint32_t h = (sw[i] >> 4) & 0x0F0F0F0Fu, tt = h | (h >> 4);
+            pk[i] = (tt & 0xFFu) | ((tt >> 8) & 0xFF00u);            /* four minima -> 16 bits */
+        }
+        const uint32_t dd = reinterpret_cast<const U32u2 *>(s + 80u)->v;    /* d | dmin << 16 */
+        o.x = pk[0] | (pk[1] << 16);
+        o.y = pk[2] | (pk[3] << 16);
+        o.z = dd >> 16;
+        o.w = 0u;
+        *reinterpret_cast<U32x4u2 *>(d + 192u) = o;
+        *reinterpret_cast<uint16_t *>(d + 208u) = (uint16_t)(dd & 0xFFFFu);
+    }
+}
+
 #include "gemv_kernels.inc"
 #include "mmq_kernels.inc"
 #include "moe_kernels.inc"
@@ -725,6 +786,8 @@ static hipError_t raise_all_lds_ceilings(void)
     if ((e = raise_lds_ceiling(k_mmq_q5_k<4, 1, 8>)) != hipSuccess) return e;
     if ((e = raise_lds_ceiling(k_mmq_q6_k<8, 1, 8>)) != hipSuccess) return e;
     if ((e = raise_lds_ceiling(k_mmq_q6_k<4, 1, 8>)) != hipSuccess) return e;
+    if ((e = raise_lds_ceiling(k_mmq_q6_k<8, 1, 8, true>)) != hipSuccess) return e;
+    if ((e = raise_lds_ceiling(k_mmq_q6_k<4, 1, 8, true>)) != hipSuccess) return e;
     if ((e = raise_lds_ceiling(k_mfma_q8_0_segments<4, 0>)) != hipSuccess) return e;
     if ((e = raise_lds_ceiling(k_mfma_q8_0_segments<4, 1>)) != hipSuccess) return e;
     if ((e = raise_lds_ceiling(k_mfma_q8_0_segments<4, 2>)) != hipSuccess) return e;
@@ -1256,13 +1319,13 @@ static void mmq5_launch(const void *d_w, size_t rows, size_t blocks, const void 
                        (const uint8_t *)d_acts, (uint32_t)n_vec, d_out, out_stride);
 }
 
-template <int TC, int RC, int WAVES>
+template <int TC, int RC, int WAVES, bool Q2 = false>
 static void mmq6_launch(const void *d_w, size_t rows, size_t blocks, const void *d_acts, size_t n_vec,
                         float *d_out, size_t out_stride, void *stream)
 {
     typedef Mmq6Geom<TC, RC, WAVES> G;
     const dim3 grid((uint32_t)((rows + G::ROWS - 1) / G::ROWS), (uint32_t)((n_vec + G::TOK - 1) / G::TOK));
-    auto kernel = k_mmq_q6_k<TC, RC, WAVES>;
+    auto kernel = k_mmq_q6_k<TC, RC, WAVES, Q2>;
     hipLaunchKernelGGL(kernel, grid, dim3(WAVES * 64), G::LDS_BYTES, pick_stream(stream),
                        (const uint8_t *)d_w, (uint32_t)rows, (uint32_t)blocks,
                        (const uint8_t *)d_acts, (uint32_t)n_vec, d_out, out_stride);
@@ -1276,7 +1339,9 @@ extern "C" int oxh_mmq(uint32_t qtype, const void *d_w, size_t rows, size_t cols
     if (rc) return rc;
     if (rows == 0 || n_vec == 0) return OXH_OK;
     if (!d_w || !d_acts || !d_out) return arg_fail("oxh_mmq: NULL pointer");
-    if ((!is_q4k(qtype) && !is_q5k(qtype) && qtype != OXH_Q6_K) || oxh_act_kind(qtype, cols) != 2) {
+    const bool wide2 = qtype == OXH_Q2_K_WIDE;
+    if ((!is_q4k(qtype) && !is_q5k(qtype) && qtype != OXH_Q6_K && !wide2) ||
+        oxh_act_kind(wide2 ? OXH_Q2_K : qtype, cols) != 2) {
         snprintf(g_err, sizeof g_err, "oxh_mmq: qtype %u with cols %zu has no MFMA kernel", qtype, cols);
         return OXH_DECLINED;
     }
@@ -1301,7 +1366,7 @@ extern "C" int oxh_mmq(uint32_t qtype, const void *d_w, size_t rows, size_t cols
         else if (((rows + 127) / 128) * ((n_vec + 63) / 64) >= need) shape = 2;
         else shape = 3;
     }
-    if (qtype == OXH_Q6_K || is_q5k(qtype)) {
+    if (qtype == OXH_Q6_K || is_q5k(qtype) || wide2) {
         /* one 16-row chunk per wave throughout: 128x128, 128x64, 64x32, 64x16 */
         if (!forced) {
             if (n_vec <= 16) shape = 4;
@@ -1315,6 +1380,14 @@ extern "C" int oxh_mmq(uint32_t qtype, const void *d_w, size_t rows, size_t cols
             else if (shape == 2) mmq5_launch<4, 1, 8>(d_w, rows, blocks, d_acts, n_vec, d_out, out_stride, stream);
             else if (shape == 3) mmq5_launch<2, 1, 4>(d_w, rows, blocks, d_acts, n_vec, d_out, out_stride, stream);
             else                 mmq5_launch<1, 1, 4>(d_w, rows, blocks, d_acts, n_vec, d_out, out_stride, stream);
+            HIP_TRY(hipGetLastError());
+            return OXH_OK;
+        }
+        if (wide2) {
+            if (shape == 1)      mmq6_launch<8, 1, 8, true>(d_w, rows, blocks, d_acts, n_vec, d_out, out_stride, stream);
+            else if (shape == 2) mmq6_launch<4, 1, 8, true>(d_w, rows, blocks, d_acts, n_vec, d_out, out_stride, stream);
+            else if (shape == 3) mmq6_launch<2, 1, 4, true>(d_w, rows, blocks, d_acts, n_vec, d_out, out_stride, stream);
+            else                 mmq6_launch<1, 1, 4, true>(d_w, rows, blocks, d_acts, n_vec, d_out, out_stride, stream);
             HIP_TRY(hipGetLastError());
             return OXH_OK;
         }
@@ -1386,6 +1459,22 @@ extern "C" int oxh_q3_k_as_q6_k(const void *d_w, size_t rows, size_t cols, void 
     const uint32_t n_blocks = (uint32_t)(rows * blocks);
     hipLaunchKernelGGL(k_q3k_to_q6k, dim3((n_blocks * 4u + 255u) / 256u), dim3(256), 0, pick_stream(stream),
                        (const uint8_t *)d_w, (uint8_t *)d_q6k, n_blocks);
+    HIP_TRY(hipGetLastError());
+    return OXH_OK;
+}
+
+extern "C" int oxh_q2_k_widen(const void *d_w, size_t rows, size_t cols, void *d_wide, void *stream)
+{
+    int rc = ensure_init();
+    if (rc) return rc;
+    if (rows == 0) return OXH_OK;
+    if (!d_w || !d_wide) return arg_fail("oxh_q2_k_widen: NULL pointer");
+    if (cols == 0 || cols % OXH_QK_K) return arg_fail("oxh_q2_k_widen: cols must be a whole number of 256-blocks");
+    const size_t blocks = cols / OXH_QK_K;
+    if (rows > 0x3FFFFFFFull / blocks) return arg_fail("oxh_q2_k_widen: matrix too large");
+    const uint32_t n_blocks = (uint32_t)(rows * blocks);
+    hipLaunchKernelGGL(k_q2k_widen, dim3((n_blocks * 4u + 255u) / 256u), dim3(256), 0, pick_stream(stream),
+                       (const uint8_t *)d_w, (uint8_t *)d_wide, n_blocks);
     HIP_TRY(hipGetLastError());
     return OXH_OK;
 }

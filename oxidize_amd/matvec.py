@@ -231,6 +231,14 @@ def q3_k_as_q6_k(d_w, rows, cols, d_q6k, stream=None):
     check(lib().oxh_q3_k_as_q6_k(ctypes.c_void_p(d_w), rows, cols, ctypes.c_void_p(d_q6k), stream))
 
 
+Q2_K_WIDE = 0x1008
+
+
+def q2_k_widen(d_w, rows, cols, d_wide, stream=None):
+    """Widen a Q2_K matrix to the 210-byte blocks oxh_mmq takes under Q2_K_WIDE."""
+    check(lib().oxh_q2_k_widen(ctypes.c_void_p(d_w), rows, cols, ctypes.c_void_p(d_wide), stream))
+
+
 def read_probe(d_buf, nbytes, stream=None):
     """One launch that only reads `nbytes` at d_buf (measurement aid)."""
     check(lib().oxh_debug_read_probe(ctypes.c_void_p(d_buf), nbytes, None, stream))

@@ -48,3 +48,30 @@ def q3k_as_q6k(w):
     out[:, 192:208] = (q3k_scales(blk[:, 96:108]) - 32).astype(np.int8).view(np.uint8)
     out[:, 208:210] = blk[:, 108:110]
     return out.reshape(-1)
+
+
+def q2k_widen(w):
+    """flat uint8 array of Q2_K blocks (oxk.c:592-622: 16 scale|min bytes, 64 bytes of 2-bit codes in
+    the element order above, f16 d, f16 dmin) -> the 210-byte blocks of the tile kernel's Q2 mode:
+    scale * code in the 6-bit fields of the Q6_K layout, minima as nibbles in bytes 192..199, dmin in
+    200..201, zeros to 207, d in 208..209"""
+    blk = np.ascontiguousarray(w, dtype=np.uint8).reshape(-1, 84)
+    sm, qs = blk[:, :16].astype(np.int32), blk[:, 16:80].astype(np.int32)
+    c6 = np.zeros((blk.shape[0], 256), np.int32)
+    for n in range(2):
+        for k in range(4):
+            for l in range(32):
+                e = 128 * n + 32 * k + l
+                c6[:, e] = ((qs[:, 32 * n + l] >> (2 * k)) & 3) * (sm[:, e // 16] & 15)
+    out = np.zeros((blk.shape[0], 210), np.uint8)
+    for n in range(2):
+        for l in range(32):
+            e = [128 * n + 32 * k + l for k in range(4)]
+            out[:, 64 * n + l] = (c6[:, e[0]] & 15) | ((c6[:, e[2]] & 15) << 4)
+            out[:, 64 * n + 32 + l] = (c6[:, e[1]] & 15) | ((c6[:, e[3]] & 15) << 4)
+            out[:, 128 + 32 * n + l] = sum((c6[:, e[k]] >> 4) << (2 * k) for k in range(4))
+    for g in range(0, 16, 2):
+        out[:, 192 + g // 2] = (sm[:, g] >> 4) | ((sm[:, g + 1] >> 4) << 4)
+    out[:, 200:202] = blk[:, 82:84]
+    out[:, 208:210] = blk[:, 80:82]
+    return out.reshape(-1)

@@ -274,11 +274,63 @@ def test_q3k_rewritten_as_q6k_bytes(oxh):
     mv.q3_k_as_q6_k(0, 0, 256, 0)           # no rows: nothing to do
 
 
+def test_q2k_widened_bytes(oxh):
+    """The device widening of Q2_K blocks against the element-by-element numpy statement."""
+    from q3k_rewrite import q2k_widen
+    g = np.load(GOLD)
+    raw = np.ascontiguousarray(g["q2_k_raw_w"]).reshape(-1)
+    rnd = np.random.default_rng(4).integers(0, 256, 84 * 1027, dtype=np.uint8)
+    for w, rows, cols in ((raw, 24, 12 * 256), (rnd, 1027, 256), (rnd[:84], 1, 256),
+                          (synth.weights(Q2K, 130, 2048, seed=8), 130, 2048)):
+        d_w = mv.DeviceBuffer.from_host(w)
+        d_o = mv.DeviceBuffer(rows * (cols // 256) * 210)
+        mv.q2_k_widen(d_w.ptr, rows, cols, d_o.ptr)
+        assert np.array_equal(d_o.download(np.uint8, rows * (cols // 256) * 210), q2k_widen(w))
+    with pytest.raises(Exception):
+        mv.q2_k_widen(d_w.ptr, 1, 200, d_o.ptr)
+
+
+@pytest.mark.parametrize("n_vec", [1, 16, 17, 40, 130])
+def test_q2k_wide_tile_kernel_on_raw_blocks(oxh, n_vec):
+    """oxh_mmq on widened raw random Q2_K blocks (every scale, minimum and code value, arbitrary f16 d and
+    dmin as far as they are finite) against the oracle's Q2_K dot of the original blocks, bit for bit,
+    through every tile shape."""
+    rows, cols = 203, 1024
+    rng = np.random.default_rng(n_vec)
+    w = rng.integers(0, 256, rows * 4 * 84, dtype=np.uint8).reshape(-1, 84)
+    w[:, 81] &= 0x3B          # |d|, |dmin| below 2: finite, products stay finite
+    w[:, 83] &= 0x3B
+    w = w.reshape(-1)
+    x = synth.normal(n_vec * cols, seed=5, stream=n_vec)
+    o = oxlibs.oracle()
+    act = np.zeros(n_vec * 4 * 292, np.uint8)
+    for v in range(n_vec):
+        o.oxo_quantize_q8_k(x[v * cols:].ctypes.data, cols, act[v * 4 * 292:].ctypes.data)
+    want = np.zeros((n_vec, rows), np.float32)
+    for v in range(n_vec):
+        for r in range(rows):
+            want[v, r] = o.oxo_dot_q2_k_q8_k(w[r * 4 * 84:].ctypes.data, 4, act[v * 4 * 292:].ctypes.data, None)
+    d_w = mv.DeviceBuffer.from_host(w)
+    d_wide = mv.DeviceBuffer(rows * 4 * 210)
+    mv.q2_k_widen(d_w.ptr, rows, cols, d_wide.ptr)
+    d_a = mv.DeviceBuffer.from_host(act)
+    d_o = mv.DeviceBuffer(n_vec * rows * 4)
+    mv.mmq(mv.Q2_K_WIDE, d_wide.ptr, rows, cols, d_a.ptr, n_vec, d_o.ptr, rows)
+    got = d_o.download(np.float32, n_vec * rows).reshape(n_vec, rows)
+    assert np.array_equal(bits(got), bits(want))
+    # the widened blocks are no GGUF type: every other entry point refuses the id
+    seg = mv.make_segments([(d_wide.ptr, d_o.ptr, rows, 0)])
+    with pytest.raises(Exception):
+        mv.gemv_segments(mv.Q2_K_WIDE, seg, cols, d_a.ptr, 1, rows)
+
+
 @pytest.mark.parametrize("qt,rows,cols,n_vec", [(Q3K, 300, 2048, 9), (Q3KS, 65, 256, 16), (Q3KL, 1, 512, 33),
-                                                (Q3K, 1000, 4096, 100), (Q3K, 4096, 4096, 512)])
-def test_q3k_prefill_batches_on_the_matrix_cores(oxh, qt, rows, cols, n_vec):
-    """More than eight vectors of Q3_K weights go through the rewrite and the Q6_K tile kernel: every
-    output still has the bits of the single-vector Q3_K dot."""
+                                                (Q3K, 1000, 4096, 100), (Q3K, 4096, 4096, 512),
+                                                (Q2K, 300, 2048, 9), (Q2K, 65, 256, 16), (Q2K, 1, 512, 33),
+                                                (Q2K, 1000, 4096, 100), (Q2K, 4096, 4096, 512)])
+def test_q23k_prefill_batches_on_the_matrix_cores(oxh, qt, rows, cols, n_vec):
+    """More than eight vectors of Q2_K / Q3_K weights go through the rewrite and the Q6_K tile kernel:
+    every output still has the bits of the single-vector dot."""
     rb = synth.row_bytes(qt, cols)
     w = synth.weights(qt, rows, cols, seed=61, stream=n_vec)
     in_stride, out_stride = cols + 8, rows + 3

@@ -351,6 +351,34 @@ def test_q3_k_rewritten_as_q6_k_is_the_same_dot_and_the_same_row():
     assert np.array_equal(a.view(np.uint32), b.view(np.uint32))
 
 
+def test_q2_k_widened_blocks_give_the_reference_bits():
+    # the widening the batch path of the library uses for Q2_K weights, and the arithmetic its tile
+    # kernel runs on the result (one integer dot with scale * code, one with the group minima spread
+    # over their elements, then dq * (d * pos - dmin * min)): float bits of the reference's Q2_K dot
+    from q3k_rewrite import q2k_widen
+    g = load("q23_k.npz")
+    w, act = g["q2_k_raw_w"], g["q2_k_raw_act"]
+    e = np.arange(256)
+    n, k, l = e // 128, (e // 32) % 4, e % 32
+    for t in range(w.shape[0]):
+        wide = q2k_widen(w[t]).reshape(-1, 210).astype(np.int64)
+        total = np.float32(0)
+        for b in range(w.shape[1]):
+            blk, a = wide[b], np.ascontiguousarray(act[t, b])
+            dq = a[:4].view(np.float32)[0]
+            q = a[4:260].view(np.int8).astype(np.int64)
+            byte = blk[64 * n + 32 * (k & 1) + l]
+            c6 = np.where(k >= 2, byte >> 4, byte & 15) | (((blk[128 + 32 * n + l] >> (2 * k)) & 3) << 4)
+            mb = blk[192 + e // 32]
+            m = np.where((e // 16) & 1, mb >> 4, mb & 15)
+            d = blk[208:210].astype(np.uint8).view(np.float16)[0].astype(np.float32)
+            dmin = blk[200:202].astype(np.uint8).view(np.float16)[0].astype(np.float32)
+            pos, mn = np.float32(int((c6 * q).sum())), np.float32(int((m * q).sum()))
+            with np.errstate(all="ignore"):
+                total = np.float32(total + np.float32(dq * np.float32(np.float32(d * pos) - np.float32(dmin * mn))))
+        assert f32bits(total) == g["q2_k_raw_scalar_bits"][t, 1]
+
+
 @pytest.mark.parametrize("qt", [8, 9, 10, 11])
 def test_q23_k_matvec_batch_and_dequant_vs_reference_goldens(qt):
     g = load("q23_k.npz")
