@@ -75,6 +75,10 @@ typedef struct {
 } Resident;
 
 static pthread_mutex_t g_lock = PTHREAD_MUTEX_INITIALIZER;
+/* Held for the whole of a matvec call, and by the calls that free device weights (taken before g_lock):
+ * the staging buffers and the library's stream are shared by every call, so concurrent callers are
+ * serialised (the reference's worker pool is one process-global resource too, include/oxidize/parallel.h:13-19). */
+static pthread_mutex_t g_call = PTHREAD_MUTEX_INITIALIZER;
 static Resident *g_res = NULL;
 static size_t g_nres = 0, g_cap = 0;
 
@@ -137,6 +141,7 @@ int oxh_weight_register(const void *h_data, size_t bytes)
 int oxh_weight_unregister(const void *h_data)
 {
     int rc = OXH_OK;
+    pthread_mutex_lock(&g_call);
     pthread_mutex_lock(&g_lock);
     for (size_t i = 0; i < g_nres; i++) {
         if (g_res[i].h == (const uint8_t *)h_data) {
@@ -148,11 +153,13 @@ int oxh_weight_unregister(const void *h_data)
         }
     }
     pthread_mutex_unlock(&g_lock);
+    pthread_mutex_unlock(&g_call);
     return rc;
 }
 
 int oxh_weight_clear(void)
 {
+    pthread_mutex_lock(&g_call);
     pthread_mutex_lock(&g_lock);
     int rc = g_nres ? oxh_stream_sync(NULL) : OXH_OK;
     for (size_t i = 0; i < g_nres; i++) {
@@ -161,6 +168,7 @@ int oxh_weight_clear(void)
     }
     g_nres = 0;
     pthread_mutex_unlock(&g_lock);
+    pthread_mutex_unlock(&g_call);
     return rc;
 }
 
@@ -284,7 +292,7 @@ static int quantize(int kind, const float *d_x, size_t in_stride, size_t n_vec,
 
 /* ─── oc_matvec_quantized ─────────────────────────────────────────────── */
 
-int oxh_matvec_quantized(uint32_t qtype, const uint8_t *data, size_t rows,
+static int mv_one(uint32_t qtype, const uint8_t *data, size_t rows,
                          size_t cols, size_t row_bytes, const float *input,
                          float *output, float *temp)
 {
@@ -392,7 +400,7 @@ static int grouped(uint32_t qtype, const uint8_t *const *datas,
     return OXH_OK;
 }
 
-int oxh_matvec_quantized_fused(const uint32_t *qtypes, const uint8_t *const *datas,
+static int mv_fused(const uint32_t *qtypes, const uint8_t *const *datas,
                                const size_t *rows, size_t cols, const size_t *row_bytes,
                                size_t n_outs, const float *input, float *const *outs,
                                float *temp)
@@ -418,7 +426,7 @@ int oxh_matvec_quantized_fused(const uint32_t *qtypes, const uint8_t *const *dat
     /* mixed types (or an all-empty group): one call per matrix, matvec.c:1579-1593 */
     if (temp == NULL) return declined("temp is NULL");
     for (size_t k = 0; k < n_outs; k++) {
-        int rc = oxh_matvec_quantized(qtypes[k], datas[k], rows[k], cols, row_bytes[k],
+        int rc = mv_one(qtypes[k], datas[k], rows[k], cols, row_bytes[k],
                                       input, outs[k], temp);
         if (rc) return rc;
         g_stats.activation_quantizations++;
@@ -428,7 +436,7 @@ int oxh_matvec_quantized_fused(const uint32_t *qtypes, const uint8_t *const *dat
     return OXH_OK;
 }
 
-int oxh_matvec_quantized_multi_input(const uint32_t *qtypes, const uint8_t *const *datas,
+static int mv_multi_input(const uint32_t *qtypes, const uint8_t *const *datas,
                                      const size_t *rows, size_t cols,
                                      const size_t *row_bytes, size_t n_outs,
                                      const float *const *inputs, float *const *outs,
@@ -453,7 +461,7 @@ int oxh_matvec_quantized_multi_input(const uint32_t *qtypes, const uint8_t *cons
     }
     if (temp == NULL) return declined("temp is NULL");
     for (size_t k = 0; k < n_outs; k++) {
-        int rc = oxh_matvec_quantized(qtypes[k], datas[k], rows[k], cols, row_bytes[k],
+        int rc = mv_one(qtypes[k], datas[k], rows[k], cols, row_bytes[k],
                                       inputs[k], outs[k], temp);
         if (rc) return rc;
         g_stats.activation_quantizations++;
@@ -465,7 +473,7 @@ int oxh_matvec_quantized_multi_input(const uint32_t *qtypes, const uint8_t *cons
 
 /* ─── oc_matvec_quantized_batch ───────────────────────────────────────── */
 
-int oxh_matvec_quantized_batch(uint32_t qtype, const uint8_t *data, size_t rows,
+static int mv_batch(uint32_t qtype, const uint8_t *data, size_t rows,
                                size_t cols, size_t row_bytes, const float *inputs,
                                size_t in_stride, float *outputs, size_t out_stride,
                                size_t n_vec, float *temp, uint8_t *act_scratch,
@@ -558,6 +566,48 @@ int oxh_matvec_quantized_batch(uint32_t qtype, const uint8_t *data, size_t rows,
                 return rc;
     }
     return oxh_stream_sync(NULL);
+}
+
+/* ─── public entry points: one call at a time ─────────────────────────── */
+
+int oxh_matvec_quantized(uint32_t qtype, const uint8_t *data, size_t rows, size_t cols, size_t row_bytes,
+                         const float *input, float *output, float *temp)
+{
+    pthread_mutex_lock(&g_call);
+    const int rc = mv_one(qtype, data, rows, cols, row_bytes, input, output, temp);
+    pthread_mutex_unlock(&g_call);
+    return rc;
+}
+
+int oxh_matvec_quantized_fused(const uint32_t *qtypes, const uint8_t *const *datas, const size_t *rows,
+                               size_t cols, const size_t *row_bytes, size_t n_outs, const float *input,
+                               float *const *outs, float *temp)
+{
+    pthread_mutex_lock(&g_call);
+    const int rc = mv_fused(qtypes, datas, rows, cols, row_bytes, n_outs, input, outs, temp);
+    pthread_mutex_unlock(&g_call);
+    return rc;
+}
+
+int oxh_matvec_quantized_multi_input(const uint32_t *qtypes, const uint8_t *const *datas, const size_t *rows,
+                                     size_t cols, const size_t *row_bytes, size_t n_outs,
+                                     const float *const *inputs, float *const *outs, float *temp)
+{
+    pthread_mutex_lock(&g_call);
+    const int rc = mv_multi_input(qtypes, datas, rows, cols, row_bytes, n_outs, inputs, outs, temp);
+    pthread_mutex_unlock(&g_call);
+    return rc;
+}
+
+int oxh_matvec_quantized_batch(uint32_t qtype, const uint8_t *data, size_t rows, size_t cols, size_t row_bytes,
+                               const float *inputs, size_t in_stride, float *outputs, size_t out_stride,
+                               size_t n_vec, float *temp, uint8_t *act_scratch, size_t act_bytes)
+{
+    pthread_mutex_lock(&g_call);
+    const int rc = mv_batch(qtype, data, rows, cols, row_bytes, inputs, in_stride, outputs, out_stride, n_vec,
+                            temp, act_scratch, act_bytes);
+    pthread_mutex_unlock(&g_call);
+    return rc;
 }
 
 /* ─── the reference's own symbols ─────────────────────────────────────── */

@@ -252,3 +252,43 @@ def test_random_fused_prologue_launch(oxh, seed):
                 h = np.zeros(r, np.float32)
                 o.oxo_swiglu_f32(want.ctypes.data, up.ctypes.data, h.ctypes.data, r)
                 assert np.all(np.abs(out[i, v, :r] - h) <= 4e-6 * np.abs(h) + 1e-30), (qt, kind, i, v)
+
+
+def test_host_calls_from_several_threads(oxh):
+    """Four threads call the host entry points at once (ctypes drops the interpreter lock during a
+    call): the library serialises them on its shared staging buffers, and every result is still the
+    oracle's to the bit.  Shapes differ per thread so that the staging buffers are regrown mid-run."""
+    import threading
+    jobs = []
+    for t, (qt, rows, cols) in enumerate([(13, 300, 4096), (16, 150, 2048), (7, 257, 896), (10, 90, 5120)]):
+        layout = BASE.get(qt, qt)
+        w = synth.weights(layout, rows, cols, seed=900 + t)
+        xs = [synth.normal(cols, seed=901, stream=10 * t + i) for i in range(6)]
+        wants = [oracle_rows(qt, layout, w, rows, cols, x)[0] for x in xs]
+        jobs.append((qt, rows, cols, synth.row_bytes(layout, cols), w, xs, wants))
+    failures = []
+
+    def worker(job):
+        qt, rows, cols, rb, w, xs, wants = job
+        temp = np.zeros(cols, np.float32)
+        scratch = np.zeros(mv.batch_scratch_bytes(cols), np.uint8)
+        try:
+            for rep in range(5):
+                for x, want in zip(xs, wants):
+                    out = np.full(rows, -3.5, np.float32)
+                    assert mv.matvec_quantized(qt, w, rows, cols, rb, x, out, temp) == 0
+                    assert np.array_equal(bits(out), bits(want))
+                xb = np.stack(xs)
+                ob = np.full((len(xs), rows), -3.5, np.float32)
+                assert mv.matvec_quantized_batch(qt, w, rows, cols, rb, xb, cols, ob, rows, len(xs), temp,
+                                                 scratch) == 0
+                assert np.array_equal(bits(ob), bits(np.stack(wants)))
+        except Exception as e:                                   # noqa: BLE001 - reported below
+            failures.append((qt, repr(e)))
+
+    threads = [threading.Thread(target=worker, args=(j,)) for j in jobs]
+    for th in threads:
+        th.start()
+    for th in threads:
+        th.join()
+    assert not failures, failures
