@@ -198,6 +198,40 @@ def secondary_figures(mv, synth):
     d_x.free()
     d_o.free()
     out["other_types_gemv_28672x4096"] = others
+    # Q2_K and Q3_K prefill (512 tokens, 14336 x 4096): the matrix is rewritten into 210-byte blocks
+    # and then runs on the Q6_K tile kernel; both steps timed, Q8_K activations already made
+    rows, cols = 14336, 4096
+    x = synth.normal(n_vec * cols, seed=0, stream=2004)
+    d_x = mv.DeviceBuffer.from_host(x)
+    d_a = mv.DeviceBuffer(n_vec * mv.act_bytes(Q6K, cols))
+    mv.quantize(Q6K, d_x.ptr, cols, n_vec, cols, d_a.ptr)
+    d_o = mv.DeviceBuffer(n_vec * rows * 4)
+    d_wide = mv.DeviceBuffer(rows * (cols // 256) * 210)
+    pre = {}
+    for name, qt in (("q2_k", 8), ("q3_k", 10)):
+        d_w = mv.DeviceBuffer.from_host(synth.weights(qt, rows, cols, seed=0, stream=8))
+        if qt == 8:
+            def rewrite():
+                mv.q2_k_widen(d_w.ptr, rows, cols, d_wide.ptr)
+            as_type = mv.Q2_K_WIDE
+        else:
+            def rewrite():
+                mv.q3_k_as_q6_k(d_w.ptr, rows, cols, d_wide.ptr)
+            as_type = Q6K
+
+        def tiles():
+            mv.mmq(as_type, d_wide.ptr, rows, cols, d_a.ptr, n_vec, d_o.ptr, rows)
+
+        us_rw = timed(rewrite, 12, mv)
+        us_mma = timed(tiles, 12, mv)
+        ops = 2.0 * rows * cols * n_vec
+        pre[name] = {"rewrite_us": round(us_rw, 2), "mfma_kernel_only_us": round(us_mma, 2),
+                     "tops": round(ops / (us_rw + us_mma) / 1e6, 1),
+                     "frac_of_int8_peak": round(ops / (us_rw + us_mma) / 1e6 / INT8_PEAK_TOPS, 4)}
+        d_w.free()
+    out["q2k_q3k_prefill_14336x4096x512"] = pre
+    for b_ in (d_x, d_a, d_o, d_wide):
+        b_.free()
     # Q8_0 lm_head (configuration 2), batch 1 and 8
     rows, cols = 151936, 896
     w = synth.weights(Q80, rows, cols, seed=0, stream=5)
