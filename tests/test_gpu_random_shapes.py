@@ -4,6 +4,8 @@ activations and its own count, ragged rows, padded output strides, with and
 without a buffer for the quantised activations (with one, launches of several
 activations run on the matrix cores).  Every output must carry the oracle's
 bits; whatever lies between the rows of a padded output must stay untouched."""
+import os
+
 import numpy as np
 import pytest
 
@@ -15,6 +17,7 @@ pytestmark = pytest.mark.gpu
 
 TYPES = (3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15, 16, 17, 18, 19, 20)
 BASE = {17: 3, 19: 5, 20: 7, 9: 10, 11: 10, 12: 13, 14: 15}      # ids that share another id's layout
+SHIFT = int(os.environ.get("OXH_TEST_SEED_SHIFT", "0"))           # other shapes from the same generators
 
 
 def bits(a):
@@ -23,7 +26,7 @@ def bits(a):
 
 @pytest.mark.parametrize("seed", range(144))
 def test_random_launch(oxh, seed):
-    rng = np.random.default_rng(1000 + seed)
+    rng = np.random.default_rng(1000 + seed + 100000 * SHIFT)
     qt = int(TYPES[seed % len(TYPES)])
     layout = BASE.get(qt, qt)
     group = synth.BLOCK_ELEMS[layout]
@@ -87,7 +90,7 @@ def test_random_host_calls(oxh, seed):
     """The reference's four entry points on host arrays with random shapes: single,
     fused (shared input, possibly mixed types and empty matrices), multi-input,
     and batch (1..40 vectors, padded strides)."""
-    rng = np.random.default_rng(5000 + seed)
+    rng = np.random.default_rng(5000 + seed + 100000 * SHIFT)
     qt = int(TYPES[seed % len(TYPES)])
     layout = BASE.get(qt, qt)
     group = synth.BLOCK_ELEMS[layout]
@@ -145,7 +148,7 @@ def test_random_host_calls(oxh, seed):
 def test_random_prefill_and_lookup(oxh, seed):
     """oxh_mmq (9..300 activations; Q4_K, Q5_K, Q6_K) with padded output stride, and
     oxh_get_rows over random ids for every type."""
-    rng = np.random.default_rng(9000 + seed)
+    rng = np.random.default_rng(9000 + seed + 100000 * SHIFT)
     o = oxlibs.oracle()
     qt = (13, 15, 16, 12, 14)[seed % 5]
     layout = BASE.get(qt, qt)
@@ -192,7 +195,7 @@ def test_random_fused_prologue_launch(oxh, seed):
     segments, one to four input vectors, optionally a paired gate/up segment.  The float
     step is read back from the device; from there on everything is exact: the quantised
     bytes, plain segments' outputs, and the two halves of a pair before silu(gate)*up."""
-    rng = np.random.default_rng(7000 + seed)
+    rng = np.random.default_rng(7000 + seed + 100000 * SHIFT)
     o = oxlibs.oracle()
     qt = int(TYPES[seed % len(TYPES)])
     layout = BASE.get(qt, qt)
