@@ -786,6 +786,8 @@ static hipError_t raise_all_lds_ceilings(void)
     if ((e = raise_lds_ceiling(k_mmq_q5_k<4, 1, 8>)) != hipSuccess) return e;
     if ((e = raise_lds_ceiling(k_mmq_q6_k<8, 1, 8>)) != hipSuccess) return e;
     if ((e = raise_lds_ceiling(k_mmq_q6_k<4, 1, 8>)) != hipSuccess) return e;
+    if ((e = raise_lds_ceiling(k_mmq_q6_k<8, 1, 4>)) != hipSuccess) return e;
+    if ((e = raise_lds_ceiling(k_mmq_q6_k<8, 1, 4, true>)) != hipSuccess) return e;
     if ((e = raise_lds_ceiling(k_mmq_q6_k<8, 1, 8, true>)) != hipSuccess) return e;
     if ((e = raise_lds_ceiling(k_mmq_q6_k<4, 1, 8, true>)) != hipSuccess) return e;
     if ((e = raise_lds_ceiling(k_mfma_q8_0_segments<4, 0>)) != hipSuccess) return e;
@@ -1353,9 +1355,10 @@ extern "C" int oxh_mmq(uint32_t qtype, const void *d_w, size_t rows, size_t cols
     if (blocks * 292u * 256u > 0xFFFFFFFFull)
         return arg_fail("oxh_mmq: cols too large");
     /* Shape: the largest tile that still gives (nearly) every CU a workgroup;
-     * OXH_MMQ_SHAPE = 1..4 forces 256x128, 128x64, 64x32, 64x16 (rows x tokens). */
+     * OXH_MMQ_SHAPE = 1..4 forces 256x128, 128x64, 64x32, 64x16 (rows x tokens), 5 the 64x128 tile
+     * that only the Q6_K kernel has (128x64 for the others). */
     static int forced = -1;
-    if (forced < 0) forced = (int)env_u32("OXH_MMQ_SHAPE", 0, 0, 4);
+    if (forced < 0) forced = (int)env_u32("OXH_MMQ_SHAPE", 0, 0, 5);
     const size_t cus = (size_t)(g_n_cu > 0 ? g_n_cu : 256);
     const size_t need = cus - cus / 8;
     int shape = forced;
@@ -1367,15 +1370,20 @@ extern "C" int oxh_mmq(uint32_t qtype, const void *d_w, size_t rows, size_t cols
         else shape = 3;
     }
     if (qtype == OXH_Q6_K || is_q5k(qtype) || wide2) {
-        /* one 16-row chunk per wave throughout: 128x128, 128x64, 64x32, 64x16 */
+        /* one 16-row chunk per wave throughout: 128x128, 128x64, 64x32, 64x16; Q6_K also has 64x128
+         * on four waves (shape 5) for matrices with too few rows to fill the chip with 128x128 tiles: the
+         * scaled weight operands a wave builds are then still reused by 128 tokens (4096 x 14336 x 512:
+         * 144 us against 167 us with 128x64 tiles) */
         if (!forced) {
             if (n_vec <= 16) shape = 4;
             else if (n_vec <= 32) shape = 3;
             else if (((rows + 127) / 128) * ((n_vec + 127) / 128) >= need) shape = 1;
+            else if (!is_q5k(qtype) && ((rows + 63) / 64) * ((n_vec + 127) / 128) >= need) shape = 5;
             else if (((rows + 127) / 128) * ((n_vec + 63) / 64) >= need) shape = 2;
             else shape = 3;
         }
         if (is_q5k(qtype)) {
+            if (shape == 5) shape = 2;
             if (shape == 1)      mmq5_launch<8, 1, 8>(d_w, rows, blocks, d_acts, n_vec, d_out, out_stride, stream);
             else if (shape == 2) mmq5_launch<4, 1, 8>(d_w, rows, blocks, d_acts, n_vec, d_out, out_stride, stream);
             else if (shape == 3) mmq5_launch<2, 1, 4>(d_w, rows, blocks, d_acts, n_vec, d_out, out_stride, stream);
@@ -1384,20 +1392,23 @@ extern "C" int oxh_mmq(uint32_t qtype, const void *d_w, size_t rows, size_t cols
             return OXH_OK;
         }
         if (wide2) {
-            if (shape == 1)      mmq6_launch<8, 1, 8, true>(d_w, rows, blocks, d_acts, n_vec, d_out, out_stride, stream);
+            if (shape == 5)      mmq6_launch<8, 1, 4, true>(d_w, rows, blocks, d_acts, n_vec, d_out, out_stride, stream);
+            else if (shape == 1) mmq6_launch<8, 1, 8, true>(d_w, rows, blocks, d_acts, n_vec, d_out, out_stride, stream);
             else if (shape == 2) mmq6_launch<4, 1, 8, true>(d_w, rows, blocks, d_acts, n_vec, d_out, out_stride, stream);
             else if (shape == 3) mmq6_launch<2, 1, 4, true>(d_w, rows, blocks, d_acts, n_vec, d_out, out_stride, stream);
             else                 mmq6_launch<1, 1, 4, true>(d_w, rows, blocks, d_acts, n_vec, d_out, out_stride, stream);
             HIP_TRY(hipGetLastError());
             return OXH_OK;
         }
-        if (shape == 1)      mmq6_launch<8, 1, 8>(d_w, rows, blocks, d_acts, n_vec, d_out, out_stride, stream);
+        if (shape == 5)      mmq6_launch<8, 1, 4>(d_w, rows, blocks, d_acts, n_vec, d_out, out_stride, stream);
+        else if (shape == 1) mmq6_launch<8, 1, 8>(d_w, rows, blocks, d_acts, n_vec, d_out, out_stride, stream);
         else if (shape == 2) mmq6_launch<4, 1, 8>(d_w, rows, blocks, d_acts, n_vec, d_out, out_stride, stream);
         else if (shape == 3) mmq6_launch<2, 1, 4>(d_w, rows, blocks, d_acts, n_vec, d_out, out_stride, stream);
         else                 mmq6_launch<1, 1, 4>(d_w, rows, blocks, d_acts, n_vec, d_out, out_stride, stream);
         HIP_TRY(hipGetLastError());
         return OXH_OK;
     }
+    if (shape == 5) shape = 2;
     if (shape == 1)      mmq_launch<8, 2, 8>(d_w, rows, blocks, d_acts, n_vec, d_out, out_stride, stream);
     else if (shape == 2) mmq_launch<4, 1, 8>(d_w, rows, blocks, d_acts, n_vec, d_out, out_stride, stream);
     else if (shape == 3) mmq_launch<2, 1, 4>(d_w, rows, blocks, d_acts, n_vec, d_out, out_stride, stream);

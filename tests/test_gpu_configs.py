@@ -143,7 +143,8 @@ def test_config3_mmq_prefill_512_tokens(oxh, rows):
     (Q4K, 14329, 256, 500),     # 256x128 tiles: 56 x 4 = 224 workgroups
     (Q4K, 4100, 512, 40),       # too few workgroups for either: 64x32 tiles, 65 x 2
     (Q6K, 7165, 512, 507),      # Q6_K: 128x128 tiles, 56 x 4
-    (Q6K, 3600, 256, 500),      # Q6_K: 128x64 tiles, 29 x 8
+    (Q6K, 3600, 256, 500),      # Q6_K: 64x128 tiles on four waves, 57 x 4
+    (Q6K, 14250, 256, 100),     # Q6_K: 128x64 tiles, 112 x 2 (223 tiles of 64x128 would leave CUs idle)
     (Q6K, 4100, 512, 40),       # Q6_K: 64x32 tiles
     (Q5K, 7165, 512, 507),      # Q5_K: 128x128 tiles, 56 x 4
     (Q5K, 3600, 256, 500),      # Q5_K: 128x64 tiles, 29 x 8
@@ -151,8 +152,8 @@ def test_config3_mmq_prefill_512_tokens(oxh, rows):
 ])
 def test_mmq_tile_variants_ragged(oxh, qtype, rows, cols, n_vec):
     """The MFMA kernel comes in several tile shapes (256x128, 128x64, 64x32,
-    64x16 rows x tokens), picked from the launch size; these cases select the
-    first three on a 256-CU device and leave the last row tile and the last
+    64x16 rows x tokens, and 64x128 for Q6_K), picked from the launch size;
+    these cases select all but 64x16 on a 256-CU device and leave the last row tile and the last
     token tile partly filled.  Every output is checked against the
     dot-instruction GEMV kernel on the same device data (two activations per
     launch: three or more would run on the matrix cores too), and a sample of
