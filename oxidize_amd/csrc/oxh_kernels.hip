@@ -1466,7 +1466,7 @@ extern "C" int oxh_q3_k_as_q6_k(const void *d_w, size_t rows, size_t cols, void 
     if (!d_w || !d_q6k) return arg_fail("oxh_q3_k_as_q6_k: NULL pointer");
     if (cols == 0 || cols % OXH_QK_K) return arg_fail("oxh_q3_k_as_q6_k: cols must be a whole number of 256-blocks");
     const size_t blocks = cols / OXH_QK_K;
-    if (rows > 0x3FFFFFFFull / blocks) return arg_fail("oxh_q3_k_as_q6_k: matrix too large");
+    if (rows > 0x3FFFFFC0ull / blocks) return arg_fail("oxh_q3_k_as_q6_k: matrix too large");
     const uint32_t n_blocks = (uint32_t)(rows * blocks);
     hipLaunchKernelGGL(k_q3k_to_q6k, dim3((n_blocks * 4u + 255u) / 256u), dim3(256), 0, pick_stream(stream),
                        (const uint8_t *)d_w, (uint8_t *)d_q6k, n_blocks);
@@ -1482,7 +1482,7 @@ extern "C" int oxh_q2_k_widen(const void *d_w, size_t rows, size_t cols, void *d
     if (!d_w || !d_wide) return arg_fail("oxh_q2_k_widen: NULL pointer");
     if (cols == 0 || cols % OXH_QK_K) return arg_fail("oxh_q2_k_widen: cols must be a whole number of 256-blocks");
     const size_t blocks = cols / OXH_QK_K;
-    if (rows > 0x3FFFFFFFull / blocks) return arg_fail("oxh_q2_k_widen: matrix too large");
+    if (rows > 0x3FFFFFC0ull / blocks) return arg_fail("oxh_q2_k_widen: matrix too large");
     const uint32_t n_blocks = (uint32_t)(rows * blocks);
     hipLaunchKernelGGL(k_q2k_widen, dim3((n_blocks * 4u + 255u) / 256u), dim3(256), 0, pick_stream(stream),
                        (const uint8_t *)d_w, (uint8_t *)d_wide, n_blocks);
