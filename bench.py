@@ -232,6 +232,33 @@ def secondary_figures(mv, synth):
     out["q2k_q3k_prefill_14336x4096x512"] = pre
     for b_ in (d_x, d_a, d_o, d_wide):
         b_.free()
+    # configuration 0 (the reference's own CPU-runnable case): one 4096 x 4096 Q4_K matvec, over 32 distinct
+    # copies in turn (302 MB: from HBM) and over one copy again and again (resident in the last-level cache)
+    rows, cols = 4096, 4096
+    w = synth.weights(Q4K, rows, cols, seed=0, stream=0)
+    copies = [mv.DeviceBuffer.from_host(w) for _ in range(32)]
+    d_x = mv.DeviceBuffer.from_host(synth.normal(cols, seed=0, stream=2005))
+    d_o = mv.DeviceBuffer(rows * 4)
+    segs = [mv.make_segments([(c.ptr, d_o.ptr, rows, 0)]) for c in copies]
+    state = {"i": 0}
+
+    def run_cold():
+        state["i"] += 1
+        mv.gemv_segments_f32(Q4K, segs[state["i"] % 32], cols, d_x.ptr, cols, None, 1, rows)
+
+    def run_hot():
+        mv.gemv_segments_f32(Q4K, segs[0], cols, d_x.ptr, cols, None, 1, rows)
+
+    nbytes = w.nbytes + 4 * cols + 4 * rows
+    us_cold, us_hot = timed(run_cold, 64, mv), timed(run_hot, 64, mv)
+    out["q4k_gemv_4096x4096_config0"] = {
+        "cold": {"us": round(us_cold, 2), "gbps": round(nbytes / us_cold / 1e3, 1)},
+        "cache_resident": {"us": round(us_hot, 2), "gbps": round(nbytes / us_hot / 1e3, 1)},
+        "note": "back-to-back launches on one stream, launch gaps included"}
+    for c in copies:
+        c.free()
+    d_x.free()
+    d_o.free()
     # Q8_0 lm_head (configuration 2), batch 1 and 8
     rows, cols = 151936, 896
     w = synth.weights(Q80, rows, cols, seed=0, stream=5)
@@ -340,9 +367,10 @@ def mmq_probe(mv, synth):
     mv.sync()
 
 
-def cpu_baseline(layers_sample=1, min_seconds=2.5):
+def cpu_baseline(layers_sample=1, min_seconds=2.5, cores=None):
     """The reference CPU path on the host cores over `layers_sample` layers of
-    the same workload (same shapes, same synthetic generator)."""
+    the same workload (same shapes, same synthetic generator); `cores` = worker
+    threads (default: up to 16, the cap of the reference's own CLI)."""
     import ctypes
 
     import numpy as np
@@ -352,7 +380,8 @@ def cpu_baseline(layers_sample=1, min_seconds=2.5):
 
     ref = oxlibs.ref()
     kind = "reference" if ref is not None else "port"
-    cores = min(16, os.cpu_count() or 1)
+    if cores is None:
+        cores = min(16, os.cpu_count() or 1)
     if ref is not None:
         ref.oc_parallel_set_threads(cores)
     else:
@@ -512,6 +541,9 @@ def main():
         out["extra"] = secondary_figures(mv, synth)
         out["extra"]["decode_chain_fused"] = chain_figure(mv, ds, args.steps)
     out["cpu_baseline"] = None if args.no_cpu else cpu_baseline()
+    if not args.no_cpu and out["cpu_baseline"]["kind"] == "reference" and isinstance(out.get("extra"), dict):
+        one = cpu_baseline(min_seconds=1.5, cores=1)
+        out["extra"]["cpu_baseline_1_thread"] = {"value": one["value"], "unit": one["unit"], "sample": one["sample"]}
     print(json.dumps(out))
     return 0
 
