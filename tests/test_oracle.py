@@ -921,3 +921,32 @@ def test_oracle_vs_live_reference_many_rows():
         ref.oc_matvec_quantized(qt, w.ctypes.data, rows, cols, rb, x.ctypes.data, b.ctypes.data, tb.ctypes.data)
         assert np.array_equal(a.view(np.uint32), b.view(np.uint32))
         assert np.array_equal(ta.view(np.uint8), tb.view(np.uint8))
+
+
+@pytest.mark.parametrize("qt", [3, 4, 5, 6, 7, 8, 10, 13, 15, 16, 18])
+def test_extreme_integers_oracle_vs_compiled_reference(qt):
+    # every code, scale and minimum at its bound, activations at +-127: the restatement must keep the
+    # reference's bits there too (the GPU test on the same inputs checks the kernels against it)
+    from extremes import TYPES, extreme_inputs, extreme_weights
+    ref = oxlibs.ref()
+    if ref is None:
+        pytest.skip("oracle/_ref was not built")
+    layout, fields = TYPES[qt]
+    rows, cols, n_vec = 130, (1024 if synth.BLOCK_ELEMS[layout] == 256 else 512), 6
+    rb = synth.row_bytes(layout, cols)
+    w = extreme_weights(layout, fields, rows, cols)
+    xs = extreme_inputs(n_vec, cols)
+    for v in range(n_vec):
+        x = np.ascontiguousarray(xs[v])
+        mine, theirs = np.zeros(rows, np.float32), np.zeros(rows, np.float32)
+        t1, t2 = np.zeros(cols, np.float32), np.zeros(cols, np.float32)
+        assert O.oxo_matvec_quantized(qt, w.ctypes.data, rows, cols, rb, x.ctypes.data, mine.ctypes.data,
+                                      t1.ctypes.data) == 0
+        ref.oc_matvec_quantized(qt, w.ctypes.data, rows, cols, rb, x.ctypes.data, theirs.ctypes.data,
+                                t2.ctypes.data)
+        nact = cols // 256 * 292 if synth.BLOCK_ELEMS[layout] == 256 else cols // 32 * 34
+        assert np.array_equal(t1.view(np.uint8)[:nact], t2.view(np.uint8)[:nact])
+        if synth.BLOCK_ELEMS[layout] == 256:
+            assert np.array_equal(mine.view(np.uint32), theirs.view(np.uint32)), (qt, v)
+        else:       # the x86 kernels of the 32-value formats sum in another order
+            assert np.allclose(mine, theirs, rtol=1e-5, atol=1e-4 * float(np.abs(theirs).max()))
