@@ -17,7 +17,11 @@
  *   oxo_scale_min_k4      KATs tests/test_oxk.c:72-103; exhaustive byte triples
  *                         vs compiled reference
  *   oxo_quantize_q8_k/0   compiled reference through oc_matvec_quantized (the
- *                         activation is left in `temp`); invariants (bsums)
+ *                         activation is left in `temp`); invariants (bsums);
+ *                         rounding ties, largest floats, subnormal scales.
+ *                         Not pinned, because the reference has no single
+ *                         answer there: blocks whose 1/d overflows (largest
+ *                         magnitude below 3.7e-37) and non-finite inputs
  *   oxo_dot_*             compiled reference scalar + dispatched kernels on the
  *                         raw-block generator of tests/test_oxk_avx2_parity.c,
  *                         closed forms, dequantised double-precision cross-check

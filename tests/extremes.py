@@ -39,3 +39,23 @@ def extreme_inputs(n_vec, cols):
     for v in range(n_vec):
         x[v] = pats[v % len(pats)]
     return x
+
+
+def quantiser_edge_inputs(n):
+    e = np.arange(n, dtype=np.float32)
+    c = {}
+    t = (e % 127) + 0.5
+    t[0] = 127.0
+    c["ties, positive"] = t.copy()                       # x / d lands on k + 0.5: round half to even
+    c["ties, negative"] = -t
+    t = ((e % 250) - 125) * 0.5
+    t[1] = 127.0
+    c["half steps"] = t.copy()
+    c["near the largest float"] = np.where(e % 3 == 0, 3.0e38, -1.7e38).astype(np.float32)
+    c["the largest float"] = np.full(n, np.finfo(np.float32).max, np.float32)
+    c["negative zeros"] = np.full(n, -0.0, np.float32)
+    c["subnormal scale"] = (np.float32(1.4e-36) * ((e % 5) - 2) / 2).astype(np.float32)      # d = 1.1e-38
+    c["smallest normal scale"] = (np.float32(1.6e-36) * ((e % 5) - 2) / 2).astype(np.float32)
+    c["smallest scale whose reciprocal is finite"] = (np.float32(3.8e-37) * ((e % 5) - 2) / 2).astype(np.float32)
+    c["one value among zeros"] = np.where(e % 256 == 200, -5.0, 0.0).astype(np.float32)
+    return c

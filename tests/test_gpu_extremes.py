@@ -14,7 +14,7 @@ from oxidize_amd import synth
 
 pytestmark = pytest.mark.gpu
 
-from extremes import TYPES, bits, extreme_inputs, extreme_weights
+from extremes import TYPES, bits, extreme_inputs, extreme_weights, quantiser_edge_inputs
 
 
 @pytest.mark.parametrize("n_vec", [1, 4, 8, 12, 40, 200])
@@ -78,3 +78,31 @@ def test_extreme_integers_large_prefill_tiles(oxh, qt, rows):
         assert o.oxo_matvec_quantized(qt, w.ctypes.data, rows, cols, rb, np.ascontiguousarray(xs[v]).ctypes.data,
                                       want.ctypes.data, temp.ctypes.data) == 0
         assert np.array_equal(bits(got[v]), bits(want)), (qt, rows, v)
+
+
+@pytest.mark.parametrize("qt", [13, 7])
+def test_quantiser_edge_inputs_bit_exact(oxh, qt):
+    """Rounding ties, magnitudes up to the largest float, subnormal block scales: the stand-alone
+    quantiser and the one fused into a GEMV launch both give the oracle's bytes.  (Blocks whose largest
+    magnitude is below 3.7e-37, where 1/d overflows, and non-finite inputs are not compared: there the
+    reference's own scalar and AVX-512 quantisers disagree with each other.)"""
+    n = 512
+    o = oxlibs.oracle()
+    fn = o.oxo_quantize_q8_k if qt == 13 else o.oxo_quantize_q8_0
+    nb = mv.act_bytes(qt, n)
+    w = synth.weights(qt, 16, n, seed=2)
+    d_w, d_o = mv.DeviceBuffer.from_host(w), mv.DeviceBuffer(64)
+    for name, x in quantiser_edge_inputs(n).items():
+        want = np.zeros(nb, np.uint8)
+        fn(x.ctypes.data, n, want.ctypes.data)
+        d_x, d_a, d_a2 = mv.DeviceBuffer.from_host(x), mv.DeviceBuffer(nb), mv.DeviceBuffer(nb)
+        mv.quantize(qt, d_x.ptr, n, 1, n, d_a.ptr)
+        assert np.array_equal(d_a.download(np.uint8, nb), want), name
+        mv.gemv_segments_f32(qt, mv.make_segments([(d_w.ptr, d_o.ptr, 16, 0)]), n, d_x.ptr, n, d_a2.ptr, 1, 16)
+        assert np.array_equal(d_a2.download(np.uint8, nb), want), name + " (fused)"
+        ref = oxlibs.ref()
+        if ref is not None:
+            out, temp = np.zeros(16, np.float32), np.zeros(n, np.float32)
+            ref.oc_matvec_quantized(qt, w.ctypes.data, 16, n, synth.row_bytes(qt, n), x.ctypes.data,
+                                    out.ctypes.data, temp.ctypes.data)
+            assert np.array_equal(temp.view(np.uint8)[:nb], want), name + " (compiled reference)"

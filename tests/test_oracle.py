@@ -950,3 +950,25 @@ def test_extreme_integers_oracle_vs_compiled_reference(qt):
             assert np.array_equal(mine.view(np.uint32), theirs.view(np.uint32)), (qt, v)
         else:       # the x86 kernels of the 32-value formats sum in another order
             assert np.allclose(mine, theirs, rtol=1e-5, atol=1e-4 * float(np.abs(theirs).max()))
+
+
+@pytest.mark.parametrize("qt", [13, 7])
+def test_quantiser_edge_inputs_oracle_vs_compiled_reference(qt):
+    # rounding ties, the largest floats, subnormal block scales (not: blocks whose 1/d overflows and
+    # non-finite inputs, where the reference's scalar and AVX-512 quantisers disagree with each other)
+    from extremes import quantiser_edge_inputs
+    ref = oxlibs.ref()
+    if ref is None:
+        pytest.skip("oracle/_ref was not built")
+    n = 512
+    fn = O.oxo_quantize_q8_k if qt == 13 else O.oxo_quantize_q8_0
+    nb = n // 256 * 292 if qt == 13 else n // 32 * 34
+    w = synth.weights(qt, 4, n, seed=2)
+    for name, x in quantiser_edge_inputs(n).items():
+        want = np.zeros(nb, np.uint8)
+        fn(x.ctypes.data, n, want.ctypes.data)
+        out, temp = np.zeros(4, np.float32), np.zeros(n, np.float32)
+        ref.oc_matvec_quantized(qt, w.ctypes.data, 4, n, synth.row_bytes(qt, n), x.ctypes.data, out.ctypes.data,
+                                temp.ctypes.data)
+        assert np.array_equal(temp.view(np.uint8)[:nb], want), name
+
