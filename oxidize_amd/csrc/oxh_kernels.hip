@@ -798,6 +798,12 @@ static hipError_t raise_all_lds_ceilings(void)
     if ((e = raise_lds_ceiling(k_mfma_q8_0_segments<4, 5>)) != hipSuccess) return e;
     if ((e = raise_lds_ceiling(k_mmq_q6_k_segments<1, 1, 4, 2>)) != hipSuccess) return e;
     if ((e = raise_lds_ceiling(k_mmq_q6_k_experts<1, 1, 4, 2>)) != hipSuccess) return e;
+    if ((e = raise_lds_ceiling(k_mmq_q6_k_experts<1, 1, 8, 2>)) != hipSuccess) return e;
+    if ((e = raise_lds_ceiling(k_mmq_q6_k_segments<1, 1, 8, 2>)) != hipSuccess) return e;
+    if ((e = raise_lds_ceiling(k_mmq_q5_k_segments<1, 1, 8, 2>)) != hipSuccess) return e;
+    if ((e = raise_lds_ceiling(k_mmq_q4_k_segments<1, 1, 8, 3>)) != hipSuccess) return e;
+    if ((e = raise_lds_ceiling(k_mmq_q45_k_experts<1, 1, 8, false, 3>)) != hipSuccess) return e;
+    if ((e = raise_lds_ceiling(k_mmq_q45_k_experts<1, 1, 8, true, 2>)) != hipSuccess) return e;
     if ((e = raise_lds_ceiling(k_mmq_q6_k_experts<4, 1, 8, 1>)) != hipSuccess) return e;
     if ((e = raise_lds_ceiling(k_mmq_q45_k_experts<4, 1, 8, false, 1>)) != hipSuccess) return e;
     if ((e = raise_lds_ceiling(k_mmq_q45_k_experts<4, 1, 8, true, 1>)) != hipSuccess) return e;
@@ -984,6 +990,18 @@ static int launch_mmq_segments(uint32_t qtype, const OxhSegment *segs, size_t n_
         if (rc) return rc;
         acts = (const uint8_t *)io.d_act_out;
     }
+    /* A launch whose 64-row tiles would give at most two workgroups per CU, but whose 128-row tiles still
+     * give nearly every CU one, takes those on eight waves with two or three super-blocks per stage:
+     * half as much again in flight per CU (OXH_MOE_WIDE_SMALL=0 switches it off). */
+    static const uint32_t wide_ok = env_u32("OXH_MOE_WIDE_SMALL", 1, 0, 1);
+    const size_t cus = (size_t)(g_n_cu > 0 ? g_n_cu : 256);
+    size_t wg64 = 0, wg128 = 0;
+    for (size_t i = 0; i < n_segs; i++) {
+        wg64 += (segs[i].rows + 63) / 64;
+        wg128 += (segs[i].rows + 127) / 128;
+    }
+    const bool wide = wide_ok && wg64 <= 2u * cus && wg128 >= cus - cus / 8;
+    const size_t tile_rows = wide ? 128 : G::ROWS;
     SegTable t;
     memset(&t, 0, sizeof t);
     uint32_t wg = 0, n = 0;
@@ -995,11 +1013,31 @@ static int launch_mmq_segments(uint32_t qtype, const OxhSegment *segs, size_t n_
         t.s[n].act_first = (uint32_t)segs[i].act_first;
         t.s[n].nv = (uint32_t)(segs[i].n_vec ? segs[i].n_vec : n_vec_default);
         t.s[n].wg_begin = wg;
-        wg += (uint32_t)((segs[i].rows + G::ROWS - 1) / G::ROWS);
+        wg += (uint32_t)((segs[i].rows + tile_rows - 1) / tile_rows);
         n++;
     }
     t.n = n;
     for (uint32_t i = 1; i < 4 && i < n; i++) t.bound[i - 1] = t.s[i].wg_begin;
+    if (wide) {
+        typedef MmqGeom<1, 1, 8> W4;
+        typedef Mmq6Geom<1, 1, 8> W6;
+        typedef MmqGeom<1, 1, 8, true> W5;
+        static_assert(W4::ROWS == 128 && W6::ROWS == 128 && W5::ROWS == 128, "128-row tiles");
+        hipStream_t ws = pick_stream(stream);
+        const uint32_t wb = (uint32_t)blocks;
+        /* super-blocks per stage: what fits the LDS (Q4_K's 144-byte rows leave room for three) */
+        if (qtype == OXH_Q6_K)
+            hipLaunchKernelGGL((k_mmq_q6_k_segments<1, 1, 8, 2>), dim3(wg), dim3(512), 2 * W6::LDS_BYTES, ws, t, wb,
+                               acts, out_stride);
+        else if (is_q5k(qtype))
+            hipLaunchKernelGGL((k_mmq_q5_k_segments<1, 1, 8, 2>), dim3(wg), dim3(512), 2 * W5::LDS_BYTES, ws, t, wb,
+                               acts, out_stride);
+        else
+            hipLaunchKernelGGL((k_mmq_q4_k_segments<1, 1, 8, 3>), dim3(wg), dim3(512), 3 * W4::LDS_BYTES, ws, t, wb,
+                               acts, out_stride);
+        HIP_TRY(hipGetLastError());
+        return OXH_OK;
+    }
     typedef Mmq6Geom<1, 1, 4> G6;                           /* same 64-row tiles */
     typedef MmqGeom<1, 1, 4, true> G5;
     static_assert(G6::ROWS == G::ROWS && G5::ROWS == G::ROWS, "segment tiling is shared by all formats");
@@ -1576,7 +1614,7 @@ extern "C" int oxh_moe_route(const float *d_logits, size_t n_tok, size_t n_exper
 
 /* one launch of the MFMA tile kernel over all experts, activation runs from device memory */
 /* one or more launches of the MFMA tile kernel over all experts, activation runs from device memory.
- * `avg_tokens` = pairs per expert on average: from about two dozen on, the 128-row x 64-token tile
+ * `pairs` = (token, expert) pairs in all; from about two dozen per expert on average on, the 128-row x 64-token tile
  * (eight waves) re-streams an expert's weights four times less often than the 64 x 16 one. */
 template <int TC, int WAVES>
 static int launch_experts_tiled(uint32_t qtype, const void *const *d_w, float *const *d_out, size_t n_mat,
@@ -1616,10 +1654,13 @@ static int launch_experts_tiled(uint32_t qtype, const void *const *d_w, float *c
         t.n = n;
         for (uint32_t i = 1; i < 4 && i < n; i++) t.bound[i - 1] = t.s[i].wg_begin;
         /* two super-blocks per stage only for the small tile (the large one has no LDS to spare) */
-        if (TC == 1 && mmq_deep_stages(wg)) {
-            if (qtype == OXH_Q6_K) OXH_EXP_LAUNCH((k_mmq_q6_k_experts<TC, 1, WAVES, TC == 1 ? 2 : 1>), G6, TC == 1 ? 2 : 1);
-            else if (is_q5k(qtype)) OXH_EXP_LAUNCH((k_mmq_q45_k_experts<TC, 1, WAVES, true, TC == 1 ? 2 : 1>), G5, TC == 1 ? 2 : 1);
-            else OXH_EXP_LAUNCH((k_mmq_q45_k_experts<TC, 1, WAVES, false, TC == 1 ? 2 : 1>), G, TC == 1 ? 2 : 1);
+        /* super-blocks per stage: what fits the LDS (Q4_K's 144-byte rows leave room for three on eight waves) */
+        constexpr int DEEP = TC == 1 ? 2 : 1;
+        constexpr int DEEP4 = TC == 1 ? (WAVES == 8 ? 3 : 2) : 1;
+        if (TC == 1 && (WAVES == 8 || mmq_deep_stages(wg))) {
+            if (qtype == OXH_Q6_K) OXH_EXP_LAUNCH((k_mmq_q6_k_experts<TC, 1, WAVES, DEEP>), G6, DEEP);
+            else if (is_q5k(qtype)) OXH_EXP_LAUNCH((k_mmq_q45_k_experts<TC, 1, WAVES, true, DEEP>), G5, DEEP);
+            else OXH_EXP_LAUNCH((k_mmq_q45_k_experts<TC, 1, WAVES, false, DEEP4>), G, DEEP4);
         } else {
             if (qtype == OXH_Q6_K) OXH_EXP_LAUNCH((k_mmq_q6_k_experts<TC, 1, WAVES, 1>), G6, 1);
             else if (is_q5k(qtype)) OXH_EXP_LAUNCH((k_mmq_q45_k_experts<TC, 1, WAVES, true, 1>), G5, 1);
@@ -1633,11 +1674,24 @@ static int launch_experts_tiled(uint32_t qtype, const void *const *d_w, float *c
 
 static int launch_experts(uint32_t qtype, const void *const *d_w, float *const *d_out, size_t n_mat,
                           size_t n_expert, size_t rows, size_t cols, const void *d_acts, size_t out_stride,
-                          const uint32_t *d_counts, const uint32_t *d_offsets, size_t avg_tokens, void *stream)
+                          const uint32_t *d_counts, const uint32_t *d_offsets, size_t pairs, void *stream)
 {
     static const uint32_t big_from = env_u32("OXH_MOE_BIG_TILE_FROM", 24, 0, 4096);     /* 0 = never */
+    const size_t avg_tokens = pairs / n_expert;
     if (big_from && avg_tokens >= big_from)
         return launch_experts_tiled<4, 8>(qtype, d_w, d_out, n_mat, n_expert, rows, cols, d_acts, out_stride,
+                                          d_counts, d_offsets, stream);
+    /* few rows per expert (a down projection): the 64-row tile would give at most two workgroups per CU;
+     * 128 rows on eight waves with two or three super-blocks per stage keep half as much again in flight
+     * (Mixtral's down projections at 16 tokens: 67 against 74 us).  Workgroups of experts without a token
+     * leave at once, so what counts is the experts that can have one; with too few of them the smaller
+     * tile spreads over more CUs. */
+    static const uint32_t wide = env_u32("OXH_MOE_WIDE_SMALL", 1, 0, 1);
+    const size_t cus = (size_t)(g_n_cu > 0 ? g_n_cu : 256);
+    const size_t live = pairs < n_expert ? (pairs ? pairs : 1) : n_expert;
+    if (wide && n_mat * n_expert * ((rows + 63) / 64) <= 2u * cus &&
+        n_mat * live * ((rows + 127) / 128) >= cus - cus / 8)
+        return launch_experts_tiled<1, 8>(qtype, d_w, d_out, n_mat, n_expert, rows, cols, d_acts, out_stride,
                                           d_counts, d_offsets, stream);
     return launch_experts_tiled<1, 4>(qtype, d_w, d_out, n_mat, n_expert, rows, cols, d_acts, out_stride,
                                       d_counts, d_offsets, stream);
@@ -1671,15 +1725,14 @@ extern "C" int oxh_moe_ffn(const OxhMoe *m, const float *d_logits, const float *
     /* 3. gate and up of every expert over its own pairs */
     const void *w_gu[2] = { m->d_w_gate, m->d_w_up };
     float *o_gu[2] = { gate, up };
-    const size_t avg_tokens = pairs / m->n_expert;
     if ((rc = launch_experts(m->qtype_gate_up, w_gu, o_gu, 2, m->n_expert, m->ffn, m->hidden, ws + l.act_x,
-                             m->ffn, counts, offsets, avg_tokens, stream))) return rc;
+                             m->ffn, counts, offsets, pairs, stream))) return rc;
     /* 4. h = silu(gate) * up, quantised; 5. down */
     if ((rc = quantize_q8_k_ex(gate, m->ffn, pairs, m->ffn, ws + l.act_h, nullptr, up, stream))) return rc;
     const void *w_dn[1] = { m->d_w_down };
     float *o_dn[1] = { y };
     if ((rc = launch_experts(m->qtype_down, w_dn, o_dn, 1, m->n_expert, m->hidden, m->ffn, ws + l.act_h,
-                             m->hidden, counts, offsets, avg_tokens, stream))) return rc;
+                             m->hidden, counts, offsets, pairs, stream))) return rc;
     /* 6. combine in ascending expert order */
     hipLaunchKernelGGL(k_moe_combine, dim3((uint32_t)((m->hidden + 255u) / 256u), (uint32_t)n_tok), dim3(256), 0,
                        pick_stream(stream), (const float *)y, m->hidden, (const int32_t *)ids, (const float *)wts,

@@ -186,6 +186,25 @@ def test_mmq_tile_variants_ragged(oxh, qtype, rows, cols, n_vec):
     assert np.array_equal(bits(got), bits(out[:, :rows]))
 
 
+@pytest.mark.parametrize("qtype", [Q4K, Q5K, Q6K])
+def test_small_batch_launch_on_128_row_tiles(oxh, qtype):
+    """Five activations over 30000 rows: 469 tiles of 64 rows would be fewer than two per CU on a 256-CU
+    device, 235 tiles of 128 rows still nearly one per CU, so the launch takes the eight-wave tile with two
+    (Q5_K, Q6_K) or three (Q4_K) super-blocks per stage; the last tile is ragged.  Bits against the oracle."""
+    rows, cols, n_vec = 30000, 768, 5
+    w = synth.weights(qtype, rows, cols, seed=12, stream=3)
+    xs = synth.normal(n_vec * cols, seed=12, stream=4).reshape(n_vec, cols)
+    d_w, d_x = mv.DeviceBuffer.from_host(w), mv.DeviceBuffer.from_host(xs)
+    d_a = mv.DeviceBuffer(n_vec * mv.act_bytes(qtype, cols))
+    d_o = mv.DeviceBuffer(n_vec * rows * 4)
+    mv.gemv_segments_f32(qtype, mv.make_segments([(d_w.ptr, d_o.ptr, rows, 0)]), cols, d_x.ptr, cols, d_a.ptr,
+                         n_vec, rows)
+    got = d_o.download(np.float32, n_vec * rows).reshape(n_vec, rows)
+    for v in range(n_vec):
+        want, _ = oracle_matvec(qtype, w, rows, cols, np.ascontiguousarray(xs[v]))
+        assert np.array_equal(bits(got[v]), bits(want)), v
+
+
 def test_config4_moe_expert_gemvs(oxh):
     ms = workloads.MoESet(seed=0, keep_host=True)
     o = oxlibs.oracle()

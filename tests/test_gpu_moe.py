@@ -245,6 +245,15 @@ def test_layer_with_prefill_sized_token_counts(oxh, qt_gu, qt_dn):
         set(range(0, n, 37))))
 
 
+@pytest.mark.parametrize("qt_gu,qt_dn", [(Q4K, Q4K), (Q4K, Q6K), (Q6K, Q5K)])
+def test_layer_whose_down_projection_takes_the_128_row_tile(oxh, qt_gu, qt_dn):
+    """8 experts x 4096 output rows: 512 workgroups of the 64-row tile (two per CU on a 256-CU device), so
+    the down launch runs on 128-row tiles of eight waves with two or three super-blocks per stage; likewise
+    9 experts x 3584 rows."""
+    check_layer(qt_gu, qt_dn, 8, 2, 4096, 256, 16, seed=31, skew=False)
+    check_layer(qt_gu, qt_dn, 9, 3, 3584, 512, 9, seed=32, skew=True)
+
+
 def test_layer_with_more_experts_than_one_launch_carries(oxh):
     """40 and 64 experts: the gate/up launch carries 16 experts, the down launch 32, so both repeat."""
     check_layer(Q4K, Q4K, 40, 4, 256, 256, 50, seed=8, skew=True)
