@@ -798,12 +798,8 @@ static hipError_t raise_all_lds_ceilings(void)
     if ((e = raise_lds_ceiling(k_mfma_q8_0_segments<4, 5>)) != hipSuccess) return e;
     if ((e = raise_lds_ceiling(k_mmq_q6_k_segments<1, 1, 4, 2>)) != hipSuccess) return e;
     if ((e = raise_lds_ceiling(k_mmq_q6_k_experts<1, 1, 4, 2>)) != hipSuccess) return e;
-    if ((e = raise_lds_ceiling(k_mmq_q6_k_experts<1, 1, 8, 2>)) != hipSuccess) return e;
-    if ((e = raise_lds_ceiling(k_mmq_q6_k_segments<1, 1, 8, 2>)) != hipSuccess) return e;
-    if ((e = raise_lds_ceiling(k_mmq_q5_k_segments<1, 1, 8, 2>)) != hipSuccess) return e;
     if ((e = raise_lds_ceiling(k_mmq_q4_k_segments<1, 1, 8, 3>)) != hipSuccess) return e;
     if ((e = raise_lds_ceiling(k_mmq_q45_k_experts<1, 1, 8, false, 3>)) != hipSuccess) return e;
-    if ((e = raise_lds_ceiling(k_mmq_q45_k_experts<1, 1, 8, true, 2>)) != hipSuccess) return e;
     if ((e = raise_lds_ceiling(k_mmq_q6_k_experts<4, 1, 8, 1>)) != hipSuccess) return e;
     if ((e = raise_lds_ceiling(k_mmq_q45_k_experts<4, 1, 8, false, 1>)) != hipSuccess) return e;
     if ((e = raise_lds_ceiling(k_mmq_q45_k_experts<4, 1, 8, true, 1>)) != hipSuccess) return e;
@@ -990,9 +986,10 @@ static int launch_mmq_segments(uint32_t qtype, const OxhSegment *segs, size_t n_
         if (rc) return rc;
         acts = (const uint8_t *)io.d_act_out;
     }
-    /* A launch whose 64-row tiles would give at most two workgroups per CU, but whose 128-row tiles still
-     * give nearly every CU one, takes those on eight waves with two or three super-blocks per stage:
-     * half as much again in flight per CU (OXH_MOE_WIDE_SMALL=0 switches it off). */
+    /* A Q4_K launch whose 64-row tiles would give at most two workgroups per CU, but whose 128-row tiles
+     * still give nearly every CU one, takes those on eight waves with three super-blocks per stage: half as
+     * much again in flight per CU (OXH_MOE_WIDE_SMALL=0 switches it off).  Q5_K and Q6_K rows leave room
+     * for two per stage only, and with two the wider tile measured slower than the 64-row one. */
     static const uint32_t wide_ok = env_u32("OXH_MOE_WIDE_SMALL", 1, 0, 1);
     const size_t cus = (size_t)(g_n_cu > 0 ? g_n_cu : 256);
     size_t wg64 = 0, wg128 = 0;
@@ -1000,7 +997,7 @@ static int launch_mmq_segments(uint32_t qtype, const OxhSegment *segs, size_t n_
         wg64 += (segs[i].rows + 63) / 64;
         wg128 += (segs[i].rows + 127) / 128;
     }
-    const bool wide = wide_ok && wg64 <= 2u * cus && wg128 >= cus - cus / 8;
+    const bool wide = wide_ok && is_q4k(qtype) && wg64 <= 2u * cus && wg128 >= cus - cus / 8;
     const size_t tile_rows = wide ? 128 : G::ROWS;
     SegTable t;
     memset(&t, 0, sizeof t);
@@ -1020,21 +1017,9 @@ static int launch_mmq_segments(uint32_t qtype, const OxhSegment *segs, size_t n_
     for (uint32_t i = 1; i < 4 && i < n; i++) t.bound[i - 1] = t.s[i].wg_begin;
     if (wide) {
         typedef MmqGeom<1, 1, 8> W4;
-        typedef Mmq6Geom<1, 1, 8> W6;
-        typedef MmqGeom<1, 1, 8, true> W5;
-        static_assert(W4::ROWS == 128 && W6::ROWS == 128 && W5::ROWS == 128, "128-row tiles");
-        hipStream_t ws = pick_stream(stream);
-        const uint32_t wb = (uint32_t)blocks;
-        /* super-blocks per stage: what fits the LDS (Q4_K's 144-byte rows leave room for three) */
-        if (qtype == OXH_Q6_K)
-            hipLaunchKernelGGL((k_mmq_q6_k_segments<1, 1, 8, 2>), dim3(wg), dim3(512), 2 * W6::LDS_BYTES, ws, t, wb,
-                               acts, out_stride);
-        else if (is_q5k(qtype))
-            hipLaunchKernelGGL((k_mmq_q5_k_segments<1, 1, 8, 2>), dim3(wg), dim3(512), 2 * W5::LDS_BYTES, ws, t, wb,
-                               acts, out_stride);
-        else
-            hipLaunchKernelGGL((k_mmq_q4_k_segments<1, 1, 8, 3>), dim3(wg), dim3(512), 3 * W4::LDS_BYTES, ws, t, wb,
-                               acts, out_stride);
+        static_assert(W4::ROWS == 128, "128-row tiles");
+        hipLaunchKernelGGL((k_mmq_q4_k_segments<1, 1, 8, 3>), dim3(wg), dim3(512), 3 * W4::LDS_BYTES,
+                           pick_stream(stream), t, (uint32_t)blocks, acts, out_stride);
         HIP_TRY(hipGetLastError());
         return OXH_OK;
     }
@@ -1653,14 +1638,15 @@ static int launch_experts_tiled(uint32_t qtype, const void *const *d_w, float *c
             }
         t.n = n;
         for (uint32_t i = 1; i < 4 && i < n; i++) t.bound[i - 1] = t.s[i].wg_begin;
-        /* two super-blocks per stage only for the small tile (the large one has no LDS to spare) */
-        /* super-blocks per stage: what fits the LDS (Q4_K's 144-byte rows leave room for three on eight waves) */
-        constexpr int DEEP = TC == 1 ? 2 : 1;
-        constexpr int DEEP4 = TC == 1 ? (WAVES == 8 ? 3 : 2) : 1;
-        if (TC == 1 && (WAVES == 8 || mmq_deep_stages(wg))) {
-            if (qtype == OXH_Q6_K) OXH_EXP_LAUNCH((k_mmq_q6_k_experts<TC, 1, WAVES, DEEP>), G6, DEEP);
-            else if (is_q5k(qtype)) OXH_EXP_LAUNCH((k_mmq_q45_k_experts<TC, 1, WAVES, true, DEEP>), G5, DEEP);
-            else OXH_EXP_LAUNCH((k_mmq_q45_k_experts<TC, 1, WAVES, false, DEEP4>), G, DEEP4);
+        /* super-blocks per stage: one in the large tile (no LDS to spare), two in the 64-row tile when the
+         * launch is small, three in the 128-row one (Q4_K only) */
+        if constexpr (TC == 1 && WAVES == 8) {
+            if (!is_q4k(qtype)) return arg_fail("moe: the 128-row small tile exists for Q4_K only");
+            OXH_EXP_LAUNCH((k_mmq_q45_k_experts<1, 1, 8, false, 3>), G, 3);
+        } else if (TC == 1 && mmq_deep_stages(wg)) {
+            if (qtype == OXH_Q6_K) OXH_EXP_LAUNCH((k_mmq_q6_k_experts<TC, 1, WAVES, 2>), G6, 2);
+            else if (is_q5k(qtype)) OXH_EXP_LAUNCH((k_mmq_q45_k_experts<TC, 1, WAVES, true, 2>), G5, 2);
+            else OXH_EXP_LAUNCH((k_mmq_q45_k_experts<TC, 1, WAVES, false, 2>), G, 2);
         } else {
             if (qtype == OXH_Q6_K) OXH_EXP_LAUNCH((k_mmq_q6_k_experts<TC, 1, WAVES, 1>), G6, 1);
             else if (is_q5k(qtype)) OXH_EXP_LAUNCH((k_mmq_q45_k_experts<TC, 1, WAVES, true, 1>), G5, 1);
@@ -1682,14 +1668,15 @@ static int launch_experts(uint32_t qtype, const void *const *d_w, float *const *
         return launch_experts_tiled<4, 8>(qtype, d_w, d_out, n_mat, n_expert, rows, cols, d_acts, out_stride,
                                           d_counts, d_offsets, stream);
     /* few rows per expert (a down projection): the 64-row tile would give at most two workgroups per CU;
-     * 128 rows on eight waves with two or three super-blocks per stage keep half as much again in flight
-     * (Mixtral's down projections at 16 tokens: 67 against 74 us).  Workgroups of experts without a token
+     * Q4_K takes 128 rows on eight waves with three super-blocks per stage, half as much again in flight
+     * (Mixtral's down projections at 16 tokens: 67 against 74 us; Q5_K and Q6_K rows leave room for two per
+     * stage only, and with two the wider tile measured slower).  Workgroups of experts without a token
      * leave at once, so what counts is the experts that can have one; with too few of them the smaller
      * tile spreads over more CUs. */
     static const uint32_t wide = env_u32("OXH_MOE_WIDE_SMALL", 1, 0, 1);
     const size_t cus = (size_t)(g_n_cu > 0 ? g_n_cu : 256);
     const size_t live = pairs < n_expert ? (pairs ? pairs : 1) : n_expert;
-    if (wide && n_mat * n_expert * ((rows + 63) / 64) <= 2u * cus &&
+    if (wide && is_q4k(qtype) && n_mat * n_expert * ((rows + 63) / 64) <= 2u * cus &&
         n_mat * live * ((rows + 127) / 128) >= cus - cus / 8)
         return launch_experts_tiled<1, 8>(qtype, d_w, d_out, n_mat, n_expert, rows, cols, d_acts, out_stride,
                                           d_counts, d_offsets, stream);

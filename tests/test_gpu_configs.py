@@ -189,8 +189,9 @@ def test_mmq_tile_variants_ragged(oxh, qtype, rows, cols, n_vec):
 @pytest.mark.parametrize("qtype", [Q4K, Q5K, Q6K])
 def test_small_batch_launch_on_128_row_tiles(oxh, qtype):
     """Five activations over 30000 rows: 469 tiles of 64 rows would be fewer than two per CU on a 256-CU
-    device, 235 tiles of 128 rows still nearly one per CU, so the launch takes the eight-wave tile with two
-    (Q5_K, Q6_K) or three (Q4_K) super-blocks per stage; the last tile is ragged.  Bits against the oracle."""
+    device, 235 tiles of 128 rows still nearly one per CU, so a Q4_K launch takes the eight-wave tile with
+    three super-blocks per stage (Q5_K and Q6_K stay on 64-row tiles with two); the last tile is ragged.
+    Bits against the oracle."""
     rows, cols, n_vec = 30000, 768, 5
     w = synth.weights(qtype, rows, cols, seed=12, stream=3)
     xs = synth.normal(n_vec * cols, seed=12, stream=4).reshape(n_vec, cols)

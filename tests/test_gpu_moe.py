@@ -248,8 +248,8 @@ def test_layer_with_prefill_sized_token_counts(oxh, qt_gu, qt_dn):
 @pytest.mark.parametrize("qt_gu,qt_dn", [(Q4K, Q4K), (Q4K, Q6K), (Q6K, Q5K)])
 def test_layer_whose_down_projection_takes_the_128_row_tile(oxh, qt_gu, qt_dn):
     """8 experts x 4096 output rows: 512 workgroups of the 64-row tile (two per CU on a 256-CU device), so
-    the down launch runs on 128-row tiles of eight waves with two or three super-blocks per stage; likewise
-    9 experts x 3584 rows."""
+    a Q4_K down launch runs on 128-row tiles of eight waves with three super-blocks per stage (the other
+    types stay on 64-row tiles with two); likewise 9 experts x 3584 rows."""
     check_layer(qt_gu, qt_dn, 8, 2, 4096, 256, 16, seed=31, skew=False)
     check_layer(qt_gu, qt_dn, 9, 3, 3584, 512, 9, seed=32, skew=True)
 
