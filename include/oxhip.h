@@ -319,6 +319,13 @@ int  oxh_free(void *d_ptr);
 int  oxh_memcpy_h2d(void *d_dst, const void *h_src, size_t bytes, void *stream);
 int  oxh_memcpy_d2h(void *h_dst, const void *d_src, size_t bytes, void *stream);
 int  oxh_memcpy_d2d(void *d_dst, const void *d_src, size_t bytes, void *stream);
+/* Rows of `width` bytes between a host matrix with `h_pitch` bytes per row and a device matrix with
+ * `d_pitch`: a padded batch travels in one copy (oc_matvec_quantized_batch's in_stride / out_stride). */
+int  oxh_memcpy2d_h2d(void *d_dst, size_t d_pitch, const void *h_src, size_t h_pitch, size_t width,
+                      size_t height, void *stream);
+int  oxh_memcpy2d_d2h(void *h_dst, size_t h_pitch, const void *d_src, size_t d_pitch, size_t width,
+                      size_t height, void *stream);
+/* A fill kernel, not a memset node: safe between oxh_graph_begin and oxh_graph_end. */
 int  oxh_memset(void *d_dst, int value, size_t bytes, void *stream);
 int  oxh_stream_create(void **stream);
 int  oxh_stream_destroy(void *stream);
@@ -400,17 +407,35 @@ uint32_t oxh_qtype_from_ggml_id(uint32_t ggml_id);
 
 /* Make the bytes at [h_data, h_data+bytes) resident in HBM and remember the
  * mapping, so later calls that pass any pointer inside that range (a whole
- * tensor or an expert slice of a stacked tensor) run without an upload.
- * Modelled on oc_cuda_init's weight upload (oxidize-c/src/backends/cuda.cu:
- * 633-712).  Unregistered weights are registered on first use.  As in the
- * reference, weights are taken to be immutable while registered: the host
- * bytes are not looked at again, so unregister before reusing the memory. */
+ * tensor or an expert slice of a stacked tensor) run without an upload and
+ * without looking at the host bytes.  Modelled on oc_cuda_init's weight upload
+ * (oxidize-c/src/backends/cuda.cu:633-712).  Registered weights are taken to
+ * be immutable, as there: unregister before reusing the memory.
+ *
+ * Weights the caller never registered keep the reference's contract, under
+ * which the host bytes are the input of every call (oxidize-c/include/oxidize/
+ * matvec.h:45-52): the device copy made on first sight serves only the exact
+ * (pointer, byte count) it was made for, every later call re-checks a
+ * fingerprint of the host bytes (length, first and last 4 KiB, 128 strided
+ * 64-byte samples; a few microseconds) and refreshes the copy when it differs,
+ * and a matrix that overlaps older cached ones replaces them.  So freeing a
+ * model and loading another at the same addresses is safe without any call
+ * here.  What the sampled fingerprint can miss is an edit of a few bytes in
+ * the middle of a matrix that stays in place: OXH_WEIGHT_CACHE=full hashes
+ * every byte on every call, OXH_WEIGHT_CACHE=off uploads on every call.
+ * OXH_WEIGHT_CACHE_MB (default 65536) bounds the bytes cached this way; the
+ * least recently used go first. */
 int oxh_weight_register(const void *h_data, size_t bytes);
+/* Drops every range, registered or cached, that contains h_data. */
 int oxh_weight_unregister(const void *h_data);
-/* Drop every registered range (the host memory may then be reused or freed). */
+/* Drop every range (the host memory may then be reused or freed). */
 int oxh_weight_clear(void);
-/* Device address backing a registered host pointer, or NULL. */
+/* Device address backing a host pointer inside a registered or cached range, or NULL. */
 const void *oxh_weight_device_ptr(const void *h_data);
+/* Counts of registered and cached ranges, the bytes cached, and how many times
+ * a cached copy was refreshed because its host bytes had changed.  Any pointer
+ * may be NULL. */
+int oxh_weight_stats(size_t *n_registered, size_t *n_cached, size_t *cached_bytes, size_t *refreshes);
 
 /* Same arguments and results as oc_matvec_quantized
  * (oxidize-c/include/oxidize/matvec.h:50-52; matvec.c:833-907): output[r] =
@@ -445,9 +470,14 @@ int oxh_matvec_quantized_batch(uint32_t qtype, const uint8_t *data,
 
 /* The reference's own symbols (matvec.h:50-52, :62-66, :72-76, :118-124,
  * :132, :146-147, :81-88).  They call the oxh_ functions above.  Because they
- * return void, a decline or failure is routed to the handler installed with
- * oxh_set_decline_handler(); with no handler installed the process prints the
- * error and aborts — it never silently computes on the CPU. */
+ * return void, a call that comes back declined or failed is handed on, with
+ * its original arguments, to the CPU functions installed with
+ * oxh_set_cpu_fallback(); failing that to the symbols oc_ref_matvec_quantized,
+ * _fused, _multi_input and _batch when the program defines them (weak
+ * references: the reference's own functions under another name); failing that
+ * the handler of oxh_set_decline_handler() is told; and with none of the three
+ * the process prints the error and aborts.  This library never computes on
+ * the CPU itself. */
 typedef struct {
     size_t activation_quantizations;
     size_t parallel_dispatches;
@@ -480,9 +510,32 @@ bool oc_matvec_fused_enabled(void);
 void oc_matvec_fused_test_reset(void);
 OcMatvecFusedTestStats oc_matvec_fused_test_stats(void);
 
+/* The caller's CPU implementations of the four entry points (the reference's
+ * own oc_matvec_quantized* under whatever names the build gives them); a NULL
+ * member falls through to the weak oc_ref_* symbol of that entry.  NULL clears
+ * the table.  Set before the first matvec call; not synchronised with calls in
+ * flight. */
+typedef struct OxhCpuFallback {
+    void (*matvec_quantized)(uint32_t qtype, const uint8_t *data, size_t rows, size_t cols, size_t row_bytes,
+                             const float *input, float *output, float *temp);
+    void (*matvec_quantized_fused)(const uint32_t *qtypes, const uint8_t *const *datas, const size_t *rows,
+                                   size_t cols, const size_t *row_bytes, size_t n_outs, const float *input,
+                                   float *const *outs, float *temp);
+    void (*matvec_quantized_multi_input)(const uint32_t *qtypes, const uint8_t *const *datas, const size_t *rows,
+                                         size_t cols, const size_t *row_bytes, size_t n_outs,
+                                         const float *const *inputs, float *const *outs, float *temp);
+    void (*matvec_quantized_batch)(uint32_t qtype, const uint8_t *data, size_t rows, size_t cols,
+                                   size_t row_bytes, const float *inputs, size_t in_stride, float *outputs,
+                                   size_t out_stride, size_t n_vec, float *temp, uint8_t *act_scratch,
+                                   size_t act_bytes);
+} OxhCpuFallback;
+void oxh_set_cpu_fallback(const OxhCpuFallback *fb);
+/* Calls handed on to a CPU fallback so far. */
+size_t oxh_cpu_fallback_calls(void);
+
 /* Called by the void oc_matvec_* symbols when the oxh_ call did not return
- * OXH_OK.  `which` is 0 single, 1 fused, 2 multi_input, 3 batch; `status` is
- * the oxh_ status.  A maintainer points this at the original CPU functions. */
+ * OXH_OK and no CPU fallback exists for that entry.  `which` is 0 single,
+ * 1 fused, 2 multi_input, 3 batch; `status` is the oxh_ status. */
 typedef void (*OxhDeclineHandler)(int which, int status, void *user);
 void oxh_set_decline_handler(OxhDeclineHandler fn, void *user);
 

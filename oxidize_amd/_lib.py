@@ -75,6 +75,8 @@ SIGNATURES = {
     "oxh_memcpy_h2d": (I, [V, V, Z, V]),
     "oxh_memcpy_d2h": (I, [V, V, Z, V]),
     "oxh_memcpy_d2d": (I, [V, V, Z, V]),
+    "oxh_memcpy2d_h2d": (I, [V, Z, V, Z, Z, Z, V]),
+    "oxh_memcpy2d_d2h": (I, [V, Z, V, Z, Z, Z, V]),
     "oxh_memset": (I, [V, I, Z, V]),
     "oxh_stream_create": (I, [ctypes.POINTER(V)]),
     "oxh_stream_destroy": (I, [V]),
@@ -105,6 +107,7 @@ SIGNATURES = {
     "oxh_weight_unregister": (I, [V]),
     "oxh_weight_clear": (I, []),
     "oxh_weight_device_ptr": (V, [V]),
+    "oxh_weight_stats": (I, [ctypes.POINTER(Z), ctypes.POINTER(Z), ctypes.POINTER(Z), ctypes.POINTER(Z)]),
     "oxh_matvec_quantized": (I, [U32, V, Z, Z, Z, V, V, V]),
     "oxh_matvec_quantized_fused": (I, [V, V, V, Z, V, Z, V, V, V]),
     "oxh_matvec_quantized_multi_input": (I, [V, V, V, Z, V, Z, V, V, V]),
@@ -119,6 +122,8 @@ SIGNATURES = {
     "oc_matvec_fused_test_reset": (None, []),
     "oc_matvec_fused_test_stats": (OcMatvecFusedTestStats, []),
     "oxh_set_decline_handler": (None, [V, V]),
+    "oxh_set_cpu_fallback": (None, [V]),
+    "oxh_cpu_fallback_calls": (Z, []),
 }
 
 _LIB = None

@@ -68,35 +68,191 @@ size_t oc_matvec_batch_scratch_bytes(size_t max_cols)
 
 /* ─── weight registry: host range -> device copy ──────────────────────── */
 
+/* Two kinds of entry.
+ *   explicit  made by oxh_weight_register (and oxh_gguf_register_all): the caller promises the bytes do
+ *             not change while registered; any pointer inside the range resolves (expert slices).
+ *   automatic made on first sight of an unregistered matrix.  The reference reads the caller's host bytes
+ *             on every call (oxidize-c/include/oxidize/matvec.h:45-52), so an address alone proves
+ *             nothing: the heap hands the same address to the next model.  An automatic entry matches
+ *             only the exact (pointer, byte count) it was made for, and every hit re-checks a
+ *             fingerprint of the host bytes; on a mismatch the device copy is refreshed in place.  A new
+ *             range that overlaps automatic entries replaces them.  Least recently used entries go once
+ *             the cached bytes pass a budget.
+ * OXH_WEIGHT_CACHE = sample (default: fingerprint of the first and last 4 KiB plus 128 strided 64-byte
+ * samples and the length), full (hash of every byte on every call), off (upload on every call). */
+typedef struct {
+    size_t off, rows, cols;     /* which sub-matrix of the range, and its shape */
+    uint32_t form;              /* OXH_PREP_* */
+    uint8_t *d;
+    size_t bytes;
+} Prepared;
+
 typedef struct {
     const uint8_t *h;
     size_t bytes;
     uint8_t *d;
+    bool automatic;
+    uint64_t print;             /* automatic entries: fingerprint of the host bytes at upload */
+    uint64_t tick;              /* last use */
+    Prepared *prep;             /* device-side rewrites of (parts of) this range, made on demand */
+    size_t n_prep;
 } Resident;
 
 static pthread_mutex_t g_lock = PTHREAD_MUTEX_INITIALIZER;
-/* Held for the whole of a matvec call, and by the calls that free device weights (taken before g_lock):
+/* Held for the whole of a matvec call, and by the calls that add or free device weights (taken before g_lock):
  * the staging buffers and the library's stream are shared by every call, so concurrent callers are
  * serialised (the reference's worker pool is one process-global resource too, include/oxidize/parallel.h:13-19). */
 static pthread_mutex_t g_call = PTHREAD_MUTEX_INITIALIZER;
 static Resident *g_res = NULL;
 static size_t g_nres = 0, g_cap = 0;
+static uint64_t g_tick = 0;
+/* g_tick when the running call began: entries used since then back a launch of this call and must
+ * stay where they are until it has finished */
+static uint64_t g_call_tick = 0;
+static size_t g_auto_bytes = 0;
 
-static Resident *find_range(const uint8_t *p, size_t bytes)
+enum { CACHE_SAMPLE = 0, CACHE_FULL = 1, CACHE_OFF = 2 };
+
+static int cache_mode(void)
+{
+    static int mode = -1;
+    if (mode < 0) {
+        const char *e = getenv("OXH_WEIGHT_CACHE");
+        mode = CACHE_SAMPLE;
+        if (e && !strcmp(e, "full")) mode = CACHE_FULL;
+        else if (e && !strcmp(e, "off")) mode = CACHE_OFF;
+    }
+    return mode;
+}
+
+/* Budget for automatic entries, OXH_WEIGHT_CACHE_MB (default 65536: a quarter of the device). */
+static size_t cache_budget(void)
+{
+    static size_t budget = 0;
+    if (!budget) {
+        const char *e = getenv("OXH_WEIGHT_CACHE_MB");
+        unsigned long long mb = e && *e ? strtoull(e, NULL, 10) : 0ull;
+        if (mb == 0ull || mb > (1ull << 24)) mb = 65536ull;
+        budget = (size_t)mb << 20;
+    }
+    return budget;
+}
+
+static uint64_t mix64(uint64_t h, uint64_t v)
+{
+    h ^= v;
+    h *= 0x9E3779B97F4A7C15ull;
+    return h ^ (h >> 29);
+}
+
+static uint64_t hash_bytes(uint64_t h, const uint8_t *p, size_t n)
+{
+    size_t i = 0;
+    for (; i + 8 <= n; i += 8) {
+        uint64_t v;
+        memcpy(&v, p + i, 8);
+        h = mix64(h, v);
+    }
+    if (i < n) {
+        uint64_t v = 0;
+        memcpy(&v, p + i, n - i);
+        h = mix64(h, v);
+    }
+    return h;
+}
+
+static uint64_t host_print(const uint8_t *p, size_t bytes)
+{
+    uint64_t h = mix64(0x6F78685F77746673ull, (uint64_t)bytes);
+    if (cache_mode() == CACHE_FULL || bytes <= 16384u) return hash_bytes(h, p, bytes);
+    h = hash_bytes(h, p, 4096u);
+    h = hash_bytes(h, p + bytes - 4096u, 4096u);
+    const size_t span = bytes - 8192u - 64u, n = 128u;
+    for (size_t i = 0; i < n; i++)
+        h = hash_bytes(h, p + 4096u + (size_t)(((unsigned __int128)span * i) / (n - 1u)), 64u);
+    return h;
+}
+
+static void drop_prepared(Resident *r)
+{
+    for (size_t i = 0; i < r->n_prep; i++) (void)oxh_free(r->prep[i].d);
+    free(r->prep);
+    r->prep = NULL;
+    r->n_prep = 0;
+}
+
+/* caller holds g_lock and has synchronised the library's stream */
+static int drop_entry(size_t i)
+{
+    Resident *r = &g_res[i];
+    drop_prepared(r);
+    if (r->automatic) g_auto_bytes -= r->bytes;
+    const int rc = oxh_free(r->d);
+    g_res[i] = g_res[g_nres - 1];
+    g_nres--;
+    return rc;
+}
+
+static bool overlaps(const Resident *r, const uint8_t *p, size_t bytes)
+{
+    return p < r->h + r->bytes && r->h < p + bytes;
+}
+
+/* explicit entries: p .. p+bytes lies inside the range (the end of one tensor is the start of the next
+ * in a mapped model file, so p itself must be inside) */
+static Resident *find_explicit(const uint8_t *p, size_t bytes)
 {
     for (size_t i = 0; i < g_nres; i++) {
-        const Resident *r = &g_res[i];
-        /* p must lie inside the range: the end of one tensor is the start of the
-         * next in a mapped model file */
-        if (p >= r->h && (size_t)(p - r->h) < r->bytes &&
+        Resident *r = &g_res[i];
+        if (!r->automatic && p >= r->h && (size_t)(p - r->h) < r->bytes &&
             bytes <= r->bytes - (size_t)(p - r->h))
-            return &g_res[i];
+            return r;
     }
     return NULL;
 }
 
-static int register_locked(const uint8_t *h, size_t bytes, Resident **out)
+static Resident *find_automatic(const uint8_t *p, size_t bytes)
 {
+    for (size_t i = 0; i < g_nres; i++)
+        if (g_res[i].automatic && g_res[i].h == p && g_res[i].bytes == bytes) return &g_res[i];
+    return NULL;
+}
+
+static int upload(uint8_t *d, const uint8_t *h, size_t bytes)
+{
+    int rc = oxh_memcpy_h2d(d, h, bytes, NULL);
+    if (!rc) rc = oxh_stream_sync(NULL);
+    return rc;
+}
+
+static int register_locked(const uint8_t *h, size_t bytes, bool automatic, Resident **out)
+{
+    /* whatever automatic entry shares bytes with the new range describes memory that now holds
+     * something else */
+    bool synced = false;
+    for (size_t i = 0; i < g_nres;) {
+        if (g_res[i].automatic && overlaps(&g_res[i], h, bytes)) {
+            if (g_res[i].tick > g_call_tick) {
+                oxh_set_error("invalid argument: %s%s", "two matrices of one call overlap in host memory", NULL);
+                return OXH_ERR_ARG;
+            }
+            if (!synced) { int rc = oxh_stream_sync(NULL); if (rc) return rc; synced = true; }
+            (void)drop_entry(i);
+        } else {
+            i++;
+        }
+    }
+    if (automatic) {
+        while (g_auto_bytes && g_auto_bytes + bytes > cache_budget()) {
+            size_t lru = g_nres;
+            for (size_t i = 0; i < g_nres; i++)
+                if (g_res[i].automatic && g_res[i].tick <= g_call_tick &&
+                    (lru == g_nres || g_res[i].tick < g_res[lru].tick)) lru = i;
+            if (lru == g_nres) break;
+            if (!synced) { int rc = oxh_stream_sync(NULL); if (rc) return rc; synced = true; }
+            (void)drop_entry(lru);
+        }
+    }
     if (g_nres == g_cap) {
         const size_t nc = g_cap ? g_cap * 2 : 64;
         Resident *n = (Resident *)realloc(g_res, nc * sizeof *n);
@@ -110,17 +266,21 @@ static int register_locked(const uint8_t *h, size_t bytes, Resident **out)
     void *d = NULL;
     int rc = oxh_malloc(&d, bytes);
     if (rc) return rc;
-    rc = oxh_memcpy_h2d(d, h, bytes, NULL);
-    if (!rc) rc = oxh_stream_sync(NULL);
-    if (rc) {
+    const uint64_t print = automatic ? host_print(h, bytes) : 0u;
+    if ((rc = upload((uint8_t *)d, h, bytes))) {
         oxh_free(d);
         return rc;
     }
-    g_res[g_nres].h = h;
-    g_res[g_nres].bytes = bytes;
-    g_res[g_nres].d = (uint8_t *)d;
-    if (out) *out = &g_res[g_nres];
-    g_nres++;
+    Resident *r = &g_res[g_nres++];
+    memset(r, 0, sizeof *r);
+    r->h = h;
+    r->bytes = bytes;
+    r->d = (uint8_t *)d;
+    r->automatic = automatic;
+    r->print = print;
+    r->tick = ++g_tick;
+    if (automatic) g_auto_bytes += bytes;
+    if (out) *out = r;
     return OXH_OK;
 }
 
@@ -130,26 +290,33 @@ int oxh_weight_register(const void *h_data, size_t bytes)
         oxh_set_error("invalid argument: %s%s", "oxh_weight_register: empty range", NULL);
         return OXH_ERR_ARG;
     }
+    int rc = oxh_init(0);
+    if (rc) return rc;
+    pthread_mutex_lock(&g_call);
+    g_call_tick = g_tick;
     pthread_mutex_lock(&g_lock);
-    int rc = OXH_OK;
-    if (!find_range((const uint8_t *)h_data, bytes))
-        rc = register_locked((const uint8_t *)h_data, bytes, NULL);
+    if (!find_explicit((const uint8_t *)h_data, bytes))
+        rc = register_locked((const uint8_t *)h_data, bytes, false, NULL);
     pthread_mutex_unlock(&g_lock);
+    pthread_mutex_unlock(&g_call);
     return rc;
 }
 
 int oxh_weight_unregister(const void *h_data)
 {
     int rc = OXH_OK;
+    const uint8_t *p = (const uint8_t *)h_data;
     pthread_mutex_lock(&g_call);
     pthread_mutex_lock(&g_lock);
-    for (size_t i = 0; i < g_nres; i++) {
-        if (g_res[i].h == (const uint8_t *)h_data) {
-            rc = oxh_stream_sync(NULL);
-            if (!rc) rc = oxh_free(g_res[i].d);
-            g_res[i] = g_res[g_nres - 1];
-            g_nres--;
-            break;
+    bool synced = false;
+    for (size_t i = 0; i < g_nres;) {
+        const Resident *r = &g_res[i];
+        if (p >= r->h && (size_t)(p - r->h) < r->bytes) {
+            if (!synced) { rc = oxh_stream_sync(NULL); synced = true; }
+            const int r2 = drop_entry(i);
+            if (!rc) rc = r2;
+        } else {
+            i++;
         }
     }
     pthread_mutex_unlock(&g_lock);
@@ -157,16 +324,22 @@ int oxh_weight_unregister(const void *h_data)
     return rc;
 }
 
+static int clear_locked(void)
+{
+    int rc = g_nres ? oxh_stream_sync(NULL) : OXH_OK;
+    while (g_nres) {
+        const int r = drop_entry(g_nres - 1);
+        if (!rc) rc = r;
+    }
+    g_auto_bytes = 0;
+    return rc;
+}
+
 int oxh_weight_clear(void)
 {
     pthread_mutex_lock(&g_call);
     pthread_mutex_lock(&g_lock);
-    int rc = g_nres ? oxh_stream_sync(NULL) : OXH_OK;
-    for (size_t i = 0; i < g_nres; i++) {
-        const int r = oxh_free(g_res[i].d);
-        if (!rc) rc = r;
-    }
-    g_nres = 0;
+    const int rc = clear_locked();
     pthread_mutex_unlock(&g_lock);
     pthread_mutex_unlock(&g_call);
     return rc;
@@ -174,24 +347,114 @@ int oxh_weight_clear(void)
 
 const void *oxh_weight_device_ptr(const void *h_data)
 {
+    const uint8_t *p = (const uint8_t *)h_data;
     pthread_mutex_lock(&g_lock);
-    const Resident *r = find_range((const uint8_t *)h_data, 0);
-    const void *d = r ? r->d + ((const uint8_t *)h_data - r->h) : NULL;
+    const Resident *r = find_explicit(p, 0);
+    if (!r)
+        for (size_t i = 0; i < g_nres && !r; i++)
+            if (g_res[i].automatic && p >= g_res[i].h && (size_t)(p - g_res[i].h) < g_res[i].bytes) r = &g_res[i];
+    const void *d = r ? r->d + (p - r->h) : NULL;
     pthread_mutex_unlock(&g_lock);
     return d;
 }
 
-/* Device address of `bytes` of weights starting at host pointer p, uploading
- * them first if no registered range covers them. */
-static int resident_ptr(const uint8_t *p, size_t bytes, const uint8_t **d)
+int oxh_weight_stats(size_t *n_explicit, size_t *n_automatic, size_t *automatic_bytes, size_t *refreshes);
+static size_t g_refreshes = 0;
+
+int oxh_weight_stats(size_t *n_explicit, size_t *n_automatic, size_t *automatic_bytes, size_t *refreshes)
 {
     pthread_mutex_lock(&g_lock);
-    Resident *r = find_range(p, bytes);
+    size_t ne = 0, na = 0;
+    for (size_t i = 0; i < g_nres; i++) {
+        if (g_res[i].automatic) na++;
+        else ne++;
+    }
+    if (n_explicit) *n_explicit = ne;
+    if (n_automatic) *n_automatic = na;
+    if (automatic_bytes) *automatic_bytes = g_auto_bytes;
+    if (refreshes) *refreshes = g_refreshes;
+    pthread_mutex_unlock(&g_lock);
+    return OXH_OK;
+}
+
+/* Device address of `bytes` of weights starting at host pointer p.  Registered ranges resolve without
+ * looking at the host bytes; anything else is uploaded on first sight and re-validated on every later
+ * call (see the registry's header; with OXH_WEIGHT_CACHE=off every hit counts as changed and is uploaded
+ * again).  The caller holds g_call.  `entry`, when not NULL, receives the registry entry. */
+static int resident_ptr(const uint8_t *p, size_t bytes, const uint8_t **d, Resident **entry)
+{
+    pthread_mutex_lock(&g_lock);
     int rc = OXH_OK;
-    if (!r) rc = register_locked(p, bytes, &r);
-    if (!rc) *d = r->d + (p - r->h);
+    if (entry) *entry = NULL;
+    Resident *r = find_explicit(p, bytes);
+    if (!r) {
+        r = find_automatic(p, bytes);
+        if (r && r->tick <= g_call_tick) {         /* validated once per call is enough */
+            const uint64_t now = cache_mode() == CACHE_OFF ? ~r->print : host_print(p, bytes);
+            if (now != r->print) {
+                /* same address and size, other contents: the caller reused the memory */
+                drop_prepared(r);
+                rc = oxh_stream_sync(NULL);
+                if (!rc) rc = upload(r->d, p, bytes);
+                r->print = cache_mode() == CACHE_OFF ? 0u : now;
+                g_refreshes++;
+            }
+        } else if (!r) {
+            rc = register_locked(p, bytes, true, &r);
+        }
+    }
+    if (!rc) {
+        r->tick = ++g_tick;
+        *d = r->d + (p - r->h);
+        if (entry) *entry = r;
+    }
     pthread_mutex_unlock(&g_lock);
     return rc;
+}
+
+static bool mul_ok(size_t a, size_t b, size_t *out);
+static int bad_arg(const char *what);
+
+/* Forms a resident matrix can be rewritten into, once, on the device. */
+#define OXH_PREP_Q3K_AS_Q6K 1u      /* oxh_q3_k_as_q6_k */
+#define OXH_PREP_Q2K_WIDE   2u      /* oxh_q2_k_widen   */
+
+/* The rewritten form of the rows x cols matrix at host pointer p inside registry entry r, made on first
+ * use and kept with the entry (the reference prepares its batch rows once per matrix as well,
+ * oxidize-c/src/compute/oxk.c:316-366, :734-745).  It goes when the entry goes or is refreshed.  The
+ * caller holds g_call. */
+static int prepared_ptr(Resident *r, const uint8_t *p, size_t rows, size_t cols, uint32_t form,
+                        const uint8_t **d)
+{
+    const size_t off = (size_t)(p - r->h);
+    for (size_t i = 0; i < r->n_prep; i++) {
+        const Prepared *q = &r->prep[i];
+        if (q->off == off && q->rows == rows && q->cols == cols && q->form == form) {
+            *d = q->d;
+            return OXH_OK;
+        }
+    }
+    size_t bytes;
+    if (!mul_ok(rows, cols / OXH_QK_K * OXH_Q6_K_BYTES, &bytes)) return bad_arg("prepared form: size overflow");
+    Prepared *np = (Prepared *)realloc(r->prep, (r->n_prep + 1) * sizeof *np);
+    if (!np) {
+        oxh_set_error("out of host memory growing the weight registry%s%s", NULL, NULL);
+        return OXH_ERR_NOMEM;
+    }
+    r->prep = np;
+    void *nd = NULL;
+    int rc = oxh_malloc(&nd, bytes);
+    if (rc) return rc;
+    if (form == OXH_PREP_Q2K_WIDE) rc = oxh_q2_k_widen(r->d + off, rows, cols, nd, NULL);
+    else                           rc = oxh_q3_k_as_q6_k(r->d + off, rows, cols, nd, NULL);
+    if (rc) {
+        (void)oxh_free(nd);
+        return rc;
+    }
+    Prepared *q = &r->prep[r->n_prep++];
+    q->off = off; q->rows = rows; q->cols = cols; q->form = form; q->d = (uint8_t *)nd; q->bytes = bytes;
+    *d = q->d;
+    return OXH_OK;
 }
 
 /* ─── device staging buffers (inputs, activations, outputs) ───────────── */
@@ -201,7 +464,7 @@ typedef struct {
     size_t bytes;
 } DevBuf;
 
-static DevBuf g_dx, g_dact, g_dout, g_dprep;
+static DevBuf g_dx, g_dact, g_dout;
 
 /* Page-locked host staging for the decode-sized entry points: the caller's
  * vectors are ordinary pageable memory, and a copy between pageable memory and
@@ -231,6 +494,28 @@ static int reserve_host(HostBuf *b, size_t bytes)
     if (rc) return rc;
     b->bytes = want;
     return OXH_OK;
+}
+
+/* oxh_shutdown: forget every device and pinned buffer made under the state that is going away. */
+void oxh_internal_host_reset(void)
+{
+    pthread_mutex_lock(&g_call);
+    pthread_mutex_lock(&g_lock);
+    (void)clear_locked();
+    pthread_mutex_unlock(&g_lock);
+    DevBuf *dv[] = { &g_dx, &g_dact, &g_dout };
+    for (size_t i = 0; i < sizeof dv / sizeof dv[0]; i++) {
+        if (dv[i]->p) (void)oxh_free(dv[i]->p);
+        dv[i]->p = NULL;
+        dv[i]->bytes = 0;
+    }
+    HostBuf *hv[] = { &g_hin, &g_hout };
+    for (size_t i = 0; i < sizeof hv / sizeof hv[0]; i++) {
+        if (hv[i]->p) (void)oxh_host_free(hv[i]->p);
+        hv[i]->p = NULL;
+        hv[i]->bytes = 0;
+    }
+    pthread_mutex_unlock(&g_call);
 }
 
 static size_t align16(size_t n) { return (n + 15u) & ~(size_t)15u; }
@@ -310,7 +595,7 @@ static int mv_one(uint32_t qtype, const uint8_t *data, size_t rows,
     int rc = oxh_init(0);
     if (rc) return rc;
     const uint8_t *d_w;
-    if ((rc = resident_ptr(data, wbytes, &d_w))) return rc;
+    if ((rc = resident_ptr(data, wbytes, &d_w, NULL))) return rc;
     /* device and pinned-host images: [output rows][quantised activation] */
     const size_t act_off = align16(obytes);
     if ((rc = reserve(&g_dx, cols * sizeof(float)))) return rc;
@@ -376,7 +661,7 @@ static int grouped(uint32_t qtype, const uint8_t *const *datas,
             const uint8_t *d_w = NULL;
             if (rows[k]) {
                 if (!datas[k] || !outs[k]) return bad_arg("grouped: NULL matrix pointer");
-                if ((rc = resident_ptr(datas[k], wbytes, &d_w))) return rc;
+                if ((rc = resident_ptr(datas[k], wbytes, &d_w, NULL))) return rc;
             }
             segs[i].d_w = d_w;
             segs[i].d_out = (float *)g_dout.p + done_rows;
@@ -494,77 +779,78 @@ static int mv_batch(uint32_t qtype, const uint8_t *data, size_t rows,
         !mul_ok(n_vec - 1, out_stride, &out_span) || !mul_ok(n_vec, abytes, &act_total) ||
         in_span > SIZE_MAX / 4 - cols || out_span > SIZE_MAX / 4 - rows)
         return bad_arg("oxh_matvec_quantized_batch: size overflow");
-    in_span += cols;
-    out_span += rows;
 
     int rc = oxh_init(0);
     if (rc) return rc;
     const uint8_t *d_w;
-    if ((rc = resident_ptr(data, wbytes, &d_w))) return rc;
-    /* Inputs travel with their host stride; outputs come back packed
-     * [n_vec][rows] and are scattered on the host so that nothing between
-     * `rows` and `out_stride` is written (tests/test_matvec_batch.c:226-230). */
-    size_t packed_out;
-    if (!mul_ok(n_vec, rows * sizeof(float), &packed_out)) return bad_arg("batch: size overflow");
-    if ((rc = reserve(&g_dx, in_span * sizeof(float)))) return rc;
+    Resident *entry;
+    if ((rc = resident_ptr(data, wbytes, &d_w, &entry))) return rc;
+    /* Inputs arrive packed [n_vec][cols] on the device and outputs come back packed [n_vec][rows]: one
+     * copy each way, two-dimensional when the host strides are padded, so that nothing between `rows`
+     * and `out_stride` is written (tests/test_matvec_batch.c:226-230). */
+    size_t packed_in, packed_out;
+    if (!mul_ok(n_vec, cols * sizeof(float), &packed_in) || !mul_ok(n_vec, rows * sizeof(float), &packed_out))
+        return bad_arg("batch: size overflow");
+    if ((rc = reserve(&g_dx, packed_in))) return rc;
     if ((rc = reserve(&g_dact, act_total))) return rc;
     if ((rc = reserve(&g_dout, packed_out))) return rc;
-    if (in_stride == cols) {
-        if ((rc = oxh_memcpy_h2d(g_dx.p, inputs, in_span * sizeof(float), NULL))) return rc;
-    } else {
-        for (size_t v = 0; v < n_vec; v++)
-            if ((rc = oxh_memcpy_h2d((float *)g_dx.p + v * in_stride, inputs + v * in_stride,
-                                     cols * sizeof(float), NULL)))
-                return rc;
-    }
+    if (in_stride == cols)
+        rc = oxh_memcpy_h2d(g_dx.p, inputs, packed_in, NULL);
+    else
+        rc = oxh_memcpy2d_h2d(g_dx.p, cols * sizeof(float), inputs, in_stride * sizeof(float),
+                              cols * sizeof(float), n_vec, NULL);
+    if (rc) return rc;
+    const float *d_x = (const float *)g_dx.p;
     /* More vectors than the GEMV kernel keeps in flight: Q4_K, Q5_K and Q6_K go to the
      * int8-MFMA kernel behind a stand-alone quantiser launch; everything else
-     * walks the batch in GEMV-sized slices with the quantisation fused in
-     * (every output is the same dot either way). */
+     * walks the batch in GEMV-sized slices (every output is the same dot either way). */
     if (n_vec > 8 && (qtype == OXH_Q4_K_S || qtype == OXH_Q4_K_M || qtype == OXH_Q5_K_S ||
                       qtype == OXH_Q5_K_M || qtype == OXH_Q6_K)) {
-        if ((rc = quantize(kind, (const float *)g_dx.p, in_stride, n_vec, cols, g_dact.p))) return rc;
+        if ((rc = quantize(kind, d_x, cols, n_vec, cols, g_dact.p))) return rc;
         if ((rc = oxh_mmq(qtype, d_w, rows, cols, g_dact.p, n_vec, (float *)g_dout.p, rows, NULL)))
             return rc;
     } else if (n_vec > 8 && (qtype == OXH_Q2_K || qtype == OXH_Q3_K_S || qtype == OXH_Q3_K_M ||
                              qtype == OXH_Q3_K_L)) {
         /* No MFMA kernel reads these blocks as they are.  Q3_K is exactly a Q6_K matrix in other bytes
-         * and Q2_K widens to 210-byte blocks with scale * code in the 6-bit fields: rewrite the matrix
-         * for this call, as the reference prepares its batch rows (oxk.c:734-745), and use that kernel */
-        size_t prep_bytes;
-        if (!mul_ok(rows, cols / OXH_QK_K * OXH_Q6_K_BYTES, &prep_bytes)) return bad_arg("batch: size overflow");
-        if ((rc = reserve(&g_dprep, prep_bytes))) return rc;
-        if (qtype == OXH_Q2_K) rc = oxh_q2_k_widen(d_w, rows, cols, g_dprep.p, NULL);
-        else                   rc = oxh_q3_k_as_q6_k(d_w, rows, cols, g_dprep.p, NULL);
-        if (rc) return rc;
-        if ((rc = quantize(kind, (const float *)g_dx.p, in_stride, n_vec, cols, g_dact.p))) return rc;
-        if ((rc = oxh_mmq(qtype == OXH_Q2_K ? OXH_Q2_K_WIDE : OXH_Q6_K, g_dprep.p, rows, cols, g_dact.p, n_vec,
+         * and Q2_K widens to 210-byte blocks with scale * code in the 6-bit fields: the rewritten matrix
+         * is made on the first batch over these weights and stays with their registry entry, as the
+         * reference prepares its batch rows (oxk.c:734-745) */
+        const uint8_t *d_prep;
+        if ((rc = prepared_ptr(entry, data, rows, cols,
+                               qtype == OXH_Q2_K ? OXH_PREP_Q2K_WIDE : OXH_PREP_Q3K_AS_Q6K, &d_prep)))
+            return rc;
+        if ((rc = quantize(kind, d_x, cols, n_vec, cols, g_dact.p))) return rc;
+        if ((rc = oxh_mmq(qtype == OXH_Q2_K ? OXH_Q2_K_WIDE : OXH_Q6_K, d_prep, rows, cols, g_dact.p, n_vec,
                           (float *)g_dout.p, rows, NULL)))
             return rc;
     } else {
-        size_t step = oxh_gemv_max_nvec_buffered(qtype, cols);
+        const size_t step = oxh_gemv_max_nvec_buffered(qtype, cols);
         if (step == 0) {
             oxh_set_error("batch: cols too wide for one workgroup%s%s", NULL, NULL);
             return OXH_ERR_TOO_WIDE;
         }
-        for (size_t v0 = 0; v0 < n_vec; v0 += step) {
-            const size_t m = n_vec - v0 < step ? n_vec - v0 : step;
-            OxhSegment seg = { d_w, (float *)g_dout.p + v0 * rows, rows, v0, 0, NULL };
-            /* with room for the quantised activations a slice of several vectors may run on
-             * the matrix cores (same results; the library decides) */
-            if ((rc = oxh_gemv_segments_f32(qtype, &seg, 1, cols, (const float *)g_dx.p, in_stride,
-                                            g_dact.p, m, rows, NULL)))
+        if (n_vec <= step) {
+            /* one launch with the quantisation fused in; with room for the quantised activations a
+             * launch of several vectors may run on the matrix cores (same results; the library decides) */
+            OxhSegment seg = { d_w, (float *)g_dout.p, rows, 0, 0, NULL };
+            if ((rc = oxh_gemv_segments_f32(qtype, &seg, 1, cols, d_x, cols, g_dact.p, n_vec, rows, NULL)))
                 return rc;
+        } else {
+            /* every activation is quantised once, then the slices run over the stored bytes */
+            if ((rc = quantize(kind, d_x, cols, n_vec, cols, g_dact.p))) return rc;
+            for (size_t v0 = 0; v0 < n_vec; v0 += step) {
+                const size_t m = n_vec - v0 < step ? n_vec - v0 : step;
+                OxhSegment seg = { d_w, (float *)g_dout.p + v0 * rows, rows, v0, 0, NULL };
+                if ((rc = oxh_gemv_segments(qtype, &seg, 1, cols, g_dact.p, m, rows, NULL))) return rc;
+            }
         }
     }
-    if (out_stride == rows) {
-        if ((rc = oxh_memcpy_d2h(outputs, g_dout.p, packed_out, NULL))) return rc;
-    } else {
-        for (size_t v = 0; v < n_vec; v++)
-            if ((rc = oxh_memcpy_d2h(outputs + v * out_stride, (float *)g_dout.p + v * rows,
-                                     rows * sizeof(float), NULL)))
-                return rc;
-    }
+    if (out_stride == rows)
+        rc = oxh_memcpy_d2h(outputs, g_dout.p, packed_out, NULL);
+    else
+        rc = oxh_memcpy2d_d2h(outputs, out_stride * sizeof(float), g_dout.p, rows * sizeof(float),
+                              rows * sizeof(float), n_vec, NULL);
+    if (rc) return rc;
     return oxh_stream_sync(NULL);
 }
 
@@ -574,6 +860,7 @@ int oxh_matvec_quantized(uint32_t qtype, const uint8_t *data, size_t rows, size_
                          const float *input, float *output, float *temp)
 {
     pthread_mutex_lock(&g_call);
+    g_call_tick = g_tick;
     const int rc = mv_one(qtype, data, rows, cols, row_bytes, input, output, temp);
     pthread_mutex_unlock(&g_call);
     return rc;
@@ -584,6 +871,7 @@ int oxh_matvec_quantized_fused(const uint32_t *qtypes, const uint8_t *const *dat
                                float *const *outs, float *temp)
 {
     pthread_mutex_lock(&g_call);
+    g_call_tick = g_tick;
     const int rc = mv_fused(qtypes, datas, rows, cols, row_bytes, n_outs, input, outs, temp);
     pthread_mutex_unlock(&g_call);
     return rc;
@@ -594,6 +882,7 @@ int oxh_matvec_quantized_multi_input(const uint32_t *qtypes, const uint8_t *cons
                                      const float *const *inputs, float *const *outs, float *temp)
 {
     pthread_mutex_lock(&g_call);
+    g_call_tick = g_tick;
     const int rc = mv_multi_input(qtypes, datas, rows, cols, row_bytes, n_outs, inputs, outs, temp);
     pthread_mutex_unlock(&g_call);
     return rc;
@@ -604,6 +893,7 @@ int oxh_matvec_quantized_batch(uint32_t qtype, const uint8_t *data, size_t rows,
                                size_t n_vec, float *temp, uint8_t *act_scratch, size_t act_bytes)
 {
     pthread_mutex_lock(&g_call);
+    g_call_tick = g_tick;
     const int rc = mv_batch(qtype, data, rows, cols, row_bytes, inputs, in_stride, outputs, out_stride, n_vec,
                             temp, act_scratch, act_bytes);
     pthread_mutex_unlock(&g_call);
@@ -612,8 +902,37 @@ int oxh_matvec_quantized_batch(uint32_t qtype, const uint8_t *data, size_t rows,
 
 /* ─── the reference's own symbols ─────────────────────────────────────── */
 
+/* They return void, so a call this library declines (or that fails) has to be finished by somebody else.
+ * In this order:
+ *   1. the CPU functions installed with oxh_set_cpu_fallback() get the call with its original arguments;
+ *   2. else the weak symbols oc_ref_matvec_quantized* do, when the program links them (the reference's
+ *      own functions renamed, e.g. objcopy --redefine-sym oc_matvec_quantized=oc_ref_matvec_quantized);
+ *   3. else the handler installed with oxh_set_decline_handler() is told;
+ *   4. else the process prints the error and aborts — it never silently computes something else. */
+extern void oc_ref_matvec_quantized(uint32_t, const uint8_t *, size_t, size_t, size_t, const float *, float *,
+                                    float *) __attribute__((weak));
+extern void oc_ref_matvec_quantized_fused(const uint32_t *, const uint8_t *const *, const size_t *, size_t,
+                                          const size_t *, size_t, const float *, float *const *, float *)
+    __attribute__((weak));
+extern void oc_ref_matvec_quantized_multi_input(const uint32_t *, const uint8_t *const *, const size_t *, size_t,
+                                                const size_t *, size_t, const float *const *, float *const *,
+                                                float *) __attribute__((weak));
+extern void oc_ref_matvec_quantized_batch(uint32_t, const uint8_t *, size_t, size_t, size_t, const float *, size_t,
+                                          float *, size_t, size_t, float *, uint8_t *, size_t)
+    __attribute__((weak));
+
+static OxhCpuFallback g_fallback;
 static OxhDeclineHandler g_handler = NULL;
 static void *g_handler_user = NULL;
+static _Atomic size_t g_forwarded = 0;
+
+void oxh_set_cpu_fallback(const OxhCpuFallback *fb)
+{
+    if (fb) g_fallback = *fb;
+    else memset(&g_fallback, 0, sizeof g_fallback);
+}
+
+size_t oxh_cpu_fallback_calls(void) { return atomic_load(&g_forwarded); }
 
 void oxh_set_decline_handler(OxhDeclineHandler fn, void *user)
 {
@@ -627,8 +946,9 @@ static void not_ok(int which, int status)
         g_handler(which, status, g_handler_user);
         return;
     }
-    fprintf(stderr, "liboxhip: oc_matvec entry %d failed with status %d: %s\n", which, status,
-            oxh_last_error());
+    fprintf(stderr, "liboxhip: oc_matvec entry %d failed with status %d: %s\n"
+            "liboxhip: no CPU fallback is installed (oxh_set_cpu_fallback, or link oc_ref_matvec_quantized*)\n",
+            which, status, oxh_last_error());
     abort();
 }
 
@@ -636,7 +956,12 @@ void oc_matvec_quantized(uint32_t qtype, const uint8_t *data, size_t rows, size_
                          size_t row_bytes, const float *input, float *output, float *temp)
 {
     const int rc = oxh_matvec_quantized(qtype, data, rows, cols, row_bytes, input, output, temp);
-    if (rc) not_ok(0, rc);
+    if (!rc) return;
+    void (*fb)(uint32_t, const uint8_t *, size_t, size_t, size_t, const float *, float *, float *) =
+        g_fallback.matvec_quantized ? g_fallback.matvec_quantized : oc_ref_matvec_quantized;
+    if (!fb) { not_ok(0, rc); return; }
+    atomic_fetch_add(&g_forwarded, 1);
+    fb(qtype, data, rows, cols, row_bytes, input, output, temp);
 }
 
 void oc_matvec_quantized_fused(const uint32_t *qtypes, const uint8_t *const *datas,
@@ -646,7 +971,13 @@ void oc_matvec_quantized_fused(const uint32_t *qtypes, const uint8_t *const *dat
 {
     const int rc = oxh_matvec_quantized_fused(qtypes, datas, rows, cols, row_bytes, n_outs,
                                               input, outs, temp);
-    if (rc) not_ok(1, rc);
+    if (!rc) return;
+    void (*fb)(const uint32_t *, const uint8_t *const *, const size_t *, size_t, const size_t *, size_t,
+               const float *, float *const *, float *) =
+        g_fallback.matvec_quantized_fused ? g_fallback.matvec_quantized_fused : oc_ref_matvec_quantized_fused;
+    if (!fb) { not_ok(1, rc); return; }
+    atomic_fetch_add(&g_forwarded, 1);
+    fb(qtypes, datas, rows, cols, row_bytes, n_outs, input, outs, temp);
 }
 
 void oc_matvec_quantized_multi_input(const uint32_t *qtypes, const uint8_t *const *datas,
@@ -657,7 +988,14 @@ void oc_matvec_quantized_multi_input(const uint32_t *qtypes, const uint8_t *cons
 {
     const int rc = oxh_matvec_quantized_multi_input(qtypes, datas, rows, cols, row_bytes,
                                                     n_outs, inputs, outs, temp);
-    if (rc) not_ok(2, rc);
+    if (!rc) return;
+    void (*fb)(const uint32_t *, const uint8_t *const *, const size_t *, size_t, const size_t *, size_t,
+               const float *const *, float *const *, float *) =
+        g_fallback.matvec_quantized_multi_input ? g_fallback.matvec_quantized_multi_input
+                                                : oc_ref_matvec_quantized_multi_input;
+    if (!fb) { not_ok(2, rc); return; }
+    atomic_fetch_add(&g_forwarded, 1);
+    fb(qtypes, datas, rows, cols, row_bytes, n_outs, inputs, outs, temp);
 }
 
 void oc_matvec_quantized_batch(uint32_t qtype, const uint8_t *data, size_t rows, size_t cols,
@@ -668,5 +1006,12 @@ void oc_matvec_quantized_batch(uint32_t qtype, const uint8_t *data, size_t rows,
     const int rc = oxh_matvec_quantized_batch(qtype, data, rows, cols, row_bytes, inputs,
                                               in_stride, outputs, out_stride, n_vec, temp,
                                               act_scratch, act_bytes);
-    if (rc) not_ok(3, rc);
+    if (!rc) return;
+    void (*fb)(uint32_t, const uint8_t *, size_t, size_t, size_t, const float *, size_t, float *, size_t, size_t,
+               float *, uint8_t *, size_t) =
+        g_fallback.matvec_quantized_batch ? g_fallback.matvec_quantized_batch : oc_ref_matvec_quantized_batch;
+    if (!fb) { not_ok(3, rc); return; }
+    atomic_fetch_add(&g_forwarded, 1);
+    fb(qtype, data, rows, cols, row_bytes, inputs, in_stride, outputs, out_stride, n_vec, temp, act_scratch,
+       act_bytes);
 }

@@ -21,6 +21,9 @@ size_t oxh_gemv_max_nvec(uint32_t qtype, size_t cols);
  * (up to 16 for Q8_0 weights, which then run on the matrix cores). */
 size_t oxh_gemv_max_nvec_buffered(uint32_t qtype, size_t cols);
 
+/* Host layer: drop the weight registry and the staging buffers (oxh_shutdown). */
+void oxh_internal_host_reset(void);
+
 #ifdef __cplusplus
 }
 #endif

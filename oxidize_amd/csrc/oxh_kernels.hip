@@ -25,6 +25,9 @@
 #include <stdlib.h>
 #include <string.h>
 
+#include <atomic>
+#include <mutex>
+
 #include "oxhip.h"
 #include "oxh_internal.h"
 
@@ -551,12 +554,15 @@ k_q2k_widen(const uint8_t *__restrict__ src, uint8_t *__restrict__ dst, uint32_t
 
 static hipError_t raise_all_lds_ceilings(void);
 
-static int g_device = -1;
+static std::atomic<int> g_device{-1};
 static hipStream_t g_stream = nullptr;
 static int g_n_cu = 0;
+static std::mutex g_init_lock;
 
 extern "C" int oxh_init(int device)
 {
+    if (g_device.load(std::memory_order_acquire) == device) return OXH_OK;
+    std::lock_guard<std::mutex> hold(g_init_lock);
     if (g_device >= 0) {
         if (device == g_device) return OXH_OK;
         return arg_fail("oxh_init: already initialised on another device");
@@ -574,17 +580,29 @@ extern "C" int oxh_init(int device)
     HIP_TRY(hipGetDeviceProperties(&prop, device));
     g_n_cu = prop.multiProcessorCount;
     HIP_TRY(hipStreamCreateWithFlags(&g_stream, hipStreamNonBlocking));
-    HIP_TRY(raise_all_lds_ceilings());
-    g_device = device;
+    const hipError_t e2 = raise_all_lds_ceilings();
+    if (e2 != hipSuccess) {
+        (void)hipStreamDestroy(g_stream);
+        g_stream = nullptr;
+        return hip_fail(e2, "hipFuncSetAttribute");
+    }
+    g_device.store(device, std::memory_order_release);
     return OXH_OK;
 }
 
+/* Everything the library made on the device goes: registered and cached weights, staging buffers, the
+ * stream.  Buffers the caller got from oxh_malloc stay the caller's. */
 extern "C" void oxh_shutdown(void)
 {
     if (g_device < 0) return;
-    if (g_stream) (void)hipStreamDestroy(g_stream);
+    oxh_internal_host_reset();
+    std::lock_guard<std::mutex> hold(g_init_lock);
+    if (g_stream) {
+        (void)hipStreamSynchronize(g_stream);
+        (void)hipStreamDestroy(g_stream);
+    }
     g_stream = nullptr;
-    g_device = -1;
+    g_device.store(-1, std::memory_order_release);
 }
 
 static int ensure_init(void)
@@ -1801,12 +1819,61 @@ extern "C" int oxh_memcpy_d2d(void *d_dst, const void *d_src, size_t bytes, void
     return OXH_OK;
 }
 
+extern "C" int oxh_memcpy2d_h2d(void *d_dst, size_t d_pitch, const void *h_src, size_t h_pitch, size_t width,
+                                size_t height, void *stream)
+{
+    int rc = ensure_init();
+    if (rc) return rc;
+    if (width == 0 || height == 0) return OXH_OK;
+    if (d_pitch < width || h_pitch < width) return arg_fail("oxh_memcpy2d_h2d: pitch < width");
+    HIP_TRY(hipMemcpy2DAsync(d_dst, d_pitch, h_src, h_pitch, width, height, hipMemcpyHostToDevice,
+                             pick_stream(stream)));
+    return OXH_OK;
+}
+
+extern "C" int oxh_memcpy2d_d2h(void *h_dst, size_t h_pitch, const void *d_src, size_t d_pitch, size_t width,
+                                size_t height, void *stream)
+{
+    int rc = ensure_init();
+    if (rc) return rc;
+    if (width == 0 || height == 0) return OXH_OK;
+    if (d_pitch < width || h_pitch < width) return arg_fail("oxh_memcpy2d_d2h: pitch < width");
+    HIP_TRY(hipMemcpy2DAsync(h_dst, h_pitch, d_src, d_pitch, width, height, hipMemcpyDeviceToHost,
+                             pick_stream(stream)));
+    return OXH_OK;
+}
+
+/* Bytes [0, bytes) of dst become `value`: byte stores up to the first 16-byte boundary and after the
+ * last, 16-byte stores between.  A kernel rather than hipMemsetAsync so that a caller may record it
+ * into a graph. */
+__global__ __launch_bounds__(256) void
+k_fill(uint8_t *__restrict__ dst, size_t bytes, uint32_t pattern)
+{
+    const size_t head = min(bytes, (size_t)((16u - ((uintptr_t)dst & 15u)) & 15u));
+    const size_t n16 = (bytes - head) / 16u;
+    const size_t tid = (size_t)blockIdx.x * blockDim.x + threadIdx.x, stride = (size_t)gridDim.x * blockDim.x;
+    u32x4 *mid = reinterpret_cast<u32x4 *>(dst + head);
+    const u32x4 v = { pattern, pattern, pattern, pattern };
+    for (size_t i = tid; i < n16; i += stride) mid[i] = v;
+    const size_t tail_at = head + n16 * 16u;
+    if (tid < head) dst[tid] = (uint8_t)pattern;
+    if (tid < bytes - tail_at) dst[tail_at + tid] = (uint8_t)pattern;
+}
+
 extern "C" int oxh_memset(void *d_dst, int value, size_t bytes, void *stream)
 {
     int rc = ensure_init();
     if (rc) return rc;
     if (bytes == 0) return OXH_OK;
-    HIP_TRY(hipMemsetAsync(d_dst, value, bytes, pick_stream(stream)));
+    if (!d_dst) return arg_fail("oxh_memset: NULL pointer");
+    const uint32_t b = (uint32_t)value & 0xFFu, pattern = b * 0x01010101u;
+    size_t blocks = (bytes / 16u + 255u) / 256u;
+    const size_t cap = (size_t)(g_n_cu > 0 ? g_n_cu : 256) * 8u;
+    if (blocks > cap) blocks = cap;
+    if (blocks == 0) blocks = 1;
+    hipLaunchKernelGGL(k_fill, dim3((uint32_t)blocks), dim3(256), 0, pick_stream(stream), (uint8_t *)d_dst, bytes,
+                       pattern);
+    HIP_TRY(hipGetLastError());
     return OXH_OK;
 }
 

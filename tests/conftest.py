@@ -20,13 +20,3 @@ def oxh():
     lib = _lib.lib()
     _lib.check(lib.oxh_init(0))
     return lib
-
-
-@pytest.fixture(autouse=True)
-def _drop_resident_weights(request):
-    """Host arrays die with each test; forget their device copies so that a
-    later array at the same address is uploaded afresh."""
-    yield
-    if request.node.get_closest_marker("gpu") is not None:
-        from oxidize_amd import _lib
-        _lib.lib().oxh_weight_clear()

@@ -121,3 +121,66 @@ def test_synthetic_generator_is_deterministic():
     assert q.min() >= -127 and q.max() <= 127
     s6 = synth.weights(16, 4, 512, seed=1).reshape(-1, 210)[:, 192:208].copy().view(np.int8)
     assert s6.min() >= -32 and s6.max() <= 31
+
+
+def test_void_symbols_hand_declined_calls_to_the_cpu_fallback():
+    """A link-time replacement must not kill the process on a shape the reference's own code handles
+    (matvec.c:833-907 falls back to its dequantise path): with a CPU fallback installed the void
+    oc_matvec_quantized* symbols forward the call with its original arguments."""
+    lib = _lib.lib()
+    o = oxlibs.oracle()
+    seen = []
+
+    ONE = ctypes.CFUNCTYPE(None, ctypes.c_uint32, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_size_t, ctypes.c_size_t,
+                           ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p)
+    BATCH = ctypes.CFUNCTYPE(None, ctypes.c_uint32, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_size_t,
+                             ctypes.c_size_t, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p, ctypes.c_size_t,
+                             ctypes.c_size_t, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t)
+
+    def cpu_one(qt, data, rows, cols, rb, x, out, temp):
+        seen.append(("one", qt, rows, cols, rb))
+        # the caller's CPU path: here the oracle's integer path over the same arguments
+        o.oxo_matvec_quantized(qt, data, rows, cols, rb, x, out, temp)
+
+    def cpu_batch(qt, data, rows, cols, rb, xs, in_stride, outs, out_stride, n_vec, temp, scratch, nscratch):
+        seen.append(("batch", qt, rows, cols, n_vec))
+
+    class Table(ctypes.Structure):
+        _fields_ = [("one", ONE), ("fused", ctypes.c_void_p), ("multi", ctypes.c_void_p), ("batch", BATCH)]
+
+    table = Table(ONE(cpu_one), None, None, BATCH(cpu_batch))
+    lib.oxh_set_cpu_fallback(ctypes.byref(table))
+    try:
+        before = lib.oxh_cpu_fallback_calls()
+        rows, cols = 4, 512
+        w = synth.weights(13, rows, cols, seed=3)
+        x = synth.normal(cols, seed=3)
+        out = np.full(rows, 9.0, np.float32)
+        temp = np.zeros(cols, np.float32)
+        lib.oc_matvec_set_fused(False)             # OC_NO_FUSED: every call is declined
+        lib.oc_matvec_quantized(13, w.ctypes.data, rows, cols, 288, x.ctypes.data, out.ctypes.data,
+                                temp.ctypes.data)
+        lib.oc_matvec_set_fused(True)
+        assert seen == [("one", 13, rows, cols, 288)]
+        want = np.zeros(rows, np.float32)
+        wtmp = np.zeros(cols, np.float32)
+        o.oxo_matvec_quantized(13, w.ctypes.data, rows, cols, 288, x.ctypes.data, want.ctypes.data,
+                               wtmp.ctypes.data)
+        assert np.array_equal(out.view(np.uint32), want.view(np.uint32))
+        # a padded row stride is declined too (matvec.c:961-985) and goes to the batch fallback
+        scratch = np.zeros(1 << 16, np.uint8)
+        lib.oc_matvec_quantized_batch(13, w.ctypes.data, rows, cols, 304, x.ctypes.data, cols, out.ctypes.data,
+                                      rows, 1, temp.ctypes.data, scratch.ctypes.data, scratch.size)
+        assert seen[-1] == ("batch", 13, rows, cols, 1)
+        assert lib.oxh_cpu_fallback_calls() == before + 2
+    finally:
+        lib.oxh_set_cpu_fallback(None)
+
+
+def test_weight_stats_and_unregister_need_no_device():
+    lib = _lib.lib()
+    n = [ctypes.c_size_t(7) for _ in range(4)]
+    assert lib.oxh_weight_stats(*[ctypes.byref(v) for v in n]) == 0
+    assert lib.oxh_init(0) != 0 or True
+    buf = np.zeros(64, np.uint8)
+    assert lib.oxh_weight_unregister(buf.ctypes.data) == 0      # nothing there: not an error

@@ -255,6 +255,9 @@ def test_expert_slices_resolve_inside_a_registered_tensor(oxh):
         assert mv.matvec_quantized(Q4K, sl, rows, cols, rb, x, out, temp) == mv.OK
         want, _ = oracle_matvec(Q4K, np.ascontiguousarray(sl), rows, cols, x)
         assert np.array_equal(bits(out), bits(want))
+    # registered ranges are the caller's promise that the bytes stay put: give it back before w is freed
+    assert oxh.oxh_weight_unregister(w.ctypes.data) == 0
+    assert oxh.oxh_weight_device_ptr(w.ctypes.data) is None
 
 
 @pytest.mark.parametrize("qtype", [Q4K, Q6K])
