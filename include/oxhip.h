@@ -276,6 +276,18 @@ int oxh_moe_workspace_bytes(const OxhMoe *m, size_t n_tok, size_t *bytes);
 int oxh_moe_ffn(const OxhMoe *m, const float *d_logits, const float *d_x, size_t x_stride,
                 size_t n_tok, float *d_out, size_t out_stride, void *d_workspace,
                 size_t workspace_bytes, void *stream);
+/* oxh_moe_ffn for callers that cannot allocate or pass a workspace (code under
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc): the
+ * workspace is a built-in device array of OXH_MOE_STATIC_WORKSPACE_BYTES per
+ * GPU, held until the process ends.  No counterpart in the reference.  The
+ * call allocates nothing and initialises nothing: oxh_init must have run.  A
+ * layer whose oxh_moe_workspace_bytes() exceeds the built-in array is refused
+ * with OXH_ERR_TOO_WIDE.  All calls on a GPU share the one array: calls that
+ * overlap in time (two streams, two threads) race; calls on one stream are
+ * ordered and safe.  Results are those of oxh_moe_ffn, bit for bit. */
+#define OXH_MOE_STATIC_WORKSPACE_BYTES (8u << 20)
+int oxh_moe_ffn_static(const OxhMoe *m, const float *d_logits, const float *d_x, size_t x_stride,
+                       size_t n_tok, float *d_out, size_t out_stride, void *stream);
 /* The routing and grouping step alone (n_expert <= 64).  ids, weights,
  * slot_pos: n_tok*top_k entries, pair (t, j) at t*top_k + j; counts,
  * offsets: per expert (offsets has n_expert + 1 entries); perm: the token of

@@ -66,6 +66,7 @@ SIGNATURES = {
     "oxh_q2_k_widen": (I, [V, Z, Z, V, V]),
     "oxh_moe_workspace_bytes": (I, [ctypes.POINTER(OxhMoe), Z, ctypes.POINTER(Z)]),
     "oxh_moe_ffn": (I, [ctypes.POINTER(OxhMoe), V, V, Z, Z, V, Z, V, Z, V]),
+    "oxh_moe_ffn_static": (I, [ctypes.POINTER(OxhMoe), V, V, Z, Z, V, Z, V]),
     "oxh_moe_route": (I, [V, Z, Z, Z, I, V, V, V, V, V, V, V]),
     "oxh_debug_moe_workspace_parts": (I, [ctypes.POINTER(OxhMoe), Z, ctypes.POINTER(Z * 12)]),
     "oxh_malloc": (I, [ctypes.POINTER(V), Z]),

@@ -553,6 +553,7 @@ k_q2k_widen(const uint8_t *__restrict__ src, uint8_t *__restrict__ dst, uint32_t
 /* ─── host side of layer 2 ────────────────────────────────────────────── */
 
 static hipError_t raise_all_lds_ceilings(void);
+static int resolve_scratch(int device);
 
 static std::atomic<int> g_device{-1};
 static hipStream_t g_stream = nullptr;
@@ -585,6 +586,13 @@ extern "C" int oxh_init(int device)
         (void)hipStreamDestroy(g_stream);
         g_stream = nullptr;
         return hip_fail(e2, "hipFuncSetAttribute");
+    }
+    /* device `device` is current: look up where its copy of the static workspace lives */
+    const int rs = resolve_scratch(device);
+    if (rs) {
+        (void)hipStreamDestroy(g_stream);
+        g_stream = nullptr;
+        return rs;
     }
     g_device.store(device, std::memory_order_release);
     return OXH_OK;
@@ -1702,20 +1710,11 @@ static int launch_experts(uint32_t qtype, const void *const *d_w, float *const *
                                       d_counts, d_offsets, stream);
 }
 
-extern "C" int oxh_moe_ffn(const OxhMoe *m, const float *d_logits, const float *d_x, size_t x_stride,
-                           size_t n_tok, float *d_out, size_t out_stride, void *d_workspace,
-                           size_t workspace_bytes, void *stream)
+/* the six launches of a layer over a workspace laid out by moe_layout(); arguments already checked */
+static int moe_ffn_run(const OxhMoe *m, const MoeLayout &l, const float *d_logits, const float *d_x, size_t x_stride,
+                       size_t n_tok, float *d_out, size_t out_stride, uint8_t *ws, void *stream)
 {
-    int rc = ensure_init();
-    if (rc) return rc;
-    MoeLayout l;
-    if ((rc = moe_layout(m, n_tok, &l))) return rc;
-    if (!d_logits || !d_x || !d_out || !d_workspace || !m->d_w_gate || !m->d_w_up || !m->d_w_down)
-        return arg_fail("oxh_moe_ffn: NULL pointer");
-    if (workspace_bytes < l.total) return arg_fail("oxh_moe_ffn: workspace too small (see oxh_moe_workspace_bytes)");
-    if (x_stride < m->hidden || out_stride < m->hidden) return arg_fail("oxh_moe_ffn: stride < hidden");
-    if ((uintptr_t)d_workspace & 255u) return arg_fail("oxh_moe_ffn: workspace must be 256-byte aligned");
-    uint8_t *ws = (uint8_t *)d_workspace;
+    int rc;
     int32_t *ids = (int32_t *)(ws + l.ids);
     float *wts = (float *)(ws + l.wts);
     uint32_t *slot_pos = (uint32_t *)(ws + l.slot_pos), *perm = (uint32_t *)(ws + l.perm);
@@ -1744,6 +1743,65 @@ extern "C" int oxh_moe_ffn(const OxhMoe *m, const float *d_logits, const float *
                        (const uint32_t *)slot_pos, (uint32_t)m->top_k, (uint32_t)m->hidden, d_out, out_stride);
     HIP_TRY(hipGetLastError());
     return OXH_OK;
+}
+
+extern "C" int oxh_moe_ffn(const OxhMoe *m, const float *d_logits, const float *d_x, size_t x_stride,
+                           size_t n_tok, float *d_out, size_t out_stride, void *d_workspace,
+                           size_t workspace_bytes, void *stream)
+{
+    int rc = ensure_init();
+    if (rc) return rc;
+    MoeLayout l;
+    if ((rc = moe_layout(m, n_tok, &l))) return rc;
+    if (!d_logits || !d_x || !d_out || !d_workspace || !m->d_w_gate || !m->d_w_up || !m->d_w_down)
+        return arg_fail("oxh_moe_ffn: NULL pointer");
+    if (workspace_bytes < l.total) return arg_fail("oxh_moe_ffn: workspace too small (see oxh_moe_workspace_bytes)");
+    if (x_stride < m->hidden || out_stride < m->hidden) return arg_fail("oxh_moe_ffn: stride < hidden");
+    if ((uintptr_t)d_workspace & 255u) return arg_fail("oxh_moe_ffn: workspace must be 256-byte aligned");
+    return moe_ffn_run(m, l, d_logits, d_x, x_stride, n_tok, d_out, out_stride, (uint8_t *)d_workspace, stream);
+}
+
+/* The workspace of oxh_moe_ffn_static: part of the library's device image, one copy per GPU, held
+ * until the process ends.  In host code `scratch` is only a handle for hipGetSymbolAddress; the
+ * device address it stands for is looked up once per device in oxh_init and kept in g_scratch. */
+static __device__ __align__(256) unsigned char scratch[OXH_MOE_STATIC_WORKSPACE_BYTES];
+#define OXH_MAX_DEVICES 64
+static uint8_t *g_scratch[OXH_MAX_DEVICES];
+
+static int resolve_scratch(int device)
+{
+    if (device < 0 || device >= OXH_MAX_DEVICES) return arg_fail("device index beyond the library's table");
+    if (g_scratch[device]) return OXH_OK;
+    void *p = nullptr;
+    HIP_TRY(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+    if (!p || ((uintptr_t)p & 255u)) return arg_fail("the static workspace has no usable device address");
+    g_scratch[device] = (uint8_t *)p;
+    return OXH_OK;
+}
+
+extern "C" int oxh_moe_ffn_static(const OxhMoe *m, const float *d_logits, const float *d_x, size_t x_stride,
+                                  size_t n_tok, float *d_out, size_t out_stride, void *stream)
+{
+    /* nothing here may allocate: no lazy initialisation either */
+    const int device = g_device.load(std::memory_order_acquire);
+    if (device < 0) return arg_fail("oxh_moe_ffn_static: call oxh_init first (this entry point allocates nothing)");
+    MoeLayout l;
+    int rc;
+    if ((rc = moe_layout(m, n_tok, &l))) return rc;
+    if (!d_logits || !d_x || !d_out || !m->d_w_gate || !m->d_w_up || !m->d_w_down)
+        return arg_fail("oxh_moe_ffn_static: NULL pointer");
+    if (x_stride < m->hidden || out_stride < m->hidden) return arg_fail("oxh_moe_ffn_static: stride < hidden");
+    if (l.total > (size_t)OXH_MOE_STATIC_WORKSPACE_BYTES) {
+        snprintf(g_err, sizeof g_err, "oxh_moe_ffn_static: this layer needs %zu bytes of workspace, the built-in "
+                 "one holds %zu; use oxh_moe_ffn with a workspace of your own", l.total,
+                 (size_t)OXH_MOE_STATIC_WORKSPACE_BYTES);
+        return OXH_ERR_TOO_WIDE;
+    }
+    uint8_t *ws = g_scratch[device];
+    if (!ws) return arg_fail("oxh_moe_ffn_static: the static workspace was not resolved at oxh_init");
+    /* every part of the workspace a launch reads has been written by an earlier launch of the same call,
+     * so nothing needs clearing between calls */
+    return moe_ffn_run(m, l, d_logits, d_x, x_stride, n_tok, d_out, out_stride, ws, stream);
 }
 
 /* ─── memory / stream / event plumbing ────────────────────────────────── */

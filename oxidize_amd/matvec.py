@@ -219,6 +219,12 @@ class MoeLayer:
                                 out_stride or self.hidden, ctypes.c_void_p(self.workspace.ptr),
                                 self.workspace.nbytes, stream))
 
+    def forward_static(self, d_logits, d_x, n_tok, d_out, x_stride=None, out_stride=None, stream=None):
+        """The same layer through oxh_moe_ffn_static: no workspace argument, nothing allocated."""
+        return lib().oxh_moe_ffn_static(ctypes.byref(self.desc), ctypes.c_void_p(d_logits), ctypes.c_void_p(d_x),
+                                        x_stride or self.hidden, n_tok, ctypes.c_void_p(d_out),
+                                        out_stride or self.hidden, stream)
+
     def parts(self, n_tok):
         """Offsets of the intermediates inside the workspace (test hook)."""
         v = (ctypes.c_size_t * 12)()
