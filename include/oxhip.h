@@ -41,6 +41,7 @@ extern "C" {
 #define OXH_ERR_NOMEM    (-5)
 #define OXH_ERR_FORMAT   (-6) /* a model file is malformed or truncated       */
 #define OXH_ERR_IO       (-7) /* a model file could not be opened or mapped   */
+#define OXH_ERR_TIMEOUT  (-8) /* a bounded wait inside a plan launch ran out  */
 
 /* GGUF quantization type ids handled here; values are ABI
  * (oxidize-c/include/oxidize/quant.h:94-110). */
@@ -200,6 +201,66 @@ int oxh_gemv_segments_fused(uint32_t qtype, const OxhSegment *segs, size_t n_seg
                             size_t cols, const float *d_x, size_t x_stride,
                             const OxhPrologue *pro, void *d_act_out, size_t n_vec,
                             size_t out_stride, void *stream);
+
+/* A chain of decode matmuls as ONE launch.  The reference's device path
+ * submits the whole token chain and replays it at about one launch per token
+ * (oxidize-c/include/oxidize/cuda.h:250-265, cuda_fast.cu); here the chain is
+ * compiled into a table in device memory and walked by one persistent kernel
+ * (a 16-wave workgroup per compute unit), which takes the launch gap, the
+ * argument fetch and the cold start of the weight stream out of every matmul:
+ * a wave requests the next operation's first weights before it has summed the
+ * rows of the current one.
+ *
+ * An operation is what one oxh_gemv_segments_fused call describes: up to four
+ * non-empty segments (each over activation 0, one vector; d_w_pair allowed),
+ * the f32 input, an optional prologue, an optional store of the quantised
+ * bytes.  Types: Q4_K, Q5_K, Q6_K; cols a multiple of 256 up to 16384.
+ * Anything else makes oxh_plan_create return OXH_DECLINED (launch those
+ * matmuls one by one).  Results are bit-identical to the same calls made one
+ * after the other.
+ *
+ * Dependencies are found from the addresses: an operation that reads or
+ * overwrites what an earlier operation wrote (or overwrites what it read)
+ * waits until every workgroup has finished that earlier one; operations
+ * without such a conflict run back to back without waiting.  Buffers that
+ * pass between operations may be ordinary oxh_malloc memory.  An operation
+ * must not store a result over one of its own inputs.
+ *
+ * All workgroups must be resident together (one per compute unit; the kernel
+ * needs the whole device, so do not run other kernels beside a plan launch).
+ * Every wait is bounded: after `polls` unsuccessful polls (about a microsecond
+ * each; default 4 000 000, OXH_PLAN_SPIN_LIMIT) the launch gives up, every
+ * workgroup leaves, and oxh_plan_status reports OXH_ERR_TIMEOUT.  A plan keeps
+ * progress counters in device memory between launches: launches of one plan
+ * must not overlap (one stream, or ordered by events); a graph may replay it. */
+typedef struct OxhPlanOp {
+    uint32_t           qtype;
+    const OxhSegment  *segs;
+    size_t             n_segs;
+    size_t             cols;
+    const float       *d_x;
+    const OxhPrologue *pro;         /* NULL: quantise d_x as it is */
+    void              *d_act_out;   /* NULL, or where the quantised bytes are also stored */
+} OxhPlanOp;
+typedef struct OxhPlan OxhPlan;
+int oxh_plan_create(const OxhPlanOp *ops, size_t n_ops, OxhPlan **plan);
+int oxh_plan_launch(OxhPlan *plan, void *stream);
+/* Waits for `stream`, then OXH_OK, or OXH_ERR_TIMEOUT when a launch since the
+ * last call gave up (the plan is reset and may be launched again). */
+int oxh_plan_status(OxhPlan *plan, void *stream);
+/* Operations, how many of them wait for an earlier one, workgroups, LDS bytes
+ * per workgroup.  Any pointer may be NULL. */
+int oxh_plan_info(const OxhPlan *plan, size_t *n_ops, size_t *n_waits, size_t *workgroups, size_t *lds_bytes);
+/* The poll limit of every wait.  With `phantom_workgroup` set the waits also
+ * expect a workgroup that does not exist, so every wait runs into the limit:
+ * the way to test the give-up path without hanging anything. */
+int oxh_plan_set_spin_limit(OxhPlan *plan, uint32_t polls, int phantom_workgroup);
+int oxh_plan_destroy(OxhPlan *plan);
+/* How a plan deals the rows of one operation's segments to `grid` workgroups of
+ * sixteen waves (pure host arithmetic): workgroups per segment and the most
+ * table rows any wave owns (a paired segment counts two per row). */
+int oxh_plan_deal(const size_t *rows, const int *paired, size_t n_segs, uint32_t grid, uint32_t *n_wg,
+                  uint32_t *rows_cap);
 
 /* Prefill matmul on int8 MFMA: out[v*out_stride + r] = dot(W[r], act[v]) for
  * v < n_vec (any count), Q8_K activations, Q4_K / Q5_K / Q6_K weights.

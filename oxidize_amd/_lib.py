@@ -10,7 +10,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, "liboxhip.so")
 
 OK, DECLINED = 0, 1
-ERR_HIP, ERR_ARG, ERR_NO_DEVICE, ERR_TOO_WIDE, ERR_NOMEM, ERR_FORMAT, ERR_IO = -1, -2, -3, -4, -5, -6, -7
+ERR_HIP, ERR_ARG, ERR_NO_DEVICE, ERR_TOO_WIDE, ERR_NOMEM, ERR_FORMAT, ERR_IO, ERR_TIMEOUT = -1, -2, -3, -4, -5, -6, -7, -8
 
 V = ctypes.c_void_p
 Z = ctypes.c_size_t
@@ -26,6 +26,11 @@ class OxhSegment(ctypes.Structure):
 class OxhPrologue(ctypes.Structure):
     _fields_ = [("kind", U32), ("eps", ctypes.c_float), ("d_b", V), ("d_out", V), ("d_add", V),
                 ("d_sum_out", V)]
+
+
+class OxhPlanOp(ctypes.Structure):
+    _fields_ = [("qtype", U32), ("segs", ctypes.POINTER(OxhSegment)), ("n_segs", Z), ("cols", Z), ("d_x", V),
+                ("pro", ctypes.POINTER(OxhPrologue)), ("d_act_out", V)]
 
 
 class OxhMoe(ctypes.Structure):
@@ -58,6 +63,13 @@ SIGNATURES = {
     "oxh_gemv_segments_f32": (I, [U32, ctypes.POINTER(OxhSegment), Z, Z, V, Z, V, Z, Z, V]),
     "oxh_gemv_segments_fused": (I, [U32, ctypes.POINTER(OxhSegment), Z, Z, V, Z,
                                     ctypes.POINTER(OxhPrologue), V, Z, Z, V]),
+    "oxh_plan_create": (I, [ctypes.POINTER(OxhPlanOp), Z, ctypes.POINTER(V)]),
+    "oxh_plan_launch": (I, [V, V]),
+    "oxh_plan_status": (I, [V, V]),
+    "oxh_plan_info": (I, [V, ctypes.POINTER(Z), ctypes.POINTER(Z), ctypes.POINTER(Z), ctypes.POINTER(Z)]),
+    "oxh_plan_set_spin_limit": (I, [V, U32, I]),
+    "oxh_plan_destroy": (I, [V]),
+    "oxh_plan_deal": (I, [ctypes.POINTER(Z), ctypes.POINTER(I), Z, U32, ctypes.POINTER(U32), ctypes.POINTER(U32)]),
     "oxh_mmq": (I, [U32, V, Z, Z, V, Z, V, Z, V]),
     "oxh_get_rows": (I, [U32, V, Z, Z, V, Z, V, Z, V]),
     "oxh_debug_subblock_sums": (I, [U32, V, Z, Z, V, V, V]),

@@ -33,18 +33,29 @@ def _run(cmd):
     return proc.stdout
 
 
-def build_oxhip(verbose=False):
-    obj_hip = os.path.join(CSRC, "oxh_kernels.o")
+HIP_UNITS = ("oxh_kernels", "oxh_plan")
+
+
+def build_oxhip(verbose=False, only=None):
+    """`only`: names of HIP translation units to recompile (the others' objects are reused)."""
+    from concurrent.futures import ThreadPoolExecutor
     obj_c = os.path.join(CSRC, "oc_matvec.o")
     obj_g = os.path.join(CSRC, "oxh_gguf.o")
     out = os.path.join(HERE, "liboxhip.so")
-    log = _run([HIPCC] + HIP_FLAGS + ["-I", INCLUDE, "-I", CSRC, "-c",
-                                     os.path.join(CSRC, "oxh_kernels.hip"), "-o", obj_hip])
+    units = [u for u in HIP_UNITS if only is None or u in only or not os.path.exists(os.path.join(CSRC, u + ".o"))]
+
+    def compile_unit(u):
+        return _run([HIPCC] + HIP_FLAGS + ["-I", INCLUDE, "-I", CSRC, "-c", os.path.join(CSRC, u + ".hip"),
+                                          "-o", os.path.join(CSRC, u + ".o")])
+
+    with ThreadPoolExecutor(max_workers=len(HIP_UNITS)) as pool:
+        log = "".join(pool.map(compile_unit, units))
+    hip_objs = [os.path.join(CSRC, u + ".o") for u in HIP_UNITS]
     log += _run([CC] + C_FLAGS + ["-I", INCLUDE, "-I", CSRC, "-c",
                                   os.path.join(CSRC, "oc_matvec.c"), "-o", obj_c])
     log += _run([CC] + C_FLAGS + ["-I", INCLUDE, "-I", CSRC, "-c",
                                   os.path.join(CSRC, "oxh_gguf.c"), "-o", obj_g])
-    log += _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", out, obj_hip, obj_c, obj_g,
+    log += _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", out] + hip_objs + [obj_c, obj_g,
                  "-lpthread", "-Wno-unused-command-line-argument"])
     if verbose and log.strip():
         print(log)

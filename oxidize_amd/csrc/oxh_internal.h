@@ -21,6 +21,11 @@ size_t oxh_gemv_max_nvec(uint32_t qtype, size_t cols);
  * (up to 16 for Q8_0 weights, which then run on the matrix cores). */
 size_t oxh_gemv_max_nvec_buffered(uint32_t qtype, size_t cols);
 
+/* Sets the thread's error text (printf-style) and returns `status`. */
+int oxh_internal_errorf(int status, const char *fmt, ...);
+/* Compute units and index of the device oxh_init() chose (0 / -1 before it ran). */
+int oxh_internal_n_cu(void);
+int oxh_internal_device(void);
 /* Host layer: drop the weight registry and the staging buffers (oxh_shutdown). */
 void oxh_internal_host_reset(void);
 

@@ -20,6 +20,7 @@
  *   -Xclang -target-feature -Xclang -packed-fp32-ops
  */
 #include <hip/hip_runtime.h>
+#include <stdarg.h>
 #include <stdint.h>
 #include <stdio.h>
 #include <stdlib.h>
@@ -44,6 +45,15 @@ extern "C" void oxh_set_error(const char *fmt, const char *a, const char *b)
     snprintf(g_err, sizeof g_err, fmt, a ? a : "", b ? b : "");
 }
 
+extern "C" int oxh_internal_errorf(int status, const char *fmt, ...)
+{
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof g_err, fmt, ap);
+    va_end(ap);
+    return status;
+}
+
 static int hip_fail(hipError_t e, const char *what)
 {
     snprintf(g_err, sizeof g_err, "HIP error in %s: %s", what, hipGetErrorString(e));
@@ -62,133 +72,7 @@ static int arg_fail(const char *what)
     return OXH_ERR_ARG;
 }
 
-/* ─── small device helpers ────────────────────────────────────────────── */
-
-typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-
-/* 16-byte vector with only 2-byte alignment: Q6_K (210 B) and Q8_0 (34 B)
- * blocks start on even addresses.  gfx9+ under HSA runs with unaligned
- * global access enabled, and the compiler emits one global_load_dwordx4. */
-struct __attribute__((packed, aligned(2))) U32x4u2 { uint32_t x, y, z, w; };
-struct __attribute__((packed, aligned(2))) U32u2 { uint32_t v; };
-
-__device__ __forceinline__ int dot4(uint32_t a, uint32_t b, int c)
-{
-    return __builtin_amdgcn_sdot4((int)a, (int)b, c, false);
-}
-
-/* Sum over the four lanes of a quad; every lane receives the total. */
-__device__ __forceinline__ int quad_sum(int v)
-{
-    v += __builtin_amdgcn_update_dpp(0, v, 0xB1, 0xF, 0xF, false); /* lanes ^1 */
-    v += __builtin_amdgcn_update_dpp(0, v, 0x4E, 0xF, 0xF, false); /* lanes ^2 */
-    return v;
-}
-
-/* Maximum over the wave; every lane receives it.  Quad and row steps are DPP
- * (xor 1, xor 2, mirror within 8, mirror within 16), the four row results
- * are combined through scalar registers. */
-__device__ __forceinline__ float dpp_max_step(float v, const int ctrl_sel)
-{
-    int o;
-    switch (ctrl_sel) {
-    case 0:  o = __builtin_amdgcn_update_dpp(0, __float_as_int(v), 0xB1, 0xF, 0xF, false); break;
-    case 1:  o = __builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x4E, 0xF, 0xF, false); break;
-    case 2:  o = __builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x141, 0xF, 0xF, false); break;
-    default: o = __builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x140, 0xF, 0xF, false); break;
-    }
-    return fmaxf(v, __int_as_float(o));
-}
-
-/* max over each aligned group of 8 lanes */
-__device__ __forceinline__ float oct_max(float v)
-{
-    v = dpp_max_step(v, 0);
-    v = dpp_max_step(v, 1);
-    v = dpp_max_step(v, 2);
-    return v;
-}
-
-__device__ __forceinline__ float wave_max(float v)
-{
-    v = oct_max(v);
-    v = dpp_max_step(v, 3);
-    const int b = __float_as_int(v);
-    const float r0 = __int_as_float(__builtin_amdgcn_readlane(b, 0));
-    const float r1 = __int_as_float(__builtin_amdgcn_readlane(b, 16));
-    const float r2 = __int_as_float(__builtin_amdgcn_readlane(b, 32));
-    const float r3 = __int_as_float(__builtin_amdgcn_readlane(b, 48));
-    return fmaxf(fmaxf(r0, r1), fmaxf(r2, r3));
-}
-
-/* binary16 -> binary32 with the hardware converter (exact for every input,
- * subnormals included: f16 denormals are never flushed on this target). */
-__device__ __forceinline__ float half_to_float_hw(uint32_t h)
-{
-    return (float)__builtin_bit_cast(_Float16, (uint16_t)h);
-}
-
-/* Exact binary16 -> binary32 including subnormals (integer-only so it does
- * not depend on the wave's denormal mode). */
-__device__ __forceinline__ float half_bits_to_float(uint32_t h)
-{
-    const uint32_t sign = (h & 0x8000u) << 16;
-    const uint32_t e = (h >> 10) & 31u;
-    const uint32_t m = h & 0x3FFu;
-    uint32_t bits;
-    if (e == 31u) {
-        bits = sign | 0x7F800000u | (m << 13);
-    } else if (e != 0u) {
-        bits = sign | ((e + 112u) << 23) | (m << 13);
-    } else if (m == 0u) {
-        bits = sign;
-    } else {
-        const uint32_t lz = (uint32_t)__clz((int)m) - 21u;   /* shifts to bit 10 */
-        bits = sign | ((113u - lz) << 23) | (((m << lz) & 0x3FFu) << 13);
-    }
-    return __uint_as_float(bits);
-}
-
-/* binary32 -> binary16 bits, round-half-UP on the dropped bits
- * (flash_attention.c:149-185). */
-__device__ __forceinline__ uint32_t float_to_half_bits_half_up(float v)
-{
-    const uint32_t u = __float_as_uint(v);
-    const uint32_t sign = (u >> 16) & 0x8000u;
-    const int e32 = (int)((u >> 23) & 0xFFu);
-    const uint32_t man = u & 0x7FFFFFu;
-    if (e32 == 255) {
-        if (man == 0u) return sign | 0x7C00u;
-        uint32_t payload = man >> 13;
-        if (payload == 0u) payload = 1u;
-        return sign | 0x7C00u | payload;
-    }
-    const int e16 = e32 - 112;
-    if (e16 >= 31) return sign | 0x7C00u;
-    if (e16 >= 1) {
-        uint32_t out = ((uint32_t)e16 << 10) | (man >> 13);
-        if (man & 0x1000u) {
-            out += 1u;
-            if (out >= 0x7C00u) return sign | 0x7C00u;
-        }
-        return sign | out;
-    }
-    if (e16 < -10) return sign;
-    const uint32_t full = man | 0x800000u;
-    const uint32_t sh = (uint32_t)(14 - e16);
-    uint32_t out = full >> sh;
-    if ((full >> (sh - 1u)) & 1u) out += 1u;
-    return sign | out;
-}
-
-__device__ __forceinline__ int quantize_one(float x, float inv)
-{
-    /* lrintf under round-to-nearest-even == v_rndne_f32 + convert */
-    int v = (int)rintf(x * inv);
-    v = v > 127 ? 127 : v;
-    v = v < -128 ? -128 : v;
-    return v;
-}
+#include "oxh_device.inc"
 
 /* ─── activation quantisers ───────────────────────────────────────────── */
 
@@ -625,6 +509,8 @@ static hipStream_t pick_stream(void *stream)
 }
 
 extern "C" void *oxh_internal_stream(void) { return (void *)g_stream; }
+extern "C" int oxh_internal_n_cu(void) { return g_n_cu; }
+extern "C" int oxh_internal_device(void) { return g_device.load(std::memory_order_acquire); }
 
 /* AL5, AL6 and AL8 are the Q4_0, Q5_0 and Q8_0 block layouts under ids of
  * their own (oxidize-c/src/compute/quantization.c:207-214; the encoder

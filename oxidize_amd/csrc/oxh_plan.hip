@@ -1,0 +1,837 @@
+/*
+ * oxh_plan.hip — a whole decode step as ONE launch.
+ *
+ * A decode step of a dense model is a fixed chain of a hundred-odd matrix-vector
+ * products (q/k/v, o, gate/up, down per layer), each a few microseconds long.
+ * Launched one by one, every product pays the gap between two kernels, the
+ * fetch of its arguments and a cold start of its weight stream; the reference's
+ * device path therefore submits the whole token chain at once
+ * (oxidize-c/include/oxidize/cuda.h:250-265).  Here the chain is compiled into a
+ * table of operations in device memory (an OxhPlan) and walked by one
+ * persistent kernel: one 16-wave workgroup per compute unit, every workgroup
+ * taking its share of the rows of every operation.
+ *
+ *   - The arithmetic is the GEMV kernels' (gemv_kernels.inc): same lane split,
+ *     same per-block f32 term, same strictly ordered per-row sum, so results
+ *     are bit-identical to oxh_gemv_segments_fused launched op by op.
+ *   - A wave asks for the first two passes of weights of the NEXT operation
+ *     as soon as its registers are free, before it sums its rows: weights do
+ *     not depend on activations, so the weight stream does not stop at an
+ *     operation boundary.
+ *   - An operation that reads what an earlier one wrote waits until every
+ *     workgroup has finished that one.  Workgroups announce progress with one
+ *     monotonic counter each; workgroup 0 gathers them and publishes the
+ *     minimum.  The eight L2 caches of the device are not coherent with each
+ *     other and a fence that makes them so costs 35 us here, so there are no
+ *     fences: everything one operation hands to another (outputs, residual
+ *     sums) is stored and loaded with system-coherent accesses that bypass the
+ *     L2s, and so are the counters.
+ *   - Every wait is bounded: after `spin_limit` polls a workgroup raises the
+ *     plan's error word and leaves, and every other workgroup leaves at its
+ *     next wait, so a launch that cannot make progress (not all workgroups
+ *     resident) ends by itself.
+ *
+ * Wave64, gfx950.  Build flags as oxh_kernels.hip.
+ */
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+
+#include "oxhip.h"
+#include "oxh_internal.h"
+
+#pragma clang fp contract(off)
+
+#include "oxh_device.inc"
+#include "gemv_kernels.inc"
+
+#define PLAN_MAX_SEGS 4
+#define PLAN_W 16u                  /* waves per workgroup */
+#define PLAN_MAX_WG 1024u
+#define PLAN_MAX_BLOCKS 64u         /* super-blocks per row: four units per wave staged at once */
+
+#define PLAN_Q4_K 0u
+#define PLAN_Q5_K 1u
+#define PLAN_Q6_K 2u
+
+/* Device addresses travel through the table as integers and become global-memory pointers in the
+ * kernel: a pointer merely loaded from memory is a generic one to the compiler, and loads through it
+ * are flat_load, counted by lgkmcnt as well as vmcnt, so that every LDS wait would wait for them. */
+typedef uint64_t gaddr;
+
+struct PlanSeg {
+    gaddr w, w2;                    /* w2: the paired matrix or 0 */
+    gaddr out;
+    uint32_t rows, wg_begin, rows_q, rows_rem;
+};
+
+struct PlanOp {
+    uint32_t kind, pro, n_segs, blocks;
+    uint32_t magic, term_stride, rows_cap, n_wg;
+    uint32_t wait;                  /* 0, or 1 + index of the operation that must be complete everywhere */
+    uint32_t signal;                /* a later operation waits for this one */
+    float eps;
+    uint32_t pad;
+    gaddr x, pro_b, pro_add;
+    gaddr pro_sum_out, pro_out;
+    gaddr act_out;
+    PlanSeg s[PLAN_MAX_SEGS];
+};
+
+/* progress counters: flags[wg], then go[0] = the published minimum, go[1] = error word */
+struct PlanSync {
+    uint32_t *flags;
+    uint32_t *go;
+    uint32_t n_wait;                /* counters gathered: the grid size (one more in the time-out test) */
+    uint32_t spin_limit;
+};
+
+struct PlanLds {
+    uint32_t act_bytes;             /* one staged activation (two are kept, used in turn) */
+    uint32_t outs_off, red_off, terms_off, terms_per_wave;   /* bytes; terms_per_wave in floats */
+};
+
+/* ─── coherent accesses ───────────────────────────────────────────────── */
+
+/* System-scope accesses (sc0 sc1) go past the per-XCD L2s to the memory side, where every XCD sees
+ * the same data.  Single words use the atomic builtins; 16-byte pieces use buffer instructions with
+ * that cache policy (a volatile generic access would compile to flat_load, which also counts as an
+ * LDS operation).  Bit 31 of the policy marks the access volatile for the compiler, so that a poll
+ * is not hoisted out of its loop and nothing moves across it. */
+#define OXH_SYSTEM_COHERENT ((int)(0x11u | 0x80000000u))
+
+typedef __amdgpu_buffer_rsrc_t CohBuf;
+
+__device__ __forceinline__ CohBuf coh_buf(const void *base)
+{
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, 0x7FFFFFFF, 0x27000);
+}
+__device__ __forceinline__ u32x4 cload16(CohBuf b, uint32_t byte_off)
+{
+    return __builtin_amdgcn_raw_buffer_load_b128(b, (int)byte_off, 0, OXH_SYSTEM_COHERENT);
+}
+__device__ __forceinline__ uint32_t cload(const uint32_t *p)
+{
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+}
+__device__ __forceinline__ void cstore(uint32_t *p, uint32_t v)
+{
+    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+}
+__device__ __forceinline__ void cstore_f32(CohBuf b, uint32_t byte_off, float v)
+{
+    __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(v), b, (int)byte_off, 0, OXH_SYSTEM_COHERENT);
+}
+__device__ __forceinline__ XRegs cload4(CohBuf b, uint32_t byte_off)
+{
+    const u32x4 v = cload16(b, byte_off);
+    XRegs r;
+    r.v0 = __uint_as_float(v.x); r.v1 = __uint_as_float(v.y);
+    r.v2 = __uint_as_float(v.z); r.v3 = __uint_as_float(v.w);
+    return r;
+}
+__device__ __forceinline__ void cstore4(CohBuf b, uint32_t byte_off, const XRegs &y)
+{
+    u32x4 v = { __float_as_uint(y.v0), __float_as_uint(y.v1), __float_as_uint(y.v2), __float_as_uint(y.v3) };
+    __builtin_amdgcn_raw_buffer_store_b128(v, b, (int)byte_off, 0, OXH_SYSTEM_COHERENT);
+}
+
+/* workgroup barrier that orders LDS only: __syncthreads() may also wait for every
+ * global load in flight, and the prefetched weights of the next operation are */
+__device__ __forceinline__ void lds_barrier()
+{
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+template <typename T>
+__device__ __forceinline__ T *gptr(gaddr v)
+{
+    typedef T __attribute__((address_space(1))) *G;
+    return (T *)reinterpret_cast<G>(v);
+}
+
+/* ─── what a wave owns of an operation ───────────────────────────────── */
+
+struct PWork {
+    WSrc src;                       /* flat block list: nblk blocks, the first n1 in src.a */
+    float *out;                     /* the segment's output vector */
+    uint32_t nblk, nrows, row0;
+    uint32_t wg_row0, wg_rows;      /* the workgroup's contiguous run of rows */
+    uint32_t kind;
+    bool paired;
+};
+
+__device__ __forceinline__ uint32_t plan_block_bytes(uint32_t kind)
+{
+    return kind == PLAN_Q6_K ? 210u : kind == PLAN_Q5_K ? 176u : 144u;
+}
+
+__device__ __forceinline__ PWork plan_work(const PlanOp *__restrict__ op, uint32_t wave)
+{
+    PWork k;
+    const uint32_t wg = blockIdx.x, n = op->n_segs;
+    uint32_t si = 0;
+#pragma unroll
+    for (uint32_t i = 1; i < PLAN_MAX_SEGS; i++)
+        if (i < n && wg >= op->s[i].wg_begin) si = i;
+    gaddr w = op->s[0].w, w2 = op->s[0].w2, out = op->s[0].out;
+    uint32_t wg_begin = op->s[0].wg_begin, q = op->s[0].rows_q, rem = op->s[0].rows_rem;
+#pragma unroll
+    for (uint32_t i = 1; i < PLAN_MAX_SEGS; i++)
+        if (si == i) {
+            w = op->s[i].w; w2 = op->s[i].w2; out = op->s[i].out;
+            wg_begin = op->s[i].wg_begin; q = op->s[i].rows_q; rem = op->s[i].rows_rem;
+        }
+    const bool idle = wg >= op->n_wg;
+    const uint32_t wi0 = (wg - wg_begin) * PLAN_W, wi = wi0 + wave;
+    k.kind = op->kind;
+    k.row0 = wi * q + min(wi, rem);
+    k.nrows = idle ? 0u : q + (wi < rem ? 1u : 0u);
+    k.wg_row0 = wi0 * q + min(wi0, rem);
+    k.wg_rows = idle ? 0u : (wi0 + PLAN_W) * q + min(wi0 + PLAN_W, rem) - k.wg_row0;
+    k.out = gptr<float>(out);
+    const uint32_t B = op->blocks;
+    const size_t off = (size_t)(k.nrows ? k.row0 : 0u) * B * plan_block_bytes(k.kind);
+    k.src.a = gptr<const uint8_t>(w + off);
+    k.src.n1 = k.nrows * B;
+    k.paired = w2 != 0u;
+    k.src.b = gptr<const uint8_t>((k.paired ? w2 : w) + off);
+    k.nblk = k.paired ? 2u * k.src.n1 : k.src.n1;
+    return k;
+}
+
+/* ─── weight register sets, untyped so that they can cross operations ── */
+
+/* named members, not an array: stores to an array from the three format branches get merged into one
+ * store at a computed index, and the set then lives in scratch memory instead of registers */
+struct WSet { u32x4 a, b, c, d, e; };      /* e: Q5_K only (kernels built without Q5_K never touch it) */
+
+__device__ __forceinline__ u32x4 as_v4(const U32x4u2 &t) { u32x4 v = { t.x, t.y, t.z, t.w }; return v; }
+__device__ __forceinline__ U32x4u2 as_u2(const u32x4 &v) { U32x4u2 t; t.x = v.x; t.y = v.y; t.z = v.z; t.w = v.w; return t; }
+
+template <bool HAS_Q5>
+__device__ __forceinline__ void wset_load(uint32_t kind, WSet &s, const WSrc &src, uint32_t g, uint32_t lane)
+{
+    const uint32_t sub = lane & 3u;
+    /* the branches produce values, the set is written once after them: stores to different members
+     * from different branches would be merged into one store at a computed address */
+    u32x4 v0, v1, v2, v3 = s.d, v4 = s.e;
+    if (kind == PLAN_Q6_K) {
+        Q6kRegs t;
+        q6k_load<true>(t, src, g, sub >> 1, sub & 1u);
+        v0 = as_v4(t.la); v1 = as_v4(t.lb); v2 = as_v4(t.hh); v3 = as_v4(t.tail);
+    } else if (HAS_Q5 && kind == PLAN_Q5_K) {
+        Q4kRegs t;
+        q4k_load<true, true>(t, src, g, sub);
+        v0 = t.hdr; v1 = t.na; v2 = t.nb; v3 = t.ha; v4 = t.hb;
+    } else {
+        Q4kRegs t;
+        q4k_load<false, true>(t, src, g, sub);
+        v0 = t.hdr; v1 = t.na; v2 = t.nb;
+    }
+    s.a = v0; s.b = v1; s.c = v2; s.d = v3;
+    if (HAS_Q5) s.e = v4;
+}
+
+template <bool HAS_Q5>
+__device__ __forceinline__ void plan_prefetch(const PWork &k, WSet &A, WSet &B, uint32_t lane)
+{
+    if (k.nblk == 0u) return;
+    const uint32_t last = k.nblk - 1u;
+    wset_load<HAS_Q5>(k.kind, A, k.src, min(lane >> 2, last), lane);
+    wset_load<HAS_Q5>(k.kind, B, k.src, min(16u + (lane >> 2), last), lane);
+}
+
+/* ─── the passes of one operation (sets A and B hold passes 0 and 1) ──── */
+
+template <bool Q5>
+__device__ __forceinline__ void
+plan_passes_q45(const WSet &A0, const WSet &B0, const PWork &k, const GemvParams &p, const uint8_t *act,
+                uint32_t act_lds, float *terms, uint32_t lane)
+{
+    const uint32_t nblk = k.nblk, B = p.blocks, s = lane & 3u;
+    Q4kRegs A, Bq;
+    A.hdr = A0.a; A.na = A0.b; A.nb = A0.c;
+    Bq.hdr = B0.a; Bq.na = B0.b; Bq.nb = B0.c;
+    if (Q5) { A.ha = A0.d; A.hb = A0.e; Bq.ha = B0.d; Bq.hb = B0.e; }
+    Q4kLane ln;
+    ln.s = s;
+    ln.hi = s >= 2u;
+    ln.sh = (s & 1u) * 16u;
+    ln.mask_a = ln.hi ? 0x0F0F0F0Fu : 0x3F3F3F3Fu;
+    ln.mask_b = ln.hi ? 0x30303030u : 0u;
+    const uint32_t last = nblk - 1u, npass = (nblk + 15u) / 16u;
+    const uint32_t lb = lane >> 2;
+    uint32_t i = 0;
+    while (i + 3u < npass) {
+        q4k_pass<1, false, Q5>(A, ln, p, act, act_lds, 1u, B, i * 16u + lb, nblk, k.row0, terms);
+        q4k_load<Q5, true>(A, k.src, min((i + 2u) * 16u + lb, last), s);
+        q4k_pass<1, false, Q5>(Bq, ln, p, act, act_lds, 1u, B, (i + 1u) * 16u + lb, nblk, k.row0, terms);
+        q4k_load<Q5, true>(Bq, k.src, min((i + 3u) * 16u + lb, last), s);
+        i += 2u;
+    }
+    const uint32_t rem = npass - i;                 /* 1, 2 or 3 */
+    q4k_pass<1, false, Q5>(A, ln, p, act, act_lds, 1u, B, i * 16u + lb, nblk, k.row0, terms);
+    if (rem == 3u) q4k_load<Q5, true>(A, k.src, min((i + 2u) * 16u + lb, last), s);
+    if (rem >= 2u) q4k_pass<1, false, Q5>(Bq, ln, p, act, act_lds, 1u, B, (i + 1u) * 16u + lb, nblk, k.row0, terms);
+    if (rem == 3u) q4k_pass<1, false, Q5>(A, ln, p, act, act_lds, 1u, B, (i + 2u) * 16u + lb, nblk, k.row0, terms);
+}
+
+__device__ __forceinline__ void
+plan_passes_q6(const WSet &A0, const WSet &B0, const PWork &k, const GemvParams &p, const uint8_t *act,
+               uint32_t act_lds, float *terms, uint32_t lane)
+{
+    const uint32_t nblk = k.nblk, B = p.blocks, u = lane & 3u, n = u >> 1, lh = u & 1u;
+    Q6kRegs A, Bq;
+    A.la = as_u2(A0.a); A.lb = as_u2(A0.b); A.hh = as_u2(A0.c); A.tail = as_u2(A0.d);
+    Bq.la = as_u2(B0.a); Bq.lb = as_u2(B0.b); Bq.hh = as_u2(B0.c); Bq.tail = as_u2(B0.d);
+    const uint32_t last = nblk - 1u, npass = (nblk + 15u) / 16u;
+    const uint32_t lb = lane >> 2;
+    uint32_t i = 0;
+    while (i + 3u < npass) {
+        q6k_pass<1, false>(A, u, p, act, act_lds, 1u, B, i * 16u + lb, nblk, k.row0, terms);
+        q6k_load<true>(A, k.src, min((i + 2u) * 16u + lb, last), n, lh);
+        q6k_pass<1, false>(Bq, u, p, act, act_lds, 1u, B, (i + 1u) * 16u + lb, nblk, k.row0, terms);
+        q6k_load<true>(Bq, k.src, min((i + 3u) * 16u + lb, last), n, lh);
+        i += 2u;
+    }
+    const uint32_t rem = npass - i;
+    q6k_pass<1, false>(A, u, p, act, act_lds, 1u, B, i * 16u + lb, nblk, k.row0, terms);
+    if (rem == 3u) q6k_load<true>(A, k.src, min((i + 2u) * 16u + lb, last), n, lh);
+    if (rem >= 2u) q6k_pass<1, false>(Bq, u, p, act, act_lds, 1u, B, (i + 1u) * 16u + lb, nblk, k.row0, terms);
+    if (rem == 3u) q6k_pass<1, false>(A, u, p, act, act_lds, 1u, B, (i + 2u) * 16u + lb, nblk, k.row0, terms);
+}
+
+/* per-row sums in block order into the workgroup's output staging; a paired operation writes
+ * silu(first) * second (the expression of row_sums_paired) */
+__device__ __forceinline__ void
+plan_row_sums(const float *terms, const PWork &k, uint32_t B, uint32_t term_stride, float *outs, uint32_t lane)
+{
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    for (uint32_t r = lane; r < k.nrows; r += 64u) {
+        const float *t = terms + __umul24(r, term_stride);
+        float v = row_sum_one<1>(t, B);
+        if (k.paired) {
+            const float u = row_sum_one<1>(t + __umul24(k.nrows, term_stride), B);
+            const float sig = 1.0f / (1.0f + expf(-v));
+            v = v * sig * u;
+        }
+        outs[k.row0 - k.wg_row0 + r] = v;
+    }
+}
+
+/* ─── activation staging: one f32 vector -> Q8_K in LDS ──────────────── */
+
+/* The vector may have been written by another workgroup a moment ago: it is read with coherent
+ * loads, and so is everything else an operation can have produced (the added vector, SwiGLU's
+ * second operand).  Norm weights are constants.  Arithmetic and order are stage_begin / stage_end's
+ * for one vector and sixteen waves, so the quantised bytes are the same. */
+template <int KIND /* 0 Q4_K/Q5_K layout, 1 Q6_K layout */, int PRO>
+__device__ __forceinline__ void
+plan_stage(const PlanOp *__restrict__ op, uint8_t *base, float *red, bool storer, uint32_t lane, uint32_t wave)
+{
+    constexpr bool RMS = PRO == GEMV_PRO_RMSNORM || PRO == GEMV_PRO_ADD_RMSNORM;
+    constexpr bool ADD = PRO == GEMV_PRO_ADD_RMSNORM;
+    const uint32_t B = op->blocks;
+    const CohBuf x = coh_buf(gptr<const float>(op->x)), add = coh_buf(gptr<const float>(op->pro_add));
+    const CohBuf bc = coh_buf(gptr<const float>(op->pro_b));
+    const float *b = gptr<const float>(op->pro_b);
+    XRegs xr[4], br[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const uint32_t unit = wave + PLAN_W * (uint32_t)i;
+        xr[i] = br[i] = XRegs{ 0.f, 0.f, 0.f, 0.f };
+        if (unit < B) {
+            const uint32_t at = unit * 256u + 4u * lane;
+            xr[i] = cload4(x, at * 4u);
+            if (ADD) {
+                const XRegs t = cload4(add, at * 4u);
+                xr[i].v0 += t.v0; xr[i].v1 += t.v1; xr[i].v2 += t.v2; xr[i].v3 += t.v3;
+            }
+            if (PRO == GEMV_PRO_SWIGLU) br[i] = cload4(bc, at * 4u);
+            else if (RMS) br[i] = x_load4(b + at);
+        }
+    }
+    float inv = 1.0f;
+    if (RMS) {
+        float ss = 0.0f;
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+            if (wave + PLAN_W * (uint32_t)i < B)
+                ss += xr[i].v0 * xr[i].v0 + xr[i].v1 * xr[i].v1 + xr[i].v2 * xr[i].v2 + xr[i].v3 * xr[i].v3;
+        ss = wave_sum_f32(ss);
+        if (lane == 0u) red[wave] = ss;
+        __syncthreads();
+        const float tot = wave_sum_f32(lane < PLAN_W ? red[lane] : 0.0f);
+        inv = 1.0f / sqrtf(tot / (float)(B * 256u) + op->eps);
+    }
+    const bool has_sout = ADD && storer && op->pro_sum_out != 0u;
+    const bool has_fout = PRO != GEMV_PRO_NONE && storer && op->pro_out != 0u;
+    const CohBuf sout = coh_buf(gptr<float>(op->pro_sum_out)), fout = coh_buf(gptr<float>(op->pro_out));
+    uint8_t *gout = (storer && op->act_out) ? gptr<uint8_t>(op->act_out) : nullptr;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const uint32_t unit = wave + PLAN_W * (uint32_t)i;
+        if (unit < B) {
+            const uint32_t at = unit * 256u + 4u * lane;
+            if (has_sout) cstore4(sout, at * 4u, xr[i]);
+            const XRegs y = prologue_apply<PRO>(xr[i], br[i], inv);
+            if (has_fout) cstore4(fout, at * 4u, y);
+            q8k_x_finish<KIND == 1>(y, B, unit, base, gout, lane);
+        }
+    }
+    /* what this workgroup stored for later operations has to be complete before it announces the
+     * operation done; the only loads in flight here are the first passes' weights, needed next anyway */
+    if (has_sout || has_fout) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+}
+
+template <int KIND>
+__device__ __forceinline__ void
+plan_stage_any(const PlanOp *__restrict__ op, uint8_t *base, float *red, bool storer, uint32_t lane, uint32_t wave)
+{
+    switch (op->pro) {
+    case GEMV_PRO_RMSNORM:     plan_stage<KIND, GEMV_PRO_RMSNORM>(op, base, red, storer, lane, wave); break;
+    case GEMV_PRO_ADD_RMSNORM: plan_stage<KIND, GEMV_PRO_ADD_RMSNORM>(op, base, red, storer, lane, wave); break;
+    case GEMV_PRO_SWIGLU:      plan_stage<KIND, GEMV_PRO_SWIGLU>(op, base, red, storer, lane, wave); break;
+    default:                   plan_stage<KIND, GEMV_PRO_NONE>(op, base, red, storer, lane, wave); break;
+    }
+}
+
+/* ─── waiting for an operation to be complete on every workgroup ──────── */
+
+/* Counters only grow (modulo 2^32): "reached" is a signed difference. */
+__device__ __forceinline__ bool reached(uint32_t v, uint32_t target) { return (int32_t)(v - target) >= 0; }
+
+__device__ __forceinline__ bool
+plan_wait(const PlanSync &sy, uint32_t target, int *s_ok, uint32_t lane, uint32_t wave)
+{
+    if (wave == 0u) {
+        bool ok = true;
+        uint32_t spins = 0;
+        if (blockIdx.x == 0u) {
+            for (;;) {
+                bool mine = true;
+                const CohBuf fb = coh_buf(sy.flags);
+                for (uint32_t k = 4u * lane; k < sy.n_wait; k += 256u) {
+                    const u32x4 f = cload16(fb, k * 4u);
+                    mine = mine && reached(f.x, target) && (k + 1u >= sy.n_wait || reached(f.y, target)) &&
+                           (k + 2u >= sy.n_wait || reached(f.z, target)) &&
+                           (k + 3u >= sy.n_wait || reached(f.w, target));
+                }
+                if (__all(mine)) break;
+                if (++spins > sy.spin_limit || cload(sy.go + 1) != 0u) { ok = false; break; }
+            }
+            if (lane == 0u) {
+                if (ok) cstore(sy.go, target);
+                else cstore(sy.go + 1, 1u);
+            }
+        } else {
+            const CohBuf gb = coh_buf(sy.go);
+            for (;;) {
+                const u32x4 g = cload16(gb, 0u);
+                if (reached(g.x, target)) break;
+                if (g.y != 0u || ++spins > sy.spin_limit) {
+                    ok = false;
+                    if (lane == 0u) cstore(sy.go + 1, 1u);
+                    break;
+                }
+            }
+        }
+        if (lane == 0u) *s_ok = ok ? 1 : 0;
+    }
+    __syncthreads();
+    return *s_ok != 0;
+}
+
+/* ─── the kernel ──────────────────────────────────────────────────────── */
+
+template <bool HAS_Q5>
+__global__ __launch_bounds__(1024) void
+k_plan(const PlanOp *__restrict__ ops, uint32_t n_ops, const PlanSync sy, const PlanLds ld)
+{
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    /* the wave index in a scalar register: everything a wave owns (rows, pointers, counts) is then
+     * scalar too */
+    const uint32_t lane = threadIdx.x & 63u, wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    /* every workgroup's counter holds the same value between launches: the end of the last one */
+    const uint32_t base = cload(sy.flags + blockIdx.x);
+    float *const outs = reinterpret_cast<float *>(lds + ld.outs_off);
+    float *const red = reinterpret_cast<float *>(lds + ld.red_off);
+    int *const s_ok = reinterpret_cast<int *>(red + 24);      /* the reduction uses slots 0..15 of 32 */
+    float *const terms = reinterpret_cast<float *>(lds + ld.terms_off) + (size_t)wave * ld.terms_per_wave;
+
+    PWork cur = plan_work(&ops[0], wave);
+    WSet A, B;
+    A.a = A.b = A.c = A.d = A.e = u32x4{ 0u, 0u, 0u, 0u };
+    B.a = B.b = B.c = B.d = B.e = A.a;
+    plan_prefetch<HAS_Q5>(cur, A, B, lane);
+
+    for (uint32_t i = 0; i < n_ops; i++) {
+        const PlanOp *op = &ops[i];
+        uint8_t *act = lds + (size_t)(i & 1u) * ld.act_bytes;
+        if (op->wait != 0u && !plan_wait(sy, base + op->wait, s_ok, lane, wave)) return;
+
+        const bool storer = blockIdx.x == 0u;
+        const uint32_t Bk = op->blocks;
+        if (op->kind == PLAN_Q6_K) plan_stage_any<1>(op, act, red, storer, lane, wave);
+        else                       plan_stage_any<0>(op, act, red, storer, lane, wave);
+        __syncthreads();
+
+        GemvParams gp;
+        gp.blocks = Bk;
+        gp.magic = op->magic;
+        gp.term_stride = op->term_stride;
+        gp.rows_cap = op->rows_cap;
+        gp.dump = nullptr;
+        if (cur.nblk != 0u) {
+            if (cur.kind == PLAN_Q6_K)      plan_passes_q6(A, B, cur, gp, act, q8k6_lds_bytes(Bk), terms, lane);
+            else if (HAS_Q5 && cur.kind == PLAN_Q5_K) plan_passes_q45<true>(A, B, cur, gp, act, q8k_lds_bytes(Bk), terms, lane);
+            else                            plan_passes_q45<false>(A, B, cur, gp, act, q8k_lds_bytes(Bk), terms, lane);
+        }
+
+        /* registers are free: the next operation's first weights, before this one's rows are summed.
+         * Wave 0 asks later: it has to see its output stores complete first, and a wait for them
+         * would wait for these loads too. */
+        const bool more = i + 1u < n_ops;
+        PWork nx = cur;
+        if (more) {
+            nx = plan_work(&ops[i + 1u], wave);
+            if (wave != 0u) plan_prefetch<HAS_Q5>(nx, A, B, lane);
+        }
+        plan_row_sums(terms, cur, Bk, op->term_stride, outs, lane);
+        lds_barrier();
+        if (wave == 0u) {
+            const CohBuf dst = coh_buf(cur.out + cur.wg_row0);
+            for (uint32_t r = lane; r < cur.wg_rows; r += 64u) cstore_f32(dst, r * 4u, outs[r]);
+            if (op->signal != 0u || !more) {
+                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                /* the last operation leaves every counter at base + n_ops + 1, the next launch's base */
+                if (lane == 0u) cstore(sy.flags + blockIdx.x, base + i + 1u + (more ? 0u : 1u));
+            }
+            if (more) plan_prefetch<HAS_Q5>(nx, A, B, lane);
+        }
+        cur = nx;
+    }
+}
+
+/* ─── host side ───────────────────────────────────────────────────────── */
+
+struct OxhPlan {
+    PlanOp *d_ops;
+    uint32_t *d_sync;               /* PLAN_MAX_WG + 4 counters, then go[4] */
+    uint32_t n_ops, grid;
+    PlanLds ld;
+    size_t lds_bytes;
+    uint32_t spin_limit, phantom;
+    bool has_q5;
+    uint32_t n_waits;               /* operations that wait (for callers' curiosity) */
+};
+
+#define PLAN_TRY(call)                                                                      \
+    do {                                                                                    \
+        hipError_t e_ = (call);                                                             \
+        if (e_ != hipSuccess)                                                               \
+            return oxh_internal_errorf(OXH_ERR_HIP, "HIP error in %s: %s", #call, hipGetErrorString(e_)); \
+    } while (0)
+
+static bool plan_kind(uint32_t qtype, uint32_t *kind)
+{
+    switch (qtype) {
+    case OXH_Q4_K_S: case OXH_Q4_K_M: *kind = PLAN_Q4_K; return true;
+    case OXH_Q5_K_S: case OXH_Q5_K_M: *kind = PLAN_Q5_K; return true;
+    case OXH_Q6_K:                    *kind = PLAN_Q6_K; return true;
+    default: return false;
+    }
+}
+
+struct Span { const char *p; size_t n; };
+static bool spans_meet(const Span &a, const Span &b)
+{
+    return a.p && b.p && a.n && b.n && a.p < b.p + b.n && b.p < a.p + a.n;
+}
+
+/* Rows of an operation dealt to workgroups: in proportion to the segments' rows (a paired segment
+ * counts twice), at most `grid` in all, every wave at most GEMV_ROWS_CAP table rows. */
+extern "C" int oxh_plan_deal(const size_t *rows, const int *paired, size_t n_segs, uint32_t grid, uint32_t *n_wg,
+                             uint32_t *rows_cap)
+{
+    size_t total_work = 0;
+    for (size_t i = 0; i < n_segs; i++) total_work += rows[i] * (paired[i] ? 2u : 1u);
+    if (total_work == 0 || grid == 0) return OXH_ERR_ARG;
+    uint32_t cap = 1, sum = 0;
+    for (size_t i = 0; i < n_segs; i++) {
+        const size_t mult = paired[i] ? 2u : 1u;
+        size_t share = ((size_t)grid * rows[i] * mult + total_work / 2) / total_work;
+        const size_t hi = (rows[i] + PLAN_W - 1) / PLAN_W;
+        if (share > hi) share = hi;
+        if (share < 1) share = 1;
+        n_wg[i] = (uint32_t)share;
+        sum += n_wg[i];
+    }
+    while (sum > grid) {            /* rounding went over: the largest share gives one back */
+        size_t big = 0;
+        for (size_t i = 1; i < n_segs; i++) if (n_wg[i] > n_wg[big]) big = i;
+        if (n_wg[big] <= 1) return OXH_ERR_TOO_WIDE;
+        n_wg[big]--;
+        sum--;
+    }
+    for (size_t i = 0; i < n_segs; i++) {
+        const size_t mult = paired[i] ? 2u : 1u;
+        const size_t waves = (size_t)n_wg[i] * PLAN_W;
+        const size_t rpw = (rows[i] + waves - 1) / waves * mult;
+        if (rpw > GEMV_ROWS_CAP) return OXH_ERR_TOO_WIDE;
+        if (rpw > cap) cap = (uint32_t)rpw;
+    }
+    *rows_cap = cap;
+    return OXH_OK;
+}
+
+extern "C" int oxh_plan_create(const OxhPlanOp *ops, size_t n_ops, OxhPlan **out)
+{
+    if (!out) return oxh_internal_errorf(OXH_ERR_ARG, "invalid argument: oxh_plan_create: NULL");
+    *out = nullptr;
+    int rc = oxh_init(oxh_internal_device() >= 0 ? oxh_internal_device() : 0);
+    if (rc) return rc;
+    if (!ops || n_ops == 0 || n_ops > 0xFFFFu)
+        return oxh_internal_errorf(OXH_ERR_ARG, "invalid argument: oxh_plan_create: 1..65535 operations");
+    const uint32_t n_cu = (uint32_t)(oxh_internal_n_cu() > 0 ? oxh_internal_n_cu() : 256);
+    const uint32_t grid = n_cu > PLAN_MAX_WG ? PLAN_MAX_WG : n_cu;
+
+    PlanOp *h = (PlanOp *)calloc(n_ops, sizeof *h);
+    Span *reads = (Span *)calloc(n_ops * 4, sizeof *reads), *writes = (Span *)calloc(n_ops * 8, sizeof *writes);
+    if (!h || !reads || !writes) {
+        free(h); free(reads); free(writes);
+        return oxh_internal_errorf(OXH_ERR_NOMEM, "out of host memory building a plan");
+    }
+    uint32_t max_act = 0, max_cap_terms = 0, max_wg_rows = 0, n_waits = 0;
+    bool has_q5 = false;
+    rc = OXH_OK;
+    for (size_t i = 0; i < n_ops && !rc; i++) {
+        const OxhPlanOp &o = ops[i];
+        PlanOp &d = h[i];
+        uint32_t kind;
+        if (!plan_kind(o.qtype, &kind) || o.cols == 0 || o.cols % OXH_QK_K || o.cols / OXH_QK_K > PLAN_MAX_BLOCKS) {
+            rc = oxh_internal_errorf(OXH_DECLINED, "plan: operation %zu (qtype %u, cols %zu) is not one a plan runs: "
+                                     "Q4_K, Q5_K or Q6_K with cols a multiple of 256 up to %u", i, o.qtype, o.cols,
+                                     PLAN_MAX_BLOCKS * 256u);
+            break;
+        }
+        if (!o.segs || o.n_segs == 0 || !o.d_x) { rc = oxh_internal_errorf(OXH_ERR_ARG, "invalid argument: plan: operation %zu has no segments or no input", i); break; }
+        d.kind = kind;
+        if (kind == PLAN_Q5_K) has_q5 = true;
+        d.blocks = (uint32_t)(o.cols / OXH_QK_K);
+        d.magic = (uint32_t)((0x100000000ull + d.blocks - 1u) / d.blocks);
+        d.term_stride = d.blocks + 1u;
+        d.x = (gaddr)(uintptr_t)o.d_x;
+        d.act_out = (gaddr)(uintptr_t)o.d_act_out;
+        d.pro = GEMV_PRO_NONE;
+        if (o.pro) {
+            const OxhPrologue &p = *o.pro;
+            if ((p.kind != OXH_PRO_RMSNORM && p.kind != OXH_PRO_SWIGLU) || !p.d_b ||
+                ((p.d_add || p.d_sum_out) && p.kind != OXH_PRO_RMSNORM) || (p.d_sum_out && !p.d_add) ||
+                (p.kind == OXH_PRO_RMSNORM && !(p.eps >= 0.0f))) {
+                rc = oxh_internal_errorf(OXH_ERR_ARG, "invalid argument: plan: operation %zu has a malformed prologue", i);
+                break;
+            }
+            d.pro = p.kind == OXH_PRO_SWIGLU ? GEMV_PRO_SWIGLU : p.d_add ? GEMV_PRO_ADD_RMSNORM : GEMV_PRO_RMSNORM;
+            d.eps = p.eps;
+            d.pro_b = (gaddr)(uintptr_t)p.d_b;
+            d.pro_add = (gaddr)(uintptr_t)p.d_add;
+            d.pro_sum_out = (gaddr)(uintptr_t)p.d_sum_out;
+            d.pro_out = (gaddr)(uintptr_t)p.d_out;
+        }
+        /* segments with rows, at most four */
+        size_t rows[PLAN_MAX_SEGS];
+        int paired[PLAN_MAX_SEGS];
+        uint32_t ns = 0;
+        for (size_t k = 0; k < o.n_segs; k++) {
+            const OxhSegment &sg = o.segs[k];
+            if (sg.rows == 0) continue;
+            if (ns == PLAN_MAX_SEGS || !sg.d_w || !sg.d_out || sg.act_first != 0 || sg.n_vec > 1 ||
+                sg.rows > 0x3FFFFFFFull / (d.blocks * 16u)) {
+                rc = oxh_internal_errorf(OXH_ERR_ARG, "invalid argument: plan: operation %zu: at most four non-empty "
+                                         "segments, each over activation 0 with one vector", i);
+                break;
+            }
+            d.s[ns].w = (gaddr)(uintptr_t)sg.d_w;
+            d.s[ns].w2 = (gaddr)(uintptr_t)sg.d_w_pair;
+            d.s[ns].out = (gaddr)(uintptr_t)sg.d_out;
+            d.s[ns].rows = (uint32_t)sg.rows;
+            rows[ns] = sg.rows;
+            paired[ns] = sg.d_w_pair != nullptr;
+            ns++;
+        }
+        if (rc) break;
+        if (ns == 0) { rc = oxh_internal_errorf(OXH_ERR_ARG, "invalid argument: plan: operation %zu has no rows", i); break; }
+        d.n_segs = ns;
+        uint32_t n_wg[PLAN_MAX_SEGS], cap = 1;
+        const int drc = oxh_plan_deal(rows, paired, ns, grid, n_wg, &cap);
+        if (drc) { rc = oxh_internal_errorf(drc, "plan: operation %zu has more rows than %u workgroups can own", i, grid); break; }
+        d.rows_cap = cap;
+        uint32_t wg = 0;
+        for (uint32_t k = 0; k < ns; k++) {
+            const size_t waves = (size_t)n_wg[k] * PLAN_W;
+            d.s[k].wg_begin = wg;
+            d.s[k].rows_q = (uint32_t)(rows[k] / waves);
+            d.s[k].rows_rem = (uint32_t)(rows[k] % waves);
+            const uint32_t per_wg = (uint32_t)((rows[k] / waves + 1) * PLAN_W);
+            if (per_wg > max_wg_rows) max_wg_rows = per_wg;
+            wg += n_wg[k];
+        }
+        d.n_wg = wg;
+        const uint32_t act = kind == PLAN_Q6_K ? q8k6_lds_bytes(d.blocks) : q8k_lds_bytes(d.blocks);
+        if (act > max_act) max_act = act;
+        if (cap * d.term_stride > max_cap_terms) max_cap_terms = cap * d.term_stride;
+
+        /* what the operation reads and writes, for the dependency scan */
+        const size_t xb = o.cols * sizeof(float);
+        Span *r = reads + i * 4, *w = writes + i * 8;
+        r[0] = Span{ (const char *)o.d_x, xb };
+        if (o.pro) {
+            r[1] = Span{ (const char *)o.pro->d_b, xb };
+            r[2] = Span{ (const char *)o.pro->d_add, xb };
+            w[0] = Span{ (const char *)o.pro->d_out, xb };
+            w[1] = Span{ (const char *)o.pro->d_sum_out, xb };
+        }
+        w[2] = Span{ (const char *)o.d_act_out, o.cols / OXH_QK_K * OXH_Q8_K_BYTES };
+        for (uint32_t k = 0; k < ns; k++) w[3 + k] = Span{ (const char *)(uintptr_t)d.s[k].out, rows[k] * sizeof(float) };
+        /* a result stored by this operation over something it reads itself: every workgroup reads
+         * while one stores */
+        for (int a = 0; a < 8 && !rc; a++)
+            for (int b = 0; b < 4; b++)
+                if (spans_meet(w[a], r[b])) {
+                    rc = oxh_internal_errorf(OXH_ERR_ARG, "invalid argument: plan: operation %zu stores over one of its own inputs", i);
+                    break;
+                }
+        /* the latest earlier operation this one must not overtake: one that wrote what this reads or
+         * writes, or read what this writes */
+        uint32_t wait = 0;
+        for (size_t j = i; j-- > 0 && !wait;) {
+            const Span *rj = reads + j * 4, *wj = writes + j * 8;
+            bool hit = false;
+            for (int a = 0; a < 8 && !hit; a++) {
+                for (int b = 0; b < 4 && !hit; b++) hit = spans_meet(wj[a], r[b]) || spans_meet(w[a], rj[b]);
+                for (int b = 0; b < 8 && !hit; b++) hit = spans_meet(wj[a], w[b]);
+            }
+            if (hit) wait = (uint32_t)j + 1u;
+        }
+        d.wait = wait;
+        if (wait) { h[wait - 1].signal = 1; n_waits++; }
+    }
+    free(reads);
+    free(writes);
+    if (rc) { free(h); return rc; }
+
+    OxhPlan *pl = (OxhPlan *)calloc(1, sizeof *pl);
+    if (!pl) { free(h); return oxh_internal_errorf(OXH_ERR_NOMEM, "out of host memory building a plan"); }
+    pl->n_ops = (uint32_t)n_ops;
+    pl->grid = grid;
+    pl->n_waits = n_waits;
+    pl->has_q5 = has_q5;
+    pl->ld.act_bytes = (max_act + 15u) & ~15u;
+    pl->ld.outs_off = 2u * pl->ld.act_bytes;
+    pl->ld.red_off = pl->ld.outs_off + ((max_wg_rows * 4u + 15u) & ~15u);
+    pl->ld.terms_off = pl->ld.red_off + 128u;
+    pl->ld.terms_per_wave = max_cap_terms;
+    pl->lds_bytes = (size_t)pl->ld.terms_off + (size_t)PLAN_W * max_cap_terms * 4u;
+    const char *sl = getenv("OXH_PLAN_SPIN_LIMIT");
+    pl->spin_limit = sl && *sl ? (uint32_t)strtoul(sl, nullptr, 10) : 4000000u;
+    if (pl->lds_bytes > 160u * 1024u) {
+        free(h); free(pl);
+        return oxh_internal_errorf(OXH_ERR_TOO_WIDE, "plan: an operation's staged activation and row tables do not fit 160 KiB of LDS");
+    }
+    const void *kernel = has_q5 ? reinterpret_cast<const void *>(k_plan<true>) : reinterpret_cast<const void *>(k_plan<false>);
+    {
+        hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        if (e != hipSuccess) { free(h); free(pl); return oxh_internal_errorf(OXH_ERR_HIP, "HIP error in hipFuncSetAttribute: %s", hipGetErrorString(e)); }
+    }
+    /* every workgroup must be resident at once: one per compute unit fits by construction when the
+     * device can hold one workgroup of this kernel per unit */
+    int per_cu = 0;
+    hipError_t e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, 1024, pl->lds_bytes);
+    if (e != hipSuccess || per_cu < 1) {
+        free(h); free(pl);
+        return oxh_internal_errorf(OXH_ERR_HIP, "plan: the device cannot hold one workgroup of the plan kernel per compute unit");
+    }
+    e = hipMalloc((void **)&pl->d_ops, n_ops * sizeof(PlanOp));
+    if (e == hipSuccess) e = hipMalloc((void **)&pl->d_sync, (PLAN_MAX_WG + 8u) * sizeof(uint32_t));
+    if (e == hipSuccess) e = hipMemcpy(pl->d_ops, h, n_ops * sizeof(PlanOp), hipMemcpyHostToDevice);
+    if (e == hipSuccess) e = hipMemset(pl->d_sync, 0, (PLAN_MAX_WG + 8u) * sizeof(uint32_t));
+    if (e == hipSuccess) e = hipDeviceSynchronize();
+    free(h);
+    if (e != hipSuccess) {
+        if (pl->d_ops) (void)hipFree(pl->d_ops);
+        if (pl->d_sync) (void)hipFree(pl->d_sync);
+        free(pl);
+        return oxh_internal_errorf(e == hipErrorOutOfMemory ? OXH_ERR_NOMEM : OXH_ERR_HIP, "plan: %s", hipGetErrorString(e));
+    }
+    *out = pl;
+    return OXH_OK;
+}
+
+extern "C" int oxh_plan_launch(OxhPlan *pl, void *stream)
+{
+    if (!pl) return oxh_internal_errorf(OXH_ERR_ARG, "invalid argument: oxh_plan_launch: NULL plan");
+    hipStream_t st = stream ? (hipStream_t)stream : (hipStream_t)oxh_internal_stream();
+    PlanSync sy;
+    sy.flags = pl->d_sync;
+    sy.go = pl->d_sync + PLAN_MAX_WG + 4u;
+    sy.n_wait = pl->grid + pl->phantom;
+    sy.spin_limit = pl->spin_limit;
+    if (pl->has_q5)
+        hipLaunchKernelGGL(k_plan<true>, dim3(pl->grid), dim3(1024), pl->lds_bytes, st, (const PlanOp *)pl->d_ops,
+                           pl->n_ops, sy, pl->ld);
+    else
+        hipLaunchKernelGGL(k_plan<false>, dim3(pl->grid), dim3(1024), pl->lds_bytes, st, (const PlanOp *)pl->d_ops,
+                           pl->n_ops, sy, pl->ld);
+    PLAN_TRY(hipGetLastError());
+    return OXH_OK;
+}
+
+extern "C" int oxh_plan_info(const OxhPlan *pl, size_t *n_ops, size_t *n_waits, size_t *workgroups, size_t *lds_bytes)
+{
+    if (!pl) return oxh_internal_errorf(OXH_ERR_ARG, "invalid argument: oxh_plan_info: NULL plan");
+    if (n_ops) *n_ops = pl->n_ops;
+    if (n_waits) *n_waits = pl->n_waits;
+    if (workgroups) *workgroups = pl->grid;
+    if (lds_bytes) *lds_bytes = pl->lds_bytes;
+    return OXH_OK;
+}
+
+extern "C" int oxh_plan_set_spin_limit(OxhPlan *pl, uint32_t polls, int phantom_workgroup)
+{
+    if (!pl) return oxh_internal_errorf(OXH_ERR_ARG, "invalid argument: oxh_plan_set_spin_limit: NULL plan");
+    pl->spin_limit = polls;
+    pl->phantom = phantom_workgroup ? 1u : 0u;
+    return OXH_OK;
+}
+
+extern "C" int oxh_plan_status(OxhPlan *pl, void *stream)
+{
+    if (!pl) return oxh_internal_errorf(OXH_ERR_ARG, "invalid argument: oxh_plan_status: NULL plan");
+    hipStream_t st = stream ? (hipStream_t)stream : (hipStream_t)oxh_internal_stream();
+    PLAN_TRY(hipStreamSynchronize(st));
+    uint32_t go[4] = { 0, 0, 0, 0 };
+    PLAN_TRY(hipMemcpy(go, pl->d_sync + PLAN_MAX_WG + 4u, sizeof go, hipMemcpyDeviceToHost));
+    if (go[1] == 0u) return OXH_OK;
+    /* a wait ran out: the counters are no longer equal, start them afresh */
+    PLAN_TRY(hipMemset(pl->d_sync, 0, (PLAN_MAX_WG + 8u) * sizeof(uint32_t)));
+    PLAN_TRY(hipDeviceSynchronize());
+    return oxh_internal_errorf(OXH_ERR_TIMEOUT, "plan: a wait between operations ran out of polls (not every workgroup "
+                               "was resident, or the limit is too small); the launch's outputs are incomplete");
+}
+
+extern "C" int oxh_plan_destroy(OxhPlan *pl)
+{
+    if (!pl) return OXH_OK;
+    hipError_t e = hipDeviceSynchronize();
+    if (pl->d_ops) (void)hipFree(pl->d_ops);
+    if (pl->d_sync) (void)hipFree(pl->d_sync);
+    free(pl);
+    if (e != hipSuccess) return oxh_internal_errorf(OXH_ERR_HIP, "HIP error in hipDeviceSynchronize: %s", hipGetErrorString(e));
+    return OXH_OK;
+}

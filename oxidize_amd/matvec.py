@@ -255,6 +255,63 @@ def debug_subblock_sums(qtype, d_w, rows, cols, d_act, d_sums, stream=None):
                                         ctypes.c_void_p(d_act), ctypes.c_void_p(d_sums), stream))
 
 
+class Plan:
+    """A chain of decode matmuls compiled into one launch (oxh_plan_*).  `ops` is a list of dicts with the
+    arguments of one gemv_segments_fused call each: qtype, segs (from make_segments), cols, d_x and
+    optionally kind / d_b / eps / d_pro_out / d_add / d_sum_out (the prologue) and d_act_out."""
+
+    def __init__(self, ops):
+        n = len(ops)
+        self._keep = []
+        arr = (_lib.OxhPlanOp * n)()
+
+        def vp(a):
+            return None if a is None else ctypes.c_void_p(a)
+        for o, d in zip(arr, ops):
+            o.qtype = d["qtype"]
+            o.segs = ctypes.cast(d["segs"], ctypes.POINTER(OxhSegment))
+            o.n_segs = len(d["segs"])
+            o.cols = d["cols"]
+            o.d_x = d["d_x"]
+            if d.get("kind"):
+                pro = OxhPrologue(d["kind"], d.get("eps", 0.0), vp(d.get("d_b")), vp(d.get("d_pro_out")),
+                                  vp(d.get("d_add")), vp(d.get("d_sum_out")))
+                self._keep.append(pro)
+                o.pro = ctypes.pointer(pro)
+            o.d_act_out = d.get("d_act_out")
+            self._keep.append(d["segs"])
+        self.handle = ctypes.c_void_p()
+        status = lib().oxh_plan_create(arr, n, ctypes.byref(self.handle))
+        if status != OK:
+            raise OxhError(status, lib().oxh_last_error().decode("utf-8", "replace"))
+
+    def launch(self, stream=None):
+        check(lib().oxh_plan_launch(self.handle, stream))
+
+    def status(self, stream=None):
+        """Waits for the stream; 0, or ERR_TIMEOUT when a launch gave up."""
+        return lib().oxh_plan_status(self.handle, stream)
+
+    def info(self):
+        v = [ctypes.c_size_t() for _ in range(4)]
+        check(lib().oxh_plan_info(self.handle, *[ctypes.byref(x) for x in v]))
+        return dict(zip(("n_ops", "n_waits", "workgroups", "lds_bytes"), [int(x.value) for x in v]))
+
+    def set_spin_limit(self, polls, phantom_workgroup=False):
+        check(lib().oxh_plan_set_spin_limit(self.handle, polls, int(phantom_workgroup)))
+
+    def destroy(self):
+        if self.handle:
+            lib().oxh_plan_destroy(self.handle)
+            self.handle = ctypes.c_void_p()
+
+    def __del__(self):
+        try:
+            self.destroy()
+        except Exception:
+            pass
+
+
 def sync(stream=None):
     check(lib().oxh_stream_sync(stream))
 

@@ -101,6 +101,16 @@ class DecodeSet:
             for op in range(len(self.ops)):
                 self.launch_op(layer, op, stream, fused)
 
+    def plan_ops(self):
+        """The step as the operation list of one persistent launch (mv.Plan): the same calls as
+        launch_step(fused=True), in the same order."""
+        ops = []
+        for layer in range(self.layers):
+            for op, (name, qt, rows, cols, _) in enumerate(self.ops):
+                ops.append(dict(qtype=qt, segs=self.segments[layer][op], cols=cols, d_x=self.x[layer][op].ptr,
+                                d_act_out=self.act[layer][op].ptr))
+        return ops
+
     def output(self, layer, op):
         rows = sum(self.ops[op][2])
         return self.out[layer][op].download(np.float32, rows)
@@ -173,6 +183,29 @@ class DecodeChain:
         h, kv, ffn = d.hidden, d.kv, d.ffn
         per_layer = 4 * ((3 * h + h + (h + 2 * kv)) + (h + h) + (3 * h + h + ffn) + (ffn + h))
         return d.weight_bytes + d.layers * per_layer
+
+    def plan_ops(self):
+        """launch_step's calls as the operation list of one persistent launch (mv.Plan); no per-stage
+        copies (capture must be off)."""
+        assert not self.capture
+        d = self.d
+        h = d.hidden
+        x, f = self.x0, self.f0
+        turn = 0
+        ops = []
+        for l in range(d.layers):
+            sg = self.segs[l]
+            x1, x2 = self.res[turn % 3], self.res[(turn + 1) % 3]
+            turn += 2
+            ops.append(dict(qtype=Q4K, segs=sg["qkv"], cols=h, d_x=x.ptr, kind=mv.PRO_RMSNORM, d_b=self.g_attn[l].ptr,
+                            eps=self.eps, d_add=f.ptr, d_sum_out=x1.ptr))
+            ops.append(dict(qtype=Q4K, segs=sg["o"], cols=h, d_x=self.qkv.ptr))
+            ops.append(dict(qtype=Q4K, segs=sg["gate_up"], cols=h, d_x=x1.ptr, kind=mv.PRO_RMSNORM,
+                            d_b=self.g_ffn[l].ptr, eps=self.eps, d_add=self.o.ptr, d_sum_out=x2.ptr))
+            ops.append(dict(qtype=Q6K, segs=sg["down"], cols=d.ffn, d_x=self.h.ptr))
+            x, f = x2, self.f
+        self.last_x = x
+        return ops
 
     def launch_step(self, stream=None):
         d = self.d

@@ -184,3 +184,31 @@ def test_weight_stats_and_unregister_need_no_device():
     assert lib.oxh_init(0) != 0 or True
     buf = np.zeros(64, np.uint8)
     assert lib.oxh_weight_unregister(buf.ctypes.data) == 0      # nothing there: not an error
+
+
+def test_plan_deals_rows_within_the_grid():
+    """How a plan spreads an operation's rows over the device is host arithmetic: never more workgroups
+    than the grid, every segment served, no wave beyond 32 table rows."""
+    lib = _lib.lib()
+
+    def deal(rows, paired, grid):
+        n = len(rows)
+        r = (ctypes.c_size_t * n)(*rows)
+        p = (ctypes.c_int * n)(*paired)
+        wg = (ctypes.c_uint32 * n)()
+        cap = ctypes.c_uint32()
+        rc = lib.oxh_plan_deal(r, p, n, grid, wg, ctypes.byref(cap))
+        return rc, list(wg), cap.value
+
+    rc, wg, cap = deal([4096, 1024, 1024], [0, 0, 0], 256)       # q/k/v: plain rounding would take 257
+    assert rc == 0 and sum(wg) <= 256 and wg[1] == wg[2] == 43 and wg[0] in (170, 171) and cap == 2
+    rc, wg, cap = deal([14336], [1], 256)                        # gate/up pair: 3.5 rows per wave, both matrices
+    assert rc == 0 and wg == [256] and cap == 8
+    rc, wg, cap = deal([4096], [0], 256)
+    assert rc == 0 and wg == [256] and cap == 1
+    rc, wg, cap = deal([100], [0], 256)                          # fewer rows than waves: 7 workgroups are enough
+    assert rc == 0 and wg == [7] and cap == 1
+    rc, wg, cap = deal([7, 9000, 3], [0, 0, 0], 304)
+    assert rc == 0 and sum(wg) <= 304 and min(wg) >= 1
+    assert deal([1 << 20], [0], 256)[0] == _lib.ERR_TOO_WIDE     # 256 rows per wave: beyond the table
+    assert deal([0], [0], 256)[0] == _lib.ERR_ARG

@@ -1,0 +1,154 @@
+"""A decode step as one persistent launch (oxh_plan_*) against the same matmuls launched one by one
+(oxh_gemv_segments_fused / _f32, themselves held to the oracle elsewhere): every output, every stored
+quantised activation and the residual stream must be bit-identical, launch after launch; and the bounded
+wait between dependent operations must give up cleanly when it cannot be satisfied."""
+import ctypes
+
+import numpy as np
+import pytest
+
+import oxlibs
+from oxidize_amd import _lib, synth
+from oxidize_amd import matvec as mv
+from oxidize_amd.workloads import DecodeChain, DecodeSet
+
+pytestmark = pytest.mark.gpu
+Q80, Q4K, Q5K, Q6K = 7, 13, 15, 16
+
+
+def bits(a):
+    return np.ascontiguousarray(a).view(np.uint32)
+
+
+@pytest.mark.parametrize("hidden,kv,ffn,layers", [(1024, 256, 2816, 3), (4096, 1024, 14336, 2), (256, 256, 512, 5)])
+def test_independent_set_matches_single_launches_and_oracle(oxh, hidden, kv, ffn, layers):
+    d = DecodeSet(hidden=hidden, kv=kv, ffn=ffn, layers=layers, seed=3, keep_host=(0,))
+    d.launch_step()
+    mv.sync()
+    want_out = [[d.output(l, op) for op in range(4)] for l in range(layers)]
+    want_act = [[d.activation(l, op) for op in range(4)] for l in range(layers)]
+    for l in range(layers):
+        for op in range(4):
+            mv.lib().oxh_memset(ctypes.c_void_p(d.out[l][op].ptr), 0xFF, d.out[l][op].nbytes, None)
+            mv.lib().oxh_memset(ctypes.c_void_p(d.act[l][op].ptr), 0xFF, d.act[l][op].nbytes, None)
+    plan = mv.Plan(d.plan_ops())
+    info = plan.info()
+    assert info["n_ops"] == 4 * layers and info["n_waits"] == 0      # nothing depends on anything here
+    for rep in range(2):
+        plan.launch()
+        assert plan.status() == 0
+        for l in range(layers):
+            for op in range(4):
+                assert np.array_equal(bits(d.output(l, op)), bits(want_out[l][op])), (rep, l, op)
+                assert np.array_equal(d.activation(l, op), want_act[l][op]), (rep, l, op)
+    # and one matrix against the oracle directly
+    o = oxlibs.oracle()
+    name, qt, rows, cols, _ = d.ops[3]
+    w, x = d.host[(0, 3, 0)], d.x_host[(0, 3)]
+    want = np.zeros(rows[0], np.float32)
+    tmp = np.zeros(cols, np.float32)
+    assert o.oxo_matvec_quantized(qt, w.ctypes.data, rows[0], cols, synth.row_bytes(qt, cols), x.ctypes.data,
+                                  want.ctypes.data, tmp.ctypes.data) == 0
+    assert np.array_equal(bits(d.output(0, 3)), bits(want))
+    plan.destroy()
+
+
+def chain_state(c):
+    d = c.d
+    return dict(qkv=c.qkv.download(np.float32, d.hidden + 2 * d.kv), o=c.o.download(np.float32, d.hidden),
+                h=c.h.download(np.float32, d.ffn), f=c.f.download(np.float32, d.hidden),
+                x=c.last_x.download(np.float32, d.hidden),
+                res=[r.download(np.float32, d.hidden) for r in c.res])
+
+
+@pytest.mark.parametrize("hidden,kv,ffn,layers", [(1024, 256, 2816, 4), (4096, 1024, 14336, 3)])
+def test_dependent_chain_matches_single_launches(oxh, hidden, kv, ffn, layers):
+    d = DecodeSet(hidden=hidden, kv=kv, ffn=ffn, layers=layers, seed=5)
+    a, b = DecodeChain(d, seed=5), DecodeChain(d, seed=5)
+    a.launch_step()
+    mv.sync()
+    want = chain_state(a)
+    assert np.all(np.isfinite(want["x"])) and float(np.abs(want["f"]).max()) > 0
+    plan = mv.Plan(b.plan_ops())
+    info = plan.info()
+    assert info["n_ops"] == 4 * layers
+    assert info["n_waits"] == 4 * layers - 1          # every operation but the first reads its predecessor's output
+    for rep in range(3):                              # the progress counters carry over from launch to launch
+        plan.launch()
+        assert plan.status() == 0
+        got = chain_state(b)
+        for k in ("qkv", "o", "h", "f", "x"):
+            assert np.array_equal(bits(got[k]), bits(want[k])), (rep, k)
+        for i in range(3):
+            assert np.array_equal(bits(got["res"][i]), bits(want["res"][i])), (rep, i)
+    # replayed from a graph, with eager work in between
+    with mv.Graph() as g:
+        plan.launch()
+    for rep in range(3):
+        mv.lib().oxh_memset(ctypes.c_void_p(b.f.ptr), 0, b.f.nbytes, None)
+        g.launch()
+        assert plan.status() == 0
+        got = chain_state(b)
+        assert np.array_equal(bits(got["f"]), bits(want["f"])) and np.array_equal(bits(got["x"]), bits(want["x"]))
+    plan.destroy()
+
+
+def test_mixed_types_with_q5k(oxh):
+    """Q5_K operations take the kernel variant that carries the fifth-bit plane."""
+    hidden, rows = 1024, 700
+    xs = [mv.DeviceBuffer.from_host(synth.normal(hidden, seed=9, stream=i)) for i in range(3)]
+    ws, outs, ops, host = [], [], [], []
+    for i, qt in enumerate((Q5K, Q4K, Q6K)):
+        w = synth.weights(qt, rows, hidden, seed=9, stream=10 + i)
+        host.append(w)
+        ws.append(mv.DeviceBuffer.from_host(w))
+        outs.append(mv.DeviceBuffer(rows * 4))
+        ops.append(dict(qtype=qt, segs=mv.make_segments([(ws[i].ptr, outs[i].ptr, rows, 0)]), cols=hidden,
+                        d_x=xs[i].ptr))
+    plan = mv.Plan(ops)
+    plan.launch()
+    assert plan.status() == 0
+    o = oxlibs.oracle()
+    for i, qt in enumerate((Q5K, Q4K, Q6K)):
+        x = synth.normal(hidden, seed=9, stream=i)
+        want = np.zeros(rows, np.float32)
+        tmp = np.zeros(hidden, np.float32)
+        assert o.oxo_matvec_quantized(qt, host[i].ctypes.data, rows, hidden, synth.row_bytes(qt, hidden),
+                                      x.ctypes.data, want.ctypes.data, tmp.ctypes.data) == 0
+        assert np.array_equal(bits(outs[i].download(np.float32, rows)), bits(want)), qt
+
+
+def test_a_wait_that_cannot_be_satisfied_gives_up(oxh):
+    """The waits expect one workgroup more than exist and may poll 300 times: every workgroup must leave,
+    the launch must end, the status must say so, and the plan must work again afterwards."""
+    d = DecodeSet(hidden=1024, kv=256, ffn=2816, layers=2, seed=7)
+    a, b = DecodeChain(d, seed=7), DecodeChain(d, seed=7)
+    a.launch_step()
+    mv.sync()
+    want = chain_state(a)
+    plan = mv.Plan(b.plan_ops())
+    plan.set_spin_limit(300, phantom_workgroup=True)
+    plan.launch()
+    assert plan.status() == _lib.ERR_TIMEOUT
+    assert b"ran out of polls" in oxh.oxh_last_error()
+    plan.set_spin_limit(4000000, phantom_workgroup=False)
+    for rep in range(2):
+        plan.launch()
+        assert plan.status() == 0
+        got = chain_state(b)
+        assert np.array_equal(bits(got["f"]), bits(want["f"])) and np.array_equal(bits(got["x"]), bits(want["x"]))
+
+
+def test_what_a_plan_declines(oxh):
+    x = mv.DeviceBuffer(4 * 32768)
+    w = mv.DeviceBuffer(1 << 20)
+    out = mv.DeviceBuffer(4 * 64)
+    seg = mv.make_segments([(w.ptr, out.ptr, 8, 0)])
+    for qt, cols in ((Q80, 1024), (Q4K, 32768), (Q4K, 1000)):
+        with pytest.raises(mv.OxhError) as e:
+            mv.Plan([dict(qtype=qt, segs=seg, cols=cols, d_x=x.ptr)])
+        assert e.value.status == mv.DECLINED
+    # an operation storing over its own input
+    with pytest.raises(mv.OxhError) as e:
+        mv.Plan([dict(qtype=Q4K, segs=mv.make_segments([(w.ptr, x.ptr, 8, 0)]), cols=1024, d_x=x.ptr)])
+    assert e.value.status == _lib.ERR_ARG
