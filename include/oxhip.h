@@ -256,6 +256,12 @@ int oxh_plan_info(const OxhPlan *plan, size_t *n_ops, size_t *n_waits, size_t *w
  * the way to test the give-up path without hanging anything. */
 int oxh_plan_set_spin_limit(OxhPlan *plan, uint32_t polls, int phantom_workgroup);
 int oxh_plan_destroy(OxhPlan *plan);
+/* Measurement aid: with d_stamps set (n_ops * workgroups * 8 uint64 of device
+ * memory, or NULL to switch it off) wave 0 of every workgroup stores the shader
+ * clock at eight points of every operation: start, dependency met, activation
+ * staged, workgroup barrier passed, passes done, rows summed, barrier passed,
+ * outputs stored and announced.  No counterpart in the reference. */
+int oxh_debug_plan_stamps(OxhPlan *plan, uint64_t *d_stamps);
 /* How a plan deals the rows of one operation's segments to `grid` workgroups of
  * sixteen waves (pure host arithmetic): workgroups per segment and the most
  * table rows any wave owns (a paired segment counts two per row). */

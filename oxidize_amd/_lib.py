@@ -69,6 +69,7 @@ SIGNATURES = {
     "oxh_plan_info": (I, [V, ctypes.POINTER(Z), ctypes.POINTER(Z), ctypes.POINTER(Z), ctypes.POINTER(Z)]),
     "oxh_plan_set_spin_limit": (I, [V, U32, I]),
     "oxh_plan_destroy": (I, [V]),
+    "oxh_debug_plan_stamps": (I, [V, V]),
     "oxh_plan_deal": (I, [ctypes.POINTER(Z), ctypes.POINTER(I), Z, U32, ctypes.POINTER(U32), ctypes.POINTER(U32)]),
     "oxh_mmq": (I, [U32, V, Z, Z, V, Z, V, Z, V]),
     "oxh_get_rows": (I, [U32, V, Z, Z, V, Z, V, Z, V]),

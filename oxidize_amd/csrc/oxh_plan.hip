@@ -86,7 +86,17 @@ struct PlanSync {
     uint32_t *go;
     uint32_t n_wait;                /* counters gathered: the grid size (one more in the time-out test) */
     uint32_t spin_limit;
+    uint64_t *stamps;               /* measurement aid: [op][workgroup][8] clock readings, or NULL */
 };
+
+#define PLAN_STAMPS 8u
+
+/* wave 0 of a workgroup notes the shader clock at phase `slot` of operation `op` */
+__device__ __forceinline__ void plan_stamp(const PlanSync &sy, uint32_t op, uint32_t slot, uint32_t lane, uint32_t wave)
+{
+    if (sy.stamps != nullptr && wave == 0u && lane == 0u)
+        sy.stamps[((size_t)op * gridDim.x + blockIdx.x) * PLAN_STAMPS + slot] = __builtin_readcyclecounter();
+}
 
 struct PlanLds {
     uint32_t act_bytes;             /* one staged activation (two are kept, used in turn) */
@@ -162,7 +172,7 @@ struct PWork {
     uint32_t nblk, nrows, row0;
     uint32_t wg_row0, wg_rows;      /* the workgroup's contiguous run of rows */
     uint32_t kind;
-    bool paired;
+    uint32_t paired;                /* 0 / 1 (a whole word: the struct is copied around as scalars) */
 };
 
 __device__ __forceinline__ uint32_t plan_block_bytes(uint32_t kind)
@@ -198,7 +208,7 @@ __device__ __forceinline__ PWork plan_work(const PlanOp *__restrict__ op, uint32
     const size_t off = (size_t)(k.nrows ? k.row0 : 0u) * B * plan_block_bytes(k.kind);
     k.src.a = gptr<const uint8_t>(w + off);
     k.src.n1 = k.nrows * B;
-    k.paired = w2 != 0u;
+    k.paired = w2 != 0u ? 1u : 0u;
     k.src.b = gptr<const uint8_t>((k.paired ? w2 : w) + off);
     k.nblk = k.paired ? 2u * k.src.n1 : k.src.n1;
     return k;
@@ -237,13 +247,12 @@ __device__ __forceinline__ void wset_load(uint32_t kind, WSet &s, const WSrc &sr
     if (HAS_Q5) s.e = v4;
 }
 
+/* pass `pass` (0 or 1) of an operation into a register set */
 template <bool HAS_Q5>
-__device__ __forceinline__ void plan_prefetch(const PWork &k, WSet &A, WSet &B, uint32_t lane)
+__device__ __forceinline__ void plan_prefetch(const PWork &k, WSet &S, uint32_t pass, uint32_t lane)
 {
     if (k.nblk == 0u) return;
-    const uint32_t last = k.nblk - 1u;
-    wset_load<HAS_Q5>(k.kind, A, k.src, min(lane >> 2, last), lane);
-    wset_load<HAS_Q5>(k.kind, B, k.src, min(16u + (lane >> 2), last), lane);
+    wset_load<HAS_Q5>(k.kind, S, k.src, min(pass * 16u + (lane >> 2), k.nblk - 1u), lane);
 }
 
 /* ─── the passes of one operation (sets A and B hold passes 0 and 1) ──── */
@@ -326,38 +335,59 @@ plan_row_sums(const float *terms, const PWork &k, uint32_t B, uint32_t term_stri
 
 /* ─── activation staging: one f32 vector -> Q8_K in LDS ──────────────── */
 
-/* The vector may have been written by another workgroup a moment ago: it is read with coherent
- * loads, and so is everything else an operation can have produced (the added vector, SwiGLU's
- * second operand).  Norm weights are constants.  Arithmetic and order are stage_begin / stage_end's
- * for one vector and sixteen waves, so the quantised bytes are the same. */
-template <int KIND /* 0 Q4_K/Q5_K layout, 1 Q6_K layout */, int PRO>
-__device__ __forceinline__ void
-plan_stage(const PlanOp *__restrict__ op, uint8_t *base, float *red, bool storer, uint32_t lane, uint32_t wave)
+/* Staging is split in two so that the loads can be placed where they hurt least in the wave's
+ * in-order memory queue: plan_stage_issue asks for this wave's (up to four) 256-value units of the
+ * input vector and of whatever the prologue combines it with; plan_stage_finish applies the prologue,
+ * quantises and writes LDS.  A vector another workgroup wrote a moment ago is read with coherent
+ * loads; inputs nobody in this launch wrote come through the caches.  Arithmetic and order are
+ * stage_begin / stage_end's for one vector and sixteen waves, so the quantised bytes are the same. */
+struct XStage {
+    XRegs x[4], t[4], b[4];
+};
+
+__device__ __forceinline__ XRegs load4_either(bool coherent, const float *base, CohBuf cb, uint32_t at)
 {
-    constexpr bool RMS = PRO == GEMV_PRO_RMSNORM || PRO == GEMV_PRO_ADD_RMSNORM;
-    constexpr bool ADD = PRO == GEMV_PRO_ADD_RMSNORM;
-    const uint32_t B = op->blocks;
-    const CohBuf x = coh_buf(gptr<const float>(op->x)), add = coh_buf(gptr<const float>(op->pro_add));
-    const CohBuf bc = coh_buf(gptr<const float>(op->pro_b));
-    const float *b = gptr<const float>(op->pro_b);
-    XRegs xr[4], br[4];
+    if (coherent) return cload4(cb, at * 4u);
+    return x_load4(base + at);
+}
+
+__device__ __forceinline__ void
+plan_stage_issue(const PlanOp *__restrict__ op, XStage &xs, bool coherent, uint32_t lane, uint32_t wave)
+{
+    const uint32_t B = op->blocks, pro = op->pro;
+    const float *x = gptr<const float>(op->x), *add = gptr<const float>(op->pro_add), *b = gptr<const float>(op->pro_b);
+    const CohBuf xc = coh_buf(x), ac = coh_buf(add), bc = coh_buf(b);
 #pragma unroll
     for (int i = 0; i < 4; i++) {
         const uint32_t unit = wave + PLAN_W * (uint32_t)i;
-        xr[i] = br[i] = XRegs{ 0.f, 0.f, 0.f, 0.f };
         if (unit < B) {
             const uint32_t at = unit * 256u + 4u * lane;
-            xr[i] = cload4(x, at * 4u);
-            if (ADD) {
-                const XRegs t = cload4(add, at * 4u);
-                xr[i].v0 += t.v0; xr[i].v1 += t.v1; xr[i].v2 += t.v2; xr[i].v3 += t.v3;
-            }
-            if (PRO == GEMV_PRO_SWIGLU) br[i] = cload4(bc, at * 4u);
-            else if (RMS) br[i] = x_load4(b + at);
+            xs.x[i] = load4_either(coherent, x, xc, at);
+            if (pro == GEMV_PRO_ADD_RMSNORM) xs.t[i] = load4_either(coherent, add, ac, at);
+            if (pro == GEMV_PRO_SWIGLU) xs.b[i] = load4_either(coherent, b, bc, at);
+            else if (pro != GEMV_PRO_NONE) xs.b[i] = x_load4(b + at);        /* norm weights: constants */
         }
     }
+}
+
+/* One instantiation per staged layout: what the prologue does is decided at run time (the branches are
+ * uniform and the float expressions are prologue_apply's), so that the quantiser is inlined twice, not
+ * eight times. */
+template <int KIND /* 0 Q4_K/Q5_K layout, 1 Q6_K layout */>
+__device__ __forceinline__ void
+plan_stage_finish(const PlanOp *__restrict__ op, const XStage &xs, uint8_t *base, float *red, bool storer,
+                  uint32_t lane, uint32_t wave)
+{
+    const uint32_t B = op->blocks, pro = op->pro;
+    const bool rms = pro == GEMV_PRO_RMSNORM || pro == GEMV_PRO_ADD_RMSNORM, add = pro == GEMV_PRO_ADD_RMSNORM;
+    XRegs xr[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        xr[i] = xs.x[i];
+        if (add) { xr[i].v0 += xs.t[i].v0; xr[i].v1 += xs.t[i].v1; xr[i].v2 += xs.t[i].v2; xr[i].v3 += xs.t[i].v3; }
+    }
     float inv = 1.0f;
-    if (RMS) {
+    if (rms) {
         float ss = 0.0f;
 #pragma unroll
         for (int i = 0; i < 4; i++)
@@ -369,8 +399,8 @@ plan_stage(const PlanOp *__restrict__ op, uint8_t *base, float *red, bool storer
         const float tot = wave_sum_f32(lane < PLAN_W ? red[lane] : 0.0f);
         inv = 1.0f / sqrtf(tot / (float)(B * 256u) + op->eps);
     }
-    const bool has_sout = ADD && storer && op->pro_sum_out != 0u;
-    const bool has_fout = PRO != GEMV_PRO_NONE && storer && op->pro_out != 0u;
+    const bool has_sout = add && storer && op->pro_sum_out != 0u;
+    const bool has_fout = pro != GEMV_PRO_NONE && storer && op->pro_out != 0u;
     const CohBuf sout = coh_buf(gptr<float>(op->pro_sum_out)), fout = coh_buf(gptr<float>(op->pro_out));
     uint8_t *gout = (storer && op->act_out) ? gptr<uint8_t>(op->act_out) : nullptr;
 #pragma unroll
@@ -379,7 +409,9 @@ plan_stage(const PlanOp *__restrict__ op, uint8_t *base, float *red, bool storer
         if (unit < B) {
             const uint32_t at = unit * 256u + 4u * lane;
             if (has_sout) cstore4(sout, at * 4u, xr[i]);
-            const XRegs y = prologue_apply<PRO>(xr[i], br[i], inv);
+            XRegs y = xr[i];
+            if (rms) y = prologue_apply<GEMV_PRO_RMSNORM>(xr[i], xs.b[i], inv);
+            else if (pro == GEMV_PRO_SWIGLU) y = prologue_apply<GEMV_PRO_SWIGLU>(xr[i], xs.b[i], inv);
             if (has_fout) cstore4(fout, at * 4u, y);
             q8k_x_finish<KIND == 1>(y, B, unit, base, gout, lane);
         }
@@ -387,18 +419,6 @@ plan_stage(const PlanOp *__restrict__ op, uint8_t *base, float *red, bool storer
     /* what this workgroup stored for later operations has to be complete before it announces the
      * operation done; the only loads in flight here are the first passes' weights, needed next anyway */
     if (has_sout || has_fout) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-}
-
-template <int KIND>
-__device__ __forceinline__ void
-plan_stage_any(const PlanOp *__restrict__ op, uint8_t *base, float *red, bool storer, uint32_t lane, uint32_t wave)
-{
-    switch (op->pro) {
-    case GEMV_PRO_RMSNORM:     plan_stage<KIND, GEMV_PRO_RMSNORM>(op, base, red, storer, lane, wave); break;
-    case GEMV_PRO_ADD_RMSNORM: plan_stage<KIND, GEMV_PRO_ADD_RMSNORM>(op, base, red, storer, lane, wave); break;
-    case GEMV_PRO_SWIGLU:      plan_stage<KIND, GEMV_PRO_SWIGLU>(op, base, red, storer, lane, wave); break;
-    default:                   plan_stage<KIND, GEMV_PRO_NONE>(op, base, red, storer, lane, wave); break;
-    }
 }
 
 /* ─── waiting for an operation to be complete on every workgroup ──────── */
@@ -464,22 +484,76 @@ k_plan(const PlanOp *__restrict__ ops, uint32_t n_ops, const PlanSync sy, const 
     int *const s_ok = reinterpret_cast<int *>(red + 24);      /* the reduction uses slots 0..15 of 32 */
     float *const terms = reinterpret_cast<float *>(lds + ld.terms_off) + (size_t)wave * ld.terms_per_wave;
 
+    /* The loop is cut between an operation's last pass and its row sums: at that point no load is in
+     * flight and no weight or input register holds anything, so nothing but scalars crosses the loop
+     * boundary.  One trip = (rows, outputs and announcement of operation i - 1), then requests,
+     * staging and passes of operation i. */
     PWork cur = plan_work(&ops[0], wave);
-    WSet A, B;
-    A.a = A.b = A.c = A.d = A.e = u32x4{ 0u, 0u, 0u, 0u };
-    B.a = B.b = B.c = B.d = B.e = A.a;
-    plan_prefetch<HAS_Q5>(cur, A, B, lane);
+    PWork prev = cur;
+    for (uint32_t i = 0;; i++) {
+        /* The lane index, made opaque once per trip: everything derived from it (sub-block masks, LDS
+         * slots, byte offsets) is then recomputed per operation in a handful of instructions instead of
+         * being kept alive across the whole loop, which costs more registers than this kernel has. */
+        uint32_t ln = lane;
+        asm volatile("" : "+v"(ln));
+        if (i > 0u) {
+            const PlanOp *po = &ops[i - 1u];
+            /* Rows first, then the workgroup's outputs go out, then (below) the requests for the next
+             * operation: those queue up in the memory pipeline (a compute unit takes in about 12 bytes
+             * per cycle), and anything placed after them in program order waits for that queue. */
+            plan_row_sums(terms, prev, po->blocks, po->term_stride, outs, ln);
+            plan_stamp(sy, i - 1u, 5, ln, wave);
+            lds_barrier();
+            plan_stamp(sy, i - 1u, 6, ln, wave);
+            if (wave == 0u) {
+                const CohBuf dst = coh_buf(prev.out + prev.wg_row0);
+                for (uint32_t r = ln; r < prev.wg_rows; r += 64u) cstore_f32(dst, r * 4u, outs[r]);
+                if (po->signal != 0u || i == n_ops) {
+                    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                    /* the last operation leaves every counter at base + n_ops + 1, the next launch's base */
+                    if (ln == 0u) cstore(sy.flags + blockIdx.x, base + i + (i == n_ops ? 1u : 0u));
+                }
+            }
+            plan_stamp(sy, i - 1u, 7, ln, wave);
+        }
+        if (i == n_ops) break;
 
-    for (uint32_t i = 0; i < n_ops; i++) {
         const PlanOp *op = &ops[i];
         uint8_t *act = lds + (size_t)(i & 1u) * ld.act_bytes;
-        if (op->wait != 0u && !plan_wait(sy, base + op->wait, s_ok, lane, wave)) return;
+        plan_stamp(sy, i, 0, ln, wave);
+        /* Loads complete in the order a wave issued them, so the order of the requests is the
+         * schedule.  An operation that depends on nothing gets its input vector requested first and
+         * both weight sets behind it; one that has to wait gets one set before the wait (that is
+         * what streams in while the wait lasts), then the input vector, then the second set. */
+        WSet A, B;
+        A.a = A.b = A.c = A.d = A.e = u32x4{ 0u, 0u, 0u, 0u };
+        B.a = B.b = B.c = B.d = B.e = A.a;
+        XStage xs;
+#pragma unroll
+        for (int u = 0; u < 4; u++) xs.x[u] = xs.t[u] = xs.b[u] = XRegs{ 0.f, 0.f, 0.f, 0.f };
+        if (op->wait == 0u) {
+            plan_stage_issue(op, xs, false, ln, wave);
+            plan_prefetch<HAS_Q5>(cur, A, 0u, ln);
+            plan_prefetch<HAS_Q5>(cur, B, 1u, ln);
+        } else {
+            plan_prefetch<HAS_Q5>(cur, A, 0u, ln);
+            if (!plan_wait(sy, base + op->wait, s_ok, ln, wave)) return;
+            plan_stage_issue(op, xs, true, ln, wave);
+            plan_prefetch<HAS_Q5>(cur, B, 1u, ln);
+        }
+        plan_stamp(sy, i, 1, ln, wave);
+        /* what this wave owns of the next operation: read from the table now, so that the table's
+         * trip from memory is over long before the passes end */
+        PWork nx = cur;
+        if (i + 1u < n_ops) nx = plan_work(&ops[i + 1u], wave);
 
         const bool storer = blockIdx.x == 0u;
         const uint32_t Bk = op->blocks;
-        if (op->kind == PLAN_Q6_K) plan_stage_any<1>(op, act, red, storer, lane, wave);
-        else                       plan_stage_any<0>(op, act, red, storer, lane, wave);
+        if (op->kind == PLAN_Q6_K) plan_stage_finish<1>(op, xs, act, red, storer, ln, wave);
+        else                       plan_stage_finish<0>(op, xs, act, red, storer, ln, wave);
+        plan_stamp(sy, i, 2, ln, wave);
         __syncthreads();
+        plan_stamp(sy, i, 3, ln, wave);
 
         GemvParams gp;
         gp.blocks = Bk;
@@ -488,32 +562,12 @@ k_plan(const PlanOp *__restrict__ ops, uint32_t n_ops, const PlanSync sy, const 
         gp.rows_cap = op->rows_cap;
         gp.dump = nullptr;
         if (cur.nblk != 0u) {
-            if (cur.kind == PLAN_Q6_K)      plan_passes_q6(A, B, cur, gp, act, q8k6_lds_bytes(Bk), terms, lane);
-            else if (HAS_Q5 && cur.kind == PLAN_Q5_K) plan_passes_q45<true>(A, B, cur, gp, act, q8k_lds_bytes(Bk), terms, lane);
-            else                            plan_passes_q45<false>(A, B, cur, gp, act, q8k_lds_bytes(Bk), terms, lane);
+            if (cur.kind == PLAN_Q6_K)      plan_passes_q6(A, B, cur, gp, act, q8k6_lds_bytes(Bk), terms, ln);
+            else if (HAS_Q5 && cur.kind == PLAN_Q5_K) plan_passes_q45<true>(A, B, cur, gp, act, q8k_lds_bytes(Bk), terms, ln);
+            else                            plan_passes_q45<false>(A, B, cur, gp, act, q8k_lds_bytes(Bk), terms, ln);
         }
-
-        /* registers are free: the next operation's first weights, before this one's rows are summed.
-         * Wave 0 asks later: it has to see its output stores complete first, and a wait for them
-         * would wait for these loads too. */
-        const bool more = i + 1u < n_ops;
-        PWork nx = cur;
-        if (more) {
-            nx = plan_work(&ops[i + 1u], wave);
-            if (wave != 0u) plan_prefetch<HAS_Q5>(nx, A, B, lane);
-        }
-        plan_row_sums(terms, cur, Bk, op->term_stride, outs, lane);
-        lds_barrier();
-        if (wave == 0u) {
-            const CohBuf dst = coh_buf(cur.out + cur.wg_row0);
-            for (uint32_t r = lane; r < cur.wg_rows; r += 64u) cstore_f32(dst, r * 4u, outs[r]);
-            if (op->signal != 0u || !more) {
-                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-                /* the last operation leaves every counter at base + n_ops + 1, the next launch's base */
-                if (lane == 0u) cstore(sy.flags + blockIdx.x, base + i + 1u + (more ? 0u : 1u));
-            }
-            if (more) plan_prefetch<HAS_Q5>(nx, A, B, lane);
-        }
+        plan_stamp(sy, i, 4, ln, wave);
+        prev = cur;
         cur = nx;
     }
 }
@@ -528,6 +582,7 @@ struct OxhPlan {
     size_t lds_bytes;
     uint32_t spin_limit, phantom;
     bool has_q5;
+    uint64_t *d_stamps;
     uint32_t n_waits;               /* operations that wait (for callers' curiosity) */
 };
 
@@ -782,6 +837,7 @@ extern "C" int oxh_plan_launch(OxhPlan *pl, void *stream)
     sy.go = pl->d_sync + PLAN_MAX_WG + 4u;
     sy.n_wait = pl->grid + pl->phantom;
     sy.spin_limit = pl->spin_limit;
+    sy.stamps = pl->d_stamps;
     if (pl->has_q5)
         hipLaunchKernelGGL(k_plan<true>, dim3(pl->grid), dim3(1024), pl->lds_bytes, st, (const PlanOp *)pl->d_ops,
                            pl->n_ops, sy, pl->ld);
@@ -807,6 +863,13 @@ extern "C" int oxh_plan_set_spin_limit(OxhPlan *pl, uint32_t polls, int phantom_
     if (!pl) return oxh_internal_errorf(OXH_ERR_ARG, "invalid argument: oxh_plan_set_spin_limit: NULL plan");
     pl->spin_limit = polls;
     pl->phantom = phantom_workgroup ? 1u : 0u;
+    return OXH_OK;
+}
+
+extern "C" int oxh_debug_plan_stamps(OxhPlan *pl, uint64_t *d_stamps)
+{
+    if (!pl) return oxh_internal_errorf(OXH_ERR_ARG, "invalid argument: oxh_debug_plan_stamps: NULL plan");
+    pl->d_stamps = d_stamps;
     return OXH_OK;
 }
 
