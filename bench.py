@@ -5,15 +5,19 @@
 
 A step is one decode token of the Llama-3-8B-shaped GEMV set: 32 layers x
 {fused q/k/v, o, fused gate/up (Q4_K), down (Q6_K)}, every GEMV preceded by
-the Q8_K quantisation of its own f32 input (fused into the GEMV kernel), 128
-launches replayed as one HIP graph.  All inputs are resident in HBM before the timed region starts.
+the Q8_K quantisation of its own f32 input (done inside the kernel).  The 128
+matmuls of a step run as ONE launch of the persistent plan kernel (oxh_plan);
+`--mode graph` runs them as 128 launches replayed as one HIP graph instead,
+and that figure is reported next to the headline one either way.  All inputs
+are resident in HBM before the timed region starts.
 
 Prints ONE JSON line.  `value` is whole-step algorithmic GB/s (packed weights
 at their on-disk size + f32 activations in + f32 outputs out, divided by the
-wall time of the K timed steps).  `roofline` is the dominant kernel (the
-Q4_K gate/up GEMV, 28672 x 4096) timed with HIP events on the launch stream.
+wall time of the K timed steps).  `roofline` is the kernel the step runs in
+(k_plan: one launch = one step), timed with HIP events on the launch stream.
 `cpu_baseline` is the reference's own CPU code (oracle/_ref, or the oracle
-port when that was never built) on this host's cores over one layer.
+port when that was never built) on this host's cores, streaming eight distinct
+layers in turn (1.1 GB: beyond the host's last-level cache).
 """
 import argparse
 import json
@@ -29,6 +33,9 @@ HBM_PEAK_GBPS = 8000.0
 # 32410.7 KiB x 2.000, WRITE_SIZE 116.57 KiB x 1.000; the factors are what the
 # same counters read for a 256 MiB device-to-device copy).  Not measured live.
 GATE_UP_TRAFFIC_BYTES = 66496518
+# HBM bytes one k_plan launch (a whole 32-layer step) moves, measured the same way; None until a
+# counter run of this kernel has been taken.
+PLAN_STEP_TRAFFIC_BYTES = None
 INT8_PEAK_TOPS = 5033.0     # dense int8 MFMA: 256 CU x 2.4 GHz x 8192 op/clk/CU
 
 
@@ -48,17 +55,25 @@ def timed(fn, reps, mv):
 def chain_figure(mv, ds, steps):
     """The same 32 layers as a dependent chain, with the float steps a decode
     layer runs between its matmuls (residual add + RMSNorm in front of q/k/v and
-    of gate/up, SwiGLU behind gate/up) fused into the four GEMV launches."""
+    of gate/up, SwiGLU behind gate/up) fused into the four matmuls of a layer:
+    as one launch of the plan kernel, and as 128 launches in a graph."""
     from oxidize_amd.workloads import DecodeChain
     chain = DecodeChain(ds)
     graph = mv.Graph()
     with graph:
         chain.launch_step()
-    us = timed(graph.launch, max(5, steps), mv)
+    us_graph = timed(graph.launch, max(5, steps), mv)
+    chain2 = DecodeChain(ds)
+    plan = mv.Plan(chain2.plan_ops())
+    us = timed(plan.launch, max(5, steps), mv)
+    assert plan.status() == 0
+    waits = plan.info()["n_waits"]
+    plan.destroy()
     nbytes = chain.bytes_per_step
     return {"us_per_step": round(us, 1), "gbps": round(nbytes / us / 1e3, 1),
             "frac_of_hbm_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBPS, 4),
-            "launches_per_step": 4 * ds.layers, "bytes_per_step": nbytes,
+            "launches_per_step": 1, "waits_per_step": waits, "bytes_per_step": nbytes,
+            "as_graph_of_128_launches_us": round(us_graph, 1),
             "note": "attention itself is outside this library: the q projection stands in for its "
                     "output so that every launch depends on the previous one"}
 
@@ -350,6 +365,10 @@ def traffic_probe(mv, ds):
     for layer in range(ds.layers):
         ds.launch_op(layer, 2)
     mv.sync()
+    plan = mv.Plan(ds.plan_ops())
+    for _ in range(3):
+        plan.launch()
+    assert plan.status() == 0
 
 
 def mmq_probe(mv, synth):
@@ -367,12 +386,22 @@ def mmq_probe(mv, synth):
     mv.sync()
 
 
-def cpu_baseline(layers_sample=1, min_seconds=2.5, cores=None):
-    """The reference CPU path on the host cores over `layers_sample` layers of
-    the same workload (same shapes, same synthetic generator); `cores` = worker
-    threads (default: up to 16, the cap of the reference's own CLI)."""
-    import ctypes
+def host_cpu_model():
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name"):
+                return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
 
+
+def cpu_baseline(layers_sample=8, min_seconds=2.5, cores=None):
+    """The reference CPU path on the host cores over `layers_sample` distinct
+    layers of the same workload in turn (same shapes, same synthetic generator:
+    138 MB a layer, so eight of them stream from DRAM rather than sit in the
+    host's caches; layers_sample=1 gives the cache-resident figure); `cores` =
+    worker threads (default: up to 16, the cap of the reference's own CLI)."""
     import numpy as np
     sys.path.insert(0, os.path.join(ROOT, "tests"))
     import oxlibs
@@ -389,42 +418,43 @@ def cpu_baseline(layers_sample=1, min_seconds=2.5, cores=None):
     orc = oxlibs.oracle()
     ops = [(13, [4096, 1024, 1024], 4096), (13, [4096], 4096), (13, [14336, 14336], 4096),
            (16, [4096], 14336)]
-    mats = []
+    layers = []
     nbytes = 0
-    for i, (qt, rows, cols) in enumerate(ops):
-        ws = [synth.weights(qt, r, cols, seed=0, stream=9000 + 10 * i + k) for k, r in enumerate(rows)]
-        x = synth.normal(cols, seed=0, stream=9900 + i)
-        outs = [np.zeros(r, np.float32) for r in rows]
-        temp = np.zeros(cols, np.float32)
-        mats.append((qt, rows, cols, ws, x, outs, temp))
-        nbytes += sum(w.nbytes for w in ws) + 4 * cols + 4 * sum(rows)
+    for layer in range(layers_sample):
+        mats = []
+        for i, (qt, rows, cols) in enumerate(ops):
+            ws = [synth.weights(qt, r, cols, seed=0, stream=9000 + 100 * layer + 10 * i + k)
+                  for k, r in enumerate(rows)]
+            x = synth.normal(cols, seed=0, stream=9900 + i)
+            outs = [np.zeros(r, np.float32) for r in rows]
+            temp = np.zeros(cols, np.float32)
+            mats.append((qt, rows, cols, ws, x, outs, temp))
+            if layer == 0:
+                nbytes += sum(w.nbytes for w in ws) + 4 * cols + 4 * sum(rows)
+        layers.append(mats)
+    fn = ref.oc_matvec_quantized_fused if ref is not None else orc.oxo_matvec_quantized_fused
 
-    def one_layer():
+    def one_layer(mats):
         for qt, rows, cols, ws, x, outs, temp in mats:
             rb = synth.row_bytes(qt, cols)
             n = len(rows)
-            if ref is not None:
-                ref.oc_matvec_quantized_fused(oxlibs.u32_array([qt] * n), oxlibs.ptr_array(ws),
-                                              oxlibs.size_array(rows), cols, oxlibs.size_array([rb] * n),
-                                              n, x.ctypes.data, oxlibs.ptr_array(outs), temp.ctypes.data)
-            else:
-                orc.oxo_matvec_quantized_fused(oxlibs.u32_array([qt] * n), oxlibs.ptr_array(ws),
-                                               oxlibs.size_array(rows), cols, oxlibs.size_array([rb] * n),
-                                               n, x.ctypes.data, oxlibs.ptr_array(outs), temp.ctypes.data)
+            fn(oxlibs.u32_array([qt] * n), oxlibs.ptr_array(ws), oxlibs.size_array(rows), cols,
+               oxlibs.size_array([rb] * n), n, x.ctypes.data, oxlibs.ptr_array(outs), temp.ctypes.data)
 
-    one_layer()
+    one_layer(layers[0])
     reps, t0 = 0, time.perf_counter()
     while True:
-        one_layer()
+        one_layer(layers[reps % layers_sample])
         reps += 1
         dt = time.perf_counter() - t0
         if dt >= min_seconds and reps >= 3:
             break
     gbps = nbytes * reps / dt / 1e9
     return {"value": round(gbps, 3), "unit": "GB/s", "cores": cores, "kind": kind,
-            "sample": "%d repetitions of one layer of the same decode set (qkv, o, gate/up Q4_K; "
-                      "down Q6_K; %.1f MB per repetition) through oc_matvec_quantized_fused, "
-                      "%.2f s wall" % (reps, nbytes / 1e6, dt)}
+            "sample": "%d layer passes over %d distinct layers of the same decode set in turn (qkv, o, gate/up "
+                      "Q4_K; down Q6_K; %.1f MB per layer, %.0f MB in all) through oc_matvec_quantized_fused, "
+                      "%.2f s wall; host CPU: %s" % (reps, layers_sample, nbytes / 1e6,
+                                                     nbytes * layers_sample / 1e6, dt, host_cpu_model())}
 
 
 def main():
@@ -434,7 +464,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--layers", type=int, default=32, help=argparse.SUPPRESS)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--no-graph", action="store_true", help="launch kernels one by one")
+    ap.add_argument("--mode", choices=["plan", "graph", "launches"], default="plan",
+                    help="a step as one persistent launch (default), as a HIP graph of 128 launches, or as 128 launches")
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary configurations")
     ap.add_argument("--probe", choices=["traffic", "mmq"], help="run a counter-collection workload and exit")
     args = ap.parse_args()
@@ -462,14 +493,15 @@ def main():
         traffic_probe(mv, ds)
         return 0
 
-    graph = None
-    if not args.no_graph:
-        graph = mv.Graph()
-        with graph:
-            ds.launch_step()
+    graph = mv.Graph()
+    with graph:
+        ds.launch_step()
+    plan = mv.Plan(ds.plan_ops())
 
     def step():
-        if graph is not None:
+        if args.mode == "plan":
+            plan.launch()
+        elif args.mode == "graph":
             graph.launch()
         else:
             ds.launch_step()
@@ -486,28 +518,44 @@ def main():
     e1.record()
     mv.sync()
     wall = time.perf_counter() - t0
+    if args.mode == "plan" and plan.status() != 0:
+        print("bench.py: a plan launch gave up on a wait: " + lib.oxh_last_error().decode(), file=sys.stderr)
+        return 1
     ev_ms = e1.ms_since(e0)
     ms_per_step = wall * 1e3 / args.steps
     value = step_bytes * args.steps / wall / 1e9
+    # the other two ways of running the same step, for the record
+    other_modes = {"plan_one_launch_us": round(timed(plan.launch, args.steps, mv), 1),
+                   "graph_of_128_launches_us": round(timed(graph.launch, args.steps, mv), 1)}
 
-    # Dominant kernel: the Q4_K gate/up GEMV (2 x 14336 rows x 4096), timed
-    # back to back over the 32 layers' distinct weights (2.1 GB per sweep, so
-    # nothing is served from cache), HIP events on the launch stream.
-    gate_up = 2
-    _, qt, rows, cols, _ = ds.ops[gate_up]
-    k_bytes = sum(w.nbytes for w in ds.weights[0][gate_up]) + 4 * cols + 4 * sum(rows)
+    # The four matmuls of a layer as single launches, each timed back to back over the 32 layers' distinct
+    # weights (nothing is served from cache), HIP events on the launch stream: what a step costs when it is
+    # launched kernel by kernel (their sum x 32 is the graph figure), and where the plan's gain comes from.
     sweeps = max(3, min(10, args.steps))
-    for layer in range(ds.layers):
-        ds.launch_op(layer, gate_up)
-    mv.sync()
-    k0, k1 = mv.Event(), mv.Event()
-    k0.record()
-    for _ in range(sweeps):
+    per_launch = {}
+    for op, (name, qt, rows, cols, _) in enumerate(ds.ops):
+        nb = sum(w.nbytes for w in ds.weights[0][op]) + 4 * cols + 4 * sum(rows)
         for layer in range(ds.layers):
-            ds.launch_op(layer, gate_up)
-    k1.record()
-    mv.sync()
-    k_us = k1.ms_since(k0) * 1e3 / (sweeps * ds.layers)
+            ds.launch_op(layer, op)
+        mv.sync()
+        k0, k1 = mv.Event(), mv.Event()
+        k0.record()
+        for _ in range(sweeps):
+            for layer in range(ds.layers):
+                ds.launch_op(layer, op)
+        k1.record()
+        mv.sync()
+        us = k1.ms_since(k0) * 1e3 / (sweeps * ds.layers)
+        per_launch[name] = {"us": round(us, 3), "bytes": nb, "gbps": round(nb / us / 1e3, 1),
+                            "frac_of_hbm_peak": round(nb / us / 1e3 / HBM_PEAK_GBPS, 4)}
+    per_launch["sum_x_layers_ms"] = round(sum(v["us"] for v in per_launch.values()) * ds.layers / 1e3, 4)
+
+    if args.mode == "plan":
+        k_name, k_bytes, k_us = "k_plan (one launch = one decode step of 128 matmuls)", step_bytes, ev_ms * 1e3 / args.steps
+        k_traffic = PLAN_STEP_TRAFFIC_BYTES if ds.layers == 32 else None
+    else:
+        k_name, k_bytes, k_us = "k_gemv_q4_k (gate/up 28672x4096)", per_launch["gate_up"]["bytes"], per_launch["gate_up"]["us"]
+        k_traffic = GATE_UP_TRAFFIC_BYTES
     achieved = k_bytes / k_us / 1e3   # GB/s
 
     out = {
@@ -525,16 +573,20 @@ def main():
         "data": "synthetic",
         "config": {"workload": "llama3-8b decode GEMV set, batch 1, 32 layers: qkv+o+gate/up Q4_K, "
                                "down Q6_K, Q8_K activations (BASELINE configs[1])",
-                   "layers": ds.layers, "launches_per_step": 4 * ds.layers,
-                   "bytes_per_step": step_bytes, "hip_graph": graph is not None},
+                   "layers": ds.layers, "mode": args.mode,
+                   "launches_per_step": 1 if args.mode == "plan" else 4 * ds.layers,
+                   "bytes_per_step": step_bytes},
         "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBPS, 2),
         "tokens_per_s_equiv": round(args.steps / wall, 1),
         "gpu_event_ms_per_step": round(ev_ms / args.steps, 4),
         "device": info,
-        "roofline": {"bound": "hbm", "kernel": "k_gemv_q4_k (gate/up 28672x4096)",
+        "roofline": {"bound": "hbm", "kernel": k_name,
                      "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": GATE_UP_TRAFFIC_BYTES,
+                     "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": k_traffic,
+                     "traffic_source": "rocprofv3 --pmc summary under profiles/ (a constant in bench.py, not live)",
                      "bytes_per_launch": k_bytes, "us_per_launch": round(k_us, 3)},
+        "step_other_modes": other_modes,
+        "single_launches": per_launch,
     }
     if not args.no_extra:
         from oxidize_amd import synth
@@ -542,8 +594,11 @@ def main():
         out["extra"]["decode_chain_fused"] = chain_figure(mv, ds, args.steps)
     out["cpu_baseline"] = None if args.no_cpu else cpu_baseline()
     if not args.no_cpu and out["cpu_baseline"]["kind"] == "reference" and isinstance(out.get("extra"), dict):
-        one = cpu_baseline(min_seconds=1.5, cores=1)
+        one = cpu_baseline(layers_sample=2, min_seconds=1.5, cores=1)
         out["extra"]["cpu_baseline_1_thread"] = {"value": one["value"], "unit": one["unit"], "sample": one["sample"]}
+        hot = cpu_baseline(layers_sample=1, min_seconds=1.5)
+        out["extra"]["cpu_baseline_cache_resident"] = {"value": hot["value"], "unit": hot["unit"], "cores": hot["cores"],
+                                                       "sample": hot["sample"]}
     print(json.dumps(out))
     return 0
 

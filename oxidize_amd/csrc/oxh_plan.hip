@@ -80,6 +80,8 @@ struct PlanOp {
     PlanSeg s[PLAN_MAX_SEGS];
 };
 
+static_assert(sizeof(PlanOp) % 16 == 0, "table rows are copied in 16-byte pieces");
+
 /* progress counters: flags[wg], then go[0] = the published minimum, go[1] = error word */
 struct PlanSync {
     uint32_t *flags;
@@ -95,12 +97,13 @@ struct PlanSync {
 __device__ __forceinline__ void plan_stamp(const PlanSync &sy, uint32_t op, uint32_t slot, uint32_t lane, uint32_t wave)
 {
     if (sy.stamps != nullptr && wave == 0u && lane == 0u)
-        sy.stamps[((size_t)op * gridDim.x + blockIdx.x) * PLAN_STAMPS + slot] = __builtin_readcyclecounter();
+        sy.stamps[((size_t)op * gridDim.x + blockIdx.x) * PLAN_STAMPS + slot] = __builtin_amdgcn_s_memrealtime();
 }
 
 struct PlanLds {
     uint32_t act_bytes;             /* one staged activation (two are kept, used in turn) */
     uint32_t outs_off, red_off, terms_off, terms_per_wave;   /* bytes; terms_per_wave in floats */
+    uint32_t table_off;             /* the operation table's copy */
 };
 
 /* ─── coherent accesses ───────────────────────────────────────────────── */
@@ -164,6 +167,35 @@ __device__ __forceinline__ T *gptr(gaddr v)
     return (T *)reinterpret_cast<G>(v);
 }
 
+/* The operation table is copied into LDS when the kernel starts: read from global memory, a row costs
+ * a trip to HBM (the weight stream flushes it out of every cache between two uses), in the middle of
+ * staging.  Fields are the same for every lane; readfirstlane says so to the compiler, and everything
+ * computed from them stays in scalar registers. */
+__device__ __forceinline__ uint32_t uni(uint32_t v) { return (uint32_t)__builtin_amdgcn_readfirstlane((int)v); }
+__device__ __forceinline__ gaddr uni(gaddr v)
+{
+    return (gaddr)uni((uint32_t)v) | ((gaddr)uni((uint32_t)(v >> 32)) << 32);
+}
+__device__ __forceinline__ float uni(float v) { return __uint_as_float(uni(__float_as_uint(v))); }
+
+/* the per-operation fields staging and the passes use */
+struct OpHead {
+    uint32_t kind, pro, blocks, magic, term_stride, rows_cap, wait, signal;
+    float eps;
+    gaddr x, pro_b, pro_add, pro_sum_out, pro_out, act_out;
+};
+
+__device__ __forceinline__ OpHead plan_head(const PlanOp *op)
+{
+    OpHead h;
+    h.kind = uni(op->kind); h.pro = uni(op->pro); h.blocks = uni(op->blocks); h.magic = uni(op->magic);
+    h.term_stride = uni(op->term_stride); h.rows_cap = uni(op->rows_cap); h.wait = uni(op->wait);
+    h.signal = uni(op->signal); h.eps = uni(op->eps);
+    h.x = uni(op->x); h.pro_b = uni(op->pro_b); h.pro_add = uni(op->pro_add);
+    h.pro_sum_out = uni(op->pro_sum_out); h.pro_out = uni(op->pro_out); h.act_out = uni(op->act_out);
+    return h;
+}
+
 /* ─── what a wave owns of an operation ───────────────────────────────── */
 
 struct PWork {
@@ -180,31 +212,26 @@ __device__ __forceinline__ uint32_t plan_block_bytes(uint32_t kind)
     return kind == PLAN_Q6_K ? 210u : kind == PLAN_Q5_K ? 176u : 144u;
 }
 
-__device__ __forceinline__ PWork plan_work(const PlanOp *__restrict__ op, uint32_t wave)
+__device__ __forceinline__ PWork plan_work(const PlanOp *op, uint32_t wave)
 {
     PWork k;
-    const uint32_t wg = blockIdx.x, n = op->n_segs;
+    const uint32_t wg = blockIdx.x, n = uni(op->n_segs);
     uint32_t si = 0;
 #pragma unroll
     for (uint32_t i = 1; i < PLAN_MAX_SEGS; i++)
-        if (i < n && wg >= op->s[i].wg_begin) si = i;
-    gaddr w = op->s[0].w, w2 = op->s[0].w2, out = op->s[0].out;
-    uint32_t wg_begin = op->s[0].wg_begin, q = op->s[0].rows_q, rem = op->s[0].rows_rem;
-#pragma unroll
-    for (uint32_t i = 1; i < PLAN_MAX_SEGS; i++)
-        if (si == i) {
-            w = op->s[i].w; w2 = op->s[i].w2; out = op->s[i].out;
-            wg_begin = op->s[i].wg_begin; q = op->s[i].rows_q; rem = op->s[i].rows_rem;
-        }
-    const bool idle = wg >= op->n_wg;
+        if (i < n && wg >= uni(op->s[i].wg_begin)) si = i;
+    const PlanSeg *sg = &op->s[si];
+    const gaddr w = uni(sg->w), w2 = uni(sg->w2), out = uni(sg->out);
+    const uint32_t wg_begin = uni(sg->wg_begin), q = uni(sg->rows_q), rem = uni(sg->rows_rem);
+    const bool idle = wg >= uni(op->n_wg);
     const uint32_t wi0 = (wg - wg_begin) * PLAN_W, wi = wi0 + wave;
-    k.kind = op->kind;
+    k.kind = uni(op->kind);
     k.row0 = wi * q + min(wi, rem);
     k.nrows = idle ? 0u : q + (wi < rem ? 1u : 0u);
     k.wg_row0 = wi0 * q + min(wi0, rem);
     k.wg_rows = idle ? 0u : (wi0 + PLAN_W) * q + min(wi0 + PLAN_W, rem) - k.wg_row0;
     k.out = gptr<float>(out);
-    const uint32_t B = op->blocks;
+    const uint32_t B = uni(op->blocks);
     const size_t off = (size_t)(k.nrows ? k.row0 : 0u) * B * plan_block_bytes(k.kind);
     k.src.a = gptr<const uint8_t>(w + off);
     k.src.n1 = k.nrows * B;
@@ -352,10 +379,10 @@ __device__ __forceinline__ XRegs load4_either(bool coherent, const float *base, 
 }
 
 __device__ __forceinline__ void
-plan_stage_issue(const PlanOp *__restrict__ op, XStage &xs, bool coherent, uint32_t lane, uint32_t wave)
+plan_stage_issue(const OpHead &op, XStage &xs, bool coherent, uint32_t lane, uint32_t wave)
 {
-    const uint32_t B = op->blocks, pro = op->pro;
-    const float *x = gptr<const float>(op->x), *add = gptr<const float>(op->pro_add), *b = gptr<const float>(op->pro_b);
+    const uint32_t B = op.blocks, pro = op.pro;
+    const float *x = gptr<const float>(op.x), *add = gptr<const float>(op.pro_add), *b = gptr<const float>(op.pro_b);
     const CohBuf xc = coh_buf(x), ac = coh_buf(add), bc = coh_buf(b);
 #pragma unroll
     for (int i = 0; i < 4; i++) {
@@ -375,10 +402,10 @@ plan_stage_issue(const PlanOp *__restrict__ op, XStage &xs, bool coherent, uint3
  * eight times. */
 template <int KIND /* 0 Q4_K/Q5_K layout, 1 Q6_K layout */>
 __device__ __forceinline__ void
-plan_stage_finish(const PlanOp *__restrict__ op, const XStage &xs, uint8_t *base, float *red, bool storer,
+plan_stage_finish(const OpHead &op, const XStage &xs, uint8_t *base, float *red, bool storer,
                   uint32_t lane, uint32_t wave)
 {
-    const uint32_t B = op->blocks, pro = op->pro;
+    const uint32_t B = op.blocks, pro = op.pro;
     const bool rms = pro == GEMV_PRO_RMSNORM || pro == GEMV_PRO_ADD_RMSNORM, add = pro == GEMV_PRO_ADD_RMSNORM;
     XRegs xr[4];
 #pragma unroll
@@ -397,12 +424,12 @@ plan_stage_finish(const PlanOp *__restrict__ op, const XStage &xs, uint8_t *base
         if (lane == 0u) red[wave] = ss;
         __syncthreads();
         const float tot = wave_sum_f32(lane < PLAN_W ? red[lane] : 0.0f);
-        inv = 1.0f / sqrtf(tot / (float)(B * 256u) + op->eps);
+        inv = 1.0f / sqrtf(tot / (float)(B * 256u) + op.eps);
     }
-    const bool has_sout = add && storer && op->pro_sum_out != 0u;
-    const bool has_fout = pro != GEMV_PRO_NONE && storer && op->pro_out != 0u;
-    const CohBuf sout = coh_buf(gptr<float>(op->pro_sum_out)), fout = coh_buf(gptr<float>(op->pro_out));
-    uint8_t *gout = (storer && op->act_out) ? gptr<uint8_t>(op->act_out) : nullptr;
+    const bool has_sout = add && storer && op.pro_sum_out != 0u;
+    const bool has_fout = pro != GEMV_PRO_NONE && storer && op.pro_out != 0u;
+    const CohBuf sout = coh_buf(gptr<float>(op.pro_sum_out)), fout = coh_buf(gptr<float>(op.pro_out));
+    uint8_t *gout = (storer && op.act_out) ? gptr<uint8_t>(op.act_out) : nullptr;
 #pragma unroll
     for (int i = 0; i < 4; i++) {
         const uint32_t unit = wave + PLAN_W * (uint32_t)i;
@@ -488,8 +515,18 @@ k_plan(const PlanOp *__restrict__ ops, uint32_t n_ops, const PlanSync sy, const 
      * flight and no weight or input register holds anything, so nothing but scalars crosses the loop
      * boundary.  One trip = (rows, outputs and announcement of operation i - 1), then requests,
      * staging and passes of operation i. */
-    PWork cur = plan_work(&ops[0], wave);
+    /* the operation table, once, into LDS */
+    {
+        const u32x4 *src = reinterpret_cast<const u32x4 *>(ops);
+        u32x4 *dst = reinterpret_cast<u32x4 *>(lds + ld.table_off);
+        const uint32_t n16 = n_ops * (uint32_t)(sizeof(PlanOp) / 16u);
+        for (uint32_t k = threadIdx.x; k < n16; k += 1024u) dst[k] = src[k];
+    }
+    __syncthreads();
+    const PlanOp *const tab = reinterpret_cast<const PlanOp *>(lds + ld.table_off);
+    PWork cur = plan_work(&tab[0], wave);
     PWork prev = cur;
+    OpHead po = plan_head(&tab[0]);
     for (uint32_t i = 0;; i++) {
         /* The lane index, made opaque once per trip: everything derived from it (sub-block masks, LDS
          * slots, byte offsets) is then recomputed per operation in a handful of instructions instead of
@@ -497,18 +534,16 @@ k_plan(const PlanOp *__restrict__ ops, uint32_t n_ops, const PlanSync sy, const 
         uint32_t ln = lane;
         asm volatile("" : "+v"(ln));
         if (i > 0u) {
-            const PlanOp *po = &ops[i - 1u];
             /* Rows first, then the workgroup's outputs go out, then (below) the requests for the next
              * operation: those queue up in the memory pipeline (a compute unit takes in about 12 bytes
              * per cycle), and anything placed after them in program order waits for that queue. */
-            plan_row_sums(terms, prev, po->blocks, po->term_stride, outs, ln);
-            plan_stamp(sy, i - 1u, 5, ln, wave);
+            plan_row_sums(terms, prev, po.blocks, po.term_stride, outs, ln);
             lds_barrier();
             plan_stamp(sy, i - 1u, 6, ln, wave);
             if (wave == 0u) {
                 const CohBuf dst = coh_buf(prev.out + prev.wg_row0);
                 for (uint32_t r = ln; r < prev.wg_rows; r += 64u) cstore_f32(dst, r * 4u, outs[r]);
-                if (po->signal != 0u || i == n_ops) {
+                if (po.signal != 0u || i == n_ops) {
                     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
                     /* the last operation leaves every counter at base + n_ops + 1, the next launch's base */
                     if (ln == 0u) cstore(sy.flags + blockIdx.x, base + i + (i == n_ops ? 1u : 0u));
@@ -518,48 +553,53 @@ k_plan(const PlanOp *__restrict__ ops, uint32_t n_ops, const PlanSync sy, const 
         }
         if (i == n_ops) break;
 
-        const PlanOp *op = &ops[i];
+        const OpHead op = plan_head(&tab[i]);
         uint8_t *act = lds + (size_t)(i & 1u) * ld.act_bytes;
         plan_stamp(sy, i, 0, ln, wave);
-        /* Loads complete in the order a wave issued them, so the order of the requests is the
-         * schedule.  An operation that depends on nothing gets its input vector requested first and
-         * both weight sets behind it; one that has to wait gets one set before the wait (that is
-         * what streams in while the wait lasts), then the input vector, then the second set. */
+        /* Loads complete in the order a wave issued them, and the compiler waits for ALL of them
+         * before the first use of the input vector (its requests sit in conditional code, which it
+         * cannot count past).  So the order of the requests is the schedule: one set of weights first
+         * (that is what streams in while a dependency is awaited and the vector is on its way), then
+         * the vector; the second set goes out once the vector has been quantised, and streams in
+         * during the workgroup barrier and the first pass. */
         WSet A, B;
         A.a = A.b = A.c = A.d = A.e = u32x4{ 0u, 0u, 0u, 0u };
         B.a = B.b = B.c = B.d = B.e = A.a;
         XStage xs;
 #pragma unroll
         for (int u = 0; u < 4; u++) xs.x[u] = xs.t[u] = xs.b[u] = XRegs{ 0.f, 0.f, 0.f, 0.f };
-        if (op->wait == 0u) {
+        if (op.wait == 0u) {
+            /* nothing to wait for: the vector goes first and is there in a microsecond */
             plan_stage_issue(op, xs, false, ln, wave);
             plan_prefetch<HAS_Q5>(cur, A, 0u, ln);
-            plan_prefetch<HAS_Q5>(cur, B, 1u, ln);
         } else {
             plan_prefetch<HAS_Q5>(cur, A, 0u, ln);
-            if (!plan_wait(sy, base + op->wait, s_ok, ln, wave)) return;
+            if (!plan_wait(sy, base + op.wait, s_ok, ln, wave)) return;
             plan_stage_issue(op, xs, true, ln, wave);
-            plan_prefetch<HAS_Q5>(cur, B, 1u, ln);
         }
         plan_stamp(sy, i, 1, ln, wave);
-        /* what this wave owns of the next operation: read from the table now, so that the table's
-         * trip from memory is over long before the passes end */
+        /* what this wave owns of the next operation */
         PWork nx = cur;
-        if (i + 1u < n_ops) nx = plan_work(&ops[i + 1u], wave);
+        if (i + 1u < n_ops) nx = plan_work(&tab[i + 1u], wave);
 
         const bool storer = blockIdx.x == 0u;
-        const uint32_t Bk = op->blocks;
-        if (op->kind == PLAN_Q6_K) plan_stage_finish<1>(op, xs, act, red, storer, ln, wave);
-        else                       plan_stage_finish<0>(op, xs, act, red, storer, ln, wave);
+        const uint32_t Bk = op.blocks;
+        if (sy.stamps != nullptr) {         /* measurement only: when has the vector arrived? */
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            plan_stamp(sy, i, 5, ln, wave);
+        }
+        if (op.kind == PLAN_Q6_K) plan_stage_finish<1>(op, xs, act, red, storer, ln, wave);
+        else                      plan_stage_finish<0>(op, xs, act, red, storer, ln, wave);
+        plan_prefetch<HAS_Q5>(cur, B, 1u, ln);
         plan_stamp(sy, i, 2, ln, wave);
         __syncthreads();
         plan_stamp(sy, i, 3, ln, wave);
 
         GemvParams gp;
         gp.blocks = Bk;
-        gp.magic = op->magic;
-        gp.term_stride = op->term_stride;
-        gp.rows_cap = op->rows_cap;
+        gp.magic = op.magic;
+        gp.term_stride = op.term_stride;
+        gp.rows_cap = op.rows_cap;
         gp.dump = nullptr;
         if (cur.nblk != 0u) {
             if (cur.kind == PLAN_Q6_K)      plan_passes_q6(A, B, cur, gp, act, q8k6_lds_bytes(Bk), terms, ln);
@@ -569,6 +609,7 @@ k_plan(const PlanOp *__restrict__ ops, uint32_t n_ops, const PlanSync sy, const 
         plan_stamp(sy, i, 4, ln, wave);
         prev = cur;
         cur = nx;
+        po = op;
     }
 }
 
@@ -792,12 +833,13 @@ extern "C" int oxh_plan_create(const OxhPlanOp *ops, size_t n_ops, OxhPlan **out
     pl->ld.red_off = pl->ld.outs_off + ((max_wg_rows * 4u + 15u) & ~15u);
     pl->ld.terms_off = pl->ld.red_off + 128u;
     pl->ld.terms_per_wave = max_cap_terms;
-    pl->lds_bytes = (size_t)pl->ld.terms_off + (size_t)PLAN_W * max_cap_terms * 4u;
+    pl->ld.table_off = (pl->ld.terms_off + PLAN_W * max_cap_terms * 4u + 15u) & ~15u;
+    pl->lds_bytes = (size_t)pl->ld.table_off + n_ops * sizeof(PlanOp);
     const char *sl = getenv("OXH_PLAN_SPIN_LIMIT");
     pl->spin_limit = sl && *sl ? (uint32_t)strtoul(sl, nullptr, 10) : 4000000u;
     if (pl->lds_bytes > 160u * 1024u) {
         free(h); free(pl);
-        return oxh_internal_errorf(OXH_ERR_TOO_WIDE, "plan: an operation's staged activation and row tables do not fit 160 KiB of LDS");
+        return oxh_internal_errorf(OXH_ERR_TOO_WIDE, "plan: the staged activation, the row tables and the table of %zu operations (%zu bytes each) do not fit 160 KiB of LDS; split the chain into several plans", n_ops, sizeof(PlanOp));
     }
     const void *kernel = has_q5 ? reinterpret_cast<const void *>(k_plan<true>) : reinterpret_cast<const void *>(k_plan<false>);
     {
