@@ -63,6 +63,8 @@ extern "C" {
 #define OXH_AL5_XS 18u     /* f16 d + thirty-two 3-bit codes (oxk.h:55) */
 #define OXH_AL6    19u     /* the Q5_0 layout */
 #define OXH_AL8    20u     /* the Q8_0 layout */
+#define OXH_IQ3_S  25u     /* codebook format, 3.44 bits per weight (oxk.h:63) */
+#define OXH_IQ1_XXXS 36u   /* codebook format, 1.19 bits per weight (quant.h:79) */
 #define OXH_QTYPE_UNKNOWN 0xffffffffu
 
 /* Block geometry (oxidize-c/include/oxidize/oxk.h:46-66). */
@@ -80,6 +82,8 @@ extern "C" {
 #define OXH_Q5_0_BYTES    22u
 #define OXH_Q5_1_BYTES    24u
 #define OXH_Q8_K_BYTES   292u
+#define OXH_IQ3_S_BYTES  110u
+#define OXH_IQ1_XXXS_BYTES 38u
 
 /* Thread-local text of the last failure on this thread ("" if none). */
 const char *oxh_last_error(void);

@@ -520,6 +520,75 @@ float oxo_dot_q5_1_q8_0(const uint8_t *row, size_t blocks, const uint8_t *act, i
     return dot_legacy(1, 1, row, blocks, act, isum);
 }
 
+/* ─── the codebook formats ────────────────────────────────────────────── */
+
+#include "iq_grids.inc"     /* OXH_IQ3S_GRID, OXH_IQ1XXXS_GRID: data shared with the kernels */
+
+float oxo_dot_iq3_s_q8_k(const uint8_t *row, size_t blocks, const uint8_t *act, int32_t *lanes)
+{
+    float acc[8] = { 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f };
+    for (size_t b = 0; b < blocks; b++) {
+        const uint8_t *w = row + b * OXO_IQ3_S_BYTES;
+        const uint8_t *a = act + b * OXO_Q8_K_BYTES;
+        float dq;
+        memcpy(&dq, a, 4);
+        const float d = oxo_f16_to_f32(rd_u16(w)) * dq;
+        const int8_t *q = (const int8_t *)(a + 4);
+        int32_t lane[8] = { 0, 0, 0, 0, 0, 0, 0, 0 };
+        for (unsigned sb = 0; sb < 8; sb++) {
+            const uint8_t *codes = w + 2 + 8 * sb, *signs = w + 74 + 4 * sb;
+            const unsigned ninth = w[66 + sb];
+            const unsigned nib = (w[106 + sb / 2] >> (4 * (sb & 1))) & 15u;
+            const int32_t ls = 2 * (int32_t)nib + 1;
+            /* value e of the sub-block: byte e%4 of the grid entry of code e/4; sign bit e%8 of byte e/8 */
+            for (unsigned e = 0; e < 32; e++) {
+                const unsigned c = e / 4;
+                const unsigned code = codes[c] | (((ninth >> c) & 1u) << 8);
+                const int32_t mag = (int32_t)((OXH_IQ3S_GRID[code] >> (8 * (e % 4))) & 0xFFu);
+                const int32_t wv = ((signs[e / 8] >> (e % 8)) & 1u) ? -mag : mag;
+                lane[e / 4] += ls * wv * (int32_t)q[32 * sb + e];
+            }
+        }
+        if (lanes) memcpy(lanes + 8 * b, lane, sizeof lane);
+        for (int j = 0; j < 8; j++) acc[j] = acc[j] + d * (float)lane[j];
+    }
+    const float s0 = acc[0] + acc[4], s1 = acc[1] + acc[5], s2 = acc[2] + acc[6], s3 = acc[3] + acc[7];
+    return (s0 + s2) + (s1 + s3);
+}
+
+float oxo_dot_iq1_xxxs_q8_k(const uint8_t *row, size_t blocks, const uint8_t *act, int32_t *sums)
+{
+    float sum = 0.0f;
+    for (size_t b = 0; b < blocks; b++) {
+        const uint8_t *w = row + b * OXO_IQ1_XXXS_BYTES;
+        const uint8_t *a = act + b * OXO_Q8_K_BYTES;
+        const float dw = oxo_f16_to_f32(rd_u16(w));
+        float da;
+        memcpy(&da, a, 4);
+        const int8_t *q = (const int8_t *)(a + 4);
+        int32_t main_sum = 0, delta_sum = 0;
+        for (unsigned g = 0; g < 8; g++) {          /* groups of 32 values */
+            const unsigned nib = (w[34 + g / 2] >> (4 * (g & 1))) & 15u;
+            const int32_t scale = 2 * (int32_t)(nib & 7u) + 1;
+            int32_t dot = 0, total = 0;
+            for (unsigned e = 0; e < 32; e++) {
+                const uint64_t entry = OXH_IQ1XXXS_GRID[w[2 + 4 * g + e / 8]];
+                dot += (int32_t)(int8_t)(entry >> (8 * (e % 8))) * (int32_t)q[32 * g + e];
+            }
+            for (unsigned h = 0; h < 2; h++) {
+                int16_t bs;
+                memcpy(&bs, a + 260 + 2 * (2 * g + h), 2);
+                total += bs;
+            }
+            main_sum += scale * dot;
+            delta_sum += scale * ((nib & 8u) ? -1 : 1) * total;
+        }
+        if (sums) { sums[2 * b] = main_sum; sums[2 * b + 1] = delta_sum; }
+        sum += dw * da * ((float)main_sum + 0.125f * (float)delta_sum);
+    }
+    return sum;
+}
+
 /* ─── eligibility ─────────────────────────────────────────────────────── */
 
 static size_t block_bytes(uint32_t qtype)
@@ -543,6 +612,8 @@ static size_t block_bytes(uint32_t qtype)
     case OXO_Q3_K_S:
     case OXO_Q3_K_M:
     case OXO_Q3_K_L: return OXO_Q3_K_BYTES;
+    case OXO_IQ3_S:  return OXO_IQ3_S_BYTES;
+    case OXO_IQ1_XXXS: return OXO_IQ1_XXXS_BYTES;
     default:         return 0;
     }
 }
@@ -567,7 +638,9 @@ int oxo_act_kind(uint32_t qtype, size_t cols)
     case OXO_Q4_K_M:
     case OXO_Q5_K_S:
     case OXO_Q5_K_M:
-    case OXO_Q6_K:   return (cols % OXO_QK_K == 0) ? 2 : 0;
+    case OXO_Q6_K:
+    case OXO_IQ1_XXXS:
+    case OXO_IQ3_S:  return (cols % OXO_QK_K == 0) ? 2 : 0;
     default:         return 0;
     }
 }
@@ -599,6 +672,8 @@ static float row_dot(uint32_t qtype, const uint8_t *row, size_t blocks,
     case OXO_Q8_0:   return oxo_dot_q8_0_q8_0(row, blocks, act, NULL);
     case OXO_AL5_XS: return oxo_dot_al5_xs_q8_0(row, blocks, act, NULL);
     case OXO_Q6_K:   return oxo_dot_q6_k_q8_k(row, blocks, act, NULL);
+    case OXO_IQ3_S:  return oxo_dot_iq3_s_q8_k(row, blocks, act, NULL);
+    case OXO_IQ1_XXXS: return oxo_dot_iq1_xxxs_q8_k(row, blocks, act, NULL);
     case OXO_Q2_K:   return oxo_dot_q2_k_q8_k(row, blocks, act, NULL);
     case OXO_Q3_K_S:
     case OXO_Q3_K_M:

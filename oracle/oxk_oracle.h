@@ -68,6 +68,8 @@ enum {
     OXO_AL5_XS = 18,    /* f16 d + 32 three-bit codes in 12 bytes */
     OXO_AL6    = 19,    /* Q5_0 layout */
     OXO_AL8    = 20,    /* Q8_0 layout */
+    OXO_IQ3_S  = 25,    /* f16 d + 64 grid codes + 8 ninth bits + 32 sign bytes + 4 scale bytes */
+    OXO_IQ1_XXXS = 36,  /* f16 d + 32 codebook indices + 4 scale|sign bytes */
 };
 
 #define OXO_QK_K        256u
@@ -80,6 +82,8 @@ enum {
 #define OXO_Q6_K_BYTES  210u
 #define OXO_Q8_0_BYTES  34u
 #define OXO_Q8_K_BYTES  292u
+#define OXO_IQ3_S_BYTES 110u
+#define OXO_IQ1_XXXS_BYTES 38u
 
 /* src/compute/oxk.c:26-56 */
 float    oxo_f16_to_f32(uint16_t h);
@@ -113,6 +117,19 @@ float oxo_dot_q6_k_q8_k(const uint8_t *row, size_t blocks, const uint8_t *act,
  * of 2-bit codes, sixteen 6-bit scales in 12 bytes, f16 d; codes 0..7 with a
  * uniform offset of 4: d*dq*(pos - 4*off)).  `grp` (optional) receives the 16
  * int32 group sums per block. */
+/* src/compute/oxk.c:1052-1116: IQ3_S.  Each 32-value sub-block: eight 9-bit codes (8 bits in qs, the
+ * ninth in qh) into a codebook of four magnitudes each, a sign bit per value, an odd scale 2*s+1 from a
+ * nibble.  The f32 part is NOT one term per block: eight float lanes, lane j taking the positions
+ * 4j..4j+3 of every sub-block, acc[j] = acc[j] + d*(float)lane[j] per block, reduced at the end as
+ * ((a0+a4)+(a2+a6)) + ((a1+a5)+(a3+a7)).  `lanes` (optional) receives the 8 int32 per block.
+ * Pinned: tests/golden/iq_types.npz (compiled reference, scalar and dispatched forms) and live;
+ * a one-hot construction that isolates every (sub-block, position) pair. */
+float oxo_dot_iq3_s_q8_k(const uint8_t *row, size_t blocks, const uint8_t *act, int32_t *lanes);
+/* src/compute/quantization.c:941-1015 (scalar branch): IQ1_XXXS.  Each group of 8 values is one byte
+ * into a codebook of {-1,0,+1}^8; per 32 values an odd scale 2*(n&7)+1 and a sign of the common offset
+ * 0.125: block term dw*da*((float)main + 0.125f*(float)delta), summed in block order.  `sums`
+ * (optional) receives {main, delta} per block.  Pinned like IQ3_S. */
+float oxo_dot_iq1_xxxs_q8_k(const uint8_t *row, size_t blocks, const uint8_t *act, int32_t *sums);
 float oxo_dot_q2_k_q8_k(const uint8_t *row, size_t blocks, const uint8_t *act, int32_t *grp);
 float oxo_dot_q3_k_q8_k(const uint8_t *row, size_t blocks, const uint8_t *act, int32_t *grp);
 /* src/compute/oxk.c:224-241 (block-sequential scalar chain).  `isum`

@@ -84,6 +84,8 @@ static const TypeRow k_types[] = {
     { 12, OXH_Q4_K_M, 256, OXH_Q4_K_BYTES },
     { 13, OXH_Q5_K_M, 256, OXH_Q5_K_BYTES },
     { 14, OXH_Q6_K, 256, OXH_Q6_K_BYTES },
+    { 21, OXH_IQ3_S, 256, OXH_IQ3_S_BYTES },
+    { 66, OXH_IQ1_XXXS, 256, OXH_IQ1_XXXS_BYTES },
     { 24, 31, 1, 1 },      /* I8  */
     { 25, 32, 1, 2 },      /* I16 */
     { 26, 33, 1, 4 },      /* I32 */

@@ -433,6 +433,7 @@ k_q2k_widen(const uint8_t *__restrict__ src, uint8_t *__restrict__ dst, uint32_t
 #include "gemv_kernels.inc"
 #include "mmq_kernels.inc"
 #include "moe_kernels.inc"
+#include "iq_kernels.inc"
 
 /* ─── host side of layer 2 ────────────────────────────────────────────── */
 
@@ -542,7 +543,9 @@ extern "C" int oxh_act_kind(uint32_t qtype, size_t cols)
     case OXH_Q4_K_M:
     case OXH_Q5_K_S:
     case OXH_Q5_K_M:
-    case OXH_Q6_K:   return (cols % OXH_QK_K == 0) ? 2 : 0;
+    case OXH_Q6_K:
+    case OXH_IQ3_S:                     /* the two codebook formats the reference's integer path takes */
+    case OXH_IQ1_XXXS: return (cols % OXH_QK_K == 0) ? 2 : 0;
     default:         return 0;
     }
 }
@@ -563,6 +566,8 @@ static size_t block_bytes(uint32_t qtype)
     case OXH_Q6_K:   return OXH_Q6_K_BYTES;
     case OXH_Q2_K:   return OXH_Q2_K_BYTES;
     case OXH_Q3_K_M: return OXH_Q3_K_BYTES;
+    case OXH_IQ3_S:  return OXH_IQ3_S_BYTES;
+    case OXH_IQ1_XXXS: return OXH_IQ1_XXXS_BYTES;
     default:         return 0;
     }
 }
@@ -668,6 +673,8 @@ static hipError_t raise_all_lds_ceilings(void)
     OXH_RAISE(k_gemv_q5_0)
     OXH_RAISE(k_gemv_q5_1)
     OXH_RAISE(k_gemv_al5_xs)
+    OXH_RAISE(k_gemv_iq3_s)
+    OXH_RAISE(k_gemv_iq1_xxxs)
 #undef OXH_RAISE
 #define OXH_RAISE_PRO1(KERNEL, PRO)                                                               \
     if ((e = raise_lds_ceiling(KERNEL<1, PRO, false>)) != hipSuccess) return e;                   \
@@ -690,6 +697,8 @@ static hipError_t raise_all_lds_ceilings(void)
     OXH_RAISE_PRO(k_gemv_q5_0_pro)
     OXH_RAISE_PRO(k_gemv_q5_1_pro)
     OXH_RAISE_PRO(k_gemv_al5_xs_pro)
+    OXH_RAISE_PRO(k_gemv_iq3_s_pro)
+    OXH_RAISE_PRO(k_gemv_iq1_xxxs_pro)
 #undef OXH_RAISE_PRO
 #undef OXH_RAISE_PRO1
     if ((e = raise_lds_ceiling(k_mmq_q4_k<8, 2, 8>)) != hipSuccess) return e;
@@ -729,11 +738,17 @@ static uint32_t act_lds_bytes(uint32_t qtype, uint32_t blocks)
     return q8k_lds_bytes(blocks);
 }
 
+static bool is_iq(uint32_t qtype) { return qtype == OXH_IQ3_S || qtype == OXH_IQ1_XXXS; }
+
+/* floats a block leaves in the term table: IQ3_S keeps eight running sums per row (oxk.c:1070-1086) */
+static uint32_t terms_per_block(uint32_t qtype) { return qtype == OXH_IQ3_S ? 8u : 1u; }
+
 static size_t gemv_lds_bytes(uint32_t qtype, uint32_t blocks, size_t n_vec, uint32_t waves,
                              uint32_t rows_cap)
 {
     return n_vec * (size_t)act_lds_bytes(qtype, blocks) +
-           (size_t)waves * n_vec * rows_cap * (blocks + 1u) * 4u;
+           (size_t)waves * n_vec * rows_cap * (terms_per_block(qtype) * blocks + 1u) * 4u +
+           (is_iq(qtype) ? IQ_TABLE_BYTES : 0u);       /* the codebook */
 }
 
 static uint32_t env_u32(const char *name, uint32_t dflt, uint32_t lo, uint32_t hi)
@@ -1002,6 +1017,7 @@ static int launch_gemv(uint32_t qtype, const OxhSegment *segs, size_t n_segs, si
     }
     if (total_rows == 0) return OXH_OK;
     if (any_pair && dump) return arg_fail("gemv: no sub-block dump of a paired launch");
+    if (is_iq(qtype) && dump) return arg_fail("gemv: no sub-block dump for the codebook formats");
     if (!any_pair && gemv_wants_mfma(qtype, io, max_nv, dump))
         return launch_mmq_segments(qtype, segs, n_segs, cols, blocks, io, n_vec_default, act_end,
                                    out_stride, stream);
@@ -1056,7 +1072,7 @@ static int launch_gemv(uint32_t qtype, const OxhSegment *segs, size_t n_segs, si
     p.magic = (uint32_t)((0x100000000ull + blocks - 1u) / blocks);
     p.act_bytes = (uint32_t)oxh_act_bytes(qtype, cols);
     p.out_stride = (uint32_t)out_stride;
-    p.term_stride = p.blocks + 1u;
+    p.term_stride = terms_per_block(qtype) * p.blocks + 1u;
     p.rows_cap = rows_cap;
     p.x = io.d_x;
     p.x_stride = (uint32_t)io.x_stride;
@@ -1131,6 +1147,8 @@ static int launch_gemv(uint32_t qtype, const OxhSegment *segs, size_t n_segs, si
     else if (qtype == OXH_Q5_0) OXH_LAUNCH_ANY(k_gemv_q5_0, k_gemv_q5_0_pro);
     else if (qtype == OXH_Q5_1) OXH_LAUNCH_ANY(k_gemv_q5_1, k_gemv_q5_1_pro);
     else if (qtype == OXH_AL5_XS) OXH_LAUNCH_ANY(k_gemv_al5_xs, k_gemv_al5_xs_pro);
+    else if (qtype == OXH_IQ3_S) OXH_LAUNCH_ANY(k_gemv_iq3_s, k_gemv_iq3_s_pro);
+    else if (qtype == OXH_IQ1_XXXS) OXH_LAUNCH_ANY(k_gemv_iq1_xxxs, k_gemv_iq1_xxxs_pro);
     else                        OXH_LAUNCH_ANY(k_gemv_q8_0, k_gemv_q8_0_pro);
 #undef OXH_LAUNCH_ANY
 #undef OXH_LAUNCH_PRO
@@ -1361,7 +1379,8 @@ extern "C" int oxh_get_rows(uint32_t qtype, const void *d_w, size_t rows, size_t
     qtype = canon_qtype(qtype);
     if (n_ids == 0) return OXH_OK;
     if (!d_w || !d_ids || !d_out) return arg_fail("oxh_get_rows: NULL pointer");
-    const size_t rb = oxh_act_kind(qtype, cols) ? oxh_row_bytes(qtype, cols) : 0;   /* every type with a matvec kernel */
+    /* every type with a matvec kernel but the codebook formats */
+    const size_t rb = (oxh_act_kind(qtype, cols) && !is_iq(qtype)) ? oxh_row_bytes(qtype, cols) : 0;
     if (rb == 0) {
         snprintf(g_err, sizeof g_err, "oxh_get_rows: qtype %u with cols %zu has no kernel here", qtype, cols);
         return OXH_DECLINED;
@@ -1440,7 +1459,9 @@ static int moe_layout(const OxhMoe *m, size_t n_tok, MoeLayout *l)
         return arg_fail("moe: n_expert must be 1..64");
     if (m->top_k == 0 || m->top_k > OXH_MOE_MAX_TOPK || m->top_k > m->n_expert)
         return arg_fail("moe: top_k must be 1..8 and at most n_expert");
-    if (oxh_act_kind(m->qtype_gate_up, m->hidden) != 2 || oxh_act_kind(m->qtype_down, m->ffn) != 2) {
+    const bool gu_ok = is_q4k(m->qtype_gate_up) || is_q5k(m->qtype_gate_up) || m->qtype_gate_up == OXH_Q6_K;
+    const bool dn_ok = is_q4k(m->qtype_down) || is_q5k(m->qtype_down) || m->qtype_down == OXH_Q6_K;
+    if (!gu_ok || !dn_ok || oxh_act_kind(m->qtype_gate_up, m->hidden) != 2 || oxh_act_kind(m->qtype_down, m->ffn) != 2) {
         snprintf(g_err, sizeof g_err, "moe: expert matrices must be Q4_K, Q5_K or Q6_K with widths in whole "
                  "256-blocks (types %u / %u, hidden %zu, ffn %zu)", m->qtype_gate_up, m->qtype_down, m->hidden, m->ffn);
         return OXH_DECLINED;

@@ -10,6 +10,7 @@ committed, this script documents how they were made.
     python tests/golden/make_golden.py dequant  # only dequant_rows.npz
     python tests/golden/make_golden.py legacy   # only legacy_formats.npz
     python tests/golden/make_golden.py q23_k    # only q23_k.npz
+    python tests/golden/make_golden.py iq       # only iq_types.npz
 
 Every array is data: inputs and the reference's outputs for them.
 """
@@ -302,6 +303,71 @@ def legacy_formats(ref):
     np.savez_compressed(os.path.join(HERE, "legacy_formats.npz"), **out)
 
 
+def iq_types(ref):
+    """iq_types.npz: IQ3_S (type id 25) and IQ1_XXXS (id 36), the two codebook formats on the reference's
+    integer path: raw-block dots (IQ3_S by its scalar and its dispatched kernel; IQ1_XXXS has one form),
+    the matvec entry points (single and batch) and a full-size checksum."""
+    rng = np.random.default_rng(20241126)
+    out = {}
+    nb, trials = 12, 24
+    F, V, Z = ctypes.c_float, ctypes.c_void_p, ctypes.c_size_t
+    forms = {"iq3_s": ("oc_oxk_dot_iq3_s_q8_k_scalar", "oc_oxk_dot_iq3_s_q8_k"),
+             "iq1_xxxs": ("oc_quant_dot_iq1_xxxs_q8_k", "oc_quant_dot_iq1_xxxs_q8_k")}
+    for name, qt, bsize in (("iq3_s", 25, 110), ("iq1_xxxs", 36, 38)):
+        w = xorshift_bytes(trials * nb * bsize, 0x9E3779B9 ^ qt).reshape(trials, nb, bsize)
+        bits = finite_scale_bits(rng, trials * nb).reshape(trials, nb)
+        w[:, :, 0] = bits & 0xFF
+        w[:, :, 1] = bits >> 8
+        act = q8k_acts(rng, trials, nb)
+        res = np.empty((trials, 2, 2), np.uint32)
+        fns = []
+        for sym in forms[name]:
+            f = getattr(ref, sym)
+            f.argtypes, f.restype = [V, Z, V], F
+            fns.append(f)
+        for t in range(trials):
+            wt, at = np.ascontiguousarray(w[t]), np.ascontiguousarray(act[t])
+            for k, blocks in enumerate((1, nb)):
+                for j, f in enumerate(fns):
+                    res[t, k, j] = np.float32(f(wt.ctypes.data, blocks, at.ctypes.data)).view(np.uint32)
+        out[name + "_raw_w"], out[name + "_raw_act"] = w, act
+        out[name + "_raw_scalar_bits"], out[name + "_raw_dispatched_bits"] = res[:, :, 0].copy(), res[:, :, 1].copy()
+    for qt, rows, cols in ((25, 40, 1280), (36, 33, 768)):
+        rb = synth.row_bytes(qt, cols)
+        wm = synth.weights(qt, rows, cols, seed=7, stream=qt)
+        x = synth.normal(cols, seed=7, stream=100 + qt)
+        o = np.zeros(rows, np.float32)
+        temp = np.zeros(cols, np.float32)
+        ref.oc_matvec_quantized(qt, wm.ctypes.data, rows, cols, rb, x.ctypes.data, o.ctypes.data,
+                                temp.ctypes.data)
+        key = "api%d_" % qt
+        out[key + "w"], out[key + "x"] = wm, x
+        out[key + "shape"] = np.array([rows, cols, rb], np.int64)
+        out[key + "out_bits"] = o.view(np.uint32).copy()
+        out[key + "act"] = temp.view(np.uint8)[:cols // 256 * 292].copy()
+        n_vec, in_stride, out_stride = 5, cols + 8, rows + 3
+        xs = synth.normal(n_vec * in_stride, seed=8, stream=qt).reshape(n_vec, in_stride)
+        outs = np.full((n_vec, out_stride), -1.0, np.float32)
+        scratch = np.zeros(ref.oc_matvec_batch_scratch_bytes(cols), np.uint8)
+        ref.oc_matvec_quantized_batch(qt, wm.ctypes.data, rows, cols, rb, xs.ctypes.data, in_stride,
+                                      outs.ctypes.data, out_stride, n_vec, temp.ctypes.data,
+                                      scratch.ctypes.data, scratch.nbytes)
+        out[key + "batch_x"] = xs
+        out[key + "batch_out_bits"] = outs.view(np.uint32).copy()
+    for qt, name in ((25, "big_iq3_s_2048x4096"), (36, "big_iq1_xxxs_2048x4096")):
+        rows, cols = 2048, 4096
+        rb = synth.row_bytes(qt, cols)
+        wm = synth.weights(qt, rows, cols, seed=0, stream=0)
+        x = synth.normal(cols, seed=0, stream=1000)
+        o = np.zeros(rows, np.float32)
+        temp = np.zeros(cols, np.float32)
+        ref.oc_matvec_quantized(qt, wm.ctypes.data, rows, cols, rb, x.ctypes.data, o.ctypes.data,
+                                temp.ctypes.data)
+        out[name + "_crc_w"] = np.array([zlib.crc32(wm.tobytes())], np.uint32)
+        out[name + "_crc_out"] = np.array([zlib.crc32(o.tobytes())], np.uint32)
+    np.savez_compressed(os.path.join(HERE, "iq_types.npz"), **out)
+
+
 def main():
     ref = oxlibs.ref()
     if ref is None:
@@ -318,6 +384,8 @@ def main():
         legacy_formats(ref)
     if only in (None, "q23_k"):
         q23_k(ref)
+    if only in (None, "iq"):
+        iq_types(ref)
     if only is not None:
         return
     rng = np.random.default_rng(20240607)

@@ -43,6 +43,8 @@ def oracle():
         lib.oxo_dot_q6_k_q8_k.argtypes = [V, Z, V, V]; lib.oxo_dot_q6_k_q8_k.restype = F
         lib.oxo_dot_q8_0_q8_0.argtypes = [V, Z, V, V]; lib.oxo_dot_q8_0_q8_0.restype = F
         lib.oxo_dot_q2_k_q8_k.argtypes = [V, Z, V, V]; lib.oxo_dot_q2_k_q8_k.restype = F
+        lib.oxo_dot_iq3_s_q8_k.argtypes = [V, Z, V, V]; lib.oxo_dot_iq3_s_q8_k.restype = F
+        lib.oxo_dot_iq1_xxxs_q8_k.argtypes = [V, Z, V, V]; lib.oxo_dot_iq1_xxxs_q8_k.restype = F
         lib.oxo_dot_q3_k_q8_k.argtypes = [V, Z, V, V]; lib.oxo_dot_q3_k_q8_k.restype = F
         for n in ("q4_0", "q4_1", "q5_0", "q5_1", "al5_xs"):
             f = getattr(lib, "oxo_dot_%s_q8_0" % n)
