@@ -230,6 +230,15 @@ int oxh_gemv_segments_fused(uint32_t qtype, const OxhSegment *segs, size_t n_seg
  * pass between operations may be ordinary oxh_malloc memory.  An operation
  * must not store a result over one of its own inputs.
  *
+ * A plan in which NO operation conflicts with an earlier one (every input is
+ * there when the launch starts) stages its inputs ahead of the chain: each
+ * vector is normalised and quantised once, by one workgroup, into device
+ * memory the plan owns (about 1.3 bytes per input value), all workgroups meet
+ * once, and from then on an operation's quantised input is copied into LDS
+ * while the previous operation runs.  Same results; oxh_plan_prestaged says
+ * whether a plan runs this way (OXH_PLAN_PRESTAGE=0 in the environment at
+ * creation keeps such a plan on the chained kernel).
+ *
  * All workgroups must be resident together (one per compute unit; the kernel
  * needs the whole device, so do not run other kernels beside a plan launch).
  * Every wait is bounded: after `polls` unsuccessful polls (about a microsecond
@@ -255,6 +264,8 @@ int oxh_plan_status(OxhPlan *plan, void *stream);
 /* Operations, how many of them wait for an earlier one, workgroups, LDS bytes
  * per workgroup.  Any pointer may be NULL. */
 int oxh_plan_info(const OxhPlan *plan, size_t *n_ops, size_t *n_waits, size_t *workgroups, size_t *lds_bytes);
+/* 1 when the plan stages its inputs ahead of the chain (see above), else 0. */
+int oxh_plan_prestaged(const OxhPlan *plan);
 /* The poll limit of every wait.  With `phantom_workgroup` set the waits also
  * expect a workgroup that does not exist, so every wait runs into the limit:
  * the way to test the give-up path without hanging anything. */

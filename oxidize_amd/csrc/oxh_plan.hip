@@ -26,6 +26,15 @@
  *     fences: everything one operation hands to another (outputs, residual
  *     sums) is stored and loaded with system-coherent accesses that bypass the
  *     L2s, and so are the counters.
+ *   - A plan none of whose operations reads what another one writes (a decode
+ *     step's matrices applied to inputs that are all there when the launch
+ *     starts) runs on a second kernel, k_plan_ext: each input vector is
+ *     normalised and quantised ONCE, by one workgroup, into a staged image in
+ *     device memory before the chain starts; after one device-wide wait every
+ *     workgroup copies the image of operation i + 1 straight into LDS while it
+ *     works on operation i.  An operation boundary then costs the row sums
+ *     and one workgroup barrier; no workgroup reads or quantises a vector that
+ *     255 others quantise as well.
  *   - Every wait is bounded: after `spin_limit` polls a workgroup raises the
  *     plan's error word and leaves, and every other workgroup leaves at its
  *     next wait, so a launch that cannot make progress (not all workgroups
@@ -77,6 +86,9 @@ struct PlanOp {
     gaddr x, pro_b, pro_add;
     gaddr pro_sum_out, pro_out;
     gaddr act_out;
+    gaddr xq;                       /* where the staged (quantised) input of this operation is kept when the
+                                     * plan stages its inputs ahead of the chain; else 0 */
+    gaddr reserved;
     PlanSeg s[PLAN_MAX_SEGS];
 };
 
@@ -104,6 +116,7 @@ struct PlanLds {
     uint32_t act_bytes;             /* one staged activation (two are kept, used in turn) */
     uint32_t outs_off, red_off, terms_off, terms_per_wave;   /* bytes; terms_per_wave in floats */
     uint32_t table_off;             /* the operation table's copy */
+    uint32_t terms_wg;              /* k_plan_ext: floats of one workgroup-wide term table (two are kept) */
 };
 
 /* ─── coherent accesses ───────────────────────────────────────────────── */
@@ -238,6 +251,49 @@ __device__ __forceinline__ PWork plan_work(const PlanOp *op, uint32_t wave)
     k.paired = w2 != 0u ? 1u : 0u;
     k.src.b = gptr<const uint8_t>((k.paired ? w2 : w) + off);
     k.nblk = k.paired ? 2u * k.src.n1 : k.src.n1;
+    return k;
+}
+
+/* The same rows dealt evenly: the workgroup's rows of the first matrix followed by its rows of the
+ * paired one form one list, and wave w takes an equal contiguous run of it (a pair of 56 rows each is
+ * seven rows per wave, where dealing pairs gives eight waves four pairs and eight waves three).  A
+ * wave's rows of the two matrices are then not the same rows, so the term table is the workgroup's
+ * (row0 = the wave's first list row) and rows are summed after a workgroup barrier. */
+__device__ __forceinline__ PWork plan_work_flat(const PlanOp *op, uint32_t wave)
+{
+    PWork k;
+    const uint32_t wg = blockIdx.x, n = uni(op->n_segs);
+    uint32_t si = 0;
+#pragma unroll
+    for (uint32_t i = 1; i < PLAN_MAX_SEGS; i++)
+        if (i < n && wg >= uni(op->s[i].wg_begin)) si = i;
+    const PlanSeg *sg = &op->s[si];
+    const gaddr w = uni(sg->w), w2 = uni(sg->w2), out = uni(sg->out);
+    const uint32_t wg_begin = uni(sg->wg_begin), sq = uni(sg->rows_q), srem = uni(sg->rows_rem);
+    const bool idle = wg >= uni(op->n_wg);
+    const uint32_t wi0 = (wg - wg_begin) * PLAN_W;
+    k.kind = uni(op->kind);
+    k.out = gptr<float>(out);
+    k.paired = w2 != 0u ? 1u : 0u;
+    k.wg_row0 = wi0 * sq + min(wi0, srem);
+    k.wg_rows = idle ? 0u : (wi0 + PLAN_W) * sq + min(wi0 + PLAN_W, srem) - k.wg_row0;
+    const uint32_t B = uni(op->blocks);
+    const gaddr rb = (gaddr)(B * plan_block_bytes(k.kind));
+    const uint32_t F = k.paired ? 2u * k.wg_rows : k.wg_rows;
+    const uint32_t q = F / PLAN_W, rem = F % PLAN_W;
+    const uint32_t f0 = wave * q + min(wave, rem), cnt = q + (wave < rem ? 1u : 0u);
+    /* rows of the first matrix in this wave's run, and where its rows of the second one start */
+    const uint32_t na = f0 < k.wg_rows ? min(cnt, k.wg_rows - f0) : 0u;
+    const uint32_t b0 = f0 < k.wg_rows ? 0u : f0 - k.wg_rows;
+    const gaddr first = w + (gaddr)(k.wg_row0 + min(f0, k.wg_rows)) * rb;
+    const gaddr second = (k.paired ? w2 : w) + (gaddr)(k.wg_row0 + b0) * rb;
+    /* a run that lies wholly in the second matrix is a one-matrix list of that one */
+    k.src.a = gptr<const uint8_t>(na != 0u ? first : second);
+    k.src.b = gptr<const uint8_t>(second);
+    k.src.n1 = (na != 0u ? na : cnt) * B;
+    k.row0 = f0;
+    k.nrows = cnt;
+    k.nblk = cnt * B;
     return k;
 }
 
@@ -613,6 +669,152 @@ k_plan(const PlanOp *__restrict__ ops, uint32_t n_ops, const PlanSync sy, const 
     }
 }
 
+/* ─── plans whose inputs are all there at launch ─────────────────────── */
+
+/* global -> LDS, 16 bytes per lane, past the L2s (the image was written by another workgroup a moment
+ * ago, and this XCD's L2 may still hold the previous launch's bytes at the same address): lane l reads
+ * base + off, its bytes land at lds_addr + 16*l.  base and lds_addr are wave-uniform. */
+__device__ __forceinline__ void plan_dma16(const uint8_t *base, uint32_t off, uint32_t lds_addr)
+{
+    asm volatile("s_mov_b32 m0, %0\n\t"
+                 "global_load_lds_dwordx4 %1, %2 sc0 sc1"
+                 :: "s"(lds_addr), "v"(off), "s"(base) : "memory");
+}
+
+__device__ __forceinline__ uint32_t plan_image_bytes(uint32_t kind, uint32_t blocks)
+{
+    return kind == PLAN_Q6_K ? q8k6_lds_bytes(blocks) : q8k_lds_bytes(blocks);
+}
+
+/* the staged input of an operation into LDS at byte address lds_addr, 1 KB pieces dealt to the waves */
+__device__ __forceinline__ void plan_image_fetch(const PlanOp *op, uint32_t lds_addr, uint32_t lane, uint32_t wave)
+{
+    const uint32_t bytes = plan_image_bytes(uni(op->kind), uni(op->blocks));
+    const uint8_t *img = gptr<const uint8_t>(uni(op->xq));
+    for (uint32_t k = wave * 1024u; k < bytes; k += PLAN_W * 1024u)
+        if (k + 16u * lane < bytes) plan_dma16(img + k, 16u * lane, lds_addr + k);
+}
+
+template <bool HAS_Q5>
+__global__ __launch_bounds__(1024) void
+k_plan_ext(const PlanOp *__restrict__ ops, uint32_t n_ops, const PlanSync sy, const PlanLds ld)
+{
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    const uint32_t lds_base = (uint32_t)(size_t)(__attribute__((address_space(3))) uint8_t *)lds;
+    const uint32_t lane = threadIdx.x & 63u, wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const uint32_t base = cload(sy.flags + blockIdx.x);
+    float *const red = reinterpret_cast<float *>(lds + ld.red_off);
+    int *const s_ok = reinterpret_cast<int *>(red + 24);
+    float *const terms_wg = reinterpret_cast<float *>(lds + ld.terms_off);
+    {
+        const u32x4 *src = reinterpret_cast<const u32x4 *>(ops);
+        u32x4 *dst = reinterpret_cast<u32x4 *>(lds + ld.table_off);
+        const uint32_t n16 = n_ops * (uint32_t)(sizeof(PlanOp) / 16u);
+        for (uint32_t k = threadIdx.x; k < n16; k += 1024u) dst[k] = src[k];
+    }
+    __syncthreads();
+    const PlanOp *const tab = reinterpret_cast<const PlanOp *>(lds + ld.table_off);
+
+    /* Inputs first: workgroup g stages the vectors of operations g, g + grid, ... exactly as the chained
+     * kernel stages them (prologue, Q8_K quantisation, the layout the passes read) and stores the LDS
+     * image with accesses every XCD sees.  The side outputs of a prologue are written here, once. */
+    for (uint32_t j = blockIdx.x; j < n_ops; j += gridDim.x) {
+        const OpHead op = plan_head(&tab[j]);
+        XStage xs;
+#pragma unroll
+        for (int u = 0; u < 4; u++) xs.x[u] = xs.t[u] = xs.b[u] = XRegs{ 0.f, 0.f, 0.f, 0.f };
+        plan_stage_issue(op, xs, false, lane, wave);
+        if (op.kind == PLAN_Q6_K) plan_stage_finish<1>(op, xs, lds, red, true, lane, wave);
+        else                      plan_stage_finish<0>(op, xs, lds, red, true, lane, wave);
+        __syncthreads();
+        const uint32_t bytes = plan_image_bytes(op.kind, op.blocks);
+        const CohBuf img = coh_buf(gptr<uint8_t>(uni(tab[j].xq)));
+        for (uint32_t k = threadIdx.x * 16u; k < bytes; k += 16384u)
+            __builtin_amdgcn_raw_buffer_store_b128(*reinterpret_cast<const u32x4 *>(lds + k), img, (int)k, 0,
+                                                   OXH_SYSTEM_COHERENT);
+        __syncthreads();
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    if (threadIdx.x == 0u) cstore(sy.flags + blockIdx.x, base + 1u);
+
+    /* One trip = requests for operation i, the workgroup barrier, rows and outputs of operation i - 1
+     * (summed from the workgroup's term table by the first wg_rows threads while the other waves go
+     * on), then the passes of operation i into the other term table.  The weight registers are free
+     * when a trip starts, so the two requested sets are not carried around the loop, and the requests go
+     * out before the barrier: the weight stream does not stop at an operation boundary.  The staged
+     * input of operation i + 1 is fetched into the other LDS buffer during operation i; the wait at
+     * the top of a trip finds it (and the output stores) long complete, and the one barrier of a trip
+     * both publishes it to the other waves and says that nobody reads the buffer it replaces. */
+    PWork cur = plan_work_flat(&tab[0], wave);
+    PWork prev = cur;
+    uint32_t p_blocks = 0, p_stride = 0;
+    for (uint32_t i = 0;; i++) {
+        uint32_t ln = lane;
+        asm volatile("" : "+v"(ln));
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        plan_stamp(sy, i < n_ops ? i : n_ops - 1u, i < n_ops ? 0u : 5u, ln, wave);
+        WSet A, B;
+        A.a = A.b = A.c = A.d = A.e = u32x4{ 0u, 0u, 0u, 0u };
+        B.a = B.b = B.c = B.d = B.e = A.a;
+        if (i < n_ops) {
+            plan_prefetch<HAS_Q5>(cur, A, 0u, ln);
+            plan_prefetch<HAS_Q5>(cur, B, 1u, ln);
+        }
+        if (i > 0u) {
+            /* every wave has finished operation i - 1 and has its pieces of this operation's input */
+            lds_barrier();
+            plan_stamp(sy, i - 1u, 6, ln, wave);
+            const float *tb = terms_wg + (size_t)((i - 1u) & 1u) * ld.terms_wg;
+            const CohBuf dst = coh_buf(prev.out + prev.wg_row0);
+            for (uint32_t r = threadIdx.x; r < prev.wg_rows; r += 1024u) {
+                float v = row_sum_one<1>(tb + __umul24(r, p_stride), p_blocks);
+                if (prev.paired) {
+                    const float u = row_sum_one<1>(tb + __umul24(prev.wg_rows + r, p_stride), p_blocks);
+                    const float sig = 1.0f / (1.0f + expf(-v));
+                    v = v * sig * u;
+                }
+                cstore_f32(dst, r * 4u, v);
+            }
+        } else {
+            /* every input is staged once every workgroup has said so */
+            if (!plan_wait(sy, base + 1u, s_ok, ln, wave)) return;
+            plan_image_fetch(&tab[0], lds_base, ln, wave);
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            __syncthreads();
+        }
+        if (i == n_ops) break;
+        if (i + 1u < n_ops) plan_image_fetch(&tab[i + 1u], lds_base + ((i + 1u) & 1u) * ld.act_bytes, ln, wave);
+        plan_stamp(sy, i, 1, ln, wave);
+
+        const PlanOp *const op = &tab[i];
+        const uint32_t Bk = uni(op->blocks);
+        const uint8_t *act = lds + (size_t)(i & 1u) * ld.act_bytes;
+        PWork nx = cur;
+        if (i + 1u < n_ops) nx = plan_work_flat(&tab[i + 1u], wave);
+        GemvParams gp;
+        gp.blocks = Bk;
+        gp.magic = uni(op->magic);
+        gp.term_stride = uni(op->term_stride);
+        gp.rows_cap = uni(op->rows_cap);
+        gp.dump = nullptr;
+        float *const terms = terms_wg + (size_t)(i & 1u) * ld.terms_wg + __umul24(cur.row0, gp.term_stride);
+        if (cur.nblk != 0u) {
+            if (cur.kind == PLAN_Q6_K)      plan_passes_q6(A, B, cur, gp, act, q8k6_lds_bytes(Bk), terms, ln);
+            else if (HAS_Q5 && cur.kind == PLAN_Q5_K) plan_passes_q45<true>(A, B, cur, gp, act, q8k_lds_bytes(Bk), terms, ln);
+            else                            plan_passes_q45<false>(A, B, cur, gp, act, q8k_lds_bytes(Bk), terms, ln);
+        }
+        plan_stamp(sy, i, 4, ln, wave);
+        prev = cur;
+        cur = nx;
+        p_blocks = Bk;
+        p_stride = gp.term_stride;
+    }
+    /* the next launch's base */
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    if (threadIdx.x == 0u) cstore(sy.flags + blockIdx.x, base + 2u);
+}
+
 /* ─── host side ───────────────────────────────────────────────────────── */
 
 struct OxhPlan {
@@ -625,7 +827,16 @@ struct OxhPlan {
     bool has_q5;
     uint64_t *d_stamps;
     uint32_t n_waits;               /* operations that wait (for callers' curiosity) */
+    bool ext;                       /* no operation depends on another: inputs are staged ahead (k_plan_ext) */
+    uint8_t *d_img;                 /* the staged inputs */
 };
+
+static const void *plan_kernel(const OxhPlan *pl)
+{
+    if (pl->ext)
+        return pl->has_q5 ? reinterpret_cast<const void *>(k_plan_ext<true>) : reinterpret_cast<const void *>(k_plan_ext<false>);
+    return pl->has_q5 ? reinterpret_cast<const void *>(k_plan<true>) : reinterpret_cast<const void *>(k_plan<false>);
+}
 
 #define PLAN_TRY(call)                                                                      \
     do {                                                                                    \
@@ -703,7 +914,8 @@ extern "C" int oxh_plan_create(const OxhPlanOp *ops, size_t n_ops, OxhPlan **out
         free(h); free(reads); free(writes);
         return oxh_internal_errorf(OXH_ERR_NOMEM, "out of host memory building a plan");
     }
-    uint32_t max_act = 0, max_cap_terms = 0, max_wg_rows = 0, n_waits = 0;
+    uint32_t max_act = 0, max_cap_terms = 0, max_wg_rows = 0, max_wg_terms = 0, n_waits = 0;
+    size_t img_bytes = 0;
     bool has_q5 = false;
     rc = OXH_OK;
     for (size_t i = 0; i < n_ops && !rc; i++) {
@@ -776,11 +988,15 @@ extern "C" int oxh_plan_create(const OxhPlanOp *ops, size_t n_ops, OxhPlan **out
             d.s[k].rows_rem = (uint32_t)(rows[k] % waves);
             const uint32_t per_wg = (uint32_t)((rows[k] / waves + 1) * PLAN_W);
             if (per_wg > max_wg_rows) max_wg_rows = per_wg;
+            const uint32_t flat = per_wg * (paired[k] ? 2u : 1u) * d.term_stride;
+            if (flat > max_wg_terms) max_wg_terms = flat;
             wg += n_wg[k];
         }
         d.n_wg = wg;
         const uint32_t act = kind == PLAN_Q6_K ? q8k6_lds_bytes(d.blocks) : q8k_lds_bytes(d.blocks);
         if (act > max_act) max_act = act;
+        d.xq = (gaddr)img_bytes;                    /* offset for now; the base is added once it exists */
+        img_bytes += (act + 255u) & ~(size_t)255u;
         if (cap * d.term_stride > max_cap_terms) max_cap_terms = cap * d.term_stride;
 
         /* what the operation reads and writes, for the dependency scan */
@@ -828,12 +1044,18 @@ extern "C" int oxh_plan_create(const OxhPlanOp *ops, size_t n_ops, OxhPlan **out
     pl->grid = grid;
     pl->n_waits = n_waits;
     pl->has_q5 = has_q5;
+    {
+        /* OXH_PLAN_PRESTAGE=0 keeps a plan of independent operations on the chained kernel */
+        const char *ps = getenv("OXH_PLAN_PRESTAGE");
+        pl->ext = n_waits == 0 && !(ps && ps[0] == '0');
+    }
     pl->ld.act_bytes = (max_act + 15u) & ~15u;
     pl->ld.outs_off = 2u * pl->ld.act_bytes;
     pl->ld.red_off = pl->ld.outs_off + ((max_wg_rows * 4u + 15u) & ~15u);
     pl->ld.terms_off = pl->ld.red_off + 128u;
     pl->ld.terms_per_wave = max_cap_terms;
-    pl->ld.table_off = (pl->ld.terms_off + PLAN_W * max_cap_terms * 4u + 15u) & ~15u;
+    pl->ld.terms_wg = (max_wg_terms + 3u) & ~3u;
+    pl->ld.table_off = (pl->ld.terms_off + (pl->ext ? 2u * pl->ld.terms_wg : PLAN_W * max_cap_terms) * 4u + 15u) & ~15u;
     pl->lds_bytes = (size_t)pl->ld.table_off + n_ops * sizeof(PlanOp);
     const char *sl = getenv("OXH_PLAN_SPIN_LIMIT");
     pl->spin_limit = sl && *sl ? (uint32_t)strtoul(sl, nullptr, 10) : 4000000u;
@@ -841,7 +1063,7 @@ extern "C" int oxh_plan_create(const OxhPlanOp *ops, size_t n_ops, OxhPlan **out
         free(h); free(pl);
         return oxh_internal_errorf(OXH_ERR_TOO_WIDE, "plan: the staged activation, the row tables and the table of %zu operations (%zu bytes each) do not fit 160 KiB of LDS; split the chain into several plans", n_ops, sizeof(PlanOp));
     }
-    const void *kernel = has_q5 ? reinterpret_cast<const void *>(k_plan<true>) : reinterpret_cast<const void *>(k_plan<false>);
+    const void *kernel = plan_kernel(pl);
     {
         hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         if (e != hipSuccess) { free(h); free(pl); return oxh_internal_errorf(OXH_ERR_HIP, "HIP error in hipFuncSetAttribute: %s", hipGetErrorString(e)); }
@@ -855,6 +1077,8 @@ extern "C" int oxh_plan_create(const OxhPlanOp *ops, size_t n_ops, OxhPlan **out
         return oxh_internal_errorf(OXH_ERR_HIP, "plan: the device cannot hold one workgroup of the plan kernel per compute unit");
     }
     e = hipMalloc((void **)&pl->d_ops, n_ops * sizeof(PlanOp));
+    if (e == hipSuccess && pl->ext) e = hipMalloc((void **)&pl->d_img, img_bytes);
+    for (size_t i = 0; i < n_ops; i++) h[i].xq = pl->ext ? (gaddr)(uintptr_t)pl->d_img + h[i].xq : 0u;
     if (e == hipSuccess) e = hipMalloc((void **)&pl->d_sync, (PLAN_MAX_WG + 8u) * sizeof(uint32_t));
     if (e == hipSuccess) e = hipMemcpy(pl->d_ops, h, n_ops * sizeof(PlanOp), hipMemcpyHostToDevice);
     if (e == hipSuccess) e = hipMemset(pl->d_sync, 0, (PLAN_MAX_WG + 8u) * sizeof(uint32_t));
@@ -862,6 +1086,7 @@ extern "C" int oxh_plan_create(const OxhPlanOp *ops, size_t n_ops, OxhPlan **out
     free(h);
     if (e != hipSuccess) {
         if (pl->d_ops) (void)hipFree(pl->d_ops);
+        if (pl->d_img) (void)hipFree(pl->d_img);
         if (pl->d_sync) (void)hipFree(pl->d_sync);
         free(pl);
         return oxh_internal_errorf(e == hipErrorOutOfMemory ? OXH_ERR_NOMEM : OXH_ERR_HIP, "plan: %s", hipGetErrorString(e));
@@ -880,12 +1105,17 @@ extern "C" int oxh_plan_launch(OxhPlan *pl, void *stream)
     sy.n_wait = pl->grid + pl->phantom;
     sy.spin_limit = pl->spin_limit;
     sy.stamps = pl->d_stamps;
-    if (pl->has_q5)
-        hipLaunchKernelGGL(k_plan<true>, dim3(pl->grid), dim3(1024), pl->lds_bytes, st, (const PlanOp *)pl->d_ops,
-                           pl->n_ops, sy, pl->ld);
-    else
-        hipLaunchKernelGGL(k_plan<false>, dim3(pl->grid), dim3(1024), pl->lds_bytes, st, (const PlanOp *)pl->d_ops,
-                           pl->n_ops, sy, pl->ld);
+#define PLAN_LAUNCH(K)                                                                                  \
+    hipLaunchKernelGGL(K, dim3(pl->grid), dim3(1024), pl->lds_bytes, st, (const PlanOp *)pl->d_ops,    \
+                       pl->n_ops, sy, pl->ld)
+    if (pl->ext) {
+        if (pl->has_q5) PLAN_LAUNCH(k_plan_ext<true>);
+        else            PLAN_LAUNCH(k_plan_ext<false>);
+    } else {
+        if (pl->has_q5) PLAN_LAUNCH(k_plan<true>);
+        else            PLAN_LAUNCH(k_plan<false>);
+    }
+#undef PLAN_LAUNCH
     PLAN_TRY(hipGetLastError());
     return OXH_OK;
 }
@@ -898,6 +1128,11 @@ extern "C" int oxh_plan_info(const OxhPlan *pl, size_t *n_ops, size_t *n_waits, 
     if (workgroups) *workgroups = pl->grid;
     if (lds_bytes) *lds_bytes = pl->lds_bytes;
     return OXH_OK;
+}
+
+extern "C" int oxh_plan_prestaged(const OxhPlan *pl)
+{
+    return pl && pl->ext ? 1 : 0;
 }
 
 extern "C" int oxh_plan_set_spin_limit(OxhPlan *pl, uint32_t polls, int phantom_workgroup)
@@ -935,6 +1170,7 @@ extern "C" int oxh_plan_destroy(OxhPlan *pl)
     if (!pl) return OXH_OK;
     hipError_t e = hipDeviceSynchronize();
     if (pl->d_ops) (void)hipFree(pl->d_ops);
+    if (pl->d_img) (void)hipFree(pl->d_img);
     if (pl->d_sync) (void)hipFree(pl->d_sync);
     free(pl);
     if (e != hipSuccess) return oxh_internal_errorf(OXH_ERR_HIP, "HIP error in hipDeviceSynchronize: %s", hipGetErrorString(e));

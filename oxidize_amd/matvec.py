@@ -295,7 +295,9 @@ class Plan:
     def info(self):
         v = [ctypes.c_size_t() for _ in range(4)]
         check(lib().oxh_plan_info(self.handle, *[ctypes.byref(x) for x in v]))
-        return dict(zip(("n_ops", "n_waits", "workgroups", "lds_bytes"), [int(x.value) for x in v]))
+        out = dict(zip(("n_ops", "n_waits", "workgroups", "lds_bytes"), [int(x.value) for x in v]))
+        out["prestaged"] = bool(lib().oxh_plan_prestaged(self.handle))
+        return out
 
     def set_spin_limit(self, polls, phantom_workgroup=False):
         check(lib().oxh_plan_set_spin_limit(self.handle, polls, int(phantom_workgroup)))

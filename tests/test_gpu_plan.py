@@ -34,6 +34,7 @@ def test_independent_set_matches_single_launches_and_oracle(oxh, hidden, kv, ffn
     plan = mv.Plan(d.plan_ops())
     info = plan.info()
     assert info["n_ops"] == 4 * layers and info["n_waits"] == 0      # nothing depends on anything here
+    assert info["prestaged"]                                          # so the inputs are staged ahead
     for rep in range(2):
         plan.launch()
         assert plan.status() == 0
@@ -116,6 +117,83 @@ def test_mixed_types_with_q5k(oxh):
         assert o.oxo_matvec_quantized(qt, host[i].ctypes.data, rows, hidden, synth.row_bytes(qt, hidden),
                                       x.ctypes.data, want.ctypes.data, tmp.ctypes.data) == 0
         assert np.array_equal(bits(outs[i].download(np.float32, rows)), bits(want)), qt
+
+
+def test_prestaged_plan_follows_its_inputs_from_launch_to_launch(oxh, monkeypatch):
+    """A plan of independent operations keeps every staged input in memory of its own and re-reads it in
+    every workgroup: new input values before a launch must reach every output of that launch (nothing
+    may come from a cache line or an image of the launch before), with and without prologues, and the
+    chained kernel must give the same bits for the same plan."""
+    hidden, ffn, eps = 1024, 3072, 1e-5
+    shapes = [(Q4K, 1800, hidden, None), (Q6K, 1024, ffn, None), (Q4K, 2 * 1536, hidden, "rms"),
+              (Q5K, 640, hidden, "add_rms"), (Q6K, 512, hidden, "swiglu"), (Q4K, 777, hidden, None)]
+    bufs, ops = [], []
+    for i, (qt, rows, cols, pro) in enumerate(shapes):
+        w = mv.DeviceBuffer.from_host(synth.weights(qt, rows, cols, seed=21, stream=i))
+        b = dict(w=w, x=mv.DeviceBuffer(cols * 4), out=mv.DeviceBuffer(rows * 4), act=mv.DeviceBuffer(mv.act_bytes(qt, cols)),
+                 g=mv.DeviceBuffer.from_host((synth.normal(cols, seed=21, stream=100 + i) * np.float32(0.1) + np.float32(1)).astype(np.float32)),
+                 add=mv.DeviceBuffer(cols * 4), pout=mv.DeviceBuffer(cols * 4), sout=mv.DeviceBuffer(cols * 4))
+        if pro == "rms" and i == 2:        # a gate/up pair
+            half = rows // 2
+            segs = mv.make_segments([(w.ptr, b["out"].ptr, half, 0, 0, w.ptr + half * synth.row_bytes(qt, cols))])
+        else:
+            segs = mv.make_segments([(w.ptr, b["out"].ptr, rows, 0)])
+        op = dict(qtype=qt, segs=segs, cols=cols, d_x=b["x"].ptr, d_act_out=b["act"].ptr)
+        if pro == "rms":
+            op.update(kind=mv.PRO_RMSNORM, d_b=b["g"].ptr, eps=eps, d_pro_out=b["pout"].ptr)
+        elif pro == "add_rms":
+            op.update(kind=mv.PRO_RMSNORM, d_b=b["g"].ptr, eps=eps, d_add=b["add"].ptr, d_sum_out=b["sout"].ptr,
+                      d_pro_out=b["pout"].ptr)
+        elif pro == "swiglu":
+            op.update(kind=mv.PRO_SWIGLU, d_b=b["add"].ptr, d_pro_out=b["pout"].ptr)
+        bufs.append(b)
+        ops.append(op)
+    plan = mv.Plan(ops)
+    assert plan.info()["prestaged"]
+    monkeypatch.setenv("OXH_PLAN_PRESTAGE", "0")
+    chained = mv.Plan(ops)
+    monkeypatch.delenv("OXH_PLAN_PRESTAGE")
+    assert not chained.info()["prestaged"] and chained.info()["n_waits"] == 0
+
+    def state():
+        out = []
+        for (qt, rows, cols, pro), b in zip(shapes, bufs):
+            n_out = rows // 2 if (pro == "rms") else rows
+            out.append((b["out"].download(np.float32, n_out), b["act"].download(np.uint8, mv.act_bytes(qt, cols)),
+                        b["pout"].download(np.float32, cols), b["sout"].download(np.float32, cols)))
+        return out
+
+    def clear():
+        for b in bufs:
+            for k in ("out", "act", "pout", "sout"):
+                mv.lib().oxh_memset(ctypes.c_void_p(b[k].ptr), 0xFF, b[k].nbytes, None)
+
+    for rep in range(3):
+        for i, ((qt, rows, cols, pro), b) in enumerate(zip(shapes, bufs)):
+            b["x"].upload(synth.normal(cols, seed=50 + rep, stream=i))
+            b["add"].upload(synth.normal(cols, seed=50 + rep, stream=40 + i))
+        clear()
+        for op in ops:          # the reference result: the same calls one by one
+            if op.get("kind"):
+                mv.gemv_segments_fused(op["qtype"], op["segs"], op["cols"], op["d_x"], op["cols"], op["kind"], op["d_b"],
+                                       op.get("eps", 0.0), op.get("d_pro_out"), op["d_act_out"], 1, 0, None,
+                                       d_add=op.get("d_add"), d_sum_out=op.get("d_sum_out"))
+            else:
+                mv.gemv_segments_f32(op["qtype"], op["segs"], op["cols"], op["d_x"], op["cols"], op["d_act_out"])
+        mv.sync()
+        want = state()
+        for p in (plan, chained):
+            clear()
+            p.launch()
+            assert p.status() == 0
+            got = state()
+            for i, (w_, g_) in enumerate(zip(want, got)):
+                assert np.array_equal(bits(w_[0]), bits(g_[0])), (rep, i, "out")
+                assert np.array_equal(w_[1], g_[1]), (rep, i, "act")
+                assert np.array_equal(bits(w_[2]), bits(g_[2])), (rep, i, "prologue out")
+                assert np.array_equal(bits(w_[3]), bits(g_[3])), (rep, i, "sum out")
+    plan.destroy()
+    chained.destroy()
 
 
 def test_a_wait_that_cannot_be_satisfied_gives_up(oxh):
