@@ -14,7 +14,8 @@ are resident in HBM before the timed region starts.
 Prints ONE JSON line.  `value` is whole-step algorithmic GB/s (packed weights
 at their on-disk size + f32 activations in + f32 outputs out, divided by the
 wall time of the K timed steps).  `roofline` is the kernel the step runs in
-(k_plan: one launch = one step), timed with HIP events on the launch stream.
+(k_plan_ext: one launch = one step, every input quantised once ahead of the
+chain), timed with HIP events on the launch stream.
 `cpu_baseline` is the reference's own CPU code (oracle/_ref, or the oracle
 port when that was never built) on this host's cores, streaming eight distinct
 layers in turn (1.1 GB: beyond the host's last-level cache).
@@ -33,9 +34,9 @@ HBM_PEAK_GBPS = 8000.0
 # 32410.7 KiB x 2.000, WRITE_SIZE 116.57 KiB x 1.000; the factors are what the
 # same counters read for a 256 MiB device-to-device copy).  Not measured live.
 GATE_UP_TRAFFIC_BYTES = 66496518
-# HBM bytes one k_plan launch (a whole 32-layer step) moves, measured the same way; None until a
-# counter run of this kernel has been taken.
-PLAN_STEP_TRAFFIC_BYTES = None
+# HBM bytes one k_plan_ext launch (a whole 32-layer step) moves, measured the same way: FETCH_SIZE
+# 2168740.9 KiB x 1.9998, WRITE_SIZE 7322.03 KiB x 1.000 (algorithmic: 4419223552, ratio 1.0067).
+PLAN_STEP_TRAFFIC_BYTES = 4448654782
 INT8_PEAK_TOPS = 5033.0     # dense int8 MFMA: 256 CU x 2.4 GHz x 8192 op/clk/CU
 
 
@@ -460,8 +461,10 @@ def cpu_baseline(layers_sample=8, min_seconds=2.5, cores=None):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=3)
+    # a launch of the step kernel takes 0.8-1.1 ms for the first thirty or so launches after the device
+    # was idle and settles after that (clock and memory power states), hence the long default warm-up
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=40)
     ap.add_argument("--layers", type=int, default=32, help=argparse.SUPPRESS)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--mode", choices=["plan", "graph", "launches"], default="plan",
@@ -551,7 +554,8 @@ def main():
     per_launch["sum_x_layers_ms"] = round(sum(v["us"] for v in per_launch.values()) * ds.layers / 1e3, 4)
 
     if args.mode == "plan":
-        k_name, k_bytes, k_us = "k_plan (one launch = one decode step of 128 matmuls)", step_bytes, ev_ms * 1e3 / args.steps
+        k_name = ("k_plan_ext" if plan.info()["prestaged"] else "k_plan") + " (one launch = one decode step of 128 matmuls)"
+        k_bytes, k_us = step_bytes, ev_ms * 1e3 / args.steps
         k_traffic = PLAN_STEP_TRAFFIC_BYTES if ds.layers == 32 else None
     else:
         k_name, k_bytes, k_us = "k_gemv_q4_k (gate/up 28672x4096)", per_launch["gate_up"]["bytes"], per_launch["gate_up"]["us"]
