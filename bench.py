@@ -275,6 +275,41 @@ def secondary_figures(mv, synth):
         c.free()
     d_x.free()
     d_o.free()
+    # the Q6_K down projection in the two layouts the decode kernels read: the file layout and the
+    # regrouped copy the decode set keeps (same bytes); eight distinct copies in turn (386 MB: from HBM)
+    rows, cols = 4096, 14336
+    w = synth.weights(Q6K, rows, cols, seed=0, stream=7)
+    plain = [mv.DeviceBuffer.from_host(w) for _ in range(8)]
+    grouped = []
+    for c in plain:
+        g = mv.DeviceBuffer(w.nbytes)
+        mv.q6_k_group(c.ptr, rows, cols, g.ptr)
+        grouped.append(g)
+    mv.sync()
+    d_x = mv.DeviceBuffer.from_host(synth.normal(cols, seed=0, stream=2006))
+    d_o = mv.DeviceBuffer(rows * 4)
+    seg_p = [mv.make_segments([(c.ptr, d_o.ptr, rows, 0)]) for c in plain]
+    seg_g = [mv.make_segments([(c.ptr, d_o.ptr, rows, 0)]) for c in grouped]
+    state = {"i": 0}
+
+    def run_plain():
+        state["i"] += 1
+        mv.gemv_segments_f32(Q6K, seg_p[state["i"] % 8], cols, d_x.ptr, cols, None, 1, rows)
+
+    def run_grouped():
+        state["i"] += 1
+        mv.gemv_segments_f32(mv.Q6_K_G8, seg_g[state["i"] % 8], cols, d_x.ptr, cols, None, 1, rows)
+
+    nbytes = w.nbytes + 4 * cols + 4 * rows
+    us_p, us_g = timed(run_plain, 64, mv), timed(run_grouped, 64, mv)
+    out["q6k_down_4096x14336_layouts"] = {
+        "file_layout": {"us": round(us_p, 2), "gbps": round(nbytes / us_p / 1e3, 1)},
+        "regrouped_in_eights": {"us": round(us_g, 2), "gbps": round(nbytes / us_g / 1e3, 1)},
+        "note": "k_gemv_q6_k against k_gemv_q6_kg, back-to-back launches, launch gaps included"}
+    for c in plain + grouped:
+        c.free()
+    d_x.free()
+    d_o.free()
     # Q8_0 lm_head (configuration 2), batch 1 and 8
     rows, cols = 151936, 896
     w = synth.weights(Q80, rows, cols, seed=0, stream=5)
@@ -578,6 +613,7 @@ def main():
         "config": {"workload": "llama3-8b decode GEMV set, batch 1, 32 layers: qkv+o+gate/up Q4_K, "
                                "down Q6_K, Q8_K activations (BASELINE configs[1])",
                    "layers": ds.layers, "mode": args.mode,
+                   "q6k_layout": "regrouped in runs of eight blocks when loaded (same bytes)" if ds.q6_grouped else "file",
                    "launches_per_step": 1 if args.mode == "plan" else 4 * ds.layers,
                    "bytes_per_step": step_bytes},
         "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBPS, 2),

@@ -313,6 +313,26 @@ int oxh_q3_k_as_q6_k(const void *d_w, size_t rows, size_t cols, void *d_q6k, voi
 #define OXH_Q2_K_WIDE 0x1008u
 int oxh_q2_k_widen(const void *d_w, size_t rows, size_t cols, void *d_wide, void *stream);
 
+/* Q6_K regrouped for decode: the same bytes, permuted inside every run of eight
+ * consecutive blocks (1680 bytes) so that the 16-byte pieces the lanes of a
+ * GEMV pass load lie next to each other and aligned:
+ *   [0..511] pieces ql[64n+16lh ..] of (block j, lane u = 2n+lh) at 16*(4j+u),
+ *   [512..1023] pieces ql[64n+32+16lh ..], [1024..1535] pieces qh[32n+16lh ..],
+ *   [1536..1663] the sixteen scales of block j at 16*j, [1664..1679] the f16 d
+ *   of block j at 2*j.
+ * The plain 210-byte blocks are only 2-byte aligned and every load instruction
+ * of a pass touches all 27 cache lines of the pass's span; regrouped, the same
+ * pass touches a third as many (decode kernels are paced by exactly that).
+ * Size and row order are unchanged; cols must be a multiple of 2048, otherwise
+ * OXH_DECLINED.  The result is a weight matrix only oxh_gemv_segments*,
+ * oxh_gemv, oxh_matvec* and plans accept, under OXH_Q6_K_G8; oxh_mmq,
+ * oxh_get_rows and the expert layer read the file layout.  The host layer keeps
+ * this form next to a registered Q6_K range by itself.  d_g8 != d_w, 16-byte
+ * aligned, rows * cols / 256 * 210 bytes.  No counterpart in the reference
+ * (its CPU kernels read the file layout, oxk.c:913-964). */
+#define OXH_Q6_K_G8 0x1009u
+int oxh_q6_k_group(const void *d_w, size_t rows, size_t cols, void *d_g8, void *stream);
+
 /* Embedding lookup: out[t*out_stride ..] = row d_ids[t] of a packed matrix,
  * expanded to f32 in the reference's dequantisation arithmetic (bit-identical
  * to oc_quant_dequant_row, oxidize-c/src/compute/quantization.c:2781-2795), so

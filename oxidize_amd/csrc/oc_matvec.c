@@ -418,6 +418,7 @@ static int bad_arg(const char *what);
 /* Forms a resident matrix can be rewritten into, once, on the device. */
 #define OXH_PREP_Q3K_AS_Q6K 1u      /* oxh_q3_k_as_q6_k */
 #define OXH_PREP_Q2K_WIDE   2u      /* oxh_q2_k_widen   */
+#define OXH_PREP_Q6K_G8     3u      /* oxh_q6_k_group   */
 
 /* The rewritten form of the rows x cols matrix at host pointer p inside registry entry r, made on first
  * use and kept with the entry (the reference prepares its batch rows once per matrix as well,
@@ -445,8 +446,9 @@ static int prepared_ptr(Resident *r, const uint8_t *p, size_t rows, size_t cols,
     void *nd = NULL;
     int rc = oxh_malloc(&nd, bytes);
     if (rc) return rc;
-    if (form == OXH_PREP_Q2K_WIDE) rc = oxh_q2_k_widen(r->d + off, rows, cols, nd, NULL);
-    else                           rc = oxh_q3_k_as_q6_k(r->d + off, rows, cols, nd, NULL);
+    if (form == OXH_PREP_Q2K_WIDE)    rc = oxh_q2_k_widen(r->d + off, rows, cols, nd, NULL);
+    else if (form == OXH_PREP_Q6K_G8) rc = oxh_q6_k_group(r->d + off, rows, cols, nd, NULL);
+    else                              rc = oxh_q3_k_as_q6_k(r->d + off, rows, cols, nd, NULL);
     if (rc) {
         (void)oxh_free(nd);
         return rc;
@@ -455,6 +457,33 @@ static int prepared_ptr(Resident *r, const uint8_t *p, size_t rows, size_t cols,
     q->off = off; q->rows = rows; q->cols = cols; q->form = form; q->d = (uint8_t *)nd; q->bytes = bytes;
     *d = q->d;
     return OXH_OK;
+}
+
+/* Q6_K for the decode kernels: the regrouped copy (oxh_q6_k_group), made the first time a GEMV runs over
+ * the matrix and kept with its registry entry next to the file layout, which the matrix-core kernel and
+ * the row lookup go on reading.  OXH_Q6K_GROUPED=0 switches it off; a matrix whose cols are not a
+ * multiple of 2048, or for which there is no memory left, stays on the file layout, and so do
+ * unregistered weights under OXH_WEIGHT_CACHE=off. */
+static int q6k_grouped_enabled(void)
+{
+    static int cached = -1;
+    if (cached < 0) {
+        const char *e = getenv("OXH_Q6K_GROUPED");
+        cached = (e && e[0] == '0') ? 0 : 1;
+    }
+    return cached;
+}
+
+static void decode_form(uint32_t *qtype, Resident *entry, const uint8_t *data, size_t rows, size_t cols,
+                        const uint8_t **d_w)
+{
+    if (*qtype != OXH_Q6_K || !entry || rows == 0 || cols % (8u * OXH_QK_K) || !q6k_grouped_enabled()) return;
+    /* a cache that uploads the bytes again on every call would regroup them on every call as well */
+    if (entry->automatic && cache_mode() == CACHE_OFF) return;
+    const uint8_t *d;
+    if (prepared_ptr(entry, data, rows, cols, OXH_PREP_Q6K_G8, &d) != OXH_OK) return;
+    *d_w = d;
+    *qtype = OXH_Q6_K_G8;
 }
 
 /* ─── device staging buffers (inputs, activations, outputs) ───────────── */
@@ -595,7 +624,10 @@ static int mv_one(uint32_t qtype, const uint8_t *data, size_t rows,
     int rc = oxh_init(0);
     if (rc) return rc;
     const uint8_t *d_w;
-    if ((rc = resident_ptr(data, wbytes, &d_w, NULL))) return rc;
+    Resident *entry = NULL;
+    if ((rc = resident_ptr(data, wbytes, &d_w, &entry))) return rc;
+    uint32_t run_type = qtype;
+    decode_form(&run_type, entry, data, rows, cols, &d_w);
     /* device and pinned-host images: [output rows][quantised activation] */
     const size_t act_off = align16(obytes);
     if ((rc = reserve(&g_dx, cols * sizeof(float)))) return rc;
@@ -607,7 +639,7 @@ static int mv_one(uint32_t qtype, const uint8_t *data, size_t rows,
     if ((rc = oxh_memcpy_h2d(g_dx.p, g_hin.p, cols * sizeof(float), NULL))) return rc;
     /* one launch: quantise the activation inside the GEMV kernel */
     OxhSegment seg = { d_w, (float *)g_dout.p, rows, 0, 0, NULL };
-    if ((rc = oxh_gemv_segments_f32(qtype, &seg, 1, cols, (const float *)g_dx.p, cols,
+    if ((rc = oxh_gemv_segments_f32(run_type, &seg, 1, cols, (const float *)g_dx.p, cols,
                                     (uint8_t *)g_dout.p + act_off, 1, rows, NULL)))
         return rc;
     if ((rc = oxh_memcpy_d2h(g_hout.p, g_dout.p, act_off + abytes, NULL))) return rc;
@@ -654,14 +686,25 @@ static int grouped(uint32_t qtype, const uint8_t *const *datas,
     size_t done_rows = 0;
     for (size_t k0 = 0; k0 < n_outs; k0 += CHUNK) {
         const size_t n = n_outs - k0 < CHUNK ? n_outs - k0 : CHUNK;
+        const uint8_t *d_plain[CHUNK], *d_alt[CHUNK];
+        bool all_alt = qtype == OXH_Q6_K;
         for (size_t i = 0; i < n; i++) {
             const size_t k = k0 + i;
             size_t wbytes;
             if (!mul_ok(rows[k], row_bytes[k], &wbytes)) return bad_arg("grouped: size overflow");
             const uint8_t *d_w = NULL;
+            Resident *entry = NULL;
             if (rows[k]) {
                 if (!datas[k] || !outs[k]) return bad_arg("grouped: NULL matrix pointer");
-                if ((rc = resident_ptr(datas[k], wbytes, &d_w, NULL))) return rc;
+                if ((rc = resident_ptr(datas[k], wbytes, &d_w, &entry))) return rc;
+            }
+            /* one launch has one weight type: the regrouped Q6_K copies are used when every matrix of
+             * the launch has one */
+            d_plain[i] = d_alt[i] = d_w;
+            if (all_alt && rows[k]) {
+                uint32_t t = qtype;
+                decode_form(&t, entry, datas[k], rows[k], cols, &d_alt[i]);
+                if (t != OXH_Q6_K_G8) all_alt = false;
             }
             segs[i].d_w = d_w;
             segs[i].d_out = (float *)g_dout.p + done_rows;
@@ -671,8 +714,9 @@ static int grouped(uint32_t qtype, const uint8_t *const *datas,
             segs[i].d_w_pair = NULL;
             done_rows += rows[k];
         }
-        if ((rc = oxh_gemv_segments_f32(qtype, segs, n, cols, (const float *)g_dx.p, cols, NULL, 1, 0,
-                                        NULL)))
+        for (size_t i = 0; i < n; i++) segs[i].d_w = all_alt ? d_alt[i] : d_plain[i];
+        if ((rc = oxh_gemv_segments_f32(all_alt ? OXH_Q6_K_G8 : qtype, segs, n, cols, (const float *)g_dx.p, cols,
+                                        NULL, 1, 0, NULL)))
             return rc;
     }
     if ((rc = oxh_memcpy_d2h(g_hout.p, g_dout.p, total_rows * sizeof(float), NULL))) return rc;

@@ -369,6 +369,38 @@ k_q3k_to_q6k(const uint8_t *__restrict__ src, uint8_t *__restrict__ dst, uint32_
     }
 }
 
+/* Q6_K blocks regrouped for the decode kernels (the layout q6k_load<.., true> reads): inside every run of
+ * eight consecutive blocks the 16-byte pieces a lane loads are stored piece-major.  One thread per
+ * 16-byte destination piece, 105 pieces per group; same bytes, same size. */
+__global__ __launch_bounds__(256) void
+k_q6k_group(const uint8_t *__restrict__ src, uint8_t *__restrict__ dst, uint32_t n_groups)
+{
+    const uint32_t t = blockIdx.x * 256u + threadIdx.x;
+    const uint32_t grp = t / 105u, piece = t - grp * 105u;
+    if (grp >= n_groups) return;
+    const uint8_t *sg = src + (size_t)grp * Q6K_GROUP_BYTES;
+    uint8_t *dg = dst + (size_t)grp * Q6K_GROUP_BYTES + 16u * piece;
+    uint16_t v[8];
+    if (piece < 104u) {
+        const uint32_t part = piece >> 5;               /* 0 la, 1 lb, 2 hh, 3 scales */
+        const uint32_t j = part < 3u ? (piece & 31u) >> 2 : piece & 7u;
+        const uint32_t u = piece & 3u, n = u >> 1, lh = u & 1u;
+        const uint32_t from = part == 0u ? 64u * n + 16u * lh
+                            : part == 1u ? 64u * n + 32u + 16u * lh
+                            : part == 2u ? 128u + 32u * n + 16u * lh : 192u;
+        const uint16_t *sp = reinterpret_cast<const uint16_t *>(sg + 210u * j + from);   /* 2-byte aligned */
+#pragma unroll
+        for (int i = 0; i < 8; i++) v[i] = sp[i];
+    } else {
+#pragma unroll
+        for (int i = 0; i < 8; i++) v[i] = *reinterpret_cast<const uint16_t *>(sg + 210u * (uint32_t)i + 208u);
+    }
+    uint32_t o[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) o[i] = (uint32_t)v[2 * i] | ((uint32_t)v[2 * i + 1] << 16);
+    *reinterpret_cast<u32x4 *>(dg) = u32x4{ o[0], o[1], o[2], o[3] };
+}
+
 /* Q2_K rows widened to 210-byte blocks for the tile kernel's Q2 mode.  A Q2_K weight is
  * d * sc * code - dmin * m with 4-bit sc and m per group of 16 and a 2-bit code (oxk.c:592-622), over
  * the groups and the element order of Q6_K.  sc * code is at most 45 and goes into the 6-bit field
@@ -546,6 +578,7 @@ extern "C" int oxh_act_kind(uint32_t qtype, size_t cols)
     case OXH_Q6_K:
     case OXH_IQ3_S:                     /* the two codebook formats the reference's integer path takes */
     case OXH_IQ1_XXXS: return (cols % OXH_QK_K == 0) ? 2 : 0;
+    case OXH_Q6_K_G8:  return (cols % (8u * OXH_QK_K) == 0) ? 2 : 0;     /* whole groups of eight blocks per row */
     default:         return 0;
     }
 }
@@ -563,7 +596,8 @@ static size_t block_bytes(uint32_t qtype)
     case OXH_Q4_K_M: return OXH_Q4_K_BYTES;
     case OXH_Q5_K_S:
     case OXH_Q5_K_M: return OXH_Q5_K_BYTES;
-    case OXH_Q6_K:   return OXH_Q6_K_BYTES;
+    case OXH_Q6_K:
+    case OXH_Q6_K_G8: return OXH_Q6_K_BYTES;
     case OXH_Q2_K:   return OXH_Q2_K_BYTES;
     case OXH_Q3_K_M: return OXH_Q3_K_BYTES;
     case OXH_IQ3_S:  return OXH_IQ3_S_BYTES;
@@ -665,6 +699,7 @@ static hipError_t raise_all_lds_ceilings(void)
     OXH_RAISE(k_gemv_q4_k)
     OXH_RAISE(k_gemv_q5_k)
     OXH_RAISE(k_gemv_q6_k)
+    OXH_RAISE(k_gemv_q6_kg)
     OXH_RAISE(k_gemv_q2_k)
     OXH_RAISE(k_gemv_q3_k)
     OXH_RAISE(k_gemv_q8_0)
@@ -689,6 +724,7 @@ static hipError_t raise_all_lds_ceilings(void)
     OXH_RAISE_PRO(k_gemv_q4_k_pro)
     OXH_RAISE_PRO(k_gemv_q5_k_pro)
     OXH_RAISE_PRO(k_gemv_q6_k_pro)
+    OXH_RAISE_PRO(k_gemv_q6_kg_pro)
     OXH_RAISE_PRO(k_gemv_q2_k_pro)
     OXH_RAISE_PRO(k_gemv_q3_k_pro)
     OXH_RAISE_PRO(k_gemv_q8_0_pro)
@@ -734,7 +770,8 @@ static uint32_t act_lds_bytes(uint32_t qtype, uint32_t blocks)
 {
     if (oxh_act_kind(qtype, 32) == 1) return q80_lds_bytes(blocks);
     qtype = canon_qtype(qtype);
-    if (qtype == OXH_Q6_K || qtype == OXH_Q2_K || qtype == OXH_Q3_K_M) return q8k6_lds_bytes(blocks);
+    if (qtype == OXH_Q6_K || qtype == OXH_Q6_K_G8 || qtype == OXH_Q2_K || qtype == OXH_Q3_K_M)
+        return q8k6_lds_bytes(blocks);
     return q8k_lds_bytes(blocks);
 }
 
@@ -1140,6 +1177,7 @@ static int launch_gemv(uint32_t qtype, const OxhSegment *segs, size_t n_segs, si
     if (is_q4k(qtype))          OXH_LAUNCH_ANY(k_gemv_q4_k, k_gemv_q4_k_pro);
     else if (is_q5k(qtype))     OXH_LAUNCH_ANY(k_gemv_q5_k, k_gemv_q5_k_pro);
     else if (qtype == OXH_Q6_K) OXH_LAUNCH_ANY(k_gemv_q6_k, k_gemv_q6_k_pro);
+    else if (qtype == OXH_Q6_K_G8) OXH_LAUNCH_ANY(k_gemv_q6_kg, k_gemv_q6_kg_pro);
     else if (qtype == OXH_Q2_K) OXH_LAUNCH_ANY(k_gemv_q2_k, k_gemv_q2_k_pro);
     else if (qtype == OXH_Q3_K_M) OXH_LAUNCH_ANY(k_gemv_q3_k, k_gemv_q3_k_pro);
     else if (qtype == OXH_Q4_0) OXH_LAUNCH_ANY(k_gemv_q4_0, k_gemv_q4_0_pro);
@@ -1380,7 +1418,7 @@ extern "C" int oxh_get_rows(uint32_t qtype, const void *d_w, size_t rows, size_t
     if (n_ids == 0) return OXH_OK;
     if (!d_w || !d_ids || !d_out) return arg_fail("oxh_get_rows: NULL pointer");
     /* every type with a matvec kernel but the codebook formats */
-    const size_t rb = (oxh_act_kind(qtype, cols) && !is_iq(qtype)) ? oxh_row_bytes(qtype, cols) : 0;
+    const size_t rb = (oxh_act_kind(qtype, cols) && !is_iq(qtype) && qtype != OXH_Q6_K_G8) ? oxh_row_bytes(qtype, cols) : 0;
     if (rb == 0) {
         snprintf(g_err, sizeof g_err, "oxh_get_rows: qtype %u with cols %zu has no kernel here", qtype, cols);
         return OXH_DECLINED;
@@ -1440,6 +1478,28 @@ extern "C" int oxh_q2_k_widen(const void *d_w, size_t rows, size_t cols, void *d
     const uint32_t n_blocks = (uint32_t)(rows * blocks);
     hipLaunchKernelGGL(k_q2k_widen, dim3((n_blocks * 4u + 255u) / 256u), dim3(256), 0, pick_stream(stream),
                        (const uint8_t *)d_w, (uint8_t *)d_wide, n_blocks);
+    HIP_TRY(hipGetLastError());
+    return OXH_OK;
+}
+
+extern "C" int oxh_q6_k_group(const void *d_w, size_t rows, size_t cols, void *d_g8, void *stream)
+{
+    int rc = ensure_init();
+    if (rc) return rc;
+    if (rows == 0) return OXH_OK;
+    if (!d_w || !d_g8) return arg_fail("oxh_q6_k_group: NULL pointer");
+    if (d_w == d_g8) return arg_fail("oxh_q6_k_group: source and destination must differ");
+    if (cols == 0 || cols % (8u * OXH_QK_K)) {
+        snprintf(g_err, sizeof g_err, "oxh_q6_k_group: cols %zu is not a multiple of 2048 (eight blocks)", cols);
+        return OXH_DECLINED;
+    }
+    if (((uintptr_t)d_w & 1u) || ((uintptr_t)d_g8 & 15u))
+        return arg_fail("oxh_q6_k_group: the source must be 2-byte and the destination 16-byte aligned");
+    const size_t groups = rows * (cols / (8u * OXH_QK_K));
+    if (groups > 0xFFFFFFFFull / 105u) return arg_fail("oxh_q6_k_group: matrix too large");
+    const uint32_t threads = (uint32_t)groups * 105u;
+    hipLaunchKernelGGL(k_q6k_group, dim3((threads + 255u) / 256u), dim3(256), 0, pick_stream(stream),
+                       (const uint8_t *)d_w, (uint8_t *)d_g8, (uint32_t)groups);
     HIP_TRY(hipGetLastError());
     return OXH_OK;
 }

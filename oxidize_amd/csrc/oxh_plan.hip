@@ -64,6 +64,7 @@
 #define PLAN_Q4_K 0u
 #define PLAN_Q5_K 1u
 #define PLAN_Q6_K 2u
+#define PLAN_Q6_KG 3u               /* Q6_K regrouped in runs of eight blocks (OXH_Q6_K_G8) */
 
 /* Device addresses travel through the table as integers and become global-memory pointers in the
  * kernel: a pointer merely loaded from memory is a generic one to the compiler, and loads through it
@@ -222,7 +223,7 @@ struct PWork {
 
 __device__ __forceinline__ uint32_t plan_block_bytes(uint32_t kind)
 {
-    return kind == PLAN_Q6_K ? 210u : kind == PLAN_Q5_K ? 176u : 144u;
+    return kind >= PLAN_Q6_K ? 210u : kind == PLAN_Q5_K ? 176u : 144u;
 }
 
 __device__ __forceinline__ PWork plan_work(const PlanOp *op, uint32_t wave)
@@ -317,6 +318,10 @@ __device__ __forceinline__ void wset_load(uint32_t kind, WSet &s, const WSrc &sr
         Q6kRegs t;
         q6k_load<true>(t, src, g, sub >> 1, sub & 1u);
         v0 = as_v4(t.la); v1 = as_v4(t.lb); v2 = as_v4(t.hh); v3 = as_v4(t.tail);
+    } else if (kind == PLAN_Q6_KG) {
+        Q6kRegs t;
+        q6k_load<true, true>(t, src, g, sub >> 1, sub & 1u);
+        v0 = as_v4(t.la); v1 = as_v4(t.lb); v2 = as_v4(t.hh); v3 = as_v4(t.tail);
     } else if (HAS_Q5 && kind == PLAN_Q5_K) {
         Q4kRegs t;
         q4k_load<true, true>(t, src, g, sub);
@@ -373,6 +378,7 @@ plan_passes_q45(const WSet &A0, const WSet &B0, const PWork &k, const GemvParams
     if (rem == 3u) q4k_pass<1, false, Q5>(A, ln, p, act, act_lds, 1u, B, (i + 2u) * 16u + lb, nblk, k.row0, terms);
 }
 
+template <bool G8>
 __device__ __forceinline__ void
 plan_passes_q6(const WSet &A0, const WSet &B0, const PWork &k, const GemvParams &p, const uint8_t *act,
                uint32_t act_lds, float *terms, uint32_t lane)
@@ -385,17 +391,17 @@ plan_passes_q6(const WSet &A0, const WSet &B0, const PWork &k, const GemvParams 
     const uint32_t lb = lane >> 2;
     uint32_t i = 0;
     while (i + 3u < npass) {
-        q6k_pass<1, false>(A, u, p, act, act_lds, 1u, B, i * 16u + lb, nblk, k.row0, terms);
-        q6k_load<true>(A, k.src, min((i + 2u) * 16u + lb, last), n, lh);
-        q6k_pass<1, false>(Bq, u, p, act, act_lds, 1u, B, (i + 1u) * 16u + lb, nblk, k.row0, terms);
-        q6k_load<true>(Bq, k.src, min((i + 3u) * 16u + lb, last), n, lh);
+        q6k_pass<1, false, G8>(A, u, p, act, act_lds, 1u, B, i * 16u + lb, nblk, k.row0, terms);
+        q6k_load<true, G8>(A, k.src, min((i + 2u) * 16u + lb, last), n, lh);
+        q6k_pass<1, false, G8>(Bq, u, p, act, act_lds, 1u, B, (i + 1u) * 16u + lb, nblk, k.row0, terms);
+        q6k_load<true, G8>(Bq, k.src, min((i + 3u) * 16u + lb, last), n, lh);
         i += 2u;
     }
     const uint32_t rem = npass - i;
-    q6k_pass<1, false>(A, u, p, act, act_lds, 1u, B, i * 16u + lb, nblk, k.row0, terms);
-    if (rem == 3u) q6k_load<true>(A, k.src, min((i + 2u) * 16u + lb, last), n, lh);
-    if (rem >= 2u) q6k_pass<1, false>(Bq, u, p, act, act_lds, 1u, B, (i + 1u) * 16u + lb, nblk, k.row0, terms);
-    if (rem == 3u) q6k_pass<1, false>(A, u, p, act, act_lds, 1u, B, (i + 2u) * 16u + lb, nblk, k.row0, terms);
+    q6k_pass<1, false, G8>(A, u, p, act, act_lds, 1u, B, i * 16u + lb, nblk, k.row0, terms);
+    if (rem == 3u) q6k_load<true, G8>(A, k.src, min((i + 2u) * 16u + lb, last), n, lh);
+    if (rem >= 2u) q6k_pass<1, false, G8>(Bq, u, p, act, act_lds, 1u, B, (i + 1u) * 16u + lb, nblk, k.row0, terms);
+    if (rem == 3u) q6k_pass<1, false, G8>(A, u, p, act, act_lds, 1u, B, (i + 2u) * 16u + lb, nblk, k.row0, terms);
 }
 
 /* per-row sums in block order into the workgroup's output staging; a paired operation writes
@@ -644,7 +650,7 @@ k_plan(const PlanOp *__restrict__ ops, uint32_t n_ops, const PlanSync sy, const 
             asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
             plan_stamp(sy, i, 5, ln, wave);
         }
-        if (op.kind == PLAN_Q6_K) plan_stage_finish<1>(op, xs, act, red, storer, ln, wave);
+        if (op.kind >= PLAN_Q6_K) plan_stage_finish<1>(op, xs, act, red, storer, ln, wave);
         else                      plan_stage_finish<0>(op, xs, act, red, storer, ln, wave);
         plan_prefetch<HAS_Q5>(cur, B, 1u, ln);
         plan_stamp(sy, i, 2, ln, wave);
@@ -658,7 +664,8 @@ k_plan(const PlanOp *__restrict__ ops, uint32_t n_ops, const PlanSync sy, const 
         gp.rows_cap = op.rows_cap;
         gp.dump = nullptr;
         if (cur.nblk != 0u) {
-            if (cur.kind == PLAN_Q6_K)      plan_passes_q6(A, B, cur, gp, act, q8k6_lds_bytes(Bk), terms, ln);
+            if (cur.kind == PLAN_Q6_K)      plan_passes_q6<false>(A, B, cur, gp, act, q8k6_lds_bytes(Bk), terms, ln);
+            else if (cur.kind == PLAN_Q6_KG) plan_passes_q6<true>(A, B, cur, gp, act, q8k6_lds_bytes(Bk), terms, ln);
             else if (HAS_Q5 && cur.kind == PLAN_Q5_K) plan_passes_q45<true>(A, B, cur, gp, act, q8k_lds_bytes(Bk), terms, ln);
             else                            plan_passes_q45<false>(A, B, cur, gp, act, q8k_lds_bytes(Bk), terms, ln);
         }
@@ -683,7 +690,7 @@ __device__ __forceinline__ void plan_dma16(const uint8_t *base, uint32_t off, ui
 
 __device__ __forceinline__ uint32_t plan_image_bytes(uint32_t kind, uint32_t blocks)
 {
-    return kind == PLAN_Q6_K ? q8k6_lds_bytes(blocks) : q8k_lds_bytes(blocks);
+    return kind >= PLAN_Q6_K ? q8k6_lds_bytes(blocks) : q8k_lds_bytes(blocks);
 }
 
 /* the staged input of an operation into LDS at byte address lds_addr, 1 KB pieces dealt to the waves */
@@ -724,7 +731,7 @@ k_plan_ext(const PlanOp *__restrict__ ops, uint32_t n_ops, const PlanSync sy, co
 #pragma unroll
         for (int u = 0; u < 4; u++) xs.x[u] = xs.t[u] = xs.b[u] = XRegs{ 0.f, 0.f, 0.f, 0.f };
         plan_stage_issue(op, xs, false, lane, wave);
-        if (op.kind == PLAN_Q6_K) plan_stage_finish<1>(op, xs, lds, red, true, lane, wave);
+        if (op.kind >= PLAN_Q6_K) plan_stage_finish<1>(op, xs, lds, red, true, lane, wave);
         else                      plan_stage_finish<0>(op, xs, lds, red, true, lane, wave);
         __syncthreads();
         const uint32_t bytes = plan_image_bytes(op.kind, op.blocks);
@@ -800,7 +807,8 @@ k_plan_ext(const PlanOp *__restrict__ ops, uint32_t n_ops, const PlanSync sy, co
         gp.dump = nullptr;
         float *const terms = terms_wg + (size_t)(i & 1u) * ld.terms_wg + __umul24(cur.row0, gp.term_stride);
         if (cur.nblk != 0u) {
-            if (cur.kind == PLAN_Q6_K)      plan_passes_q6(A, B, cur, gp, act, q8k6_lds_bytes(Bk), terms, ln);
+            if (cur.kind == PLAN_Q6_K)      plan_passes_q6<false>(A, B, cur, gp, act, q8k6_lds_bytes(Bk), terms, ln);
+            else if (cur.kind == PLAN_Q6_KG) plan_passes_q6<true>(A, B, cur, gp, act, q8k6_lds_bytes(Bk), terms, ln);
             else if (HAS_Q5 && cur.kind == PLAN_Q5_K) plan_passes_q45<true>(A, B, cur, gp, act, q8k_lds_bytes(Bk), terms, ln);
             else                            plan_passes_q45<false>(A, B, cur, gp, act, q8k_lds_bytes(Bk), terms, ln);
         }
@@ -851,6 +859,7 @@ static bool plan_kind(uint32_t qtype, uint32_t *kind)
     case OXH_Q4_K_S: case OXH_Q4_K_M: *kind = PLAN_Q4_K; return true;
     case OXH_Q5_K_S: case OXH_Q5_K_M: *kind = PLAN_Q5_K; return true;
     case OXH_Q6_K:                    *kind = PLAN_Q6_K; return true;
+    case OXH_Q6_K_G8:                 *kind = PLAN_Q6_KG; return true;
     default: return false;
     }
 }
@@ -922,9 +931,10 @@ extern "C" int oxh_plan_create(const OxhPlanOp *ops, size_t n_ops, OxhPlan **out
         const OxhPlanOp &o = ops[i];
         PlanOp &d = h[i];
         uint32_t kind;
-        if (!plan_kind(o.qtype, &kind) || o.cols == 0 || o.cols % OXH_QK_K || o.cols / OXH_QK_K > PLAN_MAX_BLOCKS) {
+        if (!plan_kind(o.qtype, &kind) || o.cols == 0 || o.cols % OXH_QK_K || o.cols / OXH_QK_K > PLAN_MAX_BLOCKS ||
+            (kind == PLAN_Q6_KG && o.cols % (8u * OXH_QK_K))) {
             rc = oxh_internal_errorf(OXH_DECLINED, "plan: operation %zu (qtype %u, cols %zu) is not one a plan runs: "
-                                     "Q4_K, Q5_K or Q6_K with cols a multiple of 256 up to %u", i, o.qtype, o.cols,
+                                     "Q4_K, Q5_K or Q6_K with cols a multiple of 256 (2048 for the regrouped Q6_K) up to %u", i, o.qtype, o.cols,
                                      PLAN_MAX_BLOCKS * 256u);
             break;
         }
@@ -993,7 +1003,7 @@ extern "C" int oxh_plan_create(const OxhPlanOp *ops, size_t n_ops, OxhPlan **out
             wg += n_wg[k];
         }
         d.n_wg = wg;
-        const uint32_t act = kind == PLAN_Q6_K ? q8k6_lds_bytes(d.blocks) : q8k_lds_bytes(d.blocks);
+        const uint32_t act = kind >= PLAN_Q6_K ? q8k6_lds_bytes(d.blocks) : q8k_lds_bytes(d.blocks);
         if (act > max_act) max_act = act;
         d.xq = (gaddr)img_bytes;                    /* offset for now; the base is added once it exists */
         img_bytes += (act + 255u) & ~(size_t)255u;

@@ -245,6 +245,14 @@ def q2_k_widen(d_w, rows, cols, d_wide, stream=None):
     check(lib().oxh_q2_k_widen(ctypes.c_void_p(d_w), rows, cols, ctypes.c_void_p(d_wide), stream))
 
 
+Q6_K_G8 = 0x1009
+
+
+def q6_k_group(d_w, rows, cols, d_g8, stream=None):
+    """Q6_K regrouped in runs of eight blocks for the decode kernels (same size; cols % 2048 == 0)."""
+    check(lib().oxh_q6_k_group(ctypes.c_void_p(d_w), rows, cols, ctypes.c_void_p(d_g8), stream))
+
+
 def read_probe(d_buf, nbytes, stream=None):
     """One launch that only reads `nbytes` at d_buf (measurement aid)."""
     check(lib().oxh_debug_read_probe(ctypes.c_void_p(d_buf), nbytes, None, stream))

@@ -19,9 +19,19 @@ LLAMA3_8B = dict(hidden=4096, kv=1024, ffn=14336, layers=32)
 
 
 class DecodeSet:
-    def __init__(self, hidden=4096, kv=1024, ffn=14336, layers=32, seed=0, keep_host=()):
+    def __init__(self, hidden=4096, kv=1024, ffn=14336, layers=32, seed=0, keep_host=(), q6_grouped=None):
+        """q6_grouped: keep the Q6_K matrices resident in the regrouped layout the decode kernels read
+        fastest (oxh_q6_k_group; same bytes, made once when the weights are loaded, as the host layer
+        does for registered weights).  Default: wherever the shape allows it (ffn % 2048 == 0)."""
         self.hidden, self.kv, self.ffn, self.layers = hidden, kv, ffn, layers
         self.seed = seed
+        if q6_grouped is None:
+            q6_grouped = ffn % 2048 == 0
+        elif q6_grouped and ffn % 2048:
+            raise ValueError("the regrouped Q6_K layout needs ffn to be a multiple of 2048")
+        self.q6_grouped = q6_grouped
+        self.qtype_run = {Q4K: Q4K, Q6K: mv.Q6_K_G8 if q6_grouped else Q6K}
+        staging = None
         # (name, qtype, [rows...], cols, input index)
         self.ops = [
             ("qkv", Q4K, [hidden, kv, kv], hidden, 0),
@@ -40,7 +50,16 @@ class DecodeSet:
                 for seg, r in enumerate(rows):
                     w = synth.weights(qt, r, cols, seed=seed, stream=stream_id)
                     stream_id += 1
-                    bufs.append(mv.DeviceBuffer.from_host(w))
+                    if qt == Q6K and q6_grouped:
+                        if staging is None or staging.nbytes < w.nbytes:
+                            staging = mv.DeviceBuffer(w.nbytes)
+                        staging.upload(w)
+                        buf = mv.DeviceBuffer(w.nbytes)
+                        mv.q6_k_group(staging.ptr, r, cols, buf.ptr)
+                        mv.sync()
+                        bufs.append(buf)
+                    else:
+                        bufs.append(mv.DeviceBuffer.from_host(w))
                     self.weight_bytes += w.nbytes
                     if layer in keep_host:
                         self.host[(layer, op, seg)] = w
@@ -89,12 +108,13 @@ class DecodeSet:
         the activation inside the GEMV kernel (fused=True, what the host API
         does), or the stand-alone quantiser followed by the GEMV."""
         name, qt, rows, cols, _ = self.ops[op]
+        run = self.qtype_run[qt]
         if fused:
-            mv.gemv_segments_f32(qt, self.segments[layer][op], cols, self.x[layer][op].ptr, cols,
+            mv.gemv_segments_f32(run, self.segments[layer][op], cols, self.x[layer][op].ptr, cols,
                                  self.act[layer][op].ptr, 1, 0, stream)
         else:
             mv.quantize(qt, self.x[layer][op].ptr, cols, 1, cols, self.act[layer][op].ptr, stream)
-            mv.gemv_segments(qt, self.segments[layer][op], cols, self.act[layer][op].ptr, 1, 0, stream)
+            mv.gemv_segments(run, self.segments[layer][op], cols, self.act[layer][op].ptr, 1, 0, stream)
 
     def launch_step(self, stream=None, fused=True):
         for layer in range(self.layers):
@@ -107,8 +127,8 @@ class DecodeSet:
         ops = []
         for layer in range(self.layers):
             for op, (name, qt, rows, cols, _) in enumerate(self.ops):
-                ops.append(dict(qtype=qt, segs=self.segments[layer][op], cols=cols, d_x=self.x[layer][op].ptr,
-                                d_act_out=self.act[layer][op].ptr))
+                ops.append(dict(qtype=self.qtype_run[qt], segs=self.segments[layer][op], cols=cols,
+                                d_x=self.x[layer][op].ptr, d_act_out=self.act[layer][op].ptr))
         return ops
 
     def output(self, layer, op):
@@ -202,7 +222,7 @@ class DecodeChain:
             ops.append(dict(qtype=Q4K, segs=sg["o"], cols=h, d_x=self.qkv.ptr))
             ops.append(dict(qtype=Q4K, segs=sg["gate_up"], cols=h, d_x=x1.ptr, kind=mv.PRO_RMSNORM,
                             d_b=self.g_ffn[l].ptr, eps=self.eps, d_add=self.o.ptr, d_sum_out=x2.ptr))
-            ops.append(dict(qtype=Q6K, segs=sg["down"], cols=d.ffn, d_x=self.h.ptr))
+            ops.append(dict(qtype=d.qtype_run[Q6K], segs=sg["down"], cols=d.ffn, d_x=self.h.ptr))
             x, f = x2, self.f
         self.last_x = x
         return ops
@@ -225,7 +245,7 @@ class DecodeChain:
             mv.gemv_segments_fused(Q4K, sg["gate_up"], h, x1.ptr, h, mv.PRO_RMSNORM, self.g_ffn[l].ptr, self.eps,
                                    cap["n2"].ptr if cap else None, None, 1, 0, stream, d_add=self.o.ptr,
                                    d_sum_out=x2.ptr)
-            mv.gemv_segments_f32(Q6K, sg["down"], d.ffn, self.h.ptr, d.ffn, None, 1, 0, stream)
+            mv.gemv_segments_f32(d.qtype_run[Q6K], sg["down"], d.ffn, self.h.ptr, d.ffn, None, 1, 0, stream)
             if cap:
                 for name, src in (("x1", x1), ("qkv", self.qkv), ("o", self.o), ("x2", x2), ("h", self.h),
                                   ("f", self.f)):
