@@ -293,6 +293,24 @@ int oxh_mmq(uint32_t qtype, const void *d_w, size_t rows, size_t cols,
             const void *d_acts, size_t n_vec, float *d_out, size_t out_stride,
             void *stream);
 
+/* oxh_mmq with options.  OXH_MMQ_RELAXED: the per-block float step of the
+ * Q4_K and Q5_K prefill tiles (256 or 128 rows x 128 tokens and 128 x 64,
+ * which a launch gets when it fills the device with them) is evaluated as dq * (dw * pos - dmin * min) with fused multiply-adds, five
+ * operations per output and block instead of the eight the reference's order
+ * takes ((dw*dq)*pos - (dmin*dq)*min, oxk.c:316-366).  The integers are the
+ * same and every block term is within an ulp or two of the exact one, so an
+ * output differs from the exact one by at most 1e-5 * |exact| + 2e-6 * r, r
+ * the root mean square of the launch's outputs (measured: 1.3e-6 * r at
+ * worst over 14336 x 4096 x 512; for outputs of unit scale that is well
+ * inside the 1e-4 + 1e-5 * |ref| the reference's own tests allow between its
+ * kernels), but it is no longer bit-identical to the CPU path.  Off unless asked for: flags = 0
+ * is oxh_mmq.  Other types and launches on the smaller tiles ignore the flag.  The host
+ * layer passes it when OXH_MMQ_RELAXED=1 is in the environment. */
+#define OXH_MMQ_RELAXED 1u
+int oxh_mmq_ex(uint32_t qtype, const void *d_w, size_t rows, size_t cols,
+               const void *d_acts, size_t n_vec, float *d_out, size_t out_stride,
+               uint32_t flags, void *stream);
+
 /* A Q3_K matrix rewritten as a Q6_K matrix that gives bit-identical results:
  * Q3_K's d * (sc - 32) * (code - 4) is Q6_K's d * sc6 * (code6 - 32) with
  * code6 = code + 28 and sc6 = sc - 32, over the same groups in the same

@@ -741,6 +741,10 @@ static hipError_t raise_all_lds_ceilings(void)
     if ((e = raise_lds_ceiling(k_mmq_q4_k<4, 1, 8>)) != hipSuccess) return e;
     if ((e = raise_lds_ceiling(k_mmq_q5_k<8, 1, 8>)) != hipSuccess) return e;
     if ((e = raise_lds_ceiling(k_mmq_q5_k<4, 1, 8>)) != hipSuccess) return e;
+    if ((e = raise_lds_ceiling(k_mmq_q4_k<8, 2, 8, true>)) != hipSuccess) return e;
+    if ((e = raise_lds_ceiling(k_mmq_q4_k<4, 1, 8, true>)) != hipSuccess) return e;
+    if ((e = raise_lds_ceiling(k_mmq_q5_k<8, 1, 8, true>)) != hipSuccess) return e;
+    if ((e = raise_lds_ceiling(k_mmq_q5_k<4, 1, 8, true>)) != hipSuccess) return e;
     if ((e = raise_lds_ceiling(k_mmq_q6_k<8, 1, 8>)) != hipSuccess) return e;
     if ((e = raise_lds_ceiling(k_mmq_q6_k<4, 1, 8>)) != hipSuccess) return e;
     if ((e = raise_lds_ceiling(k_mmq_q6_k<8, 1, 4>)) != hipSuccess) return e;
@@ -1288,25 +1292,25 @@ extern "C" int oxh_debug_subblock_sums(uint32_t qtype, const void *d_w, size_t r
     return OXH_OK;
 }
 
-template <int TC, int RC, int WAVES>
+template <int TC, int RC, int WAVES, bool RELAXED = false>
 static void mmq_launch(const void *d_w, size_t rows, size_t blocks, const void *d_acts, size_t n_vec,
                        float *d_out, size_t out_stride, void *stream)
 {
     typedef MmqGeom<TC, RC, WAVES> G;
     const dim3 grid((uint32_t)((rows + G::ROWS - 1) / G::ROWS), (uint32_t)((n_vec + G::TOK - 1) / G::TOK));
-    auto kernel = k_mmq_q4_k<TC, RC, WAVES>;
+    auto kernel = k_mmq_q4_k<TC, RC, WAVES, RELAXED>;
     hipLaunchKernelGGL(kernel, grid, dim3(WAVES * 64), G::LDS_BYTES, pick_stream(stream),
                        (const uint8_t *)d_w, (uint32_t)rows, (uint32_t)blocks,
                        (const uint8_t *)d_acts, (uint32_t)n_vec, d_out, out_stride);
 }
 
-template <int TC, int RC, int WAVES>
+template <int TC, int RC, int WAVES, bool RELAXED = false>
 static void mmq5_launch(const void *d_w, size_t rows, size_t blocks, const void *d_acts, size_t n_vec,
                         float *d_out, size_t out_stride, void *stream)
 {
     typedef MmqGeom<TC, RC, WAVES, true> G;
     const dim3 grid((uint32_t)((rows + G::ROWS - 1) / G::ROWS), (uint32_t)((n_vec + G::TOK - 1) / G::TOK));
-    auto kernel = k_mmq_q5_k<TC, RC, WAVES>;
+    auto kernel = k_mmq_q5_k<TC, RC, WAVES, RELAXED>;
     hipLaunchKernelGGL(kernel, grid, dim3(WAVES * 64), G::LDS_BYTES, pick_stream(stream),
                        (const uint8_t *)d_w, (uint32_t)rows, (uint32_t)blocks,
                        (const uint8_t *)d_acts, (uint32_t)n_vec, d_out, out_stride);
@@ -1324,9 +1328,26 @@ static void mmq6_launch(const void *d_w, size_t rows, size_t blocks, const void 
                        (const uint8_t *)d_acts, (uint32_t)n_vec, d_out, out_stride);
 }
 
+static int mmq_run(uint32_t qtype, const void *d_w, size_t rows, size_t cols, const void *d_acts, size_t n_vec,
+                   float *d_out, size_t out_stride, bool relaxed, void *stream);
+
 extern "C" int oxh_mmq(uint32_t qtype, const void *d_w, size_t rows, size_t cols,
                        const void *d_acts, size_t n_vec, float *d_out, size_t out_stride,
                        void *stream)
+{
+    return mmq_run(qtype, d_w, rows, cols, d_acts, n_vec, d_out, out_stride, false, stream);
+}
+
+extern "C" int oxh_mmq_ex(uint32_t qtype, const void *d_w, size_t rows, size_t cols,
+                          const void *d_acts, size_t n_vec, float *d_out, size_t out_stride,
+                          uint32_t flags, void *stream)
+{
+    if (flags & ~OXH_MMQ_RELAXED) return arg_fail("oxh_mmq_ex: unknown flag");
+    return mmq_run(qtype, d_w, rows, cols, d_acts, n_vec, d_out, out_stride, (flags & OXH_MMQ_RELAXED) != 0, stream);
+}
+
+static int mmq_run(uint32_t qtype, const void *d_w, size_t rows, size_t cols, const void *d_acts, size_t n_vec,
+                   float *d_out, size_t out_stride, bool relaxed, void *stream)
 {
     int rc = ensure_init();
     if (rc) return rc;
@@ -1375,7 +1396,9 @@ extern "C" int oxh_mmq(uint32_t qtype, const void *d_w, size_t rows, size_t cols
         }
         if (is_q5k(qtype)) {
             if (shape == 5) shape = 2;
-            if (shape == 1)      mmq5_launch<8, 1, 8>(d_w, rows, blocks, d_acts, n_vec, d_out, out_stride, stream);
+            if (shape == 1 && relaxed)      mmq5_launch<8, 1, 8, true>(d_w, rows, blocks, d_acts, n_vec, d_out, out_stride, stream);
+            else if (shape == 2 && relaxed) mmq5_launch<4, 1, 8, true>(d_w, rows, blocks, d_acts, n_vec, d_out, out_stride, stream);
+            else if (shape == 1) mmq5_launch<8, 1, 8>(d_w, rows, blocks, d_acts, n_vec, d_out, out_stride, stream);
             else if (shape == 2) mmq5_launch<4, 1, 8>(d_w, rows, blocks, d_acts, n_vec, d_out, out_stride, stream);
             else if (shape == 3) mmq5_launch<2, 1, 4>(d_w, rows, blocks, d_acts, n_vec, d_out, out_stride, stream);
             else                 mmq5_launch<1, 1, 4>(d_w, rows, blocks, d_acts, n_vec, d_out, out_stride, stream);
@@ -1400,7 +1423,11 @@ extern "C" int oxh_mmq(uint32_t qtype, const void *d_w, size_t rows, size_t cols
         return OXH_OK;
     }
     if (shape == 5) shape = 2;
-    if (shape == 1)      mmq_launch<8, 2, 8>(d_w, rows, blocks, d_acts, n_vec, d_out, out_stride, stream);
+    /* the relaxed f32 step exists for the two prefill tiles; smaller launches are bound by the weight
+     * stream and keep the exact one */
+    if (shape == 1 && relaxed)      mmq_launch<8, 2, 8, true>(d_w, rows, blocks, d_acts, n_vec, d_out, out_stride, stream);
+    else if (shape == 2 && relaxed) mmq_launch<4, 1, 8, true>(d_w, rows, blocks, d_acts, n_vec, d_out, out_stride, stream);
+    else if (shape == 1) mmq_launch<8, 2, 8>(d_w, rows, blocks, d_acts, n_vec, d_out, out_stride, stream);
     else if (shape == 2) mmq_launch<4, 1, 8>(d_w, rows, blocks, d_acts, n_vec, d_out, out_stride, stream);
     else if (shape == 3) mmq_launch<2, 1, 4>(d_w, rows, blocks, d_acts, n_vec, d_out, out_stride, stream);
     else                 mmq_launch<1, 1, 4>(d_w, rows, blocks, d_acts, n_vec, d_out, out_stride, stream);

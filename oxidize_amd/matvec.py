@@ -174,7 +174,14 @@ def gemv_segments_fused(qtype, segs, cols, d_x, x_stride, kind, d_b, eps=0.0, d_
                                         n_vec, out_stride, stream))
 
 
-def mmq(qtype, d_w, rows, cols, d_acts, n_vec, d_out, out_stride, stream=None):
+MMQ_RELAXED = 1
+
+
+def mmq(qtype, d_w, rows, cols, d_acts, n_vec, d_out, out_stride, stream=None, flags=0):
+    if flags:
+        check(lib().oxh_mmq_ex(qtype, ctypes.c_void_p(d_w), rows, cols, ctypes.c_void_p(d_acts),
+                               n_vec, ctypes.c_void_p(d_out), out_stride, flags, stream))
+        return
     check(lib().oxh_mmq(qtype, ctypes.c_void_p(d_w), rows, cols, ctypes.c_void_p(d_acts),
                         n_vec, ctypes.c_void_p(d_out), out_stride, stream))
 

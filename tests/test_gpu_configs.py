@@ -13,6 +13,8 @@
 import os
 import zlib
 
+import ctypes
+
 import numpy as np
 import pytest
 
@@ -235,3 +237,49 @@ def test_config4_moe_expert_gemvs(oxh):
             assert np.array_equal(bits(up[pidx]), bits(oracle_matvec(Q4K, wu, 14336, 4096, x)[0]))
             h = np.ascontiguousarray(ms.h[pidx])
             assert np.array_equal(bits(down[pidx]), bits(oracle_matvec(Q4K, wd, 4096, 14336, h)[0]))
+
+
+@pytest.mark.parametrize("qtype,rows,cols,n_vec", [
+    (Q4K, 14336, 4096, 512), (Q4K, 4096, 4096, 512), (Q4K, 3000, 2048, 130),
+    (Q5K, 7165, 512, 507), (Q5K, 3600, 256, 500), (Q6K, 2048, 1024, 300), (Q4K, 4100, 512, 20),
+])
+def test_mmq_relaxed_mode_is_opt_in_and_within_tolerance(oxh, qtype, rows, cols, n_vec):
+    """OXH_MMQ_RELAXED evaluates the float step of the Q4_K / Q5_K prefill tiles with fused multiply-adds.
+    Bar, written here: |relaxed - exact| <= 1e-5 * |exact| + 2e-6 * rms(exact) for every output (each
+    block term moves by an ulp or two of itself, and a term is of the size of the outputs' spread, not of
+    the one output it lands in); flags = 0 through the
+    same entry point stays bit-identical to oxh_mmq; types and launch sizes without a relaxed kernel
+    (Q6_K, launches on the small tiles) give the exact bits under the flag as well."""
+    w = synth.weights(qtype, rows, cols, seed=6, stream=rows)
+    xs = synth.normal(n_vec * cols, seed=6, stream=n_vec).reshape(n_vec, cols)
+    d_w = mv.DeviceBuffer.from_host(w)
+    d_x = mv.DeviceBuffer.from_host(xs)
+    d_a = mv.DeviceBuffer(n_vec * mv.act_bytes(qtype, cols))
+    mv.quantize(qtype, d_x.ptr, cols, n_vec, cols, d_a.ptr)
+    outs = []
+    for mode in ("plain", "zero", "relaxed"):
+        d_o = mv.DeviceBuffer(n_vec * rows * 4)
+        if mode == "plain":
+            mv.mmq(qtype, d_w.ptr, rows, cols, d_a.ptr, n_vec, d_o.ptr, rows)
+        elif mode == "zero":
+            assert mv.lib().oxh_mmq_ex(qtype, ctypes.c_void_p(d_w.ptr), rows, cols, ctypes.c_void_p(d_a.ptr), n_vec,
+                                       ctypes.c_void_p(d_o.ptr), rows, 0, None) == 0
+        else:
+            mv.mmq(qtype, d_w.ptr, rows, cols, d_a.ptr, n_vec, d_o.ptr, rows, flags=mv.MMQ_RELAXED)
+        mv.sync()
+        outs.append(d_o.download(np.float32, n_vec * rows))
+        d_o.free()
+    exact, zero, relaxed = outs
+    assert np.array_equal(bits(exact), bits(zero))
+    rms = float(np.sqrt(np.mean(exact.astype(np.float64) ** 2)))
+    assert np.all(np.abs(relaxed - exact) <= 1e-5 * np.abs(exact) + 2e-6 * rms)
+    # the relaxed step exists for the two prefill tiles (256 or 128 rows x 128 tokens, 128 x 64), which a
+    # launch gets when it fills the device with them
+    has_relaxed_kernel = (qtype, rows) in ((Q4K, 14336), (Q4K, 4096), (Q5K, 7165), (Q5K, 3600)) and \
+        mv.device_info()["n_cu"] == 256
+    if has_relaxed_kernel:
+        assert not np.array_equal(bits(exact), bits(relaxed))       # it is a different evaluation
+    else:
+        assert np.array_equal(bits(exact), bits(relaxed))
+    assert mv.lib().oxh_mmq_ex(qtype, ctypes.c_void_p(d_w.ptr), rows, cols, ctypes.c_void_p(d_a.ptr), n_vec,
+                               ctypes.c_void_p(d_w.ptr), rows, 2, None) != 0           # unknown flag
