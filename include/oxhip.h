@@ -311,6 +311,16 @@ int oxh_mmq_ex(uint32_t qtype, const void *d_w, size_t rows, size_t cols,
                const void *d_acts, size_t n_vec, float *d_out, size_t out_stride,
                uint32_t flags, void *stream);
 
+/* The tile (weight rows x activations per workgroup) oxh_mmq picks for a launch
+ * on a device of n_cu compute units: the largest of 256 x 128 (128 x 128 for
+ * Q5_K, Q6_K and widened Q2_K), 64 x 128 (Q6_K only), 128 x 64, 64 x 32, 64 x 16
+ * that still gives nearly every compute unit a workgroup.  Pure host arithmetic
+ * (no device needed); OXH_DECLINED for a type without a matrix-core kernel.
+ * The reference has no counterpart: its batch kernel takes four activations
+ * per weight row regardless of the shape (oxk.c:787-836). */
+int oxh_mmq_tile(uint32_t qtype, size_t rows, size_t n_vec, size_t n_cu, uint32_t *tile_rows,
+                 uint32_t *tile_tokens);
+
 /* A Q3_K matrix rewritten as a Q6_K matrix that gives bit-identical results:
  * Q3_K's d * (sc - 32) * (code - 4) is Q6_K's d * sc6 * (code6 - 32) with
  * code6 = code + 28 and sc6 = sc - 32, over the same groups in the same

@@ -75,6 +75,7 @@ SIGNATURES = {
     "oxh_plan_deal": (I, [ctypes.POINTER(Z), ctypes.POINTER(I), Z, U32, ctypes.POINTER(U32), ctypes.POINTER(U32)]),
     "oxh_mmq": (I, [U32, V, Z, Z, V, Z, V, Z, V]),
     "oxh_mmq_ex": (I, [U32, V, Z, Z, V, Z, V, Z, U32, V]),
+    "oxh_mmq_tile": (I, [U32, Z, Z, Z, ctypes.POINTER(U32), ctypes.POINTER(U32)]),
     "oxh_get_rows": (I, [U32, V, Z, Z, V, Z, V, Z, V]),
     "oxh_debug_subblock_sums": (I, [U32, V, Z, Z, V, V, V]),
     "oxh_debug_read_probe": (I, [V, Z, V, V]),

@@ -1328,6 +1328,40 @@ static void mmq6_launch(const void *d_w, size_t rows, size_t blocks, const void 
                        (const uint8_t *)d_acts, (uint32_t)n_vec, d_out, out_stride);
 }
 
+/* Which tile a matrix-core launch runs on: the largest one that still gives (nearly) every compute
+ * unit a workgroup.  1: 256 x 128 (rows x tokens; 128 x 128 for the types with one row chunk per wave:
+ * Q5_K, Q6_K, widened Q2_K), 2: 128 x 64, 3: 64 x 32, 4: 64 x 16, 5: 64 x 128 on four waves, which only the
+ * Q6_K tile code has, for matrices with too few rows to fill the device with 128 x 128 tiles (the scaled
+ * weight operands a wave builds are then still reused by 128 tokens: 4096 x 14336 x 512 takes 144 us
+ * against 167 us on 128 x 64 tiles).  Pure arithmetic: OXH_MMQ_SHAPE = 1..5 overrides it at launch. */
+static int mmq_tile_shape(uint32_t qtype, size_t rows, size_t n_vec, size_t cus)
+{
+    const size_t need = cus - cus / 8;
+    if (n_vec <= 16) return 4;
+    if (n_vec <= 32) return 3;
+    if (qtype == OXH_Q6_K || is_q5k(qtype) || qtype == OXH_Q2_K_WIDE) {
+        if (((rows + 127) / 128) * ((n_vec + 127) / 128) >= need) return 1;
+        if (!is_q5k(qtype) && ((rows + 63) / 64) * ((n_vec + 127) / 128) >= need) return 5;
+        if (((rows + 127) / 128) * ((n_vec + 63) / 64) >= need) return 2;
+        return 3;
+    }
+    if (((rows + 255) / 256) * ((n_vec + 127) / 128) >= need) return 1;
+    if (((rows + 127) / 128) * ((n_vec + 63) / 64) >= need) return 2;
+    return 3;
+}
+
+extern "C" int oxh_mmq_tile(uint32_t qtype, size_t rows, size_t n_vec, size_t n_cu, uint32_t *tile_rows,
+                            uint32_t *tile_tokens)
+{
+    const bool one_chunk = qtype == OXH_Q6_K || is_q5k(qtype) || qtype == OXH_Q2_K_WIDE;
+    if ((!is_q4k(qtype) && !one_chunk) || rows == 0 || n_vec == 0 || n_cu == 0) return OXH_DECLINED;
+    static const uint32_t tr[6] = { 0, 256, 128, 64, 64, 64 }, tt[6] = { 0, 128, 64, 32, 16, 128 };
+    const int shape = mmq_tile_shape(qtype, rows, n_vec, n_cu);
+    if (tile_rows) *tile_rows = (shape == 1 && one_chunk) ? 128u : tr[shape];
+    if (tile_tokens) *tile_tokens = tt[shape];
+    return OXH_OK;
+}
+
 static int mmq_run(uint32_t qtype, const void *d_w, size_t rows, size_t cols, const void *d_acts, size_t n_vec,
                    float *d_out, size_t out_stride, bool relaxed, void *stream);
 
@@ -1366,34 +1400,10 @@ static int mmq_run(uint32_t qtype, const void *d_w, size_t rows, size_t cols, co
     /* the kernel addresses a workgroup's rows and tokens with 32-bit lane offsets */
     if (blocks * 292u * 256u > 0xFFFFFFFFull)
         return arg_fail("oxh_mmq: cols too large");
-    /* Shape: the largest tile that still gives (nearly) every CU a workgroup;
-     * OXH_MMQ_SHAPE = 1..4 forces 256x128, 128x64, 64x32, 64x16 (rows x tokens), 5 the 64x128 tile
-     * that only the Q6_K kernel has (128x64 for the others). */
     static int forced = -1;
     if (forced < 0) forced = (int)env_u32("OXH_MMQ_SHAPE", 0, 0, 5);
-    const size_t cus = (size_t)(g_n_cu > 0 ? g_n_cu : 256);
-    const size_t need = cus - cus / 8;
-    int shape = forced;
-    if (!shape) {
-        if (n_vec <= 16) shape = 4;
-        else if (n_vec <= 32) shape = 3;
-        else if (((rows + 255) / 256) * ((n_vec + 127) / 128) >= need) shape = 1;
-        else if (((rows + 127) / 128) * ((n_vec + 63) / 64) >= need) shape = 2;
-        else shape = 3;
-    }
+    int shape = forced ? forced : mmq_tile_shape(qtype, rows, n_vec, (size_t)(g_n_cu > 0 ? g_n_cu : 256));
     if (qtype == OXH_Q6_K || is_q5k(qtype) || wide2) {
-        /* one 16-row chunk per wave throughout: 128x128, 128x64, 64x32, 64x16; Q6_K also has 64x128
-         * on four waves (shape 5) for matrices with too few rows to fill the chip with 128x128 tiles: the
-         * scaled weight operands a wave builds are then still reused by 128 tokens (4096 x 14336 x 512:
-         * 144 us against 167 us with 128x64 tiles) */
-        if (!forced) {
-            if (n_vec <= 16) shape = 4;
-            else if (n_vec <= 32) shape = 3;
-            else if (((rows + 127) / 128) * ((n_vec + 127) / 128) >= need) shape = 1;
-            else if (!is_q5k(qtype) && ((rows + 63) / 64) * ((n_vec + 127) / 128) >= need) shape = 5;
-            else if (((rows + 127) / 128) * ((n_vec + 63) / 64) >= need) shape = 2;
-            else shape = 3;
-        }
         if (is_q5k(qtype)) {
             if (shape == 5) shape = 2;
             if (shape == 1 && relaxed)      mmq5_launch<8, 1, 8, true>(d_w, rows, blocks, d_acts, n_vec, d_out, out_stride, stream);
