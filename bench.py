@@ -203,7 +203,8 @@ def secondary_figures(mv, synth):
     x = synth.normal(cols, seed=0, stream=2003)
     d_x = mv.DeviceBuffer.from_host(x)
     d_o = mv.DeviceBuffer(rows * 4)
-    for name, qt in (("q2_k", 8), ("q3_k", 10), ("q4_0", 3), ("q4_1", 4), ("q5_0", 5), ("q5_1", 6)):
+    for name, qt in (("q2_k", 8), ("q3_k", 10), ("q4_0", 3), ("q4_1", 4), ("q5_0", 5), ("q5_1", 6),
+                     ("iq3_s", 25), ("iq1_xxxs", 36)):
         w = synth.weights(qt, rows, cols, seed=0, stream=7)
         copies = [mv.DeviceBuffer.from_host(w) for _ in range(8)]
         segs = [mv.make_segments([(c.ptr, d_o.ptr, rows, 0)]) for c in copies]
