@@ -895,10 +895,20 @@ static int mv_batch(uint32_t qtype, const uint8_t *data, size_t rows,
         } else {
             /* every activation is quantised once, then the slices run over the stored bytes */
             if ((rc = quantize(kind, d_x, cols, n_vec, cols, g_dact.p))) return rc;
-            for (size_t v0 = 0; v0 < n_vec; v0 += step) {
-                const size_t m = n_vec - v0 < step ? n_vec - v0 : step;
-                OxhSegment seg = { d_w, (float *)g_dout.p + v0 * rows, rows, v0, 0, NULL };
-                if ((rc = oxh_gemv_segments(qtype, &seg, 1, cols, g_dact.p, m, rows, NULL))) return rc;
+            /* up to 32 slices per launch, each slice a segment over the same matrix with its own run of
+             * activations and its own place in the output: 512 vectors of a 32-value format are one or
+             * two launches instead of 32 or 64, and slices overlap instead of queueing behind launch gaps */
+            enum { SLICES = 32 };
+            OxhSegment segs[SLICES];
+            size_t v0 = 0;
+            while (v0 < n_vec) {
+                size_t n = 0;
+                for (; n < SLICES && v0 < n_vec; n++, v0 += step) {
+                    const size_t m = n_vec - v0 < step ? n_vec - v0 : step;
+                    const OxhSegment seg = { d_w, (float *)g_dout.p + v0 * rows, rows, v0, m, NULL };
+                    segs[n] = seg;
+                }
+                if ((rc = oxh_gemv_segments(qtype, segs, n, cols, g_dact.p, step, rows, NULL))) return rc;
             }
         }
     }

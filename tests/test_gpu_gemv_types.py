@@ -437,3 +437,21 @@ def test_every_weight_byte_influences_its_row(oxh, qtype, size):
     ob = bits(out)
     same = [i for i in range(size) if ob[1 + 2 * i] == ob[0] and ob[2 + 2 * i] == ob[0]]
     assert not same, "bytes without influence: %s" % same
+
+
+@pytest.mark.parametrize("qtype,cols,n_vec", [(Q80, 896, 600), (Q80, 4096, 33), (25, 512, 300), (3, 1024, 530)])
+def test_long_batches_of_types_without_a_tile_kernel(oxh, qtype, cols, n_vec):
+    """Batches over the 32-value and codebook formats run as slices of a few activations, up to 32 slices
+    per launch: lengths that need several launches, a last launch with one slice, a ragged last slice."""
+    rows = 70
+    rb = synth.row_bytes(qtype, cols)
+    w = synth.weights(qtype, rows, cols, seed=61, stream=cols)
+    xs = synth.normal(n_vec * (cols + 8), seed=61, stream=n_vec).reshape(n_vec, cols + 8)
+    outs = np.full((n_vec, rows + 3), -7.25, np.float32)
+    temp = np.zeros(cols, np.float32)
+    scratch = np.zeros(mv.batch_scratch_bytes(cols), np.uint8)
+    assert mv.matvec_quantized_batch(qtype, w, rows, cols, rb, xs, cols + 8, outs, rows + 3, n_vec, temp, scratch) == 0
+    assert np.all(outs[:, rows:] == -7.25)
+    for v in list(range(0, n_vec, 37)) + [n_vec - 1]:
+        want, _ = oracle_matvec(qtype, w, rows, cols, np.ascontiguousarray(xs[v, :cols]))
+        assert np.array_equal(bits(outs[v, :rows]), bits(want)), v
