@@ -235,9 +235,13 @@ int oxh_gemv_segments_fused(uint32_t qtype, const OxhSegment *segs, size_t n_seg
  * vector is normalised and quantised once, by one workgroup, into device
  * memory the plan owns (about 1.3 bytes per input value), all workgroups meet
  * once, and from then on an operation's quantised input is copied into LDS
- * while the previous operation runs.  Same results; oxh_plan_prestaged says
+ * while the previous operation runs.  Consecutive operations of such a plan
+ * that read one weight layout over vectors of one length and are short (at
+ * most three passes per wave together: q/k/v and o of a layer) are walked as
+ * one operation with several inputs.  Same results; oxh_plan_prestaged says
  * whether a plan runs this way (OXH_PLAN_PRESTAGE=0 in the environment at
- * creation keeps such a plan on the chained kernel).
+ * creation keeps such a plan on the chained kernel, OXH_PLAN_MERGE=0 keeps
+ * every operation on its own).
  *
  * All workgroups must be resident together (one per compute unit; the kernel
  * needs the whole device, so do not run other kernels beside a plan launch).

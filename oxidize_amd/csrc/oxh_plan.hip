@@ -75,6 +75,8 @@ struct PlanSeg {
     gaddr w, w2;                    /* w2: the paired matrix or 0 */
     gaddr out;
     uint32_t rows, wg_begin, rows_q, rows_rem;
+    gaddr xq;                       /* k_plan_ext: the staged input this segment multiplies (segments of one
+                                     * table row may come from different operations, see plan_merge) */
 };
 
 struct PlanOp {
@@ -219,6 +221,7 @@ struct PWork {
     uint32_t wg_row0, wg_rows;      /* the workgroup's contiguous run of rows */
     uint32_t kind;
     uint32_t paired;                /* 0 / 1 (a whole word: the struct is copied around as scalars) */
+    gaddr xq;                       /* the workgroup's segment's staged input (k_plan_ext) */
 };
 
 __device__ __forceinline__ uint32_t plan_block_bytes(uint32_t kind)
@@ -240,6 +243,7 @@ __device__ __forceinline__ PWork plan_work(const PlanOp *op, uint32_t wave)
     const bool idle = wg >= uni(op->n_wg);
     const uint32_t wi0 = (wg - wg_begin) * PLAN_W, wi = wi0 + wave;
     k.kind = uni(op->kind);
+    k.xq = uni(sg->xq);
     k.row0 = wi * q + min(wi, rem);
     k.nrows = idle ? 0u : q + (wi < rem ? 1u : 0u);
     k.wg_row0 = wi0 * q + min(wi0, rem);
@@ -274,6 +278,7 @@ __device__ __forceinline__ PWork plan_work_flat(const PlanOp *op, uint32_t wave)
     const bool idle = wg >= uni(op->n_wg);
     const uint32_t wi0 = (wg - wg_begin) * PLAN_W;
     k.kind = uni(op->kind);
+    k.xq = idle ? (gaddr)0u : uni(sg->xq);
     k.out = gptr<float>(out);
     k.paired = w2 != 0u ? 1u : 0u;
     k.wg_row0 = wi0 * sq + min(wi0, srem);
@@ -694,17 +699,19 @@ __device__ __forceinline__ uint32_t plan_image_bytes(uint32_t kind, uint32_t blo
 }
 
 /* the staged input of an operation into LDS at byte address lds_addr, 1 KB pieces dealt to the waves */
-__device__ __forceinline__ void plan_image_fetch(const PlanOp *op, uint32_t lds_addr, uint32_t lane, uint32_t wave)
+__device__ __forceinline__ void plan_image_fetch(const PlanOp *op, gaddr xq, uint32_t lds_addr, uint32_t lane, uint32_t wave)
 {
+    if (xq == 0u) return;                       /* a workgroup without rows in this operation */
     const uint32_t bytes = plan_image_bytes(uni(op->kind), uni(op->blocks));
-    const uint8_t *img = gptr<const uint8_t>(uni(op->xq));
+    const uint8_t *img = gptr<const uint8_t>(xq);
     for (uint32_t k = wave * 1024u; k < bytes; k += PLAN_W * 1024u)
         if (k + 16u * lane < bytes) plan_dma16(img + k, 16u * lane, lds_addr + k);
 }
 
 template <bool HAS_Q5>
 __global__ __launch_bounds__(1024) void
-k_plan_ext(const PlanOp *__restrict__ ops, uint32_t n_ops, const PlanSync sy, const PlanLds ld)
+k_plan_ext(const PlanOp *__restrict__ ins, uint32_t n_ins, const PlanOp *__restrict__ ops, uint32_t n_ops,
+           const PlanSync sy, const PlanLds ld)
 {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     const uint32_t lds_base = (uint32_t)(size_t)(__attribute__((address_space(3))) uint8_t *)lds;
@@ -725,8 +732,8 @@ k_plan_ext(const PlanOp *__restrict__ ops, uint32_t n_ops, const PlanSync sy, co
     /* Inputs first: workgroup g stages the vectors of operations g, g + grid, ... exactly as the chained
      * kernel stages them (prologue, Q8_K quantisation, the layout the passes read) and stores the LDS
      * image with accesses every XCD sees.  The side outputs of a prologue are written here, once. */
-    for (uint32_t j = blockIdx.x; j < n_ops; j += gridDim.x) {
-        const OpHead op = plan_head(&tab[j]);
+    for (uint32_t j = blockIdx.x; j < n_ins; j += gridDim.x) {
+        const OpHead op = plan_head(&ins[j]);
         XStage xs;
 #pragma unroll
         for (int u = 0; u < 4; u++) xs.x[u] = xs.t[u] = xs.b[u] = XRegs{ 0.f, 0.f, 0.f, 0.f };
@@ -735,7 +742,7 @@ k_plan_ext(const PlanOp *__restrict__ ops, uint32_t n_ops, const PlanSync sy, co
         else                      plan_stage_finish<0>(op, xs, lds, red, true, lane, wave);
         __syncthreads();
         const uint32_t bytes = plan_image_bytes(op.kind, op.blocks);
-        const CohBuf img = coh_buf(gptr<uint8_t>(uni(tab[j].xq)));
+        const CohBuf img = coh_buf(gptr<uint8_t>(uni(ins[j].xq)));
         for (uint32_t k = threadIdx.x * 16u; k < bytes; k += 16384u)
             __builtin_amdgcn_raw_buffer_store_b128(*reinterpret_cast<const u32x4 *>(lds + k), img, (int)k, 0,
                                                    OXH_SYSTEM_COHERENT);
@@ -786,19 +793,21 @@ k_plan_ext(const PlanOp *__restrict__ ops, uint32_t n_ops, const PlanSync sy, co
         } else {
             /* every input is staged once every workgroup has said so */
             if (!plan_wait(sy, base + 1u, s_ok, ln, wave)) return;
-            plan_image_fetch(&tab[0], lds_base, ln, wave);
+            plan_image_fetch(&tab[0], cur.xq, lds_base, ln, wave);
             asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
             __syncthreads();
         }
         if (i == n_ops) break;
-        if (i + 1u < n_ops) plan_image_fetch(&tab[i + 1u], lds_base + ((i + 1u) & 1u) * ld.act_bytes, ln, wave);
+        PWork nx = cur;
+        if (i + 1u < n_ops) {
+            nx = plan_work_flat(&tab[i + 1u], wave);
+            plan_image_fetch(&tab[i + 1u], nx.xq, lds_base + ((i + 1u) & 1u) * ld.act_bytes, ln, wave);
+        }
         plan_stamp(sy, i, 1, ln, wave);
 
         const PlanOp *const op = &tab[i];
         const uint32_t Bk = uni(op->blocks);
         const uint8_t *act = lds + (size_t)(i & 1u) * ld.act_bytes;
-        PWork nx = cur;
-        if (i + 1u < n_ops) nx = plan_work_flat(&tab[i + 1u], wave);
         GemvParams gp;
         gp.blocks = Bk;
         gp.magic = uni(op->magic);
@@ -837,6 +846,8 @@ struct OxhPlan {
     uint32_t n_waits;               /* operations that wait (for callers' curiosity) */
     bool ext;                       /* no operation depends on another: inputs are staged ahead (k_plan_ext) */
     uint8_t *d_img;                 /* the staged inputs */
+    PlanOp *d_run;                  /* k_plan_ext: the table it walks (d_ops stays the list of inputs) */
+    uint32_t n_run;
 };
 
 static const void *plan_kernel(const OxhPlan *pl)
@@ -906,6 +917,79 @@ extern "C" int oxh_plan_deal(const size_t *rows, const int *paired, size_t n_seg
     return OXH_OK;
 }
 
+
+struct PlanLimits { uint32_t max_wg_rows, max_wg_terms, max_cap_terms; };
+
+/* Deals the rows of d's segments (rows, w2 filled in) to the grid and notes what the row tables must hold. */
+static int plan_deal_op(PlanOp &d, uint32_t grid, PlanLimits &lim)
+{
+    size_t rows[PLAN_MAX_SEGS];
+    int paired[PLAN_MAX_SEGS];
+    for (uint32_t k = 0; k < d.n_segs; k++) { rows[k] = d.s[k].rows; paired[k] = d.s[k].w2 != 0u; }
+    uint32_t n_wg[PLAN_MAX_SEGS], cap = 1;
+    const int drc = oxh_plan_deal(rows, paired, d.n_segs, grid, n_wg, &cap);
+    if (drc) return drc;
+    d.rows_cap = cap;
+    uint32_t wg = 0;
+    for (uint32_t k = 0; k < d.n_segs; k++) {
+        const size_t waves = (size_t)n_wg[k] * PLAN_W;
+        d.s[k].wg_begin = wg;
+        d.s[k].rows_q = (uint32_t)(rows[k] / waves);
+        d.s[k].rows_rem = (uint32_t)(rows[k] % waves);
+        const uint32_t per_wg = (uint32_t)((rows[k] / waves + 1) * PLAN_W);
+        if (per_wg > lim.max_wg_rows) lim.max_wg_rows = per_wg;
+        const uint32_t flat = per_wg * (paired[k] ? 2u : 1u) * d.term_stride;
+        if (flat > lim.max_wg_terms) lim.max_wg_terms = flat;
+        wg += n_wg[k];
+    }
+    d.n_wg = wg;
+    if (cap * d.term_stride > lim.max_cap_terms) lim.max_cap_terms = cap * d.term_stride;
+    return OXH_OK;
+}
+
+/* Operations none of which depends on another may run in any grouping.  Consecutive ones that read
+ * the same weight layout over vectors of the same length are put into ONE table row when together
+ * they are still a short operation (at most three passes per wave on average): their segments side by
+ * side, each with the staged input of the operation it came from.  Two operations of one pass per wave
+ * each (q/k/v and o of a layer) would otherwise be two trips that each wait out a memory latency with
+ * one load in flight per wave; merged, a wave has two or three passes to overlap.  Returns the number
+ * of rows written to `run`. */
+static int plan_merge(const PlanOp *h, size_t n_ops, uint32_t grid, bool merge, PlanOp *run, size_t *n_run,
+                      PlanLimits &lim)
+{
+    const size_t limit = (size_t)grid * PLAN_W * 16u * 3u;         /* blocks: three passes per wave */
+    size_t n = 0;
+    for (size_t i = 0; i < n_ops;) {
+        PlanOp g = h[i];
+        size_t work = 0;
+        for (uint32_t k = 0; k < g.n_segs; k++) {
+            g.s[k].xq = h[i].xq;
+            work += (size_t)g.s[k].rows * (g.s[k].w2 ? 2u : 1u) * g.blocks;
+        }
+        size_t j = i + 1;
+        while (merge && j < n_ops && h[j].kind == g.kind && h[j].blocks == g.blocks &&
+               g.n_segs + h[j].n_segs <= PLAN_MAX_SEGS) {
+            size_t more = 0;
+            for (uint32_t k = 0; k < h[j].n_segs; k++)
+                more += (size_t)h[j].s[k].rows * (h[j].s[k].w2 ? 2u : 1u) * g.blocks;
+            if (work + more > limit) break;
+            for (uint32_t k = 0; k < h[j].n_segs; k++) {
+                g.s[g.n_segs] = h[j].s[k];
+                g.s[g.n_segs].xq = h[j].xq;
+                g.n_segs++;
+            }
+            work += more;
+            j++;
+        }
+        const int drc = plan_deal_op(g, grid, lim);
+        if (drc) return drc;
+        run[n++] = g;
+        i = j;
+    }
+    *n_run = n;
+    return OXH_OK;
+}
+
 extern "C" int oxh_plan_create(const OxhPlanOp *ops, size_t n_ops, OxhPlan **out)
 {
     if (!out) return oxh_internal_errorf(OXH_ERR_ARG, "invalid argument: oxh_plan_create: NULL");
@@ -923,7 +1007,8 @@ extern "C" int oxh_plan_create(const OxhPlanOp *ops, size_t n_ops, OxhPlan **out
         free(h); free(reads); free(writes);
         return oxh_internal_errorf(OXH_ERR_NOMEM, "out of host memory building a plan");
     }
-    uint32_t max_act = 0, max_cap_terms = 0, max_wg_rows = 0, max_wg_terms = 0, n_waits = 0;
+    uint32_t max_act = 0, n_waits = 0;
+    PlanLimits lim = { 0, 0, 0 };
     size_t img_bytes = 0;
     bool has_q5 = false;
     rc = OXH_OK;
@@ -986,28 +1071,12 @@ extern "C" int oxh_plan_create(const OxhPlanOp *ops, size_t n_ops, OxhPlan **out
         if (rc) break;
         if (ns == 0) { rc = oxh_internal_errorf(OXH_ERR_ARG, "invalid argument: plan: operation %zu has no rows", i); break; }
         d.n_segs = ns;
-        uint32_t n_wg[PLAN_MAX_SEGS], cap = 1;
-        const int drc = oxh_plan_deal(rows, paired, ns, grid, n_wg, &cap);
+        const int drc = plan_deal_op(d, grid, lim);
         if (drc) { rc = oxh_internal_errorf(drc, "plan: operation %zu has more rows than %u workgroups can own", i, grid); break; }
-        d.rows_cap = cap;
-        uint32_t wg = 0;
-        for (uint32_t k = 0; k < ns; k++) {
-            const size_t waves = (size_t)n_wg[k] * PLAN_W;
-            d.s[k].wg_begin = wg;
-            d.s[k].rows_q = (uint32_t)(rows[k] / waves);
-            d.s[k].rows_rem = (uint32_t)(rows[k] % waves);
-            const uint32_t per_wg = (uint32_t)((rows[k] / waves + 1) * PLAN_W);
-            if (per_wg > max_wg_rows) max_wg_rows = per_wg;
-            const uint32_t flat = per_wg * (paired[k] ? 2u : 1u) * d.term_stride;
-            if (flat > max_wg_terms) max_wg_terms = flat;
-            wg += n_wg[k];
-        }
-        d.n_wg = wg;
         const uint32_t act = kind >= PLAN_Q6_K ? q8k6_lds_bytes(d.blocks) : q8k_lds_bytes(d.blocks);
         if (act > max_act) max_act = act;
         d.xq = (gaddr)img_bytes;                    /* offset for now; the base is added once it exists */
         img_bytes += (act + 255u) & ~(size_t)255u;
-        if (cap * d.term_stride > max_cap_terms) max_cap_terms = cap * d.term_stride;
 
         /* what the operation reads and writes, for the dependency scan */
         const size_t xb = o.cols * sizeof(float);
@@ -1059,43 +1128,65 @@ extern "C" int oxh_plan_create(const OxhPlanOp *ops, size_t n_ops, OxhPlan **out
         const char *ps = getenv("OXH_PLAN_PRESTAGE");
         pl->ext = n_waits == 0 && !(ps && ps[0] == '0');
     }
+    /* the table the kernel walks: the operations themselves, or (independent operations) short
+     * neighbours merged into one row (OXH_PLAN_MERGE=0 keeps them apart) */
+    PlanOp *run = nullptr;
+    size_t n_run = n_ops;
+    if (pl->ext) {
+        const char *pm = getenv("OXH_PLAN_MERGE");
+        run = (PlanOp *)calloc(n_ops, sizeof *run);
+        if (!run) { free(h); free(pl); return oxh_internal_errorf(OXH_ERR_NOMEM, "out of host memory building a plan"); }
+        const int mrc = plan_merge(h, n_ops, grid, !(pm && pm[0] == '0'), run, &n_run, lim);
+        if (mrc) {
+            free(h); free(run); free(pl);
+            return oxh_internal_errorf(mrc, "plan: merged operations have more rows than %u workgroups can own", grid);
+        }
+    }
+    pl->n_run = (uint32_t)n_run;
     pl->ld.act_bytes = (max_act + 15u) & ~15u;
     pl->ld.outs_off = 2u * pl->ld.act_bytes;
-    pl->ld.red_off = pl->ld.outs_off + ((max_wg_rows * 4u + 15u) & ~15u);
+    pl->ld.red_off = pl->ld.outs_off + ((lim.max_wg_rows * 4u + 15u) & ~15u);
     pl->ld.terms_off = pl->ld.red_off + 128u;
-    pl->ld.terms_per_wave = max_cap_terms;
-    pl->ld.terms_wg = (max_wg_terms + 3u) & ~3u;
-    pl->ld.table_off = (pl->ld.terms_off + (pl->ext ? 2u * pl->ld.terms_wg : PLAN_W * max_cap_terms) * 4u + 15u) & ~15u;
-    pl->lds_bytes = (size_t)pl->ld.table_off + n_ops * sizeof(PlanOp);
+    pl->ld.terms_per_wave = lim.max_cap_terms;
+    pl->ld.terms_wg = (lim.max_wg_terms + 3u) & ~3u;
+    pl->ld.table_off = (pl->ld.terms_off + (pl->ext ? 2u * pl->ld.terms_wg : PLAN_W * lim.max_cap_terms) * 4u + 15u) & ~15u;
+    pl->lds_bytes = (size_t)pl->ld.table_off + n_run * sizeof(PlanOp);
     const char *sl = getenv("OXH_PLAN_SPIN_LIMIT");
     pl->spin_limit = sl && *sl ? (uint32_t)strtoul(sl, nullptr, 10) : 4000000u;
     if (pl->lds_bytes > 160u * 1024u) {
-        free(h); free(pl);
+        free(h); free(run); free(pl);
         return oxh_internal_errorf(OXH_ERR_TOO_WIDE, "plan: the staged activation, the row tables and the table of %zu operations (%zu bytes each) do not fit 160 KiB of LDS; split the chain into several plans", n_ops, sizeof(PlanOp));
     }
     const void *kernel = plan_kernel(pl);
     {
         hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-        if (e != hipSuccess) { free(h); free(pl); return oxh_internal_errorf(OXH_ERR_HIP, "HIP error in hipFuncSetAttribute: %s", hipGetErrorString(e)); }
+        if (e != hipSuccess) { free(h); free(run); free(pl); return oxh_internal_errorf(OXH_ERR_HIP, "HIP error in hipFuncSetAttribute: %s", hipGetErrorString(e)); }
     }
     /* every workgroup must be resident at once: one per compute unit fits by construction when the
      * device can hold one workgroup of this kernel per unit */
     int per_cu = 0;
     hipError_t e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, 1024, pl->lds_bytes);
     if (e != hipSuccess || per_cu < 1) {
-        free(h); free(pl);
+        free(h); free(run); free(pl);
         return oxh_internal_errorf(OXH_ERR_HIP, "plan: the device cannot hold one workgroup of the plan kernel per compute unit");
     }
     e = hipMalloc((void **)&pl->d_ops, n_ops * sizeof(PlanOp));
     if (e == hipSuccess && pl->ext) e = hipMalloc((void **)&pl->d_img, img_bytes);
+    if (e == hipSuccess && pl->ext) e = hipMalloc((void **)&pl->d_run, n_run * sizeof(PlanOp));
+    /* the staged inputs' offsets become addresses */
     for (size_t i = 0; i < n_ops; i++) h[i].xq = pl->ext ? (gaddr)(uintptr_t)pl->d_img + h[i].xq : 0u;
+    for (size_t i = 0; run && i < n_run; i++)
+        for (uint32_t k = 0; k < run[i].n_segs; k++) run[i].s[k].xq += (gaddr)(uintptr_t)pl->d_img;
     if (e == hipSuccess) e = hipMalloc((void **)&pl->d_sync, (PLAN_MAX_WG + 8u) * sizeof(uint32_t));
     if (e == hipSuccess) e = hipMemcpy(pl->d_ops, h, n_ops * sizeof(PlanOp), hipMemcpyHostToDevice);
+    if (e == hipSuccess && pl->ext) e = hipMemcpy(pl->d_run, run, n_run * sizeof(PlanOp), hipMemcpyHostToDevice);
     if (e == hipSuccess) e = hipMemset(pl->d_sync, 0, (PLAN_MAX_WG + 8u) * sizeof(uint32_t));
     if (e == hipSuccess) e = hipDeviceSynchronize();
     free(h);
+    free(run);
     if (e != hipSuccess) {
         if (pl->d_ops) (void)hipFree(pl->d_ops);
+        if (pl->d_run) (void)hipFree(pl->d_run);
         if (pl->d_img) (void)hipFree(pl->d_img);
         if (pl->d_sync) (void)hipFree(pl->d_sync);
         free(pl);
@@ -1118,14 +1209,18 @@ extern "C" int oxh_plan_launch(OxhPlan *pl, void *stream)
 #define PLAN_LAUNCH(K)                                                                                  \
     hipLaunchKernelGGL(K, dim3(pl->grid), dim3(1024), pl->lds_bytes, st, (const PlanOp *)pl->d_ops,    \
                        pl->n_ops, sy, pl->ld)
+#define PLAN_LAUNCH_EXT(K)                                                                              \
+    hipLaunchKernelGGL(K, dim3(pl->grid), dim3(1024), pl->lds_bytes, st, (const PlanOp *)pl->d_ops,    \
+                       pl->n_ops, (const PlanOp *)pl->d_run, pl->n_run, sy, pl->ld)
     if (pl->ext) {
-        if (pl->has_q5) PLAN_LAUNCH(k_plan_ext<true>);
-        else            PLAN_LAUNCH(k_plan_ext<false>);
+        if (pl->has_q5) PLAN_LAUNCH_EXT(k_plan_ext<true>);
+        else            PLAN_LAUNCH_EXT(k_plan_ext<false>);
     } else {
         if (pl->has_q5) PLAN_LAUNCH(k_plan<true>);
         else            PLAN_LAUNCH(k_plan<false>);
     }
 #undef PLAN_LAUNCH
+#undef PLAN_LAUNCH_EXT
     PLAN_TRY(hipGetLastError());
     return OXH_OK;
 }
@@ -1180,6 +1275,7 @@ extern "C" int oxh_plan_destroy(OxhPlan *pl)
     if (!pl) return OXH_OK;
     hipError_t e = hipDeviceSynchronize();
     if (pl->d_ops) (void)hipFree(pl->d_ops);
+    if (pl->d_run) (void)hipFree(pl->d_run);
     if (pl->d_img) (void)hipFree(pl->d_img);
     if (pl->d_sync) (void)hipFree(pl->d_sync);
     free(pl);

@@ -21,7 +21,7 @@ def bits(a):
 
 
 @pytest.mark.parametrize("hidden,kv,ffn,layers", [(1024, 256, 2816, 3), (4096, 1024, 14336, 2), (256, 256, 512, 5)])
-def test_independent_set_matches_single_launches_and_oracle(oxh, hidden, kv, ffn, layers):
+def test_independent_set_matches_single_launches_and_oracle(oxh, monkeypatch, hidden, kv, ffn, layers):
     d = DecodeSet(hidden=hidden, kv=kv, ffn=ffn, layers=layers, seed=3, keep_host=(0,))
     d.launch_step()
     mv.sync()
@@ -35,13 +35,25 @@ def test_independent_set_matches_single_launches_and_oracle(oxh, hidden, kv, ffn
     info = plan.info()
     assert info["n_ops"] == 4 * layers and info["n_waits"] == 0      # nothing depends on anything here
     assert info["prestaged"]                                          # so the inputs are staged ahead
+    # short neighbours of one layout (q/k/v and o) share a table row by default; the same plan with every
+    # operation in a row of its own must give the same bits
+    monkeypatch.setenv("OXH_PLAN_MERGE", "0")
+    apart = mv.Plan(d.plan_ops())
+    monkeypatch.delenv("OXH_PLAN_MERGE")
+    assert apart.info()["lds_bytes"] > info["lds_bytes"]              # a longer table
     for rep in range(2):
-        plan.launch()
-        assert plan.status() == 0
-        for l in range(layers):
-            for op in range(4):
-                assert np.array_equal(bits(d.output(l, op)), bits(want_out[l][op])), (rep, l, op)
-                assert np.array_equal(d.activation(l, op), want_act[l][op]), (rep, l, op)
+        for p in (plan, apart):
+            for l in range(layers):
+                for op in range(4):
+                    mv.lib().oxh_memset(ctypes.c_void_p(d.out[l][op].ptr), 0xFF, d.out[l][op].nbytes, None)
+                    mv.lib().oxh_memset(ctypes.c_void_p(d.act[l][op].ptr), 0xFF, d.act[l][op].nbytes, None)
+            p.launch()
+            assert p.status() == 0
+            for l in range(layers):
+                for op in range(4):
+                    assert np.array_equal(bits(d.output(l, op)), bits(want_out[l][op])), (rep, l, op)
+                    assert np.array_equal(d.activation(l, op), want_act[l][op]), (rep, l, op)
+    apart.destroy()
     # and one matrix against the oracle directly
     o = oxlibs.oracle()
     name, qt, rows, cols, _ = d.ops[3]
