@@ -242,3 +242,100 @@ def test_what_a_plan_declines(oxh):
     with pytest.raises(mv.OxhError) as e:
         mv.Plan([dict(qtype=Q4K, segs=mv.make_segments([(w.ptr, x.ptr, 8, 0)]), cols=1024, d_x=x.ptr)])
     assert e.value.status == _lib.ERR_ARG
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_random_independent_plans_match_the_launches(oxh, seed):
+    """Seeded random plans of independent operations: one to four segments of ragged sizes (fewer rows than
+    waves, rows no multiple of anything), pairs, every kind a plan takes (the regrouped Q6_K included),
+    vector lengths that make neighbours mergeable and not, prologues with side outputs; each operation is
+    also launched on its own and every output, stored activation and side output compared bit for bit,
+    on two launches with new inputs in between."""
+    rng = np.random.default_rng(1000 + seed)
+    G8 = mv.Q6_K_G8
+    kinds = [Q4K, Q4K, Q5K, Q6K, G8]
+    n_ops = int(rng.integers(3, 12))
+    ops, bufs = [], []
+    cols_choices = [256, 1024, 2048, 4096]
+    cols = int(rng.choice(cols_choices))
+    for i in range(n_ops):
+        if rng.random() < 0.4:
+            cols = int(rng.choice(cols_choices))          # else: same length as the neighbour (mergeable)
+        qt = int(rng.choice(kinds))
+        if qt == G8 and cols % 2048:
+            qt = Q6K
+        file_qt = Q6K if qt == G8 else qt
+        rb = synth.row_bytes(file_qt, cols)
+        n_seg = int(rng.integers(1, 5))
+        paired = rng.random() < 0.25
+        if paired:
+            n_seg = min(n_seg, 2)
+        seg_rows = [int(rng.choice([1, 3, 17, 100, 257, 1000, 2500, int(rng.integers(1, 3000))])) for _ in range(n_seg)]
+        total = sum(seg_rows) * (2 if paired else 1)
+        w_host = synth.weights(file_qt, total, cols, seed=seed, stream=100 + i)
+        w = mv.DeviceBuffer.from_host(w_host)
+        if qt == G8:
+            g = mv.DeviceBuffer(w_host.nbytes)
+            mv.q6_k_group(w.ptr, total, cols, g.ptr)
+            mv.sync()
+            w = g
+        b = dict(w=w, x=mv.DeviceBuffer(cols * 4), add=mv.DeviceBuffer(cols * 4), out=mv.DeviceBuffer(sum(seg_rows) * 4),
+                 act=mv.DeviceBuffer(mv.act_bytes(file_qt, cols)), pout=mv.DeviceBuffer(cols * 4), sout=mv.DeviceBuffer(cols * 4),
+                 g=mv.DeviceBuffer.from_host((synth.normal(cols, seed=seed, stream=300 + i) * np.float32(0.1) + np.float32(1)).astype(np.float32)),
+                 cols=cols, n_out=sum(seg_rows), act_bytes=mv.act_bytes(file_qt, cols))
+        items, row, out_off = [], 0, 0
+        for r in seg_rows:
+            first = w.ptr + row * rb
+            if paired:
+                items.append((first, b["out"].ptr + out_off * 4, r, 0, 0, first + r * rb))
+                row += 2 * r
+            else:
+                items.append((first, b["out"].ptr + out_off * 4, r, 0))
+                row += r
+            out_off += r
+        op = dict(qtype=qt, segs=mv.make_segments(items), cols=cols, d_x=b["x"].ptr)
+        if rng.random() < 0.5:
+            op["d_act_out"] = b["act"].ptr
+        pro = rng.random()
+        if pro < 0.2:
+            op.update(kind=mv.PRO_RMSNORM, d_b=b["g"].ptr, eps=1e-5, d_pro_out=b["pout"].ptr)
+        elif pro < 0.35:
+            op.update(kind=mv.PRO_RMSNORM, d_b=b["g"].ptr, eps=1e-5, d_add=b["add"].ptr, d_sum_out=b["sout"].ptr)
+        elif pro < 0.45:
+            op.update(kind=mv.PRO_SWIGLU, d_b=b["add"].ptr, d_pro_out=b["pout"].ptr)
+        ops.append(op)
+        bufs.append(b)
+    plan = mv.Plan(ops)
+    assert plan.info()["prestaged"]
+
+    def state():
+        return [(b["out"].download(np.float32, b["n_out"]), b["act"].download(np.uint8, b["act_bytes"]),
+                 b["pout"].download(np.float32, b["cols"]), b["sout"].download(np.float32, b["cols"])) for b in bufs]
+
+    def clear():
+        for b in bufs:
+            for k in ("out", "act", "pout", "sout"):
+                mv.lib().oxh_memset(ctypes.c_void_p(b[k].ptr), 0xFF, b[k].nbytes, None)
+
+    for rep in range(2):
+        for i, b in enumerate(bufs):
+            b["x"].upload(synth.normal(b["cols"], seed=seed * 10 + rep, stream=i))
+            b["add"].upload(synth.normal(b["cols"], seed=seed * 10 + rep, stream=50 + i))
+        clear()
+        for op in ops:
+            if op.get("kind"):
+                mv.gemv_segments_fused(op["qtype"], op["segs"], op["cols"], op["d_x"], op["cols"], op["kind"], op["d_b"],
+                                       op.get("eps", 0.0), op.get("d_pro_out"), op.get("d_act_out"), 1, 0, None,
+                                       d_add=op.get("d_add"), d_sum_out=op.get("d_sum_out"))
+            else:
+                mv.gemv_segments_f32(op["qtype"], op["segs"], op["cols"], op["d_x"], op["cols"], op.get("d_act_out"))
+        mv.sync()
+        want = state()
+        clear()
+        plan.launch()
+        assert plan.status() == 0
+        for i, (w_, g_) in enumerate(zip(want, state())):
+            for k, name in enumerate(("out", "act", "prologue out", "sum out")):
+                a, c = np.ascontiguousarray(w_[k]).view(np.uint8), np.ascontiguousarray(g_[k]).view(np.uint8)
+                assert np.array_equal(a, c), (seed, rep, i, name, ops[i]["qtype"], ops[i]["cols"])
+    plan.destroy()
