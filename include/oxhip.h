@@ -444,6 +444,13 @@ int oxh_debug_moe_workspace_parts(const OxhMoe *m, size_t n_tok, size_t parts[12
  * included.  No counterpart in the reference. */
 int oxh_debug_read_probe(const void *d_buf, size_t bytes, uint32_t *d_sink, void *stream);
 
+/* Measurement aid: the int8 matrix-core rate of the whole device (POP/s) when
+ * every v_mfma_i32_16x16x64_i8 is followed by `valu_per_mfma` (0, 1, 2 or 4)
+ * independent f32 vector instructions, with 1..4 waves per SIMD.  Synchronous
+ * (two launches, the second timed with events).  Shows whether vector work
+ * hides behind matrix work on the device.  No counterpart in the reference. */
+int oxh_debug_mfma_probe(int valu_per_mfma, int waves_per_simd, double *pops);
+
 /* Test hook: the integer sub-block sums the GEMV kernel forms, written by the
  * same device code path.  Q4_K and Q5_K: 8 int32 per super-block (S_j), Q6_K: 16 per
  * super-block, Q8_0: 1 per block; layout [row][block][j].  The reference

@@ -79,6 +79,7 @@ SIGNATURES = {
     "oxh_get_rows": (I, [U32, V, Z, Z, V, Z, V, Z, V]),
     "oxh_debug_subblock_sums": (I, [U32, V, Z, Z, V, V, V]),
     "oxh_debug_read_probe": (I, [V, Z, V, V]),
+    "oxh_debug_mfma_probe": (I, [I, I, ctypes.POINTER(ctypes.c_double)]),
     "oxh_q3_k_as_q6_k": (I, [V, Z, Z, V, V]),
     "oxh_q2_k_widen": (I, [V, Z, Z, V, V]),
     "oxh_moe_workspace_bytes": (I, [ctypes.POINTER(OxhMoe), Z, ctypes.POINTER(Z)]),

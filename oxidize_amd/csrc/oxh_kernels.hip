@@ -1273,6 +1273,71 @@ extern "C" int oxh_debug_read_probe(const void *d_buf, size_t bytes, uint32_t *d
     return OXH_OK;
 }
 
+/* Measurement aid: what the matrix cores deliver when vector instructions run beside them.  Every wave
+ * issues `iters` x 16 independent v_mfma_i32_16x16x64_i8 (four accumulators in turn) with NV plain f32
+ * multiply or add instructions, independent of the MFMAs, after each of them.  On this device the two do
+ * not overlap, within a wave or between the waves of a SIMD: a launch with NV = 4 reaches 2.6 POP/s
+ * against 4.9 POP/s with NV = 0 at any occupancy, i.e. an MFMA costs 16 cycles of the SIMD and a vector
+ * instruction 3.5 more.  That is what bounds the prefill kernel, whose exact float step and operand
+ * building are vector instructions. */
+template <int NV>
+__global__ __launch_bounds__(1024) void
+k_mfma_probe(uint32_t iters, float *__restrict__ sink)
+{
+    const uint32_t lane = threadIdx.x & 63u;
+    const v4i a = { (int)lane, 2, 3, 4 }, b = { 5, (int)lane, 7, 8 };
+    v4i c[4] = { { 0, 0, 0, 0 }, { 0, 0, 0, 0 }, { 0, 0, 0, 0 }, { 0, 0, 0, 0 } };
+    float f[4] = { (float)lane, 1.0f, 2.0f, 3.0f };
+    for (uint32_t i = 0; i < iters; i++) {
+#pragma unroll
+        for (int j = 0; j < 16; j++) {
+            c[j & 3] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b, c[j & 3], 0, 0, 0);
+#pragma unroll
+            for (int k = 0; k < NV; k++) {
+                float &v = f[(j * NV + k) & 3];
+                v = ((j * NV + k) & 4) ? v + 0.5f : v * 1.0001f;
+            }
+        }
+    }
+    if (c[0][0] + c[1][1] + c[2][2] + c[3][3] == 0x7fffffff || f[0] + f[1] + f[2] + f[3] == 12345.0f)
+        sink[0] = f[0];
+}
+
+extern "C" int oxh_debug_mfma_probe(int valu_per_mfma, int waves_per_simd, double *pops)
+{
+    int rc = ensure_init();
+    if (rc) return rc;
+    if (!pops || waves_per_simd < 1 || waves_per_simd > 4) return arg_fail("oxh_debug_mfma_probe: 1..4 waves per SIMD");
+    float *d_sink = nullptr;
+    HIP_TRY(hipMalloc((void **)&d_sink, 64));
+    const uint32_t iters = 4000, cus = (uint32_t)(g_n_cu > 0 ? g_n_cu : 256), threads = 256u * (uint32_t)waves_per_simd;
+    hipStream_t st = pick_stream(nullptr);
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    hipError_t e = hipEventCreate(&e0);
+    if (e == hipSuccess) e = hipEventCreate(&e1);
+    for (int rep = 0; rep < 2 && e == hipSuccess; rep++) {      /* the first launch warms up */
+        if (rep == 1) e = hipEventRecord(e0, st);
+        switch (valu_per_mfma) {
+        case 0: hipLaunchKernelGGL(k_mfma_probe<0>, dim3(cus), dim3(threads), 0, st, iters, d_sink); break;
+        case 1: hipLaunchKernelGGL(k_mfma_probe<1>, dim3(cus), dim3(threads), 0, st, iters, d_sink); break;
+        case 2: hipLaunchKernelGGL(k_mfma_probe<2>, dim3(cus), dim3(threads), 0, st, iters, d_sink); break;
+        case 4: hipLaunchKernelGGL(k_mfma_probe<4>, dim3(cus), dim3(threads), 0, st, iters, d_sink); break;
+        default: e = hipErrorInvalidValue; break;
+        }
+    }
+    if (e == hipSuccess) e = hipEventRecord(e1, st);
+    if (e == hipSuccess) e = hipEventSynchronize(e1);
+    float ms = 0.0f;
+    if (e == hipSuccess) e = hipEventElapsedTime(&ms, e0, e1);
+    if (e0) (void)hipEventDestroy(e0);
+    if (e1) (void)hipEventDestroy(e1);
+    (void)hipFree(d_sink);
+    if (e != hipSuccess) return valu_per_mfma == 3 || valu_per_mfma > 4 || valu_per_mfma < 0
+                                    ? arg_fail("oxh_debug_mfma_probe: valu_per_mfma is 0, 1, 2 or 4") : hip_fail(e, "oxh_debug_mfma_probe");
+    *pops = (double)cus * (threads / 64u) * iters * 16.0 * 32768.0 / ((double)ms * 1e12);
+    return OXH_OK;
+}
+
 extern "C" int oxh_debug_subblock_sums(uint32_t qtype, const void *d_w, size_t rows,
                                        size_t cols, const void *d_act, int32_t *d_sums,
                                        void *stream)
