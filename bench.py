@@ -35,8 +35,8 @@ HBM_PEAK_GBPS = 8000.0
 # same counters read for a 256 MiB device-to-device copy).  Not measured live.
 GATE_UP_TRAFFIC_BYTES = 66496518
 # HBM bytes one k_plan_ext launch (a whole 32-layer step) moves, measured the same way: FETCH_SIZE
-# 2168740.9 KiB x 1.9998, WRITE_SIZE 7322.03 KiB x 1.000 (algorithmic: 4419223552, ratio 1.0067).
-PLAN_STEP_TRAFFIC_BYTES = 4448654782
+# 2170528.0 KiB x 1.9998, WRITE_SIZE 7322.03 KiB x 1.000 (algorithmic: 4419223552, ratio 1.0075).
+PLAN_STEP_TRAFFIC_BYTES = 4452278522
 INT8_PEAK_TOPS = 5033.0     # dense int8 MFMA: 256 CU x 2.4 GHz x 8192 op/clk/CU
 
 
