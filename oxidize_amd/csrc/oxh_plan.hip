@@ -430,88 +430,168 @@ plan_row_sums(const float *terms, const PWork &k, uint32_t B, uint32_t term_stri
 /* ─── activation staging: one f32 vector -> Q8_K in LDS ──────────────── */
 
 /* Staging is split in two so that the loads can be placed where they hurt least in the wave's
- * in-order memory queue: plan_stage_issue asks for this wave's (up to four) 256-value units of the
- * input vector and of whatever the prologue combines it with; plan_stage_finish applies the prologue,
- * quantises and writes LDS.  A vector another workgroup wrote a moment ago is read with coherent
- * loads; inputs nobody in this launch wrote come through the caches.  Arithmetic and order are
- * stage_begin / stage_end's for one vector and sixteen waves, so the quantised bytes are the same. */
+ * in-order memory queue: plan_stage_issue asks for this wave's part of the input vector and of whatever
+ * the prologue combines it with; plan_stage_finish applies the prologue, quantises and writes LDS.  A
+ * vector another workgroup wrote a moment ago is read with coherent loads; inputs nobody in this launch
+ * wrote come through the caches.
+ *
+ * The launches (stage_begin / stage_end) give a wave one 256-value unit at a time, lane l holding
+ * values 4l .. 4l+3.  Here a block goes to 16 lanes: lane l of a row holds values 16l .. 16l+15 of
+ * block 4 * wave + row.  An instruction costs a 1024-thread workgroup sixteen issue slots whatever its
+ * lanes do, so the quantiser's fixed part (maximum, two divisions, slot arithmetic, stores) is paid once
+ * per four blocks instead of once per block, and for 4096 values four waves run it while twelve go on
+ * to their weight requests.  The bytes are the launches': a maximum and the integer sums do not depend
+ * on the order they are taken in, and the sum of squares is added in the launches' order.  There, lane
+ * L of wave W adds up its four squares of units W, W + 16, ... in turn, the wave adds its lanes in
+ * four exchange steps (neighbour, pair, eight, sixteen) and combines its four rows as (r0 + r1) + (r2 +
+ * r3), and the waves' sums are added the same way.  A lane here holds what four neighbouring lanes
+ * hold there: row 4w + r of waves 0..3 stands for wave W = 4w + r, walks W's units, does the first two
+ * steps in registers, and the same four exchange instructions then perform the launches' last two steps
+ * and the combination of the four rows. */
 struct XStage {
     XRegs x[4], t[4], b[4];
 };
 
-__device__ __forceinline__ XRegs load4_either(bool coherent, const float *base, CohBuf cb, uint32_t at)
-{
-    if (coherent) return cload4(cb, at * 4u);
-    return x_load4(base + at);
-}
-
+/* Every vector that may have been written in this launch is read with coherent loads, whether it was
+ * or not: choosing the instruction per load at run time gives the compiler two definitions of each
+ * register to merge, which it does with a move, and a move waits for the load (and for the weights
+ * requested before it). */
 __device__ __forceinline__ void
-plan_stage_issue(const OpHead &op, XStage &xs, bool coherent, uint32_t lane, uint32_t wave)
+plan_stage_issue(const OpHead &op, XStage &xs, uint32_t lane, uint32_t wave)
 {
-    const uint32_t B = op.blocks, pro = op.pro;
-    const float *x = gptr<const float>(op.x), *add = gptr<const float>(op.pro_add), *b = gptr<const float>(op.pro_b);
-    const CohBuf xc = coh_buf(x), ac = coh_buf(add), bc = coh_buf(b);
+    const uint32_t pro = op.pro;
+    const float *b = gptr<const float>(op.pro_b);
+    const CohBuf xc = coh_buf(gptr<const float>(op.x)), ac = coh_buf(gptr<const float>(op.pro_add)), bc = coh_buf(b);
+    const uint32_t blk = wave * 4u + (lane >> 4);
+    if (blk < op.blocks) {
+        const uint32_t at0 = blk * 256u + 16u * (lane & 15u);
 #pragma unroll
-    for (int i = 0; i < 4; i++) {
-        const uint32_t unit = wave + PLAN_W * (uint32_t)i;
-        if (unit < B) {
-            const uint32_t at = unit * 256u + 4u * lane;
-            xs.x[i] = load4_either(coherent, x, xc, at);
-            if (pro == GEMV_PRO_ADD_RMSNORM) xs.t[i] = load4_either(coherent, add, ac, at);
-            if (pro == GEMV_PRO_SWIGLU) xs.b[i] = load4_either(coherent, b, bc, at);
-            else if (pro != GEMV_PRO_NONE) xs.b[i] = x_load4(b + at);        /* norm weights: constants */
+        for (int j = 0; j < 4; j++) xs.x[j] = cload4(xc, (at0 + 4u * (uint32_t)j) * 4u);
+        if (pro == GEMV_PRO_ADD_RMSNORM) {
+#pragma unroll
+            for (int j = 0; j < 4; j++) xs.t[j] = cload4(ac, (at0 + 4u * (uint32_t)j) * 4u);
+        }
+        if (pro == GEMV_PRO_SWIGLU) {
+#pragma unroll
+            for (int j = 0; j < 4; j++) xs.b[j] = cload4(bc, (at0 + 4u * (uint32_t)j) * 4u);
+        } else if (pro != GEMV_PRO_NONE) {
+#pragma unroll
+            for (int j = 0; j < 4; j++) xs.b[j] = x_load4(b + at0 + 4u * (uint32_t)j);      /* norm weights: constants */
         }
     }
 }
 
-/* One instantiation per staged layout: what the prologue does is decided at run time (the branches are
- * uniform and the float expressions are prologue_apply's), so that the quantiser is inlined twice, not
- * eight times. */
+__device__ __forceinline__ int quantize_sum4(const XRegs &y, float inv, uint32_t &packed)
+{
+    const int q0 = quantize_one(y.v0, inv), q1 = quantize_one(y.v1, inv);
+    const int q2 = quantize_one(y.v2, inv), q3 = quantize_one(y.v3, inv);
+    packed = (uint32_t)(q0 & 255) | ((uint32_t)(q1 & 255) << 8) | ((uint32_t)(q2 & 255) << 16) |
+             ((uint32_t)(q3 & 255) << 24);
+    return q0 + q1 + q2 + q3;
+}
+
 template <int KIND /* 0 Q4_K/Q5_K layout, 1 Q6_K layout */>
 __device__ __forceinline__ void
 plan_stage_finish(const OpHead &op, const XStage &xs, uint8_t *base, float *red, bool storer,
                   uint32_t lane, uint32_t wave)
 {
+    constexpr bool Q6 = KIND == 1;
     const uint32_t B = op.blocks, pro = op.pro;
     const bool rms = pro == GEMV_PRO_RMSNORM || pro == GEMV_PRO_ADD_RMSNORM, add = pro == GEMV_PRO_ADD_RMSNORM;
+    const uint32_t blk = wave * 4u + (lane >> 4), l = lane & 15u;
     XRegs xr[4];
 #pragma unroll
-    for (int i = 0; i < 4; i++) {
-        xr[i] = xs.x[i];
-        if (add) { xr[i].v0 += xs.t[i].v0; xr[i].v1 += xs.t[i].v1; xr[i].v2 += xs.t[i].v2; xr[i].v3 += xs.t[i].v3; }
+    for (int j = 0; j < 4; j++) {
+        xr[j] = xs.x[j];
+        if (add) { xr[j].v0 += xs.t[j].v0; xr[j].v1 += xs.t[j].v1; xr[j].v2 += xs.t[j].v2; xr[j].v3 += xs.t[j].v3; }
     }
     float inv = 1.0f;
     if (rms) {
-        float ss = 0.0f;
+        if (wave < PLAN_W / 4u) {
+            /* rows beyond the vector hold zeros, the sums of the launches' idle waves */
+            float p[4];
 #pragma unroll
-        for (int i = 0; i < 4; i++)
-            if (wave + PLAN_W * (uint32_t)i < B)
-                ss += xr[i].v0 * xr[i].v0 + xr[i].v1 * xr[i].v1 + xr[i].v2 * xr[i].v2 + xr[i].v3 * xr[i].v3;
-        ss = wave_sum_f32(ss);
-        if (lane == 0u) red[wave] = ss;
+            for (int j = 0; j < 4; j++)
+                p[j] = xr[j].v0 * xr[j].v0 + xr[j].v1 * xr[j].v1 + xr[j].v2 * xr[j].v2 + xr[j].v3 * xr[j].v3;
+            /* vectors of more than sixteen blocks: the further units of the wave this row stands for,
+             * one round trip each (their values are not kept: the rows that quantise them asked for
+             * them already) */
+            if (B > PLAN_W) {
+                const CohBuf xc = coh_buf(gptr<const float>(op.x)), ac = coh_buf(gptr<const float>(op.pro_add));
+                for (uint32_t b2 = blk + PLAN_W; b2 < B; b2 += PLAN_W) {
+#pragma unroll
+                    for (int j = 0; j < 4; j++) {
+                        const uint32_t at = b2 * 256u + 16u * l + 4u * (uint32_t)j;
+                        XRegs v = cload4(xc, at * 4u);
+                        if (add) {
+                            const XRegs t = cload4(ac, at * 4u);
+                            v.v0 += t.v0; v.v1 += t.v1; v.v2 += t.v2; v.v3 += t.v3;
+                        }
+                        p[j] += v.v0 * v.v0 + v.v1 * v.v1 + v.v2 * v.v2 + v.v3 * v.v3;
+                    }
+                }
+            }
+            float q = (p[0] + p[1]) + (p[2] + p[3]);
+            q += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(q), 0xB1, 0xF, 0xF, false));
+            q += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(q), 0x4E, 0xF, 0xF, false));
+            q += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(q), 0x141, 0xF, 0xF, false));
+            q += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(q), 0x140, 0xF, 0xF, false));
+            if (l == 0u) red[blk] = q;
+        }
         __syncthreads();
-        const float tot = wave_sum_f32(lane < PLAN_W ? red[lane] : 0.0f);
-        inv = 1.0f / sqrtf(tot / (float)(B * 256u) + op.eps);
+        if (wave * 4u < B) {
+            const float tot = wave_sum_f32(lane < PLAN_W ? red[lane] : 0.0f);
+            inv = 1.0f / sqrtf(tot / (float)(B * 256u) + op.eps);
+        }
     }
     const bool has_sout = add && storer && op.pro_sum_out != 0u;
     const bool has_fout = pro != GEMV_PRO_NONE && storer && op.pro_out != 0u;
-    const CohBuf sout = coh_buf(gptr<float>(op.pro_sum_out)), fout = coh_buf(gptr<float>(op.pro_out));
-    uint8_t *gout = (storer && op.act_out) ? gptr<uint8_t>(op.act_out) : nullptr;
+    if (blk < B) {
+        const CohBuf sout = coh_buf(gptr<float>(op.pro_sum_out)), fout = coh_buf(gptr<float>(op.pro_out));
+        const uint32_t at = blk * 256u + 16u * l;
+        XRegs y[4];
 #pragma unroll
-    for (int i = 0; i < 4; i++) {
-        const uint32_t unit = wave + PLAN_W * (uint32_t)i;
-        if (unit < B) {
-            const uint32_t at = unit * 256u + 4u * lane;
-            if (has_sout) cstore4(sout, at * 4u, xr[i]);
-            XRegs y = xr[i];
-            if (rms) y = prologue_apply<GEMV_PRO_RMSNORM>(xr[i], xs.b[i], inv);
-            else if (pro == GEMV_PRO_SWIGLU) y = prologue_apply<GEMV_PRO_SWIGLU>(xr[i], xs.b[i], inv);
-            if (has_fout) cstore4(fout, at * 4u, y);
-            q8k_x_finish<KIND == 1>(y, B, unit, base, gout, lane);
+        for (int j = 0; j < 4; j++) {
+            if (has_sout) cstore4(sout, (at + 4u * (uint32_t)j) * 4u, xr[j]);
+            y[j] = xr[j];
+            if (rms) y[j] = prologue_apply<GEMV_PRO_RMSNORM>(xr[j], xs.b[j], inv);
+            else if (pro == GEMV_PRO_SWIGLU) y[j] = prologue_apply<GEMV_PRO_SWIGLU>(xr[j], xs.b[j], inv);
+            if (has_fout) cstore4(fout, (at + 4u * (uint32_t)j) * 4u, y[j]);
+        }
+        float m = fmaxf(fmaxf(fabsf(y[0].v0), fabsf(y[0].v1)), fmaxf(fabsf(y[0].v2), fabsf(y[0].v3)));
+#pragma unroll
+        for (int j = 1; j < 4; j++)
+            m = fmaxf(m, fmaxf(fmaxf(fabsf(y[j].v0), fabsf(y[j].v1)), fmaxf(fabsf(y[j].v2), fabsf(y[j].v3))));
+        m = dpp_max_step(oct_max(m), 3);                /* over the row's sixteen lanes */
+        const float d = m / 127.0f;
+        const float invd = (d != 0.0f) ? 1.0f / d : 0.0f;
+        u32x4 packed;
+        uint32_t pk;
+        int s16 = quantize_sum4(y[0], invd, pk); packed.x = pk;
+        s16 += quantize_sum4(y[1], invd, pk); packed.y = pk;
+        s16 += quantize_sum4(y[2], invd, pk); packed.z = pk;
+        s16 += quantize_sum4(y[3], invd, pk); packed.w = pk;
+        /* value dwords 4l .. 4l+3 of a block are neighbours in both staged layouts */
+        *reinterpret_cast<u32x4 *>(reinterpret_cast<uint32_t *>(base) + q8k_slot<Q6>(B, blk, 4u * l)) = packed;
+        if (Q6) {
+            const uint32_t n = l >> 3, k = (l >> 1) & 3u, lh = l & 1u;
+            reinterpret_cast<int32_t *>(base + B * 256u)[(blk * 4u + 2u * n + lh) * 4u + k] = -32 * s16;
+        } else {
+            const int bj = s16 + __builtin_amdgcn_update_dpp(0, s16, 0xB1, 0xF, 0xF, false);
+            if ((l & 1u) == 0u) {
+                const uint32_t j = l >> 1;
+                reinterpret_cast<int16_t *>(base + B * 256u)[(blk * 4u + (j >> 1)) * 2u + (j & 1u)] = (int16_t)bj;
+            }
+        }
+        if (l == 0u) reinterpret_cast<float *>(base + B * 256u + B * (Q6 ? 64u : 16u))[blk] = d;
+        if (storer && op.act_out) {
+            uint8_t *dst = gptr<uint8_t>(op.act_out) + (size_t)blk * 292u;
+            uint32_t *qs = reinterpret_cast<uint32_t *>(dst + 4) + 4u * l;
+            qs[0] = packed.x; qs[1] = packed.y; qs[2] = packed.z; qs[3] = packed.w;
+            if (l == 0u) *reinterpret_cast<float *>(dst) = d;
+            reinterpret_cast<int16_t *>(dst + 260)[l] = (int16_t)s16;
         }
     }
-    /* what this workgroup stored for later operations has to be complete before it announces the
-     * operation done; the only loads in flight here are the first passes' weights, needed next anyway */
     if (has_sout || has_fout) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 }
 
@@ -637,19 +717,25 @@ k_plan(const PlanOp *__restrict__ ops, uint32_t n_ops, const PlanSync sy, const 
         for (int u = 0; u < 4; u++) xs.x[u] = xs.t[u] = xs.b[u] = XRegs{ 0.f, 0.f, 0.f, 0.f };
         if (op.wait == 0u) {
             /* nothing to wait for: the vector goes first and is there in a microsecond */
-            plan_stage_issue(op, xs, false, ln, wave);
+            plan_stage_issue(op, xs, ln, wave);
             plan_prefetch<HAS_Q5>(cur, A, 0u, ln);
         } else {
-            plan_prefetch<HAS_Q5>(cur, A, 0u, ln);
+            /* Wave 0 polls, and a poll comes back behind everything the wave asked for before it: its
+             * own weights go out after the wait (behind its part of the vector; they are there before
+             * the vector is quantised), the other waves' before it. */
+            if (wave != 0u) plan_prefetch<HAS_Q5>(cur, A, 0u, ln);
             if (!plan_wait(sy, base + op.wait, s_ok, ln, wave)) return;
-            plan_stage_issue(op, xs, true, ln, wave);
+            plan_stage_issue(op, xs, ln, wave);
+            if (wave == 0u) plan_prefetch<HAS_Q5>(cur, A, 0u, ln);
         }
         plan_stamp(sy, i, 1, ln, wave);
         /* what this wave owns of the next operation */
         PWork nx = cur;
         if (i + 1u < n_ops) nx = plan_work(&tab[i + 1u], wave);
 
-        const bool storer = blockIdx.x == 0u;
+        /* a prologue's side outputs are one workgroup's work, and not workgroup 0's: that one gathers the
+         * counters, and whatever holds it up holds everybody up */
+        const bool storer = blockIdx.x == gridDim.x - 1u;
         const uint32_t Bk = op.blocks;
         if (sy.stamps != nullptr) {         /* measurement only: when has the vector arrived? */
             asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -737,7 +823,7 @@ k_plan_ext(const PlanOp *__restrict__ ins, uint32_t n_ins, const PlanOp *__restr
         XStage xs;
 #pragma unroll
         for (int u = 0; u < 4; u++) xs.x[u] = xs.t[u] = xs.b[u] = XRegs{ 0.f, 0.f, 0.f, 0.f };
-        plan_stage_issue(op, xs, false, lane, wave);
+        plan_stage_issue(op, xs, lane, wave);
         if (op.kind >= PLAN_Q6_K) plan_stage_finish<1>(op, xs, lds, red, true, lane, wave);
         else                      plan_stage_finish<0>(op, xs, lds, red, true, lane, wave);
         __syncthreads();
