@@ -267,6 +267,25 @@ def secondary_figures(mv, synth):
     out["q2k_q3k_prefill_14336x4096x512"] = pre
     for b_ in (d_x, d_a, d_o, d_wide):
         b_.free()
+    # the 32-value formats, 512 activations: 128 x 64 tiles, one 16x16x32 MFMA per block and token chunk
+    rows, cols, nv = 4096, 4096, 512
+    d_x = mv.DeviceBuffer.from_host(synth.normal(nv * cols, seed=0, stream=2009))
+    d_a = mv.DeviceBuffer(nv * mv.act_bytes(Q80, cols))
+    d_o = mv.DeviceBuffer(nv * rows * 4)
+    mv.quantize(Q80, d_x.ptr, cols, nv, cols, d_a.ptr)
+    pre32 = {}
+    for name, qt in (("q8_0", Q80), ("q4_0", 3), ("q5_1", 6)):
+        d_w = mv.DeviceBuffer.from_host(synth.weights(qt, rows, cols, seed=0, stream=2010 + qt))
+        us = timed(lambda: mv.mmq(qt, d_w.ptr, rows, cols, d_a.ptr, nv, d_o.ptr, rows), 20, mv)
+        ops = 2.0 * rows * cols * nv
+        pre32[name] = {"mfma_kernel_only_us": round(us, 2), "tops": round(ops / us / 1e6, 1),
+                       "frac_of_int8_peak": round(ops / us / 1e6 / INT8_PEAK_TOPS, 4)}
+        d_w.free()
+    pre32["note"] = ("exact per-block float step: four vector operations per output and 32-value block beside one "
+                     "16x16x32 MFMA per 256 outputs")
+    out["q8_0_family_prefill_4096x4096x512"] = pre32
+    for b_ in (d_x, d_a, d_o):
+        b_.free()
     # configuration 0 (the reference's own CPU-runnable case): one 4096 x 4096 Q4_K matvec, over 32 distinct
     # copies in turn (302 MB: from HBM) and over one copy again and again (resident in the last-level cache)
     rows, cols = 4096, 4096

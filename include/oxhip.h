@@ -292,7 +292,15 @@ int oxh_plan_deal(const size_t *rows, const int *paired, size_t n_segs, uint32_t
  * Replaces the prepared-row batch kernels oc_oxk_q4_k_prep_row (and
  * oc_oxk_q5_k_prep_row, oc_oxk_q6_k_prep_row) + oc_oxk_dot_q4_k_prepped_multi
  * (oxidize-c/src/compute/oxk.c:316-366, :372-373, :787-836) driven by
- * matvec_batch_prep_slice (matvec.c:1198-1228). */
+ * matvec_batch_prep_slice (matvec.c:1198-1228).
+ *
+ * The 32-value formats (Q8_0, Q4_0, Q4_1, Q5_0, Q5_1, AL5_XS and the ids that
+ * share their layouts) are taken too, against Q8_0 activations: tiles of 128
+ * rows x 64 activations, a 16x16x32 MFMA per block and 16-token chunk, the
+ * per-block float step and the block-sequential sum of oxk.c:88-241, so every
+ * output is the single-vector dot bit for bit and the matrix is streamed once
+ * per 64 activations (the reference walks such a batch four activations at a
+ * time, matvec.c:1263-1488).  Rows must be at least 16 bytes long. */
 int oxh_mmq(uint32_t qtype, const void *d_w, size_t rows, size_t cols,
             const void *d_acts, size_t n_vec, float *d_out, size_t out_stride,
             void *stream);
@@ -318,8 +326,9 @@ int oxh_mmq_ex(uint32_t qtype, const void *d_w, size_t rows, size_t cols,
 /* The tile (weight rows x activations per workgroup) oxh_mmq picks for a launch
  * on a device of n_cu compute units: the largest of 256 x 128 (128 x 128 for
  * Q5_K, Q6_K and widened Q2_K), 64 x 128 (Q6_K only), 128 x 64, 64 x 32, 64 x 16
- * that still gives nearly every compute unit a workgroup.  Pure host arithmetic
- * (no device needed); OXH_DECLINED for a type without a matrix-core kernel.
+ * that still gives nearly every compute unit a workgroup; 128 x 64 always for
+ * the 32-value formats.  Pure host arithmetic (no device needed); OXH_DECLINED
+ * for a type without a matrix-core kernel.
  * The reference has no counterpart: its batch kernel takes four activations
  * per weight row regardless of the shape (oxk.c:787-836). */
 int oxh_mmq_tile(uint32_t qtype, size_t rows, size_t n_vec, size_t n_cu, uint32_t *tile_rows,

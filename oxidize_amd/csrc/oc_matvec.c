@@ -893,22 +893,29 @@ static int mv_batch(uint32_t qtype, const uint8_t *data, size_t rows,
             if ((rc = oxh_gemv_segments_f32(qtype, &seg, 1, cols, d_x, cols, g_dact.p, n_vec, rows, NULL)))
                 return rc;
         } else {
-            /* every activation is quantised once, then the slices run over the stored bytes */
+            /* every activation is quantised once; the 32-value formats then have a token-tiled kernel on
+             * the matrix cores (the matrix is streamed once per 64 activations), the rest walk the batch in
+             * slices over the stored bytes */
             if ((rc = quantize(kind, d_x, cols, n_vec, cols, g_dact.p))) return rc;
-            /* up to 32 slices per launch, each slice a segment over the same matrix with its own run of
-             * activations and its own place in the output: 512 vectors of a 32-value format are one or
-             * two launches instead of 32 or 64, and slices overlap instead of queueing behind launch gaps */
-            enum { SLICES = 32 };
-            OxhSegment segs[SLICES];
-            size_t v0 = 0;
-            while (v0 < n_vec) {
-                size_t n = 0;
-                for (; n < SLICES && v0 < n_vec; n++, v0 += step) {
-                    const size_t m = n_vec - v0 < step ? n_vec - v0 : step;
-                    const OxhSegment seg = { d_w, (float *)g_dout.p + v0 * rows, rows, v0, m, NULL };
-                    segs[n] = seg;
+            rc = kind == 1 ? oxh_mmq(qtype, d_w, rows, cols, g_dact.p, n_vec, (float *)g_dout.p, rows, NULL)
+                           : OXH_DECLINED;
+            if (rc != OXH_OK && rc != OXH_DECLINED) return rc;
+            if (rc == OXH_DECLINED) {
+                /* up to 32 slices per launch, each slice a segment over the same matrix with its own run of
+                 * activations and its own place in the output: slices overlap instead of queueing behind
+                 * launch gaps */
+                enum { SLICES = 32 };
+                OxhSegment segs[SLICES];
+                size_t v0 = 0;
+                while (v0 < n_vec) {
+                    size_t n = 0;
+                    for (; n < SLICES && v0 < n_vec; n++, v0 += step) {
+                        const size_t m = n_vec - v0 < step ? n_vec - v0 : step;
+                        const OxhSegment seg = { d_w, (float *)g_dout.p + v0 * rows, rows, v0, m, NULL };
+                        segs[n] = seg;
+                    }
+                    if ((rc = oxh_gemv_segments(qtype, segs, n, cols, g_dact.p, step, rows, NULL))) return rc;
                 }
-                if ((rc = oxh_gemv_segments(qtype, segs, n, cols, g_dact.p, step, rows, NULL))) return rc;
             }
         }
     }

@@ -757,6 +757,12 @@ static hipError_t raise_all_lds_ceilings(void)
     if ((e = raise_lds_ceiling(k_mfma_q8_0_segments<4, 3>)) != hipSuccess) return e;
     if ((e = raise_lds_ceiling(k_mfma_q8_0_segments<4, 4>)) != hipSuccess) return e;
     if ((e = raise_lds_ceiling(k_mfma_q8_0_segments<4, 5>)) != hipSuccess) return e;
+    if ((e = raise_lds_ceiling(k_mmq_q80<0>)) != hipSuccess) return e;
+    if ((e = raise_lds_ceiling(k_mmq_q80<1>)) != hipSuccess) return e;
+    if ((e = raise_lds_ceiling(k_mmq_q80<2>)) != hipSuccess) return e;
+    if ((e = raise_lds_ceiling(k_mmq_q80<3>)) != hipSuccess) return e;
+    if ((e = raise_lds_ceiling(k_mmq_q80<4>)) != hipSuccess) return e;
+    if ((e = raise_lds_ceiling(k_mmq_q80<5>)) != hipSuccess) return e;
     if ((e = raise_lds_ceiling(k_mmq_q6_k_segments<1, 1, 4, 2>)) != hipSuccess) return e;
     if ((e = raise_lds_ceiling(k_mmq_q6_k_experts<1, 1, 4, 2>)) != hipSuccess) return e;
     if ((e = raise_lds_ceiling(k_mmq_q4_k_segments<1, 1, 8, 3>)) != hipSuccess) return e;
@@ -1415,9 +1421,28 @@ static int mmq_tile_shape(uint32_t qtype, size_t rows, size_t n_vec, size_t cus)
     return 3;
 }
 
+/* the 32-value formats with a matrix-core kernel, as its LEG parameter; -1 for everything else */
+static int mmq80_leg(uint32_t qtype)
+{
+    switch (qtype) {
+    case OXH_Q8_0:   return 0;
+    case OXH_Q4_0:   return 1;
+    case OXH_Q4_1:   return 2;
+    case OXH_Q5_0:   return 3;
+    case OXH_Q5_1:   return 4;
+    case OXH_AL5_XS: return 5;
+    default:         return -1;
+    }
+}
+
 extern "C" int oxh_mmq_tile(uint32_t qtype, size_t rows, size_t n_vec, size_t n_cu, uint32_t *tile_rows,
                             uint32_t *tile_tokens)
 {
+    if (mmq80_leg(canon_qtype(qtype)) >= 0 && rows && n_vec && n_cu) {       /* one tile for these */
+        if (tile_rows) *tile_rows = MQT_WAVES * 16u;
+        if (tile_tokens) *tile_tokens = MQT_TOK;
+        return OXH_OK;
+    }
     const bool one_chunk = qtype == OXH_Q6_K || is_q5k(qtype) || qtype == OXH_Q2_K_WIDE;
     if ((!is_q4k(qtype) && !one_chunk) || rows == 0 || n_vec == 0 || n_cu == 0) return OXH_DECLINED;
     static const uint32_t tr[6] = { 0, 256, 128, 64, 64, 64 }, tt[6] = { 0, 128, 64, 32, 16, 128 };
@@ -1452,6 +1477,38 @@ static int mmq_run(uint32_t qtype, const void *d_w, size_t rows, size_t cols, co
     if (rc) return rc;
     if (rows == 0 || n_vec == 0) return OXH_OK;
     if (!d_w || !d_acts || !d_out) return arg_fail("oxh_mmq: NULL pointer");
+    const int leg = mmq80_leg(canon_qtype(qtype));
+    if (leg >= 0 && oxh_act_kind(qtype, cols) == 1) {
+        /* 32-value blocks against Q8_0 activations: one tile shape, exact f32 step only */
+        if (out_stride < rows) return arg_fail("oxh_mmq: out_stride < rows");
+        const size_t blocks32 = cols / OXH_QK8_0;
+        if (rows > 0x7FFFFFFFull || n_vec > 0x7FFFFFFFull || blocks32 > 0xFFFFFFull)
+            return arg_fail("oxh_mmq: dimension too large");
+        if (blocks32 * block_bytes(qtype) < 16u) {
+            snprintf(g_err, sizeof g_err, "oxh_mmq: rows of qtype %u with cols %zu are shorter than 16 bytes", qtype, cols);
+            return OXH_DECLINED;
+        }
+        const uint32_t n_rt = (uint32_t)((rows + MQT_WAVES * 16u - 1u) / (MQT_WAVES * 16u));
+        const uint32_t n_tt = (uint32_t)((n_vec + MQT_TOK - 1u) / MQT_TOK);
+        const uint64_t wgs = (uint64_t)((n_rt + 7u) / 8u) * 8u * n_tt;
+        if (wgs > 0x7FFFFFFFull) return arg_fail("oxh_mmq: too many tiles");
+        hipStream_t st = pick_stream(stream);
+#define OXH_MQT(LEG) hipLaunchKernelGGL((k_mmq_q80<LEG>), dim3((uint32_t)wgs), dim3(MQT_WAVES * 64u),          \
+                                        MqtGeom<LEG>::LDS_BYTES, st, (const uint8_t *)d_w, (uint32_t)rows,     \
+                                        (uint32_t)blocks32, (const uint8_t *)d_acts, (uint32_t)n_vec, d_out,   \
+                                        out_stride, n_rt, n_tt)
+        switch (leg) {
+        case 1:  OXH_MQT(1); break;
+        case 2:  OXH_MQT(2); break;
+        case 3:  OXH_MQT(3); break;
+        case 4:  OXH_MQT(4); break;
+        case 5:  OXH_MQT(5); break;
+        default: OXH_MQT(0); break;
+        }
+#undef OXH_MQT
+        HIP_TRY(hipGetLastError());
+        return OXH_OK;
+    }
     const bool wide2 = qtype == OXH_Q2_K_WIDE;
     if ((!is_q4k(qtype) && !is_q5k(qtype) && qtype != OXH_Q6_K && !wide2) ||
         oxh_act_kind(wide2 ? OXH_Q2_K : qtype, cols) != 2) {

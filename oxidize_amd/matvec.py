@@ -186,6 +186,13 @@ def mmq(qtype, d_w, rows, cols, d_acts, n_vec, d_out, out_stride, stream=None, f
                         n_vec, ctypes.c_void_p(d_out), out_stride, stream))
 
 
+def mmq_tile(qtype, rows, n_vec, n_cu):
+    """(rows, tokens) of the workgroup tile oxh_mmq would take; host arithmetic only."""
+    r, t = ctypes.c_uint32(0), ctypes.c_uint32(0)
+    check(lib().oxh_mmq_tile(qtype, rows, n_vec, n_cu, ctypes.byref(r), ctypes.byref(t)))
+    return r.value, t.value
+
+
 def get_rows(qtype, d_w, rows, cols, d_ids, n_ids, d_out, out_stride, stream=None):
     check(lib().oxh_get_rows(qtype, ctypes.c_void_p(d_w), rows, cols, ctypes.c_void_p(d_ids), n_ids,
                              ctypes.c_void_p(d_out), out_stride, stream))

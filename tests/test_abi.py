@@ -256,6 +256,9 @@ def test_mmq_tile_choice_is_host_arithmetic():
             for n_vec in (1, 16, 17, 32, 33, 64, 100, 128, 129, 512, 2048):
                 for n_cu in (64, 256, 304):
                     assert tile(qtype, rows, n_vec, n_cu) == (0,) + rule(qtype, rows, n_vec, n_cu)
-    assert tile(Q80, 4096, 512)[0] == _lib.DECLINED
+    # the 32-value formats have one tile; the codebook formats have no matrix-core kernel
+    for qtype in (Q80, 3, 4, 5, 6, 17, 18, 19, 20):
+        assert tile(qtype, 4096, 512) == (0, 128, 64)
+    assert tile(25, 4096, 512)[0] == _lib.DECLINED
     assert tile(Q4K, 0, 512)[0] == _lib.DECLINED
     assert lib.oxh_mmq_tile(Q4K, 4096, 512, 256, None, None) == 0

@@ -455,3 +455,38 @@ def test_long_batches_of_types_without_a_tile_kernel(oxh, qtype, cols, n_vec):
     for v in list(range(0, n_vec, 37)) + [n_vec - 1]:
         want, _ = oracle_matvec(qtype, w, rows, cols, np.ascontiguousarray(xs[v, :cols]))
         assert np.array_equal(bits(outs[v, :rows]), bits(want)), v
+
+
+@pytest.mark.parametrize("qtype,rows,cols,n_vec", [
+    (Q80, 70, 896, 600),        # 28 blocks: a full step and a short one; ragged row and token tiles
+    (Q80, 130, 4096, 65),       # a second row tile of two rows, a second token tile of one token
+    (Q80, 16, 32, 64),          # one block per row
+    (3, 257, 1024, 64),         # Q4_0
+    (4, 128, 544, 100),         # Q4_1, 17 blocks: the last step is a single block
+    (5, 17, 992, 33),           # Q5_0, 31 blocks: an odd last step
+    (6, 300, 2048, 129),        # Q5_1
+    (18, 129, 1056, 70),        # AL5_XS, 33 blocks of 14 bytes: a last step shorter than one 16-byte piece
+    (20, 64, 512, 17),          # AL8: the Q8_0 layout under its own id
+])
+def test_token_tiled_kernel_of_the_32_value_formats(oxh, qtype, rows, cols, n_vec):
+    """oxh_mmq over the 32-value formats (128 rows x 64 tokens per workgroup, activations staged sixteen
+    blocks at a time): every output is the single-vector dot, bit for bit, and nothing outside the
+    rows x n_vec outputs is written."""
+    canon = {17: 3, 19: 5, 20: 7}.get(qtype, qtype)
+    w = synth.weights(canon, rows, cols, seed=83, stream=rows + cols)
+    xs = synth.normal(n_vec * cols, seed=83, stream=n_vec).reshape(n_vec, cols)
+    xs[n_vec // 2, :64] = 0.0
+    d_w = mv.DeviceBuffer.from_host(w)
+    d_x = mv.DeviceBuffer.from_host(xs)
+    d_a = mv.DeviceBuffer(n_vec * mv.act_bytes(qtype, cols))
+    mv.quantize(qtype, d_x.ptr, cols, n_vec, cols, d_a.ptr)
+    stride = rows + 3
+    d_out = mv.DeviceBuffer.from_host(np.full((n_vec, stride), -7.25, np.float32))
+    assert mv.mmq_tile(qtype, rows, n_vec, 256) == (128, 64)
+    mv.mmq(qtype, d_w.ptr, rows, cols, d_a.ptr, n_vec, d_out.ptr, stride)
+    mv.sync()
+    outs = d_out.download(np.float32, n_vec * stride).reshape(n_vec, stride)
+    assert np.all(outs[:, rows:] == -7.25)
+    for v in sorted(set(list(range(0, n_vec, 13)) + [n_vec // 2, 63 % n_vec, 64 % n_vec, n_vec - 1])):
+        want, _ = oracle_matvec(canon, w, rows, cols, np.ascontiguousarray(xs[v]))
+        assert np.array_equal(bits(outs[v, :rows]), bits(want)), v
