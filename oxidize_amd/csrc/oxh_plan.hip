@@ -20,8 +20,8 @@
  *     operation boundary.
  *   - An operation that reads what an earlier one wrote waits until every
  *     workgroup has finished that one.  Workgroups announce progress with one
- *     monotonic counter each; workgroup 0 gathers them and publishes the
- *     minimum.  The eight L2 caches of the device are not coherent with each
+ *     monotonic counter each, stored in eight copies; every workgroup reads
+ *     all counters of one copy (plan_wait).  The eight L2 caches of the device are not coherent with each
  *     other and a fence that makes them so costs 35 us here, so there are no
  *     fences: everything one operation hands to another (outputs, residual
  *     sums) is stored and loaded with system-coherent accesses that bypass the
@@ -97,11 +97,12 @@ struct PlanOp {
 
 static_assert(sizeof(PlanOp) % 16 == 0, "table rows are copied in 16-byte pieces");
 
-/* progress counters: flags[wg], then go[0] = the published minimum, go[1] = error word */
+/* progress counters: flags[copy][wg], then go[0] = the minimum workgroup 0 publishes (copies = 0), go[1] = error word */
 struct PlanSync {
     uint32_t *flags;
     uint32_t *go;
     uint32_t n_wait;                /* counters gathered: the grid size (one more in the time-out test) */
+    uint32_t copies;                /* copies of every counter that every workgroup gathers from, or 0: workgroup 0 gathers */
     uint32_t spin_limit;
     uint64_t *stamps;               /* measurement aid: [op][workgroup][8] clock readings, or NULL */
 };
@@ -600,16 +601,39 @@ plan_stage_finish(const OpHead &op, const XStage &xs, uint8_t *base, float *red,
 /* Counters only grow (modulo 2^32): "reached" is a signed difference. */
 __device__ __forceinline__ bool reached(uint32_t v, uint32_t target) { return (int32_t)(v - target) >= 0; }
 
+/* Two ways to learn that every workgroup has announced `target`:
+ *
+ * copies = 0: workgroup 0 gathers the counters and stores their minimum, the others poll that word.  A
+ * store then makes four trips through the fabric before everybody has seen it (the store, workgroup
+ * 0's poll, its store of the minimum, the others' poll), but a waiting workgroup reads one line.  The
+ * pre-staging kernel's single wait is of this kind: half the workgroups have nothing to stage and poll
+ * for microseconds while the others work (with everybody gathering, a decode step took 0.745 ms
+ * against 0.732 ms).
+ *
+ * copies = n: every counter exists n times, 4 KiB apart, a workgroup announces by storing all copies
+ * (lanes 0..n-1 of one store instruction) and every workgroup gathers for itself, from copy
+ * (workgroup % n): two trips instead of four.  With one copy the 256 pollers of the same sixteen lines
+ * are slower than the four trips (32-layer chain 1.47 ms against 1.41 ms); with eight, 32 workgroups
+ * share a copy: 1.37 ms (4: 1.38, 16: 1.38, 32: 1.39, 64: 1.40).  The chained kernel's waits are of
+ * this kind (OXH_PLAN_COPIES, 0 = the first way). */
+#define PLAN_COPIES 64u             /* room for */
+
+__device__ __forceinline__ void plan_announce(const PlanSync &sy, uint32_t value, uint32_t lane)
+{
+    if (lane < max(sy.copies, 1u)) cstore(sy.flags + lane * PLAN_MAX_WG + blockIdx.x, value);
+}
+
 __device__ __forceinline__ bool
 plan_wait(const PlanSync &sy, uint32_t target, int *s_ok, uint32_t lane, uint32_t wave)
 {
     if (wave == 0u) {
         bool ok = true;
         uint32_t spins = 0;
-        if (blockIdx.x == 0u) {
+        if (sy.copies != 0u || blockIdx.x == 0u) {
+            const CohBuf fb = coh_buf(sy.flags + (sy.copies ? blockIdx.x % sy.copies : 0u) * PLAN_MAX_WG);
             for (;;) {
                 bool mine = true;
-                const CohBuf fb = coh_buf(sy.flags);
+                const uint32_t err = cload(sy.go + 1);
                 for (uint32_t k = 4u * lane; k < sy.n_wait; k += 256u) {
                     const u32x4 f = cload16(fb, k * 4u);
                     mine = mine && reached(f.x, target) && (k + 1u >= sy.n_wait || reached(f.y, target)) &&
@@ -617,11 +641,11 @@ plan_wait(const PlanSync &sy, uint32_t target, int *s_ok, uint32_t lane, uint32_
                            (k + 3u >= sy.n_wait || reached(f.w, target));
                 }
                 if (__all(mine)) break;
-                if (++spins > sy.spin_limit || cload(sy.go + 1) != 0u) { ok = false; break; }
+                if (++spins > sy.spin_limit || err != 0u) { ok = false; break; }
             }
             if (lane == 0u) {
-                if (ok) cstore(sy.go, target);
-                else cstore(sy.go + 1, 1u);
+                if (!ok) cstore(sy.go + 1, 1u);
+                else if (sy.copies == 0u) cstore(sy.go, target);
             }
         } else {
             const CohBuf gb = coh_buf(sy.go);
@@ -693,7 +717,7 @@ k_plan(const PlanOp *__restrict__ ops, uint32_t n_ops, const PlanSync sy, const 
                 if (po.signal != 0u || i == n_ops) {
                     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
                     /* the last operation leaves every counter at base + n_ops + 1, the next launch's base */
-                    if (ln == 0u) cstore(sy.flags + blockIdx.x, base + i + (i == n_ops ? 1u : 0u));
+                    plan_announce(sy, base + i + (i == n_ops ? 1u : 0u), ln);
                 }
             }
             plan_stamp(sy, i - 1u, 7, ln, wave);
@@ -836,7 +860,7 @@ k_plan_ext(const PlanOp *__restrict__ ins, uint32_t n_ins, const PlanOp *__restr
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
-    if (threadIdx.x == 0u) cstore(sy.flags + blockIdx.x, base + 1u);
+    if (threadIdx.x < 64u) plan_announce(sy, base + 1u, threadIdx.x);
 
     /* One trip = requests for operation i, the workgroup barrier, rows and outputs of operation i - 1
      * (summed from the workgroup's term table by the first wg_rows threads while the other waves go
@@ -915,14 +939,14 @@ k_plan_ext(const PlanOp *__restrict__ ins, uint32_t n_ins, const PlanOp *__restr
     }
     /* the next launch's base */
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    if (threadIdx.x == 0u) cstore(sy.flags + blockIdx.x, base + 2u);
+    if (threadIdx.x < 64u) plan_announce(sy, base + 2u, threadIdx.x);
 }
 
 /* ─── host side ───────────────────────────────────────────────────────── */
 
 struct OxhPlan {
     PlanOp *d_ops;
-    uint32_t *d_sync;               /* PLAN_MAX_WG + 4 counters, then go[4] */
+    uint32_t *d_sync;               /* PLAN_COPIES x PLAN_MAX_WG counters, 4 spare words, then go[4] (go[1]: error word) */
     uint32_t n_ops, grid;
     PlanLds ld;
     size_t lds_bytes;
@@ -1263,10 +1287,10 @@ extern "C" int oxh_plan_create(const OxhPlanOp *ops, size_t n_ops, OxhPlan **out
     for (size_t i = 0; i < n_ops; i++) h[i].xq = pl->ext ? (gaddr)(uintptr_t)pl->d_img + h[i].xq : 0u;
     for (size_t i = 0; run && i < n_run; i++)
         for (uint32_t k = 0; k < run[i].n_segs; k++) run[i].s[k].xq += (gaddr)(uintptr_t)pl->d_img;
-    if (e == hipSuccess) e = hipMalloc((void **)&pl->d_sync, (PLAN_MAX_WG + 8u) * sizeof(uint32_t));
+    if (e == hipSuccess) e = hipMalloc((void **)&pl->d_sync, (PLAN_COPIES * PLAN_MAX_WG + 8u) * sizeof(uint32_t));
     if (e == hipSuccess) e = hipMemcpy(pl->d_ops, h, n_ops * sizeof(PlanOp), hipMemcpyHostToDevice);
     if (e == hipSuccess && pl->ext) e = hipMemcpy(pl->d_run, run, n_run * sizeof(PlanOp), hipMemcpyHostToDevice);
-    if (e == hipSuccess) e = hipMemset(pl->d_sync, 0, (PLAN_MAX_WG + 8u) * sizeof(uint32_t));
+    if (e == hipSuccess) e = hipMemset(pl->d_sync, 0, (PLAN_COPIES * PLAN_MAX_WG + 8u) * sizeof(uint32_t));
     if (e == hipSuccess) e = hipDeviceSynchronize();
     free(h);
     free(run);
@@ -1288,8 +1312,17 @@ extern "C" int oxh_plan_launch(OxhPlan *pl, void *stream)
     hipStream_t st = stream ? (hipStream_t)stream : (hipStream_t)oxh_internal_stream();
     PlanSync sy;
     sy.flags = pl->d_sync;
-    sy.go = pl->d_sync + PLAN_MAX_WG + 4u;
+    sy.go = pl->d_sync + PLAN_COPIES * PLAN_MAX_WG + 4u;
     sy.n_wait = pl->grid + pl->phantom;
+    {
+        static int copies = -1;
+        if (copies < 0) {
+            const char *pc = getenv("OXH_PLAN_COPIES");
+            const unsigned long v = pc && *pc ? strtoul(pc, nullptr, 10) : 8ul;
+            copies = v > PLAN_COPIES ? (int)PLAN_COPIES : (int)v;
+        }
+        sy.copies = pl->ext ? 0u : (uint32_t)copies;
+    }
     sy.spin_limit = pl->spin_limit;
     sy.stamps = pl->d_stamps;
 #define PLAN_LAUNCH(K)                                                                                  \
@@ -1347,10 +1380,10 @@ extern "C" int oxh_plan_status(OxhPlan *pl, void *stream)
     hipStream_t st = stream ? (hipStream_t)stream : (hipStream_t)oxh_internal_stream();
     PLAN_TRY(hipStreamSynchronize(st));
     uint32_t go[4] = { 0, 0, 0, 0 };
-    PLAN_TRY(hipMemcpy(go, pl->d_sync + PLAN_MAX_WG + 4u, sizeof go, hipMemcpyDeviceToHost));
+    PLAN_TRY(hipMemcpy(go, pl->d_sync + PLAN_COPIES * PLAN_MAX_WG + 4u, sizeof go, hipMemcpyDeviceToHost));
     if (go[1] == 0u) return OXH_OK;
     /* a wait ran out: the counters are no longer equal, start them afresh */
-    PLAN_TRY(hipMemset(pl->d_sync, 0, (PLAN_MAX_WG + 8u) * sizeof(uint32_t)));
+    PLAN_TRY(hipMemset(pl->d_sync, 0, (PLAN_COPIES * PLAN_MAX_WG + 8u) * sizeof(uint32_t)));
     PLAN_TRY(hipDeviceSynchronize());
     return oxh_internal_errorf(OXH_ERR_TIMEOUT, "plan: a wait between operations ran out of polls (not every workgroup "
                                "was resident, or the limit is too small); the launch's outputs are incomplete");
