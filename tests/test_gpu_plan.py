@@ -74,7 +74,7 @@ def chain_state(c):
                 res=[r.download(np.float32, d.hidden) for r in c.res])
 
 
-@pytest.mark.parametrize("hidden,kv,ffn,layers", [(1024, 256, 2816, 4), (4096, 1024, 14336, 3)])
+@pytest.mark.parametrize("hidden,kv,ffn,layers", [(1024, 256, 2816, 4), (4096, 1024, 14336, 3), (5120, 1024, 8192, 2), (16384, 1024, 2048, 2)])
 def test_dependent_chain_matches_single_launches(oxh, hidden, kv, ffn, layers):
     d = DecodeSet(hidden=hidden, kv=kv, ffn=ffn, layers=layers, seed=5)
     a, b = DecodeChain(d, seed=5), DecodeChain(d, seed=5)
@@ -131,12 +131,15 @@ def test_mixed_types_with_q5k(oxh):
         assert np.array_equal(bits(outs[i].download(np.float32, rows)), bits(want)), qt
 
 
-def test_prestaged_plan_follows_its_inputs_from_launch_to_launch(oxh, monkeypatch):
+@pytest.mark.parametrize("hidden,ffn", [(1024, 3072), (5120, 8192), (16384, 4096)])
+def test_prestaged_plan_follows_its_inputs_from_launch_to_launch(oxh, monkeypatch, hidden, ffn):
     """A plan of independent operations keeps every staged input in memory of its own and re-reads it in
     every workgroup: new input values before a launch must reach every output of that launch (nothing
     may come from a cache line or an image of the launch before), with and without prologues, and the
-    chained kernel must give the same bits for the same plan."""
-    hidden, ffn, eps = 1024, 3072, 1e-5
+    chained kernel must give the same bits for the same plan.  The longer vectors have more than
+    sixteen blocks: a normalising prologue then sums squares over several blocks per lane, in the
+    launches' order."""
+    eps = 1e-5
     shapes = [(Q4K, 1800, hidden, None), (Q6K, 1024, ffn, None), (Q4K, 2 * 1536, hidden, "rms"),
               (Q5K, 640, hidden, "add_rms"), (Q6K, 512, hidden, "swiglu"), (Q4K, 777, hidden, None)]
     bufs, ops = [], []
