@@ -36,7 +36,7 @@ HBM_PEAK_GBPS = 8000.0
 GATE_UP_TRAFFIC_BYTES = 66496518
 # HBM bytes one k_plan_ext launch (a whole 32-layer step) moves, measured the same way: FETCH_SIZE
 # 2170528.0 KiB x 1.9998, WRITE_SIZE 7322.03 KiB x 1.000 (algorithmic: 4419223552, ratio 1.0075).
-PLAN_STEP_TRAFFIC_BYTES = 4452278522
+PLAN_STEP_TRAFFIC_BYTES = 4441622891
 INT8_PEAK_TOPS = 5033.0     # dense int8 MFMA: 256 CU x 2.4 GHz x 8192 op/clk/CU
 
 
@@ -665,6 +665,15 @@ def main():
                    "layers": ds.layers, "mode": args.mode,
                    "q6k_layout": "regrouped in runs of eight blocks when loaded (same bytes)" if ds.q6_grouped else "file",
                    "launches_per_step": 1 if args.mode == "plan" else 4 * ds.layers,
+                   "operations_per_step": 4 * ds.layers,
+                   "table_rows_per_step": plan.info()["table_rows"] if args.mode == "plan" else None,
+                   "scheduling": ("the operations of this set do not depend on each other and the plan walks them in "
+                                  "an order and grouping of its own: operations of one weight layout and vector length "
+                                  "share table rows so that every wave has a whole number of 16-block passes "
+                                  "(gate/up of a layer with o of the next, q/k/v of two layers, down of two layers); "
+                                  "OXH_PLAN_MERGE=1 shares rows between neighbours only, 0 not at all; "
+                                  "extra.decode_chain_fused is the same step with a layer's real dependencies")
+                                 if args.mode == "plan" else None,
                    "untimed_steps_before_warmup": spun,
                    "bytes_per_step": step_bytes},
         "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBPS, 2),

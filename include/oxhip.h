@@ -235,13 +235,17 @@ int oxh_gemv_segments_fused(uint32_t qtype, const OxhSegment *segs, size_t n_seg
  * vector is normalised and quantised once, by one workgroup, into device
  * memory the plan owns (about 1.3 bytes per input value), all workgroups meet
  * once, and from then on an operation's quantised input is copied into LDS
- * while the previous operation runs.  Consecutive operations of such a plan
- * that read one weight layout over vectors of one length and are short (at
- * most three passes per wave together: q/k/v and o of a layer) are walked as
- * one operation with several inputs.  Same results; oxh_plan_prestaged says
- * whether a plan runs this way (OXH_PLAN_PRESTAGE=0 in the environment at
- * creation keeps such a plan on the chained kernel, OXH_PLAN_MERGE=0 keeps
- * every operation on its own).
+ * while the previous operation runs.  The operations of such a plan may run
+ * in any order and grouping: those that read one weight layout over vectors
+ * of one length are walked as one table row with several inputs while the row
+ * stays within eight segments and eight passes per wave (q/k/v and o of two
+ * layers: five rows per wave where one layer's are 2.5, i.e. three passes for
+ * half the waves and two for the rest; the down projections of two layers).
+ * Same results; oxh_plan_prestaged says whether a plan runs this way and
+ * oxh_plan_table_rows how many rows it walks (at creation, in the
+ * environment: OXH_PLAN_PRESTAGE=0 keeps such a plan on the chained kernel,
+ * OXH_PLAN_MERGE=0 keeps every operation on its own, OXH_PLAN_MERGE=1 merges
+ * neighbours only, within four segments and three passes per wave).
  *
  * All workgroups must be resident together (one per compute unit; the kernel
  * needs the whole device, so do not run other kernels beside a plan launch).
@@ -270,6 +274,9 @@ int oxh_plan_status(OxhPlan *plan, void *stream);
 int oxh_plan_info(const OxhPlan *plan, size_t *n_ops, size_t *n_waits, size_t *workgroups, size_t *lds_bytes);
 /* 1 when the plan stages its inputs ahead of the chain (see above), else 0. */
 int oxh_plan_prestaged(const OxhPlan *plan);
+/* Rows of the table a launch walks: the operations, or fewer where independent
+ * operations share rows.  Negative for a NULL plan. */
+int oxh_plan_table_rows(const OxhPlan *plan);
 /* The poll limit of every wait.  With `phantom_workgroup` set the waits also
  * expect a workgroup that does not exist, so every wait runs into the limit:
  * the way to test the give-up path without hanging anything. */

@@ -68,6 +68,7 @@ SIGNATURES = {
     "oxh_plan_status": (I, [V, V]),
     "oxh_plan_info": (I, [V, ctypes.POINTER(Z), ctypes.POINTER(Z), ctypes.POINTER(Z), ctypes.POINTER(Z)]),
     "oxh_plan_prestaged": (I, [V]),
+    "oxh_plan_table_rows": (I, [V]),
     "oxh_q6_k_group": (I, [V, Z, Z, V, V]),
     "oxh_plan_set_spin_limit": (I, [V, U32, I]),
     "oxh_plan_destroy": (I, [V]),

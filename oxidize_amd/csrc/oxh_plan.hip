@@ -56,7 +56,8 @@
 #include "oxh_device.inc"
 #include "gemv_kernels.inc"
 
-#define PLAN_MAX_SEGS 4
+#define PLAN_MAX_SEGS 8             /* segments of a table row */
+#define PLAN_OP_SEGS 4              /* segments of an operation as the caller gives it */
 #define PLAN_W 16u                  /* waves per workgroup */
 #define PLAN_MAX_WG 1024u
 #define PLAN_MAX_BLOCKS 64u         /* super-blocks per row: four units per wave staged at once */
@@ -1057,47 +1058,79 @@ static int plan_deal_op(PlanOp &d, uint32_t grid, PlanLimits &lim)
     return OXH_OK;
 }
 
-/* Operations none of which depends on another may run in any grouping.  Consecutive ones that read
- * the same weight layout over vectors of the same length are put into ONE table row when together
- * they are still a short operation (at most three passes per wave on average): their segments side by
- * side, each with the staged input of the operation it came from.  Two operations of one pass per wave
- * each (q/k/v and o of a layer) would otherwise be two trips that each wait out a memory latency with
- * one load in flight per wave; merged, a wave has two or three passes to overlap.  Returns the number
- * of rows written to `run`. */
-static int plan_merge(const PlanOp *h, size_t n_ops, uint32_t grid, bool merge, PlanOp *run, size_t *n_run,
-                      PlanLimits &lim)
+/* Operations none of which depends on another may run in any order and grouping.  Operations that read
+ * the same weight layout over vectors of the same length may share ONE table row: their segments side
+ * by side, each with the staged input of the operation it came from.  What is gained is whole passes:
+ * a wave takes sixteen blocks per pass and a workgroup is as slow as its busiest wave, so 40 rows of
+ * 16 blocks per workgroup (q/k/v + o of a layer: 2.5 rows per wave) cost three passes, the down
+ * projection's 3.5 passes cost four, and every row of the table costs a workgroup barrier.  Rows are
+ * filled first-fit (an operation joins the latest earlier row of its shape with room), up to
+ * `segs` segments and `passes` passes per wave on average; plan_table_cost prices the result and the
+ * caller keeps the cheapest of a few limits.  For a Llama-3-8B decode step the winner is eight passes:
+ * gate/up of a layer with o of the next (8.0 passes), q/k/v of two layers (3.0), down of two layers
+ * (7.0), all whole: 0.720 ms against 0.743 ms with only q/k/v + o of a layer sharing a row.
+ * Writes the rows to `run`, dealt to the grid. */
+static int plan_merge(const PlanOp *h, size_t n_ops, uint32_t grid, size_t passes, uint32_t max_segs, bool any_row,
+                      PlanOp *run, size_t *n_run, PlanLimits &lim)
 {
-    const size_t limit = (size_t)grid * PLAN_W * 16u * 3u;         /* blocks: three passes per wave */
+    const size_t limit = (size_t)grid * PLAN_W * 16u * passes;      /* blocks */
+    size_t *work = (size_t *)calloc(n_ops, sizeof *work);
+    if (!work) return OXH_ERR_NOMEM;
     size_t n = 0;
-    for (size_t i = 0; i < n_ops;) {
-        PlanOp g = h[i];
-        size_t work = 0;
-        for (uint32_t k = 0; k < g.n_segs; k++) {
-            g.s[k].xq = h[i].xq;
-            work += (size_t)g.s[k].rows * (g.s[k].w2 ? 2u : 1u) * g.blocks;
-        }
-        size_t j = i + 1;
-        while (merge && j < n_ops && h[j].kind == g.kind && h[j].blocks == g.blocks &&
-               g.n_segs + h[j].n_segs <= PLAN_MAX_SEGS) {
-            size_t more = 0;
-            for (uint32_t k = 0; k < h[j].n_segs; k++)
-                more += (size_t)h[j].s[k].rows * (h[j].s[k].w2 ? 2u : 1u) * g.blocks;
-            if (work + more > limit) break;
-            for (uint32_t k = 0; k < h[j].n_segs; k++) {
-                g.s[g.n_segs] = h[j].s[k];
-                g.s[g.n_segs].xq = h[j].xq;
-                g.n_segs++;
+    for (size_t i = 0; i < n_ops; i++) {
+        size_t more = 0;
+        for (uint32_t k = 0; k < h[i].n_segs; k++)
+            more += (size_t)h[i].s[k].rows * (h[i].s[k].w2 ? 2u : 1u) * h[i].blocks;
+        size_t target = n;
+        for (size_t r = n; passes != 0 && r-- > 0;) {
+            if (run[r].kind == h[i].kind && run[r].blocks == h[i].blocks &&
+                run[r].n_segs + h[i].n_segs <= max_segs && work[r] + more <= limit) {
+                target = r;
+                break;
             }
-            work += more;
-            j++;
+            if (!any_row) break;                /* neighbours only */
         }
-        const int drc = plan_deal_op(g, grid, lim);
+        if (target == n) {
+            run[n] = h[i];
+            run[n].n_segs = 0;
+            work[n] = 0;
+            n++;
+        }
+        PlanOp &g = run[target];
+        for (uint32_t k = 0; k < h[i].n_segs; k++) {
+            g.s[g.n_segs] = h[i].s[k];
+            g.s[g.n_segs].xq = h[i].xq;
+            g.n_segs++;
+        }
+        work[target] += more;
+    }
+    free(work);
+    for (size_t r = 0; r < n; r++) {
+        const int drc = plan_deal_op(run[r], grid, lim);
         if (drc) return drc;
-        run[n++] = g;
-        i = j;
     }
     *n_run = n;
     return OXH_OK;
+}
+
+/* Pass slots a dealt table takes: per row the passes of the busiest wave of its busiest workgroup
+ * (rows of a pair count twice), plus half a pass for the row's barrier and row sums. */
+static double plan_table_cost(const PlanOp *run, size_t n_run)
+{
+    double cost = 0.0;
+    for (size_t r = 0; r < n_run; r++) {
+        size_t worst = 0;
+        for (uint32_t k = 0; k < run[r].n_segs; k++) {
+            const PlanSeg &sg = run[r].s[k];
+            const size_t wg_rows = (size_t)sg.rows_q * PLAN_W + (sg.rows_rem < PLAN_W ? sg.rows_rem : PLAN_W);
+            const size_t flat = wg_rows * (sg.w2 ? 2u : 1u);
+            const size_t per_wave = (flat + PLAN_W - 1) / PLAN_W;
+            const size_t p = (per_wave * run[r].blocks + 15u) / 16u;
+            if (p > worst) worst = p;
+        }
+        cost += (double)worst + 0.5;
+    }
+    return cost;
 }
 
 extern "C" int oxh_plan_create(const OxhPlanOp *ops, size_t n_ops, OxhPlan **out)
@@ -1164,7 +1197,7 @@ extern "C" int oxh_plan_create(const OxhPlanOp *ops, size_t n_ops, OxhPlan **out
         for (size_t k = 0; k < o.n_segs; k++) {
             const OxhSegment &sg = o.segs[k];
             if (sg.rows == 0) continue;
-            if (ns == PLAN_MAX_SEGS || !sg.d_w || !sg.d_out || sg.act_first != 0 || sg.n_vec > 1 ||
+            if (ns == PLAN_OP_SEGS || !sg.d_w || !sg.d_out || sg.act_first != 0 || sg.n_vec > 1 ||
                 sg.rows > 0x3FFFFFFFull / (d.blocks * 16u)) {
                 rc = oxh_internal_errorf(OXH_ERR_ARG, "invalid argument: plan: operation %zu: at most four non-empty "
                                          "segments, each over activation 0 with one vector", i);
@@ -1243,14 +1276,41 @@ extern "C" int oxh_plan_create(const OxhPlanOp *ops, size_t n_ops, OxhPlan **out
     PlanOp *run = nullptr;
     size_t n_run = n_ops;
     if (pl->ext) {
-        const char *pm = getenv("OXH_PLAN_MERGE");
+        /* OXH_PLAN_MERGE: 0 every operation in a row of its own; 1 neighbours only, four segments, three
+         * passes per wave; 2 (default) any earlier row, eight segments, the cheapest of several pass limits
+         * (OXH_PLAN_MERGE_PASSES fixes the limit) */
+        const char *pm = getenv("OXH_PLAN_MERGE"), *pp = getenv("OXH_PLAN_MERGE_PASSES");
+        const int mode = pm && pm[0] >= '0' && pm[0] <= '2' ? pm[0] - '0' : 2;
         run = (PlanOp *)calloc(n_ops, sizeof *run);
-        if (!run) { free(h); free(pl); return oxh_internal_errorf(OXH_ERR_NOMEM, "out of host memory building a plan"); }
-        const int mrc = plan_merge(h, n_ops, grid, !(pm && pm[0] == '0'), run, &n_run, lim);
-        if (mrc) {
+        PlanOp *trial = (PlanOp *)calloc(n_ops, sizeof *trial);
+        if (!run || !trial) {
+            free(h); free(run); free(trial); free(pl);
+            return oxh_internal_errorf(OXH_ERR_NOMEM, "out of host memory building a plan");
+        }
+        const size_t fixed = pp && *pp ? strtoul(pp, nullptr, 10) : 0;
+        const size_t first = mode == 0 ? 0 : mode == 1 ? 3 : fixed ? fixed : 3, last = mode == 2 && !fixed ? 10 : first;
+        double best = -1.0;
+        PlanLimits best_lim = lim;
+        int mrc = OXH_OK;
+        for (size_t passes = first; passes <= last; passes++) {
+            PlanLimits tl = lim;
+            size_t tn = 0;
+            const int trc = plan_merge(h, n_ops, grid, passes, mode == 2 ? PLAN_MAX_SEGS : PLAN_OP_SEGS, mode == 2, trial, &tn, tl);
+            if (trc) { mrc = trc; continue; }
+            const double c = plan_table_cost(trial, tn);
+            if (best < 0.0 || c < best) {
+                best = c;
+                best_lim = tl;
+                n_run = tn;
+                memcpy(run, trial, tn * sizeof *run);
+            }
+        }
+        free(trial);
+        if (best < 0.0) {
             free(h); free(run); free(pl);
             return oxh_internal_errorf(mrc, "plan: merged operations have more rows than %u workgroups can own", grid);
         }
+        lim = best_lim;
     }
     pl->n_run = (uint32_t)n_run;
     pl->ld.act_bytes = (max_act + 15u) & ~15u;
@@ -1352,6 +1412,11 @@ extern "C" int oxh_plan_info(const OxhPlan *pl, size_t *n_ops, size_t *n_waits, 
     if (workgroups) *workgroups = pl->grid;
     if (lds_bytes) *lds_bytes = pl->lds_bytes;
     return OXH_OK;
+}
+
+extern "C" int oxh_plan_table_rows(const OxhPlan *pl)
+{
+    return pl ? (int)pl->n_run : -1;
 }
 
 extern "C" int oxh_plan_prestaged(const OxhPlan *pl)

@@ -319,6 +319,7 @@ class Plan:
         check(lib().oxh_plan_info(self.handle, *[ctypes.byref(x) for x in v]))
         out = dict(zip(("n_ops", "n_waits", "workgroups", "lds_bytes"), [int(x.value) for x in v]))
         out["prestaged"] = bool(lib().oxh_plan_prestaged(self.handle))
+        out["table_rows"] = lib().oxh_plan_table_rows(self.handle)
         return out
 
     def set_spin_limit(self, polls, phantom_workgroup=False):

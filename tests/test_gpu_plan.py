@@ -35,14 +35,18 @@ def test_independent_set_matches_single_launches_and_oracle(oxh, monkeypatch, hi
     info = plan.info()
     assert info["n_ops"] == 4 * layers and info["n_waits"] == 0      # nothing depends on anything here
     assert info["prestaged"]                                          # so the inputs are staged ahead
-    # short neighbours of one layout (q/k/v and o) share a table row by default; the same plan with every
-    # operation in a row of its own must give the same bits
+    # operations of one layout share table rows by default (q/k/v + o and the down projections of two layers
+    # at a time); neighbours only (q/k/v + o of a layer) and every operation in a row of its own must give
+    # the same bits
+    monkeypatch.setenv("OXH_PLAN_MERGE", "1")
+    neighbours = mv.Plan(d.plan_ops())
     monkeypatch.setenv("OXH_PLAN_MERGE", "0")
     apart = mv.Plan(d.plan_ops())
     monkeypatch.delenv("OXH_PLAN_MERGE")
-    assert apart.info()["lds_bytes"] > info["lds_bytes"]              # a longer table
+    assert apart.info()["table_rows"] == 4 * layers and neighbours.info()["table_rows"] == 3 * layers
+    assert info["table_rows"] < 3 * layers
     for rep in range(2):
-        for p in (plan, apart):
+        for p in (plan, neighbours, apart):
             for l in range(layers):
                 for op in range(4):
                     mv.lib().oxh_memset(ctypes.c_void_p(d.out[l][op].ptr), 0xFF, d.out[l][op].nbytes, None)
@@ -54,6 +58,7 @@ def test_independent_set_matches_single_launches_and_oracle(oxh, monkeypatch, hi
                     assert np.array_equal(bits(d.output(l, op)), bits(want_out[l][op])), (rep, l, op)
                     assert np.array_equal(d.activation(l, op), want_act[l][op]), (rep, l, op)
     apart.destroy()
+    neighbours.destroy()
     # and one matrix against the oracle directly
     o = oxlibs.oracle()
     name, qt, rows, cols, _ = d.ops[3]
