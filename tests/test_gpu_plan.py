@@ -252,7 +252,7 @@ def test_what_a_plan_declines(oxh):
     assert e.value.status == _lib.ERR_ARG
 
 
-@pytest.mark.parametrize("seed", range(6))
+@pytest.mark.parametrize("seed", range(20))
 def test_random_independent_plans_match_the_launches(oxh, seed):
     """Seeded random plans of independent operations: one to four segments of ragged sizes (fewer rows than
     waves, rows no multiple of anything), pairs, every kind a plan takes (the regrouped Q6_K included),
