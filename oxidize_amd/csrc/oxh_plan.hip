@@ -740,6 +740,9 @@ k_plan(const PlanOp *__restrict__ ops, uint32_t n_ops, const PlanSync sy, const 
         XStage xs;
 #pragma unroll
         for (int u = 0; u < 4; u++) xs.x[u] = xs.t[u] = xs.b[u] = XRegs{ 0.f, 0.f, 0.f, 0.f };
+        /* what this wave owns of the next operation: scalar arithmetic, done while nothing waits for it */
+        PWork nx = cur;
+        if (i + 1u < n_ops) nx = plan_work(&tab[i + 1u], wave);
         if (op.wait == 0u) {
             /* nothing to wait for: the vector goes first and is there in a microsecond */
             plan_stage_issue(op, xs, ln, wave);
@@ -754,9 +757,6 @@ k_plan(const PlanOp *__restrict__ ops, uint32_t n_ops, const PlanSync sy, const 
             if (wave == 0u) plan_prefetch<HAS_Q5>(cur, A, 0u, ln);
         }
         plan_stamp(sy, i, 1, ln, wave);
-        /* what this wave owns of the next operation */
-        PWork nx = cur;
-        if (i + 1u < n_ops) nx = plan_work(&tab[i + 1u], wave);
 
         /* a prologue's side outputs are one workgroup's work, and not workgroup 0's: that one gathers the
          * counters, and whatever holds it up holds everybody up */
