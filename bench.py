@@ -313,6 +313,27 @@ def secondary_figures(mv, synth):
         c.free()
     d_x.free()
     d_o.free()
+    # the host-pointer entry point itself (never `value`: inputs and outputs cross the bus on every call):
+    # oc_matvec_quantized's wall time per call from this process, weights resident after the first call
+    host_api = {}
+    for name, qt, r_, c_ in (("q4_k_4096x4096", Q4K, 4096, 4096), ("q4_k_14336x4096", Q4K, 14336, 4096),
+                             ("q6_k_4096x14336", Q6K, 4096, 14336)):
+        w = synth.weights(qt, r_, c_, seed=0, stream=11)
+        x = synth.normal(c_, seed=0, stream=2010)
+        import numpy as np
+        o_, t_ = np.zeros(r_, np.float32), np.zeros(c_, np.float32)
+        rb = synth.row_bytes(qt, c_)
+        best = None
+        for rep in range(4):
+            t0 = time.perf_counter()
+            for _ in range(100):
+                mv.matvec_quantized(qt, w, r_, c_, rb, x, o_, t_)
+            dt = (time.perf_counter() - t0) / 100 * 1e6
+            best = dt if best is None or dt < best else best
+        host_api[name] = round(best, 1)
+    from oxidize_amd import _lib
+    _lib.check(_lib.lib().oxh_weight_clear())
+    out["host_pointer_api_us_per_call"] = host_api
     # the Q6_K down projection in the two layouts the decode kernels read: the file layout and the
     # regrouped copy the decode set keeps (same bytes); eight distinct copies in turn (386 MB: from HBM)
     rows, cols = 4096, 14336

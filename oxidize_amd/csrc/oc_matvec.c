@@ -498,8 +498,15 @@ static DevBuf g_dx, g_dact, g_dout;
 /* Page-locked host staging for the decode-sized entry points: the caller's
  * vectors are ordinary pageable memory, and a copy between pageable memory and
  * the device is a synchronous two-step affair inside the runtime (about 12 us
- * each, three per call).  Staged through pinned buffers a call is one DMA in,
- * the launch, one DMA out (output and quantised activation together). */
+ * each, three per call).  Page-locked memory the device reads and writes in
+ * place, so up to HOST_DIRECT_MAX bytes a call's input is pulled out of it by a
+ * copy kernel ahead of the GEMV launch, and the GEMV kernel stores its rows (and
+ * the quantised activation) straight into it: two launches and a wait, where a
+ * DMA each way costs 7-8 us more per call than the 5-15 us the kernel runs.
+ * (Letting the GEMV read its input in place would not do: every workgroup
+ * reads the whole vector, 256 trips over the bus.)  Larger transfers keep the
+ * DMA engines. */
+#define HOST_DIRECT_MAX ((size_t)1 << 20)
 typedef struct {
     void *p;
     size_t bytes;
@@ -565,6 +572,13 @@ static int reserve(DevBuf *b, size_t bytes)
     if (rc) return rc;
     b->bytes = want;
     return OXH_OK;
+}
+
+/* The first `bytes` of the pinned input image to the device input buffer. */
+static int push_input(size_t bytes)
+{
+    if (bytes <= HOST_DIRECT_MAX) return oxh_internal_copy16(g_dx.p, g_hin.p, align16(bytes), NULL);
+    return oxh_memcpy_h2d(g_dx.p, g_hin.p, bytes, NULL);
 }
 
 static bool mul_ok(size_t a, size_t b, size_t *out)
@@ -648,13 +662,15 @@ static int mv_one(uint32_t qtype, const uint8_t *data, size_t rows,
     if ((rc = reserve_host(&g_hout, act_off + abytes))) return rc;
 
     memcpy(g_hin.p, input, cols * sizeof(float));
-    if ((rc = oxh_memcpy_h2d(g_dx.p, g_hin.p, cols * sizeof(float), NULL))) return rc;
+    if ((rc = push_input(cols * sizeof(float)))) return rc;
     /* one launch: quantise the activation inside the GEMV kernel */
-    OxhSegment seg = { d_w, (float *)g_dout.p, rows, 0, 0, NULL };
+    const bool direct = act_off + abytes <= HOST_DIRECT_MAX;
+    uint8_t *dst = direct ? (uint8_t *)g_hout.p : (uint8_t *)g_dout.p;
+    OxhSegment seg = { d_w, (float *)dst, rows, 0, 0, NULL };
     if ((rc = oxh_gemv_segments_f32(run_type, &seg, 1, cols, (const float *)g_dx.p, cols,
-                                    (uint8_t *)g_dout.p + act_off, 1, rows, NULL)))
+                                    dst + act_off, 1, rows, NULL)))
         return rc;
-    if ((rc = oxh_memcpy_d2h(g_hout.p, g_dout.p, act_off + abytes, NULL))) return rc;
+    if (!direct && (rc = oxh_memcpy_d2h(g_hout.p, g_dout.p, act_off + abytes, NULL))) return rc;
     if ((rc = oxh_stream_sync(NULL))) return rc;
     memcpy(output, g_hout.p, obytes);
     memcpy(temp, (const uint8_t *)g_hout.p + act_off, abytes);
@@ -692,7 +708,9 @@ static int grouped(uint32_t qtype, const uint8_t *const *datas,
         if (!inputs[i]) return bad_arg("grouped: NULL input");
         memcpy((float *)g_hin.p + i * cols, inputs[i], cols * sizeof(float));
     }
-    if ((rc = oxh_memcpy_h2d(g_dx.p, g_hin.p, xbytes, NULL))) return rc;
+    if ((rc = push_input(xbytes))) return rc;
+    const bool direct = total_rows * sizeof(float) <= HOST_DIRECT_MAX;
+    float *dst = direct ? (float *)g_hout.p : (float *)g_dout.p;
     enum { CHUNK = 32 };
     OxhSegment segs[CHUNK];
     size_t done_rows = 0;
@@ -719,7 +737,7 @@ static int grouped(uint32_t qtype, const uint8_t *const *datas,
                 if (t != OXH_Q6_K_G8) all_alt = false;
             }
             segs[i].d_w = d_w;
-            segs[i].d_out = (float *)g_dout.p + done_rows;
+            segs[i].d_out = dst + done_rows;
             segs[i].rows = rows[k];
             segs[i].act_first = n_inputs == 1 ? 0 : k;
             segs[i].n_vec = 0;
@@ -731,7 +749,7 @@ static int grouped(uint32_t qtype, const uint8_t *const *datas,
                                         NULL, 1, 0, NULL)))
             return rc;
     }
-    if ((rc = oxh_memcpy_d2h(g_hout.p, g_dout.p, total_rows * sizeof(float), NULL))) return rc;
+    if (!direct && (rc = oxh_memcpy_d2h(g_hout.p, g_dout.p, total_rows * sizeof(float), NULL))) return rc;
     if ((rc = oxh_stream_sync(NULL))) return rc;
     size_t off = 0;
     for (size_t k = 0; k < n_outs; k++) {

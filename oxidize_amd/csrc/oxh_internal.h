@@ -29,6 +29,11 @@ int oxh_internal_device(void);
 /* Host layer: drop the weight registry and the staging buffers (oxh_shutdown). */
 void oxh_internal_host_reset(void);
 
+/* 16-byte-granular copy by a kernel (either side may be page-locked host memory). */
+int oxh_internal_copy16(void *dst, const void *src, size_t bytes, void *stream);
+/* Wait for a stream by polling it `spins` times before blocking. */
+int oxh_internal_stream_sync_spin(void *stream, unsigned spins);
+
 #ifdef __cplusplus
 }
 #endif

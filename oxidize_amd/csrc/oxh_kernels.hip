@@ -2061,6 +2061,49 @@ extern "C" int oxh_memset(void *d_dst, int value, size_t bytes, void *stream)
     return OXH_OK;
 }
 
+/* 16-byte pieces of src to dst, both 16-byte aligned, bytes a multiple of 16.  The host layer uses it
+ * to pull a call's input out of page-locked host memory (which the device reads in place) and to push
+ * results there: for the few tens of KB of a decode call a launch costs less than a copy through the
+ * DMA engines. */
+__global__ __launch_bounds__(256) void
+k_copy16(u32x4 *__restrict__ dst, const u32x4 *__restrict__ src, size_t n16)
+{
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n16) dst[i] = src[i];
+}
+
+extern "C" int oxh_internal_copy16(void *dst, const void *src, size_t bytes, void *stream)
+{
+    int rc = ensure_init();
+    if (rc) return rc;
+    if (bytes == 0) return OXH_OK;
+    if (!dst || !src || (((uintptr_t)dst | (uintptr_t)src | bytes) & 15u))
+        return arg_fail("oxh_internal_copy16: pointers and size must be multiples of 16");
+    const size_t n16 = bytes / 16u;
+    if (n16 > ((size_t)1 << 31)) return arg_fail("oxh_internal_copy16: too large");
+    hipLaunchKernelGGL(k_copy16, dim3((uint32_t)((n16 + 255u) / 256u)), dim3(256), 0, pick_stream(stream),
+                       (u32x4 *)dst, (const u32x4 *)src, n16);
+    HIP_TRY(hipGetLastError());
+    return OXH_OK;
+}
+
+/* Wait for the stream by polling it: a blocking wait sleeps on an interrupt and wakes up some
+ * microseconds after the work is done, which a decode-sized call notices.  After `spins` polls the
+ * blocking wait takes over, so a long batch does not burn a core. */
+extern "C" int oxh_internal_stream_sync_spin(void *stream, unsigned spins)
+{
+    int rc = ensure_init();
+    if (rc) return rc;
+    hipStream_t s = pick_stream(stream);
+    for (unsigned i = 0; i < spins; i++) {
+        const hipError_t e = hipStreamQuery(s);
+        if (e == hipSuccess) return OXH_OK;
+        if (e != hipErrorNotReady) return hip_fail(e, "hipStreamQuery");
+    }
+    HIP_TRY(hipStreamSynchronize(s));
+    return OXH_OK;
+}
+
 extern "C" int oxh_stream_create(void **stream)
 {
     int rc = ensure_init();
