@@ -868,12 +868,21 @@ static int mv_batch(uint32_t qtype, const uint8_t *data, size_t rows,
     if ((rc = reserve(&g_dx, packed_in))) return rc;
     if ((rc = reserve(&g_dact, act_total))) return rc;
     if ((rc = reserve(&g_dout, packed_out))) return rc;
-    if (in_stride == cols)
+    /* a few vectors travel like a single one: through the page-locked images, in place */
+    const bool in_direct = packed_in <= HOST_DIRECT_MAX, out_direct = packed_out <= HOST_DIRECT_MAX;
+    if (in_direct) {
+        if ((rc = reserve_host(&g_hin, packed_in))) return rc;
+        for (size_t v = 0; v < n_vec; v++)
+            memcpy((float *)g_hin.p + v * cols, inputs + v * in_stride, cols * sizeof(float));
+        rc = push_input(packed_in);
+    } else if (in_stride == cols)
         rc = oxh_memcpy_h2d(g_dx.p, inputs, packed_in, NULL);
     else
         rc = oxh_memcpy2d_h2d(g_dx.p, cols * sizeof(float), inputs, in_stride * sizeof(float),
                               cols * sizeof(float), n_vec, NULL);
     if (rc) return rc;
+    if (out_direct && (rc = reserve_host(&g_hout, packed_out))) return rc;
+    float *const d_out = out_direct ? (float *)g_hout.p : (float *)g_dout.p;
     const float *d_x = (const float *)g_dx.p;
     /* More vectors than the GEMV kernel keeps in flight: Q4_K, Q5_K and Q6_K go to the
      * int8-MFMA kernel behind a stand-alone quantiser launch; everything else
@@ -881,7 +890,7 @@ static int mv_batch(uint32_t qtype, const uint8_t *data, size_t rows,
     if (n_vec > 8 && (qtype == OXH_Q4_K_S || qtype == OXH_Q4_K_M || qtype == OXH_Q5_K_S ||
                       qtype == OXH_Q5_K_M || qtype == OXH_Q6_K)) {
         if ((rc = quantize(kind, d_x, cols, n_vec, cols, g_dact.p))) return rc;
-        if ((rc = oxh_mmq_ex(qtype, d_w, rows, cols, g_dact.p, n_vec, (float *)g_dout.p, rows,
+        if ((rc = oxh_mmq_ex(qtype, d_w, rows, cols, g_dact.p, n_vec, d_out, rows,
                              mmq_relaxed_enabled() ? OXH_MMQ_RELAXED : 0u, NULL)))
             return rc;
     } else if (n_vec > 8 && (qtype == OXH_Q2_K || qtype == OXH_Q3_K_S || qtype == OXH_Q3_K_M ||
@@ -896,7 +905,7 @@ static int mv_batch(uint32_t qtype, const uint8_t *data, size_t rows,
             return rc;
         if ((rc = quantize(kind, d_x, cols, n_vec, cols, g_dact.p))) return rc;
         if ((rc = oxh_mmq(qtype == OXH_Q2_K ? OXH_Q2_K_WIDE : OXH_Q6_K, d_prep, rows, cols, g_dact.p, n_vec,
-                          (float *)g_dout.p, rows, NULL)))
+                          d_out, rows, NULL)))
             return rc;
     } else {
         const size_t step = oxh_gemv_max_nvec_buffered(qtype, cols);
@@ -907,7 +916,7 @@ static int mv_batch(uint32_t qtype, const uint8_t *data, size_t rows,
         if (n_vec <= step) {
             /* one launch with the quantisation fused in; with room for the quantised activations a
              * launch of several vectors may run on the matrix cores (same results; the library decides) */
-            OxhSegment seg = { d_w, (float *)g_dout.p, rows, 0, 0, NULL };
+            OxhSegment seg = { d_w, d_out, rows, 0, 0, NULL };
             if ((rc = oxh_gemv_segments_f32(qtype, &seg, 1, cols, d_x, cols, g_dact.p, n_vec, rows, NULL)))
                 return rc;
         } else {
@@ -915,7 +924,7 @@ static int mv_batch(uint32_t qtype, const uint8_t *data, size_t rows,
              * the matrix cores (the matrix is streamed once per 64 activations), the rest walk the batch in
              * slices over the stored bytes */
             if ((rc = quantize(kind, d_x, cols, n_vec, cols, g_dact.p))) return rc;
-            rc = kind == 1 ? oxh_mmq(qtype, d_w, rows, cols, g_dact.p, n_vec, (float *)g_dout.p, rows, NULL)
+            rc = kind == 1 ? oxh_mmq(qtype, d_w, rows, cols, g_dact.p, n_vec, d_out, rows, NULL)
                            : OXH_DECLINED;
             if (rc != OXH_OK && rc != OXH_DECLINED) return rc;
             if (rc == OXH_DECLINED) {
@@ -929,13 +938,19 @@ static int mv_batch(uint32_t qtype, const uint8_t *data, size_t rows,
                     size_t n = 0;
                     for (; n < SLICES && v0 < n_vec; n++, v0 += step) {
                         const size_t m = n_vec - v0 < step ? n_vec - v0 : step;
-                        const OxhSegment seg = { d_w, (float *)g_dout.p + v0 * rows, rows, v0, m, NULL };
+                        const OxhSegment seg = { d_w, d_out + v0 * rows, rows, v0, m, NULL };
                         segs[n] = seg;
                     }
                     if ((rc = oxh_gemv_segments(qtype, segs, n, cols, g_dact.p, step, rows, NULL))) return rc;
                 }
             }
         }
+    }
+    if (out_direct) {
+        if ((rc = oxh_stream_sync(NULL))) return rc;
+        for (size_t v = 0; v < n_vec; v++)
+            memcpy(outputs + v * out_stride, (const float *)g_hout.p + v * rows, rows * sizeof(float));
+        return OXH_OK;
     }
     if (out_stride == rows)
         rc = oxh_memcpy_d2h(outputs, g_dout.p, packed_out, NULL);
