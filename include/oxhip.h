@@ -609,7 +609,9 @@ int oxh_weight_stats(size_t *n_registered, size_t *n_cached, size_t *cached_byte
 /* Same arguments and results as oc_matvec_quantized
  * (oxidize-c/include/oxidize/matvec.h:50-52; matvec.c:833-907): output[r] =
  * dot(W[r], Q8(input)); `temp` (>= cols floats) receives the quantised
- * activation bytes exactly as the reference leaves them there. */
+ * activation bytes exactly as the reference leaves them there, for Q4_0 and
+ * AL5 followed (from the next multiple of four bytes) by the int32 sum of
+ * every 32-value block (matvec.c:198-227, :866-877). */
 int oxh_matvec_quantized(uint32_t qtype, const uint8_t *data, size_t rows,
                          size_t cols, size_t row_bytes, const float *input,
                          float *output, float *temp);

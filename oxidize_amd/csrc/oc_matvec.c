@@ -674,6 +674,19 @@ static int mv_one(uint32_t qtype, const uint8_t *data, size_t rows,
     if ((rc = oxh_stream_sync(NULL))) return rc;
     memcpy(output, g_hout.p, obytes);
     memcpy(temp, (const uint8_t *)g_hout.p + act_off, abytes);
+    /* Q4_0 and AL5: the reference leaves the int32 sum of every 32-value activation block behind the
+     * blocks, from the next multiple of four bytes on (matvec.c:198-227, :866-877); temp has the room
+     * (34 + 4 bytes per 32 floats) */
+    if (qtype == OXH_Q4_0 || qtype == OXH_AL5) {
+        uint8_t *act = (uint8_t *)temp;
+        const size_t blocks = cols / 32u, at = (abytes + 3u) & ~(size_t)3u;
+        for (size_t b = 0; b < blocks; b++) {
+            const int8_t *q = (const int8_t *)(act + b * 34u + 2u);
+            int32_t sum = 0;
+            for (int i = 0; i < 32; i++) sum += q[i];
+            memcpy(act + at + 4u * b, &sum, sizeof sum);
+        }
+    }
     return OXH_OK;
 }
 

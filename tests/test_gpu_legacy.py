@@ -57,6 +57,32 @@ def test_matvec_quantized_bits(oxh, name, qtype, rows, cols):
         assert np.all(np.abs(out - r_out) <= 1e-4 + 1e-5 * np.abs(r_out))
 
 
+@pytest.mark.parametrize("qtype", [3, 17])
+@pytest.mark.parametrize("rows,cols", [(5, 96), (64, 4096)])
+def test_block_sums_left_behind_the_activation(oxh, qtype, rows, cols):
+    """Q4_0 and AL5: the int32 sum of every activation block follows the blocks in temp, from the next
+    multiple of four bytes on (matvec.c:198-227, :866-877)."""
+    w = synth.weights(3, rows, cols, seed=43, stream=rows)        # AL5 is the Q4_0 layout under its own id
+    x = synth.normal(cols, seed=43, stream=9)
+    out = np.zeros(rows, np.float32)
+    temp = np.full(cols, np.nan, np.float32)
+    rb = synth.row_bytes(3, cols)
+    assert mv.matvec_quantized(qtype, w, rows, cols, rb, x, out, temp) == 0
+    nact, blocks = mv.act_bytes(qtype, cols), cols // 32
+    raw = temp.view(np.uint8)
+    q = raw[:nact].reshape(blocks, 34)[:, 2:].view(np.int8).astype(np.int32)
+    at = (nact + 3) & ~3
+    got = raw[at:at + 4 * blocks].view(np.int32)
+    assert np.array_equal(got, q.sum(axis=1))
+    ref = oxlibs.ref()
+    if ref is not None:
+        r_out = np.zeros(rows, np.float32)
+        r_tmp = np.full(cols, np.nan, np.float32)
+        ref.oc_matvec_quantized(qtype, w.ctypes.data, rows, cols, rb, x.ctypes.data, r_out.ctypes.data,
+                                r_tmp.ctypes.data)
+        assert np.array_equal(raw[:at + 4 * blocks], r_tmp.view(np.uint8)[:at + 4 * blocks])
+
+
 @pytest.mark.parametrize("name,qtype", LEGACY)
 def test_api_goldens_from_the_compiled_reference(oxh, name, qtype):
     g = np.load(GOLD)
