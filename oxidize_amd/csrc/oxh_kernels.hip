@@ -862,17 +862,27 @@ struct GemvIo {
     const OxhPrologue *pro; /* fused prologue in front of the quantiser, or NULL */
 };
 
-/* Q4_K with three or more activations per weight goes to the matrix cores:
- * the dot-instruction GEMV repeats its integer work per activation and stops
- * keeping up with the weight stream there (OXH_GEMV_MFMA_MIN_NV moves the
- * threshold; 0 = never).  The MFMA kernel reads Q8_K activations, so an f32
- * launch qualifies only if it has somewhere to put the quantised bytes. */
-static bool gemv_wants_mfma(uint32_t qtype, const GemvIo &io, size_t max_nv, const int32_t *dump)
+/* Q4_K, Q5_K and Q6_K with several activations per weight go to the matrix cores when the launch is
+ * large enough for them: the dot-instruction GEMV repeats its integer work per activation (a launch
+ * grows by 15-22 % per activation), while a tile kernel's workgroup needs 0.75 us per super-block of
+ * its rows whatever the batch (1.2 us for Q6_K), so a launch of few tiles is paced by that and not by
+ * the weight stream.  Measured (us, 2 / 3 / 4 / 6 / 8 activations, dot kernel against tiles):
+ * 4096 x 4096 Q4_K 5.8 / 6.5 / 7.3 / 8.8 / 10.3 against 12.4; 6144 x 4096 7.3 / 8.4 / 9.5 / 11.7 / 13.8
+ * against 12.6; 14336 x 4096 10.9 / 13.0 / 15.0 / 18.9 / 22.9 against 13.6; 28672 x 4096 15.4 / 18.7 /
+ * 21.9 / 28.3 / 34.0 against 20.6; 4096 x 14336 Q6_K 14.3 / 17.0 / 19.6 / 24.7 / 42.8 against 66.  So:
+ * tiles from four activations on where the launch has at least half a tile of 64 rows per CU, the
+ * dot kernel below that (OXH_GEMV_MFMA_MIN_NV moves the first threshold, 0 = never;
+ * OXH_GEMV_MFMA_MIN_TILES the second, in tiles).  Nine activations and more have no dot kernel.  The
+ * MFMA kernel reads Q8_K activations, so an f32 launch qualifies only if it has somewhere to put the
+ * quantised bytes. */
+static bool gemv_wants_mfma(uint32_t qtype, const GemvIo &io, size_t max_nv, const int32_t *dump, size_t tiles64)
 {
     static int min_nv = -1;
-    if (min_nv < 0) min_nv = (int)env_u32("OXH_GEMV_MFMA_MIN_NV", 3, 0, 64);
+    if (min_nv < 0) min_nv = (int)env_u32("OXH_GEMV_MFMA_MIN_NV", 4, 0, 64);
+    static const uint32_t min_tiles = env_u32("OXH_GEMV_MFMA_MIN_TILES", (uint32_t)(g_n_cu > 0 ? g_n_cu : 256) / 2u, 0, 1u << 20);
     if ((!is_q4k(qtype) && !is_q5k(qtype) && qtype != OXH_Q6_K) || dump || min_nv == 0 ||
         max_nv < (size_t)min_nv) return false;
+    if (max_nv <= OXH_MAX_NV && tiles64 < min_tiles) return false;
     /* a prologue lives in the GEMV kernels' quantiser only */
     if (io.pro) return false;
     return io.d_acts != nullptr || io.d_act_out != nullptr;
@@ -1046,7 +1056,7 @@ static int launch_gemv(uint32_t qtype, const OxhSegment *segs, size_t n_segs, si
     size_t max_nv = 0;
     bool all_one = true, any_pair = false;
     /* a paired segment walks two matrices: it counts twice wherever work is sized */
-    size_t total_work = 0;
+    size_t total_work = 0, tiles64 = 0;
     for (size_t i = 0; i < n_segs; i++) {
         const size_t nv = segs[i].n_vec ? segs[i].n_vec : n_vec;
         if (nv < 1 || nv > MQ80_TOK) return arg_fail("gemv: segment n_vec must be 1..8");
@@ -1058,6 +1068,7 @@ static int launch_gemv(uint32_t qtype, const OxhSegment *segs, size_t n_segs, si
         if (segs[i].rows > 0x3FFFFFFFull / (blocks * 16u)) return arg_fail("gemv: segment too large");
         if (segs[i].rows && (!segs[i].d_w || !segs[i].d_out)) return arg_fail("gemv: NULL segment pointer");
         total_rows += segs[i].rows;
+        tiles64 += (segs[i].rows + 63u) / 64u;
         total_work += segs[i].rows * (segs[i].d_w_pair ? 2u : 1u);
         if (segs[i].act_first > max_act) max_act = segs[i].act_first;
         if (segs[i].rows && segs[i].act_first + nv > act_end) act_end = segs[i].act_first + nv;
@@ -1065,7 +1076,7 @@ static int launch_gemv(uint32_t qtype, const OxhSegment *segs, size_t n_segs, si
     if (total_rows == 0) return OXH_OK;
     if (any_pair && dump) return arg_fail("gemv: no sub-block dump of a paired launch");
     if (is_iq(qtype) && dump) return arg_fail("gemv: no sub-block dump for the codebook formats");
-    if (!any_pair && gemv_wants_mfma(qtype, io, max_nv, dump))
+    if (!any_pair && gemv_wants_mfma(qtype, io, max_nv, dump, tiles64))
         return launch_mmq_segments(qtype, segs, n_segs, cols, blocks, io, n_vec_default, act_end,
                                    out_stride, stream);
     if (!any_pair && q80_wants_mfma(qtype, io, max_nv, blocks, dump))
