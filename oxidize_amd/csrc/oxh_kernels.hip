@@ -1419,17 +1419,21 @@ static void mmq6_launch(const void *d_w, size_t rows, size_t blocks, const void 
 static int mmq_tile_shape(uint32_t qtype, size_t rows, size_t n_vec, size_t cus)
 {
     const size_t need = cus - cus / 8;
+    /* a launch that gives no CU more than one 64 x 16 tile is paced by a workgroup's walk over the
+     * super-blocks of its rows, not by the matrix cores: the smallest tiles then put the most CUs to
+     * work (4096 x 4096 x 64: 13.3 against 14.9 us on 64 x 32 tiles; 4096 x 14336 Q6_K: 75 against 87) */
+    const bool few_tiles = ((rows + 63) / 64) * ((n_vec + 15) / 16) <= cus;
     if (n_vec <= 16) return 4;
-    if (n_vec <= 32) return 3;
+    if (n_vec <= 32) return few_tiles ? 4 : 3;
     if (qtype == OXH_Q6_K || is_q5k(qtype) || qtype == OXH_Q2_K_WIDE) {
         if (((rows + 127) / 128) * ((n_vec + 127) / 128) >= need) return 1;
         if (!is_q5k(qtype) && ((rows + 63) / 64) * ((n_vec + 127) / 128) >= need) return 5;
         if (((rows + 127) / 128) * ((n_vec + 63) / 64) >= need) return 2;
-        return 3;
+        return few_tiles ? 4 : 3;
     }
     if (((rows + 255) / 256) * ((n_vec + 127) / 128) >= need) return 1;
     if (((rows + 127) / 128) * ((n_vec + 63) / 64) >= need) return 2;
-    return 3;
+    return few_tiles ? 4 : 3;
 }
 
 /* the 32-value formats with a matrix-core kernel, as its LEG parameter; -1 for everything else */

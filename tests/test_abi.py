@@ -217,8 +217,8 @@ def test_plan_deals_rows_within_the_grid():
 def test_mmq_tile_choice_is_host_arithmetic():
     """Which tile a matrix-core launch runs on depends on the launch and the number of compute units
     only: the benchmark's two prefill shapes take the big tiles on a 256-CU device, a device with fewer
-    units takes them sooner, small batches take the small tiles, Q6_K has the 64 x 128 tile for matrices
-    with few rows."""
+    units takes them sooner, small batches take the small tiles (the smallest when that leaves no unit more
+    than one), Q6_K has the 64 x 128 tile for matrices with few rows."""
     lib = _lib.lib()
     Q4K, Q5K, Q6K, Q80, WIDE2 = 13, 15, 16, 7, 0x1008
 
@@ -232,7 +232,10 @@ def test_mmq_tile_choice_is_host_arithmetic():
     assert tile(Q4K, 4096, 512, n_cu=64) == (0, 256, 128)
     assert tile(Q4K, 14336, 16) == (0, 64, 16)
     assert tile(Q4K, 14336, 32) == (0, 64, 32)
-    assert tile(Q4K, 1000, 100) == (0, 64, 32)           # neither larger tile fills the device
+    assert tile(Q4K, 1000, 100) == (0, 64, 16)           # neither larger tile fills the device; 16 x 7 small ones
+    assert tile(Q4K, 7000, 40) == (0, 64, 32)            # 110 x 3 of the smallest would be more than one to a unit
+    assert tile(Q4K, 4096, 64) == (0, 64, 16)            # 64 x 4 = one per unit
+    assert tile(Q4K, 4096, 128) == (0, 64, 32)
     assert tile(Q5K, 28672, 512) == (0, 128, 128)        # one row chunk per wave: 128-row tiles
     assert tile(Q5K, 3600, 500) == (0, 128, 64)
     assert tile(Q6K, 4096, 512) == (0, 64, 128)          # 32 x 4 tiles of 128 x 128 are too few
@@ -241,16 +244,17 @@ def test_mmq_tile_choice_is_host_arithmetic():
     # the rule itself, stated independently: the first of the candidates with at least 7/8 of the units busy
     def rule(qtype, rows, n_vec, n_cu):
         need = n_cu - n_cu // 8
+        small = (64, 16) if -(-rows // 64) * -(-n_vec // 16) <= n_cu else (64, 32)
         if n_vec <= 16:
             return 64, 16
         if n_vec <= 32:
-            return 64, 32
+            return small
         cands = [(256, 128), (128, 64)] if qtype == Q4K else \
                 [(128, 128), (128, 64)] if qtype == Q5K else [(128, 128), (64, 128), (128, 64)]
         for tr, tt in cands:
             if -(-rows // tr) * -(-n_vec // tt) >= need:
                 return tr, tt
-        return 64, 32
+        return small
     for qtype in (Q4K, Q5K, Q6K):
         for rows in (1, 63, 64, 1000, 4096, 7165, 14336, 28672, 151936):
             for n_vec in (1, 16, 17, 32, 33, 64, 100, 128, 129, 512, 2048):
