@@ -201,3 +201,33 @@ def test_alias_type_ids_run_the_base_layout(oxh, alias, base):
         deq = np.zeros(cols, np.float32)
         assert o.oxo_dequant_row(alias, w[int(i) * rb:].ctypes.data, cols, deq.ctypes.data) == 0
         assert np.array_equal(bits(got[k]), bits(deq))
+
+
+@pytest.mark.parametrize("name,qtype", (("q8_0", 7), ("q4_0", 3), ("q5_0", 5), ("al5_xs", 18)))
+@pytest.mark.parametrize("cols", [32, 96, 416])
+def test_segment_that_starts_two_bytes_past_a_multiple_of_four(oxh, name, qtype, cols):
+    """Rows of an odd number of these blocks are 2 (mod 4) bytes long, so a segment that starts at an odd
+    row has every other block, the first one included, two bytes past a multiple of four; the kernels
+    fetch such a block from the multiple of four ahead of it or behind its first two bytes (inside the
+    matrix either way).  Rows 1.. and 3.. of a matrix as segments of their own, one and three activations."""
+    rows = 9
+    rb = synth.row_bytes(qtype, cols)
+    assert rb % 4 == 2
+    w = synth.weights(qtype, rows, cols, seed=61, stream=cols)
+    d_w = mv.DeviceBuffer.from_host(w)
+    for nv in (1, 3):
+        xs = synth.normal(nv * cols, seed=62, stream=nv).reshape(nv, cols)
+        d_x = mv.DeviceBuffer.from_host(xs)
+        d_o = mv.DeviceBuffer(2 * nv * rows * 4)
+        first = [(1, rows - 1), (3, rows - 3)]
+        segs = mv.make_segments([(d_w.ptr + r0 * rb, d_o.ptr + k * nv * rows * 4, n, 0)
+                                 for k, (r0, n) in enumerate(first)])
+        mv.gemv_segments_f32(qtype, segs, cols, d_x.ptr, cols, None, nv, rows)
+        got = d_o.download(np.float32, 2 * nv * rows).reshape(2, nv, rows)
+        for v in range(nv):
+            want, _ = oracle_matvec(qtype, w, rows, cols, xs[v])
+            for k, (r0, n) in enumerate(first):
+                assert np.array_equal(bits(got[k, v, :n]), bits(want[r0:r0 + n])), (name, cols, nv, k)
+        d_x.free()
+        d_o.free()
+    d_w.free()
