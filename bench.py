@@ -395,6 +395,43 @@ def secondary_figures(mv, synth):
     out["q8_0_lm_head_151936x896"] = q8
     for c in copies:
         c.free()
+    # configuration 2 as a whole decode step: the Qwen2.5-0.5B-shaped Q8_0 set (24 layers x {q/k/v, o,
+    # gate/up, down} + the head, every matmul quantising its own f32 input to Q8_0; matrices of 0.9-9 MB
+    # and the 145 MB head) as ONE launch (a plan over a 32-value format: the rows of all 97 operations
+    # cut into runs and dealt to the workgroups by bytes), and as a graph of 97 launches beside it
+    from oxidize_amd.workloads import DecodeSet, QWEN2_5_0_5B
+    qs = DecodeSet(qtypes=(Q80, Q80), seed=0, **QWEN2_5_0_5B)
+    w = synth.weights(Q80, rows, cols, seed=0, stream=5)
+    d_head = mv.DeviceBuffer.from_host(w)
+    d_hx = mv.DeviceBuffer.from_host(synth.normal(cols, seed=0, stream=8))
+    d_ho = mv.DeviceBuffer(rows * 4)
+    head_seg = mv.make_segments([(d_head.ptr, d_ho.ptr, rows, 0)])
+
+    def qwen_step():
+        qs.launch_step()
+        mv.gemv_segments_f32(Q80, head_seg, cols, d_hx.ptr, cols, None, 1, rows)
+
+    qwen_step()
+    mv.sync()
+    graph = mv.Graph()
+    with graph:
+        qwen_step()
+    us_graph = timed(graph.launch, 20, mv)
+    graph.destroy()
+    qplan = mv.Plan(qs.plan_ops() + [dict(qtype=Q80, segs=head_seg, cols=cols, d_x=d_hx.ptr, d_act_out=None)])
+    us = timed(qplan.launch, 20, mv)
+    assert qplan.status() == 0
+    qplan.destroy()
+    nbytes = qs.bytes_per_step + w.nbytes + 4 * (cols + rows)
+    out["q8_0_decode_step_qwen2_5_0_5b"] = {
+        "us_per_step": round(us, 1), "launches_per_step": 1, "operations_per_step": qs.layers * len(qs.ops) + 1,
+        "bytes_per_step": nbytes, "gbps": round(nbytes / us / 1e3, 1),
+        "frac_of_hbm_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBPS, 4),
+        "as_graph_of_97_launches_us": round(us_graph, 1),
+        "note": "independent operations (every input there when the launch starts); no workgroup waits for another"}
+    d_head.free()
+    d_hx.free()
+    d_ho.free()
     # What a kernel that only reads reaches on buffers the size of the decode set's matrices (launch
     # cost included; twelve distinct buffers in turn, 793 MB, so that nothing comes from the last-level
     # cache; one graph of twelve launches per replay): the ceiling the GEMV figures stand against here.

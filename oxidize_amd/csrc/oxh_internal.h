@@ -29,6 +29,14 @@ int oxh_internal_device(void);
 /* Host layer: drop the weight registry and the staging buffers (oxh_shutdown). */
 void oxh_internal_host_reset(void);
 
+/* Plans over the 32-value formats: a table of plain GEMV launches walked by one grid (oxh_kernels.hip).
+ * `ops` is an array of OxhPlanOp; which = -1 for a type without such a launch. */
+struct OxhPlanOp;
+int oxh_internal_multi_which(uint32_t qtype);
+int oxh_internal_multi_create(const struct OxhPlanOp *ops, size_t n_ops, void **handle);
+int oxh_internal_multi_launch(void *handle, void *stream);
+void oxh_internal_multi_info(const void *handle, size_t *n_items, size_t *workgroups, size_t *lds_bytes);
+int oxh_internal_multi_destroy(void *handle);
 /* 16-byte-granular copy by a kernel (either side may be page-locked host memory). */
 int oxh_internal_copy16(void *dst, const void *src, size_t bytes, void *stream);
 /* Wait for a stream by polling it `spins` times before blocking. */

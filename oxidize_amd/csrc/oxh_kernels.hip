@@ -467,6 +467,136 @@ k_q2k_widen(const uint8_t *__restrict__ src, uint8_t *__restrict__ dst, uint32_t
 #include "moe_kernels.inc"
 #include "iq_kernels.inc"
 
+/* ─── several GEMVs of one 32-value format in one launch ──────────────── */
+
+/* A run of rows of one operation, given to one workgroup: what the GEMV kernel's steps need of it, in
+ * device memory.  Workgroup b walks items[first[b]] .. items[first[b+1] - 1]. */
+struct GemvMultiItem {
+    SegInfo seg;                /* w and out already point at the run's first row; wg_begin 0 */
+    GemvParams p;               /* act_out only in the item that holds the operation's first row */
+    uint32_t same_x;            /* the previous item of this workgroup staged the same input */
+    uint32_t pad[3];
+};
+
+/* the per-format pieces of the GEMV kernels (gemv_q8_0, gemv_legacy) under one name */
+template <int WHICH> struct MultiFmt {
+    typedef LegRegs Regs;
+    static constexpr uint32_t BYTES = LegGeom<WHICH ? WHICH : 1>::BYTES;
+};
+template <> struct MultiFmt<0> {
+    typedef Q80Regs Regs;
+    static constexpr uint32_t BYTES = 34u;
+};
+template <int WHICH>
+__device__ __forceinline__ void multi_load(typename MultiFmt<WHICH>::Regs &r, const WSrc &w, uint32_t g)
+{
+    if constexpr (WHICH == 0) q80_load<false>(r, w, g);
+    else leg_load<WHICH, false>(r, w, g);
+}
+template <int WHICH>
+__device__ __forceinline__ void
+multi_pass(const typename MultiFmt<WHICH>::Regs &r, const GemvParams &p, const uint8_t *lds, uint32_t act_lds,
+           uint32_t B, uint32_t g, uint32_t nblk, uint32_t row0, float *terms)
+{
+    if constexpr (WHICH == 0) q80_pass<1, false>(r, p, lds, act_lds, 1u, B, g, nblk, row0, terms);
+    else leg_pass<WHICH, 1, false>(r, p, lds, act_lds, 1u, B, g, nblk, row0, terms);
+}
+
+/* what a wave needs of one item: the launch parameters and its share of the rows */
+struct MultiState {
+    GemvParams p;
+    WaveWork ww;
+    WSrc src;
+    uint32_t nblk, same_x;
+};
+
+template <int WHICH>
+__device__ __forceinline__ MultiState multi_state(const GemvMultiItem *it, uint32_t wave)
+{
+    MultiState st;
+    st.p = it->p;
+    st.ww.seg = it->seg;
+    st.same_x = it->same_x;
+    st.ww.seg_index = 0u;
+    st.ww.wg_in_seg = 0u;
+    const uint32_t q = st.ww.seg.rows_q, rem = st.ww.seg.rows_rem;
+    st.ww.row0 = wave * q + min(wave, rem);
+    st.ww.nrows = q + (wave < rem ? 1u : 0u);
+    bool paired;
+    st.src = wsrc_for<false>(st.ww, nullptr, st.p.blocks, MultiFmt<WHICH>::BYTES, st.nblk, paired);
+    return st;
+}
+
+/* Operations that do not depend on each other (every input there when the launch starts) in ONE
+ * launch, split in space rather than in time: the rows of all operations are cut into runs and
+ * dealt to the workgroups so that every workgroup streams about the same number of bytes, and a
+ * workgroup walks its few runs with the GEMV kernel's own steps (input quantised into LDS, passes over
+ * two register sets, ordered row sums), requesting the next run's input and first two passes of
+ * weights before it sums the rows of the current one.  No workgroup waits for another.  The matrices
+ * of a Qwen2.5-0.5B-shaped Q8_0 model are 0.9-9 MB each: launched one by one a decode step of 97
+ * matmuls takes 540 us, of which the kernels stream for a fifth, and walking the operations one after
+ * the other with the whole grid still pays 3.5 us of staging, barrier, one pass and row sums per
+ * operation.  WHICH: 0 = Q8_0, 1..5 = the LEG of gemv_legacy (Q4_0, Q4_1, Q5_0, Q5_1, AL5_XS).  A row's
+ * arithmetic does not depend on who owns it: same bits as the launches one by one. */
+template <int WHICH>
+__global__ __launch_bounds__(GEMV_MAX_THREADS) void
+k_gemv_multi(const GemvMultiItem *__restrict__ items, const uint32_t *__restrict__ first)
+{
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    typedef typename MultiFmt<WHICH>::Regs Regs;
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+    const uint32_t i0 = first[blockIdx.x], i1 = first[blockIdx.x + 1u];
+    if (i0 >= i1) return;
+    MultiState cur = multi_state<WHICH>(items + i0, wave);
+    XAhead xr = stage_begin<2, GEMV_PRO_NONE>(cur.ww.seg, cur.p, nullptr, lds, q80_lds_bytes(cur.p.blocks), 1u);
+    Regs A, Bq;
+    {
+        const uint32_t last = cur.nblk ? cur.nblk - 1u : 0u;
+        multi_load<WHICH>(A, cur.src, min(lane, last));
+        multi_load<WHICH>(Bq, cur.src, min(64u + lane, last));
+    }
+    bool staged = false;
+    for (uint32_t i = i0; i < i1; i++) {
+        /* the next item's table entry, on its way while this one is staged and walked (the last item
+         * stands in for the one after it: what is requested for that is never used) */
+        const MultiState nxt = multi_state<WHICH>(items + min(i + 1u, i1 - 1u), wave);
+        const uint32_t B = cur.p.blocks, act_lds = q80_lds_bytes(B);
+        if (!(staged && cur.same_x))
+            stage_end<2, GEMV_PRO_NONE>(xr, cur.ww.seg, cur.p, cur.ww.wg_in_seg, lds, act_lds, 1u,
+                                        reinterpret_cast<float *>(lds + act_lds));
+        staged = true;
+        __syncthreads();
+        float *const terms = reinterpret_cast<float *>(lds + act_lds) + (size_t)wave * cur.p.rows_cap * cur.p.term_stride;
+        const uint32_t nblk = cur.nblk, last = nblk ? nblk - 1u : 0u, npass = (nblk + 63u) / 64u;
+        if (nblk != 0u) {
+            uint32_t k = 0;
+            while (k + 3u < npass) {
+                multi_pass<WHICH>(A, cur.p, lds, act_lds, B, k * 64u + lane, nblk, cur.ww.row0, terms);
+                multi_load<WHICH>(A, cur.src, min((k + 2u) * 64u + lane, last));
+                multi_pass<WHICH>(Bq, cur.p, lds, act_lds, B, (k + 1u) * 64u + lane, nblk, cur.ww.row0, terms);
+                multi_load<WHICH>(Bq, cur.src, min((k + 3u) * 64u + lane, last));
+                k += 2u;
+            }
+            const uint32_t rem = npass - k;                 /* 1, 2 or 3 */
+            multi_pass<WHICH>(A, cur.p, lds, act_lds, B, k * 64u + lane, nblk, cur.ww.row0, terms);
+            if (rem == 3u) multi_load<WHICH>(A, cur.src, min((k + 2u) * 64u + lane, last));
+            if (rem >= 2u) multi_pass<WHICH>(Bq, cur.p, lds, act_lds, B, (k + 1u) * 64u + lane, nblk, cur.ww.row0, terms);
+            if (rem == 3u) multi_pass<WHICH>(A, cur.p, lds, act_lds, B, (k + 2u) * 64u + lane, nblk, cur.ww.row0, terms);
+        }
+        /* the next item's input and first weights, requested before this one's rows are summed */
+        xr = stage_begin<2, GEMV_PRO_NONE>(nxt.ww.seg, nxt.p, nullptr, lds, q80_lds_bytes(nxt.p.blocks), 1u);
+        {
+            const uint32_t nlast = nxt.nblk ? nxt.nblk - 1u : 0u;
+            multi_load<WHICH>(A, nxt.src, min(lane, nlast));
+            multi_load<WHICH>(Bq, nxt.src, min(64u + lane, nlast));
+        }
+        row_sums<1>(terms, lane, 1u, cur.ww.nrows, cur.p.rows_cap, B, cur.p.term_stride, cur.ww.seg.out,
+                    cur.p.out_stride, cur.ww.row0);
+        __syncthreads();        /* the next item keeps its terms (and maybe its input) where this one's were */
+        cur = nxt;
+    }
+}
+
 /* ─── host side of layer 2 ────────────────────────────────────────────── */
 
 static hipError_t raise_all_lds_ceilings(void);
@@ -711,6 +841,12 @@ static hipError_t raise_all_lds_ceilings(void)
     OXH_RAISE(k_gemv_iq3_s)
     OXH_RAISE(k_gemv_iq1_xxxs)
 #undef OXH_RAISE
+    if ((e = raise_lds_ceiling(k_gemv_multi<0>)) != hipSuccess) return e;
+    if ((e = raise_lds_ceiling(k_gemv_multi<1>)) != hipSuccess) return e;
+    if ((e = raise_lds_ceiling(k_gemv_multi<2>)) != hipSuccess) return e;
+    if ((e = raise_lds_ceiling(k_gemv_multi<3>)) != hipSuccess) return e;
+    if ((e = raise_lds_ceiling(k_gemv_multi<4>)) != hipSuccess) return e;
+    if ((e = raise_lds_ceiling(k_gemv_multi<5>)) != hipSuccess) return e;
 #define OXH_RAISE_PRO1(KERNEL, PRO)                                                               \
     if ((e = raise_lds_ceiling(KERNEL<1, PRO, false>)) != hipSuccess) return e;                   \
     if ((e = raise_lds_ceiling(KERNEL<0, PRO, false>)) != hipSuccess) return e;                   \
@@ -1233,6 +1369,213 @@ extern "C" int oxh_gemv_segments_f32(uint32_t qtype, const OxhSegment *segs, siz
     if (!d_x && n_segs) return arg_fail("oxh_gemv_segments_f32: NULL input");
     const GemvIo io = { nullptr, d_x, x_stride, d_act_out, nullptr };
     return launch_gemv(qtype, segs, n_segs, cols, io, n_vec, out_stride, nullptr, stream);
+}
+
+/* ─── plans over the 32-value formats (oxh_plan_* hands them here) ────── */
+
+struct GemvMulti {
+    GemvMultiItem *d_items;
+    uint32_t *d_first;
+    uint32_t n_ops, n_items, grid;
+    int which;
+    size_t lds;
+};
+
+static int mmq80_leg(uint32_t qtype);
+
+extern "C" int oxh_internal_multi_which(uint32_t qtype)
+{
+    qtype = canon_qtype(qtype);
+    if (qtype == OXH_Q8_0) return 0;
+    const int leg = mmq80_leg(qtype);
+    return leg >= 1 ? leg : -1;
+}
+
+/* Cuts the rows of all operations into runs of at most 16 x rows_cap rows (what a workgroup's term
+ * tables hold) and deals them in order: a workgroup is full when it has its share of the bytes. */
+extern "C" int oxh_internal_multi_create(const OxhPlanOp *ops, size_t n_ops, void **handle)
+{
+    int rc = ensure_init();
+    if (rc) return rc;
+    if (!ops || !handle || n_ops == 0 || n_ops > 0xFFFFu) return arg_fail("plan: 1..65535 operations");
+    *handle = nullptr;
+    const int which = oxh_internal_multi_which(ops[0].qtype);
+    if (which < 0) {
+        snprintf(g_err, sizeof g_err, "plan: qtype %u has no multi-operation launch", ops[0].qtype);
+        return OXH_DECLINED;
+    }
+    const uint32_t W = GEMV_MAX_THREADS / 64u;
+    const uint32_t n_cu = (uint32_t)(g_n_cu > 0 ? g_n_cu : 256);
+    /* pass 1: check, and add up the bytes */
+    double total = 0.0;
+    for (size_t i = 0; i < n_ops; i++) {
+        const OxhPlanOp &o = ops[i];
+        if (oxh_internal_multi_which(o.qtype) != which || o.pro || !o.segs || o.n_segs == 0 || !o.d_x ||
+            oxh_act_kind(o.qtype, o.cols) != 1) {
+            snprintf(g_err, sizeof g_err, "plan: operation %zu: the operations of a plan over a 32-value format are of "
+                     "that one format (cols a multiple of 32), without prologue, with segments and an input", i);
+            return OXH_DECLINED;
+        }
+        const size_t blocks = o.cols / OXH_QK8_0;
+        if (blocks > 0xFFFFu || gemv_lds_bytes(o.qtype, (uint32_t)blocks, 1, W, 1) > GEMV_LDS_LIMIT) {
+            snprintf(g_err, sizeof g_err, "plan: operation %zu: cols %zu too wide for one workgroup", i, o.cols);
+            return OXH_ERR_TOO_WIDE;
+        }
+        size_t live = 0;
+        for (size_t k = 0; k < o.n_segs; k++) {
+            const OxhSegment &sg = o.segs[k];
+            if (!sg.rows) continue;
+            if (sg.act_first != 0 || sg.n_vec > 1 || sg.d_w_pair || !sg.d_w || !sg.d_out || sg.rows > 0x3FFFFFFFull)
+                return arg_fail("plan: segments over activation 0, one vector, unpaired, with matrix and output");
+            total += (double)sg.rows * (double)oxh_row_bytes(o.qtype, o.cols);
+            live++;
+        }
+        if (live == 0) return arg_fail("plan: an operation has no rows");
+    }
+    const double target = total / n_cu;
+    /* pass 2: the runs.  Sized generously first (a run has at least 16 rows unless the segment ends) */
+    size_t cap_items = 0;
+    for (size_t i = 0; i < n_ops; i++)
+        for (size_t k = 0; k < ops[i].n_segs; k++) cap_items += ops[i].segs[k].rows / 16u + 2u;
+    cap_items += n_cu;
+    GemvMultiItem *h = (GemvMultiItem *)calloc(cap_items, sizeof *h);
+    uint32_t *first = (uint32_t *)calloc(n_cu + 1u, sizeof *first);
+    if (!h || !first) {
+        free(h);
+        free(first);
+        snprintf(g_err, sizeof g_err, "out of host memory building a plan");
+        return OXH_ERR_NOMEM;
+    }
+    uint32_t wg = 0, n_items = 0;
+    double used = 0.0;
+    size_t lds = 0;
+    const void *prev_x = nullptr;
+    size_t prev_cols = 0;
+    bool wg_empty = true;
+    for (size_t i = 0; i < n_ops; i++) {
+        const OxhPlanOp &o = ops[i];
+        const uint32_t blocks = (uint32_t)(o.cols / OXH_QK8_0);
+        const size_t row_bytes = oxh_row_bytes(o.qtype, o.cols);
+        uint32_t cap = GEMV_ROWS_CAP;
+        while (cap > 1u && gemv_lds_bytes(o.qtype, blocks, 1, W, cap) > GEMV_LDS_LIMIT) cap--;
+        const size_t run_max = (size_t)W * cap;
+        bool op_first = true;
+        for (size_t k = 0; k < o.n_segs; k++) {
+            const OxhSegment &sg = o.segs[k];
+            size_t r = 0;
+            while (r < sg.rows) {
+                if (!wg_empty && used >= target && wg + 1u < n_cu) {        /* this workgroup has its share */
+                    wg++;
+                    first[wg] = n_items;
+                    used = 0.0;
+                    wg_empty = true;
+                    prev_x = nullptr;
+                }
+                size_t take = sg.rows - r;
+                if (take > run_max) take = run_max;
+                const double room = target - used;
+                size_t fit = room > 0.0 ? (size_t)(room / (double)row_bytes) : 0u;
+                fit = (fit + 15u) & ~(size_t)15u;                            /* whole rows per wave, rounded up */
+                if (fit < 16u) fit = 16u;
+                if (wg + 1u < n_cu && take > fit) take = fit;
+                GemvMultiItem &it = h[n_items++];
+                it.seg.w = (const uint8_t *)sg.d_w + r * row_bytes;
+                it.seg.out = sg.d_out + r;
+                it.seg.rows = (uint32_t)take;
+                it.seg.act_first = 0;
+                it.seg.wg_begin = 0;
+                it.seg.rows_q = (uint32_t)(take / W);
+                it.seg.rows_rem = (uint32_t)(take % W);
+                it.seg.nv = 1;
+                it.p.blocks = blocks;
+                it.p.magic = (uint32_t)((0x100000000ull + blocks - 1u) / blocks);
+                it.p.act_bytes = (uint32_t)oxh_act_bytes(o.qtype, o.cols);
+                it.p.out_stride = 0;
+                it.p.term_stride = terms_per_block(o.qtype) * blocks + 1u;
+                it.p.rows_cap = (uint32_t)((take + W - 1u) / W);
+                it.p.x = o.d_x;
+                it.p.x_stride = (uint32_t)o.cols;
+                it.p.act_out = op_first ? (uint8_t *)o.d_act_out : nullptr;
+                it.same_x = (!wg_empty && prev_x == (const void *)o.d_x && prev_cols == o.cols && !it.p.act_out) ? 1u : 0u;
+                const size_t need = gemv_lds_bytes(o.qtype, blocks, 1, W, it.p.rows_cap);
+                if (need > lds) lds = need;
+                op_first = false;
+                wg_empty = false;
+                prev_x = o.d_x;
+                prev_cols = o.cols;
+                used += (double)take * (double)row_bytes;
+                r += take;
+            }
+        }
+    }
+    const uint32_t grid = wg + 1u;
+    for (uint32_t b = grid; b <= n_cu; b++) first[b] = n_items;
+    first[grid] = n_items;
+    GemvMulti *m = (GemvMulti *)calloc(1, sizeof *m);
+    if (!m) { snprintf(g_err, sizeof g_err, "out of host memory building a plan"); rc = OXH_ERR_NOMEM; }
+    if (!rc) {
+        hipError_t e = hipMalloc((void **)&m->d_items, (size_t)n_items * sizeof *h);
+        if (e == hipSuccess) e = hipMalloc((void **)&m->d_first, (size_t)(grid + 1u) * sizeof *first);
+        if (e == hipSuccess) e = hipMemcpy(m->d_items, h, (size_t)n_items * sizeof *h, hipMemcpyHostToDevice);
+        if (e == hipSuccess) e = hipMemcpy(m->d_first, first, (size_t)(grid + 1u) * sizeof *first, hipMemcpyHostToDevice);
+        if (e != hipSuccess) {
+            if (m->d_items) (void)hipFree(m->d_items);
+            if (m->d_first) (void)hipFree(m->d_first);
+            free(m);
+            m = nullptr;
+            rc = hip_fail(e, "plan table");
+        }
+    }
+    free(h);
+    free(first);
+    if (rc) return rc;
+    m->n_ops = (uint32_t)n_ops;
+    m->n_items = n_items;
+    m->grid = grid;
+    m->which = which;
+    m->lds = lds;
+    *handle = m;
+    return OXH_OK;
+}
+
+extern "C" int oxh_internal_multi_launch(void *handle, void *stream)
+{
+    GemvMulti *m = (GemvMulti *)handle;
+    if (!m) return arg_fail("plan: NULL");
+    hipStream_t st = pick_stream(stream);
+    const dim3 grid(m->grid), block(GEMV_MAX_THREADS);
+#define OXH_MULTI(WHICH) hipLaunchKernelGGL((k_gemv_multi<WHICH>), grid, block, m->lds, st, m->d_items, m->d_first)
+    switch (m->which) {
+    case 1:  OXH_MULTI(1); break;
+    case 2:  OXH_MULTI(2); break;
+    case 3:  OXH_MULTI(3); break;
+    case 4:  OXH_MULTI(4); break;
+    case 5:  OXH_MULTI(5); break;
+    default: OXH_MULTI(0); break;
+    }
+#undef OXH_MULTI
+    HIP_TRY(hipGetLastError());
+    return OXH_OK;
+}
+
+extern "C" void oxh_internal_multi_info(const void *handle, size_t *n_items, size_t *workgroups, size_t *lds_bytes)
+{
+    const GemvMulti *m = (const GemvMulti *)handle;
+    if (n_items) *n_items = m->n_items;
+    if (workgroups) *workgroups = m->grid;
+    if (lds_bytes) *lds_bytes = m->lds;
+}
+
+extern "C" int oxh_internal_multi_destroy(void *handle)
+{
+    GemvMulti *m = (GemvMulti *)handle;
+    if (!m) return OXH_OK;
+    hipError_t e = hipFree(m->d_items);
+    const hipError_t e2 = hipFree(m->d_first);
+    free(m);
+    if (e == hipSuccess) e = e2;
+    if (e != hipSuccess) return hip_fail(e, "hipFree");
+    return OXH_OK;
 }
 
 extern "C" int oxh_gemv_segments_fused(uint32_t qtype, const OxhSegment *segs, size_t n_segs,

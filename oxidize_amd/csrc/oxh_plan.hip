@@ -959,6 +959,7 @@ struct OxhPlan {
     uint8_t *d_img;                 /* the staged inputs */
     PlanOp *d_run;                  /* k_plan_ext: the table it walks (d_ops stays the list of inputs) */
     uint32_t n_run;
+    void *multi;                    /* a plan over a 32-value format: the table of GEMV launches (oxh_kernels.hip) */
 };
 
 static const void *plan_kernel(const OxhPlan *pl)
@@ -1133,6 +1134,59 @@ static double plan_table_cost(const PlanOp *run, size_t n_run)
     return cost;
 }
 
+/* Q8_0, Q4_0, Q4_1, Q5_0, Q5_1, AL5_XS (and the aliases): the operations of one such format, none of
+ * which touches what another writes, become a table of GEMV launches walked by one grid
+ * (k_gemv_multi).  No workgroup waits for another there, so a plan with a dependency is declined. */
+static int plan_create_multi(const OxhPlanOp *ops, size_t n_ops, OxhPlan **out)
+{
+    for (size_t i = 0; i < n_ops; i++) {
+        const OxhPlanOp &o = ops[i];
+        if (!o.segs || o.n_segs == 0 || !o.d_x || o.cols == 0 || o.cols % OXH_QK8_0)
+            return oxh_internal_errorf(OXH_ERR_ARG, "invalid argument: plan: operation %zu has no segments, no input or "
+                                       "cols not a multiple of 32", i);
+        const Span xi = { (const char *)o.d_x, o.cols * sizeof(float) };
+        const Span ai = { (const char *)o.d_act_out, o.cols / OXH_QK8_0 * 34u };
+        for (size_t k = 0; k < o.n_segs; k++) {
+            const Span wk = { (const char *)o.segs[k].d_out, o.segs[k].rows * sizeof(float) };
+            if (spans_meet(wk, xi) || spans_meet(wk, ai) || spans_meet(ai, xi))
+                return oxh_internal_errorf(OXH_ERR_ARG, "invalid argument: plan: operation %zu stores over one of its own inputs", i);
+        }
+        for (size_t j = 0; j < i; j++) {
+            const OxhPlanOp &e = ops[j];
+            const Span xj = { (const char *)e.d_x, e.cols * sizeof(float) };
+            const Span aj = { (const char *)e.d_act_out, e.cols / OXH_QK8_0 * 34u };
+            bool hit = spans_meet(ai, xj) || spans_meet(aj, xi) || spans_meet(ai, aj);
+            for (size_t k = 0; k < o.n_segs && !hit; k++) {
+                const Span wk = { (const char *)o.segs[k].d_out, o.segs[k].rows * sizeof(float) };
+                hit = spans_meet(wk, xj) || spans_meet(wk, aj);
+                for (size_t m = 0; m < e.n_segs && !hit; m++) {
+                    const Span wm = { (const char *)e.segs[m].d_out, e.segs[m].rows * sizeof(float) };
+                    hit = spans_meet(wk, wm);
+                }
+            }
+            for (size_t m = 0; m < e.n_segs && !hit; m++) {
+                const Span wm = { (const char *)e.segs[m].d_out, e.segs[m].rows * sizeof(float) };
+                hit = spans_meet(wm, xi) || spans_meet(wm, ai);
+            }
+            if (hit)
+                return oxh_internal_errorf(OXH_DECLINED, "plan: operation %zu depends on operation %zu; plans over the "
+                                           "32-value formats run independent operations only", i, j);
+        }
+    }
+    void *multi = nullptr;
+    const int rc = oxh_internal_multi_create(ops, n_ops, &multi);
+    if (rc) return rc;
+    OxhPlan *pl = (OxhPlan *)calloc(1, sizeof *pl);
+    if (!pl) {
+        (void)oxh_internal_multi_destroy(multi);
+        return oxh_internal_errorf(OXH_ERR_NOMEM, "out of host memory building a plan");
+    }
+    pl->multi = multi;
+    pl->n_ops = (uint32_t)n_ops;
+    *out = pl;
+    return OXH_OK;
+}
+
 extern "C" int oxh_plan_create(const OxhPlanOp *ops, size_t n_ops, OxhPlan **out)
 {
     if (!out) return oxh_internal_errorf(OXH_ERR_ARG, "invalid argument: oxh_plan_create: NULL");
@@ -1141,6 +1195,7 @@ extern "C" int oxh_plan_create(const OxhPlanOp *ops, size_t n_ops, OxhPlan **out
     if (rc) return rc;
     if (!ops || n_ops == 0 || n_ops > 0xFFFFu)
         return oxh_internal_errorf(OXH_ERR_ARG, "invalid argument: oxh_plan_create: 1..65535 operations");
+    if (oxh_internal_multi_which(ops[0].qtype) >= 0) return plan_create_multi(ops, n_ops, out);
     const uint32_t n_cu = (uint32_t)(oxh_internal_n_cu() > 0 ? oxh_internal_n_cu() : 256);
     const uint32_t grid = n_cu > PLAN_MAX_WG ? PLAN_MAX_WG : n_cu;
 
@@ -1369,6 +1424,7 @@ extern "C" int oxh_plan_create(const OxhPlanOp *ops, size_t n_ops, OxhPlan **out
 extern "C" int oxh_plan_launch(OxhPlan *pl, void *stream)
 {
     if (!pl) return oxh_internal_errorf(OXH_ERR_ARG, "invalid argument: oxh_plan_launch: NULL plan");
+    if (pl->multi) return oxh_internal_multi_launch(pl->multi, stream);
     hipStream_t st = stream ? (hipStream_t)stream : (hipStream_t)oxh_internal_stream();
     PlanSync sy;
     sy.flags = pl->d_sync;
@@ -1411,12 +1467,19 @@ extern "C" int oxh_plan_info(const OxhPlan *pl, size_t *n_ops, size_t *n_waits, 
     if (n_waits) *n_waits = pl->n_waits;
     if (workgroups) *workgroups = pl->grid;
     if (lds_bytes) *lds_bytes = pl->lds_bytes;
+    if (pl->multi) oxh_internal_multi_info(pl->multi, nullptr, workgroups, lds_bytes);
     return OXH_OK;
 }
 
 extern "C" int oxh_plan_table_rows(const OxhPlan *pl)
 {
-    return pl ? (int)pl->n_run : -1;
+    if (!pl) return -1;
+    if (pl->multi) {
+        size_t items = 0;
+        oxh_internal_multi_info(pl->multi, &items, nullptr, nullptr);
+        return (int)items;
+    }
+    return (int)pl->n_run;
 }
 
 extern "C" int oxh_plan_prestaged(const OxhPlan *pl)
@@ -1444,6 +1507,7 @@ extern "C" int oxh_plan_status(OxhPlan *pl, void *stream)
     if (!pl) return oxh_internal_errorf(OXH_ERR_ARG, "invalid argument: oxh_plan_status: NULL plan");
     hipStream_t st = stream ? (hipStream_t)stream : (hipStream_t)oxh_internal_stream();
     PLAN_TRY(hipStreamSynchronize(st));
+    if (pl->multi) return OXH_OK;              /* nothing waits in such a plan */
     uint32_t go[4] = { 0, 0, 0, 0 };
     PLAN_TRY(hipMemcpy(go, pl->d_sync + PLAN_COPIES * PLAN_MAX_WG + 4u, sizeof go, hipMemcpyDeviceToHost));
     if (go[1] == 0u) return OXH_OK;
@@ -1458,6 +1522,7 @@ extern "C" int oxh_plan_destroy(OxhPlan *pl)
 {
     if (!pl) return OXH_OK;
     hipError_t e = hipDeviceSynchronize();
+    if (pl->multi) (void)oxh_internal_multi_destroy(pl->multi);
     if (pl->d_ops) (void)hipFree(pl->d_ops);
     if (pl->d_run) (void)hipFree(pl->d_run);
     if (pl->d_img) (void)hipFree(pl->d_img);

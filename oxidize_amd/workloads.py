@@ -16,28 +16,35 @@ from . import synth
 Q80, Q4K, Q6K = 7, 13, 16
 
 LLAMA3_8B = dict(hidden=4096, kv=1024, ffn=14336, layers=32)
+QWEN2_5_0_5B = dict(hidden=896, kv=128, ffn=4864, layers=24)
 
 
 class DecodeSet:
-    def __init__(self, hidden=4096, kv=1024, ffn=14336, layers=32, seed=0, keep_host=(), q6_grouped=None):
+    def __init__(self, hidden=4096, kv=1024, ffn=14336, layers=32, seed=0, keep_host=(), q6_grouped=None,
+                 qtypes=(Q4K, Q6K)):
         """q6_grouped: keep the Q6_K matrices resident in the regrouped layout the decode kernels read
         fastest (oxh_q6_k_group; same bytes, made once when the weights are loaded, as the host layer
-        does for registered weights).  Default: wherever the shape allows it (ffn % 2048 == 0)."""
+        does for registered weights).  Default: wherever the shape allows it (ffn % 2048 == 0).
+        qtypes: weight types of (q/k/v, o, gate/up) and of the down projection; (Q80, Q80) with
+        QWEN2_5_0_5B's shapes is the reference's Q8_0 configuration."""
         self.hidden, self.kv, self.ffn, self.layers = hidden, kv, ffn, layers
         self.seed = seed
+        qt_main, qt_down = qtypes
         if q6_grouped is None:
-            q6_grouped = ffn % 2048 == 0
-        elif q6_grouped and ffn % 2048:
-            raise ValueError("the regrouped Q6_K layout needs ffn to be a multiple of 2048")
+            q6_grouped = qt_down == Q6K and ffn % 2048 == 0
+        elif q6_grouped and (ffn % 2048 or qt_down != Q6K):
+            raise ValueError("the regrouped Q6_K layout needs Q6_K weights and ffn a multiple of 2048")
         self.q6_grouped = q6_grouped
-        self.qtype_run = {Q4K: Q4K, Q6K: mv.Q6_K_G8 if q6_grouped else Q6K}
+        self.qtype_run = {qt_main: qt_main, qt_down: qt_down}
+        if qt_down == Q6K:
+            self.qtype_run[Q6K] = mv.Q6_K_G8 if q6_grouped else Q6K
         staging = None
         # (name, qtype, [rows...], cols, input index)
         self.ops = [
-            ("qkv", Q4K, [hidden, kv, kv], hidden, 0),
-            ("o", Q4K, [hidden], hidden, 1),
-            ("gate_up", Q4K, [ffn, ffn], hidden, 2),
-            ("down", Q6K, [hidden], ffn, 3),
+            ("qkv", qt_main, [hidden, kv, kv], hidden, 0),
+            ("o", qt_main, [hidden], hidden, 1),
+            ("gate_up", qt_main, [ffn, ffn], hidden, 2),
+            ("down", qt_down, [hidden], ffn, 3),
         ]
         self.weights = []      # [layer][op] -> list of DeviceBuffer (one per segment)
         self.host = {}         # (layer, op, seg) -> numpy, for layers in keep_host

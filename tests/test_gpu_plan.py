@@ -242,7 +242,7 @@ def test_what_a_plan_declines(oxh):
     w = mv.DeviceBuffer(1 << 20)
     out = mv.DeviceBuffer(4 * 64)
     seg = mv.make_segments([(w.ptr, out.ptr, 8, 0)])
-    for qt, cols in ((Q80, 1024), (Q4K, 32768), (Q4K, 1000)):
+    for qt, cols in ((25, 1024), (8, 1024), (Q4K, 32768), (Q4K, 1000)):       # IQ3_S, Q2_K: no plan; too wide; not whole blocks
         with pytest.raises(mv.OxhError) as e:
             mv.Plan([dict(qtype=qt, segs=seg, cols=cols, d_x=x.ptr)])
         assert e.value.status == mv.DECLINED
@@ -346,4 +346,68 @@ def test_random_independent_plans_match_the_launches(oxh, seed):
             for k, name in enumerate(("out", "act", "prologue out", "sum out")):
                 a, c = np.ascontiguousarray(w_[k]).view(np.uint8), np.ascontiguousarray(g_[k]).view(np.uint8)
                 assert np.array_equal(a, c), (seed, rep, i, name, ops[i]["qtype"], ops[i]["cols"])
+    plan.destroy()
+
+
+@pytest.mark.parametrize("qtype", [7, 3, 4, 5, 6, 18])
+@pytest.mark.parametrize("hidden,kv,ffn,layers", [(896, 128, 4864, 3), (256, 64, 96, 2)])
+def test_plan_over_a_32_value_format_matches_single_launches(oxh, qtype, hidden, kv, ffn, layers):
+    """Operations of one 32-value format that do not depend on each other run as one launch whose
+    workgroups share out the rows of all of them: outputs and stored activations bit for bit those of
+    the launches one by one, launch after launch, and against the oracle for one matrix."""
+    d = DecodeSet(hidden=hidden, kv=kv, ffn=ffn, layers=layers, seed=5, keep_host=(0,), qtypes=(qtype, qtype))
+    d.launch_step()
+    mv.sync()
+    want_out = [[d.output(l, op) for op in range(4)] for l in range(layers)]
+    want_act = [[d.activation(l, op) for op in range(4)] for l in range(layers)]
+    plan = mv.Plan(d.plan_ops())
+    info = plan.info()
+    # the rows of all operations are cut into runs and dealt to the workgroups: at least a run per operation
+    assert info["n_ops"] == 4 * layers and info["n_waits"] == 0 and info["table_rows"] >= 4 * layers
+    for rep in range(3):
+        for l in range(layers):
+            for op in range(4):
+                mv.lib().oxh_memset(ctypes.c_void_p(d.out[l][op].ptr), 0xFF, d.out[l][op].nbytes, None)
+                mv.lib().oxh_memset(ctypes.c_void_p(d.act[l][op].ptr), 0xFF, d.act[l][op].nbytes, None)
+        plan.launch()
+        assert plan.status() == 0
+        for l in range(layers):
+            for op in range(4):
+                assert np.array_equal(bits(d.output(l, op)), bits(want_out[l][op])), (rep, l, op)
+                assert np.array_equal(d.activation(l, op), want_act[l][op]), (rep, l, op)
+    plan.destroy()
+    o = oxlibs.oracle()
+    name, qt, rows, cols, _ = d.ops[3]
+    w, x = d.host[(0, 3, 0)], d.x_host[(0, 3)]
+    want = np.zeros(rows[0], np.float32)
+    tmp = np.zeros(cols, np.float32)
+    assert o.oxo_matvec_quantized(qt, w.ctypes.data, rows[0], cols, synth.row_bytes(qt, cols), x.ctypes.data,
+                                  want.ctypes.data, tmp.ctypes.data) == 0
+    assert np.array_equal(bits(want_out[0][3]), bits(want))
+
+
+def test_plan_over_a_32_value_format_declines_a_dependency(oxh):
+    """No workgroup waits for another in such a plan, so an operation that reads what an earlier one
+    writes cannot be part of it; nor can one of another weight format."""
+    rows, cols = 256, 256
+    w = mv.DeviceBuffer.from_host(synth.weights(7, rows, cols, seed=1))
+    x = mv.DeviceBuffer.from_host(synth.normal(cols, seed=1))
+    y = mv.DeviceBuffer(rows * 4)
+    z = mv.DeviceBuffer(rows * 4)
+    first = dict(qtype=7, segs=mv.make_segments([(w.ptr, y.ptr, rows, 0)]), cols=cols, d_x=x.ptr, d_act_out=None)
+    second = dict(qtype=7, segs=mv.make_segments([(w.ptr, z.ptr, rows, 0)]), cols=cols, d_x=y.ptr, d_act_out=None)
+    with pytest.raises(mv.OxhError) as e:
+        mv.Plan([first, second])
+    assert e.value.status == mv.DECLINED
+    w4 = mv.DeviceBuffer.from_host(synth.weights(13, rows, cols, seed=1))
+    other = dict(qtype=13, segs=mv.make_segments([(w4.ptr, z.ptr, rows, 0)]), cols=cols, d_x=x.ptr, d_act_out=None)
+    with pytest.raises(mv.OxhError) as e:
+        mv.Plan([first, other])
+    assert e.value.status == mv.DECLINED
+    independent = dict(qtype=7, segs=mv.make_segments([(w.ptr, z.ptr, rows, 0)]), cols=cols, d_x=x.ptr, d_act_out=None)
+    plan = mv.Plan([first, independent])
+    plan.launch()
+    assert plan.status() == 0
+    a, b = y.download(np.float32, rows), z.download(np.float32, rows)
+    assert np.array_equal(bits(a), bits(b)) and np.any(a != 0)
     plan.destroy()
