@@ -218,9 +218,9 @@ int oxh_gemv_segments_fused(uint32_t qtype, const OxhSegment *segs, size_t n_seg
  * An operation is what one oxh_gemv_segments_fused call describes: up to four
  * non-empty segments (each over activation 0, one vector; d_w_pair allowed),
  * the f32 input, an optional prologue, an optional store of the quantised
- * bytes.  Types: Q4_K, Q5_K, Q6_K; cols a multiple of 256 up to 16384.
- * Anything else makes oxh_plan_create return OXH_DECLINED (launch those
- * matmuls one by one).  Results are bit-identical to the same calls made one
+ * bytes.  Types: Q4_K, Q5_K, Q6_K; cols a multiple of 256 up to 16384 (the
+ * 32-value formats: see below).  Anything else makes oxh_plan_create return
+ * OXH_DECLINED (launch those matmuls one by one).  Results are bit-identical to the same calls made one
  * after the other.
  *
  * Dependencies are found from the addresses: an operation that reads or
@@ -246,6 +246,16 @@ int oxh_gemv_segments_fused(uint32_t qtype, const OxhSegment *segs, size_t n_seg
  * environment: OXH_PLAN_PRESTAGE=0 keeps such a plan on the chained kernel,
  * OXH_PLAN_MERGE=0 keeps every operation on its own, OXH_PLAN_MERGE=1 merges
  * neighbours only, within four segments and three passes per wave).
+ *
+ * Plans over the 32-value formats: when the first operation's type is Q8_0,
+ * Q4_0, Q4_1, Q5_0, Q5_1, AL5_XS or one of their aliases, every operation must
+ * be of that same type (cols a multiple of 32), without prologue and unpaired,
+ * any number of segments, and NO operation may touch what another writes
+ * (OXH_DECLINED otherwise: nothing waits in such a launch).  The rows of all
+ * operations are cut into runs and dealt to the workgroups so that each streams
+ * the same number of bytes; a workgroup walks its runs with the GEMV kernel's
+ * own steps.  Same bits as the calls one by one.  oxh_plan_table_rows gives
+ * the number of runs; nothing of the residency rule below applies.
  *
  * All workgroups must be resident together (one per compute unit; the kernel
  * needs the whole device, so do not run other kernels beside a plan launch).
