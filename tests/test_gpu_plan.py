@@ -411,3 +411,31 @@ def test_plan_over_a_32_value_format_declines_a_dependency(oxh):
     a, b = y.download(np.float32, rows), z.download(np.float32, rows)
     assert np.array_equal(bits(a), bits(b)) and np.any(a != 0)
     plan.destroy()
+
+
+@pytest.mark.parametrize("qtype", [7, 5])
+def test_plan_over_a_32_value_format_with_several_runs_of_one_input_per_workgroup(oxh, qtype):
+    """300 000 short rows: every workgroup gets three runs of the one operation (a run is at most 16 x 32
+    rows) and stages the input once; a second operation over another input follows in the same launch."""
+    rows, cols = 300000, 32
+    w = mv.DeviceBuffer.from_host(synth.weights(qtype, rows, cols, seed=9))
+    xs = [mv.DeviceBuffer.from_host(synth.normal(cols, seed=10 + k)) for k in range(2)]
+    want = []
+    for k in range(2):
+        o = mv.DeviceBuffer(rows * 4)
+        mv.gemv_segments_f32(qtype, mv.make_segments([(w.ptr, o.ptr, rows, 0)]), cols, xs[k].ptr, cols, None, 1, rows)
+        want.append(o.download(np.float32, rows))
+        o.free()
+    outs = [mv.DeviceBuffer(rows * 4) for _ in range(2)]
+    plan = mv.Plan([dict(qtype=qtype, segs=mv.make_segments([(w.ptr, outs[k].ptr, rows, 0)]), cols=cols,
+                         d_x=xs[k].ptr, d_act_out=None) for k in range(2)])
+    assert plan.info()["table_rows"] > 2 * 256
+    for rep in range(2):
+        for o in outs:
+            mv.lib().oxh_memset(ctypes.c_void_p(o.ptr), 0xFF, o.nbytes, None)
+        plan.launch()
+        assert plan.status() == 0
+        for k in range(2):
+            assert np.array_equal(bits(outs[k].download(np.float32, rows)), bits(want[k])), (rep, k)
+    assert np.any(want[0] != want[1])
+    plan.destroy()
