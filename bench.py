@@ -503,6 +503,32 @@ def traffic_probe(mv, ds):
     assert plan.status() == 0
 
 
+def q80_step_probe(mv, synth):
+    """For `rocprofv3 --pmc FETCH_SIZE` / `WRITE_SIZE` runs on k_gemv_multi: three 256 MiB device-to-device
+    copies (a kernel of known traffic to scale the counters by), then three launches of the
+    Qwen2.5-0.5B-shaped Q8_0 decode step as one plan.  Prints nothing."""
+    import ctypes
+    from oxidize_amd import _lib
+    from oxidize_amd.workloads import DecodeSet, QWEN2_5_0_5B
+    Q80 = 7
+    n = 256 << 20
+    a, b = mv.DeviceBuffer(n), mv.DeviceBuffer(n)
+    _lib.check(_lib.lib().oxh_memset(ctypes.c_void_p(a.ptr), 1, n, None))
+    for _ in range(3):
+        _lib.check(_lib.lib().oxh_memcpy_d2d(ctypes.c_void_p(b.ptr), ctypes.c_void_p(a.ptr), n, None))
+    mv.sync()
+    rows, cols = 151936, 896
+    qs = DecodeSet(qtypes=(Q80, Q80), seed=0, **QWEN2_5_0_5B)
+    d_head = mv.DeviceBuffer.from_host(synth.weights(Q80, rows, cols, seed=0, stream=5))
+    d_hx = mv.DeviceBuffer.from_host(synth.normal(cols, seed=0, stream=8))
+    d_ho = mv.DeviceBuffer(rows * 4)
+    head_seg = mv.make_segments([(d_head.ptr, d_ho.ptr, rows, 0)])
+    plan = mv.Plan(qs.plan_ops() + [dict(qtype=Q80, segs=head_seg, cols=cols, d_x=d_hx.ptr, d_act_out=None)])
+    for _ in range(3):
+        plan.launch()
+    assert plan.status() == 0
+
+
 def mmq_probe(mv, synth):
     """For `rocprofv3 --pmc` runs on the MFMA kernel: quantise 512 activations
     of 4096 values, then three 14336 x 4096 x 512 launches.  Prints nothing."""
@@ -603,7 +629,7 @@ def main():
     ap.add_argument("--mode", choices=["plan", "graph", "launches"], default="plan",
                     help="a step as one persistent launch (default), as a HIP graph of 128 launches, or as 128 launches")
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary configurations")
-    ap.add_argument("--probe", choices=["traffic", "mmq"], help="run a counter-collection workload and exit")
+    ap.add_argument("--probe", choices=["traffic", "mmq", "q80step"], help="run a counter-collection workload and exit")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this path is built and measured on ONE GPU; --gpus %d is not supported "
@@ -621,6 +647,10 @@ def main():
     if args.probe == "mmq":
         from oxidize_amd import synth
         mmq_probe(mv, synth)
+        return 0
+    if args.probe == "q80step":
+        from oxidize_amd import synth
+        q80_step_probe(mv, synth)
         return 0
 
     ds = DecodeSet(layers=args.layers, seed=0)
