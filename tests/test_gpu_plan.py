@@ -439,3 +439,64 @@ def test_plan_over_a_32_value_format_with_several_runs_of_one_input_per_workgrou
             assert np.array_equal(bits(outs[k].download(np.float32, rows)), bits(want[k])), (rep, k)
     assert np.any(want[0] != want[1])
     plan.destroy()
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_random_plans_over_a_32_value_format_match_the_launches(oxh, seed):
+    """Seeded random plans over one of the six 32-value formats: one to six segments of ragged sizes (a
+    single row, fewer rows than waves, more rows than a run holds), vector lengths from one block to 150,
+    some operations sharing an input, some storing their quantised activation; each operation is also
+    launched on its own and every output and stored activation compared bit for bit, on two launches with
+    new inputs in between."""
+    rng = np.random.default_rng(7000 + seed)
+    qt = int([7, 3, 4, 5, 6, 18][seed % 6])
+    n_ops = int(rng.integers(2, 14))
+    ops, bufs = [], []
+    shared_x = None
+    for i in range(n_ops):
+        cols = 32 * int(rng.choice([1, 3, 28, 64, 128, 150]))
+        rb = synth.row_bytes(qt, cols)
+        n_seg = int(rng.integers(1, 7))
+        seg_rows = [int(rng.choice([1, 5, 17, 100, 700, 3000, int(rng.integers(1, 9000))])) for _ in range(n_seg)]
+        total = sum(seg_rows)
+        w = mv.DeviceBuffer.from_host(synth.weights(qt, total, cols, seed=seed, stream=100 + i))
+        if shared_x is not None and shared_x[1] == cols and rng.random() < 0.5:
+            x = shared_x[0]
+        else:
+            x = mv.DeviceBuffer(cols * 4)
+            shared_x = (x, cols)
+        b = dict(w=w, x=x, out=mv.DeviceBuffer(total * 4), act=mv.DeviceBuffer(mv.act_bytes(qt, cols)), cols=cols,
+                 n_out=total, store=rng.random() < 0.5)
+        items, row = [], 0
+        for r in seg_rows:
+            items.append((w.ptr + row * rb, b["out"].ptr + row * 4, r, 0))
+            row += r
+        b["segs"] = mv.make_segments(items)
+        ops.append(dict(qtype=qt, segs=b["segs"], cols=cols, d_x=x.ptr, d_act_out=b["act"].ptr if b["store"] else None))
+        bufs.append(b)
+    plan = mv.Plan(ops)
+    assert plan.info()["n_ops"] == n_ops and plan.info()["n_waits"] == 0
+    for rep in range(2):
+        seen = set()
+        for i, b in enumerate(bufs):
+            if b["x"].ptr not in seen:
+                b["x"].upload(synth.normal(b["cols"], seed=seed, stream=500 + 20 * rep + i))
+                seen.add(b["x"].ptr)
+        want = []
+        for b in bufs:
+            mv.lib().oxh_memset(ctypes.c_void_p(b["act"].ptr), 0xEE, b["act"].nbytes, None)
+            mv.gemv_segments_f32(qt, b["segs"], b["cols"], b["x"].ptr, b["cols"], b["act"].ptr, 1, 0)
+            want.append((b["out"].download(np.float32, b["n_out"]), b["act"].download(np.uint8, b["act"].nbytes)))
+        for b in bufs:
+            mv.lib().oxh_memset(ctypes.c_void_p(b["out"].ptr), 0xFF, b["out"].nbytes, None)
+            mv.lib().oxh_memset(ctypes.c_void_p(b["act"].ptr), 0xEE, b["act"].nbytes, None)
+        plan.launch()
+        assert plan.status() == 0
+        for i, b in enumerate(bufs):
+            assert np.array_equal(bits(b["out"].download(np.float32, b["n_out"])), bits(want[i][0])), (rep, i)
+            got_act = b["act"].download(np.uint8, b["act"].nbytes)
+            if b["store"]:
+                assert np.array_equal(got_act, want[i][1]), (rep, i)
+            else:
+                assert np.all(got_act == 0xEE), (rep, i)
+    plan.destroy()
