@@ -340,6 +340,20 @@ int oxh_mmq_ex(uint32_t qtype, const void *d_w, size_t rows, size_t cols,
                const void *d_acts, size_t n_vec, float *d_out, size_t out_stride,
                uint32_t flags, void *stream);
 
+/* oxh_mmq for launches of few tiles over many columns (a 4096 x 14336 down projection under 5-64
+ * activations): a tile's workgroup walks all super-blocks of its rows at about a microsecond each, so
+ * with fewer than half a 64 x 16 tile per compute unit the launch is paced by that walk.  Here several
+ * workgroups share a tile's columns, every super-block's terms go to a workspace of
+ * cols/256 x n_vec x out_stride floats and a second launch adds them up in block order: the order the
+ * single workgroup adds them in, so the same bits.  oxh_mmq_split_workspace returns the bytes needed, or 0
+ * for a launch that would not be split (other types, more tiles, fewer than eight super-blocks, more than
+ * 64 activations); oxh_mmq_split with a smaller workspace, or none, is oxh_mmq.
+ * The reference has no counterpart (its batch kernel gives every worker whole rows, oxk.c:787-836). */
+size_t oxh_mmq_split_workspace(uint32_t qtype, size_t rows, size_t cols, size_t n_vec, size_t out_stride);
+int oxh_mmq_split(uint32_t qtype, const void *d_w, size_t rows, size_t cols,
+                  const void *d_acts, size_t n_vec, float *d_out, size_t out_stride,
+                  void *d_workspace, size_t workspace_bytes, void *stream);
+
 /* The tile (weight rows x activations per workgroup) oxh_mmq picks for a launch
  * on a device of n_cu compute units: the largest of 256 x 128 (128 x 128 for
  * Q5_K, Q6_K and widened Q2_K), 64 x 128 (Q6_K only), 128 x 64, 64 x 32, 64 x 16

@@ -77,6 +77,8 @@ SIGNATURES = {
     "oxh_mmq": (I, [U32, V, Z, Z, V, Z, V, Z, V]),
     "oxh_mmq_ex": (I, [U32, V, Z, Z, V, Z, V, Z, U32, V]),
     "oxh_mmq_tile": (I, [U32, Z, Z, Z, ctypes.POINTER(U32), ctypes.POINTER(U32)]),
+    "oxh_mmq_split_workspace": (Z, [U32, Z, Z, Z, Z]),
+    "oxh_mmq_split": (I, [U32, V, Z, Z, V, Z, V, Z, V, Z, V]),
     "oxh_get_rows": (I, [U32, V, Z, Z, V, Z, V, Z, V]),
     "oxh_debug_subblock_sums": (I, [U32, V, Z, Z, V, V, V]),
     "oxh_debug_read_probe": (I, [V, Z, V, V]),

@@ -507,7 +507,7 @@ typedef struct {
     size_t bytes;
 } DevBuf;
 
-static DevBuf g_dx, g_dact, g_dout;
+static DevBuf g_dx, g_dact, g_dout, g_dsplit;
 
 /* Page-locked host staging for the decode-sized entry points: the caller's
  * vectors are ordinary pageable memory, and a copy between pageable memory and
@@ -553,7 +553,7 @@ void oxh_internal_host_reset(void)
     pthread_mutex_lock(&g_lock);
     (void)clear_locked();
     pthread_mutex_unlock(&g_lock);
-    DevBuf *dv[] = { &g_dx, &g_dact, &g_dout };
+    DevBuf *dv[] = { &g_dx, &g_dact, &g_dout, &g_dsplit };
     for (size_t i = 0; i < sizeof dv / sizeof dv[0]; i++) {
         if (dv[i]->p) (void)oxh_free(dv[i]->p);
         dv[i]->p = NULL;
@@ -914,8 +914,17 @@ static int mv_batch(uint32_t qtype, const uint8_t *data, size_t rows,
     /* More vectors than the GEMV kernel keeps in flight: Q4_K, Q5_K and Q6_K go to the
      * int8-MFMA kernel behind a stand-alone quantiser launch; everything else
      * walks the batch in GEMV-sized slices (every output is the same dot either way). */
-    if (n_vec > 8 && (qtype == OXH_Q4_K_S || qtype == OXH_Q4_K_M || qtype == OXH_Q5_K_S ||
-                      qtype == OXH_Q5_K_M || qtype == OXH_Q6_K)) {
+    const bool kq456 = qtype == OXH_Q4_K_S || qtype == OXH_Q4_K_M || qtype == OXH_Q5_K_S || qtype == OXH_Q5_K_M ||
+                       qtype == OXH_Q6_K;
+    /* few rows, many columns, seven activations or more: the tiles' columns shared between workgroups
+     * (up to six the dot kernels are as fast: 4096 x 14336 Q6_K 24.7 us at six, 43 at eight, 28 split) */
+    const size_t split_ws = (kq456 && n_vec >= 7) ? oxh_mmq_split_workspace(qtype, rows, cols, n_vec, rows) : 0;
+    if (split_ws) {
+        if ((rc = reserve(&g_dsplit, split_ws))) return rc;
+        if ((rc = quantize(kind, d_x, cols, n_vec, cols, g_dact.p))) return rc;
+        if ((rc = oxh_mmq_split(qtype, d_w, rows, cols, g_dact.p, n_vec, d_out, rows, g_dsplit.p, g_dsplit.bytes, NULL)))
+            return rc;
+    } else if (n_vec > 8 && kq456) {
         if ((rc = quantize(kind, d_x, cols, n_vec, cols, g_dact.p))) return rc;
         if ((rc = oxh_mmq_ex(qtype, d_w, rows, cols, g_dact.p, n_vec, d_out, rows,
                              mmq_relaxed_enabled() ? OXH_MMQ_RELAXED : 0u, NULL)))

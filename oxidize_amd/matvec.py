@@ -186,6 +186,17 @@ def mmq(qtype, d_w, rows, cols, d_acts, n_vec, d_out, out_stride, stream=None, f
                         n_vec, ctypes.c_void_p(d_out), out_stride, stream))
 
 
+def mmq_split_workspace(qtype, rows, cols, n_vec, out_stride):
+    """Bytes of workspace with which mmq_split shares a tile's columns between workgroups; 0 = it would not."""
+    return int(lib().oxh_mmq_split_workspace(qtype, rows, cols, n_vec, out_stride))
+
+
+def mmq_split(qtype, d_w, rows, cols, d_acts, n_vec, d_out, out_stride, d_ws, ws_bytes, stream=None):
+    check(lib().oxh_mmq_split(qtype, ctypes.c_void_p(d_w), rows, cols, ctypes.c_void_p(d_acts), n_vec,
+                              ctypes.c_void_p(d_out), out_stride, ctypes.c_void_p(d_ws) if d_ws else None, ws_bytes,
+                              stream))
+
+
 def mmq_tile(qtype, rows, n_vec, n_cu):
     """(rows, tokens) of the workgroup tile oxh_mmq would take; host arithmetic only."""
     r, t = ctypes.c_uint32(0), ctypes.c_uint32(0)

@@ -283,3 +283,40 @@ def test_mmq_relaxed_mode_is_opt_in_and_within_tolerance(oxh, qtype, rows, cols,
         assert np.array_equal(bits(exact), bits(relaxed))
     assert mv.lib().oxh_mmq_ex(qtype, ctypes.c_void_p(d_w.ptr), rows, cols, ctypes.c_void_p(d_a.ptr), n_vec,
                                ctypes.c_void_p(d_w.ptr), rows, 2, None) != 0           # unknown flag
+
+
+@pytest.mark.parametrize("qt", [13, 15, 16])
+@pytest.mark.parametrize("rows,cols,n_vec", [(4096, 14336, 16), (1000, 4096, 5), (70, 2048, 40), (64, 8192, 64),
+                                             (3000, 2304, 17)])
+def test_mmq_with_a_tile_s_columns_shared_between_workgroups(oxh, qt, rows, cols, n_vec):
+    """oxh_mmq_split: every super-block's terms go to a workspace and are added in block order by a second
+    launch: bit for bit what oxh_mmq gives, padding between rows and out_stride untouched, and without a
+    workspace (or for a launch that would not be split) it is oxh_mmq."""
+    out_stride = rows + 3
+    w = mv.DeviceBuffer.from_host(synth.weights(qt, rows, cols, seed=rows, stream=qt))
+    x = mv.DeviceBuffer.from_host(synth.normal(n_vec * cols, seed=n_vec, stream=qt))
+    a = mv.DeviceBuffer(n_vec * mv.act_bytes(qt, cols))
+    mv.quantize(qt, x.ptr, cols, n_vec, cols, a.ptr)
+    want = mv.DeviceBuffer(n_vec * out_stride * 4)
+    got = mv.DeviceBuffer(n_vec * out_stride * 4)
+    for b in (want, got):
+        mv.lib().oxh_memset(ctypes.c_void_p(b.ptr), 0x7F, b.nbytes, None)
+    mv.mmq(qt, w.ptr, rows, cols, a.ptr, n_vec, want.ptr, out_stride)
+    need = mv.mmq_split_workspace(qt, rows, cols, n_vec, out_stride)
+    full = cols // 256 * n_vec * out_stride * 4
+    assert need == (full if (rows, cols) in ((4096, 14336), (1000, 4096), (64, 8192)) else 0)     # the others: too little to save
+    ws = mv.DeviceBuffer(full)
+    need = full                     # a launch that would not be split ignores the workspace
+    mv.mmq_split(qt, w.ptr, rows, cols, a.ptr, n_vec, got.ptr, out_stride, ws.ptr, need)
+    a_, b_ = want.download(np.uint32, n_vec * out_stride), got.download(np.uint32, n_vec * out_stride)
+    assert np.array_equal(a_, b_)
+    assert np.all(a_.reshape(n_vec, out_stride)[:, rows:] == 0x7F7F7F7F)
+    # no workspace: the plain launch
+    mv.lib().oxh_memset(ctypes.c_void_p(got.ptr), 0x7F, got.nbytes, None)
+    mv.mmq_split(qt, w.ptr, rows, cols, a.ptr, n_vec, got.ptr, out_stride, None, 0)
+    assert np.array_equal(a_, got.download(np.uint32, n_vec * out_stride))
+    # launches that are not split: many tiles, few super-blocks, a long batch
+    assert mv.mmq_split_workspace(qt, 28672, 4096, 16, 28672) == 0
+    assert mv.mmq_split_workspace(qt, 4096, 1024, 16, 4096) == 0
+    assert mv.mmq_split_workspace(qt, 4096, 14336, 512, 4096) == 0
+    assert mv.mmq_split_workspace(7, 4096, 4096, 16, 4096) == 0
