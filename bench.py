@@ -334,6 +334,47 @@ def secondary_figures(mv, synth):
     from oxidize_amd import _lib
     _lib.check(_lib.lib().oxh_weight_clear())
     out["host_pointer_api_us_per_call"] = host_api
+    # small batches over the decode matrices with few rows: the dot kernels (up to eight activations), one
+    # workgroup per 64 x 16 tile (oxh_mmq), and the tiles' columns shared between workgroups (oxh_mmq_split)
+    small = {}
+    for name, qt, r_, c_ in (("q6_k_4096x14336", Q6K, 4096, 14336), ("q4_k_4096x4096", Q4K, 4096, 4096)):
+        w = synth.weights(qt, r_, c_, seed=0, stream=12)
+        copies = [mv.DeviceBuffer.from_host(w) for _ in range(6)]
+        per = {}
+        for nv in (4, 8, 16):
+            d_x = mv.DeviceBuffer.from_host(synth.normal(nv * c_, seed=0, stream=2011))
+            d_a = mv.DeviceBuffer(nv * mv.act_bytes(qt, c_))
+            d_o = mv.DeviceBuffer(nv * r_ * 4)
+            mv.quantize(qt, d_x.ptr, c_, nv, c_, d_a.ptr)
+            need = mv.mmq_split_workspace(qt, r_, c_, nv, r_)
+            d_ws = mv.DeviceBuffer(max(need, 16))
+            segs = [mv.make_segments([(c.ptr, d_o.ptr, r_, 0)]) for c in copies]
+            state = {"i": 0}
+
+            def run_dot():
+                state["i"] += 1
+                mv.gemv_segments(qt, segs[state["i"] % 6], c_, d_a.ptr, nv, r_)
+
+            def run_tiles():
+                state["i"] += 1
+                mv.mmq(qt, copies[state["i"] % 6].ptr, r_, c_, d_a.ptr, nv, d_o.ptr, r_)
+
+            def run_split():
+                state["i"] += 1
+                mv.mmq_split(qt, copies[state["i"] % 6].ptr, r_, c_, d_a.ptr, nv, d_o.ptr, r_, d_ws.ptr, need)
+
+            row = {"one_workgroup_per_tile_us": round(timed(run_tiles, 24, mv), 1)}
+            if nv <= 8:
+                row["dot_kernel_us"] = round(timed(run_dot, 24, mv), 1)
+            if need:
+                row["columns_shared_us"] = round(timed(run_split, 24, mv), 1)
+            per["batch%d" % nv] = row
+            for b_ in (d_x, d_a, d_o, d_ws):
+                b_.free()
+        small[name] = per
+        for c in copies:
+            c.free()
+    out["small_batches_few_rows"] = small
     # the Q6_K down projection in the two layouts the decode kernels read: the file layout and the
     # regrouped copy the decode set keeps (same bytes); eight distinct copies in turn (386 MB: from HBM)
     rows, cols = 4096, 14336
