@@ -570,6 +570,28 @@ def q80_step_probe(mv, synth):
     assert plan.status() == 0
 
 
+def split_probe(mv, synth):
+    """For `rocprofv3 --kernel-trace --stats` runs on the small-batch launches whose tiles share their
+    columns between workgroups: a 4096 x 14336 Q6_K matrix under 16 activations, twelve launches of
+    oxh_mmq and twelve of oxh_mmq_split over six copies of the weights in turn.  Prints nothing."""
+    Q6K = 16
+    rows, cols, n_vec = 4096, 14336, 16
+    w = synth.weights(Q6K, rows, cols, seed=0, stream=12)
+    copies = [mv.DeviceBuffer.from_host(w) for _ in range(6)]
+    d_x = mv.DeviceBuffer.from_host(synth.normal(n_vec * cols, seed=0, stream=2011))
+    d_a = mv.DeviceBuffer(n_vec * mv.act_bytes(Q6K, cols))
+    d_o = mv.DeviceBuffer(n_vec * rows * 4)
+    mv.quantize(Q6K, d_x.ptr, cols, n_vec, cols, d_a.ptr)
+    need = mv.mmq_split_workspace(Q6K, rows, cols, n_vec, rows)
+    assert need
+    d_ws = mv.DeviceBuffer(need)
+    for i in range(12):
+        mv.mmq(Q6K, copies[i % 6].ptr, rows, cols, d_a.ptr, n_vec, d_o.ptr, rows)
+    for i in range(12):
+        mv.mmq_split(Q6K, copies[i % 6].ptr, rows, cols, d_a.ptr, n_vec, d_o.ptr, rows, d_ws.ptr, need)
+    mv.sync()
+
+
 def mmq_probe(mv, synth):
     """For `rocprofv3 --pmc` runs on the MFMA kernel: quantise 512 activations
     of 4096 values, then three 14336 x 4096 x 512 launches.  Prints nothing."""
@@ -670,7 +692,7 @@ def main():
     ap.add_argument("--mode", choices=["plan", "graph", "launches"], default="plan",
                     help="a step as one persistent launch (default), as a HIP graph of 128 launches, or as 128 launches")
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary configurations")
-    ap.add_argument("--probe", choices=["traffic", "mmq", "q80step"], help="run a counter-collection workload and exit")
+    ap.add_argument("--probe", choices=["traffic", "mmq", "q80step", "split"], help="run a counter-collection workload and exit")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this path is built and measured on ONE GPU; --gpus %d is not supported "
@@ -688,6 +710,10 @@ def main():
     if args.probe == "mmq":
         from oxidize_amd import synth
         mmq_probe(mv, synth)
+        return 0
+    if args.probe == "split":
+        from oxidize_amd import synth
+        split_probe(mv, synth)
         return 0
     if args.probe == "q80step":
         from oxidize_amd import synth
