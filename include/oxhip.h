@@ -346,8 +346,9 @@ int oxh_mmq_ex(uint32_t qtype, const void *d_w, size_t rows, size_t cols,
  * workgroups share a tile's columns, every super-block's terms go to a workspace of
  * cols/256 x n_vec x out_stride floats and a second launch adds them up in block order: the order the
  * single workgroup adds them in, so the same bits.  oxh_mmq_split_workspace returns the bytes needed, or 0
- * for a launch that would not be split (other types, more tiles, fewer than eight super-blocks, more than
- * 64 activations); oxh_mmq_split with a smaller workspace, or none, is oxh_mmq.
+ * for a launch that would not be split (types other than Q4_K, Q5_K, Q6_K and OXH_Q2_K_WIDE, more tiles,
+ * fewer than eight super-blocks, more than 64 activations); oxh_mmq_split with a smaller workspace, or
+ * none, is oxh_mmq.
  * The reference has no counterpart (its batch kernel gives every worker whole rows, oxk.c:787-836). */
 size_t oxh_mmq_split_workspace(uint32_t qtype, size_t rows, size_t cols, size_t n_vec, size_t out_stride);
 int oxh_mmq_split(uint32_t qtype, const void *d_w, size_t rows, size_t cols,

@@ -940,8 +940,12 @@ static int mv_batch(uint32_t qtype, const uint8_t *data, size_t rows,
                                qtype == OXH_Q2_K ? OXH_PREP_Q2K_WIDE : OXH_PREP_Q3K_AS_Q6K, &d_prep)))
             return rc;
         if ((rc = quantize(kind, d_x, cols, n_vec, cols, g_dact.p))) return rc;
-        if ((rc = oxh_mmq(qtype == OXH_Q2_K ? OXH_Q2_K_WIDE : OXH_Q6_K, d_prep, rows, cols, g_dact.p, n_vec,
-                          d_out, rows, NULL)))
+        const uint32_t as = qtype == OXH_Q2_K ? OXH_Q2_K_WIDE : OXH_Q6_K;
+        const size_t ws = oxh_mmq_split_workspace(as, rows, cols, n_vec, rows);
+        if (ws && (rc = reserve(&g_dsplit, ws))) return rc;
+        /* without a workspace this is oxh_mmq */
+        if ((rc = oxh_mmq_split(as, d_prep, rows, cols, g_dact.p, n_vec, d_out, rows, ws ? g_dsplit.p : NULL,
+                                ws ? g_dsplit.bytes : 0, NULL)))
             return rc;
     } else {
         const size_t step = oxh_gemv_max_nvec_buffered(qtype, cols);

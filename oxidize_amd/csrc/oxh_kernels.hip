@@ -901,6 +901,7 @@ static hipError_t raise_all_lds_ceilings(void)
     if ((e = raise_lds_ceiling(k_mmq_q80<5>)) != hipSuccess) return e;
     if ((e = raise_lds_ceiling(k_mmq_q6_k_segments<1, 1, 4, 2>)) != hipSuccess) return e;
     if ((e = raise_lds_ceiling(k_mmq_q6_k_split<2>)) != hipSuccess) return e;
+    if ((e = raise_lds_ceiling(k_mmq_q6_k_split<2, true>)) != hipSuccess) return e;
     if ((e = raise_lds_ceiling(k_mmq_q45_k_split<false, 2>)) != hipSuccess) return e;
     if ((e = raise_lds_ceiling(k_mmq_q45_k_split<true, 2>)) != hipSuccess) return e;
     if ((e = raise_lds_ceiling(k_mmq_q6_k_experts<1, 1, 4, 2>)) != hipSuccess) return e;
@@ -1828,7 +1829,7 @@ static bool mmq_split_plan(uint32_t qtype, size_t rows, size_t cols, size_t n_ve
                            uint32_t *b_per_slice, uint32_t *slices, size_t *ws_bytes)
 {
     qtype = canon_qtype(qtype);
-    if (!is_q4k(qtype) && !is_q5k(qtype) && qtype != OXH_Q6_K) return false;
+    if (!is_q4k(qtype) && !is_q5k(qtype) && qtype != OXH_Q6_K && qtype != OXH_Q2_K_WIDE) return false;
     if (rows == 0 || n_vec == 0 || n_vec > 64 || cols == 0 || cols % OXH_QK_K || out_stride < rows) return false;
     const size_t B = cols / OXH_QK_K;
     const size_t tiles = ((rows + 63) / 64) * ((n_vec + 15) / 16);
@@ -1873,6 +1874,7 @@ extern "C" int oxh_mmq_split(uint32_t qtype, const void *d_w, size_t rows, size_
         workspace_bytes < need)
         return mmq_run(qtype, d_w, rows, cols, d_acts, n_vec, d_out, out_stride, false, stream);
     if (!d_w || !d_acts || !d_out) return arg_fail("oxh_mmq_split: NULL pointer");
+    if ((uintptr_t)d_workspace % sizeof(float)) return arg_fail("oxh_mmq_split: workspace not aligned to 4 bytes");
     qtype = canon_qtype(qtype);
     const uint32_t B = (uint32_t)(cols / OXH_QK_K);
     if ((size_t)B * 292u * 256u > 0xFFFFFFFFull) return arg_fail("oxh_mmq_split: cols too large");
@@ -1886,6 +1888,9 @@ extern "C" int oxh_mmq_split(uint32_t qtype, const void *d_w, size_t rows, size_
     const size_t lds6 = 2 * G6s::LDS_BYTES, lds5 = 2 * G5s::LDS_BYTES, lds4 = 2 * G4s::LDS_BYTES;
     if (qtype == OXH_Q6_K)
         hipLaunchKernelGGL((k_mmq_q6_k_split<2>), grid, block, lds6, st, (const uint8_t *)d_w,
+                           (uint32_t)rows, B, (const uint8_t *)d_acts, (uint32_t)n_vec, terms, out_stride, per, split_stride);
+    else if (qtype == OXH_Q2_K_WIDE)
+        hipLaunchKernelGGL((k_mmq_q6_k_split<2, true>), grid, block, lds6, st, (const uint8_t *)d_w,
                            (uint32_t)rows, B, (const uint8_t *)d_acts, (uint32_t)n_vec, terms, out_stride, per, split_stride);
     else if (is_q5k(qtype))
         hipLaunchKernelGGL((k_mmq_q45_k_split<true, 2>), grid, block, lds5, st,

@@ -318,6 +318,21 @@ def test_q2k_wide_tile_kernel_on_raw_blocks(oxh, n_vec):
     mv.mmq(mv.Q2_K_WIDE, d_wide.ptr, rows, cols, d_a.ptr, n_vec, d_o.ptr, rows)
     got = d_o.download(np.float32, n_vec * rows).reshape(n_vec, rows)
     assert np.array_equal(bits(got), bits(want))
+    # the widened blocks with a tile's columns shared between workgroups (four super-blocks are too few
+    # to split: a wider matrix of the same blocks against the unsplit launch)
+    wide_rows = rows // 14
+    need = mv.mmq_split_workspace(mv.Q2_K_WIDE, wide_rows, 14 * cols, n_vec, wide_rows)
+    if n_vec <= 64:
+        assert need == 56 * n_vec * wide_rows * 4
+        d_a14 = mv.DeviceBuffer.from_host(np.tile(act.reshape(n_vec, -1), (1, 14)).reshape(-1))
+        d_ws = mv.DeviceBuffer(need)
+        d_o1, d_o2 = mv.DeviceBuffer(n_vec * wide_rows * 4), mv.DeviceBuffer(n_vec * wide_rows * 4)
+        mv.mmq(mv.Q2_K_WIDE, d_wide.ptr, wide_rows, 14 * cols, d_a14.ptr, n_vec, d_o1.ptr, wide_rows)
+        mv.mmq_split(mv.Q2_K_WIDE, d_wide.ptr, wide_rows, 14 * cols, d_a14.ptr, n_vec, d_o2.ptr, wide_rows,
+                     d_ws.ptr, need)
+        assert np.array_equal(d_o1.download(np.uint32, n_vec * wide_rows), d_o2.download(np.uint32, n_vec * wide_rows))
+    else:
+        assert need == 0
     # the widened blocks are no GGUF type: every other entry point refuses the id
     seg = mv.make_segments([(d_wide.ptr, d_o.ptr, rows, 0)])
     with pytest.raises(Exception):
