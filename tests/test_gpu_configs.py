@@ -287,7 +287,8 @@ def test_mmq_relaxed_mode_is_opt_in_and_within_tolerance(oxh, qtype, rows, cols,
 
 @pytest.mark.parametrize("qt", [13, 15, 16])
 @pytest.mark.parametrize("rows,cols,n_vec", [(4096, 14336, 16), (1000, 4096, 5), (70, 2048, 40), (64, 8192, 64),
-                                             (3000, 2304, 17)])
+                                             (3000, 2304, 17), (1, 14336, 1), (33, 5120, 3), (257, 7168, 31),
+                                             (100, 5376, 9), (2049, 6400, 18)])
 def test_mmq_with_a_tile_s_columns_shared_between_workgroups(oxh, qt, rows, cols, n_vec):
     """oxh_mmq_split: every super-block's terms go to a workspace and are added in block order by a second
     launch: bit for bit what oxh_mmq gives, padding between rows and out_stride untouched, and without a
@@ -304,7 +305,7 @@ def test_mmq_with_a_tile_s_columns_shared_between_workgroups(oxh, qt, rows, cols
     mv.mmq(qt, w.ptr, rows, cols, a.ptr, n_vec, want.ptr, out_stride)
     need = mv.mmq_split_workspace(qt, rows, cols, n_vec, out_stride)
     full = cols // 256 * n_vec * out_stride * 4
-    assert need == (full if (rows, cols) in ((4096, 14336), (1000, 4096), (64, 8192)) else 0)     # the others: too little to save
+    assert need == (0 if (rows, cols) in ((70, 2048), (3000, 2304)) else full)     # those two: too little to save
     ws = mv.DeviceBuffer(full)
     need = full                     # a launch that would not be split ignores the workspace
     mv.mmq_split(qt, w.ptr, rows, cols, a.ptr, n_vec, got.ptr, out_stride, ws.ptr, need)
