@@ -904,6 +904,10 @@ static hipError_t raise_all_lds_ceilings(void)
     if ((e = raise_lds_ceiling(k_mmq_q6_k_split<2, true>)) != hipSuccess) return e;
     if ((e = raise_lds_ceiling(k_mmq_q45_k_split<false, 2>)) != hipSuccess) return e;
     if ((e = raise_lds_ceiling(k_mmq_q45_k_split<true, 2>)) != hipSuccess) return e;
+    if ((e = raise_lds_ceiling(k_mmq_q6_k_split<2, false, 2>)) != hipSuccess) return e;
+    if ((e = raise_lds_ceiling(k_mmq_q6_k_split<2, true, 2>)) != hipSuccess) return e;
+    if ((e = raise_lds_ceiling(k_mmq_q45_k_split<false, 2, 2>)) != hipSuccess) return e;
+    if ((e = raise_lds_ceiling(k_mmq_q45_k_split<true, 2, 2>)) != hipSuccess) return e;
     if ((e = raise_lds_ceiling(k_mmq_q6_k_experts<1, 1, 4, 2>)) != hipSuccess) return e;
     if ((e = raise_lds_ceiling(k_mmq_q4_k_segments<1, 1, 8, 3>)) != hipSuccess) return e;
     if ((e = raise_lds_ceiling(k_mmq_q45_k_experts<1, 1, 8, false, 3>)) != hipSuccess) return e;
@@ -1826,13 +1830,18 @@ extern "C" int oxh_mmq(uint32_t qtype, const void *d_w, size_t rows, size_t cols
 
 /* Few tiles and many super-blocks: a tile's columns go to several workgroups (k_mmq_*_split) */
 static bool mmq_split_plan(uint32_t qtype, size_t rows, size_t cols, size_t n_vec, size_t out_stride, size_t cus,
-                           uint32_t *b_per_slice, uint32_t *slices, size_t *ws_bytes)
+                           uint32_t *b_per_slice, uint32_t *slices, size_t *ws_bytes, uint32_t *tile_tokens = nullptr)
 {
     qtype = canon_qtype(qtype);
     if (!is_q4k(qtype) && !is_q5k(qtype) && qtype != OXH_Q6_K && qtype != OXH_Q2_K_WIDE) return false;
     if (rows == 0 || n_vec == 0 || n_vec > 64 || cols == 0 || cols % OXH_QK_K || out_stride < rows) return false;
     const size_t B = cols / OXH_QK_K;
-    const size_t tiles = ((rows + 63) / 64) * ((n_vec + 15) / 16);
+    /* 64 x 16 tiles; 64 x 32 above sixteen activations unless the narrow tiles leave three quarters of
+     * the device idle anyway (a wave builds its rows' operands once per super-block whatever the tile's
+     * tokens: 4096 x 14336 Q6_K under 32 activations 44.2 -> 39.9 us, 1024 x 4096 Q4_K 7.2 -> 7.9) */
+    const size_t row_tiles = (rows + 63) / 64;
+    const size_t tile_tok = (n_vec > 16 && row_tiles * ((n_vec + 15) / 16) > cus / 4) ? 32 : 16;
+    const size_t tiles = row_tiles * ((n_vec + tile_tok - 1) / tile_tok);
     if (B < 8 || tiles > cus / 2) return false;
     const size_t want = (2 * cus) / tiles;                      /* workgroups per tile for two per CU */
     size_t per = (B + want - 1) / want;
@@ -1844,13 +1853,15 @@ static bool mmq_split_plan(uint32_t qtype, size_t rows, size_t cols, size_t n_ve
     bytes = B * n_vec * out_stride * sizeof(float);
     if (bytes > ((size_t)512 << 20)) return false;
     /* what the shorter walk saves (0.8 us a super-block) against the second launch and the terms' trip
-     * through memory (written and read once at some 4 TB/s), with two microseconds to spare: 4096 x 4096
-     * under 32 activations measured 13.6 us split against 12.7, 4096 x 14336 29.8 against 45.2 */
+     * through memory (written and read once at some 4 TB/s), with four microseconds to spare: 4096 x 4096
+     * Q4_K under 32 activations measured 12.7 us split against 12.7, under 24 11.8 against 12.9, 6144 x 4096
+     * under 17 14.0 against 13.1, 4096 x 14336 under 32 26.3 against 42.6, under 48 36.5 against 43.2 */
     const double saving_us = 0.8 * (double)(B - per), cost_us = 4.0 + 2.0 * (double)bytes / 4.0e6;
-    if (saving_us < cost_us + 2.0) return false;
+    if (saving_us < cost_us + 4.0) return false;
     if (b_per_slice) *b_per_slice = (uint32_t)per;
     if (slices) *slices = (uint32_t)n;
     if (ws_bytes) *ws_bytes = bytes;
+    if (tile_tokens) *tile_tokens = (uint32_t)tile_tok;
     return true;
 }
 
@@ -1867,10 +1878,10 @@ extern "C" int oxh_mmq_split(uint32_t qtype, const void *d_w, size_t rows, size_
 {
     int rc = ensure_init();
     if (rc) return rc;
-    uint32_t per = 0, slices = 0;
+    uint32_t per = 0, slices = 0, tile_tok = 16;
     size_t need = 0;
     const size_t cus = (size_t)(g_n_cu > 0 ? g_n_cu : 256);
-    if (!mmq_split_plan(qtype, rows, cols, n_vec, out_stride, cus, &per, &slices, &need) || !d_workspace ||
+    if (!mmq_split_plan(qtype, rows, cols, n_vec, out_stride, cus, &per, &slices, &need, &tile_tok) || !d_workspace ||
         workspace_bytes < need)
         return mmq_run(qtype, d_w, rows, cols, d_acts, n_vec, d_out, out_stride, false, stream);
     if (!d_w || !d_acts || !d_out) return arg_fail("oxh_mmq_split: NULL pointer");
@@ -1878,28 +1889,39 @@ extern "C" int oxh_mmq_split(uint32_t qtype, const void *d_w, size_t rows, size_
     qtype = canon_qtype(qtype);
     const uint32_t B = (uint32_t)(cols / OXH_QK_K);
     if ((size_t)B * 292u * 256u > 0xFFFFFFFFull) return arg_fail("oxh_mmq_split: cols too large");
-    const dim3 grid((uint32_t)((rows + 63) / 64), (uint32_t)((n_vec + 15) / 16), slices), block(4 * 64);
+    const dim3 grid((uint32_t)((rows + 63) / 64), (uint32_t)((n_vec + tile_tok - 1) / tile_tok), slices), block(4 * 64);
     const size_t split_stride = n_vec * out_stride;
     hipStream_t st = pick_stream(stream);
     float *terms = (float *)d_workspace;
-    typedef Mmq6Geom<1, 1, 4> G6s;
-    typedef MmqGeom<1, 1, 4, true> G5s;
-    typedef MmqGeom<1, 1, 4> G4s;
-    const size_t lds6 = 2 * G6s::LDS_BYTES, lds5 = 2 * G5s::LDS_BYTES, lds4 = 2 * G4s::LDS_BYTES;
-    if (qtype == OXH_Q6_K)
-        hipLaunchKernelGGL((k_mmq_q6_k_split<2>), grid, block, lds6, st, (const uint8_t *)d_w,
-                           (uint32_t)rows, B, (const uint8_t *)d_acts, (uint32_t)n_vec, terms, out_stride, per, split_stride);
-    else if (qtype == OXH_Q2_K_WIDE)
-        hipLaunchKernelGGL((k_mmq_q6_k_split<2, true>), grid, block, lds6, st, (const uint8_t *)d_w,
-                           (uint32_t)rows, B, (const uint8_t *)d_acts, (uint32_t)n_vec, terms, out_stride, per, split_stride);
-    else if (is_q5k(qtype))
-        hipLaunchKernelGGL((k_mmq_q45_k_split<true, 2>), grid, block, lds5, st,
-                           (const uint8_t *)d_w, (uint32_t)rows, B, (const uint8_t *)d_acts, (uint32_t)n_vec, terms,
-                           out_stride, per, split_stride);
-    else
-        hipLaunchKernelGGL((k_mmq_q45_k_split<false, 2>), grid, block, lds4, st,
-                           (const uint8_t *)d_w, (uint32_t)rows, B, (const uint8_t *)d_acts, (uint32_t)n_vec, terms,
-                           out_stride, per, split_stride);
+    const uint8_t *w8 = (const uint8_t *)d_w, *a8 = (const uint8_t *)d_acts;
+    const uint32_t r32 = (uint32_t)rows, n32 = (uint32_t)n_vec;
+#define OXH_SPLIT_LAUNCH(KERNEL, GEOM)                                                                        \
+    do {                                                                                                      \
+        auto kern = KERNEL;                                                                                   \
+        hipLaunchKernelGGL(kern, grid, block, 2 * GEOM::LDS_BYTES, st, w8, r32, B, a8, n32, terms, out_stride, \
+                           per, split_stride);                                                                \
+    } while (0)
+    typedef Mmq6Geom<1, 1, 4> G6a;
+    typedef Mmq6Geom<2, 1, 4> G6b;
+    typedef MmqGeom<1, 1, 4, true> G5a;
+    typedef MmqGeom<2, 1, 4, true> G5b;
+    typedef MmqGeom<1, 1, 4> G4a;
+    typedef MmqGeom<2, 1, 4> G4b;
+    const bool wide_tile = tile_tok == 32;
+    if (qtype == OXH_Q6_K) {
+        if (wide_tile) OXH_SPLIT_LAUNCH((k_mmq_q6_k_split<2, false, 2>), G6b);
+        else OXH_SPLIT_LAUNCH((k_mmq_q6_k_split<2, false, 1>), G6a);
+    } else if (qtype == OXH_Q2_K_WIDE) {
+        if (wide_tile) OXH_SPLIT_LAUNCH((k_mmq_q6_k_split<2, true, 2>), G6b);
+        else OXH_SPLIT_LAUNCH((k_mmq_q6_k_split<2, true, 1>), G6a);
+    } else if (is_q5k(qtype)) {
+        if (wide_tile) OXH_SPLIT_LAUNCH((k_mmq_q45_k_split<true, 2, 2>), G5b);
+        else OXH_SPLIT_LAUNCH((k_mmq_q45_k_split<true, 2, 1>), G5a);
+    } else {
+        if (wide_tile) OXH_SPLIT_LAUNCH((k_mmq_q45_k_split<false, 2, 2>), G4b);
+        else OXH_SPLIT_LAUNCH((k_mmq_q45_k_split<false, 2, 1>), G4a);
+    }
+#undef OXH_SPLIT_LAUNCH
     HIP_TRY(hipGetLastError());
     const size_t n_out = rows * n_vec;
     hipLaunchKernelGGL(k_mmq_sum_terms, dim3((uint32_t)((n_out + 255) / 256)), dim3(256), 0, st, terms, B, split_stride,

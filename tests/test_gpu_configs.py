@@ -288,7 +288,7 @@ def test_mmq_relaxed_mode_is_opt_in_and_within_tolerance(oxh, qtype, rows, cols,
 @pytest.mark.parametrize("qt", [13, 15, 16])
 @pytest.mark.parametrize("rows,cols,n_vec", [(4096, 14336, 16), (1000, 4096, 5), (70, 2048, 40), (64, 8192, 64),
                                              (3000, 2304, 17), (1, 14336, 1), (33, 5120, 3), (257, 7168, 31),
-                                             (100, 5376, 9), (2049, 6400, 18)])
+                                             (100, 5376, 9), (2049, 6400, 18), (4000, 14336, 45), (4096, 4096, 24)])
 def test_mmq_with_a_tile_s_columns_shared_between_workgroups(oxh, qt, rows, cols, n_vec):
     """oxh_mmq_split: every super-block's terms go to a workspace and are added in block order by a second
     launch: bit for bit what oxh_mmq gives, padding between rows and out_stride untouched, and without a
