@@ -637,6 +637,20 @@ static int mmq_relaxed_enabled(void)
     return cached;
 }
 
+/* OXH_MMQ_SPLIT_MIN_NV: activations from which a batch over few rows and many columns shares its tiles'
+ * columns between workgroups (7; 0 = never) */
+static size_t mmq_split_min_nv(void)
+{
+    static long cached = -1;
+    if (cached < 0) {
+        const char *e = getenv("OXH_MMQ_SPLIT_MIN_NV");
+        char *end = NULL;
+        const long v = (e && *e) ? strtol(e, &end, 10) : 7;
+        cached = (e && *e && (end == e || v < 0 || v > 64)) ? 7 : v;
+    }
+    return cached == 0 ? SIZE_MAX : (size_t)cached;
+}
+
 static int quantize(int kind, const float *d_x, size_t in_stride, size_t n_vec,
                     size_t cols, void *d_act)
 {
@@ -918,7 +932,7 @@ static int mv_batch(uint32_t qtype, const uint8_t *data, size_t rows,
                        qtype == OXH_Q6_K;
     /* few rows, many columns, seven activations or more: the tiles' columns shared between workgroups
      * (up to six the dot kernels are as fast: 4096 x 14336 Q6_K 24.7 us at six, 43 at eight, 28 split) */
-    const size_t split_ws = (kq456 && n_vec >= 7) ? oxh_mmq_split_workspace(qtype, rows, cols, n_vec, rows) : 0;
+    const size_t split_ws = (kq456 && n_vec >= mmq_split_min_nv()) ? oxh_mmq_split_workspace(qtype, rows, cols, n_vec, rows) : 0;
     if (split_ws) {
         if ((rc = reserve(&g_dsplit, split_ws))) return rc;
         if ((rc = quantize(kind, d_x, cols, n_vec, cols, g_dact.p))) return rc;
@@ -941,7 +955,7 @@ static int mv_batch(uint32_t qtype, const uint8_t *data, size_t rows,
             return rc;
         if ((rc = quantize(kind, d_x, cols, n_vec, cols, g_dact.p))) return rc;
         const uint32_t as = qtype == OXH_Q2_K ? OXH_Q2_K_WIDE : OXH_Q6_K;
-        const size_t ws = oxh_mmq_split_workspace(as, rows, cols, n_vec, rows);
+        const size_t ws = n_vec >= mmq_split_min_nv() ? oxh_mmq_split_workspace(as, rows, cols, n_vec, rows) : 0;
         if (ws && (rc = reserve(&g_dsplit, ws))) return rc;
         /* without a workspace this is oxh_mmq */
         if ((rc = oxh_mmq_split(as, d_prep, rows, cols, g_dact.p, n_vec, d_out, rows, ws ? g_dsplit.p : NULL,

@@ -321,3 +321,28 @@ def test_mmq_with_a_tile_s_columns_shared_between_workgroups(oxh, qt, rows, cols
     assert mv.mmq_split_workspace(qt, 4096, 1024, 16, 4096) == 0
     assert mv.mmq_split_workspace(qt, 4096, 14336, 512, 4096) == 0
     assert mv.mmq_split_workspace(7, 4096, 4096, 16, 4096) == 0
+
+
+@pytest.mark.parametrize("qt", [13, 15, 16, 10, 8])
+@pytest.mark.parametrize("rows,cols,n_vec", [(300, 5120, 9), (1000, 4096, 7), (130, 14336, 33)])
+def test_batch_entry_point_over_few_rows_and_many_columns(oxh, qt, rows, cols, n_vec):
+    """oc_matvec_quantized_batch over shapes whose tiles share their columns between workgroups (seven
+    vectors or more of a K-quant; Q2_K and Q3_K from nine on, through their rewritten forms): padded
+    strides, every output with the oracle's bits, nothing written between rows and out_stride."""
+    assert mv.mmq_split_workspace(16 if qt in (10, 8) else qt, rows, cols, n_vec, rows) > 0
+    rb = synth.row_bytes(qt, cols)
+    w = synth.weights(qt, rows, cols, seed=71, stream=n_vec)
+    in_stride, out_stride = cols + 8, rows + 3
+    xb = synth.normal(n_vec * in_stride, seed=72, stream=n_vec).reshape(n_vec, in_stride)
+    ob = np.full((n_vec, out_stride), -1.0, np.float32)
+    temp = np.zeros(cols, np.float32)
+    scratch = np.zeros(mv.batch_scratch_bytes(cols), np.uint8)
+    assert mv.matvec_quantized_batch(qt, w, rows, cols, rb, xb, in_stride, ob, out_stride, n_vec, temp,
+                                     scratch) == 0
+    assert np.all(ob[:, rows:] == -1.0)
+    o = oxlibs.oracle()
+    want = np.zeros((n_vec, out_stride), np.float32)
+    act = np.zeros(scratch.size, np.uint8)
+    assert o.oxo_matvec_quantized_batch(qt, w.ctypes.data, rows, cols, rb, xb.ctypes.data, in_stride,
+                                        want.ctypes.data, out_stride, n_vec, act.ctypes.data, act.size) == 0
+    assert np.array_equal(bits(ob[:, :rows]), bits(want[:, :rows]))
