@@ -136,11 +136,12 @@ def secondary_figures(mv, synth):
     # what bounds that kernel: int8 MFMA rate of the device with 0 / 1 / 2 / 4 independent vector instructions
     # after every MFMA, at two and four waves per SIMD (they do not overlap on this device)
     import ctypes
+    from oxidize_amd import _lib
     probe = {}
     for nv in (0, 1, 2, 4):
         for wps in (2, 4):
             pops = ctypes.c_double()
-            if mv.lib().oxh_debug_mfma_probe(nv, wps, ctypes.byref(pops)) == 0:
+            if _lib.lab().mfma_probe(nv, wps, ctypes.byref(pops)) == 0:
                 probe["valu_%d_per_mfma_%d_waves_per_simd" % (nv, wps)] = round(pops.value, 3)
     out["int8_mfma_pops_with_vector_work_beside"] = probe
     d_x.free()

@@ -287,17 +287,9 @@ int oxh_plan_prestaged(const OxhPlan *plan);
 /* Rows of the table a launch walks: the operations, or fewer where independent
  * operations share rows.  Negative for a NULL plan. */
 int oxh_plan_table_rows(const OxhPlan *plan);
-/* The poll limit of every wait.  With `phantom_workgroup` set the waits also
- * expect a workgroup that does not exist, so every wait runs into the limit:
- * the way to test the give-up path without hanging anything. */
-int oxh_plan_set_spin_limit(OxhPlan *plan, uint32_t polls, int phantom_workgroup);
+/* The poll limit of every wait (default 4 000 000, or OXH_PLAN_SPIN_LIMIT). */
+int oxh_plan_set_spin_limit(OxhPlan *plan, uint32_t polls);
 int oxh_plan_destroy(OxhPlan *plan);
-/* Measurement aid: with d_stamps set (n_ops * workgroups * 8 uint64 of device
- * memory, or NULL to switch it off) wave 0 of every workgroup stores the shader
- * clock at eight points of every operation: start, dependency met, activation
- * staged, workgroup barrier passed, passes done, rows summed, barrier passed,
- * outputs stored and announced.  No counterpart in the reference. */
-int oxh_debug_plan_stamps(OxhPlan *plan, uint64_t *d_stamps);
 /* How a plan deals the rows of one operation's segments to `grid` workgroups of
  * sixteen waves (pure host arithmetic): workgroups per segment and the most
  * table rows any wave owns (a paired segment counts two per row). */
@@ -471,36 +463,6 @@ int oxh_moe_route(const float *d_logits, size_t n_tok, size_t n_expert, size_t t
                   int32_t *d_ids, float *d_weights, uint32_t *d_counts, uint32_t *d_offsets,
                   uint32_t *d_perm, uint32_t *d_slot_pos, void *stream);
 
-/* Test hook: byte offsets inside oxh_moe_ffn's workspace of, in this order,
- * ids, weights, slot_pos, perm, counts, offsets, the gathered Q8_K activations,
- * gate, up (f32 [pair][ffn]), the Q8_K form of silu(gate)*up, the down outputs
- * (f32 [pair][hidden]), and the total size.  After a call the parity tests read
- * every intermediate from there. */
-int oxh_debug_moe_workspace_parts(const OxhMoe *m, size_t n_tok, size_t parts[12]);
-
-/* Measurement aid: one launch that only reads `bytes` of device memory (a
- * workgroup per CU, 16-byte loads, nothing computed); d_sink may be NULL.
- * Timed on a buffer the size of a weight matrix it gives the ceiling any
- * kernel streaming that matrix once can reach on the device, launch cost
- * included.  No counterpart in the reference. */
-int oxh_debug_read_probe(const void *d_buf, size_t bytes, uint32_t *d_sink, void *stream);
-
-/* Measurement aid: the int8 matrix-core rate of the whole device (POP/s) when
- * every v_mfma_i32_16x16x64_i8 is followed by `valu_per_mfma` (0, 1, 2 or 4)
- * independent f32 vector instructions, with 1..4 waves per SIMD.  Synchronous
- * (two launches, the second timed with events).  Shows whether vector work
- * hides behind matrix work on the device.  No counterpart in the reference. */
-int oxh_debug_mfma_probe(int valu_per_mfma, int waves_per_simd, double *pops);
-
-/* Test hook: the integer sub-block sums the GEMV kernel forms, written by the
- * same device code path.  Q4_K and Q5_K: 8 int32 per super-block (S_j), Q6_K: 16 per
- * super-block, Q8_0: 1 per block; layout [row][block][j].  The reference
- * exposes no such API; the values are the intermediates of
- * oxidize-c/src/compute/oxk.c:263-283, :870-886, :932-954, :234-237. */
-int oxh_debug_subblock_sums(uint32_t qtype, const void *d_w, size_t rows,
-                            size_t cols, const void *d_act, int32_t *d_sums,
-                            void *stream);
-
 /* Device memory / stream / event plumbing so that C callers never include
  * HIP headers (as cuda_mmq.h does with its void* stream). */
 int  oxh_malloc(void **d_ptr, size_t bytes);
@@ -541,6 +503,8 @@ int  oxh_graph_destroy(void *graph_exec);
 /* name (<=255 chars), compute units, clock MHz, memory bytes. */
 int  oxh_device_info(char *name, size_t name_len, int *n_cu, int *clock_mhz,
                      size_t *mem_bytes);
+/* Device memory free right now and in all (hipMemGetInfo); either may be NULL. */
+int  oxh_mem_info(size_t *free_bytes, size_t *total_bytes);
 
 /* ─── model files ─────────────────────────────────────────────────────── */
 
@@ -608,17 +572,25 @@ uint32_t oxh_qtype_from_ggml_id(uint32_t ggml_id);
  *
  * Weights the caller never registered keep the reference's contract, under
  * which the host bytes are the input of every call (oxidize-c/include/oxidize/
- * matvec.h:45-52): the device copy made on first sight serves only the exact
- * (pointer, byte count) it was made for, every later call re-checks a
- * fingerprint of the host bytes (length, first and last 4 KiB, 128 strided
- * 64-byte samples; a few microseconds) and refreshes the copy when it differs,
- * and a matrix that overlaps older cached ones replaces them.  So freeing a
- * model and loading another at the same addresses is safe without any call
- * here.  What the sampled fingerprint can miss is an edit of a few bytes in
- * the middle of a matrix that stays in place: OXH_WEIGHT_CACHE=full hashes
- * every byte on every call, OXH_WEIGHT_CACHE=off uploads on every call.
- * OXH_WEIGHT_CACHE_MB (default 65536) bounds the bytes cached this way; the
- * least recently used go first. */
+ * matvec.h:45-52), with ONE STATED LIMIT.  The device copy made on first sight
+ * serves only the exact (pointer, byte count) it was made for, and every later
+ * call re-checks the host bytes before using it (a few microseconds):
+ *   - the length, the first and last 4 KiB and 128 strided 64-byte samples:
+ *     a freed model replaced by another at the same addresses, a buffer
+ *     refilled, a matrix that overlaps older cached ones: seen on that call;
+ *   - two 16 KiB slices, hashed whole against the hashes taken of every slice
+ *     at upload, the slices taking turns from call to call: an edit of ANY
+ *     size ANYWHERE in the matrix is seen after at most
+ *     ceil(bytes / 32 KiB) calls over that matrix (1008 for 33 MB).
+ * THE LIMIT: a few bytes patched in place, between the samples, may be served
+ * from the old device copy until the rotating slices reach them.  A caller
+ * that edits weights in place and needs the very next call to see the edit
+ * calls oxh_weight_unregister(ptr) after the edit (it drops cached copies as
+ * well), or runs with OXH_WEIGHT_CACHE=full (every byte hashed on every call)
+ * or =off (uploaded on every call).  Registered ranges are never looked at.
+ * OXH_WEIGHT_CACHE_MB bounds the bytes cached this way and their rewritten
+ * forms (default: half of the device memory free when the first one is made);
+ * the least recently used go first, also when the device itself runs out. */
 int oxh_weight_register(const void *h_data, size_t bytes);
 /* Drops every range, registered or cached, that contains h_data. */
 int oxh_weight_unregister(const void *h_data);
@@ -630,6 +602,8 @@ const void *oxh_weight_device_ptr(const void *h_data);
  * a cached copy was refreshed because its host bytes had changed.  Any pointer
  * may be NULL. */
 int oxh_weight_stats(size_t *n_registered, size_t *n_cached, size_t *cached_bytes, size_t *refreshes);
+/* Cached ranges given up so far for the budget or for want of device memory. */
+size_t oxh_weight_evictions(void);
 
 /* Same arguments and results as oc_matvec_quantized
  * (oxidize-c/include/oxidize/matvec.h:50-52; matvec.c:833-907): output[r] =

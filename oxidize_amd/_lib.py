@@ -49,8 +49,19 @@ class OcMatvecFusedTestStats(ctypes.Structure):
                 ("fallback_calls", Z)]
 
 
-# name -> (restype, argtypes); every symbol include/oxhip.h declares
+class OxhLab(ctypes.Structure):
+    """include/oxhip_lab.h: test hooks and measurement aids, reached through oxh_lab()."""
+    _fields_ = [("plan_stamps", ctypes.CFUNCTYPE(I, V, V)),
+                ("plan_phantom", ctypes.CFUNCTYPE(I, V, I)),
+                ("moe_workspace_parts", ctypes.CFUNCTYPE(I, ctypes.POINTER(OxhMoe), Z, ctypes.POINTER(Z * 12))),
+                ("read_probe", ctypes.CFUNCTYPE(I, V, Z, V, V)),
+                ("mfma_probe", ctypes.CFUNCTYPE(I, I, I, ctypes.POINTER(ctypes.c_double))),
+                ("subblock_sums", ctypes.CFUNCTYPE(I, U32, V, Z, Z, V, V, V))]
+
+
+# name -> (restype, argtypes); every symbol include/oxhip.h and include/oxhip_lab.h declare
 SIGNATURES = {
+    "oxh_lab": (ctypes.POINTER(OxhLab), []),
     "oxh_last_error": (ctypes.c_char_p, []),
     "oxh_init": (I, [I]),
     "oxh_shutdown": (None, []),
@@ -70,9 +81,8 @@ SIGNATURES = {
     "oxh_plan_prestaged": (I, [V]),
     "oxh_plan_table_rows": (I, [V]),
     "oxh_q6_k_group": (I, [V, Z, Z, V, V]),
-    "oxh_plan_set_spin_limit": (I, [V, U32, I]),
+    "oxh_plan_set_spin_limit": (I, [V, U32]),
     "oxh_plan_destroy": (I, [V]),
-    "oxh_debug_plan_stamps": (I, [V, V]),
     "oxh_plan_deal": (I, [ctypes.POINTER(Z), ctypes.POINTER(I), Z, U32, ctypes.POINTER(U32), ctypes.POINTER(U32)]),
     "oxh_mmq": (I, [U32, V, Z, Z, V, Z, V, Z, V]),
     "oxh_mmq_ex": (I, [U32, V, Z, Z, V, Z, V, Z, U32, V]),
@@ -80,16 +90,12 @@ SIGNATURES = {
     "oxh_mmq_split_workspace": (Z, [U32, Z, Z, Z, Z]),
     "oxh_mmq_split": (I, [U32, V, Z, Z, V, Z, V, Z, V, Z, V]),
     "oxh_get_rows": (I, [U32, V, Z, Z, V, Z, V, Z, V]),
-    "oxh_debug_subblock_sums": (I, [U32, V, Z, Z, V, V, V]),
-    "oxh_debug_read_probe": (I, [V, Z, V, V]),
-    "oxh_debug_mfma_probe": (I, [I, I, ctypes.POINTER(ctypes.c_double)]),
     "oxh_q3_k_as_q6_k": (I, [V, Z, Z, V, V]),
     "oxh_q2_k_widen": (I, [V, Z, Z, V, V]),
     "oxh_moe_workspace_bytes": (I, [ctypes.POINTER(OxhMoe), Z, ctypes.POINTER(Z)]),
     "oxh_moe_ffn": (I, [ctypes.POINTER(OxhMoe), V, V, Z, Z, V, Z, V, Z, V]),
     "oxh_moe_ffn_static": (I, [ctypes.POINTER(OxhMoe), V, V, Z, Z, V, Z, V]),
     "oxh_moe_route": (I, [V, Z, Z, Z, I, V, V, V, V, V, V, V]),
-    "oxh_debug_moe_workspace_parts": (I, [ctypes.POINTER(OxhMoe), Z, ctypes.POINTER(Z * 12)]),
     "oxh_malloc": (I, [ctypes.POINTER(V), Z]),
     "oxh_host_alloc": (I, [ctypes.POINTER(V), Z]),
     "oxh_host_free": (I, [V]),
@@ -114,6 +120,7 @@ SIGNATURES = {
     "oxh_graph_destroy": (I, [V]),
     "oxh_device_info": (I, [ctypes.c_char_p, Z, ctypes.POINTER(I), ctypes.POINTER(I),
                             ctypes.POINTER(Z)]),
+    "oxh_mem_info": (I, [ctypes.POINTER(Z), ctypes.POINTER(Z)]),
     "oxh_gguf_open": (I, [ctypes.c_char_p, ctypes.POINTER(V)]),
     "oxh_gguf_close": (None, [V]),
     "oxh_gguf_info": (I, [V, ctypes.POINTER(U32), ctypes.POINTER(ctypes.c_uint64),
@@ -130,6 +137,7 @@ SIGNATURES = {
     "oxh_weight_clear": (I, []),
     "oxh_weight_device_ptr": (V, [V]),
     "oxh_weight_stats": (I, [ctypes.POINTER(Z), ctypes.POINTER(Z), ctypes.POINTER(Z), ctypes.POINTER(Z)]),
+    "oxh_weight_evictions": (Z, []),
     "oxh_matvec_quantized": (I, [U32, V, Z, Z, Z, V, V, V]),
     "oxh_matvec_quantized_fused": (I, [V, V, V, Z, V, Z, V, V, V]),
     "oxh_matvec_quantized_multi_input": (I, [V, V, V, Z, V, Z, V, V, V]),
@@ -171,6 +179,11 @@ def lib():
             fn.argtypes = args
         _LIB = handle
     return _LIB
+
+
+def lab():
+    """The table of test hooks and measurement aids (include/oxhip_lab.h)."""
+    return lib().oxh_lab().contents
 
 
 def check(status):

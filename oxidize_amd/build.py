@@ -36,6 +36,28 @@ def _run(cmd):
 HIP_UNITS = ("oxh_kernels", "oxh_plan")
 
 
+def exported_names():
+    """The functions the public headers declare: exactly what liboxhip.so exports."""
+    import re
+    names = set()
+    for header in ("oxhip.h", "oxhip_lab.h"):
+        text = open(os.path.join(INCLUDE, header)).read()
+        text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+        names.update(re.findall(r"\b((?:oxh|oc)_[a-z0-9_]+)\s*\(", text))
+    return sorted(names)
+
+
+def write_export_map(path):
+    """A linker version script: the declared functions are global, everything else (the kernels' host
+    stubs, the symbols the two translation units and the C host layer share, the lab functions behind
+    oxh_lab's table) stays inside the library."""
+    with open(path, "w") as f:
+        f.write("{\n  global:\n")
+        for n in exported_names():
+            f.write("    %s;\n" % n)
+        f.write("  local:\n    *;\n};\n")
+
+
 def build_oxhip(verbose=False, only=None):
     """`only`: names of HIP translation units to recompile (the others' objects are reused)."""
     from concurrent.futures import ThreadPoolExecutor
@@ -55,8 +77,10 @@ def build_oxhip(verbose=False, only=None):
                                   os.path.join(CSRC, "oc_matvec.c"), "-o", obj_c])
     log += _run([CC] + C_FLAGS + ["-I", INCLUDE, "-I", CSRC, "-c",
                                   os.path.join(CSRC, "oxh_gguf.c"), "-o", obj_g])
+    export_map = os.path.join(CSRC, "liboxhip.map")
+    write_export_map(export_map)
     log += _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", out] + hip_objs + [obj_c, obj_g,
-                 "-lpthread", "-Wno-unused-command-line-argument"])
+                 "-lpthread", "-Wl,--version-script=" + export_map, "-Wno-unused-command-line-argument"])
     if verbose and log.strip():
         print(log)
     return out

@@ -78,8 +78,18 @@ size_t oc_matvec_batch_scratch_bytes(size_t max_cols)
  *             fingerprint of the host bytes; on a mismatch the device copy is refreshed in place.  A new
  *             range that overlaps automatic entries replaces them.  Least recently used entries go once
  *             the cached bytes pass a budget.
- * OXH_WEIGHT_CACHE = sample (default: fingerprint of the first and last 4 KiB plus 128 strided 64-byte
- * samples and the length), full (hash of every byte on every call), off (upload on every call). */
+ * OXH_WEIGHT_CACHE = sample (default), full (hash of every byte on every call), off (upload on every call).
+ * What `sample` checks on every call over an automatic entry:
+ *   - the length, the first and last 4 KiB and 128 strided 64-byte samples (a reused buffer, a model
+ *     loaded over another: caught on the next call);
+ *   - SLICES_PER_CALL slices of SLICE_BYTES, hashed whole and compared with the hash the slice had when
+ *     the range was uploaded (every slice is hashed then), the slices taking turns from call to call.
+ *     An edit of any size anywhere in the range is therefore caught after at most
+ *     ceil(bytes / SLICE_BYTES / SLICES_PER_CALL) calls over that matrix, whatever it misses before.
+ * A caller that patches weights in place and needs the very next call to see it calls
+ * oxh_weight_unregister(ptr) (it drops automatic entries too), registers the range, or runs with `full`. */
+#define SLICE_BYTES ((size_t)16384u)
+#define SLICES_PER_CALL 2u
 typedef struct {
     size_t off, rows, cols;     /* which sub-matrix of the range, and its shape */
     uint32_t form;              /* OXH_PREP_* */
@@ -93,6 +103,8 @@ typedef struct {
     uint8_t *d;
     bool automatic;
     uint64_t print;             /* automatic entries: fingerprint of the host bytes at upload */
+    uint64_t *slice;            /* automatic entries in `sample` mode: hash of every SLICE_BYTES slice */
+    size_t n_slice, cursor;     /* their count; the slice the next call re-checks first */
     uint64_t tick;              /* last use */
     Prepared *prep;             /* device-side rewrites of (parts of) this range, made on demand */
     size_t n_prep;
@@ -109,7 +121,8 @@ static uint64_t g_tick = 0;
 /* g_tick when the running call began: entries used since then back a launch of this call and must
  * stay where they are until it has finished */
 static uint64_t g_call_tick = 0;
-static size_t g_auto_bytes = 0;
+static size_t g_auto_bytes = 0;       /* automatic entries and their rewritten forms */
+static size_t g_evictions = 0;
 
 enum { CACHE_SAMPLE = 0, CACHE_FULL = 1, CACHE_OFF = 2 };
 
@@ -125,15 +138,23 @@ static int cache_mode(void)
     return mode;
 }
 
-/* Budget for automatic entries, OXH_WEIGHT_CACHE_MB (default 65536: a quarter of the device). */
+/* Budget for automatic entries and the rewritten forms kept with them: OXH_WEIGHT_CACHE_MB, else half of
+ * the device memory that is free when the first automatic entry is made (other processes and the
+ * caller's own buffers are then already counted out), and never less than 256 MiB. */
 static size_t cache_budget(void)
 {
     static size_t budget = 0;
     if (!budget) {
         const char *e = getenv("OXH_WEIGHT_CACHE_MB");
         unsigned long long mb = e && *e ? strtoull(e, NULL, 10) : 0ull;
-        if (mb == 0ull || mb > (1ull << 24)) mb = 65536ull;
-        budget = (size_t)mb << 20;
+        if (mb != 0ull && mb <= (1ull << 24)) {
+            budget = (size_t)mb << 20;
+        } else {
+            size_t free_b = 0, total_b = 0;
+            if (oxh_mem_info(&free_b, &total_b) != OXH_OK || free_b == 0) free_b = (size_t)128u << 30;
+            budget = free_b / 2u;
+            if (budget < ((size_t)256u << 20)) budget = (size_t)256u << 20;
+        }
     }
     return budget;
 }
@@ -187,9 +208,45 @@ static uint64_t host_print(const uint8_t *p, size_t bytes)
     return h;
 }
 
+/* Hash of slice i of the range (the last one may be short). */
+static uint64_t slice_print(const uint8_t *p, size_t bytes, size_t i)
+{
+    const size_t at = i * SLICE_BYTES, n = bytes - at < SLICE_BYTES ? bytes - at : SLICE_BYTES;
+    return hash_bytes(mix64(0x736C696365ull, (uint64_t)i), p + at, n);
+}
+
+/* The per-slice hashes of an automatic entry, taken when its bytes go to the device (`sample` mode and
+ * ranges the fingerprint does not cover whole).  Without memory for the table the entry simply has none. */
+static void slices_take(Resident *r)
+{
+    free(r->slice);
+    r->slice = NULL;
+    r->n_slice = r->cursor = 0;
+    if (!r->automatic || cache_mode() != CACHE_SAMPLE || r->bytes <= 16384u) return;
+    const size_t n = (r->bytes + SLICE_BYTES - 1u) / SLICE_BYTES;
+    r->slice = (uint64_t *)malloc(n * sizeof *r->slice);
+    if (!r->slice) return;
+    for (size_t i = 0; i < n; i++) r->slice[i] = slice_print(r->h, r->bytes, i);
+    r->n_slice = n;
+}
+
+/* This call's turn of the rotating check: true when every slice looked at still has its hash. */
+static bool slices_hold(Resident *r)
+{
+    for (unsigned k = 0; k < SLICES_PER_CALL && r->n_slice; k++) {
+        const size_t i = r->cursor;
+        r->cursor = (i + 1u) % r->n_slice;
+        if (slice_print(r->h, r->bytes, i) != r->slice[i]) return false;
+    }
+    return true;
+}
+
 static void drop_prepared(Resident *r)
 {
-    for (size_t i = 0; i < r->n_prep; i++) (void)oxh_free(r->prep[i].d);
+    for (size_t i = 0; i < r->n_prep; i++) {
+        if (r->automatic) g_auto_bytes -= r->prep[i].bytes;
+        (void)oxh_free(r->prep[i].d);
+    }
     free(r->prep);
     r->prep = NULL;
     r->n_prep = 0;
@@ -201,6 +258,7 @@ static int drop_entry(size_t i)
     Resident *r = &g_res[i];
     drop_prepared(r);
     if (r->automatic) g_auto_bytes -= r->bytes;
+    free(r->slice);
     const int rc = oxh_free(r->d);
     g_res[i] = g_res[g_nres - 1];
     g_nres--;
@@ -239,6 +297,41 @@ static int upload(uint8_t *d, const uint8_t *h, size_t bytes)
     return rc;
 }
 
+/* Drops the least recently used automatic entry that the running call does not use (and is not `keep`).
+ * False when there is none.  The caller holds g_lock. */
+static bool evict_one(const Resident *keep, bool *synced)
+{
+    size_t lru = g_nres;
+    for (size_t i = 0; i < g_nres; i++)
+        if (g_res[i].automatic && &g_res[i] != keep && g_res[i].tick <= g_call_tick &&
+            (lru == g_nres || g_res[i].tick < g_res[lru].tick)) lru = i;
+    if (lru == g_nres) return false;
+    if (!*synced) {
+        if (oxh_stream_sync(NULL) != OXH_OK) return false;
+        *synced = true;
+    }
+    (void)drop_entry(lru);
+    return true;
+}
+
+/* Device memory for the registry.  The budget is a guess about what the device has left for us; when
+ * the allocation itself fails, automatic entries are given up, least recently used first, until it
+ * succeeds or none is left.  drop_entry moves the last entry into the freed slot, so `keep` (an entry
+ * the caller goes on using) is passed by address and re-found by the caller if it needs to. */
+static int alloc_evicting(void **d, size_t bytes, const uint8_t *keep_h, bool *synced)
+{
+    int rc = oxh_malloc(d, bytes);
+    while (rc == OXH_ERR_NOMEM) {
+        const Resident *keep = NULL;
+        for (size_t i = 0; i < g_nres && keep_h; i++)
+            if (g_res[i].h == keep_h) keep = &g_res[i];
+        if (!evict_one(keep, synced)) break;
+        g_evictions++;
+        rc = oxh_malloc(d, bytes);
+    }
+    return rc;
+}
+
 static int register_locked(const uint8_t *h, size_t bytes, bool automatic, Resident **out)
 {
     /* whatever automatic entry shares bytes with the new range describes memory that now holds
@@ -258,13 +351,8 @@ static int register_locked(const uint8_t *h, size_t bytes, bool automatic, Resid
     }
     if (automatic) {
         while (g_auto_bytes && g_auto_bytes + bytes > cache_budget()) {
-            size_t lru = g_nres;
-            for (size_t i = 0; i < g_nres; i++)
-                if (g_res[i].automatic && g_res[i].tick <= g_call_tick &&
-                    (lru == g_nres || g_res[i].tick < g_res[lru].tick)) lru = i;
-            if (lru == g_nres) break;
-            if (!synced) { int rc = oxh_stream_sync(NULL); if (rc) return rc; synced = true; }
-            (void)drop_entry(lru);
+            if (!evict_one(NULL, &synced)) break;
+            g_evictions++;
         }
     }
     if (g_nres == g_cap) {
@@ -278,7 +366,7 @@ static int register_locked(const uint8_t *h, size_t bytes, bool automatic, Resid
         g_cap = nc;
     }
     void *d = NULL;
-    int rc = oxh_malloc(&d, bytes);
+    int rc = alloc_evicting(&d, bytes, NULL, &synced);
     if (rc) return rc;
     const uint64_t print = automatic ? host_print(h, bytes) : 0u;
     if ((rc = upload((uint8_t *)d, h, bytes))) {
@@ -294,6 +382,7 @@ static int register_locked(const uint8_t *h, size_t bytes, bool automatic, Resid
     r->print = print;
     r->tick = ++g_tick;
     if (automatic) g_auto_bytes += bytes;
+    slices_take(r);
     if (out) *out = r;
     return OXH_OK;
 }
@@ -391,6 +480,14 @@ int oxh_weight_stats(size_t *n_explicit, size_t *n_automatic, size_t *automatic_
     return OXH_OK;
 }
 
+size_t oxh_weight_evictions(void)
+{
+    pthread_mutex_lock(&g_lock);
+    const size_t n = g_evictions;
+    pthread_mutex_unlock(&g_lock);
+    return n;
+}
+
 /* Device address of `bytes` of weights starting at host pointer p.  Registered ranges resolve without
  * looking at the host bytes; anything else is uploaded on first sight and re-validated on every later
  * call (see the registry's header; with OXH_WEIGHT_CACHE=off every hit counts as changed and is uploaded
@@ -405,12 +502,14 @@ static int resident_ptr(const uint8_t *p, size_t bytes, const uint8_t **d, Resid
         r = find_automatic(p, bytes);
         if (r && r->tick <= g_call_tick) {         /* validated once per call is enough */
             const uint64_t now = cache_mode() == CACHE_OFF ? ~r->print : host_print(p, bytes);
-            if (now != r->print) {
-                /* same address and size, other contents: the caller reused the memory */
+            if (now != r->print || !slices_hold(r)) {
+                /* same address and size, other contents: the caller reused or patched the memory */
                 drop_prepared(r);
                 rc = oxh_stream_sync(NULL);
                 if (!rc) rc = upload(r->d, p, bytes);
-                r->print = cache_mode() == CACHE_OFF ? 0u : now;
+                /* a copy that did not arrive must not pass for the new contents on the next call */
+                r->print = (rc || cache_mode() == CACHE_OFF) ? ~now : now;
+                if (!rc) slices_take(r);
                 g_refreshes++;
             }
         } else if (!r) {
@@ -458,7 +557,23 @@ static int prepared_ptr(Resident *r, const uint8_t *p, size_t rows, size_t cols,
     }
     r->prep = np;
     void *nd = NULL;
-    int rc = oxh_malloc(&nd, bytes);
+    /* Giving up other entries for the memory may move this one inside the table (never drop it: the
+     * running call uses it), so it is looked up again by its range. */
+    const uint8_t *const rh = r->h;
+    const size_t rbytes = r->bytes;
+    const bool rauto = r->automatic;
+    pthread_mutex_lock(&g_lock);
+    bool synced = false;
+    if (rauto)
+        while (g_auto_bytes + bytes > cache_budget() && evict_one(r, &synced)) {
+            g_evictions++;
+            for (size_t i = 0; i < g_nres; i++)
+                if (g_res[i].h == rh && g_res[i].bytes == rbytes && g_res[i].automatic == rauto) r = &g_res[i];
+        }
+    int rc = alloc_evicting(&nd, bytes, rh, &synced);
+    for (size_t i = 0; i < g_nres; i++)
+        if (g_res[i].h == rh && g_res[i].bytes == rbytes && g_res[i].automatic == rauto) r = &g_res[i];
+    pthread_mutex_unlock(&g_lock);
     if (rc) return rc;
     if (form == OXH_PREP_Q2K_WIDE)    rc = oxh_q2_k_widen(r->d + off, rows, cols, nd, NULL);
     else if (form == OXH_PREP_Q6K_G8) rc = oxh_q6_k_group(r->d + off, rows, cols, nd, NULL);
@@ -469,6 +584,7 @@ static int prepared_ptr(Resident *r, const uint8_t *p, size_t rows, size_t cols,
     }
     Prepared *q = &r->prep[r->n_prep++];
     q->off = off; q->rows = rows; q->cols = cols; q->form = form; q->d = (uint8_t *)nd; q->bytes = bytes;
+    if (r->automatic) g_auto_bytes += bytes;
     *d = q->d;
     return OXH_OK;
 }

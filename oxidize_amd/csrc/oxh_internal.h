@@ -1,5 +1,6 @@
 /* oxh_internal.h — symbols shared between the HIP translation unit and the C
- * host layer of liboxhip; not part of the public ABI. */
+ * host layer of liboxhip; not part of the public ABI: the library's export list is
+ * made from the public headers, so nothing declared here is visible outside it. */
 #ifndef OXH_INTERNAL_H
 #define OXH_INTERNAL_H
 
@@ -41,6 +42,18 @@ int oxh_internal_multi_destroy(void *handle);
 int oxh_internal_copy16(void *dst, const void *src, size_t bytes, void *stream);
 /* Wait for a stream by polling it `spins` times before blocking. */
 int oxh_internal_stream_sync_spin(void *stream, unsigned spins);
+
+
+/* The functions behind include/oxhip_lab.h's table (not exported by name). */
+struct OxhPlan;
+struct OxhMoe;
+int oxh_debug_plan_stamps(struct OxhPlan *plan, uint64_t *d_stamps);
+int oxh_debug_plan_phantom(struct OxhPlan *plan, int on);
+int oxh_debug_moe_workspace_parts(const struct OxhMoe *m, size_t n_tok, size_t parts[12]);
+int oxh_debug_read_probe(const void *d_buf, size_t bytes, uint32_t *d_sink, void *stream);
+int oxh_debug_mfma_probe(int valu_per_mfma, int waves_per_simd, double *pops);
+int oxh_debug_subblock_sums(uint32_t qtype, const void *d_w, size_t rows, size_t cols, const void *d_act,
+                            int32_t *d_sums, void *stream);
 
 #ifdef __cplusplus
 }

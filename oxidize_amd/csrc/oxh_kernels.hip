@@ -30,6 +30,7 @@
 #include <mutex>
 
 #include "oxhip.h"
+#include "oxhip_lab.h"
 #include "oxh_internal.h"
 
 #pragma clang fp contract(off)
@@ -2661,6 +2662,25 @@ extern "C" int oxh_graph_destroy(void *graph_exec)
 {
     if (graph_exec) HIP_TRY(hipGraphExecDestroy((hipGraphExec_t)graph_exec));
     return OXH_OK;
+}
+
+extern "C" int oxh_mem_info(size_t *free_bytes, size_t *total_bytes)
+{
+    int rc = ensure_init();
+    if (rc) return rc;
+    size_t f = 0, t = 0;
+    HIP_TRY(hipMemGetInfo(&f, &t));
+    if (free_bytes) *free_bytes = f;
+    if (total_bytes) *total_bytes = t;
+    return OXH_OK;
+}
+
+/* The table behind include/oxhip_lab.h. */
+extern "C" const OxhLab *oxh_lab(void)
+{
+    static const OxhLab lab = { oxh_debug_plan_stamps, oxh_debug_plan_phantom, oxh_debug_moe_workspace_parts,
+                                oxh_debug_read_probe, oxh_debug_mfma_probe, oxh_debug_subblock_sums };
+    return &lab;
 }
 
 extern "C" int oxh_device_info(char *name, size_t name_len, int *n_cu, int *clock_mhz,

@@ -106,6 +106,7 @@ struct PlanSync {
     uint32_t copies;                /* copies of every counter that every workgroup gathers from, or 0: workgroup 0 gathers */
     uint32_t spin_limit;
     uint64_t *stamps;               /* measurement aid: [op][workgroup][8] clock readings, or NULL */
+    uint32_t *host_err;             /* page-locked host word that mirrors go[1], so that the next launch can be refused */
 };
 
 #define PLAN_STAMPS 8u
@@ -645,7 +646,7 @@ plan_wait(const PlanSync &sy, uint32_t target, int *s_ok, uint32_t lane, uint32_
                 if (++spins > sy.spin_limit || err != 0u) { ok = false; break; }
             }
             if (lane == 0u) {
-                if (!ok) cstore(sy.go + 1, 1u);
+                if (!ok) { cstore(sy.go + 1, 1u); cstore(sy.host_err, 1u); }
                 else if (sy.copies == 0u) cstore(sy.go, target);
             }
         } else {
@@ -655,7 +656,7 @@ plan_wait(const PlanSync &sy, uint32_t target, int *s_ok, uint32_t lane, uint32_
                 if (reached(g.x, target)) break;
                 if (g.y != 0u || ++spins > sy.spin_limit) {
                     ok = false;
-                    if (lane == 0u) cstore(sy.go + 1, 1u);
+                    if (lane == 0u) { cstore(sy.go + 1, 1u); cstore(sy.host_err, 1u); }
                     break;
                 }
             }
@@ -960,6 +961,7 @@ struct OxhPlan {
     PlanOp *d_run;                  /* k_plan_ext: the table it walks (d_ops stays the list of inputs) */
     uint32_t n_run;
     void *multi;                    /* a plan over a 32-value format: the table of GEMV launches (oxh_kernels.hip) */
+    uint32_t *h_err;                /* page-locked: set by the kernel when a wait gave up, read before every launch */
 };
 
 static const void *plan_kernel(const OxhPlan *pl)
@@ -1403,6 +1405,8 @@ extern "C" int oxh_plan_create(const OxhPlanOp *ops, size_t n_ops, OxhPlan **out
     for (size_t i = 0; run && i < n_run; i++)
         for (uint32_t k = 0; k < run[i].n_segs; k++) run[i].s[k].xq += (gaddr)(uintptr_t)pl->d_img;
     if (e == hipSuccess) e = hipMalloc((void **)&pl->d_sync, (PLAN_COPIES * PLAN_MAX_WG + 8u) * sizeof(uint32_t));
+    if (e == hipSuccess) e = hipHostMalloc((void **)&pl->h_err, 64, hipHostMallocDefault);
+    if (e == hipSuccess) *pl->h_err = 0u;
     if (e == hipSuccess) e = hipMemcpy(pl->d_ops, h, n_ops * sizeof(PlanOp), hipMemcpyHostToDevice);
     if (e == hipSuccess && pl->ext) e = hipMemcpy(pl->d_run, run, n_run * sizeof(PlanOp), hipMemcpyHostToDevice);
     if (e == hipSuccess) e = hipMemset(pl->d_sync, 0, (PLAN_COPIES * PLAN_MAX_WG + 8u) * sizeof(uint32_t));
@@ -1414,6 +1418,7 @@ extern "C" int oxh_plan_create(const OxhPlanOp *ops, size_t n_ops, OxhPlan **out
         if (pl->d_run) (void)hipFree(pl->d_run);
         if (pl->d_img) (void)hipFree(pl->d_img);
         if (pl->d_sync) (void)hipFree(pl->d_sync);
+        if (pl->h_err) (void)hipHostFree(pl->h_err);
         free(pl);
         return oxh_internal_errorf(e == hipErrorOutOfMemory ? OXH_ERR_NOMEM : OXH_ERR_HIP, "plan: %s", hipGetErrorString(e));
     }
@@ -1425,6 +1430,13 @@ extern "C" int oxh_plan_launch(OxhPlan *pl, void *stream)
 {
     if (!pl) return oxh_internal_errorf(OXH_ERR_ARG, "invalid argument: oxh_plan_launch: NULL plan");
     if (pl->multi) return oxh_internal_multi_launch(pl->multi, stream);
+    /* A launch in which a wait gave up leaves the counters unequal: every later launch would leave at its
+     * first wait with incomplete outputs.  The kernel notes it in a host word; from then on launches
+     * are refused until oxh_plan_status has reported the failure and reset the plan.  (A launch already
+     * queued behind the failing one cannot be recalled; oxh_plan_status after it reports the same.) */
+    if (*(volatile uint32_t *)pl->h_err != 0u)
+        return oxh_internal_errorf(OXH_ERR_TIMEOUT, "plan: an earlier launch gave up at a wait between operations; "
+                                   "call oxh_plan_status to reset the plan before launching it again");
     hipStream_t st = stream ? (hipStream_t)stream : (hipStream_t)oxh_internal_stream();
     PlanSync sy;
     sy.flags = pl->d_sync;
@@ -1441,6 +1453,7 @@ extern "C" int oxh_plan_launch(OxhPlan *pl, void *stream)
     }
     sy.spin_limit = pl->spin_limit;
     sy.stamps = pl->d_stamps;
+    sy.host_err = pl->h_err;
 #define PLAN_LAUNCH(K)                                                                                  \
     hipLaunchKernelGGL(K, dim3(pl->grid), dim3(1024), pl->lds_bytes, st, (const PlanOp *)pl->d_ops,    \
                        pl->n_ops, sy, pl->ld)
@@ -1487,11 +1500,17 @@ extern "C" int oxh_plan_prestaged(const OxhPlan *pl)
     return pl && pl->ext ? 1 : 0;
 }
 
-extern "C" int oxh_plan_set_spin_limit(OxhPlan *pl, uint32_t polls, int phantom_workgroup)
+extern "C" int oxh_plan_set_spin_limit(OxhPlan *pl, uint32_t polls)
 {
     if (!pl) return oxh_internal_errorf(OXH_ERR_ARG, "invalid argument: oxh_plan_set_spin_limit: NULL plan");
     pl->spin_limit = polls;
-    pl->phantom = phantom_workgroup ? 1u : 0u;
+    return OXH_OK;
+}
+
+extern "C" int oxh_debug_plan_phantom(OxhPlan *pl, int on)
+{
+    if (!pl) return oxh_internal_errorf(OXH_ERR_ARG, "invalid argument: plan_phantom: NULL plan");
+    pl->phantom = on ? 1u : 0u;
     return OXH_OK;
 }
 
@@ -1514,6 +1533,7 @@ extern "C" int oxh_plan_status(OxhPlan *pl, void *stream)
     /* a wait ran out: the counters are no longer equal, start them afresh */
     PLAN_TRY(hipMemset(pl->d_sync, 0, (PLAN_COPIES * PLAN_MAX_WG + 8u) * sizeof(uint32_t)));
     PLAN_TRY(hipDeviceSynchronize());
+    *(volatile uint32_t *)pl->h_err = 0u;
     return oxh_internal_errorf(OXH_ERR_TIMEOUT, "plan: a wait between operations ran out of polls (not every workgroup "
                                "was resident, or the limit is too small); the launch's outputs are incomplete");
 }
@@ -1527,6 +1547,7 @@ extern "C" int oxh_plan_destroy(OxhPlan *pl)
     if (pl->d_run) (void)hipFree(pl->d_run);
     if (pl->d_img) (void)hipFree(pl->d_img);
     if (pl->d_sync) (void)hipFree(pl->d_sync);
+    if (pl->h_err) (void)hipHostFree(pl->h_err);
     free(pl);
     if (e != hipSuccess) return oxh_internal_errorf(OXH_ERR_HIP, "HIP error in hipDeviceSynchronize: %s", hipGetErrorString(e));
     return OXH_OK;

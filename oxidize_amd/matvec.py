@@ -253,7 +253,7 @@ class MoeLayer:
     def parts(self, n_tok):
         """Offsets of the intermediates inside the workspace (test hook)."""
         v = (ctypes.c_size_t * 12)()
-        check(lib().oxh_debug_moe_workspace_parts(ctypes.byref(self.desc), n_tok, ctypes.byref(v)))
+        check(_lib.lab().moe_workspace_parts(ctypes.byref(self.desc), n_tok, ctypes.byref(v)))
         return dict(zip(self.PARTS, [int(x) for x in v]))
 
 
@@ -280,11 +280,11 @@ def q6_k_group(d_w, rows, cols, d_g8, stream=None):
 
 def read_probe(d_buf, nbytes, stream=None):
     """One launch that only reads `nbytes` at d_buf (measurement aid)."""
-    check(lib().oxh_debug_read_probe(ctypes.c_void_p(d_buf), nbytes, None, stream))
+    check(_lib.lab().read_probe(ctypes.c_void_p(d_buf), nbytes, None, stream))
 
 
 def debug_subblock_sums(qtype, d_w, rows, cols, d_act, d_sums, stream=None):
-    check(lib().oxh_debug_subblock_sums(qtype, ctypes.c_void_p(d_w), rows, cols,
+    check(_lib.lab().subblock_sums(qtype, ctypes.c_void_p(d_w), rows, cols,
                                         ctypes.c_void_p(d_act), ctypes.c_void_p(d_sums), stream))
 
 
@@ -334,7 +334,8 @@ class Plan:
         return out
 
     def set_spin_limit(self, polls, phantom_workgroup=False):
-        check(lib().oxh_plan_set_spin_limit(self.handle, polls, int(phantom_workgroup)))
+        check(lib().oxh_plan_set_spin_limit(self.handle, polls))
+        check(_lib.lab().plan_phantom(self.handle, int(phantom_workgroup)))
 
     def destroy(self):
         if self.handle:

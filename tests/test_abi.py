@@ -17,10 +17,12 @@ ROOT = oxlibs.ROOT
 
 
 def declared_functions():
-    text = open(os.path.join(ROOT, "include", "oxhip.h")).read()
-    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-    names = re.findall(r"\b((?:oxh|oc)_[a-z0-9_]+)\s*\(", text)
-    return sorted(set(names))
+    names = set()
+    for header in ("oxhip.h", "oxhip_lab.h"):
+        text = open(os.path.join(ROOT, "include", header)).read()
+        text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+        names.update(re.findall(r"\b((?:oxh|oc)_[a-z0-9_]+)\s*\(", text))
+    return sorted(names)
 
 
 def test_library_exports_every_declared_symbol():

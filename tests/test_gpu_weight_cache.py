@@ -155,3 +155,57 @@ def test_cache_budget_evicts_least_recently_used(oxh):
     assert n_cached >= 1 and cached_bytes >= rows * synth.row_bytes(13, cols)
     assert oxh.oxh_weight_clear() == 0
     assert stats(oxh)[:3] == (0, 0, 0)
+
+
+def test_a_few_bytes_patched_in_place_are_seen_within_the_stated_number_of_calls(oxh):
+    """What the default cache mode guarantees for an UNREGISTERED matrix that is edited in place at the same
+    address and size (a patched tensor, a merged adapter): 64 bytes in the middle of a 33 MB matrix, between
+    the fingerprint's samples.  The per-call check re-hashes two 16 KiB slices in turn against the hashes
+    taken at upload, so the edit is seen after at most ceil(bytes / 32 KiB) calls; until then the old copy
+    may be served (the stated limit), and oxh_weight_unregister makes the very next call see it."""
+    rows, cols = 14336, 4096
+    rb = synth.row_bytes(13, cols)
+    w = synth.weights(13, rows, cols, seed=77)
+    x = synth.normal(cols, seed=78)
+    first = run(13, w, rows, cols, x)
+    assert np.array_equal(first.view(np.uint32), oracle_matvec(13, w, rows, cols, x).view(np.uint32))
+    r0 = stats(oxh)[3]
+
+    # nibble bytes of one block of row 7001 (neither in the first / last 4 KiB nor on a sample)
+    row, at = 7001, 7001 * rb + 5 * 144 + 16 + 40
+    w[at:at + 64] ^= 0x5A
+    want = oracle_matvec(13, w, rows, cols, x)
+    assert want[row] != first[row]
+    limit = -(-w.nbytes // 32768)
+    seen_after = None
+    for call in range(1, limit + 1):
+        got = run(13, w, rows, cols, x)
+        if stats(oxh)[3] == r0 + 1:
+            seen_after = call
+            assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+            break
+        assert np.array_equal(got.view(np.uint32), first.view(np.uint32))      # the old copy, whole
+    assert seen_after is not None and seen_after <= limit
+
+    # the invalidate call: a second edit, then unregister, and the next call is right
+    w[at:at + 64] ^= 0x33
+    assert oxh.oxh_weight_unregister(w.ctypes.data) == 0
+    got = run(13, w, rows, cols, x)
+    assert np.array_equal(got.view(np.uint32), oracle_matvec(13, w, rows, cols, x).view(np.uint32))
+
+
+def test_rewritten_forms_count_towards_the_cache_and_go_with_their_entry(oxh):
+    """A cached Q6_K matrix keeps a regrouped copy next to it: the bytes cached grow by both, and dropping the
+    entry returns both."""
+    rows, cols = 256, 2048
+    w = synth.weights(16, rows, cols, seed=5)
+    x = synth.normal(cols, seed=6)
+    assert oxh.oxh_weight_clear() == 0
+    got = run(16, w, rows, cols, x)
+    assert np.array_equal(got.view(np.uint32), oracle_matvec(16, w, rows, cols, x).view(np.uint32))
+    assert stats(oxh)[2] == 2 * w.nbytes
+    assert oxh.oxh_weight_unregister(w.ctypes.data) == 0
+    assert stats(oxh)[:3] == (0, 0, 0)
+    free_b, total_b = ctypes.c_size_t(0), ctypes.c_size_t(0)
+    assert oxh.oxh_mem_info(ctypes.byref(free_b), ctypes.byref(total_b)) == 0
+    assert 0 < free_b.value <= total_b.value
