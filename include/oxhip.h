@@ -65,6 +65,13 @@ extern "C" {
 #define OXH_AL8    20u     /* the Q8_0 layout */
 #define OXH_IQ3_S  25u     /* codebook format, 3.44 bits per weight (oxk.h:63) */
 #define OXH_IQ1_XXXS 36u   /* codebook format, 1.19 bits per weight (quant.h:79) */
+/* The two 4-bit codebook formats of the reference's DEQUANTISE path (quant.h:122-123): its CPU API has
+ * no integer dot for them, a row is expanded to f32 and dotted with the f32 input (matvec.c:799-831).
+ * Here: oxh_gemv_segments_f32 (f32 inputs used as they are, no quantised activations), oxh_get_rows,
+ * and, opt-in, the host entry points (OXH_F32_PATH_TYPES=1; declined otherwise, like every other type
+ * of that path). */
+#define OXH_IQ4_NL 26u     /* 18-byte blocks of 32: f16 d + 16 nibble bytes          */
+#define OXH_IQ4_XS 27u     /* 136-byte blocks of 256: f16 d, 8 six-bit scales, nibbles */
 #define OXH_QTYPE_UNKNOWN 0xffffffffu
 
 /* Block geometry (oxidize-c/include/oxidize/oxk.h:46-66). */
@@ -84,6 +91,8 @@ extern "C" {
 #define OXH_Q8_K_BYTES   292u
 #define OXH_IQ3_S_BYTES  110u
 #define OXH_IQ1_XXXS_BYTES 38u
+#define OXH_IQ4_NL_BYTES 18u
+#define OXH_IQ4_XS_BYTES 136u
 
 /* Thread-local text of the last failure on this thread ("" if none). */
 const char *oxh_last_error(void);
@@ -103,6 +112,11 @@ int oxh_act_kind(uint32_t qtype, size_t cols);
  * oc_cuda_mmq_row_bytes (cuda_mmq.h:44-48); no padding is ever added, the
  * device layout is the on-disk layout. */
 size_t oxh_row_bytes(uint32_t qtype, size_t cols);
+/* Row bytes of a type this library runs through f32 inputs instead of an integer dot (OXH_IQ4_NL,
+ * OXH_IQ4_XS; cols a whole number of blocks), 0 for every other type or width.  oxh_act_kind and
+ * oxh_row_bytes stay 0 for these, as the reference's integer path declines them
+ * (oxidize-c/src/compute/matvec.c:99-127). */
+size_t oxh_f32_path_row_bytes(uint32_t qtype, size_t cols);
 /* Bytes of one quantised activation vector of `cols` values for `qtype`. */
 size_t oxh_act_bytes(uint32_t qtype, size_t cols);
 

@@ -852,8 +852,77 @@ void oxo_swiglu_f32(const float *gate, const float *up, float *out, size_t n)
 
 /* ─── dequantisation (layout cross-check only) ────────────────────────── */
 
+/* src/compute/quant_tables.h:13-16 */
+static const int8_t iq4_values[16] = { -127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113 };
+
+size_t oxo_dequant_path_row_bytes(uint32_t qtype, size_t cols)
+{
+    if (cols == 0) return 0;
+    if (qtype == OXO_IQ4_NL) return cols % 32u ? 0 : cols / 32u * 18u;
+    if (qtype == OXO_IQ4_XS) return cols % 256u ? 0 : cols / 256u * 136u;
+    return 0;
+}
+
+/* src/compute/quantization.c:1401-1421 (IQ4_NL), :1429-1459 (IQ4_XS) */
+static void dequant_iq4(uint32_t qtype, const uint8_t *row, size_t cols, float *out)
+{
+    if (qtype == OXO_IQ4_NL) {
+        for (size_t b = 0; b < cols / 32u; b++) {
+            const uint8_t *w = row + b * 18u;
+            const float d = oxo_f16_to_f32(rd_u16(w));
+            for (unsigned j = 0; j < 16; j++) {
+                out[32 * b + j] = d * (float)iq4_values[w[2 + j] & 15u];
+                out[32 * b + j + 16] = d * (float)iq4_values[w[2 + j] >> 4];
+            }
+        }
+        return;
+    }
+    for (size_t b = 0; b < cols / 256u; b++) {
+        const uint8_t *w = row + b * 136u;
+        const float d = oxo_f16_to_f32(rd_u16(w));
+        const uint32_t high = rd_u16(w + 2);
+        for (unsigned ib = 0; ib < 8; ib++) {
+            const int32_t lo4 = (w[4 + ib / 2] >> (4 * (ib % 2))) & 15;
+            const int32_t hi2 = (int32_t)((high >> (2 * ib)) & 3u) << 4;
+            const float dl = d * (float)((lo4 | hi2) - 32);
+            for (unsigned j = 0; j < 16; j++) {
+                const uint8_t q = w[8 + 16 * ib + j];
+                out[256 * b + 32 * ib + j] = dl * (float)iq4_values[q & 15u];
+                out[256 * b + 32 * ib + j + 16] = dl * (float)iq4_values[q >> 4];
+            }
+        }
+    }
+}
+
+int oxo_matvec_dequant(uint32_t qtype, const uint8_t *data, size_t rows, size_t cols, size_t row_bytes,
+                       const float *x, double *out, double *mag)
+{
+    const size_t rb = oxo_dequant_path_row_bytes(qtype, cols);
+    if (rb == 0 || row_bytes != rb) return 1;
+    float *tmp = (float *)malloc(cols * sizeof *tmp);
+    if (!tmp) return 2;
+    for (size_t r = 0; r < rows; r++) {
+        dequant_iq4(qtype, data + r * row_bytes, cols, tmp);
+        double s = 0.0, m = 0.0;
+        for (size_t i = 0; i < cols; i++) {
+            const double t = (double)tmp[i] * (double)x[i];
+            s += t;
+            m += t < 0 ? -t : t;
+        }
+        out[r] = s;
+        if (mag) mag[r] = m;
+    }
+    free(tmp);
+    return 0;
+}
+
 int oxo_dequant_row(uint32_t qtype, const uint8_t *row, size_t cols, float *out)
 {
+    if (qtype == OXO_IQ4_NL || qtype == OXO_IQ4_XS) {
+        if (oxo_dequant_path_row_bytes(qtype, cols) == 0) return 1;
+        dequant_iq4(qtype, row, cols, out);
+        return 0;
+    }
     if (qtype == OXO_AL5) qtype = OXO_Q4_0;     /* src/compute/quantization.c:781-800 */
     if (qtype == OXO_AL6) qtype = OXO_Q5_0;
     if (qtype == OXO_AL8) qtype = OXO_Q8_0;

@@ -68,6 +68,8 @@ enum {
     OXO_AL5_XS = 18,    /* f16 d + 32 three-bit codes in 12 bytes */
     OXO_AL6    = 19,    /* Q5_0 layout */
     OXO_AL8    = 20,    /* Q8_0 layout */
+    OXO_IQ4_NL = 26,    /* f16 d + 16 nibble bytes per 32 values (dequantise path only) */
+    OXO_IQ4_XS = 27,    /* f16 d + u16 scale high bits + 4 scale nibble bytes + 128 nibble bytes per 256 */
     OXO_IQ3_S  = 25,    /* f16 d + 64 grid codes + 8 ninth bits + 32 sign bytes + 4 scale bytes */
     OXO_IQ1_XXXS = 36,  /* f16 d + 32 codebook indices + 4 scale|sign bytes */
 };
@@ -212,6 +214,16 @@ void oxo_swiglu_f32(const float *gate, const float *up, float *out, size_t n);
  * :672-721, :723-766): the checker of the embedding lookup, and an independent
  * cross-check of the layouts behind the dot functions. */
 int oxo_dequant_row(uint32_t qtype, const uint8_t *row, size_t cols, float *out);
+/* The types without an integer dot (IQ4_NL, IQ4_XS) go through the reference's dequantise loop,
+ * src/compute/matvec.c:799-831: a row expanded to f32 (src/compute/quantization.c:1401-1459, restated
+ * in oxo_dequant_row and pinned to the compiled reference's bits), then dotted with the f32 input.
+ * The reference's dot runs in SIMD lanes whose order depends on the host, so this restatement sums in
+ * double: out[r] is the exact-order-free value, mag[r] = sum |w*x| the scale a tolerance goes by.
+ * Pinned against the compiled reference's oc_matvec_quantized within 4e-6 * mag (f32 lane sums).
+ * Returns 1 for any other type or a width that is not a whole number of blocks. */
+int oxo_matvec_dequant(uint32_t qtype, const uint8_t *data, size_t rows, size_t cols, size_t row_bytes,
+                       const float *x, double *out, double *mag);
+size_t oxo_dequant_path_row_bytes(uint32_t qtype, size_t cols);
 
 #ifdef __cplusplus
 }

@@ -68,6 +68,7 @@ SIGNATURES = {
     "oxh_act_kind": (I, [U32, Z]),
     "oxh_row_bytes": (Z, [U32, Z]),
     "oxh_act_bytes": (Z, [U32, Z]),
+    "oxh_f32_path_row_bytes": (Z, [U32, Z]),
     "oxh_quantize_q8_k": (I, [V, Z, Z, Z, V, V]),
     "oxh_quantize_q8_0": (I, [V, Z, Z, Z, V, V]),
     "oxh_gemv_segments": (I, [U32, ctypes.POINTER(OxhSegment), Z, Z, V, Z, Z, V]),

@@ -776,11 +776,55 @@ static int quantize(int kind, const float *d_x, size_t in_stride, size_t n_vec,
 
 /* ─── oc_matvec_quantized ─────────────────────────────────────────────── */
 
+/* OXH_F32_PATH_TYPES=1: oc_matvec_quantized over IQ4_NL / IQ4_XS runs on the device (weights expanded
+ * against the f32 input, oxh_gemv_segments_f32).  Off by default: the reference's CPU code takes these
+ * types through its dequantise loop (matvec.c:886-907), whose results this path matches to f32 rounding,
+ * not to the bit, so the default hands them back like every other type of that loop. */
+static int f32_path_enabled(void)
+{
+    static int cached = -1;
+    if (cached < 0) {
+        const char *e = getenv("OXH_F32_PATH_TYPES");
+        cached = (e && e[0] && e[0] != '0') ? 1 : 0;
+    }
+    return cached;
+}
+
+static int mv_one_f32_path(uint32_t qtype, const uint8_t *data, size_t rows, size_t cols, size_t row_bytes,
+                           const float *input, float *output)
+{
+    if (rows == 0) return OXH_OK;
+    if (!data || !input || !output) return bad_arg("oxh_matvec_quantized: NULL pointer");
+    size_t wbytes, obytes;
+    if (!mul_ok(rows, row_bytes, &wbytes) || !mul_ok(rows, sizeof(float), &obytes) || cols > SIZE_MAX / sizeof(float))
+        return bad_arg("oxh_matvec_quantized: size overflow");
+    int rc = oxh_init(0);
+    if (rc) return rc;
+    const uint8_t *d_w;
+    if ((rc = resident_ptr(data, wbytes, &d_w, NULL))) return rc;
+    if ((rc = reserve(&g_dx, cols * sizeof(float)))) return rc;
+    if ((rc = reserve(&g_dout, obytes))) return rc;
+    if ((rc = reserve_host(&g_hin, cols * sizeof(float)))) return rc;
+    if ((rc = reserve_host(&g_hout, obytes))) return rc;
+    memcpy(g_hin.p, input, cols * sizeof(float));
+    if ((rc = push_input(cols * sizeof(float)))) return rc;
+    const bool direct = obytes <= HOST_DIRECT_MAX;
+    OxhSegment seg = { d_w, (float *)(direct ? g_hout.p : g_dout.p), rows, 0, 0, NULL };
+    if ((rc = oxh_gemv_segments_f32(qtype, &seg, 1, cols, (const float *)g_dx.p, cols, NULL, 1, rows, NULL)))
+        return rc;
+    if (!direct && (rc = oxh_memcpy_d2h(g_hout.p, g_dout.p, obytes, NULL))) return rc;
+    if ((rc = oxh_stream_sync(NULL))) return rc;
+    memcpy(output, g_hout.p, obytes);
+    return OXH_OK;
+}
+
 static int mv_one(uint32_t qtype, const uint8_t *data, size_t rows,
                          size_t cols, size_t row_bytes, const float *input,
                          float *output, float *temp)
 {
     const int kind = eligible(qtype, cols, row_bytes);
+    if (!kind && f32_path_enabled() && row_bytes != 0 && oxh_f32_path_row_bytes(qtype, cols) == row_bytes)
+        return mv_one_f32_path(qtype, data, rows, cols, row_bytes, input, output);
     if (!kind) return declined("type/shape/stride has no integer path (or it is switched off)");
     if (temp == NULL) return declined("temp is NULL");      /* matvec.c:865 */
     if (rows == 0) return OXH_OK;

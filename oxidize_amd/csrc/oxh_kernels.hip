@@ -747,6 +747,14 @@ extern "C" size_t oxh_row_bytes(uint32_t qtype, size_t cols)
     return nb * bb;
 }
 
+extern "C" size_t oxh_f32_path_row_bytes(uint32_t qtype, size_t cols)
+{
+    if (cols == 0) return 0;
+    if (qtype == OXH_IQ4_NL) return cols % OXH_QK8_0 ? 0 : cols / OXH_QK8_0 * OXH_IQ4_NL_BYTES;
+    if (qtype == OXH_IQ4_XS) return cols % OXH_QK_K ? 0 : cols / OXH_QK_K * OXH_IQ4_XS_BYTES;
+    return 0;
+}
+
 extern "C" size_t oxh_act_bytes(uint32_t qtype, size_t cols)
 {
     const int kind = oxh_act_kind(qtype, cols);
@@ -1370,12 +1378,61 @@ extern "C" int oxh_gemv_segments(uint32_t qtype, const OxhSegment *segs, size_t 
     return launch_gemv(qtype, segs, n_segs, cols, io, n_vec, out_stride, nullptr, stream);
 }
 
+/* IQ4_NL / IQ4_XS: the weights expanded on the fly against the f32 inputs themselves, a launch per
+ * segment.  There is no quantised activation to hand back. */
+static int launch_gemv_iq4(uint32_t qtype, const OxhSegment *segs, size_t n_segs, size_t cols, const float *d_x,
+                           size_t x_stride, void *d_act_out, size_t n_vec, size_t out_stride, void *stream)
+{
+    int rc = ensure_init();
+    if (rc) return rc;
+    const size_t rb = oxh_f32_path_row_bytes(qtype, cols);
+    if (rb == 0) {
+        snprintf(g_err, sizeof g_err, "oxh_gemv_segments_f32: qtype %u with cols %zu is not a whole number of blocks", qtype, cols);
+        return OXH_DECLINED;
+    }
+    if (d_act_out) return arg_fail("oxh_gemv_segments_f32: these types run on the f32 inputs, there are no quantised activations to return");
+    if (n_segs == 0) return OXH_OK;
+    if (!segs) return arg_fail("oxh_gemv_segments_f32: NULL segments");
+    if (x_stride < cols || (x_stride & 3u) || ((uintptr_t)d_x & 15u))
+        return arg_fail("oxh_gemv_segments_f32: input rows must be 16-byte aligned and x_stride >= cols");
+    const size_t lds = 64u + cols * sizeof(float);
+    if (lds > 160u * 1024u || cols > 0xFFFFFFFFull || rb > 0xFFFFFFFFull) {
+        snprintf(g_err, sizeof g_err, "oxh_gemv_segments_f32: cols %zu too wide for one workgroup's LDS", cols);
+        return OXH_ERR_TOO_WIDE;
+    }
+    const bool xs = qtype == OXH_IQ4_XS;
+    const void *kern = xs ? reinterpret_cast<const void *>(k_gemv_iq4_f32<true>) : reinterpret_cast<const void *>(k_gemv_iq4_f32<false>);
+    HIP_TRY(hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+    hipStream_t st = pick_stream(stream);
+    const uint32_t n_cu = (uint32_t)(g_n_cu > 0 ? g_n_cu : 256);
+    for (size_t k = 0; k < n_segs; k++) {
+        const OxhSegment &sg = segs[k];
+        const size_t nv = sg.n_vec ? sg.n_vec : n_vec;
+        if (sg.rows == 0 || nv == 0) continue;
+        if (!sg.d_w || !sg.d_out) return arg_fail("oxh_gemv_segments_f32: NULL segment pointer");
+        if (sg.d_w_pair) return arg_fail("oxh_gemv_segments_f32: paired segments need an integer-path type");
+        if (out_stride < sg.rows || sg.rows > 0xFFFFFFFFull || nv > 0xFFFFFFFFull)
+            return arg_fail("oxh_gemv_segments_f32: out_stride < rows or too many rows");
+        /* enough workgroups for eight waves per SIMD at most, every wave with a row */
+        const uint32_t grid = (uint32_t)((sg.rows + 3u) / 4u < 8u * n_cu ? (sg.rows + 3u) / 4u : 8u * n_cu);
+        const float *x = d_x + sg.act_first * x_stride;
+        if (xs) hipLaunchKernelGGL(k_gemv_iq4_f32<true>, dim3(grid), dim3(256), lds, st, (const uint8_t *)sg.d_w, (uint32_t)sg.rows,
+                                   (uint32_t)cols, (uint32_t)rb, x, x_stride, (uint32_t)nv, sg.d_out, out_stride);
+        else    hipLaunchKernelGGL(k_gemv_iq4_f32<false>, dim3(grid), dim3(256), lds, st, (const uint8_t *)sg.d_w, (uint32_t)sg.rows,
+                                   (uint32_t)cols, (uint32_t)rb, x, x_stride, (uint32_t)nv, sg.d_out, out_stride);
+        HIP_TRY(hipGetLastError());
+    }
+    return OXH_OK;
+}
+
 extern "C" int oxh_gemv_segments_f32(uint32_t qtype, const OxhSegment *segs, size_t n_segs,
                                      size_t cols, const float *d_x, size_t x_stride,
                                      void *d_act_out, size_t n_vec, size_t out_stride,
                                      void *stream)
 {
     if (!d_x && n_segs) return arg_fail("oxh_gemv_segments_f32: NULL input");
+    if (qtype == OXH_IQ4_NL || qtype == OXH_IQ4_XS)
+        return launch_gemv_iq4(qtype, segs, n_segs, cols, d_x, x_stride, d_act_out, n_vec, out_stride, stream);
     const GemvIo io = { nullptr, d_x, x_stride, d_act_out, nullptr };
     return launch_gemv(qtype, segs, n_segs, cols, io, n_vec, out_stride, nullptr, stream);
 }
@@ -2045,8 +2102,11 @@ extern "C" int oxh_get_rows(uint32_t qtype, const void *d_w, size_t rows, size_t
     qtype = canon_qtype(qtype);
     if (n_ids == 0) return OXH_OK;
     if (!d_w || !d_ids || !d_out) return arg_fail("oxh_get_rows: NULL pointer");
-    /* every type with a matvec kernel but the codebook formats */
-    const size_t rb = (oxh_act_kind(qtype, cols) && !is_iq(qtype) && qtype != OXH_Q6_K_G8) ? oxh_row_bytes(qtype, cols) : 0;
+    /* every type with a matvec kernel but the codebook formats of the integer path; the 4-bit codebook
+     * formats of the dequantise path */
+    const bool iq4 = qtype == OXH_IQ4_NL || qtype == OXH_IQ4_XS;
+    const size_t rb = iq4 ? oxh_f32_path_row_bytes(qtype, cols)
+                          : (oxh_act_kind(qtype, cols) && !is_iq(qtype) && qtype != OXH_Q6_K_G8) ? oxh_row_bytes(qtype, cols) : 0;
     if (rb == 0) {
         snprintf(g_err, sizeof g_err, "oxh_get_rows: qtype %u with cols %zu has no kernel here", qtype, cols);
         return OXH_DECLINED;
@@ -2062,7 +2122,13 @@ extern "C" int oxh_get_rows(uint32_t qtype, const void *d_w, size_t rows, size_t
 #define OXH_GET_ROWS(KIND)                                                                   \
     hipLaunchKernelGGL(k_get_rows<KIND>, grid, block, 0, st, w, (uint32_t)rows, (uint32_t)cols, \
                        (uint32_t)rb, d_ids, d_out, out_stride)
-    if (is_q4k(qtype))          OXH_GET_ROWS(0);
+    if (iq4) {
+        if (qtype == OXH_IQ4_XS) hipLaunchKernelGGL(k_get_rows_iq4<true>, grid, block, 0, st, w, (uint32_t)rows, (uint32_t)cols,
+                                                    (uint32_t)rb, d_ids, d_out, out_stride);
+        else                     hipLaunchKernelGGL(k_get_rows_iq4<false>, grid, block, 0, st, w, (uint32_t)rows, (uint32_t)cols,
+                                                    (uint32_t)rb, d_ids, d_out, out_stride);
+    }
+    else if (is_q4k(qtype))     OXH_GET_ROWS(0);
     else if (is_q5k(qtype))     OXH_GET_ROWS(1);
     else if (qtype == OXH_Q6_K) OXH_GET_ROWS(2);
     else if (qtype == OXH_Q4_0) OXH_GET_ROWS(4);

@@ -19,10 +19,11 @@ Q4_0, Q4_1, Q5_0, Q5_1, Q8_0, Q4_K, Q5_K, Q6_K = 3, 4, 5, 6, 7, 13, 15, 16
 Q2_K, Q3_K = 8, 10                      # Q3_K also under ids 9 and 11 (the _S and _L variants)
 AL5_XS = 18
 IQ3_S, IQ1_XXXS = 25, 36                # codebook formats: f16 d, every other byte uniform
+IQ4_NL, IQ4_XS = 26, 27                 # 4-bit codebook formats: f16 d, every other byte uniform
 BLOCK_BYTES = {Q4_0: 18, Q4_1: 20, Q5_0: 22, Q5_1: 24, Q8_0: 34, Q4_K: 144, 12: 144, Q5_K: 176, 14: 176,
-               Q6_K: 210, Q2_K: 84, 9: 110, Q3_K: 110, 11: 110, AL5_XS: 14, IQ3_S: 110, IQ1_XXXS: 38}
+               Q6_K: 210, Q2_K: 84, 9: 110, Q3_K: 110, 11: 110, AL5_XS: 14, IQ3_S: 110, IQ1_XXXS: 38, IQ4_NL: 18, IQ4_XS: 136}
 BLOCK_ELEMS = {Q4_0: 32, Q4_1: 32, Q5_0: 32, Q5_1: 32, Q8_0: 32, Q4_K: 256, 12: 256, Q5_K: 256, 14: 256,
-               Q6_K: 256, Q2_K: 256, 9: 256, Q3_K: 256, 11: 256, AL5_XS: 32, IQ3_S: 256, IQ1_XXXS: 256}
+               Q6_K: 256, Q2_K: 256, 9: 256, Q3_K: 256, 11: 256, AL5_XS: 32, IQ3_S: 256, IQ1_XXXS: 256, IQ4_NL: 32, IQ4_XS: 256}
 
 
 def _lib():
@@ -63,7 +64,7 @@ def weights(qtype, rows, cols, seed=0, stream=0, sigma=None, out=None):
     if out is None:
         out = np.empty(nbytes, dtype=np.uint8)
     assert out.dtype == np.uint8 and out.size == nbytes and out.flags.c_contiguous
-    if qtype in (Q4_0, Q4_1, Q5_0, Q5_1, AL5_XS, IQ3_S, IQ1_XXXS):
+    if qtype in (Q4_0, Q4_1, Q5_0, Q5_1, AL5_XS, IQ3_S, IQ1_XXXS, IQ4_NL, IQ4_XS):
         _lib().oxs_fill_legacy(out.ctypes.data, n_blocks, seed, stream, 0.02 if sigma is None else sigma,
                                BLOCK_BYTES[qtype], int(qtype in (Q4_1, Q5_1)))
         return out

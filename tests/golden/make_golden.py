@@ -11,6 +11,7 @@ committed, this script documents how they were made.
     python tests/golden/make_golden.py legacy   # only legacy_formats.npz
     python tests/golden/make_golden.py q23_k    # only q23_k.npz
     python tests/golden/make_golden.py iq       # only iq_types.npz
+    python tests/golden/make_golden.py iq4      # only iq4_types.npz
 
 Every array is data: inputs and the reference's outputs for them.
 """
@@ -368,6 +369,37 @@ def iq_types(ref):
     np.savez_compressed(os.path.join(HERE, "iq_types.npz"), **out)
 
 
+def iq4_types(ref):
+    """iq4_types.npz: IQ4_NL (type id 26) and IQ4_XS (id 27), the 4-bit codebook formats of the reference's
+    dequantise path: rows expanded by oc_quant_dequant_row (raw xorshift bytes behind a finite f16 scale,
+    so every nibble, scale nibble and scale high-bit pattern occurs) and oc_matvec_quantized's outputs
+    (the dequantise loop, matvec.c:799-831; float bits of THIS host's SIMD dot, held to a tolerance)."""
+    rng = np.random.default_rng(20241127)
+    out = {}
+    for name, qt, bsize, belems in (("iq4_nl", 26, 18, 32), ("iq4_xs", 27, 136, 256)):
+        rows, nb = 6, 5
+        cols, rb = nb * belems, nb * bsize
+        w = xorshift_bytes(rows * rb, 0xC0FFEE ^ qt).reshape(rows * nb, bsize)
+        bits = finite_scale_bits(rng, rows * nb)
+        w[:, 0], w[:, 1] = bits & 0xFF, bits >> 8
+        w = np.ascontiguousarray(w.reshape(-1))
+        f = np.zeros((rows, cols), np.float32)
+        for r in range(rows):
+            assert ref.oc_quant_dequant_row(qt, w[r * rb:].ctypes.data, rb, f[r].ctypes.data, cols) == 0
+        out[name + "_w"], out[name + "_bits"] = w, f.view(np.uint32).copy()
+        out[name + "_shape"] = np.array([rows, cols, rb], np.int64)
+        rows, cols = 48, 1280
+        rb = synth.row_bytes(qt, cols)
+        wm = synth.weights(qt, rows, cols, seed=9, stream=qt)
+        x = synth.normal(cols, seed=9, stream=100 + qt)
+        o = np.zeros(rows, np.float32)
+        temp = np.zeros(cols, np.float32)
+        ref.oc_matvec_quantized(qt, wm.ctypes.data, rows, cols, rb, x.ctypes.data, o.ctypes.data, temp.ctypes.data)
+        out[name + "_api_w"], out[name + "_api_x"], out[name + "_api_out"] = wm, x, o.copy()
+        out[name + "_api_shape"] = np.array([rows, cols, rb], np.int64)
+    np.savez_compressed(os.path.join(HERE, "iq4_types.npz"), **out)
+
+
 def main():
     ref = oxlibs.ref()
     if ref is None:
@@ -386,6 +418,8 @@ def main():
         q23_k(ref)
     if only in (None, "iq"):
         iq_types(ref)
+    if only in (None, "iq4"):
+        iq4_types(ref)
     if only is not None:
         return
     rng = np.random.default_rng(20240607)

@@ -65,6 +65,8 @@ def oracle():
         lib.oxo_moe_ffn.argtypes = [U32, U32, V, V, V, Z, Z, Z, Z, ctypes.c_int, V, V, Z, V]
         lib.oxo_moe_ffn.restype = ctypes.c_int
         lib.oxo_dequant_row.argtypes = [U32, V, Z, V]; lib.oxo_dequant_row.restype = ctypes.c_int
+        lib.oxo_matvec_dequant.argtypes = [U32, V, Z, Z, Z, V, V, V]; lib.oxo_matvec_dequant.restype = ctypes.c_int
+        lib.oxo_dequant_path_row_bytes.argtypes = [U32, Z]; lib.oxo_dequant_path_row_bytes.restype = Z
         lib.oxo_rms_norm_f32.argtypes = [V, V, V, Z, F]; lib.oxo_rms_norm_f32.restype = None
         lib.oxo_swiglu_f32.argtypes = [V, V, V, Z]; lib.oxo_swiglu_f32.restype = None
         _ORACLE = lib
