@@ -595,7 +595,65 @@ plan_stage_finish(const OpHead &op, const XStage &xs, uint8_t *base, float *red,
             reinterpret_cast<int16_t *>(dst + 260)[l] = (int16_t)s16;
         }
     }
-    if (has_sout || has_fout) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    /* the side outputs are acknowledged where the trip that follows the passes begins (k_plan), or after
+     * the last staged input (k_plan_ext), before the barrier that precedes the announcement: nothing
+     * else is in flight there, and here the wait would hold up the workgroup that stores them, which
+     * every other workgroup then waits for */
+}
+
+/* Vectors of at most sixteen blocks in the chained kernel, staged the launches' own way: wave w takes
+ * block w, lane l its values 4l .. 4l+3 (stage_begin / stage_end of the launches, with the loads that may
+ * see another workgroup's stores made coherent).  In a chain every wave's weights are already on their
+ * way when the vector arrives, so nothing is gained by leaving the vector to four waves of sixteen values
+ * a lane: spread over sixteen waves the dependent chain from the vector's arrival to the staged bytes is
+ * shorter (32-layer chain 1.317 ms against 1.350 ms).  Same values, same order of the sum of squares,
+ * same bytes. */
+struct XUnit {
+    XRegs x, t, b;
+};
+
+__device__ __forceinline__ void
+plan_stage_issue_unit(const OpHead &op, XUnit &xu, uint32_t lane, uint32_t wave)
+{
+    const uint32_t pro = op.pro;
+    if (wave < op.blocks) {
+        const float *b = gptr<const float>(op.pro_b);
+        const uint32_t at = (wave * 256u + 4u * lane) * 4u;
+        xu.x = cload4(coh_buf(gptr<const float>(op.x)), at);
+        if (pro == GEMV_PRO_ADD_RMSNORM) xu.t = cload4(coh_buf(gptr<const float>(op.pro_add)), at);
+        if (pro == GEMV_PRO_SWIGLU) xu.b = cload4(coh_buf(b), at);
+        else if (pro != GEMV_PRO_NONE) xu.b = x_load4(b + wave * 256u + 4u * lane);      /* norm weights: constants */
+    }
+}
+
+template <int KIND /* 0 Q4_K/Q5_K layout, 1 Q6_K layout */>
+__device__ __forceinline__ void
+plan_stage_finish_unit(const OpHead &op, const XUnit &xu, uint8_t *base, float *red, bool storer,
+                       uint32_t lane, uint32_t wave)
+{
+    const uint32_t B = op.blocks, pro = op.pro;
+    const bool rms = pro == GEMV_PRO_RMSNORM || pro == GEMV_PRO_ADD_RMSNORM, add = pro == GEMV_PRO_ADD_RMSNORM;
+    XRegs xr = xu.x;
+    if (add) { xr.v0 += xu.t.v0; xr.v1 += xu.t.v1; xr.v2 += xu.t.v2; xr.v3 += xu.t.v3; }
+    float inv = 1.0f;
+    if (rms) {
+        float ss = 0.0f;
+        if (wave < B) ss += xr.v0 * xr.v0 + xr.v1 * xr.v1 + xr.v2 * xr.v2 + xr.v3 * xr.v3;
+        ss = wave_sum_f32(ss);
+        if (lane == 0u) red[wave] = ss;
+        __syncthreads();
+        const float tot = wave_sum_f32(lane < PLAN_W ? red[lane] : 0.0f);
+        inv = 1.0f / sqrtf(tot / (float)(B * 256u) + op.eps);
+    }
+    if (wave < B) {
+        const uint32_t at = (wave * 256u + 4u * lane) * 4u;
+        if (add && storer && op.pro_sum_out != 0u) cstore4(coh_buf(gptr<float>(op.pro_sum_out)), at, xr);
+        XRegs y = xr;
+        if (rms) y = prologue_apply<GEMV_PRO_RMSNORM>(xr, xu.b, inv);
+        else if (pro == GEMV_PRO_SWIGLU) y = prologue_apply<GEMV_PRO_SWIGLU>(xr, xu.b, inv);
+        if (pro != GEMV_PRO_NONE && storer && op.pro_out != 0u) cstore4(coh_buf(gptr<float>(op.pro_out)), at, y);
+        q8k_x_finish<KIND == 1>(y, B, wave, base, (storer && op.act_out) ? gptr<uint8_t>(op.act_out) : nullptr, lane);
+    }
 }
 
 /* ─── waiting for an operation to be complete on every workgroup ──────── */
@@ -711,6 +769,10 @@ k_plan(const PlanOp *__restrict__ ops, uint32_t n_ops, const PlanSync sy, const 
              * operation: those queue up in the memory pipeline (a compute unit takes in about 12 bytes
              * per cycle), and anything placed after them in program order waits for that queue. */
             plan_row_sums(terms, prev, po.blocks, po.term_stride, outs, ln);
+            /* a prologue's side outputs (stored while staging, by any wave of one workgroup) have to be
+             * acknowledged before the workgroup announces the operation: no load is in flight here, so
+             * the wait costs nothing unless such a store is still on its way */
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
             lds_barrier();
             plan_stamp(sy, i - 1u, 6, ln, wave);
             if (wave == 0u) {
@@ -741,20 +803,30 @@ k_plan(const PlanOp *__restrict__ ops, uint32_t n_ops, const PlanSync sy, const 
         XStage xs;
 #pragma unroll
         for (int u = 0; u < 4; u++) xs.x[u] = xs.t[u] = xs.b[u] = XRegs{ 0.f, 0.f, 0.f, 0.f };
+        XUnit xu;
+        xu.x = xu.t = xu.b = XRegs{ 0.f, 0.f, 0.f, 0.f };
+        /* vectors of at most sixteen blocks: a block per wave (plan_stage_issue_unit) */
+        const bool by_unit = op.blocks <= PLAN_W;
         /* what this wave owns of the next operation: scalar arithmetic, done while nothing waits for it */
         PWork nx = cur;
         if (i + 1u < n_ops) nx = plan_work(&tab[i + 1u], wave);
         if (op.wait == 0u) {
             /* nothing to wait for: the vector goes first and is there in a microsecond */
-            plan_stage_issue(op, xs, ln, wave);
+            if (by_unit) plan_stage_issue_unit(op, xu, ln, wave);
+            else         plan_stage_issue(op, xs, ln, wave);
             plan_prefetch<HAS_Q5>(cur, A, 0u, ln);
         } else {
             /* Wave 0 polls, and a poll comes back behind everything the wave asked for before it: its
              * own weights go out after the wait (behind its part of the vector; they are there before
-             * the vector is quantised), the other waves' before it. */
+             * the vector is quantised), the other waves' before it.  (Requesting the second set here as
+             * well, which the wait would seem to have time for, measured 1.42 ms against 1.35 ms for the
+             * 32-layer chain: the requests compete with the passes the slowest workgroups are still
+             * streaming.  Two polls in flight instead of one: 1.37 ms; a pause between polls: 1.34 ms
+             * and up against 1.32 ms.) */
             if (wave != 0u) plan_prefetch<HAS_Q5>(cur, A, 0u, ln);
             if (!plan_wait(sy, base + op.wait, s_ok, ln, wave)) return;
-            plan_stage_issue(op, xs, ln, wave);
+            if (by_unit) plan_stage_issue_unit(op, xu, ln, wave);
+            else         plan_stage_issue(op, xs, ln, wave);
             if (wave == 0u) plan_prefetch<HAS_Q5>(cur, A, 0u, ln);
         }
         plan_stamp(sy, i, 1, ln, wave);
@@ -767,8 +839,13 @@ k_plan(const PlanOp *__restrict__ ops, uint32_t n_ops, const PlanSync sy, const 
             asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
             plan_stamp(sy, i, 5, ln, wave);
         }
-        if (op.kind >= PLAN_Q6_K) plan_stage_finish<1>(op, xs, act, red, storer, ln, wave);
-        else                      plan_stage_finish<0>(op, xs, act, red, storer, ln, wave);
+        if (by_unit) {
+            if (op.kind >= PLAN_Q6_K) plan_stage_finish_unit<1>(op, xu, act, red, storer, ln, wave);
+            else                      plan_stage_finish_unit<0>(op, xu, act, red, storer, ln, wave);
+        } else {
+            if (op.kind >= PLAN_Q6_K) plan_stage_finish<1>(op, xs, act, red, storer, ln, wave);
+            else                      plan_stage_finish<0>(op, xs, act, red, storer, ln, wave);
+        }
         plan_prefetch<HAS_Q5>(cur, B, 1u, ln);
         plan_stamp(sy, i, 2, ln, wave);
         __syncthreads();
