@@ -215,7 +215,7 @@ def secondary_figures(mv, synth):
     d_x = mv.DeviceBuffer.from_host(x)
     d_o = mv.DeviceBuffer(rows * 4)
     for name, qt in (("q2_k", 8), ("q3_k", 10), ("q4_0", 3), ("q4_1", 4), ("q5_0", 5), ("q5_1", 6),
-                     ("iq3_s", 25), ("iq1_xxxs", 36)):
+                     ("iq3_s", 25), ("iq1_xxxs", 36), ("iq4_nl_f32_inputs", 26), ("iq4_xs_f32_inputs", 27)):
         w = synth.weights(qt, rows, cols, seed=0, stream=7)
         copies = [mv.DeviceBuffer.from_host(w) for _ in range(8)]
         segs = [mv.make_segments([(c.ptr, d_o.ptr, rows, 0)]) for c in copies]
@@ -411,12 +411,12 @@ def secondary_figures(mv, synth):
         c.free()
     d_x.free()
     d_o.free()
-    # Q8_0 lm_head (configuration 2), batch 1 and 8
+    # Q8_0 lm_head (configuration 2), batch 1, 2, 4 and 8
     rows, cols = 151936, 896
     w = synth.weights(Q80, rows, cols, seed=0, stream=5)
     copies = [mv.DeviceBuffer.from_host(w) for _ in range(3)]
     q8 = {}
-    for nv in (1, 8):
+    for nv in (1, 2, 4, 8):
         xs = synth.normal(nv * cols, seed=0, stream=6)
         d_x = mv.DeviceBuffer.from_host(xs)
         d_o = mv.DeviceBuffer(nv * rows * 4)
@@ -437,6 +437,36 @@ def secondary_figures(mv, synth):
     out["q8_0_lm_head_151936x896"] = q8
     for c in copies:
         c.free()
+    # the feed-forward matrices of the same configuration (4864 x 896 and 896 x 4864, 4.6 MB each) at batch
+    # 1, 2, 4 and 8: 48 distinct copies in turn (222 MB), single launches, launch gaps included
+    ffn = {}
+    for name, r_, c_ in (("gate_or_up_4864x896", 4864, 896), ("down_896x4864", 896, 4864)):
+        w = synth.weights(Q80, r_, c_, seed=0, stream=9)
+        copies = [mv.DeviceBuffer.from_host(w) for _ in range(48)]
+        per = {}
+        for nv in (1, 2, 4, 8):
+            d_x = mv.DeviceBuffer.from_host(synth.normal(nv * c_, seed=0, stream=10))
+            d_o = mv.DeviceBuffer(nv * r_ * 4)
+            d_qa = mv.DeviceBuffer(nv * mv.act_bytes(Q80, c_))
+            segs = [mv.make_segments([(c.ptr, d_o.ptr, r_, 0)]) for c in copies]
+            state = {"i": 0}
+
+            def run_ffn():
+                state["i"] += 1
+                mv.gemv_segments_f32(Q80, segs[state["i"] % 48], c_, d_x.ptr, c_, d_qa.ptr, nv, r_)
+
+            us = timed(run_ffn, 96, mv)
+            nbytes = w.nbytes + nv * 4 * (c_ + r_)
+            per["batch%d" % nv] = {"us": round(us, 2), "gbps": round(nbytes / us / 1e3, 1),
+                                   "frac_of_hbm_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBPS, 4)}
+            for b_ in (d_x, d_o, d_qa):
+                b_.free()
+        ffn[name] = per
+        for c in copies:
+            c.free()
+    ffn["note"] = ("a launch over 4.6 MB is paced by its dependent chain (launch, input, quantise, one pass, row sums), "
+                   "not by the bytes: the whole-step figure below is the one that streams")
+    out["q8_0_ffn_shapes_batch_1_to_8"] = ffn
     # configuration 2 as a whole decode step: the Qwen2.5-0.5B-shaped Q8_0 set (24 layers x {q/k/v, o,
     # gate/up, down} + the head, every matmul quantising its own f32 input to Q8_0; matrices of 0.9-9 MB
     # and the 145 MB head) as ONE launch (a plan over a 32-value format: the rows of all 97 operations
@@ -832,6 +862,9 @@ def main():
                                  if args.mode == "plan" else None,
                    "untimed_steps_before_warmup": spun,
                    "bytes_per_step": step_bytes},
+        "metric_scope": ("independent operations: the benchmark's configuration 1 gives every matmul its own N(0,1) "
+                         "input, so nothing orders the 128 matmuls of a step; `dependent_chain` is the same 32 layers "
+                         "as a model runs them"),
         "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBPS, 2),
         "tokens_per_s_equiv": round(args.steps / wall, 1),
         "gpu_event_ms_per_step": round(ev_ms / args.steps, 4),
@@ -839,15 +872,19 @@ def main():
         "roofline": {"bound": "hbm", "kernel": k_name,
                      "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": k_traffic,
-                     "traffic_source": "rocprofv3 --pmc summary under profiles/ (a constant in bench.py, not live)",
+                     "traffic_source": ("historical: the rocprofv3 --pmc summary under profiles/ for this kernel and workload "
+                                        "(a constant in bench.py, not measured in this run)"),
                      "bytes_per_launch": k_bytes, "us_per_launch": round(k_us, 3)},
         "step_other_modes": other_modes,
         "single_launches": per_launch,
     }
+    # the same 32 layers with a layer's real dependencies (residual + RMSNorm and SwiGLU fused in), beside
+    # the headline and not under `extra`: the headline's operations are independent, a model's are not
+    out["dependent_chain"] = chain_figure(mv, ds, args.steps)
     if not args.no_extra:
         from oxidize_amd import synth
         out["extra"] = secondary_figures(mv, synth)
-        out["extra"]["decode_chain_fused"] = chain_figure(mv, ds, args.steps)
+        out["extra"]["decode_chain_fused"] = out["dependent_chain"]
     out["cpu_baseline"] = None if args.no_cpu else cpu_baseline()
     if not args.no_cpu and out["cpu_baseline"]["kind"] == "reference" and isinstance(out.get("extra"), dict):
         one = cpu_baseline(layers_sample=2, min_seconds=1.5, cores=1)

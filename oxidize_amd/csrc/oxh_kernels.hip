@@ -1076,6 +1076,25 @@ static int launch_q80_mfma_segments(uint32_t qtype, const OxhSegment *segs, size
         if (rc) return rc;
         acts = (const uint8_t *)io.d_act_out;
     }
+    /* Tiles of 64 rows per workgroup.  With more than eight activations staged only one workgroup fits a
+     * compute unit, and a workgroup that owned one tile would ask for its rows, wait, compute and leave
+     * with nothing on its way meanwhile: such launches give a workgroup several tiles in a row (as many as
+     * leaves every unit four workgroups or so, at most eight), the next tile's rows requested while the
+     * current one is computed and the activations staged once for all of them: vocabulary head 151936 x
+     * 896 at 16 activations 73 -> 61 us.  With eight or fewer staged, two workgroups share a unit and
+     * cover for each other; there it measured 2-4 % slower and is not used.  OXH_Q80_MFMA_GROUPS fixes
+     * the number. */
+    size_t tiles = 0, most_nv = 0;
+    for (size_t i = 0; i < n_segs; i++) {
+        tiles += (segs[i].rows + 63u) / 64u;
+        const size_t nv = segs[i].n_vec ? segs[i].n_vec : n_vec_default;
+        if (segs[i].rows && nv > most_nv) most_nv = nv;
+    }
+    static const uint32_t forced_groups = env_u32("OXH_Q80_MFMA_GROUPS", 0, 0, 64);
+    const size_t per_cu4 = 4u * (size_t)(g_n_cu > 0 ? g_n_cu : 256);
+    uint32_t groups = forced_groups ? forced_groups : (most_nv > 8u ? (uint32_t)(tiles / per_cu4) : 1u);
+    if (groups < 1u) groups = 1u;
+    if (!forced_groups && groups > 8u) groups = 8u;
     SegTable t;
     memset(&t, 0, sizeof t);
     uint32_t wg = 0, n = 0;
@@ -1087,7 +1106,7 @@ static int launch_q80_mfma_segments(uint32_t qtype, const OxhSegment *segs, size
         t.s[n].act_first = (uint32_t)segs[i].act_first;
         t.s[n].nv = (uint32_t)(segs[i].n_vec ? segs[i].n_vec : n_vec_default);
         t.s[n].wg_begin = wg;
-        wg += (uint32_t)((segs[i].rows + 63u) / 64u);
+        wg += (uint32_t)((segs[i].rows + 64u * groups - 1u) / (64u * groups));
         n++;
     }
     t.n = n;
@@ -1097,7 +1116,7 @@ static int launch_q80_mfma_segments(uint32_t qtype, const OxhSegment *segs, size
     const size_t lds = mq80_lds_bytes((uint32_t)blocks, toks, 4u);
     hipStream_t st = pick_stream(stream);
 #define OXH_MQ80(LEG) hipLaunchKernelGGL((k_mfma_q8_0_segments<4, LEG>), dim3(wg), dim3(256), lds, st, t, \
-                                         (uint32_t)blocks, acts, out_stride, toks)
+                                         (uint32_t)blocks, acts, out_stride, toks, groups)
     switch (qtype) {
     case OXH_Q4_0:   OXH_MQ80(1); break;
     case OXH_Q4_1:   OXH_MQ80(2); break;
