@@ -412,6 +412,33 @@ int oxh_q2_k_widen(const void *d_w, size_t rows, size_t cols, void *d_wide, void
 #define OXH_Q6_K_G8 0x1009u
 int oxh_q6_k_group(const void *d_w, size_t rows, size_t cols, void *d_g8, void *stream);
 
+/* Q4_K / Q5_K stored tile-major for the matrix-core tile kernels: the rows are
+ * taken in groups of sixteen, and inside a group the sixteen blocks that share
+ * a block index lie next to each other, rows ascending:
+ *   block (row r, index b) at ((r / 16) * B + b) * 16 + r % 16   blocks,
+ * B = cols / 256.  A wave of the tile kernel fetches exactly such a run per
+ * super-block: in the file layout it is sixteen pieces of 144 (176) bytes a row
+ * apart, each straddling cache lines it shares with nothing else the wave
+ * wants; tile-major it is 2304 (2816) contiguous bytes, 18 (22) whole lines.
+ * The memory pipeline charges per line touched, so an expert launch with few
+ * tokens per expert runs 10-20 % faster from this form (Mixtral's gate/up at
+ * four tokens per expert: 59 -> 53 us per 264 MB).  The blocks themselves are
+ * unchanged and so is every result, to the bit.
+ *   The last group of a matrix whose rows are not a multiple of sixteen is
+ * padded with zero blocks: oxh_tile16_bytes() gives the size (0 for a type or
+ * width without this form).  Accepted under OXH_Q4_K_T16 / OXH_Q5_K_T16 by
+ * oxh_gemv_segments and oxh_gemv_segments_f32 with d_act_out (1 to 16
+ * activations per segment, every segment starting at a group boundary; such a
+ * launch always runs on the matrix cores) and by the expert layer (OxhMoe's
+ * qtype_gate_up / qtype_down; rows per expert in whole sixteens); everything
+ * else reads the file layout and declines these ids.  d_t16 != d_w, both 16-byte
+ * aligned.  No counterpart in the reference (its kernels read the file layout,
+ * oxk.c:812-897). */
+#define OXH_Q4_K_T16 0x100Au
+#define OXH_Q5_K_T16 0x100Bu
+size_t oxh_tile16_bytes(uint32_t qtype, size_t rows, size_t cols);
+int oxh_tile16(uint32_t qtype, const void *d_w, size_t rows, size_t cols, void *d_t16, void *stream);
+
 /* Embedding lookup: out[t*out_stride ..] = row d_ids[t] of a packed matrix,
  * expanded to f32 in the reference's dequantisation arithmetic (bit-identical
  * to oc_quant_dequant_row, oxidize-c/src/compute/quantization.c:2781-2795), so

@@ -82,6 +82,8 @@ SIGNATURES = {
     "oxh_plan_prestaged": (I, [V]),
     "oxh_plan_table_rows": (I, [V]),
     "oxh_q6_k_group": (I, [V, Z, Z, V, V]),
+    "oxh_tile16_bytes": (Z, [U32, Z, Z]),
+    "oxh_tile16": (I, [U32, V, Z, Z, V, V]),
     "oxh_plan_set_spin_limit": (I, [V, U32]),
     "oxh_plan_destroy": (I, [V]),
     "oxh_plan_deal": (I, [ctypes.POINTER(Z), ctypes.POINTER(I), Z, U32, ctypes.POINTER(U32), ctypes.POINTER(U32)]),

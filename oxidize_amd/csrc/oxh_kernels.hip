@@ -710,6 +710,8 @@ extern "C" int oxh_act_kind(uint32_t qtype, size_t cols)
     case OXH_IQ3_S:                     /* the two codebook formats the reference's integer path takes */
     case OXH_IQ1_XXXS: return (cols % OXH_QK_K == 0) ? 2 : 0;
     case OXH_Q6_K_G8:  return (cols % (8u * OXH_QK_K) == 0) ? 2 : 0;     /* whole groups of eight blocks per row */
+    case OXH_Q4_K_T16:
+    case OXH_Q5_K_T16: return (cols % OXH_QK_K == 0) ? 2 : 0;
     default:         return 0;
     }
 }
@@ -724,8 +726,10 @@ static size_t block_bytes(uint32_t qtype)
     case OXH_AL5_XS: return OXH_AL5_XS_BYTES;
     case OXH_Q8_0:   return OXH_Q8_0_BYTES;
     case OXH_Q4_K_S:
+    case OXH_Q4_K_T16:
     case OXH_Q4_K_M: return OXH_Q4_K_BYTES;
     case OXH_Q5_K_S:
+    case OXH_Q5_K_T16:
     case OXH_Q5_K_M: return OXH_Q5_K_BYTES;
     case OXH_Q6_K:
     case OXH_Q6_K_G8: return OXH_Q6_K_BYTES;
@@ -928,6 +932,13 @@ static hipError_t raise_all_lds_ceilings(void)
 
 static bool is_q4k(uint32_t qtype) { return qtype == OXH_Q4_K_S || qtype == OXH_Q4_K_M; }
 static bool is_q5k(uint32_t qtype) { return qtype == OXH_Q5_K_S || qtype == OXH_Q5_K_M; }
+/* the tile-major forms of Q4_K and Q5_K, which only the MFMA tile kernels read, and the file type whose
+ * arithmetic each one keeps */
+static bool is_t16(uint32_t qtype) { return qtype == OXH_Q4_K_T16 || qtype == OXH_Q5_K_T16; }
+static uint32_t t16_base(uint32_t qtype)
+{
+    return qtype == OXH_Q4_K_T16 ? OXH_Q4_K_M : (qtype == OXH_Q5_K_T16 ? OXH_Q5_K_M : qtype);
+}
 
 static uint32_t act_lds_bytes(uint32_t qtype, uint32_t blocks)
 {
@@ -1132,7 +1143,7 @@ static int launch_q80_mfma_segments(uint32_t qtype, const OxhSegment *segs, size
 
 static int launch_mmq_segments(uint32_t qtype, const OxhSegment *segs, size_t n_segs, size_t cols, size_t blocks,
                                const GemvIo &io, size_t n_vec_default, size_t n_acts,
-                               size_t out_stride, void *stream)
+                               size_t out_stride, void *stream, uint32_t tile_major = 0u)
 {
     typedef MmqGeom<1, 1, 4> G;
     if (blocks * 292u * 256u > 0xFFFFFFFFull) return arg_fail("gemv: cols too large");
@@ -1175,7 +1186,7 @@ static int launch_mmq_segments(uint32_t qtype, const OxhSegment *segs, size_t n_
         typedef MmqGeom<1, 1, 8> W4;
         static_assert(W4::ROWS == 128, "128-row tiles");
         hipLaunchKernelGGL((k_mmq_q4_k_segments<1, 1, 8, 3>), dim3(wg), dim3(512), 3 * W4::LDS_BYTES,
-                           pick_stream(stream), t, (uint32_t)blocks, acts, out_stride);
+                           pick_stream(stream), t, (uint32_t)blocks, acts, out_stride, tile_major);
         HIP_TRY(hipGetLastError());
         return OXH_OK;
     }
@@ -1184,16 +1195,17 @@ static int launch_mmq_segments(uint32_t qtype, const OxhSegment *segs, size_t n_
     static_assert(G6::ROWS == G::ROWS && G5::ROWS == G::ROWS, "segment tiling is shared by all formats");
     hipStream_t st = pick_stream(stream);
     const uint32_t nb = (uint32_t)blocks;
-#define OXH_SEG_LAUNCH(KERNEL, GEOM, KB)                                                              \
-    hipLaunchKernelGGL((KERNEL<1, 1, 4, KB>), dim3(wg), dim3(4 * 64), (KB) * GEOM::LDS_BYTES, st, t, nb, acts, out_stride)
+#define OXH_SEG_LAUNCH(KERNEL, GEOM, KB, ...)                                                         \
+    hipLaunchKernelGGL((KERNEL<1, 1, 4, KB>), dim3(wg), dim3(4 * 64), (KB) * GEOM::LDS_BYTES, st, t, nb, acts, \
+                       out_stride, ##__VA_ARGS__)
     if (mmq_deep_stages(wg)) {
         if (qtype == OXH_Q6_K) OXH_SEG_LAUNCH(k_mmq_q6_k_segments, G6, 2);
-        else if (is_q5k(qtype)) OXH_SEG_LAUNCH(k_mmq_q5_k_segments, G5, 2);
-        else OXH_SEG_LAUNCH(k_mmq_q4_k_segments, G, 2);
+        else if (is_q5k(qtype)) OXH_SEG_LAUNCH(k_mmq_q5_k_segments, G5, 2, tile_major);
+        else OXH_SEG_LAUNCH(k_mmq_q4_k_segments, G, 2, tile_major);
     } else {
         if (qtype == OXH_Q6_K) OXH_SEG_LAUNCH(k_mmq_q6_k_segments, G6, 1);
-        else if (is_q5k(qtype)) OXH_SEG_LAUNCH(k_mmq_q5_k_segments, G5, 1);
-        else OXH_SEG_LAUNCH(k_mmq_q4_k_segments, G, 1);
+        else if (is_q5k(qtype)) OXH_SEG_LAUNCH(k_mmq_q5_k_segments, G5, 1, tile_major);
+        else OXH_SEG_LAUNCH(k_mmq_q4_k_segments, G, 1, tile_major);
     }
 #undef OXH_SEG_LAUNCH
     HIP_TRY(hipGetLastError());
@@ -1246,6 +1258,16 @@ static int launch_gemv(uint32_t qtype, const OxhSegment *segs, size_t n_segs, si
         if (segs[i].rows && segs[i].act_first + nv > act_end) act_end = segs[i].act_first + nv;
     }
     if (total_rows == 0) return OXH_OK;
+    if (is_t16(qtype)) {
+        /* tile-major weights exist for the MFMA tile kernel alone, whatever the launch's size */
+        if (any_pair || dump || io.pro || (!io.d_acts && !io.d_act_out)) {
+            snprintf(g_err, sizeof g_err, "gemv: tile-major weights (type %u) take quantised activations or a buffer "
+                     "for them, and no paired segment, prologue or sub-block dump", qtype);
+            return OXH_DECLINED;
+        }
+        return launch_mmq_segments(t16_base(qtype), segs, n_segs, cols, blocks, io, n_vec_default, act_end,
+                                   out_stride, stream, 1u);
+    }
     if (any_pair && dump) return arg_fail("gemv: no sub-block dump of a paired launch");
     if (is_iq(qtype) && dump) return arg_fail("gemv: no sub-block dump for the codebook formats");
     if (!any_pair && gemv_wants_mfma(qtype, io, max_nv, dump, tiles64))
@@ -2217,6 +2239,36 @@ extern "C" int oxh_q6_k_group(const void *d_w, size_t rows, size_t cols, void *d
     return OXH_OK;
 }
 
+extern "C" size_t oxh_tile16_bytes(uint32_t qtype, size_t rows, size_t cols)
+{
+    const uint32_t q = canon_qtype(qtype);
+    if ((!is_q4k(q) && !is_q5k(q)) || cols == 0 || cols % OXH_QK_K) return 0;
+    return (rows + 15u) / 16u * 16u * (cols / OXH_QK_K) * block_bytes(q);
+}
+
+extern "C" int oxh_tile16(uint32_t qtype, const void *d_w, size_t rows, size_t cols, void *d_t16, void *stream)
+{
+    int rc = ensure_init();
+    if (rc) return rc;
+    if (rows == 0) return OXH_OK;
+    if (!d_w || !d_t16) return arg_fail("oxh_tile16: NULL pointer");
+    if (d_w == d_t16) return arg_fail("oxh_tile16: source and destination must differ");
+    const size_t bytes = oxh_tile16_bytes(qtype, rows, cols);
+    if (!bytes) {
+        snprintf(g_err, sizeof g_err, "oxh_tile16: type %u with cols %zu is not Q4_K or Q5_K in whole 256-blocks", qtype, cols);
+        return OXH_DECLINED;
+    }
+    if (((uintptr_t)d_w & 15u) || ((uintptr_t)d_t16 & 15u))
+        return arg_fail("oxh_tile16: source and destination must be 16-byte aligned");
+    const size_t pieces = bytes / 16u;
+    if (pieces > 0xFFFFFFFFull) return arg_fail("oxh_tile16: matrix too large");
+    hipLaunchKernelGGL(k_tile16, dim3((uint32_t)((pieces + 255u) / 256u)), dim3(256), 0, pick_stream(stream),
+                       (const uint8_t *)d_w, (uint8_t *)d_t16, (uint32_t)rows, (uint32_t)(cols / OXH_QK_K),
+                       (uint32_t)(block_bytes(canon_qtype(qtype)) / 16u), (uint32_t)pieces);
+    HIP_TRY(hipGetLastError());
+    return OXH_OK;
+}
+
 /* ─── mixture of experts ──────────────────────────────────────────────── */
 
 static size_t align256(size_t v) { return (v + 255u) & ~(size_t)255u; }
@@ -2232,11 +2284,14 @@ static int moe_layout(const OxhMoe *m, size_t n_tok, MoeLayout *l)
         return arg_fail("moe: n_expert must be 1..64");
     if (m->top_k == 0 || m->top_k > OXH_MOE_MAX_TOPK || m->top_k > m->n_expert)
         return arg_fail("moe: top_k must be 1..8 and at most n_expert");
-    const bool gu_ok = is_q4k(m->qtype_gate_up) || is_q5k(m->qtype_gate_up) || m->qtype_gate_up == OXH_Q6_K;
-    const bool dn_ok = is_q4k(m->qtype_down) || is_q5k(m->qtype_down) || m->qtype_down == OXH_Q6_K;
+    /* tile-major expert matrices are stacked in whole 16-row groups */
+    const bool gu_ok = is_q4k(m->qtype_gate_up) || is_q5k(m->qtype_gate_up) || m->qtype_gate_up == OXH_Q6_K ||
+                       (is_t16(m->qtype_gate_up) && m->ffn % 16u == 0);
+    const bool dn_ok = is_q4k(m->qtype_down) || is_q5k(m->qtype_down) || m->qtype_down == OXH_Q6_K ||
+                       (is_t16(m->qtype_down) && m->hidden % 16u == 0);
     if (!gu_ok || !dn_ok || oxh_act_kind(m->qtype_gate_up, m->hidden) != 2 || oxh_act_kind(m->qtype_down, m->ffn) != 2) {
         snprintf(g_err, sizeof g_err, "moe: expert matrices must be Q4_K, Q5_K or Q6_K with widths in whole "
-                 "256-blocks (types %u / %u, hidden %zu, ffn %zu)", m->qtype_gate_up, m->qtype_down, m->hidden, m->ffn);
+                 "256-blocks, tile-major ones with rows in whole sixteens (types %u / %u, hidden %zu, ffn %zu)", m->qtype_gate_up, m->qtype_down, m->hidden, m->ffn);
         return OXH_DECLINED;
     }
     if (n_tok == 0 || n_tok > 4096) return arg_fail("moe: n_tok must be 1..4096");
@@ -2312,6 +2367,8 @@ static int launch_experts_tiled(uint32_t qtype, const void *const *d_w, float *c
                                 size_t n_expert, size_t rows, size_t cols, const void *d_acts, size_t out_stride,
                                 const uint32_t *d_counts, const uint32_t *d_offsets, void *stream)
 {
+    const uint32_t tile_major = is_t16(qtype) ? 1u : 0u;
+    qtype = t16_base(qtype);
     typedef MmqGeom<TC, 1, WAVES> G;
     typedef Mmq6Geom<TC, 1, WAVES> G6;
     typedef MmqGeom<TC, 1, WAVES, true> G5;
@@ -2322,9 +2379,9 @@ static int launch_experts_tiled(uint32_t qtype, const void *const *d_w, float *c
     const uint8_t *acts = (const uint8_t *)d_acts;
     hipStream_t st = pick_stream(stream);
     const uint32_t nb = (uint32_t)blocks;
-#define OXH_EXP_LAUNCH(KERNEL, GEOM, KB)                                                              \
+#define OXH_EXP_LAUNCH(KERNEL, GEOM, KB, ...)                                                            \
     hipLaunchKernelGGL(KERNEL, dim3(wg), dim3(WAVES * 64), (KB) * GEOM::LDS_BYTES, st, t, nb, acts, out_stride, \
-                       d_counts, d_offsets)
+                       d_counts, d_offsets, ##__VA_ARGS__)
     /* one segment per expert and matrix, at most OXH_MAX_SEGS of them per launch */
     const size_t per_launch = OXH_MAX_SEGS / n_mat;
     for (size_t e0 = 0; e0 < n_expert; e0 += per_launch) {
@@ -2348,15 +2405,15 @@ static int launch_experts_tiled(uint32_t qtype, const void *const *d_w, float *c
          * launch is small, three in the 128-row one (Q4_K only) */
         if constexpr (TC == 1 && WAVES == 8) {
             if (!is_q4k(qtype)) return arg_fail("moe: the 128-row small tile exists for Q4_K only");
-            OXH_EXP_LAUNCH((k_mmq_q45_k_experts<1, 1, 8, false, 3>), G, 3);
+            OXH_EXP_LAUNCH((k_mmq_q45_k_experts<1, 1, 8, false, 3>), G, 3, tile_major);
         } else if (TC == 1 && mmq_deep_stages(wg)) {
             if (qtype == OXH_Q6_K) OXH_EXP_LAUNCH((k_mmq_q6_k_experts<TC, 1, WAVES, 2>), G6, 2);
-            else if (is_q5k(qtype)) OXH_EXP_LAUNCH((k_mmq_q45_k_experts<TC, 1, WAVES, true, 2>), G5, 2);
-            else OXH_EXP_LAUNCH((k_mmq_q45_k_experts<TC, 1, WAVES, false, 2>), G, 2);
+            else if (is_q5k(qtype)) OXH_EXP_LAUNCH((k_mmq_q45_k_experts<TC, 1, WAVES, true, 2>), G5, 2, tile_major);
+            else OXH_EXP_LAUNCH((k_mmq_q45_k_experts<TC, 1, WAVES, false, 2>), G, 2, tile_major);
         } else {
             if (qtype == OXH_Q6_K) OXH_EXP_LAUNCH((k_mmq_q6_k_experts<TC, 1, WAVES, 1>), G6, 1);
-            else if (is_q5k(qtype)) OXH_EXP_LAUNCH((k_mmq_q45_k_experts<TC, 1, WAVES, true, 1>), G5, 1);
-            else OXH_EXP_LAUNCH((k_mmq_q45_k_experts<TC, 1, WAVES, false, 1>), G, 1);
+            else if (is_q5k(qtype)) OXH_EXP_LAUNCH((k_mmq_q45_k_experts<TC, 1, WAVES, true, 1>), G5, 1, tile_major);
+            else OXH_EXP_LAUNCH((k_mmq_q45_k_experts<TC, 1, WAVES, false, 1>), G, 1, tile_major);
         }
     }
 #undef OXH_EXP_LAUNCH
@@ -2370,6 +2427,7 @@ static int launch_experts(uint32_t qtype, const void *const *d_w, float *const *
 {
     static const uint32_t big_from = env_u32("OXH_MOE_BIG_TILE_FROM", 24, 0, 4096);     /* 0 = never */
     const size_t avg_tokens = pairs / n_expert;
+    const uint32_t file_type = t16_base(qtype);
     if (big_from && avg_tokens >= big_from)
         return launch_experts_tiled<4, 8>(qtype, d_w, d_out, n_mat, n_expert, rows, cols, d_acts, out_stride,
                                           d_counts, d_offsets, stream);
@@ -2382,7 +2440,7 @@ static int launch_experts(uint32_t qtype, const void *const *d_w, float *const *
     static const uint32_t wide = env_u32("OXH_MOE_WIDE_SMALL", 1, 0, 1);
     const size_t cus = (size_t)(g_n_cu > 0 ? g_n_cu : 256);
     const size_t live = pairs < n_expert ? (pairs ? pairs : 1) : n_expert;
-    if (wide && is_q4k(qtype) && n_mat * n_expert * ((rows + 63) / 64) <= 2u * cus &&
+    if (wide && is_q4k(file_type) && n_mat * n_expert * ((rows + 63) / 64) <= 2u * cus &&
         n_mat * live * ((rows + 127) / 128) >= cus - cus / 8)
         return launch_experts_tiled<1, 8>(qtype, d_w, d_out, n_mat, n_expert, rows, cols, d_acts, out_stride,
                                           d_counts, d_offsets, stream);

@@ -278,6 +278,19 @@ def q6_k_group(d_w, rows, cols, d_g8, stream=None):
     check(lib().oxh_q6_k_group(ctypes.c_void_p(d_w), rows, cols, ctypes.c_void_p(d_g8), stream))
 
 
+Q4_K_T16, Q5_K_T16 = 0x100A, 0x100B
+
+
+def tile16_bytes(qtype, rows, cols):
+    """Bytes of a Q4_K / Q5_K matrix stored tile-major (rows padded to whole sixteens); 0 = no such form."""
+    return int(lib().oxh_tile16_bytes(qtype, rows, cols))
+
+
+def tile16(qtype, d_w, rows, cols, d_t16, stream=None):
+    """Rewrite a Q4_K / Q5_K matrix tile-major for the matrix-core tile kernels (Q4_K_T16 / Q5_K_T16)."""
+    check(lib().oxh_tile16(qtype, ctypes.c_void_p(d_w), rows, cols, ctypes.c_void_p(d_t16), stream))
+
+
 def read_probe(d_buf, nbytes, stream=None):
     """One launch that only reads `nbytes` at d_buf (measurement aid)."""
     check(_lib.lab().read_probe(ctypes.c_void_p(d_buf), nbytes, None, stream))

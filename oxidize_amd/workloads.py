@@ -309,11 +309,14 @@ class MoESet:
     stacked expert-major as the reference stores them (llama.c:4248-4251).
     Every expert's matrices are applied only to the tokens routed to it: ONE
     launch for all experts' gate+up, ONE for all experts' down, each expert a
-    segment with its own activation count."""
+    segment with its own activation count.  tile_major: the stacks are rewritten
+    once with oxh_tile16 and the launches read that form (same results, to the bit)."""
 
-    def __init__(self, n_expert=8, top_k=2, n_tok=16, hidden=4096, ffn=14336, seed=0, keep_host=False):
+    def __init__(self, n_expert=8, top_k=2, n_tok=16, hidden=4096, ffn=14336, seed=0, keep_host=False,
+                 tile_major=False):
         self.n_expert, self.top_k, self.n_tok = n_expert, top_k, n_tok
         self.hidden, self.ffn = hidden, ffn
+        self.qtype_run = mv.Q4_K_T16 if tile_major else Q4K
         self.logits = synth.normal(n_tok * n_expert, seed=seed, stream=4242).reshape(n_tok, n_expert)
         self.ids, self.gate_w = route_top_k(self.logits, top_k)
         self.offsets, self.pair_tok = group_by_expert(self.ids, n_expert)
@@ -325,6 +328,13 @@ class MoESet:
                                          ("down", hidden, ffn, 702)):
             w = synth.weights(Q4K, n_expert * rows, cols, seed=seed, stream=stream)
             self.w[name] = mv.DeviceBuffer.from_host(w)
+            if tile_major:
+                assert rows % 16 == 0
+                tiled = mv.DeviceBuffer(mv.tile16_bytes(Q4K, n_expert * rows, cols))
+                mv.tile16(Q4K, self.w[name].ptr, n_expert * rows, cols, tiled.ptr)
+                mv.sync()
+                self.w[name].free()
+                self.w[name] = tiled
             if keep_host:
                 self.host[name] = w
         self.x_tok = synth.normal(n_tok * hidden, seed=seed, stream=4300).reshape(n_tok, hidden)
@@ -358,10 +368,10 @@ class MoESet:
 
     def launch_step(self, stream=None):
         for segs in self.seg_gu:
-            mv.gemv_segments_f32(Q4K, segs, self.hidden, self.d_xg.ptr, self.hidden, self.d_act_x.ptr, 1,
+            mv.gemv_segments_f32(self.qtype_run, segs, self.hidden, self.d_xg.ptr, self.hidden, self.d_act_x.ptr, 1,
                                  self.ffn, stream)
         for segs in self.seg_dn:
-            mv.gemv_segments_f32(Q4K, segs, self.ffn, self.d_h.ptr, self.ffn, self.d_act_h.ptr, 1,
+            mv.gemv_segments_f32(self.qtype_run, segs, self.ffn, self.d_h.ptr, self.ffn, self.d_act_h.ptr, 1,
                                  self.hidden, stream)
 
     def outputs(self):

@@ -1,0 +1,152 @@
+"""Q4_K / Q5_K stored tile-major (oxh_tile16, OXH_Q4_K_T16 / OXH_Q5_K_T16): the rewrite is checked against
+a numpy statement of the layout the header documents; the tile kernels must give from it the bits they give
+from the file layout, which other tests hold to the oracle, in segment launches and in the expert layer."""
+import numpy as np
+import pytest
+
+import oxlibs
+from oxidize_amd import synth
+from oxidize_amd import matvec as mv
+
+pytestmark = pytest.mark.gpu
+Q4K, Q5K, Q6K = 13, 15, 16
+T16 = {Q4K: mv.Q4_K_T16, Q5K: mv.Q5_K_T16}
+WB = {Q4K: 144, Q5K: 176}
+
+
+def bits(a):
+    return np.ascontiguousarray(a).view(np.uint32)
+
+
+def tile_major(w, qtype, rows, cols):
+    """block (row r, index b) at ((r // 16) * B + b) * 16 + r % 16; the last group padded with zeros"""
+    nb, wb = cols // 256, WB[qtype]
+    groups = (rows + 15) // 16
+    padded = np.zeros((groups * 16, nb, wb), np.uint8)
+    padded[:rows] = w.reshape(rows, nb, wb)
+    return np.ascontiguousarray(padded.reshape(groups, 16, nb, wb).transpose(0, 2, 1, 3)).reshape(-1)
+
+
+def tiled_copy(qtype, w, rows, cols):
+    d_w = mv.DeviceBuffer.from_host(w)
+    n = mv.tile16_bytes(qtype, rows, cols)
+    assert n == (rows + 15) // 16 * 16 * synth.row_bytes(qtype, cols)
+    d_t = mv.DeviceBuffer(n)
+    mv.tile16(qtype, d_w.ptr, rows, cols, d_t.ptr)
+    mv.sync()
+    return d_w, d_t
+
+
+@pytest.mark.parametrize("qtype", [Q4K, Q5K])
+@pytest.mark.parametrize("rows,cols", [(1, 256), (16, 512), (100, 4096), (4096, 1024), (333, 14336)])
+def test_rewrite_is_the_documented_permutation(oxh, qtype, rows, cols):
+    w = synth.weights(qtype, rows, cols, seed=41, stream=rows)
+    d_w, d_t = tiled_copy(qtype, w, rows, cols)
+    got = d_t.download(np.uint8, d_t.nbytes)
+    assert np.array_equal(got, tile_major(w, qtype, rows, cols))
+
+
+def test_sizes_and_refusals(oxh):
+    assert mv.tile16_bytes(Q6K, 64, 256) == 0
+    assert mv.tile16_bytes(Q4K, 64, 300) == 0
+    assert mv.tile16_bytes(Q4K, 17, 512) == 32 * 2 * 144
+    d = mv.DeviceBuffer(1 << 16)
+    with pytest.raises(mv.OxhError):
+        mv.tile16(Q6K, d.ptr, 16, 256, d.ptr + 32768)
+    with pytest.raises(mv.OxhError):
+        mv.tile16(Q4K, d.ptr, 16, 256, d.ptr)           # in place
+    # the plain GEMV entry point and the prefill entry point read the file layout only
+    o = mv.DeviceBuffer(64 * 4)
+    x = mv.DeviceBuffer.from_host(synth.normal(256, seed=1, stream=1))
+    with pytest.raises(mv.OxhError):
+        mv.gemv_segments_f32(mv.Q4_K_T16, mv.make_segments([(d.ptr, o.ptr, 64, 0)]), 256, x.ptr, 256, None, 1, 64)
+
+
+@pytest.mark.parametrize("qtype", [Q4K, Q5K])
+@pytest.mark.parametrize("rows,cols,n_vec", [(64, 256, 1), (100, 4096, 4), (1000, 2048, 3), (4096, 4096, 8),
+                                             (777, 1024, 16), (14336, 4096, 5), (9, 512, 2)])
+def test_segment_launch_bits_equal_the_file_layout(oxh, qtype, rows, cols, n_vec):
+    w = synth.weights(qtype, rows, cols, seed=42, stream=rows + n_vec)
+    d_w, d_t = tiled_copy(qtype, w, rows, cols)
+    x = synth.normal(n_vec * cols, seed=42, stream=7000 + rows)
+    d_x = mv.DeviceBuffer.from_host(x)
+    acts = mv.DeviceBuffer(n_vec * mv.act_bytes(qtype, cols))
+    mv.quantize(qtype, d_x.ptr, cols, n_vec, cols, acts.ptr)
+    o1, o2, o3 = (mv.DeviceBuffer(n_vec * rows * 4) for _ in range(3))
+    # the file layout through the prefill entry point (always the tile kernel), tile-major through the
+    # segment entry points, with stored activations and with the quantiser in front
+    mv.mmq(qtype, d_w.ptr, rows, cols, acts.ptr, n_vec, o1.ptr, rows)
+    mv.gemv_segments(T16[qtype], mv.make_segments([(d_t.ptr, o2.ptr, rows, 0)]), cols, acts.ptr, n_vec, rows)
+    a2 = mv.DeviceBuffer(acts.nbytes)
+    mv.gemv_segments_f32(T16[qtype], mv.make_segments([(d_t.ptr, o3.ptr, rows, 0)]), cols, d_x.ptr, cols, a2.ptr,
+                         n_vec, rows)
+    mv.sync()
+    want = o1.download(np.float32, n_vec * rows)
+    assert np.array_equal(bits(o2.download(np.float32, n_vec * rows)), bits(want))
+    assert np.array_equal(bits(o3.download(np.float32, n_vec * rows)), bits(want))
+    # vector 0 against the oracle directly
+    o = oxlibs.oracle()
+    ref = np.zeros(rows, np.float32)
+    tmp = np.zeros(cols, np.float32)
+    x0 = np.ascontiguousarray(x[:cols])
+    assert o.oxo_matvec_quantized(qtype, w.ctypes.data, rows, cols, synth.row_bytes(qtype, cols), x0.ctypes.data,
+                                  ref.ctypes.data, tmp.ctypes.data) == 0
+    assert np.array_equal(bits(want[:rows]), bits(ref))
+
+
+def test_several_segments_with_their_own_counts(oxh):
+    """Expert-style launch: slices of one tile-major stack, each over its own run of activations."""
+    cols, rows, n_exp = 1024, 192, 5
+    counts = [3, 0, 16, 1, 7]
+    w = synth.weights(Q4K, n_exp * rows, cols, seed=43, stream=5)
+    d_w, d_t = tiled_copy(Q4K, w, n_exp * rows, cols)
+    n_act = sum(counts)
+    x = synth.normal(n_act * cols, seed=43, stream=6)
+    d_x = mv.DeviceBuffer.from_host(x)
+    acts = mv.DeviceBuffer(n_act * mv.act_bytes(Q4K, cols))
+    mv.quantize(Q4K, d_x.ptr, cols, n_act, cols, acts.ptr)
+    o1, o2 = mv.DeviceBuffer(n_act * rows * 4), mv.DeviceBuffer(n_act * rows * 4)
+    rb = synth.row_bytes(Q4K, cols)
+    seg_f, seg_t, first = [], [], 0
+    for e, c in enumerate(counts):
+        if c:
+            seg_f.append((d_w.ptr + e * rows * rb, o1.ptr + first * rows * 4, rows, first, c))
+            seg_t.append((d_t.ptr + e * rows * rb, o2.ptr + first * rows * 4, rows, first, c))
+        first += c
+    for segs in seg_f:
+        # file layout one segment at a time through the prefill entry point
+        mv.mmq(Q4K, segs[0], rows, cols, acts.ptr + segs[3] * mv.act_bytes(Q4K, cols), segs[4], segs[1], rows)
+    mv.gemv_segments(mv.Q4_K_T16, mv.make_segments(seg_t), cols, acts.ptr, 1, rows)
+    mv.sync()
+    assert np.array_equal(bits(o2.download(np.float32, n_act * rows)), bits(o1.download(np.float32, n_act * rows)))
+
+
+@pytest.mark.parametrize("qt_gu,qt_dn,n_tok", [(Q4K, Q4K, 16), (Q5K, Q4K, 5), (Q4K, Q6K, 9), (Q4K, Q4K, 200)])
+def test_expert_layer_bits_equal_the_file_layout(oxh, qt_gu, qt_dn, n_tok):
+    n_expert, top_k, hidden, ffn = 8, 2, 512, 1280
+    wg = synth.weights(qt_gu, n_expert * ffn, hidden, seed=44, stream=1)
+    wu = synth.weights(qt_gu, n_expert * ffn, hidden, seed=44, stream=2)
+    wd = synth.weights(qt_dn, n_expert * hidden, ffn, seed=44, stream=3)
+    d_g, t_g = tiled_copy(qt_gu, wg, n_expert * ffn, hidden)
+    d_u, t_u = tiled_copy(qt_gu, wu, n_expert * ffn, hidden)
+    if qt_dn in T16:
+        d_d, t_d = tiled_copy(qt_dn, wd, n_expert * hidden, ffn)
+    else:
+        d_d = t_d = mv.DeviceBuffer.from_host(wd)
+    logits = synth.normal(n_tok * n_expert, seed=44, stream=4)
+    x = synth.normal(n_tok * hidden, seed=44, stream=5)
+    d_l, d_x = mv.DeviceBuffer.from_host(logits), mv.DeviceBuffer.from_host(x)
+    y1, y2 = mv.DeviceBuffer(n_tok * hidden * 4), mv.DeviceBuffer(n_tok * hidden * 4)
+    plain = mv.MoeLayer(qt_gu, qt_dn, d_g.ptr, d_u.ptr, d_d.ptr, n_expert, top_k, hidden, ffn, True, max_tok=n_tok)
+    tiled = mv.MoeLayer(T16[qt_gu], T16.get(qt_dn, qt_dn), t_g.ptr, t_u.ptr, t_d.ptr, n_expert, top_k, hidden, ffn,
+                        True, max_tok=n_tok)
+    plain.forward(d_l.ptr, d_x.ptr, n_tok, y1.ptr)
+    tiled.forward(d_l.ptr, d_x.ptr, n_tok, y2.ptr)
+    mv.sync()
+    assert np.array_equal(bits(y2.download(np.float32, n_tok * hidden)), bits(y1.download(np.float32, n_tok * hidden)))
+
+
+def test_expert_layer_declines_rows_off_the_group_size(oxh):
+    d = mv.DeviceBuffer(1 << 20)
+    with pytest.raises(mv.OxhError):
+        mv.MoeLayer(mv.Q4_K_T16, Q4K, d.ptr, d.ptr, d.ptr, 4, 2, 512, 1288, True, max_tok=4)
