@@ -436,6 +436,26 @@ int oxh_q6_k_group(const void *d_w, size_t rows, size_t cols, void *d_g8, void *
  * oxk.c:812-897). */
 #define OXH_Q4_K_T16 0x100Au
 #define OXH_Q5_K_T16 0x100Bu
+/* Q8_0 has a tile-major form too (oxh_tile16 with OXH_Q8_0; cols in whole
+ * runs of four blocks, i.e. a multiple of 128): per 16-row group and run of
+ * four blocks one 2176-byte unit, seventeen whole cache lines,
+ *   [0..1023]    blocks 4c, 4c+1 as the matrix cores' operand wants them: the
+ *                16-byte piece at 16 * (16q + r) holds row r's values 8q..8q+7
+ *                of block 4c (bytes 0-7) and of block 4c+1 (bytes 8-15),
+ *   [1024..2047] blocks 4c+2, 4c+3 likewise,
+ *   [2048..2175] the f16 scales, row r's four at 2048 + 8r,
+ * units in the order (group, run).  A wave fetches a unit with two aligned
+ * 16-byte loads per lane and one 8-byte load, straight into the operand
+ * registers, where the file layout's 34-byte blocks (2-byte aligned, a row
+ * apart) have to be carried through LDS and shifted into place; launches with
+ * 2 to 16 activations per weight then stream a large matrix at about the rate
+ * of the single-activation kernel.  Accepted under OXH_Q8_0_T16 by
+ * oxh_gemv_segments and oxh_gemv_segments_f32 with d_act_out (Q8_0
+ * activations, 1 to 16 per segment, segments starting at group boundaries);
+ * results bit-identical to OXH_Q8_0.  A wave walks all of a row group's
+ * blocks by itself, so the form pays for matrices with many rows (a
+ * vocabulary head) and not for a few hundred long ones. */
+#define OXH_Q8_0_T16 0x100Cu
 size_t oxh_tile16_bytes(uint32_t qtype, size_t rows, size_t cols);
 int oxh_tile16(uint32_t qtype, const void *d_w, size_t rows, size_t cols, void *d_t16, void *stream);
 

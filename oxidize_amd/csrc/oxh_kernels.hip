@@ -699,6 +699,7 @@ extern "C" int oxh_act_kind(uint32_t qtype, size_t cols)
     case OXH_Q5_0:
     case OXH_Q5_1:
     case OXH_AL5_XS:
+    case OXH_Q8_0_T16:
     case OXH_Q8_0:   return (cols % OXH_QK8_0 == 0) ? 1 : 0;
     case OXH_Q2_K:
     case OXH_Q3_K_M:
@@ -724,6 +725,7 @@ static size_t block_bytes(uint32_t qtype)
     case OXH_Q5_0:   return OXH_Q5_0_BYTES;
     case OXH_Q5_1:   return OXH_Q5_1_BYTES;
     case OXH_AL5_XS: return OXH_AL5_XS_BYTES;
+    case OXH_Q8_0_T16:
     case OXH_Q8_0:   return OXH_Q8_0_BYTES;
     case OXH_Q4_K_S:
     case OXH_Q4_K_T16:
@@ -855,6 +857,13 @@ static hipError_t raise_all_lds_ceilings(void)
     OXH_RAISE(k_gemv_iq1_xxxs)
 #undef OXH_RAISE
     if ((e = raise_lds_ceiling(k_gemv_multi<0>)) != hipSuccess) return e;
+    if ((e = raise_lds_ceiling(k_q80t_segments<4, 2>)) != hipSuccess) return e;
+    if ((e = raise_lds_ceiling(k_q80t_segments<8, 2>)) != hipSuccess) return e;
+    if ((e = raise_lds_ceiling(k_q80t_segments<16, 2>)) != hipSuccess) return e;
+    if ((e = raise_lds_ceiling(k_q80t_segments<4, 3>)) != hipSuccess) return e;
+    if ((e = raise_lds_ceiling(k_q80t_segments<8, 3>)) != hipSuccess) return e;
+    if ((e = raise_lds_ceiling(k_q80t_segments<16, 3>)) != hipSuccess) return e;
+    if ((e = raise_lds_ceiling(k_q80t_segments<1, 2>)) != hipSuccess) return e;
     if ((e = raise_lds_ceiling(k_gemv_multi<1>)) != hipSuccess) return e;
     if ((e = raise_lds_ceiling(k_gemv_multi<2>)) != hipSuccess) return e;
     if ((e = raise_lds_ceiling(k_gemv_multi<3>)) != hipSuccess) return e;
@@ -939,6 +948,7 @@ static uint32_t t16_base(uint32_t qtype)
 {
     return qtype == OXH_Q4_K_T16 ? OXH_Q4_K_M : (qtype == OXH_Q5_K_T16 ? OXH_Q5_K_M : qtype);
 }
+/* (OXH_Q8_0_T16, the tile-major form of Q8_0, has a kernel of its own: k_q80t_segments) */
 
 static uint32_t act_lds_bytes(uint32_t qtype, uint32_t blocks)
 {
@@ -1141,6 +1151,79 @@ static int launch_q80_mfma_segments(uint32_t qtype, const OxhSegment *segs, size
     return OXH_OK;
 }
 
+/* Tile-major Q8_0: every wave streams a run of consecutive 16-row groups straight into registers.  Eight
+ * (or four) waves share a workgroup's staged activations; a launch with fewer groups than would give every
+ * CU four four-wave workgroups runs one wave per workgroup instead, so that a small matrix still spreads
+ * over the device.  Groups per wave: as many as leave about four workgroups per CU, at most 32; measured on
+ * the 151936 x 896 head, more and shorter waves win (one group per wave 31.9 us at eight activations, two
+ * 34.0, four 37): a wave keeps two to four units on their way, and it is the number of waves that fills the
+ * memory system
+ * (OXH_Q80T_GPW fixes the number, OXH_Q80T_UNROLL = 2 or 3 the units per register set, OXH_Q80T_WAVES the
+ * waves per workgroup). */
+static int launch_q80t_segments(const OxhSegment *segs, size_t n_segs, size_t cols, size_t blocks, const GemvIo &io,
+                                size_t n_vec_default, size_t n_acts, size_t out_stride, void *stream)
+{
+    const uint8_t *acts = (const uint8_t *)io.d_acts;
+    if (!acts) {
+        int rc = oxh_quantize_q8_0(io.d_x, io.x_stride, n_acts, cols, io.d_act_out, stream);
+        if (rc) return rc;
+        acts = (const uint8_t *)io.d_act_out;
+    }
+    size_t n_groups = 0, most_nv = 0;
+    for (size_t i = 0; i < n_segs; i++) {
+        n_groups += (segs[i].rows + 15u) / 16u;
+        const size_t nv = segs[i].n_vec ? segs[i].n_vec : n_vec_default;
+        if (segs[i].rows && nv > most_nv) most_nv = nv;
+        if (segs[i].rows > 0xFFFFFFF0ull / (blocks * 34u)) return arg_fail("gemv: segment too large");
+    }
+    if (blocks % 4u) {
+        snprintf(g_err, sizeof g_err, "gemv: tile-major Q8_0 needs columns in whole runs of four blocks (cols %zu)", cols);
+        return OXH_DECLINED;
+    }
+    (void)most_nv;
+    const size_t lds = blocks * Q80T_ACT_BLOCK;
+    if (lds > GEMV_LDS_LIMIT) {
+        snprintf(g_err, sizeof g_err, "gemv: %zu columns x 16 staged activations do not fit 160 KiB of LDS", cols);
+        return OXH_ERR_TOO_WIDE;
+    }
+    static const uint32_t forced_gpw = env_u32("OXH_Q80T_GPW", 0, 0, 1024);
+    static const uint32_t unroll = env_u32("OXH_Q80T_UNROLL", 2, 2, 3);
+    static const uint32_t forced_waves = env_u32("OXH_Q80T_WAVES", 0, 0, 16);
+    const size_t cus = (size_t)(g_n_cu > 0 ? g_n_cu : 256);
+    uint32_t waves = n_groups >= 32u * cus ? 8u : (n_groups >= 16u * cus ? 4u : 1u);
+    if (forced_waves == 4u || forced_waves == 8u || forced_waves == 16u) waves = forced_waves;
+    size_t gpw = forced_gpw ? forced_gpw : n_groups / (waves * 4u * cus);
+    if (gpw < 1u) gpw = 1u;
+    if (!forced_gpw && gpw > 32u) gpw = 32u;
+    SegTable t;
+    memset(&t, 0, sizeof t);
+    uint32_t wg = 0, n = 0;
+    for (size_t i = 0; i < n_segs; i++) {
+        if (segs[i].rows == 0) continue;
+        t.s[n].w = (const uint8_t *)segs[i].d_w;
+        t.s[n].out = segs[i].d_out;
+        t.s[n].rows = (uint32_t)segs[i].rows;
+        t.s[n].act_first = (uint32_t)segs[i].act_first;
+        t.s[n].nv = (uint32_t)(segs[i].n_vec ? segs[i].n_vec : n_vec_default);
+        t.s[n].wg_begin = wg;
+        const size_t groups = (segs[i].rows + 15u) / 16u;
+        wg += (uint32_t)((groups + waves * gpw - 1u) / (waves * gpw));
+        n++;
+    }
+    t.n = n;
+    for (uint32_t i = 1; i < 4 && i < n; i++) t.bound[i - 1] = t.s[i].wg_begin;
+    hipStream_t st = pick_stream(stream);
+#define OXH_Q80T(WAVES, U) hipLaunchKernelGGL((k_q80t_segments<WAVES, U>), dim3(wg), dim3(WAVES * 64), lds, st, t, \
+                                              (uint32_t)blocks, acts, out_stride, (uint32_t)gpw)
+    if (waves == 16u) { if (unroll >= 3u) OXH_Q80T(16, 3); else OXH_Q80T(16, 2); }
+    else if (waves == 8u) { if (unroll >= 3u) OXH_Q80T(8, 3); else OXH_Q80T(8, 2); }
+    else if (waves == 4u) { if (unroll >= 3u) OXH_Q80T(4, 3); else OXH_Q80T(4, 2); }
+    else OXH_Q80T(1, 2);
+#undef OXH_Q80T
+    HIP_TRY(hipGetLastError());
+    return OXH_OK;
+}
+
 static int launch_mmq_segments(uint32_t qtype, const OxhSegment *segs, size_t n_segs, size_t cols, size_t blocks,
                                const GemvIo &io, size_t n_vec_default, size_t n_acts,
                                size_t out_stride, void *stream, uint32_t tile_major = 0u)
@@ -1258,6 +1341,14 @@ static int launch_gemv(uint32_t qtype, const OxhSegment *segs, size_t n_segs, si
         if (segs[i].rows && segs[i].act_first + nv > act_end) act_end = segs[i].act_first + nv;
     }
     if (total_rows == 0) return OXH_OK;
+    if (qtype == OXH_Q8_0_T16) {
+        if (any_pair || dump || io.pro || (!io.d_acts && !io.d_act_out)) {
+            snprintf(g_err, sizeof g_err, "gemv: tile-major Q8_0 takes quantised activations or a buffer for them, and "
+                     "no paired segment, prologue or sub-block dump");
+            return OXH_DECLINED;
+        }
+        return launch_q80t_segments(segs, n_segs, cols, blocks, io, n_vec_default, act_end, out_stride, stream);
+    }
     if (is_t16(qtype)) {
         /* tile-major weights exist for the MFMA tile kernel alone, whatever the launch's size */
         if (any_pair || dump || io.pro || (!io.d_acts && !io.d_act_out)) {
@@ -2242,6 +2333,7 @@ extern "C" int oxh_q6_k_group(const void *d_w, size_t rows, size_t cols, void *d
 extern "C" size_t oxh_tile16_bytes(uint32_t qtype, size_t rows, size_t cols)
 {
     const uint32_t q = canon_qtype(qtype);
+    if (q == OXH_Q8_0) return (cols == 0 || cols % (4u * OXH_QK8_0)) ? 0 : (rows + 15u) / 16u * (cols / (4u * OXH_QK8_0)) * Q80T_UNIT;
     if ((!is_q4k(q) && !is_q5k(q)) || cols == 0 || cols % OXH_QK_K) return 0;
     return (rows + 15u) / 16u * 16u * (cols / OXH_QK_K) * block_bytes(q);
 }
@@ -2255,8 +2347,19 @@ extern "C" int oxh_tile16(uint32_t qtype, const void *d_w, size_t rows, size_t c
     if (d_w == d_t16) return arg_fail("oxh_tile16: source and destination must differ");
     const size_t bytes = oxh_tile16_bytes(qtype, rows, cols);
     if (!bytes) {
-        snprintf(g_err, sizeof g_err, "oxh_tile16: type %u with cols %zu is not Q4_K or Q5_K in whole 256-blocks", qtype, cols);
+        snprintf(g_err, sizeof g_err, "oxh_tile16: type %u with cols %zu is not Q4_K, Q5_K or Q8_0 in whole blocks", qtype, cols);
         return OXH_DECLINED;
+    }
+    if (canon_qtype(qtype) == OXH_Q8_0) {
+        if (((uintptr_t)d_w & 1u) || ((uintptr_t)d_t16 & 15u))
+            return arg_fail("oxh_tile16: the source must be 2-byte and the destination 16-byte aligned");
+        const size_t items = bytes / Q80T_UNIT * 16u;
+        if (items > 0xFFFFFFFFull) return arg_fail("oxh_tile16: matrix too large");
+        hipLaunchKernelGGL(k_q80_tile16, dim3((uint32_t)((items + 255u) / 256u)), dim3(256), 0, pick_stream(stream),
+                           (const uint8_t *)d_w, (uint8_t *)d_t16, (uint32_t)rows, (uint32_t)(cols / OXH_QK8_0),
+                           (uint32_t)items);      /* an item = (unit, row of its group) */
+        HIP_TRY(hipGetLastError());
+        return OXH_OK;
     }
     if (((uintptr_t)d_w & 15u) || ((uintptr_t)d_t16 & 15u))
         return arg_fail("oxh_tile16: source and destination must be 16-byte aligned");

@@ -278,7 +278,7 @@ def q6_k_group(d_w, rows, cols, d_g8, stream=None):
     check(lib().oxh_q6_k_group(ctypes.c_void_p(d_w), rows, cols, ctypes.c_void_p(d_g8), stream))
 
 
-Q4_K_T16, Q5_K_T16 = 0x100A, 0x100B
+Q4_K_T16, Q5_K_T16, Q8_0_T16 = 0x100A, 0x100B, 0x100C
 
 
 def tile16_bytes(qtype, rows, cols):

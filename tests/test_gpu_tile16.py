@@ -150,3 +150,93 @@ def test_expert_layer_declines_rows_off_the_group_size(oxh):
     d = mv.DeviceBuffer(1 << 20)
     with pytest.raises(mv.OxhError):
         mv.MoeLayer(mv.Q4_K_T16, Q4K, d.ptr, d.ptr, d.ptr, 4, 2, 512, 1288, True, max_tok=4)
+
+
+# ── Q8_0 ────────────────────────────────────────────────────────────────────
+Q80 = 7
+
+
+def q80_tile_major(w, rows, cols):
+    """per (16-row group, run of four blocks) a 2176-byte unit: the 16-byte piece at 16 * (16q + r) of half h
+    holds row r's values 8q..8q+7 of block 4c + 2h (bytes 0-7) and 4c + 2h + 1 (bytes 8-15); the scales of row
+    r at 2048 + 8r; the last group padded with zeros"""
+    nb = cols // 32
+    groups, runs = (rows + 15) // 16, nb // 4
+    padded = np.zeros((groups * 16, nb, 34), np.uint8)
+    padded[:rows] = w.reshape(rows, nb, 34)
+    g = padded.reshape(groups, 16, runs, 4, 34)                              # [group][row][run][k][34]
+    out = np.zeros((groups, runs, 2176), np.uint8)
+    for k in range(4):
+        for q in range(4):
+            for r in range(16):
+                at = 1024 * (k >> 1) + 16 * (16 * q + r) + 8 * (k & 1)
+                out[:, :, at:at + 8] = g[:, r, :, k, 2 + 8 * q:10 + 8 * q]
+        for r in range(16):
+            out[:, :, 2048 + 8 * r + 2 * k:2050 + 8 * r + 2 * k] = g[:, r, :, k, 0:2]
+    return out.reshape(-1)
+
+
+@pytest.mark.parametrize("rows,cols", [(1, 128), (16, 256), (100, 896), (4864, 896), (333, 4864)])
+def test_q8_0_rewrite_is_the_documented_permutation(oxh, rows, cols):
+    w = synth.weights(Q80, rows, cols, seed=45, stream=rows)
+    d_w = mv.DeviceBuffer.from_host(w)
+    n = mv.tile16_bytes(Q80, rows, cols)
+    assert n == (rows + 15) // 16 * (cols // 128) * 2176
+    d_t = mv.DeviceBuffer(n)
+    mv.tile16(Q80, d_w.ptr, rows, cols, d_t.ptr)
+    mv.sync()
+    assert np.array_equal(d_t.download(np.uint8, n), q80_tile_major(w, rows, cols))
+
+
+@pytest.mark.parametrize("rows,cols,n_vec", [(16, 128, 1), (100, 896, 4), (1000, 896, 8), (4864, 896, 2), (896, 4864, 8),
+                                             (777, 1024, 16), (20000, 896, 5), (9, 256, 3), (4100, 2048, 12)])
+def test_q8_0_segment_launch_bits_equal_the_file_layout(oxh, rows, cols, n_vec):
+    w = synth.weights(Q80, rows, cols, seed=46, stream=rows + n_vec)
+    d_w = mv.DeviceBuffer.from_host(w)
+    d_t = mv.DeviceBuffer(mv.tile16_bytes(Q80, rows, cols))
+    mv.tile16(Q80, d_w.ptr, rows, cols, d_t.ptr)
+    x = synth.normal(n_vec * cols, seed=46, stream=8000 + rows)
+    d_x = mv.DeviceBuffer.from_host(x)
+    a1, a2 = mv.DeviceBuffer(n_vec * mv.act_bytes(Q80, cols)), mv.DeviceBuffer(n_vec * mv.act_bytes(Q80, cols))
+    o1, o2, o3 = (mv.DeviceBuffer(n_vec * rows * 4) for _ in range(3))
+    mv.gemv_segments_f32(Q80, mv.make_segments([(d_w.ptr, o1.ptr, rows, 0)]), cols, d_x.ptr, cols, a1.ptr, n_vec, rows)
+    mv.gemv_segments_f32(mv.Q8_0_T16, mv.make_segments([(d_t.ptr, o2.ptr, rows, 0)]), cols, d_x.ptr, cols, a2.ptr,
+                         n_vec, rows)
+    mv.gemv_segments(mv.Q8_0_T16, mv.make_segments([(d_t.ptr, o3.ptr, rows, 0)]), cols, a1.ptr, n_vec, rows)
+    mv.sync()
+    want = o1.download(np.float32, n_vec * rows)
+    assert np.array_equal(a1.download(np.uint8, a1.nbytes), a2.download(np.uint8, a2.nbytes))
+    assert np.array_equal(bits(o2.download(np.float32, n_vec * rows)), bits(want))
+    assert np.array_equal(bits(o3.download(np.float32, n_vec * rows)), bits(want))
+
+
+def test_q8_0_several_segments_with_their_own_counts(oxh):
+    cols, rows = 896, 208
+    counts = [3, 16, 1, 7]
+    w = synth.weights(Q80, len(counts) * rows, cols, seed=47, stream=5)
+    d_w = mv.DeviceBuffer.from_host(w)
+    d_t = mv.DeviceBuffer(mv.tile16_bytes(Q80, len(counts) * rows, cols))
+    mv.tile16(Q80, d_w.ptr, len(counts) * rows, cols, d_t.ptr)
+    n_act = sum(counts)
+    d_x = mv.DeviceBuffer.from_host(synth.normal(n_act * cols, seed=47, stream=6))
+    acts = mv.DeviceBuffer(n_act * mv.act_bytes(Q80, cols))
+    mv.quantize(Q80, d_x.ptr, cols, n_act, cols, acts.ptr)
+    o1, o2 = mv.DeviceBuffer(n_act * rows * 4), mv.DeviceBuffer(n_act * rows * 4)
+    rb = synth.row_bytes(Q80, cols)
+    seg_f, seg_t, first = [], [], 0
+    for e, c in enumerate(counts):
+        seg_f.append((d_w.ptr + e * rows * rb, o1.ptr + first * rows * 4, rows, first, c))
+        seg_t.append((d_t.ptr + e * rows * rb, o2.ptr + first * rows * 4, rows, first, c))
+        first += c
+    mv.gemv_segments(Q80, mv.make_segments(seg_f), cols, acts.ptr, 1, rows)
+    mv.gemv_segments(mv.Q8_0_T16, mv.make_segments(seg_t), cols, acts.ptr, 1, rows)
+    mv.sync()
+    assert np.array_equal(bits(o2.download(np.float32, n_act * rows)), bits(o1.download(np.float32, n_act * rows)))
+
+
+def test_q8_0_widths_off_the_run_size_are_declined(oxh):
+    assert mv.tile16_bytes(Q80, 64, 96) == 0
+    assert mv.tile16_bytes(Q80, 17, 256) == 2 * 2 * 2176
+    d = mv.DeviceBuffer(1 << 16)
+    with pytest.raises(mv.OxhError):
+        mv.tile16(Q80, d.ptr, 16, 96, d.ptr + 32768)
