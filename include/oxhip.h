@@ -450,9 +450,10 @@ int oxh_q6_k_group(const void *d_w, size_t rows, size_t cols, void *d_g8, void *
  * apart) have to be carried through LDS and shifted into place; launches with
  * 2 to 16 activations per weight then stream a large matrix at about the rate
  * of the single-activation kernel.  Accepted under OXH_Q8_0_T16 by
- * oxh_gemv_segments and oxh_gemv_segments_f32 with d_act_out (Q8_0
- * activations, 1 to 16 per segment, segments starting at group boundaries);
- * results bit-identical to OXH_Q8_0.  A wave walks all of a row group's
+ * oxh_gemv_segments (Q8_0 activations) and oxh_gemv_segments_f32 (the
+ * workgroups quantise the f32 inputs themselves; d_act_out may be NULL), 1 to
+ * 16 activations per segment, segments starting at group boundaries; results
+ * bit-identical to OXH_Q8_0.  A wave walks all of a row group's
  * blocks by itself, so the form pays for matrices with many rows (a
  * vocabulary head) and not for a few hundred long ones. */
 #define OXH_Q8_0_T16 0x100Cu

@@ -857,13 +857,12 @@ static hipError_t raise_all_lds_ceilings(void)
     OXH_RAISE(k_gemv_iq1_xxxs)
 #undef OXH_RAISE
     if ((e = raise_lds_ceiling(k_gemv_multi<0>)) != hipSuccess) return e;
-    if ((e = raise_lds_ceiling(k_q80t_segments<4, 2>)) != hipSuccess) return e;
-    if ((e = raise_lds_ceiling(k_q80t_segments<8, 2>)) != hipSuccess) return e;
-    if ((e = raise_lds_ceiling(k_q80t_segments<16, 2>)) != hipSuccess) return e;
-    if ((e = raise_lds_ceiling(k_q80t_segments<4, 3>)) != hipSuccess) return e;
-    if ((e = raise_lds_ceiling(k_q80t_segments<8, 3>)) != hipSuccess) return e;
-    if ((e = raise_lds_ceiling(k_q80t_segments<16, 3>)) != hipSuccess) return e;
-    if ((e = raise_lds_ceiling(k_q80t_segments<1, 2>)) != hipSuccess) return e;
+    if ((e = raise_lds_ceiling(k_q80t_segments<4, 2, false>)) != hipSuccess) return e;
+    if ((e = raise_lds_ceiling(k_q80t_segments<8, 2, false>)) != hipSuccess) return e;
+    if ((e = raise_lds_ceiling(k_q80t_segments<1, 2, false>)) != hipSuccess) return e;
+    if ((e = raise_lds_ceiling(k_q80t_segments<4, 2, true>)) != hipSuccess) return e;
+    if ((e = raise_lds_ceiling(k_q80t_segments<8, 2, true>)) != hipSuccess) return e;
+    if ((e = raise_lds_ceiling(k_q80t_segments<1, 2, true>)) != hipSuccess) return e;
     if ((e = raise_lds_ceiling(k_gemv_multi<1>)) != hipSuccess) return e;
     if ((e = raise_lds_ceiling(k_gemv_multi<2>)) != hipSuccess) return e;
     if ((e = raise_lds_ceiling(k_gemv_multi<3>)) != hipSuccess) return e;
@@ -1158,17 +1157,10 @@ static int launch_q80_mfma_segments(uint32_t qtype, const OxhSegment *segs, size
  * the 151936 x 896 head, more and shorter waves win (one group per wave 31.9 us at eight activations, two
  * 34.0, four 37): a wave keeps two to four units on their way, and it is the number of waves that fills the
  * memory system
- * (OXH_Q80T_GPW fixes the number, OXH_Q80T_UNROLL = 2 or 3 the units per register set, OXH_Q80T_WAVES the
- * waves per workgroup). */
+ * (OXH_Q80T_GPW fixes the number, OXH_Q80T_WAVES the waves per workgroup). */
 static int launch_q80t_segments(const OxhSegment *segs, size_t n_segs, size_t cols, size_t blocks, const GemvIo &io,
                                 size_t n_vec_default, size_t n_acts, size_t out_stride, void *stream)
 {
-    const uint8_t *acts = (const uint8_t *)io.d_acts;
-    if (!acts) {
-        int rc = oxh_quantize_q8_0(io.d_x, io.x_stride, n_acts, cols, io.d_act_out, stream);
-        if (rc) return rc;
-        acts = (const uint8_t *)io.d_act_out;
-    }
     size_t n_groups = 0, most_nv = 0;
     for (size_t i = 0; i < n_segs; i++) {
         n_groups += (segs[i].rows + 15u) / 16u;
@@ -1180,18 +1172,33 @@ static int launch_q80t_segments(const OxhSegment *segs, size_t n_segs, size_t co
         snprintf(g_err, sizeof g_err, "gemv: tile-major Q8_0 needs columns in whole runs of four blocks (cols %zu)", cols);
         return OXH_DECLINED;
     }
-    (void)most_nv;
     const size_t lds = blocks * Q80T_ACT_BLOCK;
     if (lds > GEMV_LDS_LIMIT) {
         snprintf(g_err, sizeof g_err, "gemv: %zu columns x 16 staged activations do not fit 160 KiB of LDS", cols);
         return OXH_ERR_TOO_WIDE;
     }
     static const uint32_t forced_gpw = env_u32("OXH_Q80T_GPW", 0, 0, 1024);
-    static const uint32_t unroll = env_u32("OXH_Q80T_UNROLL", 2, 2, 3);
-    static const uint32_t forced_waves = env_u32("OXH_Q80T_WAVES", 0, 0, 16);
+    static const uint32_t forced_waves = env_u32("OXH_Q80T_WAVES", 0, 0, 8);
     const size_t cus = (size_t)(g_n_cu > 0 ? g_n_cu : 256);
     uint32_t waves = n_groups >= 32u * cus ? 8u : (n_groups >= 16u * cus ? 4u : 1u);
-    if (forced_waves == 4u || forced_waves == 8u || forced_waves == 16u) waves = forced_waves;
+    if (forced_waves == 1u || forced_waves == 4u || forced_waves == 8u) waves = forced_waves;
+    /* f32 inputs: with one or two activations per segment the workgroups quantise them themselves while
+     * they stage them (a launch less: head at one activation 27.4 against 30 us); with more, that work,
+     * repeated by every workgroup, costs more than the quantiser's launch (eight activations 36 against 32 us),
+     * and one-wave workgroups would each repeat all of it.  Without a buffer for the blocks there is no
+     * choice.  (OXH_Q80T_FUSE_NV moves the threshold.) */
+    static const uint32_t fuse_nv = env_u32("OXH_Q80T_FUSE_NV", 2, 0, 16);
+    bool fused = false;
+    uint8_t *acts = (uint8_t *)const_cast<void *>(io.d_acts);
+    if (!acts) {
+        fused = !io.d_act_out || (most_nv <= fuse_nv && waves >= 4u);
+        acts = (uint8_t *)io.d_act_out;
+        if (fused && io.x_stride > 0xFFFFFFFFull) return arg_fail("gemv: stride too large");
+        if (!fused) {
+            int rc = oxh_quantize_q8_0(io.d_x, io.x_stride, n_acts, cols, io.d_act_out, stream);
+            if (rc) return rc;
+        }
+    }
     size_t gpw = forced_gpw ? forced_gpw : n_groups / (waves * 4u * cus);
     if (gpw < 1u) gpw = 1u;
     if (!forced_gpw && gpw > 32u) gpw = 32u;
@@ -1213,12 +1220,12 @@ static int launch_q80t_segments(const OxhSegment *segs, size_t n_segs, size_t co
     t.n = n;
     for (uint32_t i = 1; i < 4 && i < n; i++) t.bound[i - 1] = t.s[i].wg_begin;
     hipStream_t st = pick_stream(stream);
-#define OXH_Q80T(WAVES, U) hipLaunchKernelGGL((k_q80t_segments<WAVES, U>), dim3(wg), dim3(WAVES * 64), lds, st, t, \
-                                              (uint32_t)blocks, acts, out_stride, (uint32_t)gpw)
-    if (waves == 16u) { if (unroll >= 3u) OXH_Q80T(16, 3); else OXH_Q80T(16, 2); }
-    else if (waves == 8u) { if (unroll >= 3u) OXH_Q80T(8, 3); else OXH_Q80T(8, 2); }
-    else if (waves == 4u) { if (unroll >= 3u) OXH_Q80T(4, 3); else OXH_Q80T(4, 2); }
-    else OXH_Q80T(1, 2);
+#define OXH_Q80T(WAVES, FUSED) hipLaunchKernelGGL((k_q80t_segments<WAVES, 2, FUSED>), dim3(wg), dim3(WAVES * 64), lds, \
+                                                  st, t, (uint32_t)blocks, acts, out_stride, (uint32_t)gpw, io.d_x,   \
+                                                  (uint32_t)io.x_stride)
+    if (waves == 8u) { if (fused) OXH_Q80T(8, true); else OXH_Q80T(8, false); }
+    else if (waves == 4u) { if (fused) OXH_Q80T(4, true); else OXH_Q80T(4, false); }
+    else { if (fused) OXH_Q80T(1, true); else OXH_Q80T(1, false); }
 #undef OXH_Q80T
     HIP_TRY(hipGetLastError());
     return OXH_OK;
@@ -1342,9 +1349,8 @@ static int launch_gemv(uint32_t qtype, const OxhSegment *segs, size_t n_segs, si
     }
     if (total_rows == 0) return OXH_OK;
     if (qtype == OXH_Q8_0_T16) {
-        if (any_pair || dump || io.pro || (!io.d_acts && !io.d_act_out)) {
-            snprintf(g_err, sizeof g_err, "gemv: tile-major Q8_0 takes quantised activations or a buffer for them, and "
-                     "no paired segment, prologue or sub-block dump");
+        if (any_pair || dump || io.pro) {
+            snprintf(g_err, sizeof g_err, "gemv: tile-major Q8_0 takes no paired segment, prologue or sub-block dump");
             return OXH_DECLINED;
         }
         return launch_q80t_segments(segs, n_segs, cols, blocks, io, n_vec_default, act_end, out_stride, stream);

@@ -208,6 +208,12 @@ def test_q8_0_segment_launch_bits_equal_the_file_layout(oxh, rows, cols, n_vec):
     assert np.array_equal(a1.download(np.uint8, a1.nbytes), a2.download(np.uint8, a2.nbytes))
     assert np.array_equal(bits(o2.download(np.float32, n_vec * rows)), bits(want))
     assert np.array_equal(bits(o3.download(np.float32, n_vec * rows)), bits(want))
+    # f32 inputs with nowhere to put the quantised blocks: the workgroups quantise for themselves
+    o4 = mv.DeviceBuffer(n_vec * rows * 4)
+    mv.gemv_segments_f32(mv.Q8_0_T16, mv.make_segments([(d_t.ptr, o4.ptr, rows, 0)]), cols, d_x.ptr, cols, None,
+                         n_vec, rows)
+    mv.sync()
+    assert np.array_equal(bits(o4.download(np.float32, n_vec * rows)), bits(want))
 
 
 def test_q8_0_several_segments_with_their_own_counts(oxh):
