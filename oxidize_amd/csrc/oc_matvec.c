@@ -532,6 +532,7 @@ static int bad_arg(const char *what);
 #define OXH_PREP_Q3K_AS_Q6K 1u      /* oxh_q3_k_as_q6_k */
 #define OXH_PREP_Q2K_WIDE   2u      /* oxh_q2_k_widen   */
 #define OXH_PREP_Q6K_G8     3u      /* oxh_q6_k_group   */
+#define OXH_PREP_Q80_T16    4u      /* oxh_tile16 of a Q8_0 matrix */
 
 /* The rewritten form of the rows x cols matrix at host pointer p inside registry entry r, made on first
  * use and kept with the entry (the reference prepares its batch rows once per matrix as well,
@@ -549,7 +550,11 @@ static int prepared_ptr(Resident *r, const uint8_t *p, size_t rows, size_t cols,
         }
     }
     size_t bytes;
-    if (!mul_ok(rows, cols / OXH_QK_K * OXH_Q6_K_BYTES, &bytes)) return bad_arg("prepared form: size overflow");
+    if (form == OXH_PREP_Q80_T16) {
+        bytes = oxh_tile16_bytes(OXH_Q8_0, rows, cols);
+        if (!bytes) return bad_arg("prepared form: no tile-major form of this width");
+    } else if (!mul_ok(rows, cols / OXH_QK_K * OXH_Q6_K_BYTES, &bytes))
+        return bad_arg("prepared form: size overflow");
     Prepared *np = (Prepared *)realloc(r->prep, (r->n_prep + 1) * sizeof *np);
     if (!np) {
         oxh_set_error("out of host memory growing the weight registry%s%s", NULL, NULL);
@@ -575,7 +580,8 @@ static int prepared_ptr(Resident *r, const uint8_t *p, size_t rows, size_t cols,
         if (g_res[i].h == rh && g_res[i].bytes == rbytes && g_res[i].automatic == rauto) r = &g_res[i];
     pthread_mutex_unlock(&g_lock);
     if (rc) return rc;
-    if (form == OXH_PREP_Q2K_WIDE)    rc = oxh_q2_k_widen(r->d + off, rows, cols, nd, NULL);
+    if (form == OXH_PREP_Q80_T16)     rc = oxh_tile16(OXH_Q8_0, r->d + off, rows, cols, nd, NULL);
+    else if (form == OXH_PREP_Q2K_WIDE) rc = oxh_q2_k_widen(r->d + off, rows, cols, nd, NULL);
     else if (form == OXH_PREP_Q6K_G8) rc = oxh_q6_k_group(r->d + off, rows, cols, nd, NULL);
     else                              rc = oxh_q3_k_as_q6_k(r->d + off, rows, cols, nd, NULL);
     if (rc) {
@@ -614,6 +620,35 @@ static void decode_form(uint32_t *qtype, Resident *entry, const uint8_t *data, s
     if (prepared_ptr(entry, data, rows, cols, OXH_PREP_Q6K_G8, &d) != OXH_OK) return;
     *d_w = d;
     *qtype = OXH_Q6_K_G8;
+}
+
+/* Q8_0 for batches of 2 to 16: the tile-major copy (oxh_tile16), made the first time such a batch runs
+ * over a matrix with enough rows to fill the device one 16-row group per wave (sixteen groups per compute
+ * unit; a vocabulary head) and kept with its registry entry next to the file layout, which single
+ * vectors and longer batches go on reading.  OXH_Q80_TILED=0 switches it off; no memory left, a width
+ * that is not a multiple of 128, or OXH_WEIGHT_CACHE=off leave the call on the file layout. */
+static int q80_tiled_enabled(void)
+{
+    static int cached = -1;
+    if (cached < 0) {
+        const char *e = getenv("OXH_Q80_TILED");
+        cached = (e && e[0] == '0') ? 0 : 1;
+    }
+    return cached;
+}
+
+static void batch_form(uint32_t *qtype, Resident *entry, const uint8_t *data, size_t rows, size_t cols, size_t n_vec,
+                       const uint8_t **d_w)
+{
+    const int n_cu = oxh_internal_n_cu();
+    if (*qtype != OXH_Q8_0 || !entry || n_vec < 2 || n_vec > 16 || cols % (4u * OXH_QK8_0) || !q80_tiled_enabled() ||
+        n_cu <= 0 || rows / 16u < 16u * (size_t)n_cu)
+        return;
+    if (entry->automatic && cache_mode() == CACHE_OFF) return;
+    const uint8_t *d;
+    if (prepared_ptr(entry, data, rows, cols, OXH_PREP_Q80_T16, &d) != OXH_OK) return;
+    *d_w = d;
+    *qtype = OXH_Q8_0_T16;
 }
 
 /* ─── device staging buffers (inputs, activations, outputs) ───────────── */
@@ -1130,8 +1165,11 @@ static int mv_batch(uint32_t qtype, const uint8_t *data, size_t rows,
         if (n_vec <= step) {
             /* one launch with the quantisation fused in; with room for the quantised activations a
              * launch of several vectors may run on the matrix cores (same results; the library decides) */
-            OxhSegment seg = { d_w, d_out, rows, 0, 0, NULL };
-            if ((rc = oxh_gemv_segments_f32(qtype, &seg, 1, cols, d_x, cols, g_dact.p, n_vec, rows, NULL)))
+            uint32_t run_type = qtype;
+            const uint8_t *run_w = d_w;
+            batch_form(&run_type, entry, data, rows, cols, n_vec, &run_w);
+            OxhSegment seg = { run_w, d_out, rows, 0, 0, NULL };
+            if ((rc = oxh_gemv_segments_f32(run_type, &seg, 1, cols, d_x, cols, g_dact.p, n_vec, rows, NULL)))
                 return rc;
         } else {
             /* every activation is quantised once; the 32-value formats then have a token-tiled kernel on

@@ -246,3 +246,43 @@ def test_q8_0_widths_off_the_run_size_are_declined(oxh):
     d = mv.DeviceBuffer(1 << 16)
     with pytest.raises(mv.OxhError):
         mv.tile16(Q80, d.ptr, 16, 96, d.ptr + 32768)
+
+
+def test_host_batch_keeps_a_tile_major_copy_of_a_tall_q8_0_matrix(oxh):
+    """oc_matvec_quantized_batch over a Q8_0 matrix with enough rows for a 16-row group per wave: batches of
+    2 to 16 run from a tile-major copy kept with the registry entry (counted in the cache's bytes), single
+    vectors and refilled buffers keep giving the oracle's bits."""
+    import ctypes
+    rows, cols, n_vec = 70000, 128, 4
+    rb = synth.row_bytes(Q80, cols)
+    w = synth.weights(Q80, rows, cols, seed=48, stream=1)
+    xs = synth.normal(n_vec * cols, seed=48, stream=2).reshape(n_vec, cols)
+    temp = np.zeros(cols, np.float32)
+    scratch = np.zeros(mv.batch_scratch_bytes(cols), np.uint8)
+
+    def cached_bytes():
+        v = [ctypes.c_size_t(0) for _ in range(4)]
+        assert oxh.oxh_weight_stats(*[ctypes.byref(t) for t in v]) == 0
+        return int(v[2].value)
+
+    def check():
+        outs = np.zeros((n_vec, rows), np.float32)
+        assert mv.matvec_quantized_batch(Q80, w, rows, cols, rb, xs, cols, outs, rows, n_vec, temp, scratch) == 0
+        o = oxlibs.oracle()
+        for v in range(n_vec):
+            want = np.zeros(rows, np.float32)
+            x = np.ascontiguousarray(xs[v])
+            assert o.oxo_matvec_quantized(Q80, w.ctypes.data, rows, cols, rb, x.ctypes.data, want.ctypes.data,
+                                          temp.ctypes.data) == 0
+            assert np.array_equal(bits(outs[v]), bits(want))
+
+    assert oxh.oxh_weight_clear() == 0
+    check()
+    assert cached_bytes() == w.nbytes + mv.tile16_bytes(Q80, rows, cols)
+    check()                                                 # the kept copy again
+    assert cached_bytes() == w.nbytes + mv.tile16_bytes(Q80, rows, cols)
+    w[:] = synth.weights(Q80, rows, cols, seed=49, stream=1)      # same buffer, other matrix: both copies go
+    check()
+    assert cached_bytes() == w.nbytes + mv.tile16_bytes(Q80, rows, cols)
+    assert oxh.oxh_cpu_fallback_calls() == 0
+    assert oxh.oxh_weight_clear() == 0
