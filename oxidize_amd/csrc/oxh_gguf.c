@@ -86,6 +86,8 @@ static const TypeRow k_types[] = {
     { 14, OXH_Q6_K, 256, OXH_Q6_K_BYTES },
     { 21, OXH_IQ3_S, 256, OXH_IQ3_S_BYTES },
     { 66, OXH_IQ1_XXXS, 256, OXH_IQ1_XXXS_BYTES },
+    { 20, OXH_IQ4_NL, 32, OXH_IQ4_NL_BYTES },    /* quantization.c:2954-2955 */
+    { 23, OXH_IQ4_XS, 256, OXH_IQ4_XS_BYTES },
     { 24, 31, 1, 1 },      /* I8  */
     { 25, 32, 1, 2 },      /* I16 */
     { 26, 33, 1, 4 },      /* I32 */
@@ -474,7 +476,9 @@ int oxh_gguf_register_all(OxhGguf *g, size_t *n_registered, size_t *bytes)
     for (size_t i = 0; i < g->n_tensors; i++) {
         OxhTensor *t = &g->tensors[i];
         if (t->resident) { n++; total += t->nbytes; continue; }
-        if (t->n_dims < 2 || t->nbytes == 0 || !oxh_act_kind(t->qtype, t->cols)) continue;
+        /* types with an integer path, and those that run on f32 inputs on the device */
+        if (t->n_dims < 2 || t->nbytes == 0 ||
+            (!oxh_act_kind(t->qtype, t->cols) && !oxh_f32_path_row_bytes(t->qtype, t->cols))) continue;
         const int rc = oxh_weight_register(t->data, t->nbytes);
         if (rc != OXH_OK) return rc;
         t->resident = 1;

@@ -1074,13 +1074,19 @@ static bool mmq_deep_stages(uint32_t wg)
 /* Launches over a 32-value format (Q8_0, Q4_0, Q4_1, Q5_0, Q5_1, AL5_XS) with five or more
  * activations per weight go to the MFMA kernel (OXH_Q80_MFMA_MIN_NV moves the threshold, 0 = never)
  * when the quantised activations exist or have somewhere to go and the staged activations fit LDS. */
-static bool q80_wants_mfma(uint32_t qtype, const GemvIo &io, size_t max_nv, size_t blocks, const int32_t *dump)
+static bool q80_wants_mfma(uint32_t qtype, const GemvIo &io, size_t max_nv, size_t blocks, const int32_t *dump,
+                           size_t tiles64)
 {
     static int min_nv = -1;
     if (min_nv < 0) min_nv = (int)env_u32("OXH_Q80_MFMA_MIN_NV", 5, 0, 64);
+    /* as for the K-quants, a launch of few tiles is paced by a wave's walk over its rows' blocks and stays on
+     * the dot kernel while that takes the batch (Q8_0, 5 / 6 / 8 activations: 4864 x 896 7.3 / 8.1 / 9.7 against
+     * 9.4 us, 896 x 4864 13.4 / 14.8 / 17.9 against 25.8 us); OXH_Q80_MFMA_MIN_TILES moves the threshold */
+    static const uint32_t min_tiles = env_u32("OXH_Q80_MFMA_MIN_TILES", (uint32_t)(g_n_cu > 0 ? g_n_cu : 256) / 2u, 0, 1u << 20);
     if (oxh_act_kind(qtype, 32) != 1 || dump || io.pro || min_nv == 0 || max_nv < (size_t)min_nv ||
         max_nv > MQ80_TOK)
         return false;
+    if (max_nv <= OXH_MAX_NV && tiles64 < min_tiles) return false;
     if (blocks * block_bytes(qtype) < 16u) return false;        /* rows shorter than one 16-byte piece */
     if ((size_t)mq80_lds_bytes((uint32_t)blocks, max_nv > 8 ? 16u : 8u, 4u) > GEMV_LDS_LIMIT) return false;
     return io.d_acts != nullptr || io.d_act_out != nullptr;
@@ -1370,7 +1376,7 @@ static int launch_gemv(uint32_t qtype, const OxhSegment *segs, size_t n_segs, si
     if (!any_pair && gemv_wants_mfma(qtype, io, max_nv, dump, tiles64))
         return launch_mmq_segments(qtype, segs, n_segs, cols, blocks, io, n_vec_default, act_end,
                                    out_stride, stream);
-    if (!any_pair && q80_wants_mfma(qtype, io, max_nv, blocks, dump))
+    if (!any_pair && q80_wants_mfma(qtype, io, max_nv, blocks, dump, tiles64))
         return launch_q80_mfma_segments(qtype, segs, n_segs, cols, blocks, io, n_vec_default, act_end,
                                         out_stride, stream);
     /* only that kernel takes 9 to 16 activations per weight */

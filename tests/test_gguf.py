@@ -126,6 +126,7 @@ def test_on_disk_type_ids_map_like_the_reference():
     lib = _lib.lib()
     table = {0: 0, 1: 1, 30: 2, 2: 3, 3: 4, 6: 5, 7: 6, 8: 7, 10: 8, 11: 9, 12: 13, 13: 15, 14: 16,
              24: 31, 25: 32, 26: 33, 27: 34, 28: 35,
+             21: 25, 66: 36, 20: 26, 23: 27,               # IQ3_S, IQ1_XXXS, IQ4_NL, IQ4_XS (:2949-2958)
              240: 17, 241: 20, 242: 19, 243: 18}           # AL family (quantization.c:2943-2947)
     for ggml, q in table.items():
         assert lib.oxh_qtype_from_ggml_id(ggml) == q
