@@ -641,6 +641,40 @@ def split_probe(mv, synth):
     mv.sync()
 
 
+def head_probe(mv, synth):
+    """For `rocprofv3` runs on the Q8_0 kernels of 2-16 activations: the 151936 x 896 vocabulary head at
+    eight activations, six launches from the file layout (k_mfma_q8_0_segments) and six from the tile-major
+    copy (k_q80t_segments), three copies of the weights in turn.  Prints nothing."""
+    Q80 = 7
+    rows, cols, nv = 151936, 896, 8
+    w = synth.weights(Q80, rows, cols, seed=0, stream=5)
+    copies = [mv.DeviceBuffer.from_host(w) for _ in range(3)]
+    tiled = [mv.DeviceBuffer(mv.tile16_bytes(Q80, rows, cols)) for _ in range(3)]
+    for c, t in zip(copies, tiled):
+        mv.tile16(Q80, c.ptr, rows, cols, t.ptr)
+    d_x = mv.DeviceBuffer.from_host(synth.normal(nv * cols, seed=0, stream=6))
+    d_o = mv.DeviceBuffer(nv * rows * 4)
+    d_qa = mv.DeviceBuffer(nv * mv.act_bytes(Q80, cols))
+    for qt, bufs in ((Q80, copies), (mv.Q8_0_T16, tiled)):
+        for i in range(6):
+            segs = mv.make_segments([(bufs[i % 3].ptr, d_o.ptr, rows, 0)])
+            mv.gemv_segments_f32(qt, segs, cols, d_x.ptr, cols, d_qa.ptr, nv, rows)
+    mv.sync()
+
+
+def moe_probe(mv, synth):
+    """For `rocprofv3` runs on the expert launches of configuration 4 (8 experts, top-2, 16 tokens, Q4_K):
+    six steps from the file layout, then six from tile-major expert stacks.  Prints nothing."""
+    from oxidize_amd.workloads import MoESet
+    for tile_major in (False, True):
+        ms = MoESet(seed=0, tile_major=tile_major)
+        for _ in range(6):
+            ms.launch_step()
+        mv.sync()
+        for buf in list(ms.w.values()) + [ms.d_xg, ms.d_h, ms.d_gate, ms.d_up, ms.d_down, ms.d_act_x, ms.d_act_h]:
+            buf.free()
+
+
 def mmq_probe(mv, synth):
     """For `rocprofv3 --pmc` runs on the MFMA kernel: quantise 512 activations
     of 4096 values, then three 14336 x 4096 x 512 launches.  Prints nothing."""
@@ -741,7 +775,7 @@ def main():
     ap.add_argument("--mode", choices=["plan", "graph", "launches"], default="plan",
                     help="a step as one persistent launch (default), as a HIP graph of 128 launches, or as 128 launches")
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary configurations")
-    ap.add_argument("--probe", choices=["traffic", "mmq", "q80step", "split"], help="run a counter-collection workload and exit")
+    ap.add_argument("--probe", choices=["traffic", "mmq", "q80step", "split", "head", "moe"], help="run a counter-collection workload and exit")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this path is built and measured on ONE GPU; --gpus %d is not supported "
@@ -763,6 +797,10 @@ def main():
     if args.probe == "split":
         from oxidize_amd import synth
         split_probe(mv, synth)
+        return 0
+    if args.probe in ("head", "moe"):
+        from oxidize_amd import synth
+        (head_probe if args.probe == "head" else moe_probe)(mv, synth)
         return 0
     if args.probe == "q80step":
         from oxidize_amd import synth
