@@ -2480,8 +2480,12 @@ extern "C" int oxh_moe_route(const float *d_logits, size_t n_tok, size_t n_exper
 template <int TC, int WAVES>
 static int launch_experts_tiled(uint32_t qtype, const void *const *d_w, float *const *d_out, size_t n_mat,
                                 size_t n_expert, size_t rows, size_t cols, const void *d_acts, size_t out_stride,
-                                const uint32_t *d_counts, const uint32_t *d_offsets, void *stream)
+                                const uint32_t *d_counts, const uint32_t *d_offsets, size_t max_tokens, void *stream)
 {
+    /* sixteen-token tiles take the token tile from the grid's second dimension: as many as an expert that
+     * every token chose would need */
+    const uint32_t ny = TC == 1 ? (uint32_t)((max_tokens + 15u) / 16u ? (max_tokens + 15u) / 16u : 1u) : 1u;
+    if (ny > 65535u) return arg_fail("moe: too many tokens for the sixteen-token tile");
     const uint32_t tile_major = is_t16(qtype) ? 1u : 0u;
     qtype = t16_base(qtype);
     typedef MmqGeom<TC, 1, WAVES> G;
@@ -2495,7 +2499,7 @@ static int launch_experts_tiled(uint32_t qtype, const void *const *d_w, float *c
     hipStream_t st = pick_stream(stream);
     const uint32_t nb = (uint32_t)blocks;
 #define OXH_EXP_LAUNCH(KERNEL, GEOM, KB, ...)                                                            \
-    hipLaunchKernelGGL(KERNEL, dim3(wg), dim3(WAVES * 64), (KB) * GEOM::LDS_BYTES, st, t, nb, acts, out_stride, \
+    hipLaunchKernelGGL(KERNEL, dim3(wg, ny), dim3(WAVES * 64), (KB) * GEOM::LDS_BYTES, st, t, nb, acts, out_stride, \
                        d_counts, d_offsets, ##__VA_ARGS__)
     /* one segment per expert and matrix, at most OXH_MAX_SEGS of them per launch */
     const size_t per_launch = OXH_MAX_SEGS / n_mat;
@@ -2538,14 +2542,15 @@ static int launch_experts_tiled(uint32_t qtype, const void *const *d_w, float *c
 
 static int launch_experts(uint32_t qtype, const void *const *d_w, float *const *d_out, size_t n_mat,
                           size_t n_expert, size_t rows, size_t cols, const void *d_acts, size_t out_stride,
-                          const uint32_t *d_counts, const uint32_t *d_offsets, size_t pairs, void *stream)
+                          const uint32_t *d_counts, const uint32_t *d_offsets, size_t pairs, size_t max_tokens,
+                          void *stream)
 {
     static const uint32_t big_from = env_u32("OXH_MOE_BIG_TILE_FROM", 24, 0, 4096);     /* 0 = never */
     const size_t avg_tokens = pairs / n_expert;
     const uint32_t file_type = t16_base(qtype);
     if (big_from && avg_tokens >= big_from)
         return launch_experts_tiled<4, 8>(qtype, d_w, d_out, n_mat, n_expert, rows, cols, d_acts, out_stride,
-                                          d_counts, d_offsets, stream);
+                                          d_counts, d_offsets, max_tokens, stream);
     /* few rows per expert (a down projection): the 64-row tile would give at most two workgroups per CU;
      * Q4_K takes 128 rows on eight waves with three super-blocks per stage, half as much again in flight
      * (Mixtral's down projections at 16 tokens: 67 against 74 us; Q5_K and Q6_K rows leave room for two per
@@ -2558,9 +2563,9 @@ static int launch_experts(uint32_t qtype, const void *const *d_w, float *const *
     if (wide && is_q4k(file_type) && n_mat * n_expert * ((rows + 63) / 64) <= 2u * cus &&
         n_mat * live * ((rows + 127) / 128) >= cus - cus / 8)
         return launch_experts_tiled<1, 8>(qtype, d_w, d_out, n_mat, n_expert, rows, cols, d_acts, out_stride,
-                                          d_counts, d_offsets, stream);
+                                          d_counts, d_offsets, max_tokens, stream);
     return launch_experts_tiled<1, 4>(qtype, d_w, d_out, n_mat, n_expert, rows, cols, d_acts, out_stride,
-                                      d_counts, d_offsets, stream);
+                                      d_counts, d_offsets, max_tokens, stream);
 }
 
 /* the six launches of a layer over a workspace laid out by moe_layout(); arguments already checked */
@@ -2583,13 +2588,13 @@ static int moe_ffn_run(const OxhMoe *m, const MoeLayout &l, const float *d_logit
     const void *w_gu[2] = { m->d_w_gate, m->d_w_up };
     float *o_gu[2] = { gate, up };
     if ((rc = launch_experts(m->qtype_gate_up, w_gu, o_gu, 2, m->n_expert, m->ffn, m->hidden, ws + l.act_x,
-                             m->ffn, counts, offsets, pairs, stream))) return rc;
+                             m->ffn, counts, offsets, pairs, n_tok, stream))) return rc;
     /* 4. h = silu(gate) * up, quantised; 5. down */
     if ((rc = quantize_q8_k_ex(gate, m->ffn, pairs, m->ffn, ws + l.act_h, nullptr, up, stream))) return rc;
     const void *w_dn[1] = { m->d_w_down };
     float *o_dn[1] = { y };
     if ((rc = launch_experts(m->qtype_down, w_dn, o_dn, 1, m->n_expert, m->hidden, m->ffn, ws + l.act_h,
-                             m->hidden, counts, offsets, pairs, stream))) return rc;
+                             m->hidden, counts, offsets, pairs, n_tok, stream))) return rc;
     /* 6. combine in ascending expert order */
     hipLaunchKernelGGL(k_moe_combine, dim3((uint32_t)((m->hidden + 255u) / 256u), (uint32_t)n_tok), dim3(256), 0,
                        pick_stream(stream), (const float *)y, m->hidden, (const int32_t *)ids, (const float *)wts,
