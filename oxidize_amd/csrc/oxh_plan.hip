@@ -114,9 +114,13 @@ struct PlanSync {
 #define PLAN_STAMPS 8u
 
 /* wave 0 of a workgroup notes the shader clock at phase `slot` of operation `op` */
+/* ON: the kernel variant a plan runs once clock stamps have been asked for (a measurement hook).  The
+ * ordinary variants carry none of it: the chained kernel is short of scalar registers, and the stamps' pointer
+ * and tests alone cost it five scalars kept in vector lanes and 20 us per 128-operation step. */
+template <bool ON>
 __device__ __forceinline__ void plan_stamp(const PlanSync &sy, uint32_t op, uint32_t slot, uint32_t lane, uint32_t wave)
 {
-    if (sy.stamps != nullptr && wave == 0u && lane == 0u)
+    if (ON && sy.stamps != nullptr && wave == 0u && lane == 0u)
         sy.stamps[((size_t)op * gridDim.x + blockIdx.x) * PLAN_STAMPS + slot] = __builtin_amdgcn_s_memrealtime();
 }
 
@@ -737,7 +741,7 @@ plan_wait(const PlanSync &sy, uint32_t target, int *s_ok, uint32_t lane, uint32_
 
 /* ─── the kernel ──────────────────────────────────────────────────────── */
 
-template <bool HAS_Q5>
+template <bool HAS_Q5, bool STAMPS = false>
 __global__ __launch_bounds__(1024) void
 k_plan(const PlanOp *__restrict__ ops, uint32_t n_ops, const PlanSync sy, const PlanLds ld)
 {
@@ -784,7 +788,7 @@ k_plan(const PlanOp *__restrict__ ops, uint32_t n_ops, const PlanSync sy, const 
              * the wait costs nothing unless such a store is still on its way */
             asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
             lds_barrier();
-            plan_stamp(sy, i - 1u, 6, ln, wave);
+            plan_stamp<STAMPS>(sy, i - 1u, 6, ln, wave);
             if (wave == 0u) {
                 const CohBuf dst = coh_buf(prev.out + prev.wg_row0);
                 for (uint32_t r = ln; r < prev.wg_rows; r += 64u) cstore_f32(dst, r * 4u, outs[r]);
@@ -794,13 +798,13 @@ k_plan(const PlanOp *__restrict__ ops, uint32_t n_ops, const PlanSync sy, const 
                     plan_announce(sy, base + i + (i == n_ops ? 1u : 0u), ln);
                 }
             }
-            plan_stamp(sy, i - 1u, 7, ln, wave);
+            plan_stamp<STAMPS>(sy, i - 1u, 7, ln, wave);
         }
         if (i == n_ops) break;
 
         const OpHead op = plan_head(&tab[i]);
         uint8_t *act = lds + (size_t)(i & 1u) * ld.act_bytes;
-        plan_stamp(sy, i, 0, ln, wave);
+        plan_stamp<STAMPS>(sy, i, 0, ln, wave);
         /* Loads complete in the order a wave issued them, and the compiler waits for ALL of them
          * before the first use of the input vector (its requests sit in conditional code, which it
          * cannot count past).  So the order of the requests is the schedule: one set of weights first
@@ -839,15 +843,15 @@ k_plan(const PlanOp *__restrict__ ops, uint32_t n_ops, const PlanSync sy, const 
             else         plan_stage_issue(op, xs, ln, wave);
             if (wave == 0u) plan_prefetch<HAS_Q5>(cur, A, 0u, ln);
         }
-        plan_stamp(sy, i, 1, ln, wave);
+        plan_stamp<STAMPS>(sy, i, 1, ln, wave);
 
         /* a prologue's side outputs are one workgroup's work, and not workgroup 0's: that one gathers the
          * counters, and whatever holds it up holds everybody up */
         const bool storer = blockIdx.x == gridDim.x - 1u;
         const uint32_t Bk = op.blocks;
-        if (sy.stamps != nullptr) {         /* measurement only: when has the vector arrived? */
+        if (STAMPS && sy.stamps != nullptr) {         /* measurement only: when has the vector arrived? */
             asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-            plan_stamp(sy, i, 5, ln, wave);
+            plan_stamp<STAMPS>(sy, i, 5, ln, wave);
         }
         if (by_unit) {
             if (op.kind >= PLAN_Q6_K) plan_stage_finish_unit<1>(op, xu, act, red, storer, ln, wave);
@@ -857,9 +861,9 @@ k_plan(const PlanOp *__restrict__ ops, uint32_t n_ops, const PlanSync sy, const 
             else                      plan_stage_finish<0>(op, xs, act, red, storer, ln, wave);
         }
         plan_prefetch<HAS_Q5>(cur, B, 1u, ln);
-        plan_stamp(sy, i, 2, ln, wave);
+        plan_stamp<STAMPS>(sy, i, 2, ln, wave);
         __syncthreads();
-        plan_stamp(sy, i, 3, ln, wave);
+        plan_stamp<STAMPS>(sy, i, 3, ln, wave);
 
         GemvParams gp;
         gp.blocks = Bk;
@@ -873,7 +877,7 @@ k_plan(const PlanOp *__restrict__ ops, uint32_t n_ops, const PlanSync sy, const 
             else if (HAS_Q5 && cur.kind == PLAN_Q5_K) plan_passes_q45<true>(A, B, cur, gp, act, q8k_lds_bytes(Bk), terms, ln);
             else                            plan_passes_q45<false>(A, B, cur, gp, act, q8k_lds_bytes(Bk), terms, ln);
         }
-        plan_stamp(sy, i, 4, ln, wave);
+        plan_stamp<STAMPS>(sy, i, 4, ln, wave);
         prev = cur;
         cur = nx;
         po = op;
@@ -907,7 +911,7 @@ __device__ __forceinline__ void plan_image_fetch(const PlanOp *op, gaddr xq, uin
         if (k + 16u * lane < bytes) plan_dma16(img + k, 16u * lane, lds_addr + k);
 }
 
-template <bool HAS_Q5>
+template <bool HAS_Q5, bool STAMPS = false>
 __global__ __launch_bounds__(1024) void
 k_plan_ext(const PlanOp *__restrict__ ins, uint32_t n_ins, const PlanOp *__restrict__ ops, uint32_t n_ops,
            const PlanSync sy, const PlanLds ld)
@@ -966,7 +970,7 @@ k_plan_ext(const PlanOp *__restrict__ ins, uint32_t n_ins, const PlanOp *__restr
         uint32_t ln = lane;
         asm volatile("" : "+v"(ln));
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        plan_stamp(sy, i < n_ops ? i : n_ops - 1u, i < n_ops ? 0u : 5u, ln, wave);
+        plan_stamp<STAMPS>(sy, i < n_ops ? i : n_ops - 1u, i < n_ops ? 0u : 5u, ln, wave);
         WSet A, B;
         A.a = A.b = A.c = A.d = A.e = u32x4{ 0u, 0u, 0u, 0u };
         B.a = B.b = B.c = B.d = B.e = A.a;
@@ -977,7 +981,7 @@ k_plan_ext(const PlanOp *__restrict__ ins, uint32_t n_ins, const PlanOp *__restr
         if (i > 0u) {
             /* every wave has finished operation i - 1 and has its pieces of this operation's input */
             lds_barrier();
-            plan_stamp(sy, i - 1u, 6, ln, wave);
+            plan_stamp<STAMPS>(sy, i - 1u, 6, ln, wave);
             const float *tb = terms_wg + (size_t)((i - 1u) & 1u) * ld.terms_wg;
             const CohBuf dst = coh_buf(prev.out + prev.wg_row0);
             for (uint32_t r = threadIdx.x; r < prev.wg_rows; r += 1024u) {
@@ -1002,7 +1006,7 @@ k_plan_ext(const PlanOp *__restrict__ ins, uint32_t n_ins, const PlanOp *__restr
             nx = plan_work_flat(&tab[i + 1u], wave);
             plan_image_fetch(&tab[i + 1u], nx.xq, lds_base + ((i + 1u) & 1u) * ld.act_bytes, ln, wave);
         }
-        plan_stamp(sy, i, 1, ln, wave);
+        plan_stamp<STAMPS>(sy, i, 1, ln, wave);
 
         const PlanOp *const op = &tab[i];
         const uint32_t Bk = uni(op->blocks);
@@ -1020,7 +1024,7 @@ k_plan_ext(const PlanOp *__restrict__ ins, uint32_t n_ins, const PlanOp *__restr
             else if (HAS_Q5 && cur.kind == PLAN_Q5_K) plan_passes_q45<true>(A, B, cur, gp, act, q8k_lds_bytes(Bk), terms, ln);
             else                            plan_passes_q45<false>(A, B, cur, gp, act, q8k_lds_bytes(Bk), terms, ln);
         }
-        plan_stamp(sy, i, 4, ln, wave);
+        plan_stamp<STAMPS>(sy, i, 4, ln, wave);
         prev = cur;
         cur = nx;
         p_blocks = Bk;
@@ -1053,6 +1057,9 @@ struct OxhPlan {
 
 static const void *plan_kernel(const OxhPlan *pl)
 {
+    /* with clock stamps attached (plans without Q5_K only): the variants that write them */
+    if (pl->d_stamps != nullptr && !pl->has_q5)
+        return pl->ext ? reinterpret_cast<const void *>(k_plan_ext<false, true>) : reinterpret_cast<const void *>(k_plan<false, true>);
     if (pl->ext)
         return pl->has_q5 ? reinterpret_cast<const void *>(k_plan_ext<true>) : reinterpret_cast<const void *>(k_plan_ext<false>);
     return pl->has_q5 ? reinterpret_cast<const void *>(k_plan<true>) : reinterpret_cast<const void *>(k_plan<false>);
@@ -1553,12 +1560,15 @@ extern "C" int oxh_plan_launch(OxhPlan *pl, void *stream)
 #define PLAN_LAUNCH_EXT(K)                                                                              \
     hipLaunchKernelGGL(K, dim3(pl->grid), dim3(1024), pl->lds_bytes, st, (const PlanOp *)pl->d_ops,    \
                        pl->n_ops, (const PlanOp *)pl->d_run, pl->n_run, sy, pl->ld)
+    const bool stamped = pl->d_stamps != nullptr && !pl->has_q5;     /* as plan_kernel() */
     if (pl->ext) {
-        if (pl->has_q5) PLAN_LAUNCH_EXT(k_plan_ext<true>);
-        else            PLAN_LAUNCH_EXT(k_plan_ext<false>);
+        if (stamped)         PLAN_LAUNCH_EXT((k_plan_ext<false, true>));
+        else if (pl->has_q5) PLAN_LAUNCH_EXT(k_plan_ext<true>);
+        else                 PLAN_LAUNCH_EXT(k_plan_ext<false>);
     } else {
-        if (pl->has_q5) PLAN_LAUNCH(k_plan<true>);
-        else            PLAN_LAUNCH(k_plan<false>);
+        if (stamped)         PLAN_LAUNCH((k_plan<false, true>));
+        else if (pl->has_q5) PLAN_LAUNCH(k_plan<true>);
+        else                 PLAN_LAUNCH(k_plan<false>);
     }
 #undef PLAN_LAUNCH
 #undef PLAN_LAUNCH_EXT
@@ -1611,6 +1621,7 @@ extern "C" int oxh_debug_plan_stamps(OxhPlan *pl, uint64_t *d_stamps)
 {
     if (!pl) return oxh_internal_errorf(OXH_ERR_ARG, "invalid argument: oxh_debug_plan_stamps: NULL plan");
     pl->d_stamps = d_stamps;
+    PLAN_TRY(hipFuncSetAttribute(plan_kernel(pl), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
     return OXH_OK;
 }
 
