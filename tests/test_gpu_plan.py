@@ -216,6 +216,36 @@ def test_prestaged_plan_follows_its_inputs_from_launch_to_launch(oxh, monkeypatc
     chained.destroy()
 
 
+def test_clock_stamps_run_the_stamped_kernels_with_the_same_bits(oxh):
+    """The measurement hook swaps in the kernel variants that write clock stamps (the ordinary ones carry no
+    stamp code): same outputs, and every workgroup leaves stamps for every operation."""
+    hidden, kv, ffn, layers = 1024, 256, 2816, 2
+    d = DecodeSet(hidden=hidden, kv=kv, ffn=ffn, layers=layers, seed=6)
+    a, b = DecodeChain(d, seed=6), DecodeChain(d, seed=6)
+    a.launch_step()
+    mv.sync()
+    want = chain_state(a)
+    plan = mv.Plan(b.plan_ops())
+    n_ops, grid = 4 * layers, plan.info()["workgroups"]
+    stamps = mv.DeviceBuffer(n_ops * grid * 8 * 8)
+    _lib.check(_lib.lib().oxh_memset(ctypes.c_void_p(stamps.ptr), 0, stamps.nbytes, None))
+    plan.launch()                                       # the ordinary kernel
+    assert plan.status() == 0
+    assert not stamps.download(np.uint64, n_ops * grid * 8).any()
+    _lib.check(_lib.lab().plan_stamps(plan.handle, ctypes.c_void_p(stamps.ptr)))
+    for rep in range(2):
+        plan.launch()                                   # the stamped one
+        assert plan.status() == 0
+        got = chain_state(b)
+        for k in ("qkv", "o", "h", "f", "x"):
+            assert np.array_equal(bits(got[k]), bits(want[k])), (rep, k)
+    st = stamps.download(np.uint64, n_ops * grid * 8).reshape(n_ops, grid, 8)
+    assert (st[:, :, 0] != 0).all()                     # slot 0: the operation's start, by every workgroup
+    assert (st[1:, :, 0].astype(np.int64) - st[:-1, :, 0].astype(np.int64) > 0).all()   # in order
+    _lib.check(_lib.lab().plan_stamps(plan.handle, None))
+    plan.destroy()
+
+
 def test_a_wait_that_cannot_be_satisfied_gives_up(oxh):
     """The waits expect one workgroup more than exist and may poll 300 times: every workgroup must leave,
     the launch must end, the status must say so, and the plan must work again afterwards."""
