@@ -511,6 +511,51 @@ def secondary_figures(mv, synth):
         "frac_of_hbm_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBPS, 4),
         "as_graph_of_97_launches_us": round(us_graph, 1),
         "note": "independent operations (every input there when the launch starts); no workgroup waits for another"}
+    # the same step for a batch of eight activations per matmul, as a graph of launches (a plan over a 32-value
+    # format takes one activation per operation): the layers from the file layout (dot or matrix-core kernel by
+    # launch size), the head from a tile-major copy
+    nvb = 8
+    bx, bo, ba, bsegs = [], [], [], []
+    for layer in range(qs.layers):
+        for op, (name, qt, rows_, cols_, _) in enumerate(qs.ops):
+            tot = sum(rows_)
+            x = mv.DeviceBuffer.from_host(synth.normal(nvb * cols_, seed=0, stream=500000 + layer * 8 + op))
+            o = mv.DeviceBuffer(nvb * tot * 4)
+            aq = mv.DeviceBuffer(nvb * mv.act_bytes(qt, cols_))
+            items, off = [], 0
+            for seg, r_ in enumerate(rows_):
+                items.append((qs.weights[layer][op][seg].ptr, o.ptr + off * 4, r_, 0))
+                off += r_
+            bx.append(x); bo.append(o); ba.append(aq)
+            bsegs.append((mv.make_segments(items), cols_, tot))
+    d_head16 = mv.DeviceBuffer(mv.tile16_bytes(Q80, rows, cols))
+    mv.tile16(Q80, d_head.ptr, rows, cols, d_head16.ptr)
+    d_hx8 = mv.DeviceBuffer.from_host(synth.normal(nvb * cols, seed=0, stream=9))
+    d_ho8 = mv.DeviceBuffer(nvb * rows * 4)
+    d_ha8 = mv.DeviceBuffer(nvb * mv.act_bytes(Q80, cols))
+    head16_seg = mv.make_segments([(d_head16.ptr, d_ho8.ptr, rows, 0)])
+
+    def qwen_step_batch():
+        for (segs, cols_, tot), x, aq in zip(bsegs, bx, ba):
+            mv.gemv_segments_f32(Q80, segs, cols_, x.ptr, cols_, aq.ptr, nvb, tot)
+        mv.gemv_segments_f32(mv.Q8_0_T16, head16_seg, cols, d_hx8.ptr, cols, d_ha8.ptr, nvb, rows)
+
+    qwen_step_batch()
+    mv.sync()
+    graph = mv.Graph()
+    with graph:
+        qwen_step_batch()
+    us_b = timed(graph.launch, 20, mv)
+    graph.destroy()
+    out["q8_0_decode_step_qwen2_5_0_5b"]["batch8_as_graph_of_launches_us"] = round(us_b, 1)
+    out["q8_0_decode_step_qwen2_5_0_5b"]["batch8_note"] = (
+        "eight activations per matmul, 97 operations as a graph (the layers' matrices from the file layout, the "
+        "145 MB head from its tile-major copy); per activation %.1f us against %.1f us for the batch-1 step as one "
+        "launch: launches over matrices of 0.9-9 MB are paced by their own dependent chain (8-18 us each at eight "
+        "activations), so eight single-activation plan launches (%.0f us) beat one batched step of launches"
+        % (us_b / nvb, us, nvb * us))
+    for b_ in bx + bo + ba + [d_head16, d_hx8, d_ho8, d_ha8]:
+        b_.free()
     d_head.free()
     d_hx.free()
     d_ho.free()
