@@ -554,6 +554,72 @@ def secondary_figures(mv, synth):
         "launch: launches over matrices of 0.9-9 MB are paced by their own dependent chain (8-18 us each at eight "
         "activations), so eight single-activation plan launches (%.0f us) beat one batched step of launches"
         % (us_b / nvb, us, nvb * us))
+    # The same eight-activation step with EVERY matrix tile-major and the independent operations of one input
+    # width grouped into launches of up to 32 segments (each segment its own run of eight activations): every
+    # launch then has thousands of 16-row groups to deal to its waves, where a launch over one small matrix
+    # has a few hundred.  Inputs are quantised by one launch per width.
+    groups = {}
+    for idx, ((segs_, cols_, tot), x) in enumerate(zip(bsegs, bx)):
+        groups.setdefault(cols_, []).append(idx)
+    tiled_keep, launches = [], []
+    for cols_, idxs in groups.items():
+        n_in = len(idxs) * nvb
+        xin = mv.DeviceBuffer(n_in * cols_ * 4)
+        for j, idx in enumerate(idxs):
+            _lib_check_copy(xin.ptr + j * nvb * cols_ * 4, bx[idx].ptr, nvb * cols_ * 4)
+        aq = mv.DeviceBuffer(n_in * mv.act_bytes(Q80, cols_))
+        items = []
+        for j, idx in enumerate(idxs):
+            layer, op = divmod(idx, len(qs.ops))
+            name, qt, rows_, _, _ = qs.ops[op]
+            off = 0
+            for seg, r_ in enumerate(rows_):
+                t16 = mv.DeviceBuffer(mv.tile16_bytes(Q80, r_, cols_))
+                mv.tile16(Q80, qs.weights[layer][op][seg].ptr, r_, cols_, t16.ptr)
+                tiled_keep.append(t16)
+                items.append((t16.ptr, bo[idx].ptr + off * 4, r_, j * nvb, nvb, sum(rows_)))
+                off += r_
+        tiled_keep += [xin, aq]
+        # segments of one launch share the output stride: group them by it
+        by_stride = {}
+        for it in items:
+            by_stride.setdefault(it[5], []).append(it[:5])
+        for stride, its in by_stride.items():
+            for k in range(0, len(its), 32):
+                launches.append((mv.make_segments(its[k:k + 32]), cols_, aq, stride))
+        launches.append(("quantize", cols_, xin, aq, n_in))
+    mv.sync()
+
+    def qwen_step_tiled():
+        for l in launches:
+            if l[0] == "quantize":
+                mv.quantize(Q80, l[2].ptr, l[1], l[4], l[1], l[3].ptr)
+        for l in launches:
+            if l[0] != "quantize":
+                mv.gemv_segments(mv.Q8_0_T16, l[0], l[1], l[2].ptr, nvb, l[3])
+        mv.gemv_segments_f32(mv.Q8_0_T16, head16_seg, cols, d_hx8.ptr, cols, d_ha8.ptr, nvb, rows)
+
+    import numpy as np
+    probe_idx = (len(bo) - 1, 2, 0)                     # a down projection, a gate/up, a q/k/v
+    before = [bo[i].download(np.uint32, bo[i].nbytes // 4).copy() for i in probe_idx]
+    for i in probe_idx:
+        _lib_check_memset(bo[i])
+    qwen_step_tiled()
+    mv.sync()
+    for i, want in zip(probe_idx, before):              # the file layout's bits
+        assert np.array_equal(bo[i].download(np.uint32, bo[i].nbytes // 4), want)
+    graph = mv.Graph()
+    with graph:
+        qwen_step_tiled()
+    us_t = timed(graph.launch, 20, mv)
+    graph.destroy()
+    n_l = sum(1 for l in launches) + 2
+    out["q8_0_decode_step_qwen2_5_0_5b"]["batch8_tile_major_grouped_us"] = round(us_t, 1)
+    out["q8_0_decode_step_qwen2_5_0_5b"]["batch8_tile_major_grouped_note"] = (
+        "every matrix tile-major (oxh_tile16), the independent operations of one input width grouped into launches "
+        "of up to 32 segments: %d launches per step, %.1f us per activation" % (n_l, us_t / nvb))
+    for b_ in tiled_keep:
+        b_.free()
     for b_ in bx + bo + ba + [d_head16, d_hx8, d_ho8, d_ha8]:
         b_.free()
     d_head.free()
@@ -615,6 +681,12 @@ def secondary_figures(mv, synth):
         "note": "oxh_moe_ffn as one graph: route + group, gather + Q8_K, gate/up of all experts, "
                 "silu(gate)*up + Q8_K, down of all experts, combine; no host step between them"}
     return out
+
+
+def _lib_check_copy(dst, src, nbytes):
+    import ctypes
+    from oxidize_amd import _lib
+    _lib.check(_lib.lib().oxh_memcpy_d2d(ctypes.c_void_p(dst), ctypes.c_void_p(src), nbytes, None))
 
 
 def traffic_probe(mv, ds):

@@ -859,6 +859,8 @@ static hipError_t raise_all_lds_ceilings(void)
     if ((e = raise_lds_ceiling(k_gemv_multi<0>)) != hipSuccess) return e;
     if ((e = raise_lds_ceiling(k_q80t_segments<4, 2, false>)) != hipSuccess) return e;
     if ((e = raise_lds_ceiling(k_q80t_segments<8, 2, false>)) != hipSuccess) return e;
+    if ((e = raise_lds_ceiling(k_q80t_segments<16, 2, false>)) != hipSuccess) return e;
+    if ((e = raise_lds_ceiling(k_q80t_segments<16, 2, true>)) != hipSuccess) return e;
     if ((e = raise_lds_ceiling(k_q80t_segments<1, 2, false>)) != hipSuccess) return e;
     if ((e = raise_lds_ceiling(k_q80t_segments<4, 2, true>)) != hipSuccess) return e;
     if ((e = raise_lds_ceiling(k_q80t_segments<8, 2, true>)) != hipSuccess) return e;
@@ -1184,10 +1186,20 @@ static int launch_q80t_segments(const OxhSegment *segs, size_t n_segs, size_t co
         return OXH_ERR_TOO_WIDE;
     }
     static const uint32_t forced_gpw = env_u32("OXH_Q80T_GPW", 0, 0, 1024);
-    static const uint32_t forced_waves = env_u32("OXH_Q80T_WAVES", 0, 0, 8);
+    static const uint32_t forced_waves = env_u32("OXH_Q80T_WAVES", 0, 0, 16);
     const size_t cus = (size_t)(g_n_cu > 0 ? g_n_cu : 256);
-    uint32_t waves = n_groups >= 32u * cus ? 8u : (n_groups >= 16u * cus ? 4u : 1u);
-    if (forced_waves == 1u || forced_waves == 4u || forced_waves == 8u) waves = forced_waves;
+    /* Waves per workgroup: a wave per row group is all the parallelism there is, so the smallest workgroup
+     * with which every group's wave is resident at once (a compute unit holds 32 waves, and as many
+     * workgroups as their staged activations leave LDS for: one, for 4864 columns); launches with more
+     * groups than that run in rounds of eight-wave workgroups.  24 matrices of 896 x 4864 in one launch
+     * (1344 groups, 87 KB of LDS per workgroup): one wave per workgroup is one wave per compute unit. */
+    const size_t wg_per_cu = lds ? (160u * 1024u / lds ? 160u * 1024u / lds : 1u) : 1u;
+    uint32_t waves = 8u;
+    for (uint32_t w = 1u; w <= 16u; w = w == 1u ? 4u : 2u * w) {
+        const size_t per_cu = wg_per_cu * w < 32u ? wg_per_cu * w : 32u;
+        if (cus * per_cu >= n_groups) { waves = w; break; }
+    }
+    if (forced_waves == 1u || forced_waves == 4u || forced_waves == 8u || forced_waves == 16u) waves = forced_waves;
     /* f32 inputs: with one or two activations per segment the workgroups quantise them themselves while
      * they stage them (a launch less: head at one activation 27.4 against 30 us); with more, that work,
      * repeated by every workgroup, costs more than the quantiser's launch (eight activations 36 against 32 us),
@@ -1229,7 +1241,8 @@ static int launch_q80t_segments(const OxhSegment *segs, size_t n_segs, size_t co
 #define OXH_Q80T(WAVES, FUSED) hipLaunchKernelGGL((k_q80t_segments<WAVES, 2, FUSED>), dim3(wg), dim3(WAVES * 64), lds, \
                                                   st, t, (uint32_t)blocks, acts, out_stride, (uint32_t)gpw, io.d_x,   \
                                                   (uint32_t)io.x_stride)
-    if (waves == 8u) { if (fused) OXH_Q80T(8, true); else OXH_Q80T(8, false); }
+    if (waves == 16u) { if (fused) OXH_Q80T(16, true); else OXH_Q80T(16, false); }
+    else if (waves == 8u) { if (fused) OXH_Q80T(8, true); else OXH_Q80T(8, false); }
     else if (waves == 4u) { if (fused) OXH_Q80T(4, true); else OXH_Q80T(4, false); }
     else { if (fused) OXH_Q80T(1, true); else OXH_Q80T(1, false); }
 #undef OXH_Q80T
