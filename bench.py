@@ -571,7 +571,7 @@ def secondary_figures(mv, synth):
     groups = {}
     for idx, ((segs_, cols_, tot), x) in enumerate(zip(bsegs, bx)):
         groups.setdefault(cols_, []).append(idx)
-    tiled_keep, launches = [], []
+    tiled_keep, launches, t16_of = [], [], {}
     for cols_, idxs in groups.items():
         n_in = len(idxs) * nvb
         xin = mv.DeviceBuffer(n_in * cols_ * 4)
@@ -587,6 +587,7 @@ def secondary_figures(mv, synth):
                 t16 = mv.DeviceBuffer(mv.tile16_bytes(Q80, r_, cols_))
                 mv.tile16(Q80, qs.weights[layer][op][seg].ptr, r_, cols_, t16.ptr)
                 tiled_keep.append(t16)
+                t16_of[(idx, seg)] = t16
                 items.append((t16.ptr, bo[idx].ptr + off * 4, r_, j * nvb, nvb, sum(rows_)))
                 off += r_
         tiled_keep += [xin, aq]
@@ -628,6 +629,39 @@ def secondary_figures(mv, synth):
     out["q8_0_decode_step_qwen2_5_0_5b"]["batch8_tile_major_grouped_note"] = (
         "every matrix tile-major (oxh_tile16), the independent operations of one input width grouped into launches "
         "of up to 32 segments: %d launches per step, %.1f us per activation" % (n_l, us_t / nvb))
+    # ... and as ONE launch: a plan over the tile-major matrices, eight activations per segment, every operation
+    # quantising its own f32 input (the matrices cut into runs of whole row groups, dealt by units streamed)
+    plan_ops = []
+    for idx, (segs_, cols_, tot) in enumerate(bsegs):
+        layer, op = divmod(idx, len(qs.ops))
+        rows_ = qs.ops[op][2]
+        items, off = [], 0
+        for seg, r_ in enumerate(rows_):
+            items.append((t16_of[(idx, seg)].ptr, bo[idx].ptr + off * 4, r_, 0, nvb))
+            off += r_
+        plan_ops.append(dict(qtype=mv.Q8_0_T16, segs=mv.make_segments(items), cols=cols_, d_x=bx[idx].ptr,
+                             d_act_out=None, out_stride=tot))
+    plan_ops.append(dict(qtype=mv.Q8_0_T16, segs=mv.make_segments([(d_head16.ptr, d_ho8.ptr, rows, 0, nvb)]), cols=cols,
+                         d_x=d_hx8.ptr, d_act_out=None, out_stride=rows))
+    tplan = mv.Plan(plan_ops)
+    head_before = d_ho8.download(np.uint32, nvb * rows).copy()
+    for i in probe_idx:
+        _lib_check_memset(bo[i])
+    _lib_check_memset(d_ho8)
+    tplan.launch()
+    assert tplan.status() == 0
+    for i, want in zip(probe_idx, before):
+        assert np.array_equal(bo[i].download(np.uint32, bo[i].nbytes // 4), want)
+    assert np.array_equal(d_ho8.download(np.uint32, nvb * rows), head_before)
+    us_p = timed(tplan.launch, 20, mv)
+    t_info = tplan.info()
+    tplan.destroy()
+    step_bytes8 = qs.weight_bytes + w.nbytes
+    out["q8_0_decode_step_qwen2_5_0_5b"]["batch8_tile_major_plan_us"] = round(us_p, 1)
+    out["q8_0_decode_step_qwen2_5_0_5b"]["batch8_tile_major_plan_note"] = (
+        "the same 97 operations at eight activations each as ONE launch (a plan over OXH_Q8_0_T16 operations, %d "
+        "workgroups): %.1f us per activation, %.2f TB/s of weight bytes, bit-checked against the file-layout outputs"
+        % (t_info["workgroups"], us_p / nvb, step_bytes8 / us_p / 1e6))
     for b_ in tiled_keep:
         b_.free()
     for b_ in bx + bo + ba + [d_head16, d_hx8, d_ho8, d_ha8]:

@@ -271,6 +271,17 @@ int oxh_gemv_segments_fused(uint32_t qtype, const OxhSegment *segs, size_t n_seg
  * own steps.  Same bits as the calls one by one.  oxh_plan_table_rows gives
  * the number of runs; nothing of the residency rule below applies.
  *
+ * Plans over tile-major Q8_0 (OXH_Q8_0_T16, see oxh_tile16): every operation
+ * of that form (cols a multiple of 128), independent of each other as above,
+ * without prologue and unpaired; a segment may carry up to sixteen activations
+ * (its n_vec, from row act_first of d_x on, the rows cols floats apart; d_act_out,
+ * when given, receives the Q8_0 blocks of the same rows), activation v's rows
+ * going out_stride floats after activation v - 1's.  The matrices are cut into
+ * runs of whole 16-row groups and dealt so that every workgroup streams the
+ * same amount; same bits as oxh_gemv_segments_f32 segment by segment.  This
+ * is how many small matrices are batched: a Qwen2.5-0.5B-shaped step of 97
+ * matmuls at eight activations each is one launch.
+ *
  * All workgroups must be resident together (one per compute unit; the kernel
  * needs the whole device, so do not run other kernels beside a plan launch).
  * Every wait is bounded: after `polls` unsuccessful polls (about a microsecond
@@ -286,6 +297,8 @@ typedef struct OxhPlanOp {
     const float       *d_x;
     const OxhPrologue *pro;         /* NULL: quantise d_x as it is */
     void              *d_act_out;   /* NULL, or where the quantised bytes are also stored */
+    size_t             out_stride;  /* floats from one activation's outputs to the next one's (tile-major
+                                       plans with several activations per segment); otherwise unused, 0 */
 } OxhPlanOp;
 typedef struct OxhPlan OxhPlan;
 int oxh_plan_create(const OxhPlanOp *ops, size_t n_ops, OxhPlan **plan);

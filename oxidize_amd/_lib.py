@@ -30,7 +30,7 @@ class OxhPrologue(ctypes.Structure):
 
 class OxhPlanOp(ctypes.Structure):
     _fields_ = [("qtype", U32), ("segs", ctypes.POINTER(OxhSegment)), ("n_segs", Z), ("cols", Z), ("d_x", V),
-                ("pro", ctypes.POINTER(OxhPrologue)), ("d_act_out", V)]
+                ("pro", ctypes.POINTER(OxhPrologue)), ("d_act_out", V), ("out_stride", Z)]
 
 
 class OxhMoe(ctypes.Structure):

@@ -642,8 +642,8 @@ static void batch_form(uint32_t *qtype, Resident *entry, const uint8_t *data, si
 {
     const int n_cu = oxh_internal_n_cu();
     if (*qtype != OXH_Q8_0 || !entry || n_vec < 2 || n_vec > 16 || cols % (4u * OXH_QK8_0) || !q80_tiled_enabled() ||
-        n_cu <= 0 || rows / 16u < 16u * (size_t)n_cu)
-        return;
+        n_cu <= 0 || rows / 16u < 16u * (size_t)n_cu || cols / OXH_QK8_0 * 576u > 160u * 1024u)
+        return;                                     /* the last: what the tile-major kernel's workgroup holds in LDS */
     if (entry->automatic && cache_mode() == CACHE_OFF) return;
     const uint8_t *d;
     if (prepared_ptr(entry, data, rows, cols, OXH_PREP_Q80_T16, &d) != OXH_OK) return;

@@ -517,6 +517,10 @@ __device__ __forceinline__ MultiState multi_state(const GemvMultiItem *it, uint3
     MultiState st;
     st.p = it->p;
     st.ww.seg = it->seg;
+    st.ww.seg.w = as_global(st.ww.seg.w);
+    st.ww.seg.out = as_global(st.ww.seg.out);
+    st.p.x = as_global(st.p.x);
+    st.p.act_out = as_global(st.p.act_out);
     st.same_x = it->same_x;
     st.ww.seg_index = 0u;
     st.ww.wg_in_seg = 0u;
@@ -860,6 +864,8 @@ static hipError_t raise_all_lds_ceilings(void)
     if ((e = raise_lds_ceiling(k_q80t_segments<4, 2, false>)) != hipSuccess) return e;
     if ((e = raise_lds_ceiling(k_q80t_segments<8, 2, false>)) != hipSuccess) return e;
     if ((e = raise_lds_ceiling(k_q80t_segments<16, 2, false>)) != hipSuccess) return e;
+    if ((e = raise_lds_ceiling(k_q80t_multi<8, 2>)) != hipSuccess) return e;
+    if ((e = raise_lds_ceiling(k_q80t_multi<16, 2>)) != hipSuccess) return e;
     if ((e = raise_lds_ceiling(k_q80t_segments<16, 2, true>)) != hipSuccess) return e;
     if ((e = raise_lds_ceiling(k_q80t_segments<1, 2, false>)) != hipSuccess) return e;
     if ((e = raise_lds_ceiling(k_q80t_segments<4, 2, true>)) != hipSuccess) return e;
@@ -1180,8 +1186,8 @@ static int launch_q80t_segments(const OxhSegment *segs, size_t n_segs, size_t co
         snprintf(g_err, sizeof g_err, "gemv: tile-major Q8_0 needs columns in whole runs of four blocks (cols %zu)", cols);
         return OXH_DECLINED;
     }
-    const size_t lds = blocks * Q80T_ACT_BLOCK;
-    if (lds > GEMV_LDS_LIMIT) {
+    const size_t image = blocks * Q80T_ACT_BLOCK;
+    if (image > GEMV_LDS_LIMIT) {
         snprintf(g_err, sizeof g_err, "gemv: %zu columns x 16 staged activations do not fit 160 KiB of LDS", cols);
         return OXH_ERR_TOO_WIDE;
     }
@@ -1193,13 +1199,14 @@ static int launch_q80t_segments(const OxhSegment *segs, size_t n_segs, size_t co
      * workgroups as their staged activations leave LDS for: one, for 4864 columns); launches with more
      * groups than that run in rounds of eight-wave workgroups.  24 matrices of 896 x 4864 in one launch
      * (1344 groups, 87 KB of LDS per workgroup): one wave per workgroup is one wave per compute unit. */
-    const size_t wg_per_cu = lds ? (160u * 1024u / lds ? 160u * 1024u / lds : 1u) : 1u;
     uint32_t waves = 8u;
     for (uint32_t w = 1u; w <= 16u; w = w == 1u ? 4u : 2u * w) {
+        const size_t wg_per_cu = GEMV_LDS_LIMIT / image ? GEMV_LDS_LIMIT / image : 1u;
         const size_t per_cu = wg_per_cu * w < 32u ? wg_per_cu * w : 32u;
         if (cus * per_cu >= n_groups) { waves = w; break; }
     }
     if (forced_waves == 1u || forced_waves == 4u || forced_waves == 8u || forced_waves == 16u) waves = forced_waves;
+    const size_t lds = image;
     /* f32 inputs: with one or two activations per segment the workgroups quantise them themselves while
      * they stage them (a launch less: head at one activation 27.4 against 30 us); with more, that work,
      * repeated by every workgroup, costs more than the quantiser's launch (eight activations 36 against 32 us),
@@ -1598,20 +1605,202 @@ extern "C" int oxh_gemv_segments_f32(uint32_t qtype, const OxhSegment *segs, siz
 
 struct GemvMulti {
     GemvMultiItem *d_items;
+    Q80tItem *d_titems;         /* which == MULTI_TILED */
     uint32_t *d_first;
-    uint32_t n_ops, n_items, grid;
+    uint32_t n_ops, n_items, grid, waves;
     int which;
     size_t lds;
 };
+#define MULTI_TILED 6           /* tile-major Q8_0, up to sixteen activations per segment */
 
 static int mmq80_leg(uint32_t qtype);
 
 extern "C" int oxh_internal_multi_which(uint32_t qtype)
 {
+    if (qtype == OXH_Q8_0_T16) return MULTI_TILED;
     qtype = canon_qtype(qtype);
     if (qtype == OXH_Q8_0) return 0;
     const int leg = mmq80_leg(qtype);
     return leg >= 1 ? leg : -1;
+}
+
+/* Plans over tile-major Q8_0.  Every segment is cut into runs of whole 16-row groups, a run's cost for
+ * its workgroup being the units its busiest wave streams (groups shared between the waves, a group's
+ * units = blocks / 4), and the runs are dealt to the least loaded workgroup in turn, the segments with
+ * the longest rows first (their runs are the coarsest), each workgroup taking as many rounds of a
+ * segment as still fit its share: a workgroup's items are few and mostly consecutive runs of one
+ * operation, so its activations are staged once. */
+static int multi_create_tiled(const OxhPlanOp *ops, size_t n_ops, void **handle)
+{
+    const uint32_t n_cu = (uint32_t)(g_n_cu > 0 ? g_n_cu : 256);
+    static const uint32_t forced_waves = env_u32("OXH_Q80T_PLAN_WAVES", 0, 0, 16);
+    struct Piece { uint32_t op, seg, runs, groups, nv; };
+    size_t n_pieces = 0, max_blocks = 0;
+    for (size_t i = 0; i < n_ops; i++) {
+        const OxhPlanOp &o = ops[i];
+        if (o.qtype != OXH_Q8_0_T16 || o.pro || !o.segs || o.n_segs == 0 || !o.d_x || o.cols == 0 || o.cols % 128u) {
+            snprintf(g_err, sizeof g_err, "plan: operation %zu: the operations of a plan over tile-major Q8_0 are all of "
+                     "that form (cols a multiple of 128), without prologue, with segments and an input", i);
+            return OXH_DECLINED;
+        }
+        const size_t blocks = o.cols / OXH_QK8_0;
+        if (blocks * Q80T_ACT_BLOCK > GEMV_LDS_LIMIT) {
+            snprintf(g_err, sizeof g_err, "plan: operation %zu: cols %zu too wide for one workgroup", i, o.cols);
+            return OXH_ERR_TOO_WIDE;
+        }
+        if (blocks > max_blocks) max_blocks = blocks;
+        size_t live = 0;
+        for (size_t k = 0; k < o.n_segs; k++) {
+            const OxhSegment &sg = o.segs[k];
+            if (!sg.rows) continue;
+            const size_t nv = sg.n_vec ? sg.n_vec : 1u;
+            if (nv > 16u || sg.d_w_pair || !sg.d_w || !sg.d_out || sg.rows > 0x3FFFFFFFull || sg.act_first > 0xFFFFFFu)
+                return arg_fail("plan: tile-major segments have 1..16 activations, a matrix and an output, and are unpaired");
+            if (nv > 1u && (o.out_stride == 0 || o.out_stride > 0xFFFFFFFFull))
+                return arg_fail("plan: an operation with several activations per segment needs out_stride");
+            live++;
+        }
+        if (live == 0) return arg_fail("plan: an operation has no rows");
+        n_pieces += live;
+    }
+    /* LDS of a workgroup: the widest operation's staged activations.  Sixteen waves, one workgroup per
+     * compute unit (eight: two where LDS holds two) */
+    const size_t lds = max_blocks * Q80T_ACT_BLOCK;
+    const uint32_t waves = forced_waves == 8u || forced_waves == 16u ? forced_waves : 16u;
+    const uint32_t per_cu = (waves == 8u && 2u * lds <= GEMV_LDS_LIMIT) ? 2u : 1u;
+    const uint32_t n_wg = n_cu * per_cu;
+
+    Piece *pieces = (Piece *)calloc(n_pieces, sizeof *pieces);
+    double *load = (double *)calloc(n_wg, sizeof *load);
+    uint32_t *count = (uint32_t *)calloc(n_wg + 1u, sizeof *count);
+    if (!pieces || !load || !count) {
+        free(pieces); free(load); free(count);
+        snprintf(g_err, sizeof g_err, "out of host memory building a plan");
+        return OXH_ERR_NOMEM;
+    }
+    size_t np = 0, cap_items = 0;
+    double total = 0.0;
+    for (size_t i = 0; i < n_ops; i++)
+        for (size_t k = 0; k < ops[i].n_segs; k++) {
+            const OxhSegment &sg = ops[i].segs[k];
+            if (!sg.rows) continue;
+            Piece &pc = pieces[np++];
+            pc.op = (uint32_t)i;
+            pc.seg = (uint32_t)k;
+            pc.runs = (uint32_t)(ops[i].cols / 128u);
+            pc.groups = (uint32_t)((sg.rows + 15u) / 16u);
+            pc.nv = (uint32_t)(sg.n_vec ? sg.n_vec : 1u);
+            total += (double)pc.groups / waves * pc.runs;
+            cap_items += pc.groups / waves + 2u;
+        }
+    /* longest rows first; the order of the operations otherwise (insertion sort: stable) */
+    for (size_t a = 1; a < np; a++) {
+        const Piece key = pieces[a];
+        size_t b = a;
+        while (b > 0 && pieces[b - 1].runs < key.runs) { pieces[b] = pieces[b - 1]; b--; }
+        pieces[b] = key;
+    }
+    struct Dealt { Q80tItem it; uint32_t wg; };
+    Dealt *dealt = (Dealt *)calloc(cap_items, sizeof *dealt);
+    if (!dealt) {
+        free(pieces); free(load); free(count);
+        snprintf(g_err, sizeof g_err, "out of host memory building a plan");
+        return OXH_ERR_NOMEM;
+    }
+    const double target = total / n_wg;
+    size_t n_items = 0;
+    for (size_t a = 0; a < np; a++) {
+        const Piece &pc = pieces[a];
+        const OxhPlanOp &o = ops[pc.op];
+        const OxhSegment &sg = o.segs[pc.seg];
+        const uint32_t B = 4u * pc.runs;
+        /* the first run of a segment stores the quantised activations unless an earlier segment of the
+         * operation has stored the same ones */
+        bool keep = o.d_act_out != nullptr;
+        for (size_t k = 0; k < pc.seg && keep; k++) {
+            const OxhSegment &e = o.segs[k];
+            if (e.rows && e.act_first == sg.act_first && (e.n_vec ? e.n_vec : 1u) >= pc.nv) keep = false;
+        }
+        uint32_t g = 0;
+        while (g < pc.groups) {
+            uint32_t wg = 0;
+            for (uint32_t w = 1; w < n_wg; w++) if (load[w] < load[wg]) wg = w;
+            const double room = target - load[wg];
+            uint32_t rounds = room >= (double)pc.runs ? (uint32_t)(room / (double)pc.runs) : 1u;
+            if (rounds > 0xFFFFu) rounds = 0xFFFFu;
+            uint32_t take = pc.groups - g;
+            if (take > rounds * waves) take = rounds * waves;
+            if (n_items >= cap_items) {          /* cannot happen: every item but a segment's last is a whole round */
+                free(pieces); free(load); free(count); free(dealt);
+                return arg_fail("plan: item table overflow");
+            }
+            Dealt &d = dealt[n_items++];
+            d.wg = wg;
+            d.it.w = (const uint8_t *)sg.d_w + (size_t)g * pc.runs * Q80T_UNIT;
+            d.it.out = sg.d_out;
+            d.it.x = o.d_x + sg.act_first * o.cols;
+            d.it.keep = keep ? (uint8_t *)o.d_act_out + sg.act_first * (size_t)B * 34u : nullptr;
+            d.it.row0 = 16u * g;
+            d.it.rows = (uint32_t)sg.rows;
+            d.it.groups = take;
+            d.it.B = B;
+            d.it.nv = pc.nv;
+            d.it.out_stride = (uint32_t)o.out_stride;
+            d.it.same_x = 0;
+            d.it.pad = 0;
+            keep = false;
+            load[wg] += (double)((take + waves - 1u) / waves) * pc.runs;
+            count[wg + 1u]++;
+            g += take;
+        }
+    }
+    /* the table in workgroup order (a workgroup's items in the order they were dealt) */
+    Q80tItem *h = (Q80tItem *)calloc(n_items ? n_items : 1u, sizeof *h);
+    uint32_t *first = count;                    /* counts -> first indices, in place */
+    uint32_t *fill = (uint32_t *)calloc(n_wg, sizeof *fill);
+    if (!h || !fill) {
+        free(pieces); free(load); free(count); free(dealt); free(h); free(fill);
+        snprintf(g_err, sizeof g_err, "out of host memory building a plan");
+        return OXH_ERR_NOMEM;
+    }
+    for (uint32_t w = 0; w < n_wg; w++) first[w + 1u] += first[w];
+    for (size_t k = 0; k < n_items; k++) {
+        const uint32_t w = dealt[k].wg;
+        const uint32_t at = first[w] + fill[w]++;
+        h[at] = dealt[k].it;
+        if (fill[w] > 1u) {
+            const Q80tItem &pv = h[at - 1u];
+            h[at].same_x = (pv.x == h[at].x && pv.B == h[at].B && pv.nv == h[at].nv && !h[at].keep) ? 1u : 0u;
+        }
+    }
+    free(pieces); free(load); free(dealt); free(fill);
+    int rc = OXH_OK;
+    GemvMulti *m = (GemvMulti *)calloc(1, sizeof *m);
+    if (!m) { snprintf(g_err, sizeof g_err, "out of host memory building a plan"); rc = OXH_ERR_NOMEM; }
+    if (!rc) {
+        hipError_t e = hipMalloc((void **)&m->d_titems, (n_items ? n_items : 1u) * sizeof *h);
+        if (e == hipSuccess) e = hipMalloc((void **)&m->d_first, (size_t)(n_wg + 1u) * sizeof *first);
+        if (e == hipSuccess) e = hipMemcpy(m->d_titems, h, (n_items ? n_items : 1u) * sizeof *h, hipMemcpyHostToDevice);
+        if (e == hipSuccess) e = hipMemcpy(m->d_first, first, (size_t)(n_wg + 1u) * sizeof *first, hipMemcpyHostToDevice);
+        if (e != hipSuccess) {
+            if (m->d_titems) (void)hipFree(m->d_titems);
+            if (m->d_first) (void)hipFree(m->d_first);
+            free(m);
+            m = nullptr;
+            rc = hip_fail(e, "plan table");
+        }
+    }
+    free(h);
+    free(count);
+    if (rc) return rc;
+    m->n_ops = (uint32_t)n_ops;
+    m->n_items = (uint32_t)n_items;
+    m->grid = n_wg;
+    m->waves = waves;
+    m->which = MULTI_TILED;
+    m->lds = lds;
+    *handle = m;
+    return OXH_OK;
 }
 
 /* Cuts the rows of all operations into runs of at most 16 x rows_cap rows (what a workgroup's term
@@ -1627,6 +1816,7 @@ extern "C" int oxh_internal_multi_create(const OxhPlanOp *ops, size_t n_ops, voi
         snprintf(g_err, sizeof g_err, "plan: qtype %u has no multi-operation launch", ops[0].qtype);
         return OXH_DECLINED;
     }
+    if (which == MULTI_TILED) return multi_create_tiled(ops, n_ops, handle);
     const uint32_t W = GEMV_MAX_THREADS / 64u;
     const uint32_t n_cu = (uint32_t)(g_n_cu > 0 ? g_n_cu : 256);
     /* pass 1: check, and add up the bytes */
@@ -1766,6 +1956,15 @@ extern "C" int oxh_internal_multi_launch(void *handle, void *stream)
     GemvMulti *m = (GemvMulti *)handle;
     if (!m) return arg_fail("plan: NULL");
     hipStream_t st = pick_stream(stream);
+    if (m->which == MULTI_TILED) {
+        const dim3 tgrid(m->grid);
+        if (m->waves == 16u)
+            hipLaunchKernelGGL((k_q80t_multi<16, 2>), tgrid, dim3(1024), m->lds, st, m->d_titems, m->d_first);
+        else
+            hipLaunchKernelGGL((k_q80t_multi<8, 2>), tgrid, dim3(512), m->lds, st, m->d_titems, m->d_first);
+        HIP_TRY(hipGetLastError());
+        return OXH_OK;
+    }
     const dim3 grid(m->grid), block(GEMV_MAX_THREADS);
 #define OXH_MULTI(WHICH) hipLaunchKernelGGL((k_gemv_multi<WHICH>), grid, block, m->lds, st, m->d_items, m->d_first)
     switch (m->which) {
@@ -1793,7 +1992,7 @@ extern "C" int oxh_internal_multi_destroy(void *handle)
 {
     GemvMulti *m = (GemvMulti *)handle;
     if (!m) return OXH_OK;
-    hipError_t e = hipFree(m->d_items);
+    hipError_t e = hipFree(m->which == MULTI_TILED ? (void *)m->d_titems : (void *)m->d_items);
     const hipError_t e2 = hipFree(m->d_first);
     free(m);
     if (e == hipSuccess) e = e2;

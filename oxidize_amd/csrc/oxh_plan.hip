@@ -1233,6 +1233,26 @@ static double plan_table_cost(const PlanOp *run, size_t n_run)
 /* Q8_0, Q4_0, Q4_1, Q5_0, Q5_1, AL5_XS (and the aliases): the operations of one such format, none of
  * which touches what another writes, become a table of GEMV launches walked by one grid
  * (k_gemv_multi).  No workgroup waits for another there, so a plan with a dependency is declined. */
+/* What one operation of such a plan reads and writes: input rows and their quantised blocks over the
+ * activations its segments name (one, except in plans over tile-major Q8_0), and per segment the rows of
+ * every activation, out_stride floats apart. */
+static size_t multi_acts(const OxhPlanOp &o)
+{
+    size_t n = 1;
+    for (size_t k = 0; k < o.n_segs; k++) {
+        const size_t end = o.segs[k].act_first + (o.segs[k].n_vec ? o.segs[k].n_vec : 1u);
+        if (o.segs[k].rows && end > n) n = end;
+    }
+    return n;
+}
+
+static Span multi_out_span(const OxhPlanOp &o, size_t k)
+{
+    const size_t nv = o.segs[k].n_vec ? o.segs[k].n_vec : 1u;
+    const Span s = { (const char *)o.segs[k].d_out, ((nv - 1u) * o.out_stride + o.segs[k].rows) * sizeof(float) };
+    return s;
+}
+
 static int plan_create_multi(const OxhPlanOp *ops, size_t n_ops, OxhPlan **out)
 {
     for (size_t i = 0; i < n_ops; i++) {
@@ -1240,28 +1260,32 @@ static int plan_create_multi(const OxhPlanOp *ops, size_t n_ops, OxhPlan **out)
         if (!o.segs || o.n_segs == 0 || !o.d_x || o.cols == 0 || o.cols % OXH_QK8_0)
             return oxh_internal_errorf(OXH_ERR_ARG, "invalid argument: plan: operation %zu has no segments, no input or "
                                        "cols not a multiple of 32", i);
-        const Span xi = { (const char *)o.d_x, o.cols * sizeof(float) };
-        const Span ai = { (const char *)o.d_act_out, o.cols / OXH_QK8_0 * 34u };
+        for (size_t k = 0; k < o.n_segs; k++)
+            if (o.segs[k].act_first > 0xFFFFFFu || o.segs[k].n_vec > 16u || o.segs[k].rows > 0x3FFFFFFFull ||
+                o.out_stride > 0xFFFFFFFFull || o.cols > 0xFFFFFFu)
+                return oxh_internal_errorf(OXH_ERR_ARG, "invalid argument: plan: operation %zu: a segment's activations, "
+                                           "rows or the output stride are out of range", i);
+        const size_t acts_i = multi_acts(o);
+        const Span xi = { (const char *)o.d_x, acts_i * o.cols * sizeof(float) };
+        const Span ai = { (const char *)o.d_act_out, acts_i * (o.cols / OXH_QK8_0) * 34u };
         for (size_t k = 0; k < o.n_segs; k++) {
-            const Span wk = { (const char *)o.segs[k].d_out, o.segs[k].rows * sizeof(float) };
+            const Span wk = multi_out_span(o, k);
             if (spans_meet(wk, xi) || spans_meet(wk, ai) || spans_meet(ai, xi))
                 return oxh_internal_errorf(OXH_ERR_ARG, "invalid argument: plan: operation %zu stores over one of its own inputs", i);
         }
         for (size_t j = 0; j < i; j++) {
             const OxhPlanOp &e = ops[j];
-            const Span xj = { (const char *)e.d_x, e.cols * sizeof(float) };
-            const Span aj = { (const char *)e.d_act_out, e.cols / OXH_QK8_0 * 34u };
+            const size_t acts_j = multi_acts(e);
+            const Span xj = { (const char *)e.d_x, acts_j * e.cols * sizeof(float) };
+            const Span aj = { (const char *)e.d_act_out, acts_j * (e.cols / OXH_QK8_0) * 34u };
             bool hit = spans_meet(ai, xj) || spans_meet(aj, xi) || spans_meet(ai, aj);
             for (size_t k = 0; k < o.n_segs && !hit; k++) {
-                const Span wk = { (const char *)o.segs[k].d_out, o.segs[k].rows * sizeof(float) };
+                const Span wk = multi_out_span(o, k);
                 hit = spans_meet(wk, xj) || spans_meet(wk, aj);
-                for (size_t m = 0; m < e.n_segs && !hit; m++) {
-                    const Span wm = { (const char *)e.segs[m].d_out, e.segs[m].rows * sizeof(float) };
-                    hit = spans_meet(wk, wm);
-                }
+                for (size_t m = 0; m < e.n_segs && !hit; m++) hit = spans_meet(wk, multi_out_span(e, m));
             }
             for (size_t m = 0; m < e.n_segs && !hit; m++) {
-                const Span wm = { (const char *)e.segs[m].d_out, e.segs[m].rows * sizeof(float) };
+                const Span wm = multi_out_span(e, m);
                 hit = spans_meet(wm, xi) || spans_meet(wm, ai);
             }
             if (hit)

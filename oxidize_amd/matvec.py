@@ -304,7 +304,8 @@ def debug_subblock_sums(qtype, d_w, rows, cols, d_act, d_sums, stream=None):
 class Plan:
     """A chain of decode matmuls compiled into one launch (oxh_plan_*).  `ops` is a list of dicts with the
     arguments of one gemv_segments_fused call each: qtype, segs (from make_segments), cols, d_x and
-    optionally kind / d_b / eps / d_pro_out / d_add / d_sum_out (the prologue) and d_act_out."""
+    optionally kind / d_b / eps / d_pro_out / d_add / d_sum_out (the prologue), d_act_out and out_stride
+    (plans over Q8_0_T16 whose segments carry several activations)."""
 
     def __init__(self, ops):
         n = len(ops)
@@ -325,6 +326,7 @@ class Plan:
                 self._keep.append(pro)
                 o.pro = ctypes.pointer(pro)
             o.d_act_out = d.get("d_act_out")
+            o.out_stride = d.get("out_stride", 0)
             self._keep.append(d["segs"])
         self.handle = ctypes.c_void_p()
         status = lib().oxh_plan_create(arr, n, ctypes.byref(self.handle))

@@ -5,7 +5,7 @@ import numpy as np
 import pytest
 
 import oxlibs
-from oxidize_amd import synth
+from oxidize_amd import _lib, synth
 from oxidize_amd import matvec as mv
 
 pytestmark = pytest.mark.gpu
@@ -286,3 +286,123 @@ def test_host_batch_keeps_a_tile_major_copy_of_a_tall_q8_0_matrix(oxh):
     assert cached_bytes() == w.nbytes + mv.tile16_bytes(Q80, rows, cols)
     assert oxh.oxh_cpu_fallback_calls() == 0
     assert oxh.oxh_weight_clear() == 0
+
+
+# ── plans over tile-major Q8_0: many matrices, several activations each, one launch ─────────────────────────
+class _TiledOp:
+    """One operation: segments over their own matrices and runs of activations of one f32 input, its outputs
+    [activation][all segments' rows]; the file layout's launch beside the tile-major plan entry."""
+
+    def __init__(self, cols, segs, seed, keep_acts=True):
+        self.cols, self.segs = cols, segs                    # segs: [(rows, act_first, n_vec)]
+        self.n_act = max(a + n for _, a, n in segs)
+        self.total = sum(r for r, _, _ in segs)
+        self.d_x = mv.DeviceBuffer.from_host(synth.normal(self.n_act * cols, seed=seed, stream=1))
+        self.out_file, self.out_plan = mv.DeviceBuffer(16 * self.total * 4), mv.DeviceBuffer(16 * self.total * 4)
+        for b in (self.out_file, self.out_plan):
+            b.upload(np.full(16 * self.total, np.float32(-7.0)))
+        self.acts_file = mv.DeviceBuffer(self.n_act * mv.act_bytes(Q80, cols))
+        self.acts_plan = mv.DeviceBuffer(self.n_act * mv.act_bytes(Q80, cols)) if keep_acts else None
+        self.keep = []
+        file_items, plan_items, off = [], [], 0
+        for k, (rows, first, n_vec) in enumerate(segs):
+            w = synth.weights(Q80, rows, cols, seed=seed, stream=10 + k)
+            d_w = mv.DeviceBuffer.from_host(w)
+            d_t = mv.DeviceBuffer(mv.tile16_bytes(Q80, rows, cols))
+            mv.tile16(Q80, d_w.ptr, rows, cols, d_t.ptr)
+            self.keep += [d_w, d_t]
+            file_items.append((d_w.ptr, self.out_file.ptr + off * 4, rows, first, n_vec))
+            plan_items.append((d_t.ptr, self.out_plan.ptr + off * 4, rows, first, n_vec))
+            off += rows
+        self.file_items = file_items
+        self.file_segs, self.plan_segs = mv.make_segments(file_items), mv.make_segments(plan_items)
+
+    def launch_file_layout(self):
+        """the quantiser, then every segment from the file layout, at most eight activations per launch (what
+        the dot kernel takes)"""
+        mv.quantize(Q80, self.d_x.ptr, self.cols, self.n_act, self.cols, self.acts_file.ptr)
+        for d_w, d_out, rows, first, n_vec in self.file_items:
+            for v0 in range(0, n_vec, 8):
+                n = min(8, n_vec - v0)
+                mv.gemv_segments(Q80, mv.make_segments([(d_w, d_out + v0 * self.total * 4, rows, first + v0, n)]),
+                                 self.cols, self.acts_file.ptr, 1, self.total)
+
+    def plan_op(self):
+        return dict(qtype=mv.Q8_0_T16, segs=self.plan_segs, cols=self.cols, d_x=self.d_x.ptr,
+                    d_act_out=None if self.acts_plan is None else self.acts_plan.ptr, out_stride=self.total)
+
+    def check(self):
+        n = 16 * self.total
+        assert np.array_equal(bits(self.out_plan.download(np.float32, n)), bits(self.out_file.download(np.float32, n)))
+        if self.acts_plan is not None:                       # the blocks of every activation a segment names
+            got = self.acts_plan.download(np.uint8, self.acts_plan.nbytes).reshape(self.n_act, -1)
+            want = self.acts_file.download(np.uint8, self.acts_file.nbytes).reshape(self.n_act, -1)
+            named = sorted({v for _, first, n in self.segs for v in range(first, first + n)})
+            assert np.array_equal(got[named], want[named])
+
+
+def test_q8_0_tile_major_plan_gives_the_launches_bits(oxh):
+    """Operations of different widths, ragged row counts, several segments with their own runs of activations,
+    with and without the quantised blocks stored: one launch, the bits of the file layout's launches (which
+    other tests hold to the oracle), nothing written beyond a segment's rows and activations."""
+    ops = [_TiledOp(896, [(896, 0, 8), (128, 0, 8), (128, 0, 8)], seed=60),
+           _TiledOp(4864, [(896, 0, 8)], seed=61),
+           _TiledOp(896, [(4864, 0, 5), (4864, 0, 5)], seed=62, keep_acts=False),
+           _TiledOp(128, [(1, 0, 1), (17, 1, 16), (333, 3, 2)], seed=63),
+           _TiledOp(1024, [(50000, 2, 3)], seed=64),
+           _TiledOp(256, [(15, 0, 16)], seed=65, keep_acts=False)]
+    for o in ops:
+        o.launch_file_layout()
+    plan = mv.Plan([o.plan_op() for o in ops])
+    info = plan.info()
+    assert info["n_ops"] == len(ops) and info["n_waits"] == 0
+    assert info["lds_bytes"] == 4864 // 32 * 576                  # the widest staged image
+    for _ in range(2):                                       # a plan is launched again and again
+        plan.launch()
+    assert plan.status() == 0
+    for o in ops:
+        o.check()
+    plan.destroy()
+
+
+def test_q8_0_tile_major_plan_of_one_small_operation(oxh):
+    o = _TiledOp(128, [(16, 0, 1)], seed=66)
+    o.launch_file_layout()
+    plan = mv.Plan([o.plan_op()])
+    plan.launch()
+    assert plan.status() == 0
+    o.check()
+    plan.destroy()
+
+
+def test_q8_0_tile_major_plan_refusals(oxh):
+    a, b = _TiledOp(896, [(64, 0, 4)], seed=67), _TiledOp(896, [(64, 0, 4)], seed=68)
+    # an operation of another form among them
+    other = dict(qtype=Q80, segs=a.file_segs, cols=896, d_x=a.d_x.ptr)
+    with pytest.raises(mv.OxhError) as e:
+        mv.Plan([a.plan_op(), other])
+    assert e.value.status == mv.DECLINED
+    # several activations and no stride
+    op = a.plan_op()
+    op["out_stride"] = 0
+    with pytest.raises(mv.OxhError) as e:
+        mv.Plan([op])
+    assert e.value.status == _lib.ERR_ARG
+    # more activations than a tile holds
+    op = a.plan_op()
+    op["segs"] = mv.make_segments([(a.keep[1].ptr, a.out_plan.ptr, 64, 0, 17)])
+    with pytest.raises(mv.OxhError) as e:
+        mv.Plan([op])
+    assert e.value.status == _lib.ERR_ARG
+    # a width that is not whole runs of four blocks
+    op = a.plan_op()
+    op["cols"] = 96
+    with pytest.raises(mv.OxhError) as e:
+        mv.Plan([op])
+    assert e.value.status == mv.DECLINED
+    # an operation that reads what another writes
+    op = b.plan_op()
+    op["d_x"] = a.out_plan.ptr
+    with pytest.raises(mv.OxhError) as e:
+        mv.Plan([a.plan_op(), op])
+    assert e.value.status == mv.DECLINED
