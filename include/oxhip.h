@@ -278,7 +278,10 @@ int oxh_gemv_segments_fused(uint32_t qtype, const OxhSegment *segs, size_t n_seg
  * when given, receives the Q8_0 blocks of the same rows), activation v's rows
  * going out_stride floats after activation v - 1's.  The matrices are cut into
  * runs of whole 16-row groups and dealt so that every workgroup streams the
- * same amount; same bits as oxh_gemv_segments_f32 segment by segment.  This
+ * same amount; same bits as oxh_gemv_segments_f32 segment by segment.  (The
+ * independence check takes a segment's outputs as one span from its first
+ * activation's first row to its last one's last row: outputs of different
+ * operations interleaved in one buffer are declined.)  This
  * is how many small matrices are batched: a Qwen2.5-0.5B-shaped step of 97
  * matmuls at eight activations each is one launch.
  *
