@@ -1207,12 +1207,13 @@ static int launch_q80t_segments(const OxhSegment *segs, size_t n_segs, size_t co
     }
     if (forced_waves == 1u || forced_waves == 4u || forced_waves == 8u || forced_waves == 16u) waves = forced_waves;
     const size_t lds = image;
-    /* f32 inputs: with one or two activations per segment the workgroups quantise them themselves while
-     * they stage them (a launch less: head at one activation 27.4 against 30 us); with more, that work,
-     * repeated by every workgroup, costs more than the quantiser's launch (eight activations 36 against 32 us),
-     * and one-wave workgroups would each repeat all of it.  Without a buffer for the blocks there is no
-     * choice.  (OXH_Q80T_FUSE_NV moves the threshold.) */
-    static const uint32_t fuse_nv = env_u32("OXH_Q80T_FUSE_NV", 2, 0, 16);
+    /* f32 inputs: with up to four activations per segment the workgroups quantise them themselves while
+     * they stage them (a launch less: head at one activation 28.4 against 30 us, at four 30.5 against 31.1);
+     * with more, that work, repeated by every workgroup, costs what the quantiser's launch costs (eight
+     * activations 32.6 against 32.1 us, sixteen 39 against 33.5), and one-wave workgroups would each repeat
+     * all of it.  Without a buffer for the blocks there is no choice.  (OXH_Q80T_FUSE_NV moves the
+     * threshold.) */
+    static const uint32_t fuse_nv = env_u32("OXH_Q80T_FUSE_NV", 4, 0, 16);
     bool fused = false;
     uint8_t *acts = (uint8_t *)const_cast<void *>(io.d_acts);
     if (!acts) {
