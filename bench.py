@@ -727,6 +727,99 @@ def secondary_figures(mv, synth):
     return out
 
 
+def batched_step_figure(mv, synth, ds, single_us):
+    """Configuration 1's set at eight and sixteen activations per matmul (a batch of sequences decoding
+    together): not a launch per matmul (at that size q/k/v, o and down are launches of 64-96 row tiles on
+    256 CUs) but the independent matmuls of one shape grouped into launches of up to 32 segments, each segment
+    its own matrix and run of activations, Q4_K from tile-major copies: 7 matmul launches + 4 quantising
+    launches per step."""
+    import numpy as np
+    Q4K, Q6K = 13, 16
+    layers = ds.layers
+    keep, w_run = [], {}
+    for layer in range(layers):
+        for op, (name, qt, rows_, cols_, _) in enumerate(ds.ops):
+            for seg, r_ in enumerate(rows_):
+                if qt == Q4K:
+                    t = mv.DeviceBuffer(mv.tile16_bytes(Q4K, r_, cols_))
+                    mv.tile16(Q4K, ds.weights[layer][op][seg].ptr, r_, cols_, t.ptr)
+                elif ds.q6_grouped:                     # the tile kernel reads Q6_K in the file layout
+                    t = mv.DeviceBuffer.from_host(synth.weights(Q6K, r_, cols_, seed=ds.seed, stream=layer * 7 + 6))
+                else:
+                    t = ds.weights[layer][op][seg]
+                if t is not ds.weights[layer][op][seg]:
+                    keep.append(t)
+                w_run[(layer, op, seg)] = t
+    mv.sync()
+    res = {}
+    for nv in (8, 16):
+        bufs, launches, outs = [], [], {}
+        for op, (name, qt, rows_, cols_, _) in enumerate(ds.ops):
+            tot, n_in = sum(rows_), layers * nv
+            xin = mv.DeviceBuffer.from_host(synth.normal(n_in * cols_, seed=0, stream=900 + op))
+            aq = mv.DeviceBuffer(n_in * mv.act_bytes(qt, cols_))
+            bufs += [xin, aq]
+            items = []
+            for layer in range(layers):
+                o = mv.DeviceBuffer(nv * tot * 4)
+                bufs.append(o)
+                outs[(layer, op)] = (o, xin.ptr + layer * nv * cols_ * 4)
+                off = 0
+                for seg, r_ in enumerate(rows_):
+                    items.append((w_run[(layer, op, seg)].ptr, o.ptr + off * 4, r_, layer * nv, nv))
+                    off += r_
+            launches.append(("quantize", qt, cols_, xin, aq, n_in))
+            for k in range(0, len(items), 32):
+                launches.append(("gemv", mv.Q4_K_T16 if qt == Q4K else qt, mv.make_segments(items[k:k + 32]), cols_, aq, tot))
+
+        def step():
+            for l in launches:
+                if l[0] == "quantize":
+                    mv.quantize(l[1], l[3].ptr, l[2], l[5], l[2], l[4].ptr)
+                else:
+                    mv.gemv_segments(l[1], l[2], l[3], l[4].ptr, nv, l[5])
+
+        step()
+        mv.sync()
+        if nv == 8:
+            # the bits of a launch of its own over the file layout (which the tests hold to the oracle)
+            for layer, op in ((layers - 1, 0), (0, 3)):
+                name, qt, rows_, cols_, _ = ds.ops[op]
+                o, x_ptr = outs[(layer, op)]
+                tot = sum(rows_)
+                ref, a_ref = mv.DeviceBuffer(nv * tot * 4), mv.DeviceBuffer(nv * mv.act_bytes(qt, cols_))
+                items, off = [], 0
+                for seg, r_ in enumerate(rows_):
+                    w = ds.weights[layer][op][seg] if qt == Q4K else w_run[(layer, op, seg)]
+                    items.append((w.ptr, ref.ptr + off * 4, r_, 0))
+                    off += r_
+                mv.gemv_segments_f32(qt, mv.make_segments(items), cols_, x_ptr, cols_, a_ref.ptr, nv, tot)
+                mv.sync()
+                assert np.array_equal(o.download(np.uint32, nv * tot), ref.download(np.uint32, nv * tot))
+                ref.free()
+                a_ref.free()
+        graph = mv.Graph()
+        with graph:
+            step()
+        us = timed(graph.launch, 10, mv)
+        graph.destroy()
+        res["batch%d" % nv] = {"us_per_step": round(us, 1), "us_per_activation": round(us / nv, 1),
+                               "launches_per_step": len(launches),
+                               "weight_gbps": round(ds.weight_bytes / us / 1e3, 1),
+                               "frac_of_hbm_peak": round(ds.weight_bytes / us / 1e3 / HBM_PEAK_GBPS, 4)}
+        for b_ in bufs:
+            b_.free()
+    for b_ in keep:
+        b_.free()
+    res["note"] = ("the 128 matmuls of a Llama-3-8B-shaped step with 8 / 16 activations each, the matmuls of one shape "
+                   "grouped 32 segments to a launch (oxh_gemv_segments over OXH_Q4_K_T16 copies and file-layout Q6_K, "
+                   "one quantising launch per shape), replayed as a graph; two operations bit-checked against launches "
+                   "of their own.  The single-activation step takes %.0f us as one launch: per activation this is "
+                   "%.1fx / %.1fx less" % (single_us, single_us / res["batch8"]["us_per_activation"],
+                                           single_us / res["batch16"]["us_per_activation"]))
+    return res
+
+
 def _lib_check_copy(dst, src, nbytes):
     import ctypes
     from oxidize_amd import _lib
@@ -1102,6 +1195,7 @@ def main():
         from oxidize_amd import synth
         out["extra"] = secondary_figures(mv, synth)
         out["extra"]["decode_chain_fused"] = out["dependent_chain"]
+        out["extra"]["decode_step_llama3_8b_batch_8_16"] = batched_step_figure(mv, synth, ds, ev_ms * 1e3 / args.steps)
     out["cpu_baseline"] = None if args.no_cpu else cpu_baseline()
     if not args.no_cpu and out["cpu_baseline"]["kind"] == "reference" and isinstance(out.get("extra"), dict):
         one = cpu_baseline(layers_sample=2, min_seconds=1.5, cores=1)
