@@ -268,3 +268,30 @@ def test_mmq_tile_choice_is_host_arithmetic():
     assert tile(25, 4096, 512)[0] == _lib.DECLINED
     assert tile(Q4K, 0, 512)[0] == _lib.DECLINED
     assert lib.oxh_mmq_tile(Q4K, 4096, 512, 256, None, None) == 0
+
+
+def test_bindings_lay_the_structs_out_as_the_header_does(tmp_path):
+    """The ctypes structures of the bindings against the C compiler's view of include/oxhip.h: size and
+    the offset of every field (a field added to the header and not to the bindings would shift what
+    follows it)."""
+    import subprocess
+    structs = {"OxhSegment": _lib.OxhSegment, "OxhPrologue": _lib.OxhPrologue, "OxhPlanOp": _lib.OxhPlanOp,
+               "OxhMoe": _lib.OxhMoe, "OxhTensor": _lib.OxhTensor}
+    lines = ['#include <stdio.h>', '#include <stddef.h>', '#include "oxhip.h"', 'int main(void) {']
+    for name, cls in structs.items():
+        lines.append('printf("%s size %%zu\\n", sizeof(%s));' % (name, name))
+        for field, _ in cls._fields_:
+            lines.append('printf("%s %s %%zu\\n", offsetof(%s, %s));' % (name, field, name, field))
+    lines += ['return 0; }']
+    src = tmp_path / "layout.c"
+    src.write_text("\n".join(lines))
+    exe = tmp_path / "layout"
+    subprocess.run(["gcc", "-std=c11", "-I", os.path.join(ROOT, "include"), "-o", str(exe), str(src)], check=True)
+    seen = {}
+    for line in subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout.splitlines():
+        name, field, value = line.split()
+        seen[(name, field)] = int(value)
+    for name, cls in structs.items():
+        assert seen[(name, "size")] == ctypes.sizeof(cls), name
+        for field, _ in cls._fields_:
+            assert seen[(name, field)] == getattr(cls, field).offset, (name, field)
