@@ -768,16 +768,12 @@ def batched_step_figure(mv, synth, ds, single_us):
                 for seg, r_ in enumerate(rows_):
                     items.append((w_run[(layer, op, seg)].ptr, o.ptr + off * 4, r_, layer * nv, nv))
                     off += r_
-            launches.append(("quantize", qt, cols_, xin, aq, n_in))
-            for k in range(0, len(items), 32):
-                launches.append(("gemv", mv.Q4_K_T16 if qt == Q4K else qt, mv.make_segments(items[k:k + 32]), cols_, aq, tot))
+            # one call per shape: its 32-96 segments go out as launches of 32 over activations quantised once
+            launches.append((mv.Q4_K_T16 if qt == Q4K else qt, mv.make_segments(items), cols_, xin, aq, tot))
 
         def step():
-            for l in launches:
-                if l[0] == "quantize":
-                    mv.quantize(l[1], l[3].ptr, l[2], l[5], l[2], l[4].ptr)
-                else:
-                    mv.gemv_segments(l[1], l[2], l[3], l[4].ptr, nv, l[5])
+            for qt_, segs_, cols_, xin, aq, tot in launches:
+                mv.gemv_segments_f32(qt_, segs_, cols_, xin.ptr, cols_, aq.ptr, nv, tot)
 
         step()
         mv.sync()
@@ -804,7 +800,8 @@ def batched_step_figure(mv, synth, ds, single_us):
         us = timed(graph.launch, 10, mv)
         graph.destroy()
         res["batch%d" % nv] = {"us_per_step": round(us, 1), "us_per_activation": round(us / nv, 1),
-                               "launches_per_step": len(launches),
+                               "calls_per_step": len(launches),
+                               "launches_per_step": sum(1 + (len(l[1]) + 31) // 32 for l in launches),
                                "weight_gbps": round(ds.weight_bytes / us / 1e3, 1),
                                "frac_of_hbm_peak": round(ds.weight_bytes / us / 1e3 / HBM_PEAK_GBPS, 4)}
         for b_ in bufs:
@@ -812,7 +809,7 @@ def batched_step_figure(mv, synth, ds, single_us):
     for b_ in keep:
         b_.free()
     res["note"] = ("the 128 matmuls of a Llama-3-8B-shaped step with 8 / 16 activations each, the matmuls of one shape "
-                   "grouped 32 segments to a launch (oxh_gemv_segments over OXH_Q4_K_T16 copies and file-layout Q6_K, "
+                   "in one oxh_gemv_segments_f32 call (32 segments to a launch, OXH_Q4_K_T16 copies and file-layout Q6_K, "
                    "one quantising launch per shape), replayed as a graph; two operations bit-checked against launches "
                    "of their own.  The single-activation step takes %.0f us as one launch: per activation this is "
                    "%.1fx / %.1fx less" % (single_us, single_us / res["batch8"]["us_per_activation"],

@@ -159,7 +159,9 @@ typedef struct OxhSegment {
  * matvec_fused_multi_input_slice (matvec.c:640-797) and the small-batch
  * rows path (matvec.c:1079-1102); the device analogue is
  * oc_cuda_mmq_matvec / _matvec_expert (cuda_mmq.h:57-72).  Segments live in
- * HOST memory and are copied into the launch. */
+ * HOST memory and are copied into the launch; a launch takes 32 of them, a
+ * call with more runs as launches of 32 (over f32 inputs: quantised once for
+ * all, which needs d_act_out; no prologue then). */
 int oxh_gemv_segments(uint32_t qtype, const OxhSegment *segs, size_t n_segs,
                       size_t cols, const void *d_acts, size_t n_vec,
                       size_t out_stride, void *stream);

@@ -1340,11 +1340,37 @@ static int launch_gemv(uint32_t qtype, const OxhSegment *segs, size_t n_segs, si
     if (!segs || (!io.d_acts && !io.d_x)) return arg_fail("gemv: NULL pointer");
     if (n_vec < 1 || n_vec > MQ80_TOK) return arg_fail("gemv: n_vec must be 1..8");
     const size_t n_vec_default = n_vec;
-    if (n_segs > OXH_MAX_SEGS) return arg_fail("gemv: more than 32 segments in one launch");
     const int kind = oxh_act_kind(qtype, cols);
     if (!kind) {
         snprintf(g_err, sizeof g_err, "gemv: qtype %u with cols %zu has no integer path", qtype, cols);
         return OXH_DECLINED;
+    }
+    if (n_segs > OXH_MAX_SEGS) {
+        /* A launch's segment table holds 32: more segments go out in launches of 32, over activations that
+         * are quantised once for all of them (f32 inputs need the buffer for the quantised bytes). */
+        if (dump || io.pro) return arg_fail("gemv: more than 32 segments take no prologue and no sub-block dump");
+        GemvIo each = io;
+        if (!io.d_acts) {
+            if (!io.d_act_out) return arg_fail("gemv: more than 32 segments over f32 inputs need d_act_out");
+            size_t act_end = 0;
+            for (size_t i = 0; i < n_segs; i++) {
+                const size_t nv = segs[i].n_vec ? segs[i].n_vec : n_vec;
+                if (nv > MQ80_TOK || segs[i].act_first > 0xFFFFFFFFull) return arg_fail("gemv: segment n_vec or act_first out of range");
+                if (segs[i].rows && segs[i].act_first + nv > act_end) act_end = segs[i].act_first + nv;
+            }
+            if (act_end == 0) return OXH_OK;
+            rc = kind == 2 ? oxh_quantize_q8_k(io.d_x, io.x_stride, act_end, cols, io.d_act_out, stream)
+                           : oxh_quantize_q8_0(io.d_x, io.x_stride, act_end, cols, io.d_act_out, stream);
+            if (rc) return rc;
+            each.d_acts = io.d_act_out;
+            each.d_x = nullptr;
+            each.d_act_out = nullptr;
+        }
+        for (size_t k = 0; k < n_segs; k += OXH_MAX_SEGS) {
+            const size_t n = n_segs - k < OXH_MAX_SEGS ? n_segs - k : OXH_MAX_SEGS;
+            if ((rc = launch_gemv(qtype, segs + k, n, cols, each, n_vec, out_stride, nullptr, stream))) return rc;
+        }
+        return OXH_OK;
     }
     const size_t blocks = kind == 2 ? cols / OXH_QK_K : cols / OXH_QK8_0;
     if (blocks > 0xFFFFu) {

@@ -490,3 +490,41 @@ def test_token_tiled_kernel_of_the_32_value_formats(oxh, qtype, rows, cols, n_ve
     for v in sorted(set(list(range(0, n_vec, 13)) + [n_vec // 2, 63 % n_vec, 64 % n_vec, n_vec - 1])):
         want, _ = oracle_matvec(canon, w, rows, cols, np.ascontiguousarray(xs[v]))
         assert np.array_equal(bits(outs[v, :rows]), bits(want)), v
+
+
+@pytest.mark.parametrize("qtype,rows,cols,n_vec", [(Q4K, 40, 512, 3), (Q80, 33, 256, 1), (Q6K, 70, 256, 8)])
+def test_a_call_with_more_than_32_segments_runs_as_launches_of_32(oxh, qtype, rows, cols, n_vec):
+    """Seventy segments, each its own matrix and run of activations, in one call: the bits of the same
+    segments in calls of at most 32, over quantised activations and over f32 inputs with a buffer for the
+    quantised bytes; f32 inputs without one are refused."""
+    from oxidize_amd import _lib
+    n_seg = 70
+    rb = synth.row_bytes(qtype, cols)
+    w = synth.weights(qtype, n_seg * rows, cols, seed=97)
+    d_w = mv.DeviceBuffer.from_host(w)
+    n_act = n_seg * n_vec
+    d_x = mv.DeviceBuffer.from_host(synth.normal(n_act * cols, seed=97, stream=1))
+    nact = mv.act_bytes(qtype, cols)
+    a_ref, a_all = mv.DeviceBuffer(n_act * nact), mv.DeviceBuffer(n_act * nact)
+    outs = [mv.DeviceBuffer(n_act * rows * 4) for _ in range(3)]
+    for o in outs:
+        o.upload(np.full(n_act * rows, np.float32(-3.0)))
+
+    def items(o):
+        return [(d_w.ptr + s * rows * rb, o.ptr + s * n_vec * rows * 4, rows, s * n_vec, n_vec) for s in range(n_seg)]
+
+    mv.quantize(qtype, d_x.ptr, cols, n_act, cols, a_ref.ptr)
+    it = items(outs[0])
+    for k in range(0, n_seg, 32):
+        mv.gemv_segments(qtype, mv.make_segments(it[k:k + 32]), cols, a_ref.ptr, 1, rows)
+    mv.gemv_segments(qtype, mv.make_segments(items(outs[1])), cols, a_ref.ptr, 1, rows)
+    mv.gemv_segments_f32(qtype, mv.make_segments(items(outs[2])), cols, d_x.ptr, cols, a_all.ptr, 1, rows)
+    mv.sync()
+    want = outs[0].download(np.float32, n_act * rows)
+    assert not np.any(want == np.float32(-3.0))
+    assert np.array_equal(bits(outs[1].download(np.float32, n_act * rows)), bits(want))
+    assert np.array_equal(bits(outs[2].download(np.float32, n_act * rows)), bits(want))
+    assert np.array_equal(a_all.download(np.uint8, n_act * nact), a_ref.download(np.uint8, n_act * nact))
+    with pytest.raises(mv.OxhError) as e:
+        mv.gemv_segments_f32(qtype, mv.make_segments(items(outs[2])), cols, d_x.ptr, cols, None, 1, rows)
+    assert e.value.status == _lib.ERR_ARG
