@@ -870,6 +870,54 @@ def q80_step_probe(mv, synth):
     assert plan.status() == 0
 
 
+def q80_batch_probe(mv, synth):
+    """For `rocprofv3 --pmc FETCH_SIZE` / `WRITE_SIZE` runs on k_q80t_multi: three 256 MiB device-to-device
+    copies (known traffic), then three launches of the Qwen2.5-0.5B-shaped Q8_0 step at eight activations per
+    matmul as one plan over tile-major copies.  Prints nothing."""
+    import ctypes
+    from oxidize_amd import _lib
+    from oxidize_amd.workloads import DecodeSet, QWEN2_5_0_5B
+    Q80, nvb = 7, 8
+    n = 256 << 20
+    a, b = mv.DeviceBuffer(n), mv.DeviceBuffer(n)
+    _lib.check(_lib.lib().oxh_memset(ctypes.c_void_p(a.ptr), 1, n, None))
+    for _ in range(3):
+        _lib.check(_lib.lib().oxh_memcpy_d2d(ctypes.c_void_p(b.ptr), ctypes.c_void_p(a.ptr), n, None))
+    mv.sync()
+    rows, cols = 151936, 896
+    qs = DecodeSet(qtypes=(Q80, Q80), seed=0, **QWEN2_5_0_5B)
+    keep, ops = [], []
+
+    def tiled(d_w, r_, c_):
+        t = mv.DeviceBuffer(mv.tile16_bytes(Q80, r_, c_))
+        mv.tile16(Q80, d_w.ptr, r_, c_, t.ptr)
+        keep.append(t)
+        return t
+
+    for layer in range(qs.layers):
+        for op, (name, qt, rows_, cols_, _) in enumerate(qs.ops):
+            tot = sum(rows_)
+            x = mv.DeviceBuffer.from_host(synth.normal(nvb * cols_, seed=0, stream=500000 + layer * 8 + op))
+            o = mv.DeviceBuffer(nvb * tot * 4)
+            keep += [x, o]
+            items, off = [], 0
+            for seg, r_ in enumerate(rows_):
+                items.append((tiled(qs.weights[layer][op][seg], r_, cols_).ptr, o.ptr + off * 4, r_, 0, nvb))
+                off += r_
+            ops.append(dict(qtype=mv.Q8_0_T16, segs=mv.make_segments(items), cols=cols_, d_x=x.ptr, d_act_out=None,
+                            out_stride=tot))
+    d_head = mv.DeviceBuffer.from_host(synth.weights(Q80, rows, cols, seed=0, stream=5))
+    hx = mv.DeviceBuffer.from_host(synth.normal(nvb * cols, seed=0, stream=9))
+    ho = mv.DeviceBuffer(nvb * rows * 4)
+    ops.append(dict(qtype=mv.Q8_0_T16, segs=mv.make_segments([(tiled(d_head, rows, cols).ptr, ho.ptr, rows, 0, nvb)]),
+                    cols=cols, d_x=hx.ptr, d_act_out=None, out_stride=rows))
+    mv.sync()
+    plan = mv.Plan(ops)
+    for _ in range(3):
+        plan.launch()
+    assert plan.status() == 0
+
+
 def split_probe(mv, synth):
     """For `rocprofv3 --kernel-trace --stats` runs on the small-batch launches whose tiles share their
     columns between workgroups: a 4096 x 14336 Q6_K matrix under 16 activations, twelve launches of
@@ -1026,7 +1074,7 @@ def main():
     ap.add_argument("--mode", choices=["plan", "graph", "launches"], default="plan",
                     help="a step as one persistent launch (default), as a HIP graph of 128 launches, or as 128 launches")
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary configurations")
-    ap.add_argument("--probe", choices=["traffic", "mmq", "q80step", "split", "head", "moe"], help="run a counter-collection workload and exit")
+    ap.add_argument("--probe", choices=["traffic", "mmq", "q80step", "q80batch", "split", "head", "moe"], help="run a counter-collection workload and exit")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this path is built and measured on ONE GPU; --gpus %d is not supported "
@@ -1056,6 +1104,10 @@ def main():
     if args.probe == "q80step":
         from oxidize_amd import synth
         q80_step_probe(mv, synth)
+        return 0
+    if args.probe == "q80batch":
+        from oxidize_amd import synth
+        q80_batch_probe(mv, synth)
         return 0
 
     ds = DecodeSet(layers=args.layers, seed=0)
