@@ -40,14 +40,19 @@ PLAN_STEP_TRAFFIC_BYTES = 4441622891
 INT8_PEAK_TOPS = 5033.0     # dense int8 MFMA: 256 CU x 2.4 GHz x 8192 op/clk/CU
 
 
-def timed(fn, reps, mv, spin_ms=15.0):
-    """Average microseconds of fn() over `reps` back-to-back calls (HIP events), after `spin_ms` milliseconds
-    of the same calls untimed: between two legs the host generates and uploads data while the device idles,
-    and the first tens of launches after that run slower (an expert step 171 us where it settles at 161)."""
+LEG_SPINUP_MS = 15.0        # --leg-spinup-ms
+
+
+def timed(fn, reps, mv):
+    """Average microseconds of fn() over `reps` back-to-back calls (HIP events), after LEG_SPINUP_MS
+    milliseconds of the same calls untimed: between two legs the host generates and uploads data while the
+    device idles, and the first tens of launches after that run slower (an expert step 171 us where it settles
+    at 161).  Runs under a tracing profiler pass --leg-spinup-ms 0: the untimed calls multiply the dispatches
+    it has to record."""
     fn()
     mv.sync()
     t_spin = time.perf_counter()
-    while (time.perf_counter() - t_spin) * 1e3 < spin_ms:
+    while (time.perf_counter() - t_spin) * 1e3 < LEG_SPINUP_MS:
         for _ in range(4):
             fn()
         mv.sync()
@@ -1078,6 +1083,7 @@ def cpu_baseline(layers_sample=8, min_seconds=2.5, cores=None):
 
 
 def main():
+    global LEG_SPINUP_MS
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     # a launch of the step kernel takes 0.8-1.1 ms for the first thirty or so launches after the device
@@ -1086,6 +1092,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=40)
     ap.add_argument("--spinup-ms", type=float, default=60.0,
                     help="untimed milliseconds of the same step before the warm-up steps (device clocks settle)")
+    ap.add_argument("--leg-spinup-ms", type=float, default=LEG_SPINUP_MS,
+                    help="untimed milliseconds of the same calls in front of every other timed leg (0 under a tracing profiler)")
     ap.add_argument("--layers", type=int, default=32, help=argparse.SUPPRESS)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--mode", choices=["plan", "graph", "launches"], default="plan",
@@ -1093,6 +1101,7 @@ def main():
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary configurations")
     ap.add_argument("--probe", choices=["traffic", "mmq", "q80step", "q80batch", "split", "head", "moe"], help="run a counter-collection workload and exit")
     args = ap.parse_args()
+    LEG_SPINUP_MS = max(0.0, args.leg_spinup_ms)
     if args.gpus != 1:
         print("bench.py: this path is built and measured on ONE GPU; --gpus %d is not supported "
               "(the work would shard by output rows across GPUs; nothing here launches a second rank)" % args.gpus, file=sys.stderr)
