@@ -40,7 +40,7 @@ PLAN_STEP_TRAFFIC_BYTES = 4441622891
 INT8_PEAK_TOPS = 5033.0     # dense int8 MFMA: 256 CU x 2.4 GHz x 8192 op/clk/CU
 
 
-LEG_SPINUP_MS = 15.0        # --leg-spinup-ms
+LEG_SPINUP_MS = 50.0        # --leg-spinup-ms
 
 
 def timed(fn, reps, mv):
