@@ -1271,10 +1271,12 @@ static int launch_mmq_segments(uint32_t qtype, const OxhSegment *segs, size_t n_
         acts = (const uint8_t *)io.d_act_out;
     }
     /* A Q4_K launch whose 64-row tiles would give at most two workgroups per CU, but whose 128-row tiles
-     * still give nearly every CU one, takes those on eight waves with three super-blocks per stage: half as
-     * much again in flight per CU (OXH_MOE_WIDE_SMALL=0 switches it off).  Q5_K and Q6_K rows leave room
-     * for two per stage only, and with two the wider tile measured slower than the 64-row one. */
-    static const uint32_t wide_ok = env_u32("OXH_MOE_WIDE_SMALL", 1, 0, 1);
+     * still give nearly every CU one, can take those on eight waves with three super-blocks per stage: half as
+     * much again in flight per CU.  Off by default (OXH_MOE_WIDE_SMALL=1 switches it on): launched
+     * continuously, Mixtral's down projections at 16 tokens run faster on the 64-row tiles with two
+     * super-blocks per stage (an expert step 154.5 against 158.5 us); the wider tile only won when the
+     * launches were timed right after an idle period. */
+    static const uint32_t wide_ok = env_u32("OXH_MOE_WIDE_SMALL", 0, 0, 1);
     const size_t cus = (size_t)(g_n_cu > 0 ? g_n_cu : 256);
     size_t wg64 = 0, wg128 = 0;
     for (size_t i = 0; i < n_segs; i++) {
@@ -2790,13 +2792,13 @@ static int launch_experts(uint32_t qtype, const void *const *d_w, float *const *
     if (big_from && avg_tokens >= big_from)
         return launch_experts_tiled<4, 8>(qtype, d_w, d_out, n_mat, n_expert, rows, cols, d_acts, out_stride,
                                           d_counts, d_offsets, max_tokens, stream);
-    /* few rows per expert (a down projection): the 64-row tile would give at most two workgroups per CU;
-     * Q4_K takes 128 rows on eight waves with three super-blocks per stage, half as much again in flight
-     * (Mixtral's down projections at 16 tokens: 67 against 74 us; Q5_K and Q6_K rows leave room for two per
-     * stage only, and with two the wider tile measured slower).  Workgroups of experts without a token
-     * leave at once, so what counts is the experts that can have one; with too few of them the smaller
-     * tile spreads over more CUs. */
-    static const uint32_t wide = env_u32("OXH_MOE_WIDE_SMALL", 1, 0, 1);
+    /* few rows per expert (a down projection): the 64-row tile gives at most two workgroups per CU; Q4_K
+     * can take 128 rows on eight waves with three super-blocks per stage instead, half as much again in
+     * flight (OXH_MOE_WIDE_SMALL=1).  Off by default: launched continuously, Mixtral's down projections at
+     * 16 tokens run faster on the 64-row tiles with two super-blocks per stage (the layer 163 against 169 us;
+     * the wider tile only won when the launches were timed right after an idle period).  Workgroups of
+     * experts without a token leave at once, so what counts is the experts that can have one. */
+    static const uint32_t wide = env_u32("OXH_MOE_WIDE_SMALL", 0, 0, 1);
     const size_t cus = (size_t)(g_n_cu > 0 ? g_n_cu : 256);
     const size_t live = pairs < n_expert ? (pairs ? pairs : 1) : n_expert;
     if (wide && is_q4k(file_type) && n_mat * n_expert * ((rows + 63) / 64) <= 2u * cus &&

@@ -246,12 +246,31 @@ def test_layer_with_prefill_sized_token_counts(oxh, qt_gu, qt_dn):
 
 
 @pytest.mark.parametrize("qt_gu,qt_dn", [(Q4K, Q4K), (Q4K, Q6K), (Q6K, Q5K)])
-def test_layer_whose_down_projection_takes_the_128_row_tile(oxh, qt_gu, qt_dn):
-    """8 experts x 4096 output rows: 512 workgroups of the 64-row tile (two per CU on a 256-CU device), so
-    a Q4_K down launch runs on 128-row tiles of eight waves with three super-blocks per stage (the other
-    types stay on 64-row tiles with two); likewise 9 experts x 3584 rows."""
+def test_layer_whose_down_projection_gives_two_workgroups_per_cu(oxh, qt_gu, qt_dn):
+    """8 experts x 4096 output rows: 512 workgroups of the 64-row tile (two per CU on a 256-CU device), which
+    then stage two super-blocks per barrier; likewise 9 experts x 3584 rows.  (With OXH_MOE_WIDE_SMALL=1 a
+    Q4_K down launch of this size runs on 128-row tiles of eight waves instead: the test below.)"""
     check_layer(qt_gu, qt_dn, 8, 2, 4096, 256, 16, seed=31, skew=False)
     check_layer(qt_gu, qt_dn, 9, 3, 3584, 512, 9, seed=32, skew=True)
+
+
+def test_the_128_row_tile_when_switched_on(oxh):
+    """OXH_MOE_WIDE_SMALL=1 is read once per process: the layers above, the Mixtral-shaped layer and
+    configuration 4's expert launches over host-made lists, in a process of their own with the switch on,
+    against the same oracle checks."""
+    import os
+    import subprocess
+    import sys
+    if os.environ.get("OXH_MOE_WIDE_SMALL") == "1":
+        pytest.skip("this is the process with the switch on")
+    env = dict(os.environ, OXH_MOE_WIDE_SMALL="1")
+    proc = subprocess.run([sys.executable, "-m", "pytest", "-x", "-q", "-p", "no:cacheprovider", "--timeout", "120",
+                           "--timeout-method", "thread",
+                           "tests/test_gpu_moe.py::test_layer_whose_down_projection_gives_two_workgroups_per_cu",
+                           "tests/test_gpu_moe.py::test_mixtral_shape_sampled_and_graph_replay",
+                           "tests/test_gpu_configs.py::test_config4_moe_expert_gemvs"],
+                          cwd=oxlibs.ROOT, env=env, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=300)
+    assert proc.returncode == 0 and " passed" in proc.stdout, proc.stdout[-2000:]
 
 
 def test_layer_with_more_experts_than_one_launch_carries(oxh):
